@@ -1,0 +1,59 @@
+/* t2sp_hip.h — the thin C-ABI layer over the HIP kernels (gfx950).
+ *
+ * Plain pointers and sizes only.  Every pointer is a DEVICE pointer unless a
+ * comment says otherwise; `stream` is a hipStream_t passed as void* (NULL = the
+ * default stream).  Calls enqueue work and return without synchronising.
+ * Return value: T2SP_OK, or a negative code (same numbering as the Halide error
+ * codes the reference's generated interface returns,
+ * Halide/src/runtime/HalideRuntime.h:957-1143).
+ *
+ * The operator entry points that take halide_buffer_t* (gemm-interface.h,
+ * conv-interface.h, capsule-interface.h, mttkrp-interface.h) validate their
+ * buffers, stage data, and then call the functions declared here.
+ */
+#ifndef T2SP_HIP_H
+#define T2SP_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define T2SP_OK 0
+#define T2SP_ERR_SHAPE (-8)   /* halide_error_code_constraint_violated */
+#define T2SP_ERR_LAUNCH (-23) /* halide_error_code_device_run_failed   */
+
+/* Tile configurations of the SGEMM kernel (cfg argument). */
+#define T2SP_GEMM_CFG_AUTO 0
+#define T2SP_GEMM_CFG_256x256 1
+#define T2SP_GEMM_CFG_128x128 2
+#define T2SP_GEMM_CFG_64x128 3
+#define T2SP_GEMM_CFG_SCALAR 99
+
+/* C[i,j] = sum_k A[i,k] * B[k,j], fp32, row-major with leading dimensions in
+ * elements.  Replaces the device side of the reference's SGEMM pipeline: the
+ * kernels of t2s/tests/performance/gemm/bitstream/a10/a.cl:67-770 launched by
+ * halide_opencl_wait_for_kernels_finish (t2s/src/AOT-OpenCL-Runtime.cpp:312-397). */
+int t2sp_sgemm_f32(const float *A, const float *B, float *C, int M, int N, int K, int64_t lda,
+                   int64_t ldb, int64_t ldc, int cfg, void *stream);
+
+/* Same product, written straight into the reference's 6-D tiled output
+ * c(jjj, iii, jj, ii, j, i) (t2s/tests/performance/gemm/gemm-run-fpga.cpp:69;
+ * row = iii + III*ii + III*II*i, col = jjj + JJJ*jj + JJJ*JJ*j, gemm.cpp:39-41).
+ * strides6[d] is the element stride of output dimension d.  Replaces the
+ * unloader kernel plus the host deserializer loop of the generated interface. */
+int t2sp_sgemm_f32_tiled(const float *A, const float *B, float *C, int M, int N, int K,
+                         int64_t lda, int64_t ldb, int jjj, int iii, int jj, int ii,
+                         const int64_t *strides6, int cfg, void *stream);
+
+/* x[i] = u(seed, i), i in [0,n): the seeded uniform[-1,1) generator shared with
+ * the CPU checker (same bits for the same seed and index).  The reference's
+ * drivers fill their inputs with unseeded random() (gemm-run-fpga.cpp:57-67);
+ * this is the seeded replacement the benchmark configurations ask for. */
+int t2sp_fill_uniform_f32(float *x, int64_t n, uint64_t seed, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* T2SP_HIP_H */

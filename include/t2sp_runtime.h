@@ -1,0 +1,27 @@
+/* t2sp_runtime.h — the few runtime calls a driver may use next to the operator
+ * entry points.  They stand in for pieces of t2s/src/AOT-OpenCL-Runtime.cpp. */
+#ifndef T2SP_RUNTIME_H
+#define T2SP_RUNTIME_H
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* GPU time, in nanoseconds, of the kernels of the most recent operator call
+ * (hipEvent bracket on the library stream).  Counterpart of the
+ * "latest end - earliest start" figure the reference writes to exec_time.txt
+ * (t2s/src/AOT-OpenCL-Runtime.cpp:358-396) and reads back with ExecTime()
+ * (t2s/src/Roofline.cpp:113-140), and of the value the oneAPI-flavour entry
+ * returns (t2s/src/CodeGen_OneAPI_Dev.cpp:3554-3617). */
+double t2sp_last_kernel_ns(void);
+
+/* Frees the cached device allocations the entry points keep between calls
+ * (counterpart of halide_device_and_host_free, AOT-OpenCL-Runtime.cpp:280-295). */
+void t2sp_release(void);
+
+/* Number of HIP devices visible; 0 when there is none. */
+int t2sp_device_count(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

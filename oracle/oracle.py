@@ -1,0 +1,173 @@
+"""ctypes front end of liboracle.so (oracle.c): TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg import this
+module.  Arrays are numpy float32; every tensor is described by element strides
+per logical index, so one function covers every memory layout (see oracle.c for
+the reference file:line each function follows).
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+
+ACC_F32, ACC_F32_FMA, ACC_F64 = 0, 1, 2
+ORDER_GOLDEN, ORDER_URE = 0, 1
+
+_lib = None
+
+
+def build():
+    """Compile oracle.c into liboracle.so (gcc only)."""
+    subprocess.check_call(["make", "-C", _HERE, "-B", "liboracle.so"], stdout=subprocess.DEVNULL)
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        i64, fp, ip = ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p
+        _lib.oracle_fill_uniform.argtypes = [fp, i64, ctypes.c_uint64]
+        _lib.oracle_gemm.argtypes = [fp, fp, fp] + [i64] * 11 + [ctypes.c_int, ctypes.c_int]
+        _lib.oracle_gemm_literal.argtypes = [fp, fp, fp] + [i64] * 5
+        _lib.oracle_conv.argtypes = [fp, fp, fp, ip, ip, ip, ip, i64, i64, i64, i64, ctypes.c_int,
+                                     i64, ctypes.c_int, ctypes.c_int]
+        _lib.oracle_capsule.argtypes = [fp, fp, fp, ip, ip, ip, ip, i64, i64, ctypes.c_int, i64,
+                                        ctypes.c_int, ctypes.c_int]
+        _lib.oracle_mttkrp.argtypes = [fp, fp, fp, fp, ip, ip, ip, ip, ip, i64, i64, ctypes.c_int,
+                                       ctypes.c_int]
+        _lib.oracle_mttkrp_literal.argtypes = [fp, fp, fp, fp] + [i64] * 6
+        _lib.oracle_max_threads.restype = ctypes.c_int
+        for f in (_lib.oracle_fill_uniform, _lib.oracle_gemm, _lib.oracle_gemm_literal,
+                  _lib.oracle_conv, _lib.oracle_capsule, _lib.oracle_mttkrp,
+                  _lib.oracle_mttkrp_literal):
+            f.restype = None
+    return _lib
+
+
+def _p(a):
+    assert a.dtype == np.float32
+    return a.ctypes.data
+
+
+def _i64(seq):
+    return np.asarray(list(seq), dtype=np.int64)
+
+
+def _estrides(a):
+    assert all(s % a.itemsize == 0 for s in a.strides)
+    return [s // a.itemsize for s in a.strides]
+
+
+def fill_uniform(shape, seed):
+    """float32 array of `shape` (C order) with x.flat[i] = u(seed, i) in [-1, 1)."""
+    x = np.empty(shape, dtype=np.float32)
+    lib().oracle_fill_uniform(_p(x), x.size, ctypes.c_uint64(seed))
+    return x
+
+
+def gemm(A, B, acc=ACC_F32, rows=None, threads=0):
+    """C = A @ B for 2-D float32 views A[M,K], B[K,N] (any strides).
+
+    Returns the full M x N array; when `rows` = (row0, nrows) only those rows
+    are computed and an nrows x N array is returned."""
+    M, K = A.shape
+    K2, N = B.shape
+    assert K == K2
+    row0, nrows = (0, M) if rows is None else rows
+    C = np.zeros((nrows, N), dtype=np.float32)
+    sa, sb = _estrides(A), _estrides(B)
+    lib().oracle_gemm(_p(A), _p(B), C.ctypes.data - row0 * N * 4, M, N, K, sa[0], sa[1], sb[0], sb[1],
+                      N, 1, row0, nrows, acc, threads)
+    return C
+
+
+def gemm_literal(A, B, rows=None):
+    A = np.ascontiguousarray(A)
+    B = np.ascontiguousarray(B)
+    M, K = A.shape
+    N = B.shape[1]
+    row0, nrows = (0, M) if rows is None else rows
+    C = np.zeros((nrows, N), dtype=np.float32)
+    lib().oracle_gemm_literal(_p(A), _p(B), C.ctypes.data - row0 * N * 4, M, N, K, row0, nrows)
+    return C
+
+
+def conv(I, W, stride=(1, 1), order=ORDER_GOLDEN, cii=1, acc=ACC_F32, n_range=None, co_range=None,
+         threads=0):
+    """O[n,co,y,x] = sum I[n,ci,y*sy+ky,x*sx+kx] * W[co,ci,ky,kx].
+
+    I, W are 4-D float32 views indexed (n,ci,y,x) and (co,ci,ky,kx) with any
+    strides; "y" is the axis the reference calls y (kernel tap ky runs fastest
+    in its golden loop).  Returns O indexed (n,co,y,x), C-contiguous, zero
+    outside the requested n/co ranges."""
+    N, CI, IY, IX = I.shape
+    CO, CI2, KY, KX = W.shape
+    assert CI == CI2
+    sy, sx = stride
+    OY, OX = (IY - KY) // sy + 1, (IX - KX) // sx + 1
+    O = np.zeros((N, CO, OY, OX), dtype=np.float32)
+    n0, n1 = (0, N) if n_range is None else n_range
+    c0, c1 = (0, CO) if co_range is None else co_range
+    dims = _i64([N, CI, CO, OY, OX, KY, KX, sy, sx])
+    si, sw, so = _i64(_estrides(I)), _i64(_estrides(W)), _i64(_estrides(O))
+    lib().oracle_conv(_p(I), _p(W), _p(O), dims.ctypes.data, si.ctypes.data, sw.ctypes.data,
+                      so.ctypes.data, n0, n1, c0, c1, order, cii, acc, threads)
+    return O
+
+
+def capsule(P, W, stride=2, order=ORDER_GOLDEN, cii=1, acc=ACC_F32, n_range=None, threads=0):
+    """V[n,co,y,x,mx,my] = sum P[n,ci,y*S+ky,x*S+kx,mx,mk] * W[co,ci,ky,kx,mk,my].
+
+    P is a 6-D view indexed (n,ci,y,x,mx,mk), W is indexed (co,ci,ky,kx,mk,my).
+    Returns V indexed (n,co,y,x,mx,my), C-contiguous."""
+    N, CI, IY, IX, MX, MK = P.shape
+    CO, CI2, KY, KX, MK2, MY = W.shape
+    assert CI == CI2 and MK == MK2
+    OY, OX = (IY - KY) // stride + 1, (IX - KX) // stride + 1
+    V = np.zeros((N, CO, OY, OX, MX, MY), dtype=np.float32)
+    n0, n1 = (0, N) if n_range is None else n_range
+    dims = _i64([N, CI, CO, OY, OX, KY, KX, stride, MX, MY, MK])
+    sp, sw, sv = _i64(_estrides(P)), _i64(_estrides(W)), _i64(_estrides(V))
+    lib().oracle_capsule(_p(P), _p(W), _p(V), dims.ctypes.data, sp.ctypes.data, sw.ctypes.data,
+                         sv.ctypes.data, n0, n1, order, cii, acc, threads)
+    return V
+
+
+def mttkrp(B, C, D, acc=ACC_F32, i_range=None, threads=0):
+    """A[i,r] = sum_k (sum_j B[i,j,k] C[j,r]) D[k,r] in the reference's two-step order.
+
+    B is a 3-D view indexed (i,j,k); C (j,r); D (k,r).  Returns A (i,r)."""
+    I, J, K = B.shape
+    J2, R = C.shape
+    K2, R2 = D.shape
+    assert J == J2 and K == K2 and R == R2
+    A = np.zeros((I, R), dtype=np.float32)
+    i0, i1 = (0, I) if i_range is None else i_range
+    dims = _i64([I, J, K, R])
+    sb, sc, sd, sa = (_i64(_estrides(x)) for x in (B, C, D, A))
+    lib().oracle_mttkrp(_p(B), _p(C), _p(D), _p(A), dims.ctypes.data, sb.ctypes.data, sc.ctypes.data,
+                        sd.ctypes.data, sa.ctypes.data, i0, i1, acc, threads)
+    return A
+
+
+def mttkrp_literal(a, b, c, i_range=None):
+    """util.h:498-515 on dense reference-layout arrays: a[k][i][l], c[j][l], b[j][k] -> d[j][i]
+    (numpy C order; the reference's first index is the last numpy axis)."""
+    K, I, L = a.shape
+    J = c.shape[0]
+    assert c.shape == (J, L) and b.shape == (J, K)
+    a, b, c = (np.ascontiguousarray(x) for x in (a, b, c))
+    d = np.zeros((J, I), dtype=np.float32)
+    i0, i1 = (0, I) if i_range is None else i_range
+    lib().oracle_mttkrp_literal(_p(a), _p(b), _p(c), _p(d), L, I, J, K, i0, i1)
+    return d
+
+
+def max_threads():
+    return lib().oracle_max_threads()

@@ -1,0 +1,46 @@
+"""Loader of libt2sp_mi355x.so (built in-tree by t2sp_amd/csrc/Makefile)."""
+import ctypes
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(_HERE, "libt2sp_mi355x.so")
+_lib = None
+
+
+def lib_path():
+    return _LIB
+
+
+def build(jobs=8):
+    """Compile every HIP/C++ source for gfx950 into libt2sp_mi355x.so."""
+    subprocess.check_call(["make", "-C", os.path.join(_HERE, "csrc"), "-B", "-j%d" % jobs])
+
+
+def lib():
+    """The loaded library.  Raises if it has not been built: there is no fallback."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB):
+            raise RuntimeError(
+                "%s is missing: run `python -c 'import __graft_entry__ as g; g.build()'` "
+                "or `make -C t2sp_amd/csrc` first (no CPU fallback exists)" % _LIB)
+        _lib = ctypes.CDLL(_LIB)
+        _declare(_lib)
+    return _lib
+
+
+def _declare(L):
+    from .buffer import halide_buffer_t
+    bp = ctypes.POINTER(halide_buffer_t)
+    vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    L.gemm.argtypes = [bp, bp, bp]
+    L.GEMM.argtypes = [bp, bp, bp]
+    L.t2sp_gemm_with_cfg.argtypes = [bp, bp, bp, i32]
+    L.t2sp_sgemm_f32.argtypes = [vp, vp, vp, i32, i32, i32, i64, i64, i64, i32, vp]
+    L.t2sp_sgemm_f32_tiled.argtypes = [vp, vp, vp, i32, i32, i32, i64, i64, i32, i32, i32, i32,
+                                       ctypes.POINTER(i64), i32, vp]
+    L.t2sp_fill_uniform_f32.argtypes = [vp, i64, ctypes.c_uint64, vp]
+    L.t2sp_last_kernel_ns.restype = ctypes.c_double
+    L.t2sp_release.restype = None
+    L.t2sp_device_count.restype = i32

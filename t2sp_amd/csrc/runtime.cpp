@@ -1,0 +1,213 @@
+// runtime.cpp — see runtime.hpp.
+#include "runtime.hpp"
+
+#include <atomic>
+
+namespace t2sp {
+
+std::mutex &api_mutex() {
+    static std::mutex m;
+    return m;
+}
+
+// The entry points run on the default stream: it orders against work the caller
+// queued on it (for example a framework that filled a pre-staged device buffer).
+hipStream_t api_stream() { return nullptr; }
+
+static std::atomic<double> g_last_kernel_ns{0.0};
+static hipEvent_t g_ev0 = nullptr, g_ev1 = nullptr;
+
+int report(int code, const char *op, const char *what) {
+    if (code != 0) fprintf(stderr, "t2sp: %s: %s (error %d)\n", op, what, code);
+    return code;
+}
+
+int check_buffer(const halide_buffer_t *b, const char *op, const char *name, int dims_a,
+                 int dims_b, Span *span) {
+    char msg[160];
+    if (!b) {
+        snprintf(msg, sizeof msg, "buffer argument %s is NULL", name);
+        return report(halide_error_code_buffer_argument_is_null, op, msg);
+    }
+    if (b->type.code != halide_type_float || b->type.bits != 32 || b->type.lanes != 1) {
+        snprintf(msg, sizeof msg, "%s has type code %d bits %d lanes %d, expected float32", name,
+                 (int)b->type.code, (int)b->type.bits, (int)b->type.lanes);
+        return report(halide_error_code_bad_type, op, msg);
+    }
+    if (b->dimensions != dims_a && b->dimensions != dims_b) {
+        snprintf(msg, sizeof msg, "%s has %d dimensions, expected %d%s", name, b->dimensions, dims_a,
+                 dims_b != dims_a ? " (or the tiled form)" : "");
+        return report(halide_error_code_bad_dimensions, op, msg);
+    }
+    if (!b->dim) {
+        snprintf(msg, sizeof msg, "%s has no dimension array", name);
+        return report(halide_error_code_buffer_is_null, op, msg);
+    }
+    int64_t elements = 1, spn = 1;
+    for (int d = 0; d < b->dimensions; d++) {
+        if (b->dim[d].extent < 0) {
+            snprintf(msg, sizeof msg, "%s dimension %d has negative extent %d", name, d,
+                     b->dim[d].extent);
+            return report(halide_error_code_buffer_extents_negative, op, msg);
+        }
+        if (b->dim[d].stride < 0) {
+            snprintf(msg, sizeof msg, "%s dimension %d has negative stride", name, d);
+            return report(halide_error_code_constraint_violated, op, msg);
+        }
+        elements *= b->dim[d].extent;
+        spn += (int64_t)(b->dim[d].extent > 0 ? b->dim[d].extent - 1 : 0) * b->dim[d].stride;
+    }
+    if (b->dimensions > 0 && b->dim[0].stride != 1) {
+        snprintf(msg, sizeof msg, "%s.stride.0 is %d, must be 1", name, b->dim[0].stride);
+        return report(halide_error_code_constraint_violated, op, msg);
+    }
+    if (!b->host && !b->device) {
+        snprintf(msg, sizeof msg, "%s has neither host nor device memory", name);
+        return report(halide_error_code_host_is_null, op, msg);
+    }
+    if ((b->flags & halide_buffer_flag_host_dirty) && (b->flags & halide_buffer_flag_device_dirty)) {
+        snprintf(msg, sizeof msg, "%s is dirty on both host and device", name);
+        return report(halide_error_code_host_and_device_dirty, op, msg);
+    }
+    if (span) {
+        span->elements = elements;
+        span->span = elements == 0 ? 0 : spn;
+    }
+    return 0;
+}
+
+void *DevicePool::get(size_t bytes) {
+    if (bytes == 0) bytes = 16;
+    Block *best = nullptr;
+    for (auto &b : blocks_)
+        if (!b.busy && b.bytes >= bytes && (!best || b.bytes < best->bytes)) best = &b;
+    if (best && best->bytes <= 2 * bytes + (1u << 20)) {
+        best->busy = true;
+        return best->p;
+    }
+    void *p = nullptr;
+    if (hipMalloc(&p, bytes) != hipSuccess) {
+        // drop idle blocks and retry once
+        for (size_t i = 0; i < blocks_.size();) {
+            if (!blocks_[i].busy) {
+                (void)hipFree(blocks_[i].p);
+                blocks_.erase(blocks_.begin() + i);
+            } else {
+                i++;
+            }
+        }
+        (void)hipGetLastError();
+        if (hipMalloc(&p, bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+    }
+    blocks_.push_back({p, bytes, true});
+    return p;
+}
+
+void DevicePool::put(void *p) {
+    for (auto &b : blocks_)
+        if (b.p == p) b.busy = false;
+}
+
+void DevicePool::release_all() {
+    for (auto &b : blocks_) (void)hipFree(b.p);
+    blocks_.clear();
+}
+
+DevicePool &pool() {
+    static DevicePool p;
+    return p;
+}
+
+Staged::~Staged() {
+    if (pooled_ && ptr_) pool().put(ptr_);
+}
+
+int Staged::input(const halide_buffer_t *b, const Span &s, const char *op) {
+    span_ = s.span;
+    const size_t bytes = (size_t)s.span * sizeof(float);
+    if (b->device) {
+        ptr_ = reinterpret_cast<float *>(b->device);
+        if ((b->flags & halide_buffer_flag_host_dirty) && b->host && bytes)
+            if (hipMemcpyAsync(ptr_, b->host, bytes, hipMemcpyHostToDevice, api_stream()) != hipSuccess)
+                return report(halide_error_code_copy_to_device_failed, op, "host to device copy failed");
+        return 0;
+    }
+    ptr_ = static_cast<float *>(pool().get(bytes));
+    if (!ptr_) return report(halide_error_code_device_malloc_failed, op, "device allocation failed");
+    pooled_ = true;
+    if (bytes && hipMemcpyAsync(ptr_, b->host, bytes, hipMemcpyHostToDevice, api_stream()) != hipSuccess)
+        return report(halide_error_code_copy_to_device_failed, op, "host to device copy failed");
+    return 0;
+}
+
+int Staged::output(halide_buffer_t *b, const Span &s, const char *op) {
+    span_ = s.span;
+    out_ = b;
+    const size_t bytes = (size_t)s.span * sizeof(float);
+    if (b->device) {
+        ptr_ = reinterpret_cast<float *>(b->device);
+        return 0;
+    }
+    ptr_ = static_cast<float *>(pool().get(bytes));
+    if (!ptr_) return report(halide_error_code_device_malloc_failed, op, "device allocation failed");
+    pooled_ = true;
+    if (s.span != s.elements && bytes)
+        if (hipMemcpyAsync(ptr_, b->host, bytes, hipMemcpyHostToDevice, api_stream()) != hipSuccess)
+            return report(halide_error_code_copy_to_device_failed, op, "host to device copy failed");
+    return 0;
+}
+
+int Staged::finish(const char *op) {
+    if (!out_) return 0;
+    if (!pooled_) {
+        out_->flags |= halide_buffer_flag_device_dirty;
+        out_->flags &= ~(uint64_t)halide_buffer_flag_host_dirty;
+        return 0;
+    }
+    const size_t bytes = (size_t)span_ * sizeof(float);
+    if (bytes && hipMemcpy(out_->host, ptr_, bytes, hipMemcpyDeviceToHost) != hipSuccess)
+        return report(halide_error_code_copy_to_host_failed, op, "device to host copy failed");
+    out_->flags &= ~(uint64_t)(halide_buffer_flag_device_dirty | halide_buffer_flag_host_dirty);
+    return 0;
+}
+
+KernelTimer::KernelTimer() {
+    if (!g_ev0) {
+        (void)hipEventCreate(&g_ev0);
+        (void)hipEventCreate(&g_ev1);
+    }
+    (void)hipEventRecord(g_ev0, api_stream());
+}
+
+int KernelTimer::stop_and_sync(const char *op) {
+    (void)hipEventRecord(g_ev1, api_stream());
+    if (hipStreamSynchronize(api_stream()) != hipSuccess) {
+        (void)hipGetLastError();
+        return report(halide_error_code_device_run_failed, op, "kernel execution failed");
+    }
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, g_ev0, g_ev1) == hipSuccess) g_last_kernel_ns = (double)ms * 1e6;
+    return 0;
+}
+
+}  // namespace t2sp
+
+extern "C" double t2sp_last_kernel_ns(void) { return t2sp::g_last_kernel_ns.load(); }
+
+extern "C" void t2sp_release(void) {
+    std::lock_guard<std::mutex> lock(t2sp::api_mutex());
+    (void)hipDeviceSynchronize();
+    t2sp::pool().release_all();
+}
+
+extern "C" int t2sp_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return n;
+}
