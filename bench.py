@@ -1,0 +1,176 @@
+#!/usr/bin/env python3
+"""bench.py — throughput of the hot path on one MI355X.
+
+A step is one pass of the hot path over one batch of synthetic input: one SGEMM
+C = A*B at M=N=K=8192 (fp32, row-major, A and B uniform[-1,1) from a seed),
+inputs resident in HBM before the timed region starts.  One JSON line is
+printed:
+  value/unit      whole-job TFLOP/s over the timed region (2*M*N*K flop per step)
+  roofline        dominant kernel against the fp32 MFMA peak; `achieved` comes
+                  from HIP events around every launch in the timed region, on the
+                  stream the kernel is launched on
+  cpu_baseline    the CPU restatement of the reference's golden loop, timed on
+                  this host on a bounded sample of the same workload
+  parity          relative Frobenius / max-abs error of this run's result against
+                  the CPU oracle on sampled rows
+  others          the remaining benchmark configurations (SGEMM sweep; conv,
+                  capsule, MTTKRP once built), each with its own TFLOP/s and
+                  fraction of peak
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3   # 256 CU x 256 flop/clk/CU x 2.4 GHz
+PEAK_HBM_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-others", action="store_true", help="skip the non-headline configurations")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
+    return ap.parse_args()
+
+
+def time_launches(torch, launch, steps, warmup):
+    """Run `launch` warmup+steps times; return (ms_per_step over the bracketed region,
+    average per-launch ms from events recorded on the launch stream)."""
+    for _ in range(warmup):
+        launch()
+    torch.cuda.synchronize()
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    t0 = time.perf_counter()
+    evs[0].record()
+    for i in range(steps):
+        launch()
+        evs[i + 1].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    per = [evs[i].elapsed_time(evs[i + 1]) for i in range(steps)]
+    return wall_ms, sum(per) / len(per), min(per)
+
+
+def sgemm_case(torch, t2sp_amd, M, N, K, steps, warmup, seed=1):
+    L = t2sp_amd.lib()
+    A = t2sp_amd.fill_uniform(torch.empty(M, K, device="cuda"), seed)
+    B = t2sp_amd.fill_uniform(torch.empty(K, N, device="cuda"), seed + 1)
+    C = torch.empty(M, N, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        rc = L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, stream)
+        if rc != 0:
+            raise RuntimeError("t2sp_sgemm_f32 returned %d" % rc)
+
+    wall_ms, avg_ms, min_ms = time_launches(torch, launch, steps, warmup)
+    flop = 2.0 * M * N * K
+    return dict(A=A, B=B, C=C, wall_ms=wall_ms, avg_ms=avg_ms, min_ms=min_ms, flop=flop)
+
+
+def cpu_baseline_gemm(oracle, M, N, K, budget_s):
+    """The reference's golden loop (gemm-run-fpga.cpp:74-86) restated in C, one thread, on a
+    sample of output rows of the same M x N x K problem, extrapolated linearly."""
+    import numpy as np
+    A = oracle.fill_uniform((8, K), 1)
+    B = oracle.fill_uniform((K, N), 2)
+    t0 = time.perf_counter()
+    oracle.gemm_literal(A, B, rows=(0, 1))
+    one = time.perf_counter() - t0
+    rows = int(max(1, min(8, budget_s / max(one, 1e-6))))
+    t0 = time.perf_counter()
+    oracle.gemm_literal(A, B, rows=(0, rows))
+    dt = time.perf_counter() - t0
+    gflops = 2.0 * rows * N * K / dt / 1e9
+    # the same arithmetic, loops reordered over independent outputs, all host threads
+    threads = oracle.max_threads()
+    Am = oracle.fill_uniform((64, K), 1)
+    t0 = time.perf_counter()
+    oracle.gemm(Am, B)
+    dt_mt = time.perf_counter() - t0
+    return {
+        "value": round(gflops / 1e3, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+        "sample": "golden loop (i,j,k order, scalar accumulator) on %d of %d output rows of the %dx%dx%d SGEMM, "
+                  "single thread, %.1f s; extrapolated full problem: %.0f s" % (rows, M, M, N, K, dt, dt / rows * M),
+        "all_threads": {"value": round(2.0 * 64 * N * K / dt_mt / 1e12, 6), "unit": "TFLOP/s", "cores": threads,
+                        "sample": "same per-element arithmetic, outputs vectorised and spread over OpenMP threads, "
+                                  "64 of %d rows, %.2f s" % (M, dt_mt)},
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus %d is not supported (every box has one GPU, "
+              "and the path shards without exchange: see DESIGN.md)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import numpy as np
+    import torch
+    import t2sp_amd
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    t2sp_amd.lib()
+
+    M = N = K = 8192
+    r = sgemm_case(torch, t2sp_amd, M, N, K, args.steps, args.warmup)
+    tflops = r["flop"] / (r["wall_ms"] * 1e-3) / 1e12
+    kernel_tflops = r["flop"] / (r["avg_ms"] * 1e-3) / 1e12
+
+    out = {
+        "metric": "fp32 TFLOPS + % of fp32-MFMA peak, SGEMM 8192^3 on 1 MI355X",
+        "value": round(tflops, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(r["wall_ms"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "SGEMM C=A*B, M=N=K=8192, fp32 row-major, uniform[-1,1) seeds 1,2 (configs[1])",
+                   "entry": "t2sp_sgemm_f32", "inputs": "resident in HBM"},
+        "pct_of_peak": round(100.0 * tflops / PEAK_FP32_MFMA_TFLOPS, 2),
+        "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 3), "peak": PEAK_FP32_MFMA_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(kernel_tflops / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+                     "kernel": "sgemm_kernel<256x256x16>", "avg_launch_ms": round(r["avg_ms"], 4),
+                     "best_launch_ms": round(r["min_ms"], 4), "flop_per_launch": r["flop"]},
+    }
+
+    from oracle import oracle
+    rows = np.unique(np.concatenate([[0, M - 1], np.random.default_rng(0).integers(0, M, 30)]))
+    idx = torch.as_tensor(rows, device="cuda")
+    ref = oracle.gemm(r["A"][idx].cpu().numpy(), r["B"].cpu().numpy())
+    got = r["C"][idx].cpu().numpy().astype(np.float64)
+    out["parity"] = {"rel_frobenius": float(np.linalg.norm(got - ref) / np.linalg.norm(ref)),
+                     "max_abs": float(np.abs(got - ref).max()), "rows_checked": int(len(rows)),
+                     "against": "CPU oracle, sequential float32 golden loop"}
+    del r
+
+    if not args.no_others:
+        others = {}
+        for (m, n, k) in [(4096, 16384, 2048), (16384, 4096, 8192), (1024, 1024, 1024)]:
+            c = sgemm_case(torch, t2sp_amd, m, n, k, max(5, args.steps // 2), 2)
+            tf = c["flop"] / (c["avg_ms"] * 1e-3) / 1e12
+            others["sgemm_%dx%dx%d" % (m, n, k)] = {"TFLOP/s": round(tf, 3), "frac_of_peak": round(tf / PEAK_FP32_MFMA_TFLOPS, 4),
+                                                    "avg_launch_ms": round(c["avg_ms"], 4)}
+            del c
+        try:
+            from t2sp_amd import bench_ops
+            others.update(bench_ops.run_all(torch, max(5, args.steps // 2), 2, PEAK_FP32_MFMA_TFLOPS))
+        except ImportError:
+            pass
+        out["others"] = others
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline_gemm(oracle, M, N, K, args.cpu_seconds)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

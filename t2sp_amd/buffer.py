@@ -77,6 +77,9 @@ class HalideBuffer:
         assert isinstance(a, np.ndarray) and a.dtype == np.float32
         assert all(s % 4 == 0 for s in a.strides)
         ext, st = cls._dims_of(a.shape, [s // 4 for s in a.strides])
+        if a.size == 0:  # numpy gives empty arrays arbitrary strides; describe them densely
+            st = [int(np.prod(ext[:d], dtype=np.int64)) if d else 1 for d in range(len(ext))]
+            st = [max(x, 1) for x in st]
         return cls(ext, st, host=a.ctypes.data, keep=a)
 
     @classmethod

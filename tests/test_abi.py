@@ -1,0 +1,105 @@
+"""CPU-only checks of the boundary: the library loads, exports every symbol the
+headers in include/ declare, and the entry points reject bad arguments with the
+reference's error codes before any device work (Halide/src/AddImageChecks.cpp:352-636,
+codes Halide/src/runtime/HalideRuntime.h:957-1143)."""
+import ctypes
+import glob
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+import t2sp_amd
+from t2sp_amd.buffer import HalideBuffer, halide_buffer_t
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    names = set()
+    for h in glob.glob(os.path.join(ROOT, "include", "*.h")):
+        text = re.sub(r"/\*.*?\*/", "", open(h).read(), flags=re.S)
+        text = re.sub(r"//[^\n]*", "", text)
+        for m in re.finditer(r"^(?:int|double|void)\s+(\w+)\s*\(", text, flags=re.M):
+            names.add(m.group(1))
+    return names
+
+
+def test_library_exports_every_declared_symbol():
+    L = t2sp_amd.lib()
+    names = declared_symbols()
+    assert {"gemm", "GEMM", "t2sp_sgemm_f32", "t2sp_last_kernel_ns"} <= names
+    missing = [n for n in sorted(names) if not hasattr(L, n)]
+    assert not missing, missing
+
+
+def test_headers_compile_as_c_and_cpp(tmp_path):
+    inc = os.path.join(ROOT, "include")
+    headers = sorted(os.path.basename(h) for h in glob.glob(os.path.join(inc, "*.h")))
+    src = "".join('#include "%s"\n' % h for h in headers) + "int main(void){return sizeof(halide_buffer_t)==56?0:1;}\n"
+    for ext, cc in ((".c", "gcc"), (".cpp", "g++")):
+        f = tmp_path / ("t" + ext)
+        f.write_text(src)
+        exe = str(tmp_path / ("t" + ext + ".out"))
+        subprocess.check_call([cc, "-Wall", "-Werror", "-I", inc, str(f), "-o", exe])
+        assert subprocess.call([exe]) == 0
+
+
+def test_struct_layout_matches_header():
+    assert ctypes.sizeof(halide_buffer_t) == 56
+    assert halide_buffer_t.host.offset == 16 and halide_buffer_t.flags.offset == 24
+    assert halide_buffer_t.type.offset == 32 and halide_buffer_t.dimensions.offset == 36
+    assert halide_buffer_t.dim.offset == 40
+
+
+def test_numpy_buffer_follows_halide_dimension_order():
+    a = np.zeros((3, 5, 7), np.float32)
+    b = HalideBuffer.from_numpy(a)
+    dims = [(b.struct.dim[d].extent, b.struct.dim[d].stride) for d in range(3)]
+    assert dims == [(7, 1), (5, 7), (3, 35)]
+
+
+def _buf(shape, **kw):
+    return HalideBuffer.from_numpy(np.zeros(shape, np.float32), **kw)
+
+
+def test_gemm_rejects_bad_arguments_without_a_device():
+    L = t2sp_amd.lib()
+    a, b, c = _buf((8, 4)), _buf((4, 12)), _buf((8, 12))
+    assert L.gemm(None, b.ref, c.ref) == -12                 # buffer argument is NULL
+    assert L.gemm(a.ref, b.ref, None) == -12
+    bad_type = _buf((8, 4))
+    bad_type.struct.type.bits = 64
+    assert L.gemm(bad_type.ref, b.ref, c.ref) == -3          # bad type
+    assert L.gemm(_buf((2, 8, 4)).ref, b.ref, c.ref) == -43  # bad dimensions
+    assert L.gemm(a.ref, b.ref, _buf((8, 12, 1)).ref) == -43
+    assert L.gemm(a.ref, _buf((3, 12)).ref, c.ref) == -4     # B too small: out of bounds
+    assert L.gemm(a.ref, _buf((5, 12)).ref, c.ref) == -8     # constraint violated
+    assert L.gemm(a.ref, b.ref, _buf((8, 8)).ref) == -4      # C too small
+    nohost = _buf((8, 4))
+    nohost.struct.host = None
+    assert L.gemm(nohost.ref, b.ref, c.ref) == -34           # host is NULL
+    strided = HalideBuffer.from_numpy(np.zeros((8, 8), np.float32)[:, ::2])
+    assert L.gemm(strided.ref, b.ref, c.ref) == -8           # stride.0 must be 1
+    both = _buf((8, 4))
+    both.struct.flags = 3
+    assert L.gemm(both.ref, b.ref, c.ref) == -37             # dirty on host and device
+    neg = _buf((8, 4))
+    neg.struct.dim[1].extent = -1
+    assert L.gemm(neg.ref, b.ref, c.ref) == -28
+
+
+def test_thin_layer_rejects_bad_shapes():
+    L = t2sp_amd.lib()
+    assert L.t2sp_sgemm_f32(None, None, None, 0, 4, 4, 4, 4, 4, 0, None) == -8
+    assert L.t2sp_sgemm_f32(None, None, None, 4, 4, 4, 4, 4, 4, 12345, None) in (-8, -23)
+    assert L.t2sp_fill_uniform_f32(None, -1, 0, None) == -8
+    assert L.t2sp_fill_uniform_f32(None, 0, 0, None) == 0
+
+
+def test_python_mirror_raises_with_code():
+    with pytest.raises(t2sp_amd.T2spError) as e:
+        t2sp_amd.gemm(np.zeros((8, 4), np.float32), np.zeros((5, 12), np.float32))
+    assert e.value.code == -8

@@ -1,0 +1,159 @@
+"""GPU parity tests of the SGEMM path, called through the C entry points
+`gemm` / `GEMM` (include/gemm-interface.h) and the thin layer (include/t2sp_hip.h).
+
+Bar: relative Frobenius error <= 1e-5 against the CPU oracle's sequential
+float32 golden loop on the same seeded inputs (max-abs error is printed), and
+exact equality where the inputs make float32 sums order-independent."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import t2sp_amd
+from conftest import rel_fro
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+CFGS = [0, 1, 2, 3]
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+    assert torch.cuda.is_available()
+    return torch
+
+
+def detile(Ct):
+    """(I, J, II, JJ, III, JJJ) tiled result -> flat (M, N), per gemm.cpp:39-41."""
+    I, J, II, JJ, III, JJJ = Ct.shape
+    return Ct.transpose(0, 2, 4, 1, 3, 5).reshape(I * II * III, J * JJ * JJJ)
+
+
+@pytest.mark.parametrize("cfg", CFGS)
+def test_config1_1024_cubed_seed0_host_buffers(oracle, cfg):
+    """BASELINE config 1: M=N=K=1024, uniform[-1,1) from seed 0, host buffers in and out."""
+    A, B = oracle.fill_uniform((1024, 1024), 0), oracle.fill_uniform((1024, 1024), 1)
+    ref = oracle.gemm(A, B)
+    C = t2sp_amd.gemm(A, B, cfg=cfg)
+    err, mx = rel_fro(C, ref)
+    print("cfg %d rel_fro %.3e max_abs %.3e" % (cfg, err, mx))
+    assert err <= TOL
+    err_fma, _ = rel_fro(C, oracle.gemm(A, B, acc=oracle.ACC_F32_FMA))
+    err64, _ = rel_fro(C, oracle.gemm(A, B, acc=oracle.ACC_F64))
+    assert err_fma <= TOL and err64 <= TOL
+
+
+def test_device_buffers_and_fill_match_cpu_generator(oracle, torch_cuda):
+    torch = torch_cuda
+    M, N, K = 512, 768, 640
+    A = t2sp_amd.fill_uniform(torch.empty(M, K, device="cuda"), 5)
+    B = t2sp_amd.fill_uniform(torch.empty(K, N, device="cuda"), 6)
+    assert (A.cpu().numpy() == oracle.fill_uniform((M, K), 5)).all()
+    assert (B.cpu().numpy() == oracle.fill_uniform((K, N), 6)).all()
+    C = torch.full((M, N), float("nan"), device="cuda")
+    t2sp_amd.gemm(A, B, out=C)
+    torch.cuda.synchronize()
+    err, _ = rel_fro(C.cpu().numpy(), oracle.gemm(A.cpu().numpy(), B.cpu().numpy()))
+    assert err <= TOL
+    assert t2sp_amd.last_kernel_ns() > 0
+
+
+@pytest.mark.parametrize("K", [64, 2048])
+def test_aot_boundary_closed_form_tiled_output(oracle, K):
+    """The reference's AOT boundary test (correctness/aot/gemm-run.cpp:36-80): A[i,k]=k+i,
+    B[k,j]=j-k into the tiled result(JJJ,III,JJ,II,J,I) through `GEMM`, with its constants
+    III=2, II=4, JJJ=4, JJ=4, outermost 2x2.  At K=64 the closed form is exact in float32;
+    at the test's own K=2048 the reference's tolerance (0.5% per element) applies."""
+    III, II, JJJ, JJ, OI, OJ = 2, 4, 4, 4, 2, 2
+    M, N = III * II * OI, JJJ * JJ * OJ
+    i, j, k = np.arange(M), np.arange(N), np.arange(K)
+    A = (k[None, :] + i[:, None]).astype(np.float32)
+    B = (j[None, :] - k[:, None]).astype(np.float32)
+    S1, S2 = K * (K - 1) // 2, (K - 1) * K * (2 * K - 1) // 6
+    want = (j[None, :] - i[:, None]) * S1 + i[:, None] * j[None, :] * K - S2
+    Ct = np.full(t2sp_amd.gemm_tiled_shape(M, N, III, II, JJJ, JJ), np.nan, np.float32)
+    a, b, c = (t2sp_amd.HalideBuffer.from_numpy(x) for x in (A, B, Ct))
+    assert c.struct.dimensions == 6
+    assert t2sp_amd.lib().GEMM(a.ref, b.ref, c.ref) == 0
+    got = detile(Ct)
+    if K == 64:
+        assert (got == want).all()
+    else:
+        assert (np.abs(got - want) <= 0.005 * np.abs(want)).all()
+        assert rel_fro(got, oracle.gemm(A, B))[0] <= TOL
+
+
+@pytest.mark.parametrize("tiles", [(16, 4, 8, 2), (10, 32, 8, 32), (2, 32, 4, 32), (5, 3, 6, 7)])
+def test_tiled_output_is_a_relayout_of_flat(oracle, tiles):
+    """FPGA-flavour 6-D output (gemm-run-fpga.cpp:69-86) vs GPU-flavour flat output
+    (gemm-run-gpu.cpp:45-62) for the GPU constants (III,II,JJJ,JJ)=(16,4,8,2), the A10
+    constants (10,32,8,32) (gemm/const-parameters.h:23-52) and odd tile sizes."""
+    III, II, JJJ, JJ = tiles
+    M, N, K = III * II * 2, JJJ * JJ * 3, 96
+    A, B = oracle.fill_uniform((M, K), 7), oracle.fill_uniform((K, N), 8)
+    flat = t2sp_amd.gemm(A, B)
+    tiled = t2sp_amd.gemm(A, B, tiles=tiles)
+    assert (detile(tiled) == flat).all()
+    assert rel_fro(flat, oracle.gemm(A, B))[0] <= TOL
+
+
+@pytest.mark.parametrize("cfg", CFGS)
+def test_small_integers_exact(cfg):
+    """Entries in {-1,0,1,2}: exact in any order (Halide/apps/cuda_mat_mul/runner.cpp:19-35)."""
+    rng = np.random.default_rng(3)
+    A = rng.integers(-1, 3, (512, 1024)).astype(np.float32)
+    B = rng.integers(-1, 3, (1024, 384)).astype(np.float32)
+    assert (t2sp_amd.gemm(A, B, cfg=cfg) == A.astype(np.int64) @ B.astype(np.int64)).all()
+
+
+@pytest.mark.parametrize("shape", [(1, 4, 4), (33, 8, 12), (100, 36, 20), (257, 516, 40), (320, 256, 512),
+                                   (300, 200, 100), (64, 128, 8), (5, 7, 3), (130, 130, 130)])
+def test_ragged_shapes(oracle, shape):
+    """Shapes that are not tile multiples, including ones only the scalar kernel can take."""
+    M, N, K = shape
+    A, B = oracle.fill_uniform((M, K), 9), oracle.fill_uniform((K, N), 10)
+    ref = oracle.gemm(A, B)
+    for cfg in CFGS:
+        C = np.full((M, N), np.nan, np.float32)
+        t2sp_amd.gemm(A, B, out=C, cfg=cfg)
+        assert rel_fro(C, ref)[0] <= TOL, (shape, cfg)
+
+
+def test_padded_leading_dimensions(oracle):
+    M, N, K = 128, 256, 64
+    Ap, Bp, Cp = (oracle.fill_uniform(s, 11 + i) for i, s in enumerate([(M, K + 12), (K, N + 4), (M, N + 8)]))
+    A, B, C = Ap[:, :K], Bp[:, :N], Cp[:, :N]
+    keep = Cp[:, N:].copy()
+    t2sp_amd.gemm(A, B, out=C)
+    assert rel_fro(C, oracle.gemm(np.ascontiguousarray(A), np.ascontiguousarray(B)))[0] <= TOL
+    assert (Cp[:, N:] == keep).all()          # padding columns of C untouched
+
+
+def test_empty_extents():
+    C = np.full((16, 8), np.nan, np.float32)
+    t2sp_amd.gemm(np.zeros((16, 0), np.float32), np.zeros((0, 8), np.float32), out=C)
+    assert (C == 0).all()                     # empty reduction
+    t2sp_amd.gemm(np.zeros((0, 4), np.float32), np.zeros((4, 8), np.float32), out=np.zeros((0, 8), np.float32))
+
+
+@pytest.mark.parametrize("shape", [(8192, 8192, 8192), (4096, 16384, 2048), (16384, 4096, 8192)])
+def test_config2_full_size_sampled_rows_and_identity(oracle, torch_cuda, shape):
+    """BASELINE config 2 at full size, on the device.  The oracle checks 48 sampled rows;
+    the whole result is covered by a size-independent property: A @ I == A exactly."""
+    torch = torch_cuda
+    M, N, K = shape
+    A = t2sp_amd.fill_uniform(torch.empty(M, K, device="cuda"), 21)
+    B = t2sp_amd.fill_uniform(torch.empty(K, N, device="cuda"), 22)
+    C = t2sp_amd.gemm(A, B)
+    torch.cuda.synchronize()
+    rows = np.unique(np.concatenate([[0, M - 1], np.random.default_rng(0).integers(0, M, 46)]))
+    An, Bn = A[torch.as_tensor(rows, device="cuda")].cpu().numpy(), B.cpu().numpy()
+    ref = oracle.gemm(An, Bn)
+    err, mx = rel_fro(C[torch.as_tensor(rows, device="cuda")].cpu().numpy(), ref)
+    print("shape %s rel_fro %.3e max_abs %.3e" % (shape, err, mx))
+    assert err <= TOL
+    del B, C
+    if K == N:
+        eye = torch.eye(K, device="cuda")
+        assert torch.equal(t2sp_amd.gemm(A, eye), A)

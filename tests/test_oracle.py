@@ -1,0 +1,309 @@
+"""Pins of the CPU oracle (oracle/oracle.c) — CPU only.
+
+The oracle restates the reference's golden loops; before it may judge the HIP
+kernels it is itself checked here against what the reference's own tests hold
+(closed-form inputs, SEQUENTIAL/CONSTANT fixtures, exact-equality checks) and
+against what the mathematics fixes (integer-exact einsum, special cases that
+reduce one operator to another, step-by-step float32 emulation of the stated
+summation order).  None of these retypes the oracle's own loop nest.
+"""
+import numpy as np
+import pytest
+from numpy.lib.stride_tricks import as_strided
+
+from oracle import oracle as o
+
+
+def seq_f32(terms_a, terms_b):
+    """Sequential float32 accumulation acc = fl(acc + fl(a*b)) over axis 0."""
+    acc = np.zeros(terms_a.shape[1:], dtype=np.float32)
+    for t in range(terms_a.shape[0]):
+        acc = (acc + (terms_a[t] * terms_b[t]).astype(np.float32)).astype(np.float32)
+    return acc
+
+
+def ints(shape, lo, hi, seed):
+    return np.random.default_rng(seed).integers(lo, hi, size=shape).astype(np.float32)
+
+
+# ----------------------------------------------------------------------------- fill
+def test_fill_is_counter_based_and_in_range():
+    x = o.fill_uniform((1000,), 7)
+    y = o.fill_uniform((10, 100), 7)
+    assert (x == y.ravel()).all()
+    assert x.min() >= -1.0 and x.max() < 1.0
+    assert abs(float(x.mean())) < 0.1 and 0.5 < float(x.std()) < 0.65
+    assert not (o.fill_uniform((1000,), 8) == x).all()
+    # values sit on the 2^-23 grid
+    assert (np.round((x.astype(np.float64) + 1) * 2 ** 23) == (x.astype(np.float64) + 1) * 2 ** 23).all()
+
+
+def test_fill_known_answer():
+    """splitmix64 restated with Python integers."""
+    M = (1 << 64) - 1
+
+    def sm(z):
+        z = (z + 0x9E3779B97F4A7C15) & M
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & M
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & M
+        return z ^ (z >> 31)
+
+    seed = 12345
+    base = sm(seed)
+    want = np.array([np.float32((sm((base + i) & M) >> 40) / 8388608.0) - np.float32(1.0) for i in range(16)],
+                    dtype=np.float32)
+    assert (o.fill_uniform((16,), seed) == want).all()
+
+
+# ----------------------------------------------------------------------------- gemm
+def test_gemm_closed_form_kat():
+    """A[i,k]=k+i, B[k,j]=j-k (correctness/aot/gemm-run.cpp:49-59) has the closed form
+    C[i,j] = (j-i)*S1 + i*j*K - S2; exact in float32 at this K."""
+    M, N, K = 48, 40, 64
+    i, j, k = np.arange(M), np.arange(N), np.arange(K)
+    A = (k[None, :] + i[:, None]).astype(np.float32)
+    B = (j[None, :] - k[:, None]).astype(np.float32)
+    S1, S2 = K * (K - 1) // 2, (K - 1) * K * (2 * K - 1) // 6
+    want = (j[None, :] - i[:, None]) * S1 + i[:, None] * j[None, :] * K - S2
+    for acc in (o.ACC_F32, o.ACC_F32_FMA, o.ACC_F64):
+        assert (o.gemm(A, B, acc=acc) == want.astype(np.float32)).all()
+    assert (o.gemm_literal(A, B) == want.astype(np.float32)).all()
+
+
+def test_gemm_sequential_fixture_exact():
+    """SEQUENTIAL fixture b(i,j)=i+j+1 (correctness/util/util.h:52-64) at the I=J=64, K=256 of
+    correctness/gemm/gemm.cpp:140-159, product c(i,j)=sum_k a(k,i)*b(k,j) (util.h:415-426).
+    Every partial sum stays below 2^24, which is why the reference can assert == there."""
+    I, J, K = 64, 64, 256
+    a = (np.arange(K)[None, :] + np.arange(I)[:, None] + 1).astype(np.float32)  # a(k,i) as [i][k]
+    b = (np.arange(K)[:, None] + np.arange(J)[None, :] + 1).astype(np.float32)  # b(k,j) as [k][j]
+    want = a.astype(np.int64) @ b.astype(np.int64)
+    assert want.max() < 2 ** 24
+    for acc in (o.ACC_F32, o.ACC_F32_FMA):
+        assert (o.gemm(a, b, acc=acc) == want).all()
+    assert (o.gemm_literal(a, b) == want).all()
+
+
+def test_gemm_small_integers_exact():
+    """Entries in {-1,0,1,2}: every partial sum is an exact integer, so any order gives the
+    same float32 result (the check of Halide/apps/cuda_mat_mul/runner.cpp:19-35)."""
+    A, B = ints((96, 256), -1, 3, 0), ints((256, 80), -1, 3, 1)
+    want = A.astype(np.int64) @ B.astype(np.int64)
+    for acc in (o.ACC_F32, o.ACC_F32_FMA, o.ACC_F64):
+        assert (o.gemm(A, B, acc=acc) == want).all()
+
+
+def test_gemm_random_order_and_fma():
+    A, B = o.fill_uniform((40, 300), 1), o.fill_uniform((300, 24), 2)
+    want = seq_f32(A.T[:, :, None] * np.ones((1, 1, 24), np.float32), B[:, None, :] * np.ones((1, 40, 1), np.float32))
+    got = o.gemm(A, B)
+    assert (got == want).all()                      # ascending-k, separate multiply and add
+    assert (o.gemm_literal(A, B) == want).all()
+    exact = A.astype(np.float64) @ B.astype(np.float64)
+    fma = o.gemm(A, B, acc=o.ACC_F32_FMA)
+    assert (fma != got).any()                       # a distinct arithmetic
+    assert np.abs(fma - exact).max() < 2e-5 and np.abs(got - exact).max() < 2e-5
+    assert np.abs(o.gemm(A, B, acc=o.ACC_F64) - exact).max() < 1e-6
+
+
+def test_gemm_strides_rows_identity_transpose():
+    A, B = ints((32, 48), -3, 4, 3), ints((48, 20), -3, 4, 4)
+    C = o.gemm(A, B)
+    assert (o.gemm(B.T.copy().T, np.eye(20, dtype=np.float32)) == B).all()
+    assert (o.gemm(B.T, A.T) == C.T).all()          # transposed strided views
+    part = o.gemm(A, B, rows=(8, 5))
+    assert (part == C[8:13]).all()
+    for threads in (1, 3):
+        assert (o.gemm(A, B, threads=threads) == C).all()
+
+
+# ----------------------------------------------------------------------------- conv
+def conv_terms(I, W, order, cii=1, stride=(1, 1)):
+    """Terms of every output in the stated reduction order, for the emulation."""
+    N, CI, IY, IX = I.shape
+    CO, _, KY, KX = W.shape
+    sy, sx = stride
+    OY, OX = (IY - KY) // sy + 1, (IX - KX) // sx + 1
+    ta, tb = [], []
+    if order == o.ORDER_GOLDEN:
+        seq = [(ci, ky, kx) for ci in range(CI) for kx in range(KX) for ky in range(KY)]
+    else:
+        seq = [(cii_ + cii * cio, ky, kx) for cio in range(CI // cii) for kx in range(KX)
+               for ky in range(KY) for cii_ in range(cii)]
+    for ci, ky, kx in seq:
+        patch = I[:, ci, ky:ky + sy * OY:sy, kx:kx + sx * OX:sx]          # n,y,x
+        ta.append(np.broadcast_to(patch[:, None], (N, CO, OY, OX)))
+        tb.append(np.broadcast_to(W[None, :, ci, ky, kx, None, None], (N, CO, OY, OX)))
+    return np.stack(ta), np.stack(tb)
+
+
+def test_conv_integer_exact_and_constants():
+    I, W = ints((2, 6, 9, 8), -2, 3, 5), ints((4, 6, 3, 3), -2, 3, 6)
+    win = np.lib.stride_tricks.sliding_window_view(I.astype(np.int64), (3, 3), axis=(2, 3))  # n,ci,y,x,ky,kx
+    want = np.einsum("niyxpq,oipq->noyx", win, W.astype(np.int64))
+    for order in (o.ORDER_GOLDEN, o.ORDER_URE):
+        for acc in (o.ACC_F32, o.ACC_F32_FMA, o.ACC_F64):
+            assert (o.conv(I, W, order=order, cii=2, acc=acc) == want).all()
+    ones = o.conv(np.ones((1, 5, 6, 6), np.float32), np.ones((3, 5, 3, 3), np.float32))
+    assert (ones == 5 * 9).all()
+    delta = np.zeros((1, 1, 3, 3), np.float32)
+    delta[0, 0, 2, 1] = 1.0                                                  # ky=2, kx=1
+    X = o.fill_uniform((2, 1, 8, 7), 3)
+    assert (o.conv(X, delta) == X[:, :, 2:8, 1:6]).all()
+
+
+def test_conv_orders_match_stepwise_float32():
+    I, W = o.fill_uniform((1, 8, 6, 6), 10), o.fill_uniform((3, 8, 3, 3), 11)
+    g = o.conv(I, W, order=o.ORDER_GOLDEN)
+    u = o.conv(I, W, order=o.ORDER_URE, cii=4)
+    assert (g == seq_f32(*conv_terms(I, W, o.ORDER_GOLDEN))).all()
+    assert (u == seq_f32(*conv_terms(I, W, o.ORDER_URE, cii=4))).all()
+    assert (g != u).any()
+    exact = np.einsum("niyxpq,oipq->noyx",
+                      np.lib.stride_tricks.sliding_window_view(I.astype(np.float64), (3, 3), axis=(2, 3)), W.astype(np.float64))
+    assert np.abs(g - exact).max() < 1e-5 and np.abs(o.conv(I, W, acc=o.ACC_F64) - exact).max() < 1e-6
+
+
+def test_conv_1x1_is_gemm_and_stride():
+    I, W = o.fill_uniform((2, 16, 5, 4), 12), o.fill_uniform((6, 16, 1, 1), 13)
+    got = o.conv(I, W)
+    as_gemm = o.gemm(W[:, :, 0, 0], I.transpose(1, 0, 2, 3).reshape(16, -1)).reshape(6, 2, 5, 4).transpose(1, 0, 2, 3)
+    assert (got == as_gemm).all()
+    X, K = ints((1, 2, 9, 9), -2, 3, 14), ints((2, 2, 3, 3), -2, 3, 15)
+    assert (o.conv(X, K, stride=(2, 2)) == o.conv(X, K)[:, :, ::2, ::2]).all()
+
+
+def test_conv_reference_packed_layout_views():
+    """The 2-D packed buffers of conv-run-fpga.cpp:49-69 (I: [ix][iy][n][ci], K: [ky][ci][kx][co])
+    viewed through strides give the same result as dense arrays; partial n/co ranges too."""
+    N, CI, CO, IY, IX = 2, 4, 3, 6, 5
+    I, W = ints((N, CI, IY, IX), -2, 3, 16), ints((CO, CI, 3, 3), -2, 3, 17)
+    want = o.conv(I, W)
+    Ip = np.ascontiguousarray(I.transpose(3, 2, 0, 1))           # [ix][iy][n][ci]
+    Wp = np.ascontiguousarray(W.transpose(2, 1, 3, 0))           # [ky][ci][kx][co]
+    Iv = Ip.transpose(2, 3, 1, 0)                                # logical (n,ci,y,x)
+    Wv = Wp.transpose(3, 1, 0, 2)                                # logical (co,ci,ky,kx)
+    assert (o.conv(Iv, Wv) == want).all()
+    part = o.conv(I, W, n_range=(1, 2), co_range=(1, 3))
+    assert (part[1, 1:3] == want[1, 1:3]).all() and (part[0] == 0).all()
+
+
+# ----------------------------------------------------------------------------- capsule
+def test_capsule_constant_fixture():
+    """CONSTANT(=1) inputs: every vote is CI*KX*KY*MK (correctness/multi-projection/capsule.cpp:75-102)."""
+    N, CI, CO = 1, 32, 2
+    P = np.ones((N, CI, 7, 7, 4, 4), np.float32)
+    W = np.ones((CO, CI, 3, 3, 4, 4), np.float32)
+    for order in (o.ORDER_GOLDEN, o.ORDER_URE):
+        V = o.capsule(P, W, stride=2, order=order, cii=4)
+        assert V.shape == (N, CO, 3, 3, 4, 4) and (V == 32 * 9 * 4).all()
+
+
+def capsule_exact(P, W, stride, dtype):
+    win = np.lib.stride_tricks.sliding_window_view(P.astype(dtype), (W.shape[2], W.shape[3]), axis=(2, 3))
+    win = win[:, :, ::stride, ::stride]                          # n,ci,y,x,mx,mk,ky,kx
+    return np.einsum("niyxakpq,oipqkb->noyxab", win, W.astype(dtype))
+
+
+def test_capsule_integer_exact_and_fp64():
+    P, W = ints((2, 3, 7, 5, 4, 4), -2, 3, 20), ints((5, 3, 3, 3, 4, 4), -2, 3, 21)
+    want = capsule_exact(P, W, 2, np.int64)
+    for order in (o.ORDER_GOLDEN, o.ORDER_URE):
+        for acc in (o.ACC_F32, o.ACC_F32_FMA, o.ACC_F64):
+            assert (o.capsule(P, W, stride=2, order=order, cii=3, acc=acc) == want).all()
+    Pr, Wr = o.fill_uniform(P.shape, 22), o.fill_uniform(W.shape, 23)
+    exact = capsule_exact(Pr, Wr, 2, np.float64)
+    assert np.abs(o.capsule(Pr, Wr) - exact).max() < 1e-5
+    assert np.abs(o.capsule(Pr, Wr, acc=o.ACC_F64) - exact).max() < 1e-6
+
+
+def test_capsule_orders_match_stepwise_float32():
+    P, W = o.fill_uniform((1, 4, 5, 5, 2, 3), 24), o.fill_uniform((2, 4, 3, 3, 3, 2), 25)
+    N, CI, _, _, MX, MK = P.shape
+    CO, MY = W.shape[0], W.shape[5]
+
+    def terms(seq):
+        ta, tb = [], []
+        for ci, ky, kx, mk in seq:
+            p = P[:, ci, ky:ky + 3:2, kx:kx + 3:2, :, mk]                        # n,y,x,mx
+            ta.append(np.broadcast_to(p[:, None, :, :, :, None], (N, CO, 2, 2, MX, MY)))
+            tb.append(np.broadcast_to(W[None, :, ci, ky, kx, mk, None, None, None, :], (N, CO, 2, 2, MX, MY)))
+        return np.stack(ta), np.stack(tb)
+
+    golden = [(ci, ky, kx, mk) for kx in range(3) for ky in range(3) for mk in range(MK) for ci in range(CI)]
+    ure = [(cii + 2 * cio, ky, kx, mk) for mk in range(MK) for cio in range(CI // 2) for kx in range(3)
+           for ky in range(3) for cii in range(2)]
+    g, u = o.capsule(P, W), o.capsule(P, W, order=o.ORDER_URE, cii=2)
+    assert (g == seq_f32(*terms(golden))).all()
+    assert (u == seq_f32(*terms(ure))).all()
+    assert (g != u).any()
+
+
+def test_capsule_scalar_poses_is_strided_conv():
+    P, W = ints((2, 5, 9, 7, 1, 1), -2, 3, 26), ints((3, 5, 3, 3, 1, 1), -2, 3, 27)
+    V = o.capsule(P, W, stride=2)
+    C = o.conv(P[..., 0, 0], W[..., 0, 0], stride=(2, 2))
+    assert (V[..., 0, 0] == C).all()
+
+
+def test_capsule_reference_layout_views():
+    """oneAPI-flavour dense layouts P(MK,MX,CI,IY,IX,N), W(MY,MK,CI,CO,KY,KX)
+    (oneapi/src/oneapi-target-6-run.cpp:52-99) through strided views."""
+    P, W = ints((2, 3, 5, 5, 4, 4), -2, 3, 28), ints((4, 3, 3, 3, 4, 4), -2, 3, 29)
+    want = o.capsule(P, W)
+    Pm = np.ascontiguousarray(P.transpose(0, 3, 2, 1, 4, 5))     # [n][ix][iy][ci][mx][mk]
+    Wm = np.ascontiguousarray(W.transpose(3, 2, 0, 1, 4, 5))     # [kx][ky][co][ci][mk][my]
+    assert (o.capsule(Pm.transpose(0, 3, 2, 1, 4, 5), Wm.transpose(2, 3, 1, 0, 4, 5)) == want).all()
+
+
+# ----------------------------------------------------------------------------- mttkrp
+def mttkrp_bruteforce(a, b, c, L, I, J, K):
+    """util.h:498-515 restated with Python loops over reference-indexed accessors."""
+    A = lambda l, i, k: a[k, i, l]
+    Cc = lambda l, j: c[j, l]
+    Bb = lambda k, j: b[j, k]
+    d = np.zeros((J, I), np.float32)
+    for i in range(I):
+        for j in range(J):
+            dij = np.float32(0)
+            for k in range(K):
+                e = np.float32(0)
+                for l in range(L):
+                    e = np.float32(e + np.float32(A(l, i, k) * Cc(l, j)))
+                dij = np.float32(dij + np.float32(e * Bb(k, j)))
+            d[j, i] = dij
+    return d
+
+
+def test_mttkrp_bruteforce_and_literal():
+    L, I, J, K = 5, 4, 3, 6                                       # reference's template names
+    a, c, b = o.fill_uniform((K, I, L), 30), o.fill_uniform((J, L), 31), o.fill_uniform((J, K), 32)
+    want = mttkrp_bruteforce(a, b, c, L, I, J, K)
+    assert (o.mttkrp_literal(a, b, c) == want).all()
+    # same data through the strided entry: B[i,j,k] = a(l=j, i, k), C[j,r] = c(l=j, r), D[k,r] = b(k, r)
+    got = o.mttkrp(a.transpose(1, 2, 0), c.T, b.T)
+    assert (got == want.T).all()
+    assert (o.mttkrp(a.transpose(1, 2, 0), c.T, b.T, i_range=(1, 3))[1:3] == want.T[1:3]).all()
+
+
+def test_mttkrp_closed_forms():
+    I, J, K, R = 6, 7, 5, 4
+    ones = o.mttkrp(np.ones((I, J, K), np.float32), np.ones((J, R), np.float32), np.ones((K, R), np.float32))
+    assert (ones == J * K).all()
+    u, v, w = ints((I,), -3, 4, 33), ints((J,), -3, 4, 34), ints((K,), -3, 4, 35)
+    C, D = ints((J, R), -3, 4, 36), ints((K, R), -3, 4, 37)
+    B = np.einsum("i,j,k->ijk", u, v, w).astype(np.float32)
+    want = u[:, None].astype(np.int64) * (v.astype(np.int64) @ C.astype(np.int64))[None, :] * (w.astype(np.int64) @ D.astype(np.int64))[None, :]
+    for acc in (o.ACC_F32, o.ACC_F32_FMA, o.ACC_F64):
+        assert (o.mttkrp(B, C, D, acc=acc) == want).all()
+    Br, Cr, Dr = o.fill_uniform((I, J, K), 38), o.fill_uniform((J, R), 39), o.fill_uniform((K, R), 40)
+    exact = np.einsum("ijk,jr,kr->ir", Br.astype(np.float64), Cr.astype(np.float64), Dr.astype(np.float64))
+    assert np.abs(o.mttkrp(Br, Cr, Dr) - exact).max() < 1e-5
+    assert np.abs(o.mttkrp(Br, Cr, Dr, acc=o.ACC_F64) - exact).max() < 1e-6
+
+
+def test_mttkrp_single_k_is_gemm():
+    I, J, R = 9, 33, 5
+    B, C = o.fill_uniform((I, J, 1), 41), o.fill_uniform((J, R), 42)
+    got = o.mttkrp(B, C, np.ones((1, R), np.float32))
+    assert (got == o.gemm(B[:, :, 0], C)).all()
