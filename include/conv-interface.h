@@ -1,0 +1,35 @@
+/* conv-interface.h — host interface of the 2-D convolution pipeline.
+ *
+ * Same name and signature as the header the reference generates with
+ * compile_to_host("conv-interface", {I, K}, "conv", ...)
+ * (t2s/tests/performance/conv/conv.cpp:99-101), called as conv(i, k, o) in
+ * conv-run-fpga.cpp:69.  Returns 0 or a negative halide_error_code_t.
+ */
+#ifndef T2SP_CONV_INTERFACE_H
+#define T2SP_CONV_INTERFACE_H
+#include "t2sp_buffer.h"
+#include "t2sp_runtime.h"
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* O[n,co,y,x] = sum_{ci,kx,ky} I[n,ci,y+ky,x+kx] * K[co,ci,ky,kx]  (stride 1, no padding).
+ * Argument forms (dimension 0 first):
+ *   I(IY, IX, CI, N), K(KY, KX, CI, CO)   4-D, as in oneapi/src/oneapi-target-5-run.cpp:100-106;
+ *                                         dense buffers are NCHW / OIHW memory with y as "W"
+ *   I(CI*N, IY*IX),   K(CO*KX, CI*KY)     packed 2-D, as in conv-run-fpga.cpp:49-66
+ *   O(OY, OX, CO, N)                      4-D, or
+ *   O(COOO, YYY, XXX, COO, YY, XX, Y, X, CO, N)  the 10-D tiled output of conv-run-fpga.cpp:68
+ * Packed inputs need the 10-D output (N, CO and the image size are read from it).
+ * Device-resident buffers: see gemm-interface.h. */
+int conv(struct halide_buffer_t *I, struct halide_buffer_t *K, struct halide_buffer_t *O);
+
+/* conv() with a forced tile configuration (T2SP_CFG_* of t2sp_hip.h); no counterpart in
+ * the reference. */
+int t2sp_conv_with_cfg(struct halide_buffer_t *I, struct halide_buffer_t *K,
+                       struct halide_buffer_t *O, int cfg);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -27,7 +27,7 @@ int gemm(struct halide_buffer_t *A, struct halide_buffer_t *B, struct halide_buf
  * (t2s/tests/correctness/aot/gemm-generate.cpp:176, gemm-run.cpp:62). */
 int GEMM(struct halide_buffer_t *A, struct halide_buffer_t *B, struct halide_buffer_t *C);
 
-/* gemm() with a forced tile configuration (T2SP_GEMM_CFG_* of t2sp_hip.h);
+/* gemm() with a forced tile configuration (T2SP_CFG_* of t2sp_hip.h);
  * for benchmarks and tests, no counterpart in the reference. */
 int t2sp_gemm_with_cfg(struct halide_buffer_t *A, struct halide_buffer_t *B,
                        struct halide_buffer_t *C, int cfg);

@@ -24,12 +24,14 @@ extern "C" {
 #define T2SP_ERR_SHAPE (-8)   /* halide_error_code_constraint_violated */
 #define T2SP_ERR_LAUNCH (-23) /* halide_error_code_device_run_failed   */
 
-/* Tile configurations of the SGEMM kernel (cfg argument). */
-#define T2SP_GEMM_CFG_AUTO 0
-#define T2SP_GEMM_CFG_256x256 1
-#define T2SP_GEMM_CFG_128x128 2
-#define T2SP_GEMM_CFG_64x128 3
-#define T2SP_GEMM_CFG_SCALAR 99
+/* Tile configurations of the MFMA kernels (cfg argument of every operator). */
+#define T2SP_CFG_AUTO 0
+#define T2SP_CFG_256x256 1
+#define T2SP_CFG_128x128 2
+#define T2SP_CFG_64x128 3
+#define T2SP_CFG_SCALAR 99
+
+#define T2SP_MAX_DIMS 10
 
 /* C[i,j] = sum_k A[i,k] * B[k,j], fp32, row-major with leading dimensions in
  * elements.  Replaces the device side of the reference's SGEMM pipeline: the
@@ -46,6 +48,24 @@ int t2sp_sgemm_f32(const float *A, const float *B, float *C, int M, int N, int K
 int t2sp_sgemm_f32_tiled(const float *A, const float *B, float *C, int M, int N, int K,
                          int64_t lda, int64_t ldb, int jjj, int iii, int jj, int ii,
                          const int64_t *strides6, int cfg, void *stream);
+
+/* O[n,co,h,w] = sum_{ci,kh,kw} I[n,ci,h+kh,w+kw] * W[co,ci,kh,kw], stride 1, valid
+ * padding, fp32.  si4/sw4/so4 are element strides of the logical indices
+ * (n,ci,h,w), (co,ci,kh,kw), (n,co,h,w); "w" is the innermost spatial axis (the
+ * one the reference calls y).  Dense NCHW/OIHW with OW % 4 == 0 takes the
+ * implicit-GEMM MFMA kernel, anything else a scalar kernel.  Replaces the device
+ * side of the reference's conv pipeline (t2s/tests/performance/conv/conv.cpp:59-65,
+ * conv/bitstream/a10/a.cl). */
+int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, int CI, int CO, int OH,
+                    int OW, int KH, int KW, const int64_t *si4, const int64_t *sw4,
+                    const int64_t *so4, int cfg, void *stream);
+
+/* dst[sum_d c_d*dst_strides[d]] = src[sum_d c_d*src_strides[d]] for every coordinate c of the
+ * box `extents` (nd <= T2SP_MAX_DIMS, dimension 0 fastest).  Device-side replacement of the
+ * host serializer/deserializer loops the reference's generated interface runs around its
+ * pipeline (t2s/src/Stensor.cpp:228-249,270-279). */
+int t2sp_relayout_f32(const float *src, float *dst, int nd, const int *extents,
+                      const int64_t *src_strides, const int64_t *dst_strides, void *stream);
 
 /* x[i] = u(seed, i), i in [0,n): the seeded uniform[-1,1) generator shared with
  * the CPU checker (same bits for the same seed and index).  The reference's

@@ -40,6 +40,11 @@ def _declare(L):
     L.t2sp_sgemm_f32.argtypes = [vp, vp, vp, i32, i32, i32, i64, i64, i64, i32, vp]
     L.t2sp_sgemm_f32_tiled.argtypes = [vp, vp, vp, i32, i32, i32, i64, i64, i32, i32, i32, i32,
                                        ctypes.POINTER(i64), i32, vp]
+    L.conv.argtypes = [bp, bp, bp]
+    L.t2sp_conv_with_cfg.argtypes = [bp, bp, bp, i32]
+    p64, p32 = ctypes.POINTER(i64), ctypes.POINTER(i32)
+    L.t2sp_conv2d_f32.argtypes = [vp, vp, vp] + [i32] * 7 + [p64, p64, p64, i32, vp]
+    L.t2sp_relayout_f32.argtypes = [vp, vp, i32, p32, p64, p64, vp]
     L.t2sp_fill_uniform_f32.argtypes = [vp, i64, ctypes.c_uint64, vp]
     L.t2sp_last_kernel_ns.restype = ctypes.c_double
     L.t2sp_release.restype = None

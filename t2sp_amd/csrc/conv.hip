@@ -1,0 +1,179 @@
+// conv.hip — 2-D convolution as an implicit GEMM on fp32 MFMA tiles.
+//
+//   O[n,co,h,w] = sum_{ci,kh,kw} I[n,ci,h+kh,w+kw] * W[co,ci,kh,kw]     (stride 1, valid padding)
+//
+// Replaces the reference's conv device pipeline (t2s/tests/performance/conv/conv.cpp:59-65 as
+// compiled to conv/bitstream/a10/a.cl).  GEMM view: D[co][p] with p = (n,h,w) flattened, w
+// fastest; reduction index k = (ci,kh,kw), the memory order of the weights.
+//   * weights  -> KC tile ([co][k], k contiguous): plain rows of the CO x (CI*KH*KW) matrix
+//   * input    -> RC tile ([k][p], p contiguous): im2col formed on the fly; a thread loads 4
+//                 consecutive w of one (n,ci,h+kh) row, 4-byte aligned (kw shifts the start)
+//   * output   -> a lane ends up with 4 consecutive w of one (n,co,h) row: 128-bit stores
+// "w" is the innermost spatial axis of the buffers (the one the reference calls y).
+#include "mfma_core.hpp"
+#include "gemm_loaders.hpp"
+#include "t2sp_hip.h"
+
+namespace t2sp {
+
+typedef float v4f_u __attribute__((ext_vector_type(4), aligned(4)));
+
+struct ConvArgs {
+    const float *I, *W;
+    float *O;
+    int N, CI, CO, OH, OW, KH, KW;
+    int64_t si_n, si_c, si_h;   // input strides (w stride is 1)
+    int64_t sw_o;               // weight stride of co (ci,kh,kw are dense)
+    int64_t so_n, so_c, so_h;   // output strides (w stride is 1)
+    int P, KRED;                // N*OH*OW, CI*KH*KW
+    int tiles_m, tiles_n, group_m;
+};
+
+// Input operand: for reduction row k = (ci,kh,kw) and 4 consecutive output pixels of one image
+// row, the 4 input pixels at (ci, h+kh, w+kw .. w+kw+3).
+template <class Cfg, bool EDGE>
+struct Im2colRcLoader {
+    const float *base[Cfg::B_VEC];   // pixel part of the address (n, h, w), fixed for the block
+    bool col_ok[Cfg::B_VEC];
+    int k[Cfg::B_VEC];               // reduction row this slot loads next
+    v4f reg[Cfg::B_VEC];
+    const ConvArgs &g;
+    __device__ Im2colRcLoader(const ConvArgs &g_, int p0) : g(g_) {
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
+            int p = p0 + s.col;
+            col_ok[i] = !EDGE || p < g.P;
+            if (!col_ok[i]) p = 0;
+            const int hw = g.OH * g.OW;
+            const int n = p / hw, rem = p - n * hw;
+            const int h = rem / g.OW, w = rem - h * g.OW;
+            base[i] = g.I + n * g.si_n + h * g.si_h + w;
+            k[i] = s.k;
+        }
+    }
+    __device__ __forceinline__ void fetch() {
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            const int khw = g.KH * g.KW;
+            const int ci = k[i] / khw, r = k[i] - ci * khw;
+            const int kh = r / g.KW, kw = r - kh * g.KW;
+            if (!EDGE || (col_ok[i] && k[i] < g.KRED))
+                reg[i] = *reinterpret_cast<const v4f_u *>(base[i] + ci * g.si_c + kh * g.si_h + kw);
+            else
+                reg[i] = v4f{0.f, 0.f, 0.f, 0.f};
+            k[i] += Cfg::BK;
+        }
+    }
+    __device__ __forceinline__ void commit(float *stage) const {
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
+            *reinterpret_cast<v4f *>(stage + s.k * Cfg::LDB + s.col) = reg[i];
+        }
+    }
+};
+
+template <class Cfg, bool EDGE>
+__global__ void __launch_bounds__(Cfg::NTHREADS) conv_kernel(const ConvArgs g) {
+    extern __shared__ __align__(16) float smem[];
+    int tm, tn;
+    tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, g.group_m, tm, tn);
+    const int co0 = tm * Cfg::BM, p0 = tn * Cfg::BN;
+    RowMajorKcLoader<Cfg, EDGE> la(g.W, g.sw_o, co0, g.CO, g.KRED);
+    Im2colRcLoader<Cfg, EDGE> lb(g, p0);
+    Accum<Cfg> acc;
+    mainloop<Cfg>(acc, la, lb, (g.KRED + Cfg::BK - 1) / Cfg::BK, smem);
+    const int hw = g.OH * g.OW;
+    drain<Cfg>(acc, [&](int row, int col, v4f v) {
+        const int co = co0 + row, p = p0 + col;
+        if (EDGE && (co >= g.CO || p >= g.P)) return;
+        const int n = p / hw, rem = p - n * hw;
+        const int h = rem / g.OW, w = rem - h * g.OW;
+        *reinterpret_cast<v4f *>(g.O + n * g.so_n + co * g.so_c + h * g.so_h + w) = v;
+    });
+}
+
+// Any strides, any sizes: one thread per output, reduction in (ci,kh,kw) order.
+struct ConvGenericArgs {
+    const float *I, *W;
+    float *O;
+    int N, CI, CO, OH, OW, KH, KW;
+    int64_t si[4], sw[4], so[4];   // (n,c,h,w), (co,ci,kh,kw), (n,co,h,w)
+};
+__global__ void conv_scalar_kernel(const ConvGenericArgs g) {
+    const int64_t total = (int64_t)g.N * g.CO * g.OH * g.OW;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total;
+         t += (int64_t)gridDim.x * blockDim.x) {
+        const int w = t % g.OW, h = (t / g.OW) % g.OH, co = (t / ((int64_t)g.OW * g.OH)) % g.CO;
+        const int n = t / ((int64_t)g.OW * g.OH * g.CO);
+        float acc = 0.f;
+        for (int ci = 0; ci < g.CI; ci++)
+            for (int kh = 0; kh < g.KH; kh++)
+                for (int kw = 0; kw < g.KW; kw++)
+                    acc = fmaf(g.I[n * g.si[0] + ci * g.si[1] + (h + kh) * g.si[2] + (w + kw) * g.si[3]],
+                               g.W[co * g.sw[0] + ci * g.sw[1] + kh * g.sw[2] + kw * g.sw[3]], acc);
+        g.O[n * g.so[0] + co * g.so[1] + h * g.so[2] + w * g.so[3]] = acc;
+    }
+}
+
+template <class Cfg>
+static int launch_conv(ConvArgs g, hipStream_t stream) {
+    g.tiles_m = (g.CO + Cfg::BM - 1) / Cfg::BM;
+    g.tiles_n = (g.P + Cfg::BN - 1) / Cfg::BN;
+    g.group_m = g.tiles_m;   // all output channels of a pixel tile run together: the input tile is shared in L2
+    const bool edge = (g.CO % Cfg::BM) || (g.P % Cfg::BN) || (g.KRED % Cfg::BK);
+    const size_t smem = Cfg::SMEM_FLOATS * sizeof(float);
+    auto kern = edge ? conv_kernel<Cfg, true> : conv_kernel<Cfg, false>;
+    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)smem) != hipSuccess)
+        return T2SP_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(Cfg::NTHREADS), smem, stream, g);
+    return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+}
+
+using ConvL = TileCfg<256, 256, 16, 4, 2, STYLE_RC>;
+using ConvM = TileCfg<128, 128, 16, 4, 1, STYLE_RC>;
+using ConvS = TileCfg<64, 128, 16, 2, 1, STYLE_RC>;
+
+}  // namespace t2sp
+
+extern "C" int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, int CI, int CO,
+                               int OH, int OW, int KH, int KW, const int64_t *si4,
+                               const int64_t *sw4, const int64_t *so4, int cfg, void *stream) {
+    using namespace t2sp;
+    if (N <= 0 || CI <= 0 || CO <= 0 || OH <= 0 || OW <= 0 || KH <= 0 || KW <= 0 || !si4 || !sw4 || !so4)
+        return T2SP_ERR_SHAPE;
+    if ((int64_t)N * OH * OW > INT32_MAX || (int64_t)CI * KH * KW > INT32_MAX) return T2SP_ERR_SHAPE;
+    const bool fast = cfg != T2SP_CFG_SCALAR && si4[3] == 1 && so4[3] == 1 && sw4[3] == 1 &&
+                      sw4[2] == KW && sw4[1] == (int64_t)KH * KW && sw4[0] % 4 == 0 && OW % 4 == 0 &&
+                      (CI * KH * KW) % 4 == 0 && so4[0] % 4 == 0 && so4[1] % 4 == 0 && so4[2] % 4 == 0 &&
+                      ((uintptr_t)W % 16 == 0) && ((uintptr_t)O % 16 == 0) && ((uintptr_t)I % 4 == 0);
+    if (!fast) {
+        ConvGenericArgs a{I, W, O, N, CI, CO, OH, OW, KH, KW, {}, {}, {}};
+        for (int d = 0; d < 4; d++) { a.si[d] = si4[d]; a.sw[d] = sw4[d]; a.so[d] = so4[d]; }
+        const int64_t total = (int64_t)N * CO * OH * OW;
+        const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
+        hipLaunchKernelGGL(conv_scalar_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+        return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+    }
+    ConvArgs g{};
+    g.I = I; g.W = W; g.O = O;
+    g.N = N; g.CI = CI; g.CO = CO; g.OH = OH; g.OW = OW; g.KH = KH; g.KW = KW;
+    g.si_n = si4[0]; g.si_c = si4[1]; g.si_h = si4[2];
+    g.sw_o = sw4[0];
+    g.so_n = so4[0]; g.so_c = so4[1]; g.so_h = so4[2];
+    g.P = N * OH * OW; g.KRED = CI * KH * KW;
+    if (cfg == T2SP_CFG_AUTO) {
+        auto tiles = [&](int bm, int bn) { return (int64_t)((CO + bm - 1) / bm) * ((g.P + bn - 1) / bn); };
+        if (tiles(256, 256) >= 200) cfg = T2SP_CFG_256x256;
+        else if (tiles(128, 128) >= 200) cfg = T2SP_CFG_128x128;
+        else cfg = T2SP_CFG_64x128;
+    }
+    switch (cfg) {
+        case T2SP_CFG_256x256: return launch_conv<ConvL>(g, (hipStream_t)stream);
+        case T2SP_CFG_128x128: return launch_conv<ConvM>(g, (hipStream_t)stream);
+        case T2SP_CFG_64x128: return launch_conv<ConvS>(g, (hipStream_t)stream);
+        default: return T2SP_ERR_SHAPE;
+    }
+}

@@ -7,85 +7,10 @@
 // row-major or the reference's 6-D tiled output
 // c(jjj, iii, jj, ii, j, i)  (gemm-run-fpga.cpp:69, gemm.cpp:39-41).
 #include "mfma_core.hpp"
+#include "gemm_loaders.hpp"
 #include "t2sp_hip.h"
 
 namespace t2sp {
-
-// A operand: rows of a row-major matrix, k contiguous.
-template <class Cfg, bool EDGE>
-struct RowMajorKcLoader {
-    const float *p[Cfg::A_VEC];
-    bool row_ok[Cfg::A_VEC];
-    int kpos[Cfg::A_VEC];
-    v4f reg[Cfg::A_VEC];
-    int K;
-    __device__ RowMajorKcLoader(const float *A, int64_t lda, int m0, int M, int K_) : K(K_) {
-#pragma unroll
-        for (int i = 0; i < Cfg::A_VEC; i++) {
-            KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
-            row_ok[i] = !EDGE || (m0 + s.row < M);
-            kpos[i] = s.k;
-            p[i] = A + (int64_t)(m0 + (row_ok[i] ? s.row : 0)) * lda + s.k;
-        }
-    }
-    __device__ __forceinline__ void fetch() {
-#pragma unroll
-        for (int i = 0; i < Cfg::A_VEC; i++) {
-            if (!EDGE || (row_ok[i] && kpos[i] < K))
-                reg[i] = *reinterpret_cast<const v4f *>(p[i]);
-            else
-                reg[i] = v4f{0.f, 0.f, 0.f, 0.f};
-            p[i] += Cfg::BK;
-            kpos[i] += Cfg::BK;
-        }
-    }
-    __device__ __forceinline__ void commit(float *stage) const {
-#pragma unroll
-        for (int i = 0; i < Cfg::A_VEC; i++) {
-            KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
-            *reinterpret_cast<v4f *>(stage + s.row * Cfg::LDA + s.k) = reg[i];
-        }
-    }
-};
-
-// B operand: k-rows of a row-major matrix, columns contiguous.
-template <class Cfg, bool EDGE>
-struct RowMajorRcLoader {
-    const float *p[Cfg::B_VEC];
-    bool col_ok[Cfg::B_VEC];
-    int kpos[Cfg::B_VEC];
-    v4f reg[Cfg::B_VEC];
-    int64_t step;
-    int K;
-    __device__ RowMajorRcLoader(const float *B, int64_t ldb, int n0, int N, int K_)
-        : step((int64_t)Cfg::BK * ldb), K(K_) {
-#pragma unroll
-        for (int i = 0; i < Cfg::B_VEC; i++) {
-            RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
-            col_ok[i] = !EDGE || (n0 + s.col < N);
-            kpos[i] = s.k;
-            p[i] = B + (int64_t)s.k * ldb + n0 + (col_ok[i] ? s.col : 0);
-        }
-    }
-    __device__ __forceinline__ void fetch() {
-#pragma unroll
-        for (int i = 0; i < Cfg::B_VEC; i++) {
-            if (!EDGE || (col_ok[i] && kpos[i] < K))
-                reg[i] = *reinterpret_cast<const v4f *>(p[i]);
-            else
-                reg[i] = v4f{0.f, 0.f, 0.f, 0.f};
-            p[i] += step;
-            kpos[i] += Cfg::BK;
-        }
-    }
-    __device__ __forceinline__ void commit(float *stage) const {
-#pragma unroll
-        for (int i = 0; i < Cfg::B_VEC; i++) {
-            RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
-            *reinterpret_cast<v4f *>(stage + s.k * Cfg::LDB + s.col) = reg[i];
-        }
-    }
-};
 
 struct GemmArgs {
     const float *A, *B;
@@ -170,22 +95,22 @@ static int dispatch(GemmArgs g, int cfg, hipStream_t stream) {
     const bool vec_ok = g.K % 4 == 0 && g.N % 4 == 0 && g.lda % 4 == 0 && g.ldb % 4 == 0 &&
                         ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
                         ((uintptr_t)g.C % 16 == 0) && (g.tiled || g.ldc % 4 == 0);
-    if (cfg == T2SP_GEMM_CFG_SCALAR || !vec_ok) {
+    if (cfg == T2SP_CFG_SCALAR || !vec_ok) {
         hipLaunchKernelGGL(sgemm_scalar_kernel, dim3((g.N + 255) / 256, g.M), dim3(256), 0, stream, g);
         return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
     }
-    if (cfg == T2SP_GEMM_CFG_AUTO) {
+    if (cfg == T2SP_CFG_AUTO) {
         auto tiles = [&](int bm, int bn) {
             return (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
         };
-        if (tiles(256, 256) >= 200) cfg = T2SP_GEMM_CFG_256x256;
-        else if (tiles(128, 128) >= 200) cfg = T2SP_GEMM_CFG_128x128;
-        else cfg = T2SP_GEMM_CFG_64x128;
+        if (tiles(256, 256) >= 200) cfg = T2SP_CFG_256x256;
+        else if (tiles(128, 128) >= 200) cfg = T2SP_CFG_128x128;
+        else cfg = T2SP_CFG_64x128;
     }
     switch (cfg) {
-        case T2SP_GEMM_CFG_256x256: return launch<GemmL>(g, stream);
-        case T2SP_GEMM_CFG_128x128: return launch<GemmM>(g, stream);
-        case T2SP_GEMM_CFG_64x128: return launch<GemmS>(g, stream);
+        case T2SP_CFG_256x256: return launch<GemmL>(g, stream);
+        case T2SP_CFG_128x128: return launch<GemmM>(g, stream);
+        case T2SP_CFG_64x128: return launch<GemmS>(g, stream);
         default: return T2SP_ERR_SHAPE;
     }
 }

@@ -1,0 +1,176 @@
+// host_conv.cpp — the operator entry point  int conv(I, K, O).
+//
+// Drop-in for the host function the reference generates from
+// t2s/tests/performance/conv/conv.cpp:99-101 (compile_to_host("conv-interface", {I, K},
+// "conv", ...)) and calls from conv-run-fpga.cpp:69.  Accepted argument forms
+// (dimension 0 first, as Halide lists them):
+//   4-D  I(IY, IX, CI, N), K(KY, KX, CI, CO)                     oneapi/src/oneapi-target-5-run.cpp:100-106
+//   2-D  I(CI*N, IY*IX),   K(CO*KX, CI*KY)  (packed)             conv-run-fpga.cpp:49-66, conv.cpp:51-54
+//   O    4-D (OY, OX, CO, N), or the 10-D tiled
+//        (COOO, YYY, XXX, COO, YY, XX, Y, X, CO, N)              conv-run-fpga.cpp:68, conv.cpp:39-44
+// with  O[n,co,y,x] = sum_{ci,kx,ky} I[n,ci,y+ky,x+kx] * K[co,ci,ky,kx].  All sizes come from
+// the buffers; the packed form needs the 10-D output to recover N, CO and the image size.
+// The 4-D form with dense I/K/O is the benchmark's NCHW/OIHW layout and goes to the MFMA
+// kernel directly; other forms are re-laid on the device first, which is what the
+// reference's host serializer/deserializer loops do on the CPU.
+#include "conv-interface.h"
+#include "runtime.hpp"
+#include "t2sp_hip.h"
+
+using namespace t2sp;
+
+namespace {
+struct Logical4 {
+    int64_t ext[4];
+    int64_t str[4];
+};
+
+bool dense_nchw(const Logical4 &t) {
+    return t.str[3] == 1 && t.str[2] == t.ext[3] && t.str[1] == t.ext[2] * t.ext[3] &&
+           t.str[0] == t.ext[1] * t.ext[2] * t.ext[3];
+}
+}  // namespace
+
+static int conv_impl(halide_buffer_t *I, halide_buffer_t *K, halide_buffer_t *O, int cfg) {
+    static const char *op = "conv";
+    std::lock_guard<std::mutex> lock(api_mutex());
+    Span si, sk, so;
+    int err;
+    if ((err = check_buffer(I, op, "I", 4, 2, &si))) return err;
+    if ((err = check_buffer(K, op, "K", 4, 2, &sk))) return err;
+    if ((err = check_buffer(O, op, "O", 4, 10, &so))) return err;
+    const bool packed = I->dimensions == 2;
+    if ((K->dimensions == 2) != packed)
+        return report(halide_error_code_bad_dimensions, op, "I and K must both be 4-D or both be packed 2-D");
+    if (packed && O->dimensions != 10)
+        return report(halide_error_code_bad_dimensions, op, "packed 2-D inputs need the 10-D tiled output");
+
+    // Output: logical (n, co, h, w) with w = the reference's y (innermost), h = its x.
+    int64_t N, CO, OH, OW;
+    const halide_dimension_t *od = O->dim;
+    if (O->dimensions == 4) {
+        OW = od[0].extent; OH = od[1].extent; CO = od[2].extent; N = od[3].extent;
+    } else {
+        CO = (int64_t)od[0].extent * od[3].extent * od[8].extent;
+        OW = (int64_t)od[1].extent * od[4].extent * od[6].extent;
+        OH = (int64_t)od[2].extent * od[5].extent * od[7].extent;
+        N = od[9].extent;
+    }
+    Logical4 li{}, lk{};
+    int64_t CI, KH, KW;
+    if (!packed) {
+        CI = I->dim[2].extent; KW = K->dim[0].extent; KH = K->dim[1].extent;
+        if (K->dim[2].extent != CI || K->dim[3].extent != CO)
+            return report(halide_error_code_constraint_violated, op, "K extents must be (KY, KX, CI, CO)");
+        if (I->dim[0].extent < OW + KW - 1 || I->dim[1].extent < OH + KH - 1 || I->dim[3].extent < N)
+            return report(halide_error_code_access_out_of_bounds, op, "I is smaller than the region the output needs");
+        for (int d = 0; d < 4; d++) { li.str[3 - d] = I->dim[d].stride; lk.str[3 - d] = K->dim[d].stride; }
+    } else {
+        if (N == 0 || CO == 0) return 0;
+        if (I->dim[0].extent % N || K->dim[0].extent % CO)
+            return report(halide_error_code_constraint_violated, op, "packed extents do not divide by N / CO");
+        CI = I->dim[0].extent / N; KH = K->dim[0].extent / CO;
+        if (CI == 0 || K->dim[1].extent % CI)
+            return report(halide_error_code_constraint_violated, op, "K.extent.1 must be CI*KY");
+        KW = K->dim[1].extent / CI;
+        const int64_t IW = OW + KW - 1, IH = OH + KH - 1;
+        if (I->dim[1].extent < IW * IH)
+            return report(halide_error_code_access_out_of_bounds, op, "I is smaller than the region the output needs");
+        const int64_t s1 = I->dim[1].stride, k1 = K->dim[1].stride;
+        li.str[0] = CI; li.str[1] = 1; li.str[3] = s1; li.str[2] = IW * s1;           // (n,ci,h,w)
+        lk.str[0] = 1; lk.str[2] = CO; lk.str[1] = k1; lk.str[3] = CI * k1;            // (co,ci,kh,kw)
+    }
+    if (N == 0 || CO == 0 || OH == 0 || OW == 0) return 0;
+    if (CI == 0 || KH == 0 || KW == 0)
+        return report(halide_error_code_constraint_violated, op, "empty reduction extents");
+    const int64_t IW = OW + KW - 1, IH = OH + KH - 1;
+    li.ext[0] = N; li.ext[1] = CI; li.ext[2] = IH; li.ext[3] = IW;
+    lk.ext[0] = CO; lk.ext[1] = CI; lk.ext[2] = KH; lk.ext[3] = KW;
+    if (N * OH * OW > INT32_MAX || CI * KH * KW > INT32_MAX)
+        return report(halide_error_code_buffer_extents_too_large, op, "problem too large for 32-bit tile indices");
+
+    Staged di, dk, dout;
+    if ((err = di.input(I, si, op))) return err;
+    if ((err = dk.input(K, sk, op))) return err;
+    if ((err = dout.output(O, so, op))) return err;
+    KernelTimer timer;
+
+    // Operands the MFMA kernel can read in place stay where they are; the rest are re-laid into
+    // dense NCHW / OIHW temporaries.
+    const float *pi = di.ptr(), *pk = dk.ptr();
+    float *tmp_i = nullptr, *tmp_k = nullptr, *tmp_o = nullptr;
+    struct Release {
+        float **p[3];
+        ~Release() { for (auto q : p) if (*q) pool().put(*q); }
+    } release{{&tmp_i, &tmp_k, &tmp_o}};
+    const bool out_direct = O->dimensions == 4 && od[0].stride == 1 && OW % 4 == 0 && od[1].stride % 4 == 0 &&
+                            od[2].stride % 4 == 0 && od[3].stride % 4 == 0 && ((uintptr_t)dout.ptr() % 16 == 0);
+    const bool fast_shape = OW % 4 == 0 && (CI * KH * KW) % 4 == 0;
+    Logical4 ci4 = li, ck4 = lk;
+    if (fast_shape && cfg != T2SP_CFG_SCALAR) {
+        if (li.str[3] != 1) {
+            const int64_t elems = N * CI * IH * IW;
+            tmp_i = static_cast<float *>(pool().get(elems * sizeof(float)));
+            if (!tmp_i) return report(halide_error_code_device_malloc_failed, op, "device allocation failed");
+            const int ext[4] = {(int)IW, (int)IH, (int)CI, (int)N};
+            const int64_t ss[4] = {li.str[3], li.str[2], li.str[1], li.str[0]};
+            const int64_t ds[4] = {1, IW, IW * IH, IW * IH * CI};
+            if ((err = t2sp_relayout_f32(pi, tmp_i, 4, ext, ss, ds, api_stream()))) return report(err, op, "relayout failed");
+            pi = tmp_i;
+            ci4.str[3] = 1; ci4.str[2] = IW; ci4.str[1] = IW * IH; ci4.str[0] = IW * IH * CI;
+        }
+        if (!dense_nchw(lk) || ((uintptr_t)pk % 16)) {
+            const int64_t elems = CO * CI * KH * KW;
+            tmp_k = static_cast<float *>(pool().get(elems * sizeof(float)));
+            if (!tmp_k) return report(halide_error_code_device_malloc_failed, op, "device allocation failed");
+            const int ext[4] = {(int)KW, (int)KH, (int)CI, (int)CO};
+            const int64_t ss[4] = {lk.str[3], lk.str[2], lk.str[1], lk.str[0]};
+            const int64_t ds[4] = {1, KW, KW * KH, KW * KH * CI};
+            if ((err = t2sp_relayout_f32(pk, tmp_k, 4, ext, ss, ds, api_stream()))) return report(err, op, "relayout failed");
+            pk = tmp_k;
+            ck4.str[3] = 1; ck4.str[2] = KW; ck4.str[1] = KW * KH; ck4.str[0] = KW * KH * CI;
+        }
+    }
+    int64_t so4[4];
+    float *po = dout.ptr();
+    const bool via_tmp_o = !(out_direct || (O->dimensions == 4 && !(fast_shape && cfg != T2SP_CFG_SCALAR)));
+    if (via_tmp_o) {
+        tmp_o = static_cast<float *>(pool().get(N * CO * OH * OW * sizeof(float)));
+        if (!tmp_o) return report(halide_error_code_device_malloc_failed, op, "device allocation failed");
+        po = tmp_o;
+        so4[3] = 1; so4[2] = OW; so4[1] = OW * OH; so4[0] = OW * OH * CO;
+    } else {
+        for (int d = 0; d < 4; d++) so4[3 - d] = od[d].stride;
+    }
+    err = t2sp_conv2d_f32(pi, pk, po, (int)N, (int)CI, (int)CO, (int)OH, (int)OW, (int)KH, (int)KW, ci4.str,
+                          ck4.str, so4, cfg, api_stream());
+    if (err) return report(err, op, "kernel launch failed");
+    if (via_tmp_o) {
+        int ext[T2SP_MAX_DIMS];
+        int64_t ss[T2SP_MAX_DIMS], ds[T2SP_MAX_DIMS];
+        const int nd = O->dimensions;
+        for (int d = 0; d < nd; d++) { ext[d] = od[d].extent; ds[d] = od[d].stride; }
+        if (nd == 4) {
+            ss[0] = so4[3]; ss[1] = so4[2]; ss[2] = so4[1]; ss[3] = so4[0];
+        } else {
+            const int64_t COOO = od[0].extent, YYY = od[1].extent, XXX = od[2].extent, COO = od[3].extent,
+                          YY = od[4].extent, XX = od[5].extent;
+            ss[0] = so4[1]; ss[3] = COOO * so4[1]; ss[8] = COOO * COO * so4[1];        // cooo, coo, co
+            ss[1] = so4[3]; ss[4] = YYY * so4[3];  ss[6] = YYY * YY * so4[3];          // yyy, yy, y
+            ss[2] = so4[2]; ss[5] = XXX * so4[2];  ss[7] = XXX * XX * so4[2];          // xxx, xx, x
+            ss[9] = so4[0];                                                            // n
+        }
+        if ((err = t2sp_relayout_f32(tmp_o, dout.ptr(), nd, ext, ss, ds, api_stream())))
+            return report(err, op, "relayout failed");
+    }
+    if ((err = timer.stop_and_sync(op))) return err;
+    return dout.finish(op);
+}
+
+extern "C" int conv(halide_buffer_t *I, halide_buffer_t *K, halide_buffer_t *O) {
+    return conv_impl(I, K, O, T2SP_CFG_AUTO);
+}
+
+extern "C" int t2sp_conv_with_cfg(halide_buffer_t *I, halide_buffer_t *K, halide_buffer_t *O, int cfg) {
+    return conv_impl(I, K, O, cfg);
+}

@@ -69,13 +69,13 @@ static int gemm_impl(halide_buffer_t *A, halide_buffer_t *B, halide_buffer_t *C,
 }
 
 extern "C" int gemm(halide_buffer_t *A, halide_buffer_t *B, halide_buffer_t *C) {
-    return gemm_impl(A, B, C, T2SP_GEMM_CFG_AUTO);
+    return gemm_impl(A, B, C, T2SP_CFG_AUTO);
 }
 
 // Name used by the reference's AOT boundary test
 // (t2s/tests/correctness/aot/gemm-generate.cpp:176, gemm-run.cpp:62).
 extern "C" int GEMM(halide_buffer_t *A, halide_buffer_t *B, halide_buffer_t *C) {
-    return gemm_impl(A, B, C, T2SP_GEMM_CFG_AUTO);
+    return gemm_impl(A, B, C, T2SP_CFG_AUTO);
 }
 
 extern "C" int t2sp_gemm_with_cfg(halide_buffer_t *A, halide_buffer_t *B, halide_buffer_t *C, int cfg) {

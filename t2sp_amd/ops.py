@@ -60,6 +60,24 @@ def gemm(A, B, out=None, tiles=None, cfg=0):
     return out
 
 
+def conv(I, W, out=None, cfg=0):
+    """O = conv2d(I, W), stride 1, no padding, through the `conv` entry point
+    (include/conv-interface.h).
+
+    4-D form: I (N, CI, IH, IW), W (CO, CI, KH, KW) -> O (N, CO, OH, OW); dense arrays are
+    the NCHW / OIHW layout.  The reference's packed 2-D inputs and 10-D tiled output
+    (t2s/tests/performance/conv/conv-run-fpga.cpp:49-68) are accepted too, passed as numpy
+    arrays whose axes are the reversed Halide dimensions; `out` must then be given."""
+    if out is None:
+        assert I.ndim == 4 and W.ndim == 4
+        N, _, IH, IW = I.shape
+        CO, _, KH, KW = W.shape
+        out = _empty_like_kind(I, (N, CO, IH - KH + 1, IW - KW + 1))
+    i, w, o = HalideBuffer.wrap(I), HalideBuffer.wrap(W), HalideBuffer.wrap(out)
+    _check("conv", lib().t2sp_conv_with_cfg(i.ref, w.ref, o.ref, int(cfg)))
+    return out
+
+
 def fill_uniform(t, seed):
     """Fill a contiguous torch CUDA float32 tensor with u(seed, i) in [-1, 1)."""
     import torch
