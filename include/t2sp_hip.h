@@ -14,6 +14,7 @@
 #ifndef T2SP_HIP_H
 #define T2SP_HIP_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -59,6 +60,29 @@ int t2sp_sgemm_f32_tiled(const float *A, const float *B, float *C, int M, int N,
 int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, int CI, int CO, int OH,
                     int OW, int KH, int KW, const int64_t *si4, const int64_t *sw4,
                     const int64_t *so4, int cfg, void *stream);
+
+/* V[n,co,h,w,mx,my] = sum_{ci,kh,kw,mk} P[n,ci,S*h+kh,S*w+kw,mx,mk] * W[co,ci,kh,kw,mk,my].
+ * dims11 = {N, CI, CO, OH, OW, KH, KW, S, MX, MY, MK}; sp6/sw6/sv6 are element strides of the
+ * logical indices (n,ci,h,w,mx,mk), (co,ci,kh,kw,mk,my), (n,co,h,w,mx,my).  4x4 poses with the
+ * innermost pose index contiguous take the MFMA kernel, anything else a scalar kernel.  When the
+ * reduction is split over workgroups (`splits` > 1, or chosen automatically with 0) partial
+ * tiles go through `workspace`, which must hold t2sp_capsule_workspace_bytes(...) bytes.
+ * Replaces the device side of the reference's capsule pipeline
+ * (t2s/tests/performance/capsule/capsule.cpp:60-66, capsule/bitstream/a10/a.cl). */
+size_t t2sp_capsule_workspace_bytes(const int *dims11, int cfg, int splits);
+int t2sp_capsule_f32(const float *P, const float *W, float *V, const int *dims11, const int64_t *sp6,
+                     const int64_t *sw6, const int64_t *sv6, int cfg, int splits, float *workspace,
+                     size_t workspace_bytes, void *stream);
+
+/* A[i,r] = sum_{j,k} B[i,j,k] * C[j,r] * D[k,r].  sb3/sc2/sd2/sa2 are element strides of
+ * (i,j,k), (j,r), (k,r), (i,r).  The layout of the reference's golden helper (j contiguous in B
+ * and C, i contiguous in A; t2s/tests/performance/util/util.h:498-515) takes the MFMA kernel,
+ * anything else a scalar kernel.  Workspace as for t2sp_capsule_f32. */
+size_t t2sp_mttkrp_workspace_bytes(int I, int J, int K, int R, int cfg, int splits);
+int t2sp_mttkrp_f32(const float *B, const float *C, const float *D, float *A, int I, int J, int K,
+                    int R, const int64_t *sb3, const int64_t *sc2, const int64_t *sd2,
+                    const int64_t *sa2, int cfg, int splits, float *workspace,
+                    size_t workspace_bytes, void *stream);
 
 /* dst[sum_d c_d*dst_strides[d]] = src[sum_d c_d*src_strides[d]] for every coordinate c of the
  * box `extents` (nd <= T2SP_MAX_DIMS, dimension 0 fastest).  Device-side replacement of the

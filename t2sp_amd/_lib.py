@@ -45,6 +45,17 @@ def _declare(L):
     p64, p32 = ctypes.POINTER(i64), ctypes.POINTER(i32)
     L.t2sp_conv2d_f32.argtypes = [vp, vp, vp] + [i32] * 7 + [p64, p64, p64, i32, vp]
     L.t2sp_relayout_f32.argtypes = [vp, vp, i32, p32, p64, p64, vp]
+    L.capsule.argtypes = [bp, bp, bp]
+    L.t2sp_capsule_with_cfg.argtypes = [bp, bp, bp, i32, i32]
+    L.mttkrp.argtypes = [bp, bp, bp, bp]
+    L.t2sp_mttkrp_with_cfg.argtypes = [bp, bp, bp, bp, i32, i32]
+    sz = ctypes.c_size_t
+    L.t2sp_capsule_workspace_bytes.argtypes = [p32, i32, i32]
+    L.t2sp_capsule_workspace_bytes.restype = sz
+    L.t2sp_capsule_f32.argtypes = [vp, vp, vp, p32, p64, p64, p64, i32, i32, vp, sz, vp]
+    L.t2sp_mttkrp_workspace_bytes.argtypes = [i32, i32, i32, i32, i32, i32]
+    L.t2sp_mttkrp_workspace_bytes.restype = sz
+    L.t2sp_mttkrp_f32.argtypes = [vp, vp, vp, vp, i32, i32, i32, i32, p64, p64, p64, p64, i32, i32, vp, sz, vp]
     L.t2sp_fill_uniform_f32.argtypes = [vp, i64, ctypes.c_uint64, vp]
     L.t2sp_last_kernel_ns.restype = ctypes.c_double
     L.t2sp_release.restype = None

@@ -91,6 +91,26 @@ class HalideBuffer:
         return cls(ext, st, device=t.data_ptr(), keep=t)
 
     @classmethod
+    def from_axes(cls, x, axes):
+        """Buffer whose Halide dimension d is axis axes[d] of the numpy array / torch tensor x."""
+        if isinstance(x, np.ndarray):
+            assert x.dtype == np.float32 and all(s % 4 == 0 for s in x.strides)
+            shape, strides = x.shape, [s // 4 for s in x.strides]
+            kw = dict(host=x.ctypes.data)
+        else:
+            import torch
+            assert x.is_cuda and x.dtype == torch.float32
+            shape, strides = tuple(x.shape), x.stride()
+            kw = dict(device=x.data_ptr())
+        assert sorted(axes) == list(range(len(shape)))
+        ext = [int(shape[a]) for a in axes]
+        st = [int(strides[a]) if shape[a] != 1 else 1 for a in axes]
+        for d in range(1, len(st)):          # size-1 axes carry no stride information
+            if ext[d] == 1:
+                st[d] = st[d - 1] * max(ext[d - 1], 1)
+        return cls(ext, st, keep=x, **kw)
+
+    @classmethod
     def wrap(cls, x):
         if isinstance(x, cls):
             return x

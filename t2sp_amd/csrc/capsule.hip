@@ -1,0 +1,281 @@
+// capsule.hip — capsule convolution over 4x4 pose matrices on fp32 MFMA tiles.
+//
+//   V[n,co,h,w,mx,my] = sum_{ci,kh,kw,mk} P[n,ci,S*h+kh,S*w+kw,mx,mk] * W[co,ci,kh,kw,mk,my]
+//
+// Replaces the reference's capsule device pipeline (t2s/tests/performance/capsule/capsule.cpp:
+// 60-66 as compiled to capsule/bitstream/a10/a.cl).  The 4x4 pose product is folded into the
+// reduction of one GEMM:  D[(n,h,w,mx)][(co,my)], k = (ci,kh,kw,mk) with mk fastest.
+//   * poses   -> KC tile: the 4 mk of one pose row are contiguous, one 128-bit load per slot
+//   * weights -> RC tile: the 4 my of one (co,ci,kh,kw,mk) are contiguous, one 128-bit load
+//   * votes   -> a lane ends up with the 4 my of one (n,co,h,w,mx): one 128-bit store
+// All other strides are free, so the same kernel serves pose-innermost layouts with the
+// channel axis inside or outside the image axes.  The benchmark shape has only 49 tiles of
+// 128 rows, so the reduction is split over several workgroups (splitk.hpp).
+#include "mfma_core.hpp"
+#include "splitk.hpp"
+#include "t2sp_hip.h"
+
+namespace t2sp {
+
+struct CapsuleArgs {
+    const float *P, *W;
+    float *V;
+    int N, CI, CO, OH, OW, KH, KW, S, MX;          // MK = MY = 4
+    int64_t sp[5];   // P strides of (n, ci, h, w, mx); mk stride is 1
+    int64_t sw[5];   // W strides of (co, ci, kh, kw, mk); my stride is 1
+    int64_t sv[5];   // V strides of (n, co, h, w, mx); my stride is 1
+    int ROWS, COLS, KRED;   // N*OH*OW*MX, CO*4, CI*KH*KW*4
+    int tiles_m, tiles_n, splits, Mp, Np;
+    float *scratch;
+};
+
+struct CapsuleOutMap {
+    float *V;
+    int OH, OW, MX, ROWS, COLS;
+    int64_t sv[5];
+    __device__ __forceinline__ void store(int row, int col, v4f v) const {
+        if (row >= ROWS || col >= COLS) return;
+        const int mx = row % MX, pix = row / MX;
+        const int w = pix % OW, h = (pix / OW) % OH, n = pix / (OW * OH);
+        *reinterpret_cast<v4f *>(V + n * sv[0] + (col >> 2) * sv[1] + h * sv[2] + w * sv[3] + mx * sv[4]) = v;
+    }
+};
+
+template <class Cfg>
+struct PoseKcLoader {
+    const float *base[Cfg::A_VEC];
+    bool ok[Cfg::A_VEC];
+    int k[Cfg::A_VEC];
+    v4f reg[Cfg::A_VEC];
+    const CapsuleArgs &g;
+    __device__ PoseKcLoader(const CapsuleArgs &g_, int m0, int k_begin) : g(g_) {
+#pragma unroll
+        for (int i = 0; i < Cfg::A_VEC; i++) {
+            KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
+            int row = m0 + s.row;
+            ok[i] = row < g.ROWS;
+            if (!ok[i]) row = 0;
+            const int mx = row % g.MX, pix = row / g.MX;
+            const int w = pix % g.OW, h = (pix / g.OW) % g.OH, n = pix / (g.OW * g.OH);
+            base[i] = g.P + n * g.sp[0] + (int64_t)h * g.S * g.sp[2] + (int64_t)w * g.S * g.sp[3] + mx * g.sp[4];
+            k[i] = k_begin + s.k;
+        }
+    }
+    __device__ __forceinline__ void fetch() {
+#pragma unroll
+        for (int i = 0; i < Cfg::A_VEC; i++) {
+            const int q = k[i] >> 2;                       // (ci, kh, kw)
+            const int kw = q % g.KW, kh = (q / g.KW) % g.KH, ci = q / (g.KW * g.KH);
+            if (ok[i] && k[i] < g.KRED)
+                reg[i] = *reinterpret_cast<const v4f *>(base[i] + ci * g.sp[1] + kh * g.sp[2] + kw * g.sp[3]);
+            else
+                reg[i] = v4f{0.f, 0.f, 0.f, 0.f};
+            k[i] += Cfg::BK;
+        }
+    }
+    __device__ __forceinline__ void commit(float *stage) const {
+#pragma unroll
+        for (int i = 0; i < Cfg::A_VEC; i++) {
+            KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
+            *reinterpret_cast<v4f *>(stage + s.row * Cfg::LDA + s.k) = reg[i];
+        }
+    }
+};
+
+template <class Cfg>
+struct PoseWeightRcLoader {
+    const float *base[Cfg::B_VEC];
+    bool ok[Cfg::B_VEC];
+    int k[Cfg::B_VEC];
+    v4f reg[Cfg::B_VEC];
+    const CapsuleArgs &g;
+    __device__ PoseWeightRcLoader(const CapsuleArgs &g_, int n0, int k_begin) : g(g_) {
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
+            const int col = n0 + s.col;
+            ok[i] = col < g.COLS;
+            base[i] = g.W + (ok[i] ? (col >> 2) : 0) * g.sw[0];
+            k[i] = k_begin + s.k;
+        }
+    }
+    __device__ __forceinline__ void fetch() {
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            const int mk = k[i] & 3, q = k[i] >> 2;
+            const int kw = q % g.KW, kh = (q / g.KW) % g.KH, ci = q / (g.KW * g.KH);
+            if (ok[i] && k[i] < g.KRED)
+                reg[i] = *reinterpret_cast<const v4f *>(base[i] + ci * g.sw[1] + kh * g.sw[2] + kw * g.sw[3] +
+                                                        mk * g.sw[4]);
+            else
+                reg[i] = v4f{0.f, 0.f, 0.f, 0.f};
+            k[i] += Cfg::BK;
+        }
+    }
+    __device__ __forceinline__ void commit(float *stage) const {
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
+            *reinterpret_cast<v4f *>(stage + s.k * Cfg::LDB + s.col) = reg[i];
+        }
+    }
+};
+
+template <class Cfg>
+__global__ void __launch_bounds__(Cfg::NTHREADS) capsule_kernel(const CapsuleArgs g) {
+    extern __shared__ __align__(16) float smem[];
+    const int tile = blockIdx.x / g.splits, split = blockIdx.x % g.splits;
+    const int tm = tile / g.tiles_n, tn = tile % g.tiles_n;
+    const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
+    int kt0, kt1;
+    split_range((g.KRED + Cfg::BK - 1) / Cfg::BK, g.splits, split, kt0, kt1);
+    PoseKcLoader<Cfg> la(g, m0, kt0 * Cfg::BK);
+    PoseWeightRcLoader<Cfg> lb(g, n0, kt0 * Cfg::BK);
+    Accum<Cfg> acc;
+    mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem);
+    if (g.splits == 1) {
+        CapsuleOutMap map{g.V, g.OH, g.OW, g.MX, g.ROWS, g.COLS, {g.sv[0], g.sv[1], g.sv[2], g.sv[3], g.sv[4]}};
+        drain<Cfg>(acc, [&](int row, int col, v4f v) { map.store(m0 + row, n0 + col, v); });
+    } else {
+        store_partial<Cfg>(acc, g.scratch, split, m0, n0, g.Mp, g.Np);
+    }
+}
+
+// Any pose sizes and strides: one thread per vote element, reduction in (ci,kh,kw,mk) order.
+struct CapsuleGenericArgs {
+    const float *P, *W;
+    float *V;
+    int N, CI, CO, OH, OW, KH, KW, S, MX, MY, MK;
+    int64_t sp[6], sw[6], sv[6];
+};
+__global__ void capsule_scalar_kernel(const CapsuleGenericArgs g) {
+    const int64_t total = (int64_t)g.N * g.CO * g.OH * g.OW * g.MX * g.MY;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total;
+         t += (int64_t)gridDim.x * blockDim.x) {
+        int64_t r = t;
+        const int my = r % g.MY; r /= g.MY;
+        const int mx = r % g.MX; r /= g.MX;
+        const int w = r % g.OW; r /= g.OW;
+        const int h = r % g.OH; r /= g.OH;
+        const int co = r % g.CO;
+        const int n = (int)(r / g.CO);
+        float acc = 0.f;
+        for (int ci = 0; ci < g.CI; ci++)
+            for (int kh = 0; kh < g.KH; kh++)
+                for (int kw = 0; kw < g.KW; kw++)
+                    for (int mk = 0; mk < g.MK; mk++)
+                        acc = fmaf(g.P[n * g.sp[0] + ci * g.sp[1] + (h * g.S + kh) * g.sp[2] +
+                                       (w * g.S + kw) * g.sp[3] + mx * g.sp[4] + mk * g.sp[5]],
+                                   g.W[co * g.sw[0] + ci * g.sw[1] + kh * g.sw[2] + kw * g.sw[3] +
+                                       mk * g.sw[4] + my * g.sw[5]],
+                                   acc);
+        g.V[n * g.sv[0] + co * g.sv[1] + h * g.sv[2] + w * g.sv[3] + mx * g.sv[4] + my * g.sv[5]] = acc;
+    }
+}
+
+using CapsM = TileCfg<128, 128, 16, 4, 1, STYLE_RC>;
+using CapsS = TileCfg<64, 128, 16, 2, 1, STYLE_RC>;
+using CapsL = TileCfg<256, 256, 16, 4, 2, STYLE_RC>;
+
+struct CapsulePlan {
+    int cfg, splits, Mp, Np;
+    size_t scratch_bytes;
+};
+
+static CapsulePlan plan_capsule(int rows, int cols, int kred, int cfg, int splits) {
+    CapsulePlan p{};
+    if (cfg == T2SP_CFG_AUTO) {
+        const int64_t t128 = (int64_t)((rows + 127) / 128) * ((cols + 127) / 128);
+        const int64_t t256 = (int64_t)((rows + 255) / 256) * ((cols + 255) / 256);
+        cfg = (t256 >= 200 && cols > 128) ? T2SP_CFG_256x256 : (t128 >= 24 ? T2SP_CFG_128x128 : T2SP_CFG_64x128);
+    }
+    const int bm = cfg == T2SP_CFG_256x256 ? 256 : cfg == T2SP_CFG_128x128 ? 128 : 64;
+    const int bn = cfg == T2SP_CFG_256x256 ? 256 : 128;
+    const int tiles = ((rows + bm - 1) / bm) * ((cols + bn - 1) / bn);
+    const int ktiles = (kred + 15) / 16;
+    if (splits <= 0) {
+        // fill the 256 CUs about once, keep at least 8 k-tiles per split
+        splits = tiles >= 200 ? 1 : (256 + tiles / 2) / tiles;
+        if (splits > ktiles / 8) splits = ktiles / 8;
+        if (splits < 1) splits = 1;
+    }
+    if (splits > ktiles) splits = ktiles;
+    p.cfg = cfg; p.splits = splits;
+    p.Mp = (rows + bm - 1) / bm * bm;
+    p.Np = (cols + bn - 1) / bn * bn;
+    p.scratch_bytes = splits > 1 ? (size_t)splits * p.Mp * p.Np * sizeof(float) : 0;
+    return p;
+}
+
+template <class Cfg>
+static int launch_capsule(CapsuleArgs g, hipStream_t stream) {
+    g.tiles_m = g.Mp / Cfg::BM;
+    g.tiles_n = g.Np / Cfg::BN;
+    const size_t smem = Cfg::SMEM_FLOATS * sizeof(float);
+    auto kern = capsule_kernel<Cfg>;
+    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+        return T2SP_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * g.splits), dim3(Cfg::NTHREADS), smem, stream, g);
+    if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
+    if (g.splits > 1) {
+        CapsuleOutMap map{g.V, g.OH, g.OW, g.MX, g.ROWS, g.COLS, {g.sv[0], g.sv[1], g.sv[2], g.sv[3], g.sv[4]}};
+        if (launch_splitk_reduce<true>(g.scratch, g.splits, g.Mp, g.Np, map, stream) != hipSuccess)
+            return T2SP_ERR_LAUNCH;
+    }
+    return T2SP_OK;
+}
+
+}  // namespace t2sp
+
+static bool capsule_fast(const int *d, const int64_t *sp6, const int64_t *sw6, const int64_t *sv6,
+                         const float *P, const float *W, const float *V) {
+    const int MY = d[9], MK = d[10];
+    if (MY != 4 || MK != 4) return false;
+    if (sp6[5] != 1 || sw6[5] != 1 || sv6[5] != 1) return false;
+    for (int i = 0; i < 5; i++)
+        if (sp6[i] % 4 || sw6[i] % 4 || sv6[i] % 4) return false;
+    return ((uintptr_t)P % 16 == 0) && ((uintptr_t)W % 16 == 0) && ((uintptr_t)V % 16 == 0);
+}
+
+extern "C" size_t t2sp_capsule_workspace_bytes(const int *dims11, int cfg, int splits) {
+    const int *d = dims11;
+    if (!d) return 0;
+    const int64_t rows = (int64_t)d[0] * d[3] * d[4] * d[8], cols = (int64_t)d[2] * 4, kred = (int64_t)d[1] * d[5] * d[6] * 4;
+    if (rows <= 0 || rows > INT32_MAX || cols > INT32_MAX || kred > INT32_MAX) return 0;
+    return t2sp::plan_capsule((int)rows, (int)cols, (int)kred, cfg, splits).scratch_bytes;
+}
+
+extern "C" int t2sp_capsule_f32(const float *P, const float *W, float *V, const int *dims11,
+                                const int64_t *sp6, const int64_t *sw6, const int64_t *sv6, int cfg,
+                                int splits, float *workspace, size_t workspace_bytes, void *stream) {
+    using namespace t2sp;
+    if (!dims11 || !sp6 || !sw6 || !sv6) return T2SP_ERR_SHAPE;
+    const int *d = dims11;   // N, CI, CO, OH, OW, KH, KW, S, MX, MY, MK
+    for (int i = 0; i < 11; i++)
+        if (d[i] <= 0) return T2SP_ERR_SHAPE;
+    const int64_t rows = (int64_t)d[0] * d[3] * d[4] * d[8], cols = (int64_t)d[2] * 4,
+                  kred = (int64_t)d[1] * d[5] * d[6] * 4;
+    if (rows > INT32_MAX / 2 || cols > INT32_MAX / 2 || kred > INT32_MAX / 2) return T2SP_ERR_SHAPE;
+    if (cfg == T2SP_CFG_SCALAR || !capsule_fast(d, sp6, sw6, sv6, P, W, V)) {
+        CapsuleGenericArgs a{P, W, V, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], d[8], d[9], d[10], {}, {}, {}};
+        for (int i = 0; i < 6; i++) { a.sp[i] = sp6[i]; a.sw[i] = sw6[i]; a.sv[i] = sv6[i]; }
+        const int64_t total = (int64_t)d[0] * d[2] * d[3] * d[4] * d[8] * d[9];
+        const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
+        hipLaunchKernelGGL(capsule_scalar_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+        return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+    }
+    const CapsulePlan p = plan_capsule((int)rows, (int)cols, (int)kred, cfg, splits);
+    if (p.scratch_bytes > workspace_bytes || (p.scratch_bytes && !workspace)) return T2SP_ERR_SHAPE;
+    CapsuleArgs g{};
+    g.P = P; g.W = W; g.V = V;
+    g.N = d[0]; g.CI = d[1]; g.CO = d[2]; g.OH = d[3]; g.OW = d[4]; g.KH = d[5]; g.KW = d[6]; g.S = d[7]; g.MX = d[8];
+    for (int i = 0; i < 5; i++) { g.sp[i] = sp6[i]; g.sw[i] = sw6[i]; g.sv[i] = sv6[i]; }
+    g.ROWS = (int)rows; g.COLS = (int)cols; g.KRED = (int)kred;
+    g.splits = p.splits; g.Mp = p.Mp; g.Np = p.Np; g.scratch = workspace;
+    switch (p.cfg) {
+        case T2SP_CFG_256x256: return launch_capsule<CapsL>(g, (hipStream_t)stream);
+        case T2SP_CFG_128x128: return launch_capsule<CapsM>(g, (hipStream_t)stream);
+        case T2SP_CFG_64x128: return launch_capsule<CapsS>(g, (hipStream_t)stream);
+        default: return T2SP_ERR_SHAPE;
+    }
+}

@@ -1,0 +1,260 @@
+// mttkrp.hip — matricised tensor times Khatri-Rao product on fp32 MFMA tiles.
+//
+//   A[i,r] = sum_{j,k} B[i,j,k] * C[j,r] * D[k,r]
+//
+// The reference holds only a golden loop for this operator
+// (t2s/tests/performance/util/util.h:498-515, d(i,j) = sum_k (sum_l a(l,i,k) c(l,j)) b(k,j));
+// its buffers a(l,i,k), c(l,j), b(k,j), d(i,j) are B[i,j,k] with j innermost, C[j,r] with j
+// innermost, D[k,r] with k innermost and A[i,r] with i innermost.
+// GEMM view: rows i, columns r, reduction index (k, j) with j fastest.
+//   * B tensor -> KC tile: 4 consecutive j of one (i,k), one 128-bit load; B is read once
+//   * Khatri-Rao operand -> KC tile [r][(k,j)]: C[j..j+3, r] loaded as 128 bits and multiplied
+//     in registers by D[k,r] before it is written to LDS; it is never materialised in memory
+//   * A -> a lane ends up with 4 consecutive i of one column r: one 128-bit store
+// Only (I/BM)*(R/BN) output tiles exist, so the (k,j) reduction is split over many workgroups
+// (splitk.hpp) and B streams through all CUs.
+#include "mfma_core.hpp"
+#include "splitk.hpp"
+#include "t2sp_hip.h"
+
+namespace t2sp {
+
+struct MttkrpArgs {
+    const float *B, *C, *D;
+    float *A;
+    int I, J, K, R;
+    int64_t sb_i, sb_k;   // B strides of i and k (j stride 1)
+    int64_t sc_r;         // C stride of r (j stride 1)
+    int64_t sd_k, sd_r;   // D strides
+    int64_t sa_r;         // A stride of r (i stride 1)
+    int tiles_m, tiles_n, splits, Mp, Np;
+    float *scratch;
+};
+
+struct MttkrpOutMap {
+    float *A;
+    int I, R;
+    int64_t sa_r;
+    __device__ __forceinline__ void store(int row, int col, v4f v) const {
+        if (row >= I || col >= R) return;
+        *reinterpret_cast<v4f *>(A + col * sa_r + row) = v;
+    }
+};
+
+// B tensor rows: slot (row i, 4 consecutive j) of reduction tile kt: k = kt / (J/BK).
+template <class Cfg>
+struct TensorKcLoader {
+    const float *p[Cfg::A_VEC];
+    bool ok[Cfg::A_VEC];
+    v4f reg[Cfg::A_VEC];
+    int kt, tiles_per_k;
+    int64_t sb_k;
+    __device__ TensorKcLoader(const MttkrpArgs &g, int m0, int kt0)
+        : kt(kt0), tiles_per_k(g.J / Cfg::BK), sb_k(g.sb_k) {
+#pragma unroll
+        for (int i = 0; i < Cfg::A_VEC; i++) {
+            KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
+            ok[i] = m0 + s.row < g.I;
+            p[i] = g.B + (int64_t)(ok[i] ? m0 + s.row : 0) * g.sb_i + s.k;
+        }
+    }
+    __device__ __forceinline__ void fetch() {
+        const int k = kt / tiles_per_k, j0 = (kt - k * tiles_per_k) * Cfg::BK;
+#pragma unroll
+        for (int i = 0; i < Cfg::A_VEC; i++) {
+            if (ok[i])
+                reg[i] = *reinterpret_cast<const v4f *>(p[i] + k * sb_k + j0);
+            else
+                reg[i] = v4f{0.f, 0.f, 0.f, 0.f};
+        }
+        kt++;
+    }
+    __device__ __forceinline__ void commit(float *stage) const {
+#pragma unroll
+        for (int i = 0; i < Cfg::A_VEC; i++) {
+            KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
+            *reinterpret_cast<v4f *>(stage + s.row * Cfg::LDA + s.k) = reg[i];
+        }
+    }
+};
+
+// Khatri-Rao rows: slot (column r, 4 consecutive j) of reduction tile kt holds
+// C[j..j+3, r] * D[k, r], formed in registers.
+template <class Cfg>
+struct KhatriRaoKcLoader {
+    const float *pc[Cfg::B_VEC];
+    const float *pd[Cfg::B_VEC];
+    bool ok[Cfg::B_VEC];
+    v4f reg[Cfg::B_VEC];
+    float dval[Cfg::B_VEC];
+    int kt, tiles_per_k;
+    int64_t sd_k;
+    __device__ KhatriRaoKcLoader(const MttkrpArgs &g, int n0, int kt0)
+        : kt(kt0), tiles_per_k(g.J / Cfg::BK), sd_k(g.sd_k) {
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
+            ok[i] = n0 + s.row < g.R;
+            const int r = ok[i] ? n0 + s.row : 0;
+            pc[i] = g.C + (int64_t)r * g.sc_r + s.k;
+            pd[i] = g.D + (int64_t)r * g.sd_r;
+        }
+    }
+    __device__ __forceinline__ void fetch() {
+        const int k = kt / tiles_per_k, j0 = (kt - k * tiles_per_k) * Cfg::BK;
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            if (ok[i]) {
+                reg[i] = *reinterpret_cast<const v4f *>(pc[i] + j0);
+                dval[i] = pd[i][k * sd_k];
+            } else {
+                reg[i] = v4f{0.f, 0.f, 0.f, 0.f};
+                dval[i] = 0.f;
+            }
+        }
+        kt++;
+    }
+    __device__ __forceinline__ void commit(float *stage) const {
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
+            *reinterpret_cast<v4f *>(stage + s.row * Cfg::LDB + s.k) = reg[i] * dval[i];
+        }
+    }
+};
+
+template <class Cfg>
+__global__ void __launch_bounds__(Cfg::NTHREADS) mttkrp_kernel(const MttkrpArgs g) {
+    extern __shared__ __align__(16) float smem[];
+    const int tile = blockIdx.x % (g.tiles_m * g.tiles_n), split = blockIdx.x / (g.tiles_m * g.tiles_n);
+    const int tm = tile % g.tiles_m, tn = tile / g.tiles_m;
+    const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
+    int kt0, kt1;
+    split_range(g.K * (g.J / Cfg::BK), g.splits, split, kt0, kt1);
+    TensorKcLoader<Cfg> la(g, m0, kt0);
+    KhatriRaoKcLoader<Cfg> lb(g, n0, kt0);
+    Accum<Cfg> acc;
+    mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem);
+    if (g.splits == 1) {
+        MttkrpOutMap map{g.A, g.I, g.R, g.sa_r};
+        drain<Cfg>(acc, [&](int row, int col, v4f v) { map.store(m0 + row, n0 + col, v); });
+    } else {
+        store_partial<Cfg>(acc, g.scratch, split, m0, n0, g.Mp, g.Np);
+    }
+}
+
+// Any strides and sizes: one thread per output, in the reference's two-step order.
+struct MttkrpGenericArgs {
+    const float *B, *C, *D;
+    float *A;
+    int I, J, K, R;
+    int64_t sb[3], sc[2], sd[2], sa[2];
+};
+__global__ void mttkrp_scalar_kernel(const MttkrpGenericArgs g) {
+    const int64_t total = (int64_t)g.I * g.R;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total;
+         t += (int64_t)gridDim.x * blockDim.x) {
+        const int i = t % g.I, r = t / g.I;
+        float acc = 0.f;
+        for (int k = 0; k < g.K; k++) {
+            float e = 0.f;
+            for (int j = 0; j < g.J; j++)
+                e = fmaf(g.B[i * g.sb[0] + j * g.sb[1] + k * g.sb[2]], g.C[j * g.sc[0] + r * g.sc[1]], e);
+            acc = fmaf(e, g.D[k * g.sd[0] + r * g.sd[1]], acc);
+        }
+        g.A[i * g.sa[0] + r * g.sa[1]] = acc;
+    }
+}
+
+using MttL = TileCfg<256, 256, 16, 4, 2, STYLE_KC>;   // 8 waves, 64x128 per wave
+using MttM = TileCfg<128, 128, 16, 2, 2, STYLE_KC>;   // 4 waves, 64x64 per wave
+using MttS = TileCfg<64, 64, 16, 2, 1, STYLE_KC>;     // 2 waves, 32x64 per wave
+
+struct MttkrpPlan {
+    int cfg, splits, Mp, Np;
+    size_t scratch_bytes;
+};
+
+static MttkrpPlan plan_mttkrp(int I, int J, int K, int R, int cfg, int splits) {
+    MttkrpPlan p{};
+    if (cfg == T2SP_CFG_AUTO)
+        cfg = (I >= 256 && R >= 256) ? T2SP_CFG_256x256 : (I >= 128 && R >= 128) ? T2SP_CFG_128x128 : T2SP_CFG_64x128;
+    const int bm = cfg == T2SP_CFG_256x256 ? 256 : cfg == T2SP_CFG_128x128 ? 128 : 64;
+    const int bn = bm;
+    const int tiles = ((I + bm - 1) / bm) * ((R + bn - 1) / bn);
+    const int64_t ktiles = (int64_t)K * (J / 16);
+    if (splits <= 0) {
+        splits = tiles >= 200 ? 1 : (256 + tiles / 2) / tiles;
+        if (splits > ktiles / 16) splits = (int)(ktiles / 16);
+        if (splits < 1) splits = 1;
+    }
+    if (splits > ktiles) splits = (int)ktiles;
+    p.cfg = cfg; p.splits = splits;
+    p.Mp = (I + bm - 1) / bm * bm;
+    p.Np = (R + bn - 1) / bn * bn;
+    p.scratch_bytes = splits > 1 ? (size_t)splits * p.Mp * p.Np * sizeof(float) : 0;
+    return p;
+}
+
+template <class Cfg>
+static int launch_mttkrp(MttkrpArgs g, hipStream_t stream) {
+    g.tiles_m = g.Mp / Cfg::BM;
+    g.tiles_n = g.Np / Cfg::BN;
+    const size_t smem = Cfg::SMEM_FLOATS * sizeof(float);
+    auto kern = mttkrp_kernel<Cfg>;
+    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+        return T2SP_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * g.splits), dim3(Cfg::NTHREADS), smem, stream, g);
+    if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
+    if (g.splits > 1) {
+        MttkrpOutMap map{g.A, g.I, g.R, g.sa_r};
+        if (launch_splitk_reduce<false>(g.scratch, g.splits, g.Mp, g.Np, map, stream) != hipSuccess)
+            return T2SP_ERR_LAUNCH;
+    }
+    return T2SP_OK;
+}
+
+static bool mttkrp_fast(int I, int J, const int64_t *sb3, const int64_t *sc2, const int64_t *sd2,
+                        const int64_t *sa2, const float *B, const float *C, const float *A) {
+    (void)sd2;
+    return J % 16 == 0 && I % 4 == 0 && sb3[1] == 1 && sc2[0] == 1 && sa2[0] == 1 && sb3[0] % 4 == 0 &&
+           sb3[2] % 4 == 0 && sc2[1] % 4 == 0 && sa2[1] % 4 == 0 && ((uintptr_t)B % 16 == 0) &&
+           ((uintptr_t)C % 16 == 0) && ((uintptr_t)A % 16 == 0);
+}
+
+}  // namespace t2sp
+
+extern "C" size_t t2sp_mttkrp_workspace_bytes(int I, int J, int K, int R, int cfg, int splits) {
+    if (I <= 0 || J <= 0 || K <= 0 || R <= 0) return 0;
+    return t2sp::plan_mttkrp(I, J, K, R, cfg, splits).scratch_bytes;
+}
+
+extern "C" int t2sp_mttkrp_f32(const float *B, const float *C, const float *D, float *A, int I, int J,
+                               int K, int R, const int64_t *sb3, const int64_t *sc2,
+                               const int64_t *sd2, const int64_t *sa2, int cfg, int splits,
+                               float *workspace, size_t workspace_bytes, void *stream) {
+    using namespace t2sp;
+    if (I <= 0 || J <= 0 || K <= 0 || R <= 0 || !sb3 || !sc2 || !sd2 || !sa2) return T2SP_ERR_SHAPE;
+    if ((int64_t)K * J > INT32_MAX) return T2SP_ERR_SHAPE;
+    if (cfg == T2SP_CFG_SCALAR || !mttkrp_fast(I, J, sb3, sc2, sd2, sa2, B, C, A)) {
+        MttkrpGenericArgs a{B, C, D, A, I, J, K, R, {sb3[0], sb3[1], sb3[2]}, {sc2[0], sc2[1]},
+                            {sd2[0], sd2[1]}, {sa2[0], sa2[1]}};
+        const int64_t total = (int64_t)I * R;
+        const int blocks = (int)((total + 63) / 64 < 65536 ? (total + 63) / 64 : 65536);
+        hipLaunchKernelGGL(mttkrp_scalar_kernel, dim3(blocks), dim3(64), 0, (hipStream_t)stream, a);
+        return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+    }
+    const MttkrpPlan p = plan_mttkrp(I, J, K, R, cfg, splits);
+    if (p.scratch_bytes > workspace_bytes || (p.scratch_bytes && !workspace)) return T2SP_ERR_SHAPE;
+    MttkrpArgs g{};
+    g.B = B; g.C = C; g.D = D; g.A = A;
+    g.I = I; g.J = J; g.K = K; g.R = R;
+    g.sb_i = sb3[0]; g.sb_k = sb3[2]; g.sc_r = sc2[1]; g.sd_k = sd2[0]; g.sd_r = sd2[1]; g.sa_r = sa2[1];
+    g.splits = p.splits; g.Mp = p.Mp; g.Np = p.Np; g.scratch = workspace;
+    switch (p.cfg) {
+        case T2SP_CFG_256x256: return launch_mttkrp<MttL>(g, (hipStream_t)stream);
+        case T2SP_CFG_128x128: return launch_mttkrp<MttM>(g, (hipStream_t)stream);
+        case T2SP_CFG_64x128: return launch_mttkrp<MttS>(g, (hipStream_t)stream);
+        default: return T2SP_ERR_SHAPE;
+    }
+}

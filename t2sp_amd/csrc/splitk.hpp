@@ -1,0 +1,69 @@
+// splitk.hpp — splitting the reduction of one output tile over several workgroups.
+//
+// Operators whose output has too few tiles to fill 256 CUs (capsule conv at small batch,
+// MTTKRP, small SGEMM) give each tile to S workgroups, each reducing a contiguous slice of k.
+// Every workgroup stores its partial tile into scratch laid out as S planes of the (padded)
+// output matrix; a second kernel adds the S planes in ascending order (so the result does not
+// depend on scheduling) and hands each group of four sums to the operator's output map.
+// Plane layout follows the direction in which a lane's four values are adjacent:
+//   RC tiles: plane[row][col], four consecutive columns per lane
+//   KC tiles: plane[col][row], four consecutive rows per lane
+#pragma once
+#include "mfma_core.hpp"
+
+namespace t2sp {
+
+// k-tiles [begin, end) of split s out of S over `ktiles` tiles (sizes differ by at most one).
+__device__ __host__ inline void split_range(int ktiles, int S, int s, int &begin, int &end) {
+    const int base = ktiles / S, extra = ktiles % S;
+    begin = s * base + (s < extra ? s : extra);
+    end = begin + base + (s < extra ? 1 : 0);
+}
+
+template <class Cfg>
+__device__ __forceinline__ void store_partial(const Accum<Cfg> &acc, float *scratch, int split,
+                                              int m0, int n0, int Mp, int Np) {
+    float *plane = scratch + (size_t)split * Mp * Np;
+    drain<Cfg>(acc, [&](int row, int col, v4f v) {
+        if constexpr (Cfg::BSTYLE == STYLE_RC)
+            *reinterpret_cast<v4f *>(plane + (size_t)(m0 + row) * Np + n0 + col) = v;
+        else
+            *reinterpret_cast<v4f *>(plane + (size_t)(n0 + col) * Mp + m0 + row) = v;
+    });
+}
+
+// OutMap: __device__ void store(int row, int col, v4f v) const — writes D[row][col..col+3]
+// (ALONG_COLS) or D[row..row+3][col] (!ALONG_COLS), ignoring out-of-range positions.
+template <bool ALONG_COLS, class OutMap>
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *scratch, int S, int Mp,
+                                                             int Np, const OutMap map) {
+    const size_t plane = (size_t)Mp * Np;
+    const size_t groups = plane / 4;
+    for (size_t g = (size_t)blockIdx.x * blockDim.x + threadIdx.x; g < groups;
+         g += (size_t)gridDim.x * blockDim.x) {
+        v4f sum = *reinterpret_cast<const v4f *>(scratch + g * 4);
+        for (int s = 1; s < S; s++) sum += *reinterpret_cast<const v4f *>(scratch + s * plane + g * 4);
+        int row, col;
+        if (ALONG_COLS) {
+            row = (int)(g / (Np / 4));
+            col = (int)(g % (Np / 4)) * 4;
+        } else {
+            col = (int)(g / (Mp / 4));
+            row = (int)(g % (Mp / 4)) * 4;
+        }
+        map.store(row, col, sum);
+    }
+}
+
+template <bool ALONG_COLS, class OutMap>
+inline hipError_t launch_splitk_reduce(const float *scratch, int S, int Mp, int Np, const OutMap &map,
+                                       hipStream_t stream) {
+    const size_t groups = (size_t)Mp * Np / 4;
+    size_t blocks = (groups + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL((splitk_reduce_kernel<ALONG_COLS, OutMap>), dim3((unsigned)blocks), dim3(256), 0,
+                       stream, scratch, S, Mp, Np, map);
+    return hipGetLastError();
+}
+
+}  // namespace t2sp

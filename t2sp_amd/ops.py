@@ -78,6 +78,62 @@ def conv(I, W, out=None, cfg=0):
     return out
 
 
+def _alloc_inner_first(ref, shape, inner_axis):
+    """Array of logical `shape` whose axis `inner_axis` is contiguous and the rest C-ordered."""
+    order = [a for a in range(len(shape)) if a != inner_axis] + [inner_axis]
+    base = _empty_like_kind(ref, tuple(shape[a] for a in order))
+    inv = [order.index(a) for a in range(len(shape))]
+    return base.permute(*inv) if _is_torch(base) else base.transpose(inv)
+
+
+def capsule(P, W, out=None, stride=2, cfg=0, splits=0):
+    """Capsule convolution through the `capsule` entry point (include/capsule-interface.h).
+
+    P: (N, CI, IY, IX, MX, MK) poses, W: (CO, CI, KY, KX, MK, MY) weights ->
+    V: (N, CO, OY, OX, MX, MY) votes, V[n,co,y,x] = sum P[n,ci,S*y+ky,S*x+kx] @ W[co,ci,ky,kx]
+    (4x4 matrix products).  Any strides with the last axis contiguous; dense C-order arrays are
+    the layout [n][ci][y][x][mx][mk].  `stride` only sizes a freshly allocated output: the entry
+    point recovers S from the image sizes, as the C interface has no such argument."""
+    N, CI, IY, IX, MX, MK = P.shape
+    CO, _, KY, KX, _, MY = W.shape
+    if out is None:
+        out = _empty_like_kind(P, (N, CO, (IY - KY) // stride + 1, (IX - KX) // stride + 1, MX, MY))
+    p = HalideBuffer.from_axes(P, [5, 4, 1, 2, 3, 0])
+    w = HalideBuffer.from_axes(W, [5, 4, 1, 0, 2, 3])
+    v = HalideBuffer.from_axes(out, [5, 4, 1, 2, 3, 0])
+    _check("capsule", lib().t2sp_capsule_with_cfg(p.ref, w.ref, v.ref, int(cfg), int(splits)))
+    return out
+
+
+def mttkrp_reference_layout(B, C, D):
+    """Views of B (i,j,k), C (j,r), D (k,r) re-laid as the reference's golden helper stores them
+    (t2s/tests/performance/util/util.h:498-515): j contiguous in B and C, k contiguous in D."""
+    if _is_torch(B):
+        return (B.permute(2, 0, 1).contiguous().permute(1, 2, 0), C.t().contiguous().t(),
+                D.t().contiguous().t())
+    return (np.ascontiguousarray(B.transpose(2, 0, 1)).transpose(1, 2, 0),
+            np.ascontiguousarray(C.T).T, np.ascontiguousarray(D.T).T)
+
+
+def mttkrp(B, C, D, out=None, cfg=0, splits=0):
+    """A[i,r] = sum_{j,k} B[i,j,k] C[j,r] D[k,r] through the `mttkrp` entry point
+    (include/mttkrp-interface.h).
+
+    B: (I, J, K), C: (J, R), D: (K, R) -> A: (I, R), all indexed logically; the entry point
+    wants the reference helper's memory layout (see mttkrp_reference_layout), i.e. unit stride
+    along j in B and C, along k in D and along i in A, and rejects anything else with -8."""
+    I, J, K = B.shape
+    R = C.shape[1]
+    if out is None:
+        out = _alloc_inner_first(B, (I, R), 0)
+    b = HalideBuffer.from_axes(B, [1, 0, 2])
+    c = HalideBuffer.from_axes(C, [0, 1])
+    d = HalideBuffer.from_axes(D, [0, 1])
+    a = HalideBuffer.from_axes(out, [0, 1])
+    _check("mttkrp", lib().t2sp_mttkrp_with_cfg(b.ref, c.ref, d.ref, a.ref, int(cfg), int(splits)))
+    return out
+
+
 def fill_uniform(t, seed):
     """Fill a contiguous torch CUDA float32 tensor with u(seed, i) in [-1, 1)."""
     import torch
