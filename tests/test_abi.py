@@ -91,12 +91,39 @@ def test_gemm_rejects_bad_arguments_without_a_device():
     assert L.gemm(neg.ref, b.ref, c.ref) == -28
 
 
+def test_other_entries_reject_bad_arguments_without_a_device():
+    L = t2sp_amd.lib()
+    i4, k4, o4 = _buf((2, 4, 6, 6)), _buf((8, 4, 3, 3)), _buf((2, 8, 4, 4))
+    assert L.conv(None, k4.ref, o4.ref) == -12
+    assert L.conv(i4.ref, k4.ref, _buf((2, 8, 4)).ref) == -43
+    assert L.conv(_buf((36, 8)).ref, k4.ref, o4.ref) == -43           # packed I with 4-D K
+    assert L.conv(_buf((36, 8)).ref, _buf((12, 24)).ref, o4.ref) == -43  # packed inputs need 10-D O
+    assert L.conv(i4.ref, _buf((8, 5, 3, 3)).ref, o4.ref) == -8       # CI mismatch
+    assert L.conv(_buf((2, 4, 5, 6)).ref, k4.ref, o4.ref) == -4       # input too small
+    p, w, v = _buf((1, 5, 5, 4, 4, 4)), _buf((3, 3, 2, 4, 4, 4)), _buf((1, 2, 2, 2, 4, 4))
+    assert L.capsule(p.ref, w.ref, None) == -12
+    assert L.capsule(_buf((4, 5, 5, 4, 4)).ref, w.ref, v.ref) == -43
+    assert L.capsule(p.ref, _buf((3, 3, 2, 5, 4, 4)).ref, v.ref) == -8   # CI mismatch
+    assert L.capsule(_buf((1, 2, 2, 4, 4, 4)).ref, w.ref, v.ref) == -4   # image smaller than kernel
+    b = HalideBuffer.from_axes(np.zeros((5, 6, 8), np.float32), [2, 1, 0])
+    c, d, a = _buf((7, 8)), _buf((7, 5)), _buf((7, 6))
+    assert L.mttkrp(b.ref, c.ref, d.ref, None) == -12
+    assert L.mttkrp(b.ref, _buf((7, 9)).ref, d.ref, a.ref) == -8
+    assert L.mttkrp(b.ref, _buf((7, 4)).ref, d.ref, a.ref) == -4
+    assert L.mttkrp(_buf((6, 8)).ref, c.ref, d.ref, a.ref) == -43
+
+
 def test_thin_layer_rejects_bad_shapes():
     L = t2sp_amd.lib()
     assert L.t2sp_sgemm_f32(None, None, None, 0, 4, 4, 4, 4, 4, 0, None) == -8
     assert L.t2sp_sgemm_f32(None, None, None, 4, 4, 4, 4, 4, 4, 12345, None) in (-8, -23)
     assert L.t2sp_fill_uniform_f32(None, -1, 0, None) == -8
     assert L.t2sp_fill_uniform_f32(None, 0, 0, None) == 0
+    assert L.t2sp_conv2d_f32(None, None, None, 1, 1, 1, 0, 4, 3, 3, None, None, None, 0, None) == -8
+    assert L.t2sp_mttkrp_f32(None, None, None, None, 0, 4, 4, 4, None, None, None, None, 0, 0, None, 0, None) == -8
+    assert L.t2sp_capsule_f32(None, None, None, None, None, None, None, 0, 0, None, 0, None) == -8
+    assert L.t2sp_relayout_f32(None, None, 11, None, None, None, None) == -8
+    assert L.t2sp_mttkrp_workspace_bytes(512, 512, 512, 256, 1, 128) == 128 * 512 * 256 * 4
 
 
 def test_python_mirror_raises_with_code():

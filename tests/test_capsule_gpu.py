@@ -1,0 +1,79 @@
+"""GPU parity tests of the capsule convolution path through `capsule`
+(include/capsule-interface.h).  Arrays are indexed P (n,ci,y,x,mx,mk), W (co,ci,ky,kx,mk,my),
+V (n,co,y,x,mx,my), the oracle's convention."""
+import numpy as np
+import pytest
+
+import t2sp_amd
+from conftest import rel_fro
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+
+def test_constant_fixture_exact():
+    """CONSTANT(=1) inputs: every vote is CI*KX*KY*MK = 1152 at CI=32
+    (correctness/multi-projection/capsule.cpp:75-102)."""
+    P = np.ones((2, 32, 15, 15, 4, 4), np.float32)
+    W = np.ones((8, 32, 3, 3, 4, 4), np.float32)
+    V = t2sp_amd.capsule(P, W)
+    assert V.shape == (2, 8, 7, 7, 4, 4) and (V == 1152).all()
+
+
+@pytest.mark.parametrize("cfg,splits", [(0, 0), (2, 1), (2, 3), (3, 2), (1, 2), (99, 0)])
+def test_tiny_constants_parity_golden_and_ure_order(oracle, cfg, splits):
+    """The TINY sizes of capsule/const-parameters.h:43-52 with N=4 (capsule-run-fpga.cpp:37-39):
+    16 -> 16 channels, 15x15 -> 7x7, against both reduction orders the reference uses."""
+    P, W = oracle.fill_uniform((4, 16, 15, 15, 4, 4), 1), oracle.fill_uniform((16, 16, 3, 3, 4, 4), 2)
+    got = t2sp_amd.capsule(P, W, cfg=cfg, splits=splits)
+    for order, cii in ((oracle.ORDER_GOLDEN, 1), (oracle.ORDER_URE, 4)):
+        err, mx = rel_fro(got, oracle.capsule(P, W, order=order, cii=cii))
+        assert err <= TOL, (cfg, splits, order, err, mx)
+
+
+def test_integers_exact_and_identity_weights(oracle):
+    rng = np.random.default_rng(0)
+    P = rng.integers(-2, 3, (2, 8, 9, 7, 4, 4)).astype(np.float32)
+    W = rng.integers(-2, 3, (6, 8, 3, 3, 4, 4)).astype(np.float32)
+    assert (t2sp_amd.capsule(P, W) == oracle.capsule(P, W)).all()
+    Wi = np.zeros((8, 8, 3, 3, 4, 4), np.float32)
+    for c in range(8):
+        Wi[c, c, 1, 2] = np.eye(4)
+    Pr = oracle.fill_uniform(P.shape, 3)
+    assert (t2sp_amd.capsule(Pr, Wi) == Pr[:, :, 1:9:2, 2:7:2]).all()
+
+
+def test_oneapi_memory_layout_and_other_strides(oracle):
+    """Memory laid out as the oneAPI driver fills it (oneapi/src/oneapi-target-6-run.cpp:52-99):
+    P [n][ix][iy][ci][mx][mk], W [kx][ky][co][ci][mk][my]; plus a stride-1 and a stride-3 case."""
+    P, W = oracle.fill_uniform((2, 8, 7, 9, 4, 4), 4), oracle.fill_uniform((4, 8, 3, 3, 4, 4), 5)
+    ref = oracle.capsule(P, W)
+    Pm = np.ascontiguousarray(P.transpose(0, 3, 2, 1, 4, 5)).transpose(0, 3, 2, 1, 4, 5)
+    Wm = np.ascontiguousarray(W.transpose(3, 2, 0, 1, 4, 5)).transpose(2, 3, 1, 0, 4, 5)
+    assert not Pm.flags["C_CONTIGUOUS"]
+    assert rel_fro(t2sp_amd.capsule(Pm, Wm), ref)[0] <= TOL
+    for s, iy in ((1, 5), (3, 9)):
+        Ps = oracle.fill_uniform((1, 4, iy, iy, 4, 4), 6)
+        got = t2sp_amd.capsule(Ps, W[:, :4], stride=s)
+        assert rel_fro(got, oracle.capsule(Ps, np.ascontiguousarray(W[:, :4]), stride=s))[0] <= TOL
+
+
+def test_other_pose_sizes_take_the_scalar_kernel(oracle):
+    P, W = oracle.fill_uniform((1, 3, 5, 5, 2, 3), 7), oracle.fill_uniform((2, 3, 3, 3, 3, 5), 8)
+    assert rel_fro(t2sp_amd.capsule(P, W), oracle.capsule(P, W))[0] <= TOL
+
+
+def test_config4_full_size(oracle):
+    """BASELINE config 4: N=32, CI=CO=32, 15x15 -> 7x7, 3x3, stride 2, on the device, whole
+    result against the oracle."""
+    import torch
+    P = t2sp_amd.fill_uniform(torch.empty(32, 32, 15, 15, 4, 4, device="cuda"), 41)
+    W = t2sp_amd.fill_uniform(torch.empty(32, 32, 3, 3, 4, 4, device="cuda"), 42)
+    V = t2sp_amd.capsule(P, W)
+    torch.cuda.synchronize()
+    ref = oracle.capsule(P.cpu().numpy(), W.cpu().numpy())
+    err, mx = rel_fro(V.cpu().numpy(), ref)
+    print("capsule full size rel_fro %.3e max_abs %.3e" % (err, mx))
+    assert err <= TOL
+    V2 = t2sp_amd.capsule(P, W)
+    assert torch.equal(V, V2)          # the split reduction is added in a fixed order

@@ -1,0 +1,130 @@
+"""GPU parity tests of the 2-D convolution path through `conv` (include/conv-interface.h).
+
+Oracle convention: logical I (n, ci, y, x), W (co, ci, ky, kx) with y the reference's innermost
+spatial axis.  The 4-D buffers of the entry point are I(IY, IX, CI, N), K(KY, KX, CI, CO),
+O(OY, OX, CO, N), i.e. numpy arrays indexed [n][ci][x][y]: arrays below are built in oracle
+order and handed over with the two spatial axes swapped."""
+import numpy as np
+import pytest
+
+import t2sp_amd
+from conftest import rel_fro
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+
+def run(I, W, cfg=0, out=None):
+    """Oracle-ordered (n,c,y,x) arrays -> entry point -> oracle-ordered result."""
+    O = t2sp_amd.conv(np.ascontiguousarray(I.transpose(0, 1, 3, 2)), np.ascontiguousarray(W.transpose(0, 1, 3, 2)), cfg=cfg)
+    return O.transpose(0, 1, 3, 2)
+
+
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 99])
+def test_small_parity_golden_and_ure_order(oracle, cfg):
+    I, W = oracle.fill_uniform((2, 32, 14, 10), 1), oracle.fill_uniform((24, 32, 3, 3), 2)
+    got = run(I, W, cfg)
+    for order, cii in ((oracle.ORDER_GOLDEN, 1), (oracle.ORDER_URE, 8)):
+        err, mx = rel_fro(got, oracle.conv(I, W, order=order, cii=cii))
+        assert err <= TOL, (cfg, order, err, mx)
+    assert rel_fro(got, oracle.conv(I, W, acc=oracle.ACC_F32_FMA))[0] <= TOL
+
+
+def test_integers_exact_and_special_kernels(oracle):
+    rng = np.random.default_rng(0)
+    I = rng.integers(-2, 3, (3, 16, 10, 14)).astype(np.float32)
+    W = rng.integers(-2, 3, (8, 16, 3, 3)).astype(np.float32)
+    assert (run(I, W) == oracle.conv(I, W)).all()
+    assert (run(np.ones((1, 8, 6, 6), np.float32), np.ones((4, 8, 3, 3), np.float32)) == 8 * 9).all()
+    delta = np.zeros((16, 16, 3, 3), np.float32)
+    for c in range(16):
+        delta[c, c, 2, 1] = 1.0
+    X = oracle.fill_uniform((2, 16, 10, 9), 3)
+    assert (run(X, delta) == X[:, :, 2:10, 1:8]).all()
+
+
+def test_1x1_kernel_is_gemm(oracle):
+    I, W = oracle.fill_uniform((2, 64, 8, 8), 4), oracle.fill_uniform((32, 64, 1, 1), 5)
+    got = run(I, W)
+    as_gemm = oracle.gemm(W[:, :, 0, 0], I.transpose(1, 0, 2, 3).reshape(64, -1)).reshape(32, 2, 8, 8).transpose(1, 0, 2, 3)
+    assert rel_fro(got, as_gemm)[0] <= TOL
+
+
+@pytest.mark.parametrize("shape", [(1, 3, 5, 7, 6, 3, 3), (2, 5, 3, 4, 4, 2, 3), (1, 8, 8, 9, 8, 1, 1), (2, 4, 6, 12, 5, 5, 5)])
+def test_ragged_shapes(oracle, shape):
+    """Sizes the vector path cannot take (OY not a multiple of 4, odd reductions) and edge tiles."""
+    N, CI, CO, OY, OX, KY, KX = shape
+    I, W = oracle.fill_uniform((N, CI, OY + KY - 1, OX + KX - 1), 6), oracle.fill_uniform((CO, CI, KY, KX), 7)
+    assert rel_fro(run(I, W), oracle.conv(I, W))[0] <= TOL
+
+
+def test_strided_4d_buffers(oracle):
+    """Padded rows / channels in I and O, and an input larger than the output needs."""
+    N, CI, CO, OY, OX = 2, 8, 8, 8, 6
+    Ibig = oracle.fill_uniform((N, CI + 1, OX + 2 + 1, OY + 2 + 6), 8)       # [n][ci][x][y], padded
+    Iv = Ibig[:, :CI, :OX + 2, :OY + 2]
+    W = oracle.fill_uniform((CO, CI, 3, 3), 9)
+    Obig = np.full((N, CO, OX, OY + 4), np.nan, np.float32)
+    Ov = Obig[..., :OY]
+    t2sp_amd.conv(Iv, W, out=Ov)
+    ref = oracle.conv(np.ascontiguousarray(Iv).transpose(0, 1, 3, 2), W.transpose(0, 1, 3, 2)).transpose(0, 1, 3, 2)
+    assert rel_fro(Ov, ref)[0] <= TOL
+    assert np.isnan(Obig[..., OY:]).all()
+
+
+def tiled_view(O10):
+    """10-D tiled output (numpy axes reversed: n,co,x,y,xx,yy,coo,xxx,yyy,cooo) -> (n,co,y,x)."""
+    N, CO, X, Y, XX, YY, COO, XXX, YYY, COOO = O10.shape
+    t = O10.transpose(0, 1, 6, 9, 3, 5, 8, 2, 4, 7)       # n, co,coo,cooo, y,yy,yyy, x,xx,xxx
+    return t.reshape(N, CO * COO * COOO, Y * YY * YYY, X * XX * XXX)
+
+
+@pytest.mark.parametrize("consts", [
+    dict(CII=4, CI=4, COOO=4, COO=4, CO=4, YYY=4, XXX=4, YY=1, XX=1, Y=1, X=1, N=4),       # TINY
+    dict(CII=8, CI=2, COOO=8, COO=1, CO=2, YYY=8, XXX=1, YY=2, XX=2, Y=1, X=3, N=2),       # GPU-like
+    dict(CII=4, CI=3, COOO=2, COO=3, CO=2, YYY=5, XXX=2, YY=2, XX=1, Y=1, X=3, N=1),       # odd tiles
+])
+def test_reference_packed_inputs_and_tiled_output(oracle, consts):
+    """The FPGA-flavour call of conv-run-fpga.cpp:49-93: packed 2-D I and K, 10-D tiled O,
+    with the TINY constants of conv/const-parameters.h:37-48 and two other sets."""
+    c = consts
+    TCI, TCO = c["CII"] * c["CI"], c["COOO"] * c["COO"] * c["CO"]
+    OY, OX, N = c["YYY"] * c["YY"] * c["Y"], c["XXX"] * c["XX"] * c["X"], c["N"]
+    I, W = oracle.fill_uniform((N, TCI, OY + 2, OX + 2), 10), oracle.fill_uniform((TCO, TCI, 3, 3), 11)
+    ref = oracle.conv(I, W)
+    Ip = np.ascontiguousarray(I.transpose(3, 2, 0, 1)).reshape((OX + 2) * (OY + 2), N * TCI)   # i(ci+CI*n, iy+IY*ix)
+    Kp = np.ascontiguousarray(W.transpose(2, 1, 3, 0)).reshape(3 * TCI, 3 * TCO)               # k(co+CO*kx, ci+CI*ky)
+    O10 = np.full((N, c["CO"], c["X"], c["Y"], c["XX"], c["YY"], c["COO"], c["XXX"], c["YYY"], c["COOO"]), np.nan, np.float32)
+    t2sp_amd.conv(Ip, Kp, out=O10)
+    assert rel_fro(tiled_view(O10), ref)[0] <= TOL
+    # oneAPI flavour: 4-D inputs with the same tiled output (oneapi-target-5-run.cpp:100-106,150-190)
+    O10b = np.full_like(O10, np.nan)
+    t2sp_amd.conv(np.ascontiguousarray(I.transpose(0, 1, 3, 2)), np.ascontiguousarray(W.transpose(0, 1, 3, 2)), out=O10b)
+    assert (O10b == O10).all()
+
+
+def test_packed_inputs_need_tiled_output():
+    with pytest.raises(t2sp_amd.T2spError) as e:
+        t2sp_amd.conv(np.zeros((36, 8), np.float32), np.zeros((12, 12), np.float32), out=np.zeros((1, 4, 4, 4), np.float32))
+    assert e.value.code == -43
+
+
+def test_config3_full_size_sampled_and_shift_property(oracle):
+    """BASELINE config 3 on the device: N=64, CI=CO=256, 56x56 output, 3x3.  The oracle checks two
+    images x 24 channels; a one-hot kernel gives an exact shifted copy of the whole input."""
+    import torch
+    N, C, OH = 64, 256, 56
+    I = t2sp_amd.fill_uniform(torch.empty(N, C, OH + 2, OH + 2, device="cuda"), 31)
+    W = t2sp_amd.fill_uniform(torch.empty(C, C, 3, 3, device="cuda"), 32)
+    O = t2sp_amd.conv(I, W)
+    torch.cuda.synchronize()
+    In, Wn = I[[0, N - 1]].cpu().numpy().transpose(0, 1, 3, 2), W.cpu().numpy().transpose(0, 1, 3, 2)
+    cos = slice(100, 124)
+    ref = oracle.conv(In, Wn, co_range=(cos.start, cos.stop))[:, cos]
+    got = O[[0, N - 1]][:, cos].cpu().numpy().transpose(0, 1, 3, 2)
+    err, mx = rel_fro(got, ref)
+    print("conv full size rel_fro %.3e max_abs %.3e" % (err, mx))
+    assert err <= TOL
+    Wd = torch.zeros_like(W)
+    Wd[torch.arange(C), torch.arange(C), 1, 2] = 1.0
+    assert torch.equal(t2sp_amd.conv(I, Wd), I[:, :, 1:OH + 1, 2:OH + 2])
