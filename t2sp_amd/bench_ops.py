@@ -1,0 +1,97 @@
+"""Timed launches of the non-headline benchmark configurations (conv, capsule, MTTKRP),
+used by bench.py's `others` block.  Inputs are synthetic, seeded, resident in HBM."""
+import ctypes
+
+from . import ops
+from ._lib import lib
+
+i64 = ctypes.c_int64
+
+
+def _time(torch, launch, steps, warmup):
+    for _ in range(warmup):
+        launch()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        launch()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def _entry(tf, peak, ms, **extra):
+    d = {"TFLOP/s": round(tf, 3), "frac_of_peak": round(tf / peak, 4), "avg_launch_ms": round(ms, 5)}
+    d.update(extra)
+    return d
+
+
+def conv_config3(torch, steps, warmup, peak):
+    L = lib()
+    N, CI, CO, OH, OW = 64, 256, 256, 56, 56
+    I = ops.fill_uniform(torch.empty(N, CI, OH + 2, OW + 2, device="cuda"), 1)
+    W = ops.fill_uniform(torch.empty(CO, CI, 3, 3, device="cuda"), 2)
+    O = torch.empty(N, CO, OH, OW, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    si, sw, so = ((i64 * 4)(*t.stride()) for t in (I, W, O))
+
+    def launch():
+        rc = L.t2sp_conv2d_f32(I.data_ptr(), W.data_ptr(), O.data_ptr(), N, CI, CO, OH, OW, 3, 3, si, sw, so, 0, s)
+        assert rc == 0, rc
+
+    ms = _time(torch, launch, steps, warmup)
+    flop = 2.0 * N * CO * OH * OW * CI * 9
+    return _entry(flop / ms / 1e9, peak, ms, workload="N=64 CI=CO=256 56x56 out 3x3 NCHW (configs[2])")
+
+
+def capsule_config4(torch, steps, warmup, peak):
+    L = lib()
+    N, CI, CO = 32, 32, 32
+    P = ops.fill_uniform(torch.empty(N, CI, 15, 15, 4, 4, device="cuda"), 1)
+    W = ops.fill_uniform(torch.empty(CO, CI, 3, 3, 4, 4, device="cuda"), 2)
+    V = torch.empty(N, CO, 7, 7, 4, 4, device="cuda")
+    dims = (ctypes.c_int * 11)(N, CI, CO, 7, 7, 3, 3, 2, 4, 4, 4)
+    sp, sw, sv = ((i64 * 6)(*t.stride()) for t in (P, W, V))
+    nbytes = L.t2sp_capsule_workspace_bytes(dims, 0, 0)
+    ws = torch.empty(max(nbytes // 4, 1), device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        rc = L.t2sp_capsule_f32(P.data_ptr(), W.data_ptr(), V.data_ptr(), dims, sp, sw, sv, 0, 0, ws.data_ptr(), nbytes, s)
+        assert rc == 0, rc
+
+    ms = _time(torch, launch, max(steps, 200), max(warmup, 20))
+    flop = 2.0 * N * CO * 49 * 16 * CI * 9 * 4
+    return _entry(flop / ms / 1e9, peak, ms, workload="N=32 CI=CO=32 15x15->7x7 3x3 s2 4x4 poses (configs[3])",
+                  note="back-to-back launches; includes the split-reduction kernel")
+
+
+def mttkrp_config5(torch, steps, warmup, peak):
+    L = lib()
+    I = J = K = 512
+    R = 256
+    B = ops.fill_uniform(torch.empty(K, I, J, device="cuda"), 1).permute(1, 2, 0)
+    C = ops.fill_uniform(torch.empty(R, J, device="cuda"), 2).t()
+    D = ops.fill_uniform(torch.empty(R, K, device="cuda"), 3).t()
+    A = torch.empty(R, I, device="cuda").t()
+    nbytes = L.t2sp_mttkrp_workspace_bytes(I, J, K, R, 0, 0)
+    ws = torch.empty(max(nbytes // 4, 1), device="cuda")
+    sb, sc, sd, sa = (i64 * 3)(*B.stride()), (i64 * 2)(*C.stride()), (i64 * 2)(*D.stride()), (i64 * 2)(*A.stride())
+    s = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        rc = L.t2sp_mttkrp_f32(B.data_ptr(), C.data_ptr(), D.data_ptr(), A.data_ptr(), I, J, K, R, sb, sc, sd, sa,
+                               0, 0, ws.data_ptr(), nbytes, s)
+        assert rc == 0, rc
+
+    ms = _time(torch, launch, steps, warmup)
+    flop = 2.0 * I * J * K * R + J * K * R
+    return _entry(flop / ms / 1e9, peak, ms, workload="I=J=K=512 R=256, helper layout (configs[4])",
+                  note="includes the split-reduction kernel")
+
+
+def run_all(torch, steps, warmup, peak):
+    return {"conv2d": conv_config3(torch, steps, warmup, peak),
+            "capsule": capsule_config4(torch, steps, warmup, peak),
+            "mttkrp": mttkrp_config5(torch, steps, warmup, peak)}
