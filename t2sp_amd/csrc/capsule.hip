@@ -45,10 +45,10 @@ template <class Cfg>
 struct PoseKcLoader {
     const float *base[Cfg::A_VEC];
     bool ok[Cfg::A_VEC];
-    int k[Cfg::A_VEC];
-    v4f reg[Cfg::A_VEC];
+    v4f reg[2][Cfg::A_VEC];
+    int k0;
     const CapsuleArgs &g;
-    __device__ PoseKcLoader(const CapsuleArgs &g_, int m0, int k_begin) : g(g_) {
+    __device__ PoseKcLoader(const CapsuleArgs &g_, int m0, int k_begin) : k0(k_begin), g(g_) {
 #pragma unroll
         for (int i = 0; i < Cfg::A_VEC; i++) {
             KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
@@ -58,26 +58,26 @@ struct PoseKcLoader {
             const int mx = row % g.MX, pix = row / g.MX;
             const int w = pix % g.OW, h = (pix / g.OW) % g.OH, n = pix / (g.OW * g.OH);
             base[i] = g.P + n * g.sp[0] + (int64_t)h * g.S * g.sp[2] + (int64_t)w * g.S * g.sp[3] + mx * g.sp[4];
-            k[i] = k_begin + s.k;
         }
     }
+    template <int S>
     __device__ __forceinline__ void fetch() {
 #pragma unroll
         for (int i = 0; i < Cfg::A_VEC; i++) {
-            const int q = k[i] >> 2;                       // (ci, kh, kw)
+            KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
+            const int k = k0 + s.k;
+            const int q = k >> 2;                       // (ci, kh, kw)
             const int kw = q % g.KW, kh = (q / g.KW) % g.KH, ci = q / (g.KW * g.KH);
-            if (ok[i] && k[i] < g.KRED)
-                reg[i] = *reinterpret_cast<const v4f *>(base[i] + ci * g.sp[1] + kh * g.sp[2] + kw * g.sp[3]);
-            else
-                reg[i] = v4f{0.f, 0.f, 0.f, 0.f};
-            k[i] += Cfg::BK;
+            reg[S][i] = load_or_zero(base[i] + ci * g.sp[1] + kh * g.sp[2] + kw * g.sp[3], ok[i] && k < g.KRED, g.P);
         }
+        k0 += Cfg::BK;
     }
+    template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
 #pragma unroll
         for (int i = 0; i < Cfg::A_VEC; i++) {
             KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
-            *reinterpret_cast<v4f *>(stage + s.row * Cfg::LDA + s.k) = reg[i];
+            *reinterpret_cast<v4f *>(stage + s.row * Cfg::LDA + s.k) = reg[S][i];
         }
     }
 };
@@ -86,37 +86,37 @@ template <class Cfg>
 struct PoseWeightRcLoader {
     const float *base[Cfg::B_VEC];
     bool ok[Cfg::B_VEC];
-    int k[Cfg::B_VEC];
-    v4f reg[Cfg::B_VEC];
+    v4f reg[2][Cfg::B_VEC];
+    int k0;
     const CapsuleArgs &g;
-    __device__ PoseWeightRcLoader(const CapsuleArgs &g_, int n0, int k_begin) : g(g_) {
+    __device__ PoseWeightRcLoader(const CapsuleArgs &g_, int n0, int k_begin) : k0(k_begin), g(g_) {
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
             const int col = n0 + s.col;
             ok[i] = col < g.COLS;
             base[i] = g.W + (ok[i] ? (col >> 2) : 0) * g.sw[0];
-            k[i] = k_begin + s.k;
         }
     }
+    template <int S>
     __device__ __forceinline__ void fetch() {
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
-            const int mk = k[i] & 3, q = k[i] >> 2;
+            RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
+            const int k = k0 + s.k;
+            const int mk = k & 3, q = k >> 2;
             const int kw = q % g.KW, kh = (q / g.KW) % g.KH, ci = q / (g.KW * g.KH);
-            if (ok[i] && k[i] < g.KRED)
-                reg[i] = *reinterpret_cast<const v4f *>(base[i] + ci * g.sw[1] + kh * g.sw[2] + kw * g.sw[3] +
-                                                        mk * g.sw[4]);
-            else
-                reg[i] = v4f{0.f, 0.f, 0.f, 0.f};
-            k[i] += Cfg::BK;
+            reg[S][i] = load_or_zero(base[i] + ci * g.sw[1] + kh * g.sw[2] + kw * g.sw[3] + mk * g.sw[4],
+                                     ok[i] && k < g.KRED, g.W);
         }
+        k0 += Cfg::BK;
     }
+    template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
-            *reinterpret_cast<v4f *>(stage + s.k * Cfg::LDB + s.col) = reg[i];
+            *reinterpret_cast<v4f *>(stage + s.k * Cfg::LDB + s.col) = reg[S][i];
         }
     }
 };
@@ -199,7 +199,7 @@ static CapsulePlan plan_capsule(int rows, int cols, int kred, int cfg, int split
         if (splits > ktiles / 8) splits = ktiles / 8;
         if (splits < 1) splits = 1;
     }
-    if (splits > ktiles) splits = ktiles;
+    if (splits > (ktiles + 1) / 2) splits = (ktiles + 1) / 2;
     p.cfg = cfg; p.splits = splits;
     p.Mp = (rows + bm - 1) / bm * bm;
     p.Np = (cols + bn - 1) / bn * bn;

@@ -35,10 +35,10 @@ template <class Cfg, bool EDGE>
 struct Im2colRcLoader {
     const float *base[Cfg::B_VEC];   // pixel part of the address (n, h, w), fixed for the block
     bool col_ok[Cfg::B_VEC];
-    int k[Cfg::B_VEC];               // reduction row this slot loads next
-    v4f reg[Cfg::B_VEC];
+    v4f reg[2][Cfg::B_VEC];
+    int k0;                          // first reduction row of the tile fetched next
     const ConvArgs &g;
-    __device__ Im2colRcLoader(const ConvArgs &g_, int p0) : g(g_) {
+    __device__ Im2colRcLoader(const ConvArgs &g_, int p0) : k0(0), g(g_) {
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
@@ -49,27 +49,34 @@ struct Im2colRcLoader {
             const int n = p / hw, rem = p - n * hw;
             const int h = rem / g.OW, w = rem - h * g.OW;
             base[i] = g.I + n * g.si_n + h * g.si_h + w;
-            k[i] = s.k;
         }
     }
+    template <int S>
     __device__ __forceinline__ void fetch() {
+        const int khw = g.KH * g.KW;
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
-            const int khw = g.KH * g.KW;
-            const int ci = k[i] / khw, r = k[i] - ci * khw;
+            RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
+            const int k = k0 + s.k;
+            const int ci = k / khw, r = k - ci * khw;
             const int kh = r / g.KW, kw = r - kh * g.KW;
-            if (!EDGE || (col_ok[i] && k[i] < g.KRED))
-                reg[i] = *reinterpret_cast<const v4f_u *>(base[i] + ci * g.si_c + kh * g.si_h + kw);
-            else
-                reg[i] = v4f{0.f, 0.f, 0.f, 0.f};
-            k[i] += Cfg::BK;
+            const float *ptr = base[i] + ci * g.si_c + kh * g.si_h + kw;
+            if (EDGE) {
+                const bool ok = col_ok[i] && k < g.KRED;
+                const v4f_u v = *reinterpret_cast<const v4f_u *>(ok ? ptr : g.I);
+                reg[S][i] = ok ? (v4f)v : v4f{0.f, 0.f, 0.f, 0.f};
+            } else {
+                reg[S][i] = *reinterpret_cast<const v4f_u *>(ptr);
+            }
         }
+        k0 += (EDGE || k0 + 2 * Cfg::BK <= g.KRED) ? Cfg::BK : 0;
     }
+    template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
-            *reinterpret_cast<v4f *>(stage + s.k * Cfg::LDB + s.col) = reg[i];
+            *reinterpret_cast<v4f *>(stage + s.k * Cfg::LDB + s.col) = reg[S][i];
         }
     }
 };
@@ -83,7 +90,7 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) conv_kernel(const ConvArgs g) {
     RowMajorKcLoader<Cfg, EDGE> la(g.W, g.sw_o, co0, g.CO, g.KRED);
     Im2colRcLoader<Cfg, EDGE> lb(g, p0);
     Accum<Cfg> acc;
-    mainloop<Cfg>(acc, la, lb, (g.KRED + Cfg::BK - 1) / Cfg::BK, smem);
+    mainloop<Cfg>(acc, la, lb, ktiles_even<Cfg>(g.KRED), smem);
     const int hw = g.OH * g.OW;
     drain<Cfg>(acc, [&](int row, int col, v4f v) {
         const int co = co0 + row, p = p0 + col;
@@ -122,7 +129,7 @@ static int launch_conv(ConvArgs g, hipStream_t stream) {
     g.tiles_m = (g.CO + Cfg::BM - 1) / Cfg::BM;
     g.tiles_n = (g.P + Cfg::BN - 1) / Cfg::BN;
     g.group_m = g.tiles_m;   // all output channels of a pixel tile run together: the input tile is shared in L2
-    const bool edge = (g.CO % Cfg::BM) || (g.P % Cfg::BN) || (g.KRED % Cfg::BK);
+    const bool edge = (g.CO % Cfg::BM) || (g.P % Cfg::BN) || (g.KRED % (2 * Cfg::BK));
     const size_t smem = Cfg::SMEM_FLOATS * sizeof(float);
     auto kern = edge ? conv_kernel<Cfg, true> : conv_kernel<Cfg, false>;
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,

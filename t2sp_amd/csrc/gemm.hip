@@ -41,7 +41,7 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) sgemm_kernel(const GemmArgs g) 
     RowMajorKcLoader<Cfg, EDGE> la(g.A, g.lda, m0, g.M, g.K);
     RowMajorRcLoader<Cfg, EDGE> lb(g.B, g.ldb, n0, g.N, g.K);
     Accum<Cfg> acc;
-    mainloop<Cfg>(acc, la, lb, (g.K + Cfg::BK - 1) / Cfg::BK, smem);
+    mainloop<Cfg>(acc, la, lb, ktiles_even<Cfg>(g.K), smem);
     drain<Cfg>(acc, [&](int row, int col, v4f v) {
         const int r = m0 + row, c = n0 + col;
         if (EDGE && (r >= g.M || c >= g.N)) return;
@@ -76,7 +76,7 @@ static int launch(GemmArgs g, hipStream_t stream) {
     g.tiles_n = (g.N + Cfg::BN - 1) / Cfg::BN;
     // bands of about sqrt(32) tile-rows keep a XCD's resident tiles near-square
     g.group_m = g.tiles_m >= 4 ? 4 : g.tiles_m;
-    const bool edge = (g.M % Cfg::BM) || (g.N % Cfg::BN) || (g.K % Cfg::BK);
+    const bool edge = (g.M % Cfg::BM) || (g.N % Cfg::BN) || (g.K % (2 * Cfg::BK));
     const size_t smem = Cfg::SMEM_FLOATS * sizeof(float);
     auto kern = edge ? sgemm_kernel<Cfg, true> : sgemm_kernel<Cfg, false>;
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,

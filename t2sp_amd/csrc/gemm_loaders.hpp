@@ -1,4 +1,10 @@
 // gemm_loaders.hpp — tile loaders for operands that are plain row-major matrices.
+//
+// Loader contract (see mainloop in mfma_core.hpp): fetch<S>() loads the next k-tile into
+// register slot S and steps to the following one; it may be called for up to two tiles past
+// the end of the reduction, whose data is never multiplied.  EDGE loaders predicate every load
+// (rows/columns outside the matrix and k >= K read as 0); plain loaders assume full tiles and
+// stay on the last tile instead of stepping past the end of the matrix.
 #pragma once
 #include "mfma_core.hpp"
 
@@ -8,35 +14,40 @@ namespace t2sp {
 template <class Cfg, bool EDGE>
 struct RowMajorKcLoader {
     const float *p[Cfg::A_VEC];
+    const float *safe;
     bool row_ok[Cfg::A_VEC];
-    int kpos[Cfg::A_VEC];
-    v4f reg[Cfg::A_VEC];
-    int K;
-    __device__ RowMajorKcLoader(const float *A, int64_t lda, int m0, int M, int K_) : K(K_) {
+    v4f reg[2][Cfg::A_VEC];
+    int k0, K;
+    __device__ RowMajorKcLoader(const float *A, int64_t lda, int m0, int M, int K_, int k_begin = 0)
+        : safe(A), k0(k_begin), K(K_) {
 #pragma unroll
         for (int i = 0; i < Cfg::A_VEC; i++) {
             KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
             row_ok[i] = !EDGE || (m0 + s.row < M);
-            kpos[i] = s.k;
-            p[i] = A + (int64_t)(m0 + (row_ok[i] ? s.row : 0)) * lda + s.k;
+            p[i] = A + (int64_t)(m0 + (row_ok[i] ? s.row : 0)) * lda + k_begin + s.k;
         }
     }
+    template <int S>
     __device__ __forceinline__ void fetch() {
 #pragma unroll
         for (int i = 0; i < Cfg::A_VEC; i++) {
-            if (!EDGE || (row_ok[i] && kpos[i] < K))
-                reg[i] = *reinterpret_cast<const v4f *>(p[i]);
+            KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
+            if (EDGE)
+                reg[S][i] = load_or_zero(p[i], row_ok[i] && k0 + s.k < K, safe);
             else
-                reg[i] = v4f{0.f, 0.f, 0.f, 0.f};
-            p[i] += Cfg::BK;
-            kpos[i] += Cfg::BK;
+                reg[S][i] = *reinterpret_cast<const v4f *>(p[i]);
         }
+        const int step = (EDGE || k0 + 2 * Cfg::BK <= K) ? Cfg::BK : 0;
+        k0 += step;
+#pragma unroll
+        for (int i = 0; i < Cfg::A_VEC; i++) p[i] += step;
     }
+    template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
 #pragma unroll
         for (int i = 0; i < Cfg::A_VEC; i++) {
             KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
-            *reinterpret_cast<v4f *>(stage + s.row * Cfg::LDA + s.k) = reg[i];
+            *reinterpret_cast<v4f *>(stage + s.row * Cfg::LDA + s.k) = reg[S][i];
         }
     }
 };
@@ -45,39 +56,50 @@ struct RowMajorKcLoader {
 template <class Cfg, bool EDGE>
 struct RowMajorRcLoader {
     const float *p[Cfg::B_VEC];
+    const float *safe;
     bool col_ok[Cfg::B_VEC];
-    int kpos[Cfg::B_VEC];
-    v4f reg[Cfg::B_VEC];
-    int64_t step;
-    int K;
-    __device__ RowMajorRcLoader(const float *B, int64_t ldb, int n0, int N, int K_)
-        : step((int64_t)Cfg::BK * ldb), K(K_) {
+    v4f reg[2][Cfg::B_VEC];
+    int64_t ldb;
+    int k0, K;
+    __device__ RowMajorRcLoader(const float *B, int64_t ldb_, int n0, int N, int K_, int k_begin = 0)
+        : safe(B), ldb(ldb_), k0(k_begin), K(K_) {
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
             col_ok[i] = !EDGE || (n0 + s.col < N);
-            kpos[i] = s.k;
-            p[i] = B + (int64_t)s.k * ldb + n0 + (col_ok[i] ? s.col : 0);
+            p[i] = B + (int64_t)(k_begin + s.k) * ldb + n0 + (col_ok[i] ? s.col : 0);
         }
     }
+    template <int S>
     __device__ __forceinline__ void fetch() {
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
-            if (!EDGE || (col_ok[i] && kpos[i] < K))
-                reg[i] = *reinterpret_cast<const v4f *>(p[i]);
+            RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
+            if (EDGE)
+                reg[S][i] = load_or_zero(p[i], col_ok[i] && k0 + s.k < K, safe);
             else
-                reg[i] = v4f{0.f, 0.f, 0.f, 0.f};
-            p[i] += step;
-            kpos[i] += Cfg::BK;
+                reg[S][i] = *reinterpret_cast<const v4f *>(p[i]);
         }
+        const bool adv = EDGE || k0 + 2 * Cfg::BK <= K;
+        const int64_t step = adv ? (int64_t)Cfg::BK * ldb : 0;
+        k0 += adv ? Cfg::BK : 0;
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) p[i] += step;
     }
+    template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
-            *reinterpret_cast<v4f *>(stage + s.k * Cfg::LDB + s.col) = reg[i];
+            *reinterpret_cast<v4f *>(stage + s.k * Cfg::LDB + s.col) = reg[S][i];
         }
     }
 };
+
+// Number of k-tiles the mainloop runs for a reduction of length K: rounded up to a pair.
+template <class Cfg>
+__device__ __host__ inline int ktiles_even(int K) {
+    return ((K + 2 * Cfg::BK - 1) / (2 * Cfg::BK)) * 2;
+}
 
 }  // namespace t2sp

@@ -60,10 +60,18 @@ struct TileCfg {
     static constexpr int B_VEC = BN * BK / 4 / NTHREADS;
     static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be a multiple of 32x32");
     static_assert(BSTYLE == STYLE_KC || TN % 128 == 0, "RC wave tiles are 128-column groups");
-    static_assert(BK % 8 == 0, "BK must be a multiple of 8");
+    static_assert(BK % 16 == 0, "BK must be a multiple of 16 (an even number of k-slices of 8)");
     static_assert(A_VEC * 4 * NTHREADS == BM * BK && A_VEC >= 1, "A tile must split evenly");
     static_assert(B_VEC * 4 * NTHREADS == BN * BK && B_VEC >= 1, "B tile must split evenly");
 };
+
+// 128-bit global load that is predicated without a branch (a branch would split the basic
+// block the MFMA/memory interleave is scheduled in): an invalid slot reads `safe` and yields 0.
+template <class V = float __attribute__((ext_vector_type(4)))>
+__device__ __forceinline__ V load_or_zero(const float *ptr, bool valid, const float *safe) {
+    const V v = *reinterpret_cast<const V *>(valid ? ptr : safe);
+    return valid ? v : V{0.f, 0.f, 0.f, 0.f};
+}
 
 // Position, inside a KC tile of ROWS x BK, of the f-th float4 of the tile.
 template <int BK>
@@ -92,87 +100,146 @@ struct Accum {
     }
 };
 
-// One k-tile (BK) of multiply-accumulate from the LDS stages As/Bs.
+// Operand fragments of one wave for one k-slice of 8: what the MFMAs of that slice read.
 template <class Cfg>
-__device__ __forceinline__ void mma_ktile(Accum<Cfg> &acc, const float *__restrict__ As,
-                                          const float *__restrict__ Bs, int wm, int wn, int lane) {
+struct Frag {
+    static constexpr int NB = Cfg::NT;   // RC: (NT/4 groups) x 4 k-pairs; KC: NT column tiles
+    v4f a[Cfg::MT];
+    v4f b[NB];
+};
+
+template <class Cfg>
+__device__ __forceinline__ void load_frag(Frag<Cfg> &f, const float *__restrict__ As,
+                                          const float *__restrict__ Bs, int kk, int wm, int wn,
+                                          int lane) {
     const int l32 = lane & 31, lhi = lane >> 5;
-    const float *a_base = As + (wm * Cfg::TM + l32) * Cfg::LDA + 4 * lhi;
+    const float *a_base = As + (wm * Cfg::TM + l32) * Cfg::LDA + 4 * lhi + kk * 8;
 #pragma unroll
-    for (int kk = 0; kk < Cfg::BK / 8; kk++) {
-        v4f a[Cfg::MT];
+    for (int mi = 0; mi < Cfg::MT; mi++)
+        f.a[mi] = *reinterpret_cast<const v4f *>(a_base + mi * 32 * Cfg::LDA);
+    if constexpr (Cfg::BSTYLE == STYLE_RC) {
 #pragma unroll
-        for (int mi = 0; mi < Cfg::MT; mi++)
-            a[mi] = *reinterpret_cast<const v4f *>(a_base + mi * 32 * Cfg::LDA + kk * 8);
-        if constexpr (Cfg::BSTYLE == STYLE_RC) {
-            constexpr int NG = Cfg::NT / 4;
-            v4f b[NG][4];
-#pragma unroll
-            for (int g = 0; g < NG; g++)
-#pragma unroll
-                for (int j = 0; j < 4; j++)
-                    b[g][j] = *reinterpret_cast<const v4f *>(
-                        Bs + (kk * 8 + j + 4 * lhi) * Cfg::LDB + wn * Cfg::TN + g * 128 + 4 * l32);
+        for (int g = 0; g < Cfg::NT / 4; g++)
 #pragma unroll
             for (int j = 0; j < 4; j++)
+                f.b[g * 4 + j] = *reinterpret_cast<const v4f *>(
+                    Bs + (kk * 8 + j + 4 * lhi) * Cfg::LDB + wn * Cfg::TN + g * 128 + 4 * l32);
+    } else {
+        const float *b_base = Bs + (wn * Cfg::TN + l32) * Cfg::LDB + 4 * lhi + kk * 8;
 #pragma unroll
-                for (int mi = 0; mi < Cfg::MT; mi++)
-#pragma unroll
-                    for (int g = 0; g < NG; g++)
-#pragma unroll
-                        for (int c = 0; c < 4; c++)
-                            acc.t[mi][g * 4 + c] = __builtin_amdgcn_mfma_f32_32x32x2f32(
-                                a[mi][j], b[g][j][c], acc.t[mi][g * 4 + c], 0, 0, 0);
-        } else {
-            const float *b_base = Bs + (wn * Cfg::TN + l32) * Cfg::LDB + 4 * lhi;
-            v4f b[Cfg::NT];
-#pragma unroll
-            for (int ni = 0; ni < Cfg::NT; ni++)
-                b[ni] = *reinterpret_cast<const v4f *>(b_base + ni * 32 * Cfg::LDB + kk * 8);
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-#pragma unroll
-                for (int mi = 0; mi < Cfg::MT; mi++)
-#pragma unroll
-                    for (int ni = 0; ni < Cfg::NT; ni++)
-                        acc.t[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(
-                            a[mi][j], b[ni][j], acc.t[mi][ni], 0, 0, 0);
-        }
+        for (int ni = 0; ni < Cfg::NT; ni++)
+            f.b[ni] = *reinterpret_cast<const v4f *>(b_base + ni * 32 * Cfg::LDB);
     }
 }
 
-// The pipelined mainloop.  ALoader/BLoader expose
-//   void fetch()                 issue the global loads of the next k-tile into registers
-//   void commit(float *stage)    write those registers into an LDS stage
-// and are constructed by the operator kernel for the block's tile origin.
+// The MFMAs of one k-slice of 8.  Consecutive MFMAs write different accumulator tiles.
+template <class Cfg>
+__device__ __forceinline__ void mma_frag(Accum<Cfg> &acc, const Frag<Cfg> &f) {
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int mi = 0; mi < Cfg::MT; mi++) {
+            if constexpr (Cfg::BSTYLE == STYLE_RC) {
+#pragma unroll
+                for (int g = 0; g < Cfg::NT / 4; g++)
+#pragma unroll
+                    for (int c = 0; c < 4; c++)
+                        acc.t[mi][g * 4 + c] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                            f.a[mi][j], f.b[g * 4 + j][c], acc.t[mi][g * 4 + c], 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int ni = 0; ni < Cfg::NT; ni++)
+                    acc.t[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                        f.a[mi][j], f.b[ni][j], acc.t[mi][ni], 0, 0, 0);
+            }
+        }
+}
+
+// Instruction classes of __builtin_amdgcn_sched_group_barrier.
+enum : int { SG_MFMA = 0x008, SG_VMEM_READ = 0x020, SG_DS_READ = 0x100, SG_DS_WRITE = 0x200 };
+
+// Ask the scheduler to emit `n_mem` memory instructions of class `mask` one at a time, each
+// followed by `mfma_between` MFMAs, so that a burst of loads or stores never holds up the
+// wave's in-order issue while the matrix pipe runs dry.
+#define T2SP_INTERLEAVE(mask, n_mem, mfma_between)                       \
+    _Pragma("unroll") for (int _i = 0; _i < (n_mem); _i++) {             \
+        __builtin_amdgcn_sched_group_barrier((mask), 1, 0);              \
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, (mfma_between), 0);\
+    }
+
+// The pipelined mainloop.  ALoader/BLoader expose, for register slot S in {0,1},
+//   void fetch<S>()                 issue the global loads of the next k-tile into slot S
+//   void commit<S>(float *stage)    write slot S into an LDS stage
+// and are constructed by the operator kernel for the block's tile origin and first k-tile.
+//
+// Software pipeline (KK = BK/8 slices per k-tile):
+//   * global -> registers runs two k-tiles ahead (two register slots), registers -> LDS one
+//     k-tile ahead (two LDS stages), LDS -> fragments one slice ahead (two fragment sets);
+//   * while slices 0..KK-2 of tile t are multiplied, tile t+2 is fetched, tile t+1 is written
+//     to the other LDS stage and the next slice's fragments are read; after the barrier the
+//     first fragments of tile t+1 are read while the last slice of tile t is multiplied;
+//   * loads and stores are interleaved one by one between MFMAs: a wave issues in order, so a
+//     burst of memory instructions that backs up in the address path would starve the MFMA pipe.
+template <class Cfg, int S, class ALoader, class BLoader>
+__device__ __forceinline__ void mainloop_body(Accum<Cfg> &acc, ALoader &la, BLoader &lb,
+                                              Frag<Cfg> (&frag)[2], float *smem, int wm, int wn,
+                                              int lane) {
+    constexpr int KK = Cfg::BK / 8;
+    constexpr int CUR = S;   // tile parity == LDS stage == register slot that held it
+    float *a_cur = smem + CUR * Cfg::A_STAGE, *a_nxt = smem + (CUR ^ 1) * Cfg::A_STAGE;
+    float *b_cur = smem + 2 * Cfg::A_STAGE + CUR * Cfg::B_STAGE;
+    float *b_nxt = smem + 2 * Cfg::A_STAGE + (CUR ^ 1) * Cfg::B_STAGE;
+    constexpr int MFMA_PER_SLICE = 4 * Cfg::MT * Cfg::NT;
+    constexpr int N_DS_READ = Cfg::MT + Cfg::NT;
+    constexpr int N_VMEM = Cfg::A_VEC + Cfg::B_VEC;
+    la.template fetch<S>();
+    lb.template fetch<S>();
+#pragma unroll
+    for (int kk = 0; kk < KK - 1; kk++) {
+        load_frag<Cfg>(frag[(kk + 1) & 1], a_cur, b_cur, kk + 1, wm, wn, lane);
+        mma_frag<Cfg>(acc, frag[kk & 1]);
+    }
+    la.template commit<S ^ 1>(a_nxt);
+    lb.template commit<S ^ 1>(b_nxt);
+    {
+        constexpr int N_MEM = 2 * N_VMEM + (KK - 1) * N_DS_READ;
+        constexpr int TOTAL = (KK - 1) * MFMA_PER_SLICE;
+        constexpr int GAP = TOTAL / N_MEM > 0 ? TOTAL / N_MEM : 1;
+        T2SP_INTERLEAVE(SG_DS_READ, N_DS_READ, GAP)
+        T2SP_INTERLEAVE(SG_VMEM_READ, N_VMEM, GAP)
+        T2SP_INTERLEAVE(SG_DS_READ, (KK - 2) * N_DS_READ, GAP)
+        T2SP_INTERLEAVE(SG_DS_WRITE, N_VMEM, GAP)
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    load_frag<Cfg>(frag[0], a_nxt, b_nxt, 0, wm, wn, lane);
+    mma_frag<Cfg>(acc, frag[(KK - 1) & 1]);
+    T2SP_INTERLEAVE(SG_DS_READ, N_DS_READ, 2)
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// `ktiles` must be even (callers round the reduction up to a pair of k-tiles; loaders return
+// zeros, or re-read valid data that is never multiplied, for tiles past the end).  fetch() is
+// called for two tiles past the last one and commit() for one.
 template <class Cfg, class ALoader, class BLoader>
 __device__ __forceinline__ void mainloop(Accum<Cfg> &acc, ALoader &la, BLoader &lb, int ktiles,
                                          float *smem) {
-    // Stage addresses are formed as offsets from the one LDS array so that the
-    // compiler keeps them in the LDS address space (ds_read/ds_write, lgkmcnt only).
-    auto a_stage = [&](int s) { return smem + s * Cfg::A_STAGE; };
-    auto b_stage = [&](int s) { return smem + 2 * Cfg::A_STAGE + s * Cfg::B_STAGE; };
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
     acc.clear();
-    la.fetch();
-    lb.fetch();
-    la.commit(a_stage(0));
-    lb.commit(b_stage(0));
+    la.template fetch<0>();
+    lb.template fetch<0>();
+    la.template commit<0>(smem);
+    lb.template commit<0>(smem + 2 * Cfg::A_STAGE);
+    la.template fetch<1>();
+    lb.template fetch<1>();
     __syncthreads();
-    for (int kt = 0; kt < ktiles; kt++) {
-        const int cur = kt & 1;
-        const bool more = kt + 1 < ktiles;
-        if (more) {
-            la.fetch();
-            lb.fetch();
-        }
-        mma_ktile<Cfg>(acc, a_stage(cur), b_stage(cur), wm, wn, lane);
-        if (more) {
-            la.commit(a_stage(cur ^ 1));
-            lb.commit(b_stage(cur ^ 1));
-        }
-        __syncthreads();
+    Frag<Cfg> frag[2];
+    load_frag<Cfg>(frag[0], smem, smem + 2 * Cfg::A_STAGE, 0, wm, wn, lane);
+    for (int kt = 0; kt < ktiles; kt += 2) {
+        mainloop_body<Cfg, 0>(acc, la, lb, frag, smem, wm, wn, lane);
+        mainloop_body<Cfg, 1>(acc, la, lb, frag, smem, wm, wn, lane);
     }
 }
 

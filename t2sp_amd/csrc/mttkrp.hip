@@ -45,12 +45,13 @@ struct MttkrpOutMap {
 template <class Cfg>
 struct TensorKcLoader {
     const float *p[Cfg::A_VEC];
+    const float *safe;
     bool ok[Cfg::A_VEC];
-    v4f reg[Cfg::A_VEC];
-    int kt, tiles_per_k;
+    v4f reg[2][Cfg::A_VEC];
+    int kt, tiles_per_k, total;
     int64_t sb_k;
     __device__ TensorKcLoader(const MttkrpArgs &g, int m0, int kt0)
-        : kt(kt0), tiles_per_k(g.J / Cfg::BK), sb_k(g.sb_k) {
+        : safe(g.B), kt(kt0), tiles_per_k(g.J / Cfg::BK), total(g.K * (g.J / Cfg::BK)), sb_k(g.sb_k) {
 #pragma unroll
         for (int i = 0; i < Cfg::A_VEC; i++) {
             KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
@@ -58,22 +59,21 @@ struct TensorKcLoader {
             p[i] = g.B + (int64_t)(ok[i] ? m0 + s.row : 0) * g.sb_i + s.k;
         }
     }
+    template <int S>
     __device__ __forceinline__ void fetch() {
-        const int k = kt / tiles_per_k, j0 = (kt - k * tiles_per_k) * Cfg::BK;
+        const bool in = kt < total;
+        const int t = in ? kt : 0;
+        const int k = t / tiles_per_k, j0 = (t - k * tiles_per_k) * Cfg::BK;
 #pragma unroll
-        for (int i = 0; i < Cfg::A_VEC; i++) {
-            if (ok[i])
-                reg[i] = *reinterpret_cast<const v4f *>(p[i] + k * sb_k + j0);
-            else
-                reg[i] = v4f{0.f, 0.f, 0.f, 0.f};
-        }
+        for (int i = 0; i < Cfg::A_VEC; i++) reg[S][i] = load_or_zero(p[i] + k * sb_k + j0, ok[i] && in, safe);
         kt++;
     }
+    template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
 #pragma unroll
         for (int i = 0; i < Cfg::A_VEC; i++) {
             KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
-            *reinterpret_cast<v4f *>(stage + s.row * Cfg::LDA + s.k) = reg[i];
+            *reinterpret_cast<v4f *>(stage + s.row * Cfg::LDA + s.k) = reg[S][i];
         }
     }
 };
@@ -84,13 +84,14 @@ template <class Cfg>
 struct KhatriRaoKcLoader {
     const float *pc[Cfg::B_VEC];
     const float *pd[Cfg::B_VEC];
+    const float *safe;
     bool ok[Cfg::B_VEC];
-    v4f reg[Cfg::B_VEC];
-    float dval[Cfg::B_VEC];
-    int kt, tiles_per_k;
+    v4f reg[2][Cfg::B_VEC];
+    float dval[2][Cfg::B_VEC];
+    int kt, tiles_per_k, total;
     int64_t sd_k;
     __device__ KhatriRaoKcLoader(const MttkrpArgs &g, int n0, int kt0)
-        : kt(kt0), tiles_per_k(g.J / Cfg::BK), sd_k(g.sd_k) {
+        : safe(g.C), kt(kt0), tiles_per_k(g.J / Cfg::BK), total(g.K * (g.J / Cfg::BK)), sd_k(g.sd_k) {
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
@@ -100,25 +101,24 @@ struct KhatriRaoKcLoader {
             pd[i] = g.D + (int64_t)r * g.sd_r;
         }
     }
+    template <int S>
     __device__ __forceinline__ void fetch() {
-        const int k = kt / tiles_per_k, j0 = (kt - k * tiles_per_k) * Cfg::BK;
+        const bool in = kt < total;
+        const int t = in ? kt : 0;
+        const int k = t / tiles_per_k, j0 = (t - k * tiles_per_k) * Cfg::BK;
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
-            if (ok[i]) {
-                reg[i] = *reinterpret_cast<const v4f *>(pc[i] + j0);
-                dval[i] = pd[i][k * sd_k];
-            } else {
-                reg[i] = v4f{0.f, 0.f, 0.f, 0.f};
-                dval[i] = 0.f;
-            }
+            reg[S][i] = load_or_zero(pc[i] + j0, ok[i] && in, safe);
+            dval[S][i] = pd[i][k * sd_k];
         }
         kt++;
     }
+    template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
-            *reinterpret_cast<v4f *>(stage + s.row * Cfg::LDB + s.k) = reg[i] * dval[i];
+            *reinterpret_cast<v4f *>(stage + s.row * Cfg::LDB + s.k) = reg[S][i] * dval[S][i];
         }
     }
 };
@@ -188,7 +188,7 @@ static MttkrpPlan plan_mttkrp(int I, int J, int K, int R, int cfg, int splits) {
         if (splits > ktiles / 16) splits = (int)(ktiles / 16);
         if (splits < 1) splits = 1;
     }
-    if (splits > ktiles) splits = (int)ktiles;
+    if (splits > (ktiles + 1) / 2) splits = (int)((ktiles + 1) / 2);
     p.cfg = cfg; p.splits = splits;
     p.Mp = (I + bm - 1) / bm * bm;
     p.Np = (R + bn - 1) / bn * bn;

@@ -13,11 +13,15 @@
 
 namespace t2sp {
 
-// k-tiles [begin, end) of split s out of S over `ktiles` tiles (sizes differ by at most one).
+// k-tiles [begin, end) of split s out of S over `ktiles` tiles.  Ranges are whole pairs of
+// tiles (the mainloop runs an even number); the last range may end one tile past `ktiles`, which
+// the loaders fill with zeros.  Sizes differ by at most one pair.
 __device__ __host__ inline void split_range(int ktiles, int S, int s, int &begin, int &end) {
-    const int base = ktiles / S, extra = ktiles % S;
-    begin = s * base + (s < extra ? s : extra);
-    end = begin + base + (s < extra ? 1 : 0);
+    const int pairs = (ktiles + 1) / 2;
+    const int base = pairs / S, extra = pairs % S;
+    const int b = s * base + (s < extra ? s : extra);
+    begin = 2 * b;
+    end = 2 * (b + base + (s < extra ? 1 : 0));
 }
 
 template <class Cfg>
