@@ -41,36 +41,56 @@ struct CapsuleOutMap {
     }
 };
 
-template <class Cfg>
+// Both loaders address their tensor with 32-bit element offsets from the base pointer:
+// a fixed per-slot part (the output row / column) plus the window walk over (ci,kh,kw).
+// KPAD: the reduction length is not a whole number of k-tile pairs, so slots past its end
+// must read as zero; otherwise tiles past the end are fetched but never multiplied and the
+// walk simply stops on the last tile.  Rows/columns outside the matrix read row/column 0:
+// whatever they accumulate is never stored.
+template <class Cfg, bool KPAD>
 struct PoseKcLoader {
-    const float *base[Cfg::A_VEC];
-    bool ok[Cfg::A_VEC];
+    int base_off[Cfg::A_VEC];
+    WindowSlot slot[Cfg::A_VEC];
     v4f reg[2][Cfg::A_VEC];
     int k0;
+    WindowParams wp;
     const CapsuleArgs &g;
-    __device__ PoseKcLoader(const CapsuleArgs &g_, int m0, int k_begin) : k0(k_begin), g(g_) {
+    __device__ PoseKcLoader(const CapsuleArgs &g_, int m0, int k_begin, const int *tab) : k0(k_begin), g(g_) {
+        wp.tab = tab;
+        wp.win = g.KH * g.KW;
+        wp.stride_c = (int)g.sp[1];
+        wp.step_r = (Cfg::BK / 4) % wp.win;
+        wp.step_coff = ((Cfg::BK / 4) / wp.win) * (int)g.sp[1];
 #pragma unroll
         for (int i = 0; i < Cfg::A_VEC; i++) {
             KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
             int row = m0 + s.row;
-            ok[i] = row < g.ROWS;
-            if (!ok[i]) row = 0;
+            if (row >= g.ROWS) row = 0;
             const int mx = row % g.MX, pix = row / g.MX;
             const int w = pix % g.OW, h = (pix / g.OW) % g.OH, n = pix / (g.OW * g.OH);
-            base[i] = g.P + n * g.sp[0] + (int64_t)h * g.S * g.sp[2] + (int64_t)w * g.S * g.sp[3] + mx * g.sp[4];
+            base_off[i] = (int)(n * g.sp[0] + h * g.S * g.sp[2] + w * g.S * g.sp[3] + mx * g.sp[4]);
+            int q = (k_begin + s.k) >> 2;
+            if (q >= g.KRED / 4) q = 0;
+            slot[i].init(wp, q);
         }
     }
     template <int S>
     __device__ __forceinline__ void fetch() {
+        const bool go = k0 + 2 * Cfg::BK <= g.KRED;
 #pragma unroll
         for (int i = 0; i < Cfg::A_VEC; i++) {
             KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
-            const int k = k0 + s.k;
-            const int q = k >> 2;                       // (ci, kh, kw)
-            const int kw = q % g.KW, kh = (q / g.KW) % g.KH, ci = q / (g.KW * g.KH);
-            reg[S][i] = load_or_zero(base[i] + ci * g.sp[1] + kh * g.sp[2] + kw * g.sp[3], ok[i] && k < g.KRED, g.P);
+            const uint32_t off = (uint32_t)(base_off[i] + slot[i].offset());
+            if (KPAD) {
+                const bool ok = k0 + s.k < g.KRED;
+                const v4f v = *reinterpret_cast<const v4f *>(g.P + (ok ? off : 0u));
+                reg[S][i] = ok ? v : v4f{0.f, 0.f, 0.f, 0.f};
+            } else {
+                reg[S][i] = *reinterpret_cast<const v4f *>(g.P + off);
+            }
+            slot[i].advance(wp, go);
         }
-        k0 += Cfg::BK;
+        k0 += (KPAD || go) ? Cfg::BK : 0;
     }
     template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
@@ -82,34 +102,48 @@ struct PoseKcLoader {
     }
 };
 
-template <class Cfg>
+template <class Cfg, bool KPAD>
 struct PoseWeightRcLoader {
-    const float *base[Cfg::B_VEC];
-    bool ok[Cfg::B_VEC];
+    int base_off[Cfg::B_VEC];
+    WindowSlot slot[Cfg::B_VEC];
     v4f reg[2][Cfg::B_VEC];
     int k0;
+    WindowParams wp;
     const CapsuleArgs &g;
-    __device__ PoseWeightRcLoader(const CapsuleArgs &g_, int n0, int k_begin) : k0(k_begin), g(g_) {
+    __device__ PoseWeightRcLoader(const CapsuleArgs &g_, int n0, int k_begin, const int *tab) : k0(k_begin), g(g_) {
+        wp.tab = tab;
+        wp.win = g.KH * g.KW;
+        wp.stride_c = (int)g.sw[1];
+        wp.step_r = (Cfg::BK / 4) % wp.win;
+        wp.step_coff = ((Cfg::BK / 4) / wp.win) * (int)g.sw[1];
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
-            const int col = n0 + s.col;
-            ok[i] = col < g.COLS;
-            base[i] = g.W + (ok[i] ? (col >> 2) : 0) * g.sw[0];
+            int col = n0 + s.col;
+            if (col >= g.COLS) col = 0;
+            base_off[i] = (int)((col >> 2) * g.sw[0] + ((k_begin + s.k) & 3) * g.sw[4]);
+            int q = (k_begin + s.k) >> 2;
+            if (q >= g.KRED / 4) q = 0;
+            slot[i].init(wp, q);
         }
     }
     template <int S>
     __device__ __forceinline__ void fetch() {
+        const bool go = k0 + 2 * Cfg::BK <= g.KRED;
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
-            const int k = k0 + s.k;
-            const int mk = k & 3, q = k >> 2;
-            const int kw = q % g.KW, kh = (q / g.KW) % g.KH, ci = q / (g.KW * g.KH);
-            reg[S][i] = load_or_zero(base[i] + ci * g.sw[1] + kh * g.sw[2] + kw * g.sw[3] + mk * g.sw[4],
-                                     ok[i] && k < g.KRED, g.W);
+            const uint32_t off = (uint32_t)(base_off[i] + slot[i].offset());
+            if (KPAD) {
+                const bool ok = k0 + s.k < g.KRED;
+                const v4f v = *reinterpret_cast<const v4f *>(g.W + (ok ? off : 0u));
+                reg[S][i] = ok ? v : v4f{0.f, 0.f, 0.f, 0.f};
+            } else {
+                reg[S][i] = *reinterpret_cast<const v4f *>(g.W + off);
+            }
+            slot[i].advance(wp, go);
         }
-        k0 += Cfg::BK;
+        k0 += (KPAD || go) ? Cfg::BK : 0;
     }
     template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
@@ -121,16 +155,21 @@ struct PoseWeightRcLoader {
     }
 };
 
-template <class Cfg>
+template <class Cfg, bool KPAD>
 __global__ void __launch_bounds__(Cfg::NTHREADS) capsule_kernel(const CapsuleArgs g) {
     extern __shared__ __align__(16) float smem[];
+    int *tab_p = reinterpret_cast<int *>(smem + Cfg::SMEM_FLOATS);
+    int *tab_w = tab_p + g.KH * g.KW;
+    fill_window_table(tab_p, g.KH, g.KW, (int)g.sp[2], (int)g.sp[3]);
+    fill_window_table(tab_w, g.KH, g.KW, (int)g.sw[2], (int)g.sw[3]);
+    __syncthreads();
     const int tile = blockIdx.x / g.splits, split = blockIdx.x % g.splits;
     const int tm = tile / g.tiles_n, tn = tile % g.tiles_n;
     const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
     int kt0, kt1;
     split_range((g.KRED + Cfg::BK - 1) / Cfg::BK, g.splits, split, kt0, kt1);
-    PoseKcLoader<Cfg> la(g, m0, kt0 * Cfg::BK);
-    PoseWeightRcLoader<Cfg> lb(g, n0, kt0 * Cfg::BK);
+    PoseKcLoader<Cfg, KPAD> la(g, m0, kt0 * Cfg::BK, tab_p);
+    PoseWeightRcLoader<Cfg, KPAD> lb(g, n0, kt0 * Cfg::BK, tab_w);
     Accum<Cfg> acc;
     mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem);
     if (g.splits == 1) {
@@ -211,8 +250,8 @@ template <class Cfg>
 static int launch_capsule(CapsuleArgs g, hipStream_t stream) {
     g.tiles_m = g.Mp / Cfg::BM;
     g.tiles_n = g.Np / Cfg::BN;
-    const size_t smem = Cfg::SMEM_FLOATS * sizeof(float);
-    auto kern = capsule_kernel<Cfg>;
+    const size_t smem = Cfg::SMEM_FLOATS * sizeof(float) + 2 * (size_t)g.KH * g.KW * sizeof(int);
+    auto kern = (g.KRED % (2 * Cfg::BK)) ? capsule_kernel<Cfg, true> : capsule_kernel<Cfg, false>;
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * g.splits), dim3(Cfg::NTHREADS), smem, stream, g);
@@ -230,7 +269,14 @@ static int launch_capsule(CapsuleArgs g, hipStream_t stream) {
 static bool capsule_fast(const int *d, const int64_t *sp6, const int64_t *sw6, const int64_t *sv6,
                          const float *P, const float *W, const float *V) {
     const int MY = d[9], MK = d[10];
-    if (MY != 4 || MK != 4) return false;
+    if (MY != 4 || MK != 4 || d[5] * d[6] > 4096) return false;
+    // 32-bit element offsets: every tensor must span fewer than 2^31 elements
+    const int64_t span_p = (int64_t)(d[0] - 1) * sp6[0] + (int64_t)(d[1] - 1) * sp6[1] +
+                           (int64_t)((d[3] - 1) * d[7] + d[5] - 1) * sp6[2] +
+                           (int64_t)((d[4] - 1) * d[7] + d[6] - 1) * sp6[3] + (int64_t)(d[8] - 1) * sp6[4] + 3;
+    const int64_t span_w = (int64_t)(d[2] - 1) * sw6[0] + (int64_t)(d[1] - 1) * sw6[1] + (int64_t)(d[5] - 1) * sw6[2] +
+                           (int64_t)(d[6] - 1) * sw6[3] + 3 * sw6[4] + 3;
+    if (span_p >= INT32_MAX || span_w >= INT32_MAX) return false;
     if (sp6[5] != 1 || sw6[5] != 1 || sv6[5] != 1) return false;
     for (int i = 0; i < 5; i++)
         if (sp6[i] % 4 || sw6[i] % 4 || sv6[i] % 4) return false;

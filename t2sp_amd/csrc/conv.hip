@@ -22,23 +22,31 @@ struct ConvArgs {
     const float *I, *W;
     float *O;
     int N, CI, CO, OH, OW, KH, KW;
-    int64_t si_n, si_c, si_h;   // input strides (w stride is 1)
+    int si_n, si_c, si_h;       // input strides in elements (w stride is 1); the input spans < 2^31 elements
     int64_t sw_o;               // weight stride of co (ci,kh,kw are dense)
     int64_t so_n, so_c, so_h;   // output strides (w stride is 1)
     int P, KRED;                // N*OH*OW, CI*KH*KW
     int tiles_m, tiles_n, group_m;
+    int p_begin;                // first output pixel this launch covers
 };
 
 // Input operand: for reduction row k = (ci,kh,kw) and 4 consecutive output pixels of one image
 // row, the 4 input pixels at (ci, h+kh, w+kw .. w+kw+3).
 template <class Cfg, bool EDGE>
 struct Im2colRcLoader {
-    const float *base[Cfg::B_VEC];   // pixel part of the address (n, h, w), fixed for the block
+    int base_off[Cfg::B_VEC];        // pixel part of the element offset (n, h, w), fixed for the block
     bool col_ok[Cfg::B_VEC];
+    WindowSlot slot[Cfg::B_VEC];     // window part of the reduction row this slot loads next
     v4f reg[2][Cfg::B_VEC];
     int k0;                          // first reduction row of the tile fetched next
+    WindowParams wp;
     const ConvArgs &g;
-    __device__ Im2colRcLoader(const ConvArgs &g_, int p0) : k0(0), g(g_) {
+    __device__ Im2colRcLoader(const ConvArgs &g_, int p0, const int *tab) : k0(0), g(g_) {
+        wp.tab = tab;
+        wp.win = g.KH * g.KW;
+        wp.stride_c = g.si_c;
+        wp.step_r = Cfg::BK % wp.win;
+        wp.step_coff = (Cfg::BK / wp.win) * g.si_c;
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
@@ -48,28 +56,27 @@ struct Im2colRcLoader {
             const int hw = g.OH * g.OW;
             const int n = p / hw, rem = p - n * hw;
             const int h = rem / g.OW, w = rem - h * g.OW;
-            base[i] = g.I + n * g.si_n + h * g.si_h + w;
+            base_off[i] = n * g.si_n + h * g.si_h + w;
+            slot[i].init(wp, s.k);
         }
     }
     template <int S>
     __device__ __forceinline__ void fetch() {
-        const int khw = g.KH * g.KW;
+        const bool go = EDGE || k0 + 2 * Cfg::BK <= g.KRED;
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
-            const int k = k0 + s.k;
-            const int ci = k / khw, r = k - ci * khw;
-            const int kh = r / g.KW, kw = r - kh * g.KW;
-            const float *ptr = base[i] + ci * g.si_c + kh * g.si_h + kw;
+            const uint32_t off = (uint32_t)(base_off[i] + slot[i].offset());
             if (EDGE) {
-                const bool ok = col_ok[i] && k < g.KRED;
-                const v4f_u v = *reinterpret_cast<const v4f_u *>(ok ? ptr : g.I);
+                const bool ok = col_ok[i] && k0 + s.k < g.KRED;
+                const v4f_u v = *reinterpret_cast<const v4f_u *>(g.I + (ok ? off : 0u));
                 reg[S][i] = ok ? (v4f)v : v4f{0.f, 0.f, 0.f, 0.f};
             } else {
-                reg[S][i] = *reinterpret_cast<const v4f_u *>(ptr);
+                reg[S][i] = *reinterpret_cast<const v4f_u *>(g.I + off);
             }
+            slot[i].advance(wp, go);
         }
-        k0 += (EDGE || k0 + 2 * Cfg::BK <= g.KRED) ? Cfg::BK : 0;
+        k0 += go ? Cfg::BK : 0;
     }
     template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
@@ -84,11 +91,14 @@ struct Im2colRcLoader {
 template <class Cfg, bool EDGE>
 __global__ void __launch_bounds__(Cfg::NTHREADS) conv_kernel(const ConvArgs g) {
     extern __shared__ __align__(16) float smem[];
+    int *tab = reinterpret_cast<int *>(smem + Cfg::SMEM_FLOATS);
+    fill_window_table(tab, g.KH, g.KW, g.si_h, 1);
+    __syncthreads();
     int tm, tn;
     tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, g.group_m, tm, tn);
-    const int co0 = tm * Cfg::BM, p0 = tn * Cfg::BN;
+    const int co0 = tm * Cfg::BM, p0 = g.p_begin + tn * Cfg::BN;
     RowMajorKcLoader<Cfg, EDGE> la(g.W, g.sw_o, co0, g.CO, g.KRED);
-    Im2colRcLoader<Cfg, EDGE> lb(g, p0);
+    Im2colRcLoader<Cfg, EDGE> lb(g, p0, tab);
     Accum<Cfg> acc;
     mainloop<Cfg>(acc, la, lb, ktiles_even<Cfg>(g.KRED), smem);
     const int hw = g.OH * g.OW;
@@ -124,13 +134,16 @@ __global__ void conv_scalar_kernel(const ConvGenericArgs g) {
     }
 }
 
+// Launches the tiles covering output pixels [p_begin, p_end); p_begin is a multiple of BN.
 template <class Cfg>
-static int launch_conv(ConvArgs g, hipStream_t stream) {
+static int launch_conv(ConvArgs g, int p_begin, int p_end, hipStream_t stream) {
+    if (p_end <= p_begin) return T2SP_OK;
+    g.p_begin = p_begin;
     g.tiles_m = (g.CO + Cfg::BM - 1) / Cfg::BM;
-    g.tiles_n = (g.P + Cfg::BN - 1) / Cfg::BN;
+    g.tiles_n = (p_end - p_begin + Cfg::BN - 1) / Cfg::BN;
     g.group_m = g.tiles_m;   // all output channels of a pixel tile run together: the input tile is shared in L2
-    const bool edge = (g.CO % Cfg::BM) || (g.P % Cfg::BN) || (g.KRED % (2 * Cfg::BK));
-    const size_t smem = Cfg::SMEM_FLOATS * sizeof(float);
+    const bool edge = (g.CO % Cfg::BM) || ((p_end - p_begin) % Cfg::BN) || (g.KRED % (2 * Cfg::BK));
+    const size_t smem = Cfg::SMEM_FLOATS * sizeof(float) + (size_t)g.KH * g.KW * sizeof(int);
     auto kern = edge ? conv_kernel<Cfg, true> : conv_kernel<Cfg, false>;
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)smem) != hipSuccess)
@@ -152,35 +165,49 @@ extern "C" int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, 
     if (N <= 0 || CI <= 0 || CO <= 0 || OH <= 0 || OW <= 0 || KH <= 0 || KW <= 0 || !si4 || !sw4 || !so4)
         return T2SP_ERR_SHAPE;
     if ((int64_t)N * OH * OW > INT32_MAX || (int64_t)CI * KH * KW > INT32_MAX) return T2SP_ERR_SHAPE;
+    const int64_t in_span = (int64_t)(N - 1) * si4[0] + (int64_t)(CI - 1) * si4[1] +
+                            (int64_t)(OH + KH - 2) * si4[2] + (OW + KW - 2);
     const bool fast = cfg != T2SP_CFG_SCALAR && si4[3] == 1 && so4[3] == 1 && sw4[3] == 1 &&
                       sw4[2] == KW && sw4[1] == (int64_t)KH * KW && sw4[0] % 4 == 0 && OW % 4 == 0 &&
-                      (CI * KH * KW) % 4 == 0 && so4[0] % 4 == 0 && so4[1] % 4 == 0 && so4[2] % 4 == 0 &&
+                      (CI * KH * KW) % 4 == 0 && KH * KW <= 4096 && in_span < INT32_MAX &&
+                      so4[0] % 4 == 0 && so4[1] % 4 == 0 && so4[2] % 4 == 0 &&
                       ((uintptr_t)W % 16 == 0) && ((uintptr_t)O % 16 == 0) && ((uintptr_t)I % 4 == 0);
+    hipStream_t st = (hipStream_t)stream;
     if (!fast) {
         ConvGenericArgs a{I, W, O, N, CI, CO, OH, OW, KH, KW, {}, {}, {}};
         for (int d = 0; d < 4; d++) { a.si[d] = si4[d]; a.sw[d] = sw4[d]; a.so[d] = so4[d]; }
         const int64_t total = (int64_t)N * CO * OH * OW;
         const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
-        hipLaunchKernelGGL(conv_scalar_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+        hipLaunchKernelGGL(conv_scalar_kernel, dim3(blocks), dim3(256), 0, st, a);
         return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
     }
     ConvArgs g{};
     g.I = I; g.W = W; g.O = O;
     g.N = N; g.CI = CI; g.CO = CO; g.OH = OH; g.OW = OW; g.KH = KH; g.KW = KW;
-    g.si_n = si4[0]; g.si_c = si4[1]; g.si_h = si4[2];
+    g.si_n = (int)si4[0]; g.si_c = (int)si4[1]; g.si_h = (int)si4[2];
     g.sw_o = sw4[0];
     g.so_n = so4[0]; g.so_c = so4[1]; g.so_h = so4[2];
     g.P = N * OH * OW; g.KRED = CI * KH * KW;
-    if (cfg == T2SP_CFG_AUTO) {
-        auto tiles = [&](int bm, int bn) { return (int64_t)((CO + bm - 1) / bm) * ((g.P + bn - 1) / bn); };
-        if (tiles(256, 256) >= 200) cfg = T2SP_CFG_256x256;
-        else if (tiles(128, 128) >= 200) cfg = T2SP_CFG_128x128;
-        else cfg = T2SP_CFG_64x128;
-    }
     switch (cfg) {
-        case T2SP_CFG_256x256: return launch_conv<ConvL>(g, (hipStream_t)stream);
-        case T2SP_CFG_128x128: return launch_conv<ConvM>(g, (hipStream_t)stream);
-        case T2SP_CFG_64x128: return launch_conv<ConvS>(g, (hipStream_t)stream);
+        case T2SP_CFG_256x256: return launch_conv<ConvL>(g, 0, g.P, st);
+        case T2SP_CFG_128x128: return launch_conv<ConvM>(g, 0, g.P, st);
+        case T2SP_CFG_64x128: return launch_conv<ConvS>(g, 0, g.P, st);
+        case T2SP_CFG_AUTO: break;
         default: return T2SP_ERR_SHAPE;
     }
+    // Automatic choice.  One 256x256 tile occupies a CU, so big tiles run in rounds of 256 (the
+    // CU count); a partial last round would leave most CUs idle for a whole tile time.  Whole
+    // rounds of big tiles are therefore launched first and the remaining pixels are covered with
+    // 128x128 tiles (several per CU), which finish in a fraction of a round.
+    constexpr int CUS = 256;
+    const int tiles_m = (CO + 255) / 256;
+    const int rounds = (int)(((int64_t)tiles_m * (g.P / 256)) / CUS);
+    if (CO >= 256 && CUS % tiles_m == 0 && rounds >= 1) {
+        const int p_split = rounds * (CUS / tiles_m) * 256;
+        const int rc = launch_conv<ConvL>(g, 0, p_split, st);
+        if (rc != T2SP_OK) return rc;
+        return launch_conv<ConvM>(g, p_split, g.P, st);
+    }
+    if ((int64_t)((CO + 127) / 128) * ((g.P + 127) / 128) >= 128) return launch_conv<ConvM>(g, 0, g.P, st);
+    return launch_conv<ConvS>(g, 0, g.P, st);
 }

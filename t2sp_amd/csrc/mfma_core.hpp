@@ -73,6 +73,46 @@ __device__ __forceinline__ V load_or_zero(const float *ptr, bool valid, const fl
     return valid ? v : V{0.f, 0.f, 0.f, 0.f};
 }
 
+// Division-free, multiply-free walk over a reduction index q = c * WIN + r, r = kh * KW + kw,
+// that advances by a fixed step per k-tile (convolution windows).  The element offset of q is
+//     c * stride_c + tab[r],   tab[r] = (r / KW) * stride_h + (r % KW) * stride_w,
+// with `tab` a small table in LDS filled once per workgroup.  A loader slot keeps r, the
+// running c * stride_c and the table entry of its next fetch, and updates them with a few
+// 32-bit adds and one LDS read per k-tile.  (Integer division and 64-bit address arithmetic
+// per slot per k-tile cost as much issue time as the MFMAs themselves on small tiles.)
+struct WindowParams {
+    const int *tab;     // LDS, `win` entries
+    int win;            // KH * KW
+    int stride_c;
+    int step_r;         // (q step per k-tile) % win
+    int step_coff;      // (q step per k-tile) / win * stride_c
+};
+struct WindowSlot {
+    int r, coff, woff;
+    __device__ __forceinline__ void init(const WindowParams &w, int q) {
+        const int c = q / w.win;
+        r = q - c * w.win;
+        coff = c * w.stride_c;
+        woff = w.tab[r];
+    }
+    __device__ __forceinline__ int offset() const { return coff + woff; }
+    // `go` is uniform: false once the next tile would lie past the end of the reduction
+    __device__ __forceinline__ void advance(const WindowParams &w, bool go) {
+        r += go ? w.step_r : 0;
+        coff += go ? w.step_coff : 0;
+        const bool wrap = r >= w.win;
+        r -= wrap ? w.win : 0;
+        coff += wrap ? w.stride_c : 0;
+        woff = w.tab[r];
+    }
+};
+// Fill the window table; call from every thread before the first __syncthreads().
+__device__ __forceinline__ void fill_window_table(int *tab, int kh_extent, int kw_extent, int stride_h,
+                                                  int stride_w) {
+    for (int r = threadIdx.x; r < kh_extent * kw_extent; r += blockDim.x)
+        tab[r] = (r / kw_extent) * stride_h + (r % kw_extent) * stride_w;
+}
+
 // Position, inside a KC tile of ROWS x BK, of the f-th float4 of the tile.
 template <int BK>
 struct KcSlot {
