@@ -28,6 +28,10 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3   # 256 CU x 256 flop/clk/CU x 2.4 GHz
 PEAK_HBM_GBS = 8000.0
+# Bytes the L2s fetch from / write to the fabric per SGEMM 8192^3 launch: rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (two runs of this script with --calibrate-copy), each scaled by what the same counter reads
+# for the 256 MiB calibration copy (x1.999 and x1.000); summary in profiles/all_kernels_hbm_traffic_pmc.md.
+SGEMM_8192_TRAFFIC_BYTES = 3.49e9
 
 
 def parse():
@@ -38,6 +42,9 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-others", action="store_true", help="skip the non-headline configurations")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="first run a plain device copy of 256 MiB three times (a kernel of known HBM traffic, "
+                         "used to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
     return ap.parse_args()
 
 
@@ -121,6 +128,18 @@ def main():
         sys.exit(1)
     t2sp_amd.lib()
 
+    if args.calibrate_copy:
+        import ctypes
+        n = 64 * 1024 * 1024
+        src, dst = torch.ones(n, device="cuda"), torch.empty(n, device="cuda")
+        ext, st = (ctypes.c_int * 1)(n), (ctypes.c_int64 * 1)(1)
+        for _ in range(3):
+            rc = t2sp_amd.lib().t2sp_relayout_f32(src.data_ptr(), dst.data_ptr(), 1, ext, st, st,
+                                                  torch.cuda.current_stream().cuda_stream)
+            assert rc == 0
+        torch.cuda.synchronize()
+        del src, dst
+
     M = N = K = 8192
     r = sgemm_case(torch, t2sp_amd, M, N, K, args.steps, args.warmup)
     tflops = r["flop"] / (r["wall_ms"] * 1e-3) / 1e12
@@ -135,7 +154,8 @@ def main():
                    "entry": "t2sp_sgemm_f32", "inputs": "resident in HBM"},
         "pct_of_peak": round(100.0 * tflops / PEAK_FP32_MFMA_TFLOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 3), "peak": PEAK_FP32_MFMA_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(kernel_tflops / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+                     "unit": "TFLOP/s", "frac": round(kernel_tflops / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": SGEMM_8192_TRAFFIC_BYTES,
+                     "traffic_note": "bytes per launch, L2<->fabric, from rocprofv3 FETCH_SIZE+WRITE_SIZE scaled by a copy kernel; algorithmic 8.05e8",
                      "kernel": "sgemm_kernel<256x256x16>", "avg_launch_ms": round(r["avg_ms"], 4),
                      "best_launch_ms": round(r["min_ms"], 4), "flop_per_launch": r["flop"]},
     }
@@ -153,14 +173,14 @@ def main():
     if not args.no_others:
         others = {}
         for (m, n, k) in [(4096, 16384, 2048), (16384, 4096, 8192), (1024, 1024, 1024)]:
-            c = sgemm_case(torch, t2sp_amd, m, n, k, max(5, args.steps // 2), 2)
+            c = sgemm_case(torch, t2sp_amd, m, n, k, max(5, args.steps // 2), 5)
             tf = c["flop"] / (c["avg_ms"] * 1e-3) / 1e12
             others["sgemm_%dx%dx%d" % (m, n, k)] = {"TFLOP/s": round(tf, 3), "frac_of_peak": round(tf / PEAK_FP32_MFMA_TFLOPS, 4),
                                                     "avg_launch_ms": round(c["avg_ms"], 4)}
             del c
         try:
             from t2sp_amd import bench_ops
-            others.update(bench_ops.run_all(torch, max(5, args.steps // 2), 2, PEAK_FP32_MFMA_TFLOPS))
+            others.update(bench_ops.run_all(torch, max(5, args.steps // 2), 5, PEAK_FP32_MFMA_TFLOPS))
         except ImportError:
             pass
         out["others"] = others
