@@ -113,11 +113,24 @@ __device__ __forceinline__ void fill_window_table(int *tab, int kh_extent, int k
         tab[r] = (r / kw_extent) * stride_h + (r % kw_extent) * stride_w;
 }
 
-// Position, inside a KC tile of ROWS x BK, of the f-th float4 of the tile.
+// Position, inside a KC tile of ROWS x BK, of the f-th float4 of the tile.  With BK = 16 a row
+// is 4 float4, so the 8 lanes that a 128-bit LDS write serves per cycle cover two rows; rows r
+// and r+1 are 20 floats apart and their 16-bank windows overlap, rows r and r+4 (80 floats = 16
+// banks apart) do not.  Slots are therefore dealt to rows in the order 0,4,1,5,2,6,3,7 inside
+// every block of 8 rows.  The global side is unaffected: a row is still 4 adjacent lanes.
 template <int BK>
 struct KcSlot {
     int row, k;
-    __device__ explicit KcSlot(int f) : row(f / (BK / 4)), k((f % (BK / 4)) * 4) {}
+    __device__ explicit KcSlot(int f) {
+        if constexpr (BK == 16) {
+            const int j = (f >> 2) & 7;
+            row = ((f >> 5) << 3) + (j >> 1) + ((j & 1) << 2);
+            k = (f & 3) << 2;
+        } else {
+            row = f / (BK / 4);
+            k = (f % (BK / 4)) * 4;
+        }
+    }
 };
 // Position, inside an RC tile of BK x COLS, of the f-th float4.
 template <int COLS>
