@@ -30,6 +30,7 @@ extern "C" {
 #define T2SP_CFG_256x256 1
 #define T2SP_CFG_128x128 2
 #define T2SP_CFG_64x128 3
+#define T2SP_CFG_32x128 4 /* one wavefront per tile: for problems with few outputs */
 #define T2SP_CFG_SCALAR 99
 
 #define T2SP_MAX_DIMS 10

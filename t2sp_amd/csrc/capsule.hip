@@ -215,6 +215,7 @@ __global__ void capsule_scalar_kernel(const CapsuleGenericArgs g) {
 using CapsM = TileCfg<128, 128, 16, 4, 1, STYLE_RC>;
 using CapsS = TileCfg<64, 128, 16, 2, 1, STYLE_RC>;
 using CapsL = TileCfg<256, 256, 16, 4, 2, STYLE_RC>;
+using CapsW = TileCfg<32, 128, 16, 1, 1, STYLE_RC>;   // one wave per tile
 
 struct CapsulePlan {
     int cfg, splits, Mp, Np;
@@ -228,7 +229,7 @@ static CapsulePlan plan_capsule(int rows, int cols, int kred, int cfg, int split
         const int64_t t256 = (int64_t)((rows + 255) / 256) * ((cols + 255) / 256);
         cfg = (t256 >= 200 && cols > 128) ? T2SP_CFG_256x256 : (t128 >= 24 ? T2SP_CFG_128x128 : T2SP_CFG_64x128);
     }
-    const int bm = cfg == T2SP_CFG_256x256 ? 256 : cfg == T2SP_CFG_128x128 ? 128 : 64;
+    const int bm = cfg == T2SP_CFG_256x256 ? 256 : cfg == T2SP_CFG_128x128 ? 128 : cfg == T2SP_CFG_64x128 ? 64 : 32;
     const int bn = cfg == T2SP_CFG_256x256 ? 256 : 128;
     const int tiles = ((rows + bm - 1) / bm) * ((cols + bn - 1) / bn);
     const int ktiles = (kred + 15) / 16;
@@ -322,6 +323,7 @@ extern "C" int t2sp_capsule_f32(const float *P, const float *W, float *V, const 
         case T2SP_CFG_256x256: return launch_capsule<CapsL>(g, (hipStream_t)stream);
         case T2SP_CFG_128x128: return launch_capsule<CapsM>(g, (hipStream_t)stream);
         case T2SP_CFG_64x128: return launch_capsule<CapsS>(g, (hipStream_t)stream);
+        case T2SP_CFG_32x128: return launch_capsule<CapsW>(g, (hipStream_t)stream);
         default: return T2SP_ERR_SHAPE;
     }
 }

@@ -45,8 +45,17 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *scratch
     const size_t groups = plane / 4;
     for (size_t g = (size_t)blockIdx.x * blockDim.x + threadIdx.x; g < groups;
          g += (size_t)gridDim.x * blockDim.x) {
-        v4f sum = *reinterpret_cast<const v4f *>(scratch + g * 4);
-        for (int s = 1; s < S; s++) sum += *reinterpret_cast<const v4f *>(scratch + s * plane + g * 4);
+        const float *p = scratch + g * 4;
+        v4f sum = *reinterpret_cast<const v4f *>(p);
+        int s = 1;
+        for (; s + 3 < S; s += 4) {   // four loads in flight; the additions stay in ascending order
+            const v4f a = *reinterpret_cast<const v4f *>(p + (size_t)s * plane);
+            const v4f b = *reinterpret_cast<const v4f *>(p + (size_t)(s + 1) * plane);
+            const v4f c = *reinterpret_cast<const v4f *>(p + (size_t)(s + 2) * plane);
+            const v4f d = *reinterpret_cast<const v4f *>(p + (size_t)(s + 3) * plane);
+            sum = (((sum + a) + b) + c) + d;
+        }
+        for (; s < S; s++) sum += *reinterpret_cast<const v4f *>(p + (size_t)s * plane);
         int row, col;
         if (ALONG_COLS) {
             row = (int)(g / (Np / 4));
