@@ -55,12 +55,16 @@ int t2sp_sgemm_f32_tiled(const float *A, const float *B, float *C, int M, int N,
  * padding, fp32.  si4/sw4/so4 are element strides of the logical indices
  * (n,ci,h,w), (co,ci,kh,kw), (n,co,h,w); "w" is the innermost spatial axis (the
  * one the reference calls y).  Dense NCHW/OIHW with OW % 4 == 0 takes the
- * implicit-GEMM MFMA kernel, anything else a scalar kernel.  Replaces the device
+ * implicit-GEMM MFMA kernel, anything else a scalar kernel.  `workspace` (optional, may be
+ * NULL; t2sp_conv2d_workspace_bytes gives its size) lets the last, partial round of tiles split
+ * its reduction over all CUs.  Replaces the device
  * side of the reference's conv pipeline (t2s/tests/performance/conv/conv.cpp:59-65,
  * conv/bitstream/a10/a.cl). */
+size_t t2sp_conv2d_workspace_bytes(int N, int CI, int CO, int OH, int OW, int KH, int KW);
 int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, int CI, int CO, int OH,
                     int OW, int KH, int KW, const int64_t *si4, const int64_t *sw4,
-                    const int64_t *so4, int cfg, void *stream);
+                    const int64_t *so4, int cfg, float *workspace, size_t workspace_bytes,
+                    void *stream);
 
 /* V[n,co,h,w,mx,my] = sum_{ci,kh,kw,mk} P[n,ci,S*h+kh,S*w+kw,mx,mk] * W[co,ci,kh,kw,mk,my].
  * dims11 = {N, CI, CO, OH, OW, KH, KW, S, MX, MY, MK}; sp6/sw6/sv6 are element strides of the

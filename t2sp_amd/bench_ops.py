@@ -43,9 +43,12 @@ def conv_config3(torch, steps, warmup, peak):
     O = torch.empty(N, CO, OH, OW, device="cuda")
     s = torch.cuda.current_stream().cuda_stream
     si, sw, so = ((i64 * 4)(*t.stride()) for t in (I, W, O))
+    nbytes = L.t2sp_conv2d_workspace_bytes(N, CI, CO, OH, OW, 3, 3)
+    ws = torch.empty(max(nbytes // 4, 1), device="cuda")
 
     def launch():
-        rc = L.t2sp_conv2d_f32(I.data_ptr(), W.data_ptr(), O.data_ptr(), N, CI, CO, OH, OW, 3, 3, si, sw, so, 0, s)
+        rc = L.t2sp_conv2d_f32(I.data_ptr(), W.data_ptr(), O.data_ptr(), N, CI, CO, OH, OW, 3, 3, si, sw, so, 0,
+                               ws.data_ptr(), nbytes, s)
         assert rc == 0, rc
 
     ms = _time(torch, launch, steps, warmup)

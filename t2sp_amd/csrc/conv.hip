@@ -12,6 +12,7 @@
 // "w" is the innermost spatial axis of the buffers (the one the reference calls y).
 #include "mfma_core.hpp"
 #include "gemm_loaders.hpp"
+#include "splitk.hpp"
 #include "t2sp_hip.h"
 
 namespace t2sp {
@@ -28,6 +29,23 @@ struct ConvArgs {
     int P, KRED;                // N*OH*OW, CI*KH*KW
     int tiles_m, tiles_n, group_m;
     int p_begin;                // first output pixel this launch covers
+    int splits;                 // workgroups per tile along the reduction (1 = none)
+    int Mp, Np;                 // padded extents of one partial plane (CO, pixels of this launch)
+    float *scratch;
+};
+
+struct ConvOutMap {
+    float *O;
+    int CO, P, OH, OW, p_begin;
+    int64_t so_n, so_c, so_h;
+    __device__ __forceinline__ void store(int row, int col, v4f v) const {
+        const int p = p_begin + col;
+        if (row >= CO || p >= P) return;
+        const int hw = OH * OW;
+        const int n = p / hw, rem = p - n * hw;
+        const int h = rem / OW, w = rem - h * OW;
+        *reinterpret_cast<v4f *>(O + n * so_n + row * so_c + h * so_h + w) = v;
+    }
 };
 
 // Input operand: for reduction row k = (ci,kh,kw) and 4 consecutive output pixels of one image
@@ -41,7 +59,7 @@ struct Im2colRcLoader {
     int k0;                          // first reduction row of the tile fetched next
     WindowParams wp;
     const ConvArgs &g;
-    __device__ Im2colRcLoader(const ConvArgs &g_, int p0, const int *tab) : k0(0), g(g_) {
+    __device__ Im2colRcLoader(const ConvArgs &g_, int p0, const int *tab, int k_begin) : k0(k_begin), g(g_) {
         wp.tab = tab;
         wp.win = g.KH * g.KW;
         wp.stride_c = g.si_c;
@@ -57,7 +75,7 @@ struct Im2colRcLoader {
             const int n = p / hw, rem = p - n * hw;
             const int h = rem / g.OW, w = rem - h * g.OW;
             base_off[i] = n * g.si_n + h * g.si_h + w;
-            slot[i].init(wp, s.k);
+            slot[i].init(wp, (k_begin + s.k < g.KRED) ? k_begin + s.k : 0);
         }
     }
     template <int S>
@@ -94,13 +112,20 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) conv_kernel(const ConvArgs g) {
     int *tab = reinterpret_cast<int *>(smem + Cfg::SMEM_FLOATS);
     fill_window_table(tab, g.KH, g.KW, g.si_h, 1);
     __syncthreads();
+    const int tile = blockIdx.x / g.splits, split = blockIdx.x - tile * g.splits;
     int tm, tn;
-    tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, g.group_m, tm, tn);
+    tile_coords(tile, g.tiles_m, g.tiles_n, g.group_m, tm, tn);
     const int co0 = tm * Cfg::BM, p0 = g.p_begin + tn * Cfg::BN;
-    RowMajorKcLoader<Cfg, EDGE> la(g.W, g.sw_o, co0, g.CO, g.KRED);
-    Im2colRcLoader<Cfg, EDGE> lb(g, p0, tab);
+    int kt0 = 0, kt1 = ktiles_even<Cfg>(g.KRED);
+    if (g.splits > 1) split_range((g.KRED + Cfg::BK - 1) / Cfg::BK, g.splits, split, kt0, kt1);
+    RowMajorKcLoader<Cfg, EDGE> la(g.W, g.sw_o, co0, g.CO, g.KRED, kt0 * Cfg::BK);
+    Im2colRcLoader<Cfg, EDGE> lb(g, p0, tab, kt0 * Cfg::BK);
     Accum<Cfg> acc;
-    mainloop<Cfg>(acc, la, lb, ktiles_even<Cfg>(g.KRED), smem);
+    mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem);
+    if (g.splits > 1) {
+        store_partial<Cfg>(acc, g.scratch, split, co0, p0 - g.p_begin, g.Mp, g.Np);
+        return;
+    }
     const int hw = g.OH * g.OW;
     drain<Cfg>(acc, [&](int row, int col, v4f v) {
         const int co = co0 + row, p = p0 + col;
@@ -135,21 +160,63 @@ __global__ void conv_scalar_kernel(const ConvGenericArgs g) {
 }
 
 // Launches the tiles covering output pixels [p_begin, p_end); p_begin is a multiple of BN.
+// With splits > 1 every tile's reduction is shared by `splits` workgroups through `scratch`
+// and a second kernel adds the partial planes.
 template <class Cfg>
-static int launch_conv(ConvArgs g, int p_begin, int p_end, hipStream_t stream) {
+static int launch_conv(ConvArgs g, int p_begin, int p_end, int splits, float *scratch, hipStream_t stream) {
     if (p_end <= p_begin) return T2SP_OK;
     g.p_begin = p_begin;
     g.tiles_m = (g.CO + Cfg::BM - 1) / Cfg::BM;
     g.tiles_n = (p_end - p_begin + Cfg::BN - 1) / Cfg::BN;
     g.group_m = g.tiles_m;   // all output channels of a pixel tile run together: the input tile is shared in L2
+    g.splits = splits;
+    g.Mp = g.tiles_m * Cfg::BM;
+    g.Np = g.tiles_n * Cfg::BN;
+    g.scratch = scratch;
     const bool edge = (g.CO % Cfg::BM) || ((p_end - p_begin) % Cfg::BN) || (g.KRED % (2 * Cfg::BK));
     const size_t smem = Cfg::SMEM_FLOATS * sizeof(float) + (size_t)g.KH * g.KW * sizeof(int);
     auto kern = edge ? conv_kernel<Cfg, true> : conv_kernel<Cfg, false>;
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(Cfg::NTHREADS), smem, stream, g);
-    return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * splits), dim3(Cfg::NTHREADS), smem, stream, g);
+    if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
+    if (splits > 1) {
+        ConvOutMap map{g.O, g.CO, g.P, g.OH, g.OW, p_begin, g.so_n, g.so_c, g.so_h};
+        if (launch_splitk_reduce<true>(scratch, splits, g.Mp, g.Np, map, stream) != hipSuccess) return T2SP_ERR_LAUNCH;
+    }
+    return T2SP_OK;
+}
+
+// How the automatic configuration covers the pixels: whole rounds of 256x256 tiles up to
+// p_split, then 128x128 tiles whose reduction is split `splits` ways so that the remainder
+// also spreads over all CUs.
+struct ConvPlan {
+    bool two_phase;
+    int p_split, splits;
+    size_t scratch_bytes;
+};
+static ConvPlan plan_conv(int CO, int P, int KRED) {
+    constexpr int CUS = 256;
+    ConvPlan p{false, 0, 1, 0};
+    const int tiles_m = (CO + 255) / 256;
+    const int rounds = (int)(((int64_t)tiles_m * (P / 256)) / CUS);
+    if (CO >= 256 && CUS % tiles_m == 0 && rounds >= 1) {
+        p.two_phase = true;
+        p.p_split = rounds * (CUS / tiles_m) * 256;
+        const int rem_tiles = ((CO + 127) / 128) * ((P - p.p_split + 127) / 128);
+        if (rem_tiles > 0 && rem_tiles < 128) {
+            int s = CUS / rem_tiles;
+            const int pairs = ((KRED + 15) / 16 + 1) / 2;
+            if (s > pairs / 4) s = pairs / 4;
+            if (s > 8) s = 8;
+            if (s > 1) {
+                p.splits = s;
+                p.scratch_bytes = (size_t)s * ((CO + 127) / 128 * 128) * ((P - p.p_split + 127) / 128 * 128) * sizeof(float);
+            }
+        }
+    }
+    return p;
 }
 
 using ConvL = TileCfg<256, 256, 16, 4, 2, STYLE_RC>;
@@ -158,9 +225,16 @@ using ConvS = TileCfg<64, 128, 16, 2, 1, STYLE_RC>;
 
 }  // namespace t2sp
 
+extern "C" size_t t2sp_conv2d_workspace_bytes(int N, int CI, int CO, int OH, int OW, int KH, int KW) {
+    if (N <= 0 || CI <= 0 || CO <= 0 || OH <= 0 || OW <= 0 || KH <= 0 || KW <= 0) return 0;
+    if ((int64_t)N * OH * OW > INT32_MAX || (int64_t)CI * KH * KW > INT32_MAX) return 0;
+    return t2sp::plan_conv(CO, N * OH * OW, CI * KH * KW).scratch_bytes;
+}
+
 extern "C" int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, int CI, int CO,
                                int OH, int OW, int KH, int KW, const int64_t *si4,
-                               const int64_t *sw4, const int64_t *so4, int cfg, void *stream) {
+                               const int64_t *sw4, const int64_t *so4, int cfg, float *workspace,
+                               size_t workspace_bytes, void *stream) {
     using namespace t2sp;
     if (N <= 0 || CI <= 0 || CO <= 0 || OH <= 0 || OW <= 0 || KH <= 0 || KW <= 0 || !si4 || !sw4 || !so4)
         return T2SP_ERR_SHAPE;
@@ -189,25 +263,24 @@ extern "C" int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, 
     g.so_n = so4[0]; g.so_c = so4[1]; g.so_h = so4[2];
     g.P = N * OH * OW; g.KRED = CI * KH * KW;
     switch (cfg) {
-        case T2SP_CFG_256x256: return launch_conv<ConvL>(g, 0, g.P, st);
-        case T2SP_CFG_128x128: return launch_conv<ConvM>(g, 0, g.P, st);
-        case T2SP_CFG_64x128: return launch_conv<ConvS>(g, 0, g.P, st);
+        case T2SP_CFG_256x256: return launch_conv<ConvL>(g, 0, g.P, 1, nullptr, st);
+        case T2SP_CFG_128x128: return launch_conv<ConvM>(g, 0, g.P, 1, nullptr, st);
+        case T2SP_CFG_64x128: return launch_conv<ConvS>(g, 0, g.P, 1, nullptr, st);
         case T2SP_CFG_AUTO: break;
         default: return T2SP_ERR_SHAPE;
     }
     // Automatic choice.  One 256x256 tile occupies a CU, so big tiles run in rounds of 256 (the
     // CU count); a partial last round would leave most CUs idle for a whole tile time.  Whole
     // rounds of big tiles are therefore launched first and the remaining pixels are covered with
-    // 128x128 tiles (several per CU), which finish in a fraction of a round.
-    constexpr int CUS = 256;
-    const int tiles_m = (CO + 255) / 256;
-    const int rounds = (int)(((int64_t)tiles_m * (g.P / 256)) / CUS);
-    if (CO >= 256 && CUS % tiles_m == 0 && rounds >= 1) {
-        const int p_split = rounds * (CUS / tiles_m) * 256;
-        const int rc = launch_conv<ConvL>(g, 0, p_split, st);
+    // 128x128 tiles; when those are too few to occupy the CUs their reduction is split as well
+    // (needs the workspace; without it the remainder runs unsplit).
+    const ConvPlan plan = plan_conv(CO, g.P, g.KRED);
+    if (plan.two_phase) {
+        const int rc = launch_conv<ConvL>(g, 0, plan.p_split, 1, nullptr, st);
         if (rc != T2SP_OK) return rc;
-        return launch_conv<ConvM>(g, p_split, g.P, st);
+        const bool split = plan.splits > 1 && workspace && workspace_bytes >= plan.scratch_bytes;
+        return launch_conv<ConvM>(g, plan.p_split, g.P, split ? plan.splits : 1, split ? workspace : nullptr, st);
     }
-    if ((int64_t)((CO + 127) / 128) * ((g.P + 127) / 128) >= 128) return launch_conv<ConvM>(g, 0, g.P, st);
-    return launch_conv<ConvS>(g, 0, g.P, st);
+    if ((int64_t)((CO + 127) / 128) * ((g.P + 127) / 128) >= 128) return launch_conv<ConvM>(g, 0, g.P, 1, nullptr, st);
+    return launch_conv<ConvS>(g, 0, g.P, 1, nullptr, st);
 }

@@ -142,8 +142,11 @@ static int conv_impl(halide_buffer_t *I, halide_buffer_t *K, halide_buffer_t *O,
     } else {
         for (int d = 0; d < 4; d++) so4[3 - d] = od[d].stride;
     }
+    const size_t ws_bytes = t2sp_conv2d_workspace_bytes((int)N, (int)CI, (int)CO, (int)OH, (int)OW, (int)KH, (int)KW);
+    float *ws = ws_bytes ? static_cast<float *>(pool().get(ws_bytes)) : nullptr;   // optional: NULL just disables the split
     err = t2sp_conv2d_f32(pi, pk, po, (int)N, (int)CI, (int)CO, (int)OH, (int)OW, (int)KH, (int)KW, ci4.str,
-                          ck4.str, so4, cfg, api_stream());
+                          ck4.str, so4, cfg, ws, ws ? ws_bytes : 0, api_stream());
+    struct PutWs { float *p; ~PutWs() { if (p) pool().put(p); } } put_ws{ws};
     if (err) return report(err, op, "kernel launch failed");
     if (via_tmp_o) {
         int ext[T2SP_MAX_DIMS];

@@ -119,7 +119,7 @@ def test_thin_layer_rejects_bad_shapes():
     assert L.t2sp_sgemm_f32(None, None, None, 4, 4, 4, 4, 4, 4, 12345, None) in (-8, -23)
     assert L.t2sp_fill_uniform_f32(None, -1, 0, None) == -8
     assert L.t2sp_fill_uniform_f32(None, 0, 0, None) == 0
-    assert L.t2sp_conv2d_f32(None, None, None, 1, 1, 1, 0, 4, 3, 3, None, None, None, 0, None) == -8
+    assert L.t2sp_conv2d_f32(None, None, None, 1, 1, 1, 0, 4, 3, 3, None, None, None, 0, None, 0, None) == -8
     assert L.t2sp_mttkrp_f32(None, None, None, None, 0, 4, 4, 4, None, None, None, None, 0, 0, None, 0, None) == -8
     assert L.t2sp_capsule_f32(None, None, None, None, None, None, None, 0, 0, None, 0, None) == -8
     assert L.t2sp_relayout_f32(None, None, 11, None, None, None, None) == -8
