@@ -1,0 +1,21 @@
+"""The C++ drivers of tests/drivers (written like the reference's *-run-fpga.cpp programs:
+build buffers, call the entry point, re-check every output with a naive loop, print Success)
+run against the built library on the GPU.  They are compiled by __graft_entry__.build() /
+`make -C tests/drivers` with the host compiler only."""
+import os
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+BIN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "drivers", "bin")
+
+
+@pytest.mark.parametrize("name", ["gemm-run", "conv-run", "capsule-run", "mttkrp-run"])
+def test_driver_prints_success(name):
+    exe = os.path.join(BIN, name)
+    assert os.path.exists(exe), "build the drivers first: make -C tests/drivers"
+    p = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    print(p.stdout, p.stderr)
+    assert p.returncode == 0
+    assert p.stdout.strip().splitlines()[-1] == "Success"
