@@ -51,6 +51,18 @@ int t2sp_sgemm_f32_tiled(const float *A, const float *B, float *C, int M, int N,
                          int64_t lda, int64_t ldb, int jjj, int iii, int jj, int ii,
                          const int64_t *strides6, int cfg, void *stream);
 
+/* BLAS form, row-major: C = alpha * op(A) * op(B) + beta * Cin with op(X) = X or X^T (transa /
+ * transb non-zero: A stored K x M, B stored N x K).  Cin may be NULL (beta is then ignored) or
+ * equal to C (in place).  A transposed A is first re-laid into `workspace`
+ * (t2sp_sgemm_ex_workspace_bytes); B^T runs natively.  Device side of the reference's 8-argument
+ * gemm(opa, opb, alpha, beta, A, B, C, O) pipeline behind its BLAS wrapper
+ * (t2s/peppers/blas/level3/gemm/release/a10/blas-gemm.cpp:28-47). */
+size_t t2sp_sgemm_ex_workspace_bytes(int transa, int M, int N, int K);
+int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, float alpha, const float *A,
+                      int64_t lda, const float *B, int64_t ldb, float beta, const float *Cin,
+                      int64_t ldcin, float *C, int64_t ldc, int cfg, float *workspace,
+                      size_t workspace_bytes, void *stream);
+
 /* O[n,co,h,w] = sum_{ci,kh,kw} I[n,ci,h+kh,w+kw] * W[co,ci,kh,kw], stride 1, valid
  * padding, fp32.  si4/sw4/so4 are element strides of the logical indices
  * (n,ci,h,w), (co,ci,kh,kw), (n,co,h,w); "w" is the innermost spatial axis (the

@@ -40,6 +40,12 @@ def _declare(L):
     L.t2sp_sgemm_f32.argtypes = [vp, vp, vp, i32, i32, i32, i64, i64, i64, i32, vp]
     L.t2sp_sgemm_f32_tiled.argtypes = [vp, vp, vp, i32, i32, i32, i64, i64, i32, i32, i32, i32,
                                        ctypes.POINTER(i64), i32, vp]
+    f32 = ctypes.c_float
+    L.t2sp_gemm_ex.argtypes = [i32, i32, f32, f32, bp, bp, bp, bp]
+    L.t2sp_sgemm_ex_workspace_bytes.argtypes = [i32, i32, i32, i32]
+    L.t2sp_sgemm_ex_workspace_bytes.restype = ctypes.c_size_t
+    L.t2sp_sgemm_ex_f32.argtypes = [i32, i32, i32, i32, i32, f32, vp, i64, vp, i64, f32, vp, i64, vp, i64, i32, vp,
+                                    ctypes.c_size_t, vp]
     L.conv.argtypes = [bp, bp, bp]
     L.t2sp_conv_with_cfg.argtypes = [bp, bp, bp, i32]
     p64, p32 = ctypes.POINTER(i64), ctypes.POINTER(i32)

@@ -23,6 +23,11 @@ struct GemmArgs {
     int tiled, t_jjj, t_iii, t_jj, t_ii;
     int64_t s[6];
     int tiles_m, tiles_n, group_m;
+    // C = alpha * A*B + beta * Cin (Cin read through ldcin); scale == 0 means plain C = A*B
+    int scale;
+    float alpha, beta;
+    const float *Cin;
+    int64_t ldcin;
 };
 
 __device__ __forceinline__ int64_t tiled_offset(const GemmArgs &g, int row, int col) {
@@ -32,45 +37,69 @@ __device__ __forceinline__ int64_t tiled_offset(const GemmArgs &g, int row, int 
            (cj / g.t_jj) * g.s[4] + (ri / g.t_ii) * g.s[5];
 }
 
-template <class Cfg, bool EDGE>
+// One accumulator element to memory, with the optional alpha/beta scaling of the BLAS form.
+__device__ __forceinline__ void gemm_store1(const GemmArgs &g, int r, int c, float v) {
+    if (g.scale) v = g.alpha * v + (g.beta != 0.f ? g.beta * g.Cin[(int64_t)r * g.ldcin + c] : 0.f);
+    if (g.tiled)
+        g.C[tiled_offset(g, r, c)] = v;
+    else
+        g.C[(int64_t)r * g.ldc + c] = v;
+}
+
+// BT = false: B is row-major K x N (columns contiguous, RC tile).
+// BT = true:  B is stored transposed, N x K with k contiguous (KC tile): C = A * B^T.
+template <class Cfg, bool EDGE, bool BT>
 __global__ void __launch_bounds__(Cfg::NTHREADS) sgemm_kernel(const GemmArgs g) {
     extern __shared__ __align__(16) float smem[];
     int tm, tn;
     tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, g.group_m, tm, tn);
     const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
     RowMajorKcLoader<Cfg, EDGE> la(g.A, g.lda, m0, g.M, g.K);
-    RowMajorRcLoader<Cfg, EDGE> lb(g.B, g.ldb, n0, g.N, g.K);
     Accum<Cfg> acc;
-    mainloop<Cfg>(acc, la, lb, ktiles_even<Cfg>(g.K), smem);
-    drain<Cfg>(acc, [&](int row, int col, v4f v) {
-        const int r = m0 + row, c = n0 + col;
-        if (EDGE && (r >= g.M || c >= g.N)) return;
-        if (!g.tiled) {
-            *reinterpret_cast<v4f *>(g.C + (int64_t)r * g.ldc + c) = v;
-        } else if (g.s[0] == 1 && g.t_jjj % 4 == 0) {
-            *reinterpret_cast<v4f *>(g.C + tiled_offset(g, r, c)) = v;
-        } else {
+    if constexpr (BT) {
+        RowMajorKcLoaderB<Cfg, EDGE> lb(g.B, g.ldb, n0, g.N, g.K);
+        mainloop<Cfg>(acc, la, lb, ktiles_even<Cfg>(g.K), smem);
+        drain<Cfg>(acc, [&](int row, int col, v4f v) {   // v = D[row..row+3][col]
+            const int c = n0 + col;
+            if (EDGE && c >= g.N) return;
+            for (int e = 0; e < 4; e++)
+                if (!EDGE || m0 + row + e < g.M) gemm_store1(g, m0 + row + e, c, v[e]);
+        });
+    } else {
+        RowMajorRcLoader<Cfg, EDGE> lb(g.B, g.ldb, n0, g.N, g.K);
+        mainloop<Cfg>(acc, la, lb, ktiles_even<Cfg>(g.K), smem);
+        drain<Cfg>(acc, [&](int row, int col, v4f v) {   // v = D[row][col..col+3]
+            const int r = m0 + row, c = n0 + col;
+            if (EDGE && (r >= g.M || c >= g.N)) return;
+            if (g.scale) {
+                v = v * g.alpha;
+                if (g.beta != 0.f) v += *reinterpret_cast<const v4f *>(g.Cin + (int64_t)r * g.ldcin + c) * g.beta;
+            }
+            if (!g.tiled) {
+                *reinterpret_cast<v4f *>(g.C + (int64_t)r * g.ldc + c) = v;
+            } else if (g.s[0] == 1 && g.t_jjj % 4 == 0) {
+                *reinterpret_cast<v4f *>(g.C + tiled_offset(g, r, c)) = v;
+            } else {
 #pragma unroll
-            for (int e = 0; e < 4; e++) g.C[tiled_offset(g, r, c + e)] = v[e];
-        }
-    });
+                for (int e = 0; e < 4; e++) g.C[tiled_offset(g, r, c + e)] = v[e];
+            }
+        });
+    }
 }
 
 // Fallback for shapes the vector loaders cannot take (K or N not a multiple
 // of 4, or operands not 16-byte aligned): one thread per output, sequential k.
-__global__ void sgemm_scalar_kernel(const GemmArgs g) {
+__global__ void sgemm_scalar_kernel(const GemmArgs g, int bt) {
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     const int r = blockIdx.y;
     if (c >= g.N) return;
     float acc = 0.f;
-    for (int k = 0; k < g.K; k++) acc = fmaf(g.A[(int64_t)r * g.lda + k], g.B[(int64_t)k * g.ldb + c], acc);
-    if (g.tiled)
-        g.C[tiled_offset(g, r, c)] = acc;
-    else
-        g.C[(int64_t)r * g.ldc + c] = acc;
+    for (int k = 0; k < g.K; k++)
+        acc = fmaf(g.A[(int64_t)r * g.lda + k], bt ? g.B[(int64_t)c * g.ldb + k] : g.B[(int64_t)k * g.ldb + c], acc);
+    gemm_store1(g, r, c, acc);
 }
 
-template <class Cfg>
+template <class Cfg, bool BT>
 static int launch(GemmArgs g, hipStream_t stream) {
     g.tiles_m = (g.M + Cfg::BM - 1) / Cfg::BM;
     g.tiles_n = (g.N + Cfg::BN - 1) / Cfg::BN;
@@ -78,7 +107,7 @@ static int launch(GemmArgs g, hipStream_t stream) {
     g.group_m = g.tiles_m >= 4 ? 4 : g.tiles_m;
     const bool edge = (g.M % Cfg::BM) || (g.N % Cfg::BN) || (g.K % (2 * Cfg::BK));
     const size_t smem = Cfg::SMEM_FLOATS * sizeof(float);
-    auto kern = edge ? sgemm_kernel<Cfg, true> : sgemm_kernel<Cfg, false>;
+    auto kern = edge ? sgemm_kernel<Cfg, true, BT> : sgemm_kernel<Cfg, false, BT>;
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
@@ -89,14 +118,19 @@ static int launch(GemmArgs g, hipStream_t stream) {
 using GemmL = TileCfg<256, 256, 16, 4, 2, STYLE_RC>;  // 8 waves, 64x128 per wave
 using GemmM = TileCfg<128, 128, 16, 4, 1, STYLE_RC>;  // 4 waves, 32x128 per wave
 using GemmS = TileCfg<64, 128, 16, 2, 1, STYLE_RC>;   // 2 waves, 32x128 per wave
+using GemmW = TileCfg<32, 128, 16, 1, 1, STYLE_RC>;   // 1 wave per tile
+using GemmLT = TileCfg<256, 256, 16, 4, 2, STYLE_KC>;  // B^T forms: both operands k-contiguous
+using GemmMT = TileCfg<128, 128, 16, 2, 2, STYLE_KC>;
+using GemmST = TileCfg<64, 64, 16, 2, 1, STYLE_KC>;
 
-static int dispatch(GemmArgs g, int cfg, hipStream_t stream) {
+static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream) {
     if (g.M <= 0 || g.N <= 0 || g.K <= 0) return T2SP_ERR_SHAPE;
-    const bool vec_ok = g.K % 4 == 0 && g.N % 4 == 0 && g.lda % 4 == 0 && g.ldb % 4 == 0 &&
+    const bool vec_ok = g.K % 4 == 0 && (bt || g.N % 4 == 0) && g.lda % 4 == 0 && g.ldb % 4 == 0 &&
                         ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
-                        ((uintptr_t)g.C % 16 == 0) && (g.tiled || g.ldc % 4 == 0);
+                        ((uintptr_t)g.C % 16 == 0) && (g.tiled || g.ldc % 4 == 0) &&
+                        (!g.scale || (g.ldcin % 4 == 0 && (uintptr_t)g.Cin % 16 == 0));
     if (cfg == T2SP_CFG_SCALAR || !vec_ok) {
-        hipLaunchKernelGGL(sgemm_scalar_kernel, dim3((g.N + 255) / 256, g.M), dim3(256), 0, stream, g);
+        hipLaunchKernelGGL(sgemm_scalar_kernel, dim3((g.N + 255) / 256, g.M), dim3(256), 0, stream, g, bt ? 1 : 0);
         return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
     }
     if (cfg == T2SP_CFG_AUTO) {
@@ -107,10 +141,20 @@ static int dispatch(GemmArgs g, int cfg, hipStream_t stream) {
         else if (tiles(128, 128) >= 200) cfg = T2SP_CFG_128x128;
         else cfg = T2SP_CFG_64x128;
     }
+    if (bt) {
+        switch (cfg) {
+            case T2SP_CFG_256x256: return launch<GemmLT, true>(g, stream);
+            case T2SP_CFG_128x128: return launch<GemmMT, true>(g, stream);
+            case T2SP_CFG_64x128:
+            case T2SP_CFG_32x128: return launch<GemmST, true>(g, stream);
+            default: return T2SP_ERR_SHAPE;
+        }
+    }
     switch (cfg) {
-        case T2SP_CFG_256x256: return launch<GemmL>(g, stream);
-        case T2SP_CFG_128x128: return launch<GemmM>(g, stream);
-        case T2SP_CFG_64x128: return launch<GemmS>(g, stream);
+        case T2SP_CFG_256x256: return launch<GemmL, false>(g, stream);
+        case T2SP_CFG_128x128: return launch<GemmM, false>(g, stream);
+        case T2SP_CFG_64x128: return launch<GemmS, false>(g, stream);
+        case T2SP_CFG_32x128: return launch<GemmW, false>(g, stream);
         default: return T2SP_ERR_SHAPE;
     }
 }
@@ -123,7 +167,7 @@ extern "C" int t2sp_sgemm_f32(const float *A, const float *B, float *C, int M, i
     g.A = A; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K;
     g.lda = lda; g.ldb = ldb; g.ldc = ldc;
     g.tiled = 0;
-    return t2sp::dispatch(g, cfg, (hipStream_t)stream);
+    return t2sp::dispatch(g, cfg, false, (hipStream_t)stream);
 }
 
 extern "C" int t2sp_sgemm_f32_tiled(const float *A, const float *B, float *C, int M, int N, int K,
@@ -135,5 +179,36 @@ extern "C" int t2sp_sgemm_f32_tiled(const float *A, const float *B, float *C, in
     g.lda = lda; g.ldb = ldb; g.ldc = 0;
     g.tiled = 1; g.t_jjj = jjj; g.t_iii = iii; g.t_jj = jj; g.t_ii = ii;
     for (int d = 0; d < 6; d++) g.s[d] = strides6[d];
-    return t2sp::dispatch(g, cfg, (hipStream_t)stream);
+    return t2sp::dispatch(g, cfg, false, (hipStream_t)stream);
+}
+
+extern "C" size_t t2sp_sgemm_ex_workspace_bytes(int transa, int M, int N, int K) {
+    (void)N;
+    return (transa && M > 0 && K > 0) ? (size_t)M * K * sizeof(float) : 0;
+}
+
+extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, float alpha, const float *A,
+                                 int64_t lda, const float *B, int64_t ldb, float beta, const float *Cin,
+                                 int64_t ldcin, float *C, int64_t ldc, int cfg, float *workspace,
+                                 size_t workspace_bytes, void *stream) {
+    if (M <= 0 || N <= 0 || K <= 0) return T2SP_ERR_SHAPE;
+    const float *a = A;
+    int64_t la = lda;
+    if (transa) {
+        // A is stored K x M: bring it to M x K first (the MFMA loaders want k contiguous in A)
+        if (!workspace || workspace_bytes < (size_t)M * K * sizeof(float)) return T2SP_ERR_SHAPE;
+        const int ext[2] = {K, M};
+        const int64_t ss[2] = {lda, 1}, ds[2] = {1, K};
+        const int rc = t2sp_relayout_f32(A, workspace, 2, ext, ss, ds, stream);
+        if (rc != T2SP_OK) return rc;
+        a = workspace;
+        la = K;
+    }
+    t2sp::GemmArgs g{};
+    g.A = a; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K;
+    g.lda = la; g.ldb = ldb; g.ldc = ldc;
+    g.tiled = 0;
+    g.scale = 1; g.alpha = alpha; g.beta = beta; g.Cin = Cin ? Cin : C; g.ldcin = Cin ? ldcin : ldc;
+    if (!Cin) g.beta = 0.f;
+    return t2sp::dispatch(g, cfg, transb != 0, (hipStream_t)stream);
 }

@@ -96,6 +96,48 @@ struct RowMajorRcLoader {
     }
 };
 
+// B operand stored transposed (N x K, k contiguous): the same loader as for A, sized by the
+// B-side constants of the tile.
+template <class Cfg, bool EDGE>
+struct RowMajorKcLoaderB {
+    const float *p[Cfg::B_VEC];
+    const float *safe;
+    bool row_ok[Cfg::B_VEC];
+    v4f reg[2][Cfg::B_VEC];
+    int k0, K;
+    __device__ RowMajorKcLoaderB(const float *B, int64_t ldb, int n0, int N, int K_) : safe(B), k0(0), K(K_) {
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
+            row_ok[i] = !EDGE || (n0 + s.row < N);
+            p[i] = B + (int64_t)(n0 + (row_ok[i] ? s.row : 0)) * ldb + s.k;
+        }
+    }
+    template <int S>
+    __device__ __forceinline__ void fetch() {
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
+            if (EDGE)
+                reg[S][i] = load_or_zero(p[i], row_ok[i] && k0 + s.k < K, safe);
+            else
+                reg[S][i] = *reinterpret_cast<const v4f *>(p[i]);
+        }
+        const int step = (EDGE || k0 + 2 * Cfg::BK <= K) ? Cfg::BK : 0;
+        k0 += step;
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) p[i] += step;
+    }
+    template <int S>
+    __device__ __forceinline__ void commit(float *stage) const {
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
+            *reinterpret_cast<v4f *>(stage + s.row * Cfg::LDB + s.k) = reg[S][i];
+        }
+    }
+};
+
 // Number of k-tiles the mainloop runs for a reduction of length K: rounded up to a pair.
 template <class Cfg>
 __device__ __host__ inline int ktiles_even(int K) {

@@ -60,6 +60,23 @@ def gemm(A, B, out=None, tiles=None, cfg=0):
     return out
 
 
+def gemm_ex(opa, opb, alpha, beta, A, B, C=None, out=None, tiles=None):
+    """O = alpha * op(A) @ op(B) + beta * C through `t2sp_gemm_ex` (include/blas-gemm.h), the
+    counterpart of the reference's gemm(opa, opb, alpha, beta, A, B, C, O)
+    (t2s/peppers/blas/level3/gemm/release/a10/blas-gemm.cpp:47).
+
+    A is (M, K), or (K, M) when opa; B is (K, N), or (N, K) when opb; C (M, N) or None."""
+    M = A.shape[1] if opa else A.shape[0]
+    N = B.shape[0] if opb else B.shape[1]
+    if out is None:
+        out = _empty_like_kind(A, (M, N) if tiles is None else gemm_tiled_shape(M, N, *tiles))
+    a, b, o = HalideBuffer.wrap(A), HalideBuffer.wrap(B), HalideBuffer.wrap(out)
+    c = HalideBuffer.wrap(C) if C is not None else None
+    _check("gemm_ex", lib().t2sp_gemm_ex(int(bool(opa)), int(bool(opb)), float(alpha), float(beta), a.ref, b.ref,
+                                         c.ref if c is not None else None, o.ref))
+    return out
+
+
 def conv(I, W, out=None, cfg=0):
     """O = conv2d(I, W), stride 1, no padding, through the `conv` entry point
     (include/conv-interface.h).
