@@ -28,6 +28,10 @@ int capsule(struct halide_buffer_t *P, struct halide_buffer_t *W, struct halide_
 int t2sp_capsule_with_cfg(struct halide_buffer_t *P, struct halide_buffer_t *W,
                           struct halide_buffer_t *V, int cfg, int splits);
 
+/* capsule() that returns the kernel time in ns (negative error code on failure), like the oneAPI
+ * flavour of the reference's entry (t2s/tests/performance/oneapi/src/oneapi-target-4-run.cpp:99). */
+double capsule_ns(struct halide_buffer_t *P, struct halide_buffer_t *W, struct halide_buffer_t *V);
+
 #ifdef __cplusplus
 }
 #endif

@@ -29,6 +29,10 @@ int conv(struct halide_buffer_t *I, struct halide_buffer_t *K, struct halide_buf
 int t2sp_conv_with_cfg(struct halide_buffer_t *I, struct halide_buffer_t *K,
                        struct halide_buffer_t *O, int cfg);
 
+/* conv() that returns the kernel time in ns (negative error code on failure), like the oneAPI
+ * flavour of the reference's entry (t2s/tests/performance/oneapi/src/oneapi-target-4-run.cpp:99). */
+double conv_ns(struct halide_buffer_t *I, struct halide_buffer_t *K, struct halide_buffer_t *O);
+
 #ifdef __cplusplus
 }
 #endif

@@ -32,6 +32,10 @@ int GEMM(struct halide_buffer_t *A, struct halide_buffer_t *B, struct halide_buf
 int t2sp_gemm_with_cfg(struct halide_buffer_t *A, struct halide_buffer_t *B,
                        struct halide_buffer_t *C, int cfg);
 
+/* gemm() that returns the kernel time in ns (negative error code on failure), like the oneAPI
+ * flavour of the reference's entry (t2s/tests/performance/oneapi/src/oneapi-target-4-run.cpp:99). */
+double gemm_ns(struct halide_buffer_t *A, struct halide_buffer_t *B, struct halide_buffer_t *C);
+
 #ifdef __cplusplus
 }
 #endif

@@ -24,6 +24,10 @@ int mttkrp(struct halide_buffer_t *B, struct halide_buffer_t *C, struct halide_b
 int t2sp_mttkrp_with_cfg(struct halide_buffer_t *B, struct halide_buffer_t *C,
                          struct halide_buffer_t *D, struct halide_buffer_t *A, int cfg, int splits);
 
+/* mttkrp() that returns the kernel time in ns (negative error code on failure), like the oneAPI
+ * flavour of the reference's entry (t2s/tests/performance/oneapi/src/oneapi-target-4-run.cpp:99). */
+double mttkrp_ns(struct halide_buffer_t *B, struct halide_buffer_t *C, struct halide_buffer_t *D, struct halide_buffer_t *A);
+
 #ifdef __cplusplus
 }
 #endif

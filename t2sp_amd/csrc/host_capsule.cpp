@@ -77,3 +77,11 @@ extern "C" int capsule(halide_buffer_t *P, halide_buffer_t *W, halide_buffer_t *
 extern "C" int t2sp_capsule_with_cfg(halide_buffer_t *P, halide_buffer_t *W, halide_buffer_t *V, int cfg, int splits) {
     return capsule_impl(P, W, V, cfg, splits);
 }
+
+// The oneAPI flavour of the reference's entry returns the kernel time in nanoseconds
+// (double exec_time = capsule(device_selector, ...), t2s/src/CodeGen_OneAPI_Dev.cpp:3554-3617); this is
+// that form: the time on success, the negative error code otherwise.
+extern "C" double capsule_ns(halide_buffer_t *P, halide_buffer_t *W, halide_buffer_t *V) {
+    const int rc = capsule(P, W, V);
+    return rc == 0 ? t2sp_last_kernel_ns() : (double)rc;
+}

@@ -177,3 +177,11 @@ extern "C" int conv(halide_buffer_t *I, halide_buffer_t *K, halide_buffer_t *O) 
 extern "C" int t2sp_conv_with_cfg(halide_buffer_t *I, halide_buffer_t *K, halide_buffer_t *O, int cfg) {
     return conv_impl(I, K, O, cfg);
 }
+
+// The oneAPI flavour of the reference's entry returns the kernel time in nanoseconds
+// (double exec_time = conv(device_selector, ...), t2s/src/CodeGen_OneAPI_Dev.cpp:3554-3617); this is
+// that form: the time on success, the negative error code otherwise.
+extern "C" double conv_ns(halide_buffer_t *I, halide_buffer_t *K, halide_buffer_t *O) {
+    const int rc = conv(I, K, O);
+    return rc == 0 ? t2sp_last_kernel_ns() : (double)rc;
+}

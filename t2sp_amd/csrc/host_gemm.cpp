@@ -81,3 +81,11 @@ extern "C" int GEMM(halide_buffer_t *A, halide_buffer_t *B, halide_buffer_t *C) 
 extern "C" int t2sp_gemm_with_cfg(halide_buffer_t *A, halide_buffer_t *B, halide_buffer_t *C, int cfg) {
     return gemm_impl(A, B, C, cfg);
 }
+
+// The oneAPI flavour of the reference's entry returns the kernel time in nanoseconds
+// (double exec_time = gemm(device_selector, ...), t2s/src/CodeGen_OneAPI_Dev.cpp:3554-3617); this is
+// that form: the time on success, the negative error code otherwise.
+extern "C" double gemm_ns(halide_buffer_t *A, halide_buffer_t *B, halide_buffer_t *C) {
+    const int rc = gemm(A, B, C);
+    return rc == 0 ? t2sp_last_kernel_ns() : (double)rc;
+}

@@ -77,3 +77,11 @@ extern "C" int t2sp_mttkrp_with_cfg(halide_buffer_t *B, halide_buffer_t *C, hali
                                     halide_buffer_t *A, int cfg, int splits) {
     return mttkrp_impl(B, C, D, A, cfg, splits);
 }
+
+// The oneAPI flavour of the reference's entry returns the kernel time in nanoseconds
+// (double exec_time = mttkrp(device_selector, ...), t2s/src/CodeGen_OneAPI_Dev.cpp:3554-3617); this is
+// that form: the time on success, the negative error code otherwise.
+extern "C" double mttkrp_ns(halide_buffer_t *B, halide_buffer_t *C, halide_buffer_t *D, halide_buffer_t *A) {
+    const int rc = mttkrp(B, C, D, A);
+    return rc == 0 ? t2sp_last_kernel_ns() : (double)rc;
+}

@@ -2,6 +2,7 @@
 #include "runtime.hpp"
 
 #include <atomic>
+#include <stdlib.h>
 
 namespace t2sp {
 
@@ -190,6 +191,18 @@ int KernelTimer::stop_and_sync(const char *op) {
     }
     float ms = 0.f;
     if (hipEventElapsedTime(&ms, g_ev0, g_ev1) == hipSuccess) g_last_kernel_ns = (double)ms * 1e6;
+    // Optional file in the reference's exec_time.txt format (AOT-OpenCL-Runtime.cpp:380-394):
+    // overall ns on the first line, then "<kernel_name> <ns>" lines.  The reference's drivers ask
+    // for "kernel_unloader", the last kernel of its pipeline, so that name is written too.
+    if (const char *file = getenv("T2SP_EXEC_TIME_FILE")) {
+        if (*file) {
+            if (FILE *fp = fopen(file, "w")) {
+                const double ns = g_last_kernel_ns.load();
+                fprintf(fp, "%f\nkernel_%s %lf\nkernel_unloader %lf\n", ns, op, ns, ns);
+                fclose(fp);
+            }
+        }
+    }
     return 0;
 }
 

@@ -31,8 +31,10 @@ def test_library_exports_every_declared_symbol():
     L = t2sp_amd.lib()
     names = declared_symbols()
     assert {"gemm", "GEMM", "t2sp_sgemm_f32", "t2sp_last_kernel_ns"} <= names
-    # sgemm has C++ linkage, like the reference's blas-gemm.h: look its mangled name up instead
-    mangled = {"sgemm": "_Z5sgemmcciiifPfiS_ifS_i"}
+    # sgemm and the Roofline.h helpers have C++ linkage, like the reference's own headers: look their
+    # mangled names up instead
+    mangled = {"sgemm": "_Z5sgemmcciiifPfiS_ifS_i", "DSPs": "_Z4DSPsv", "FMax": "_Z4FMaxv",
+               "ExecTime": "_Z8ExecTimePKc", "roofline": "_Z8rooflineddddd"}
     missing = [n for n in sorted(names) if not hasattr(L, mangled.get(n, n))]
     assert not missing, missing
     assert {"sgemm", "t2sp_gemm_ex", "t2sp_conv2d_workspace_bytes", "t2sp_mttkrp_workspace_bytes"} <= names

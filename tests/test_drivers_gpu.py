@@ -11,11 +11,11 @@ pytestmark = pytest.mark.gpu
 BIN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "drivers", "bin")
 
 
-@pytest.mark.parametrize("name", ["gemm-run", "conv-run", "capsule-run", "mttkrp-run", "sgemm-run"])
-def test_driver_prints_success(name):
+@pytest.mark.parametrize("name", ["gemm-run", "conv-run", "capsule-run", "mttkrp-run", "sgemm-run", "gemm-large-run"])
+def test_driver_prints_success(name, tmp_path):
     exe = os.path.join(BIN, name)
     assert os.path.exists(exe), "build the drivers first: make -C tests/drivers"
-    p = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    p = subprocess.run([exe], capture_output=True, text=True, timeout=100, cwd=str(tmp_path))
     print(p.stdout, p.stderr)
     assert p.returncode == 0
     assert p.stdout.strip().splitlines()[-1] == "Success"
