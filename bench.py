@@ -93,9 +93,12 @@ def sgemm_case(torch, t2sp_amd, M, N, K, steps, warmup, seed=1, min_warm_ms=0.0)
     B = t2sp_amd.fill_uniform(torch.empty(K, N, device="cuda"), seed + 1)
     C = torch.empty(M, N, device="cuda")
     stream = torch.cuda.current_stream().cuda_stream
+    nbytes = L.t2sp_sgemm_workspace_bytes(M, N, K)
+    ws = torch.empty(max(nbytes // 4, 1), device="cuda")
 
     def launch():
-        rc = L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, stream)
+        rc = L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, ws.data_ptr(), nbytes,
+                              stream)
         if rc != 0:
             raise RuntimeError("t2sp_sgemm_f32 returned %d" % rc)
 

@@ -38,9 +38,13 @@ extern "C" {
 /* C[i,j] = sum_k A[i,k] * B[k,j], fp32, row-major with leading dimensions in
  * elements.  Replaces the device side of the reference's SGEMM pipeline: the
  * kernels of t2s/tests/performance/gemm/bitstream/a10/a.cl:67-770 launched by
- * halide_opencl_wait_for_kernels_finish (t2s/src/AOT-OpenCL-Runtime.cpp:312-397). */
+ * halide_opencl_wait_for_kernels_finish (t2s/src/AOT-OpenCL-Runtime.cpp:312-397).
+ * `workspace` is optional (NULL allowed): products with fewer output tiles than CUs use it
+ * (t2sp_sgemm_workspace_bytes) to split the reduction over more workgroups. */
+size_t t2sp_sgemm_workspace_bytes(int M, int N, int K);
 int t2sp_sgemm_f32(const float *A, const float *B, float *C, int M, int N, int K, int64_t lda,
-                   int64_t ldb, int64_t ldc, int cfg, void *stream);
+                   int64_t ldb, int64_t ldc, int cfg, float *workspace, size_t workspace_bytes,
+                   void *stream);
 
 /* Same product, written straight into the reference's 6-D tiled output
  * c(jjj, iii, jj, ii, j, i) (t2s/tests/performance/gemm/gemm-run-fpga.cpp:69;
@@ -49,7 +53,8 @@ int t2sp_sgemm_f32(const float *A, const float *B, float *C, int M, int N, int K
  * unloader kernel plus the host deserializer loop of the generated interface. */
 int t2sp_sgemm_f32_tiled(const float *A, const float *B, float *C, int M, int N, int K,
                          int64_t lda, int64_t ldb, int jjj, int iii, int jj, int ii,
-                         const int64_t *strides6, int cfg, void *stream);
+                         const int64_t *strides6, int cfg, float *workspace, size_t workspace_bytes,
+                         void *stream);
 
 /* BLAS form, row-major: C = alpha * op(A) * op(B) + beta * Cin with op(X) = X or X^T (transa /
  * transb non-zero: A stored K x M, B stored N x K).  Cin may be NULL (beta is then ignored) or

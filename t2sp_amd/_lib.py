@@ -37,9 +37,11 @@ def _declare(L):
     L.gemm.argtypes = [bp, bp, bp]
     L.GEMM.argtypes = [bp, bp, bp]
     L.t2sp_gemm_with_cfg.argtypes = [bp, bp, bp, i32]
-    L.t2sp_sgemm_f32.argtypes = [vp, vp, vp, i32, i32, i32, i64, i64, i64, i32, vp]
+    L.t2sp_sgemm_f32.argtypes = [vp, vp, vp, i32, i32, i32, i64, i64, i64, i32, vp, ctypes.c_size_t, vp]
+    L.t2sp_sgemm_workspace_bytes.argtypes = [i32, i32, i32]
+    L.t2sp_sgemm_workspace_bytes.restype = ctypes.c_size_t
     L.t2sp_sgemm_f32_tiled.argtypes = [vp, vp, vp, i32, i32, i32, i64, i64, i32, i32, i32, i32,
-                                       ctypes.POINTER(i64), i32, vp]
+                                       ctypes.POINTER(i64), i32, vp, ctypes.c_size_t, vp]
     f32 = ctypes.c_float
     L.t2sp_gemm_ex.argtypes = [i32, i32, f32, f32, bp, bp, bp, bp]
     L.t2sp_sgemm_ex_workspace_bytes.argtypes = [i32, i32, i32, i32]

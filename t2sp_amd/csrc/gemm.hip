@@ -8,6 +8,7 @@
 // c(jjj, iii, jj, ii, j, i)  (gemm-run-fpga.cpp:69, gemm.cpp:39-41).
 #include "mfma_core.hpp"
 #include "gemm_loaders.hpp"
+#include "splitk.hpp"
 #include "t2sp_hip.h"
 
 namespace t2sp {
@@ -28,6 +29,9 @@ struct GemmArgs {
     float alpha, beta;
     const float *Cin;
     int64_t ldcin;
+    // reduction split over `splits` workgroups per tile (1 = none): partial planes in scratch
+    int splits, Mp, Np;
+    float *scratch;
 };
 
 __device__ __forceinline__ int64_t tiled_offset(const GemmArgs &g, int row, int col) {
@@ -46,15 +50,32 @@ __device__ __forceinline__ void gemm_store1(const GemmArgs &g, int r, int c, flo
         g.C[(int64_t)r * g.ldc + c] = v;
 }
 
+// Where the sum of the partial planes of a split reduction goes (plain C = A*B only).
+struct GemmOutMap {
+    GemmArgs g;
+    __device__ __forceinline__ void store(int row, int col, v4f v) const {
+        if (row >= g.M || col >= g.N) return;
+        if (!g.tiled) {
+            *reinterpret_cast<v4f *>(g.C + (int64_t)row * g.ldc + col) = v;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) g.C[tiled_offset(g, row, col + e)] = v[e];
+        }
+    }
+};
+
 // BT = false: B is row-major K x N (columns contiguous, RC tile).
 // BT = true:  B is stored transposed, N x K with k contiguous (KC tile): C = A * B^T.
 template <class Cfg, bool EDGE, bool BT>
 __global__ void __launch_bounds__(Cfg::NTHREADS) sgemm_kernel(const GemmArgs g) {
     extern __shared__ __align__(16) float smem[];
+    const int tile = blockIdx.x / g.splits, split = blockIdx.x - tile * g.splits;
     int tm, tn;
-    tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, g.group_m, tm, tn);
+    tile_coords(tile, g.tiles_m, g.tiles_n, g.group_m, tm, tn);
     const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
-    RowMajorKcLoader<Cfg, EDGE> la(g.A, g.lda, m0, g.M, g.K);
+    int kt0 = 0, kt1 = ktiles_even<Cfg>(g.K);
+    if (g.splits > 1) split_range((g.K + Cfg::BK - 1) / Cfg::BK, g.splits, split, kt0, kt1);
+    RowMajorKcLoader<Cfg, EDGE> la(g.A, g.lda, m0, g.M, g.K, kt0 * Cfg::BK);
     Accum<Cfg> acc;
     if constexpr (BT) {
         RowMajorKcLoaderB<Cfg, EDGE> lb(g.B, g.ldb, n0, g.N, g.K);
@@ -66,8 +87,12 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) sgemm_kernel(const GemmArgs g) 
                 if (!EDGE || m0 + row + e < g.M) gemm_store1(g, m0 + row + e, c, v[e]);
         });
     } else {
-        RowMajorRcLoader<Cfg, EDGE> lb(g.B, g.ldb, n0, g.N, g.K);
-        mainloop<Cfg>(acc, la, lb, ktiles_even<Cfg>(g.K), smem);
+        RowMajorRcLoader<Cfg, EDGE> lb(g.B, g.ldb, n0, g.N, g.K, kt0 * Cfg::BK);
+        mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem);
+        if (g.splits > 1) {
+            store_partial<Cfg>(acc, g.scratch, split, m0, n0, g.Mp, g.Np);
+            return;
+        }
         drain<Cfg>(acc, [&](int row, int col, v4f v) {   // v = D[row][col..col+3]
             const int r = m0 + row, c = n0 + col;
             if (EDGE && (r >= g.M || c >= g.N)) return;
@@ -100,9 +125,13 @@ __global__ void sgemm_scalar_kernel(const GemmArgs g, int bt) {
 }
 
 template <class Cfg, bool BT>
-static int launch(GemmArgs g, hipStream_t stream) {
+static int launch(GemmArgs g, hipStream_t stream, int splits = 1, float *scratch = nullptr) {
     g.tiles_m = (g.M + Cfg::BM - 1) / Cfg::BM;
     g.tiles_n = (g.N + Cfg::BN - 1) / Cfg::BN;
+    g.splits = BT ? 1 : splits;
+    g.Mp = g.tiles_m * Cfg::BM;
+    g.Np = g.tiles_n * Cfg::BN;
+    g.scratch = scratch;
     // bands of about sqrt(32) tile-rows keep a XCD's resident tiles near-square
     g.group_m = g.tiles_m >= 4 ? 4 : g.tiles_m;
     const bool edge = (g.M % Cfg::BM) || (g.N % Cfg::BN) || (g.K % (2 * Cfg::BK));
@@ -111,8 +140,13 @@ static int launch(GemmArgs g, hipStream_t stream) {
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(Cfg::NTHREADS), smem, stream, g);
-    return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * g.splits), dim3(Cfg::NTHREADS), smem, stream, g);
+    if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
+    if (g.splits > 1) {
+        GemmOutMap map{g};
+        if (launch_splitk_reduce<true>(scratch, g.splits, g.Mp, g.Np, map, stream) != hipSuccess) return T2SP_ERR_LAUNCH;
+    }
+    return T2SP_OK;
 }
 
 using GemmL = TileCfg<256, 256, 16, 4, 2, STYLE_RC>;  // 8 waves, 64x128 per wave
@@ -123,7 +157,37 @@ using GemmLT = TileCfg<256, 256, 16, 4, 2, STYLE_KC>;  // B^T forms: both operan
 using GemmMT = TileCfg<128, 128, 16, 2, 2, STYLE_KC>;
 using GemmST = TileCfg<64, 64, 16, 2, 1, STYLE_KC>;
 
-static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream) {
+// Tile configuration and reduction split for a plain product.  Large problems take 256x256
+// tiles; when those would leave CUs idle the tile shrinks, and when even 128x128 tiles are fewer
+// than the 256 CUs the reduction is split so that about one workgroup per CU exists (needs a
+// workspace; without one the product runs unsplit).
+struct GemmPlan {
+    int cfg, splits;
+    size_t scratch_bytes;
+};
+static GemmPlan plan_gemm(int M, int N, int K) {
+    auto tiles = [&](int bm, int bn) { return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+    GemmPlan p{T2SP_CFG_64x128, 1, 0};
+    if (tiles(256, 256) >= 200) p.cfg = T2SP_CFG_256x256;
+    else if (tiles(128, 128) >= 200) p.cfg = T2SP_CFG_128x128;
+    else {
+        const int bm = tiles(128, 128) >= 32 ? 128 : 64;
+        p.cfg = bm == 128 ? T2SP_CFG_128x128 : T2SP_CFG_64x128;
+        const int64_t t = tiles(bm, 128);
+        const int pairs = ((K + 15) / 16 + 1) / 2;
+        int s = (int)((256 + t / 2) / t);
+        if (s > pairs / 4) s = pairs / 4;
+        if (s > 16) s = 16;
+        if (s > 1) {
+            p.splits = s;
+            p.scratch_bytes = (size_t)s * ((M + bm - 1) / bm * bm) * ((N + 127) / 128 * 128) * sizeof(float);
+        }
+    }
+    return p;
+}
+
+static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *workspace = nullptr,
+                    size_t workspace_bytes = 0) {
     if (g.M <= 0 || g.N <= 0 || g.K <= 0) return T2SP_ERR_SHAPE;
     const bool vec_ok = g.K % 4 == 0 && (bt || g.N % 4 == 0) && g.lda % 4 == 0 && g.ldb % 4 == 0 &&
                         ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
@@ -133,13 +197,11 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream) {
         hipLaunchKernelGGL(sgemm_scalar_kernel, dim3((g.N + 255) / 256, g.M), dim3(256), 0, stream, g, bt ? 1 : 0);
         return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
     }
+    int splits = 1;
     if (cfg == T2SP_CFG_AUTO) {
-        auto tiles = [&](int bm, int bn) {
-            return (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
-        };
-        if (tiles(256, 256) >= 200) cfg = T2SP_CFG_256x256;
-        else if (tiles(128, 128) >= 200) cfg = T2SP_CFG_128x128;
-        else cfg = T2SP_CFG_64x128;
+        const GemmPlan p = plan_gemm(g.M, g.N, g.K);
+        cfg = p.cfg;
+        if (!bt && !g.scale && p.splits > 1 && workspace && workspace_bytes >= p.scratch_bytes) splits = p.splits;
     }
     if (bt) {
         switch (cfg) {
@@ -152,8 +214,8 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream) {
     }
     switch (cfg) {
         case T2SP_CFG_256x256: return launch<GemmL, false>(g, stream);
-        case T2SP_CFG_128x128: return launch<GemmM, false>(g, stream);
-        case T2SP_CFG_64x128: return launch<GemmS, false>(g, stream);
+        case T2SP_CFG_128x128: return launch<GemmM, false>(g, stream, splits, workspace);
+        case T2SP_CFG_64x128: return launch<GemmS, false>(g, stream, splits, workspace);
         case T2SP_CFG_32x128: return launch<GemmW, false>(g, stream);
         default: return T2SP_ERR_SHAPE;
     }
@@ -161,25 +223,32 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream) {
 
 }  // namespace t2sp
 
+extern "C" size_t t2sp_sgemm_workspace_bytes(int M, int N, int K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    return t2sp::plan_gemm(M, N, K).scratch_bytes;
+}
+
 extern "C" int t2sp_sgemm_f32(const float *A, const float *B, float *C, int M, int N, int K,
-                              int64_t lda, int64_t ldb, int64_t ldc, int cfg, void *stream) {
+                              int64_t lda, int64_t ldb, int64_t ldc, int cfg, float *workspace,
+                              size_t workspace_bytes, void *stream) {
     t2sp::GemmArgs g{};
     g.A = A; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K;
     g.lda = lda; g.ldb = ldb; g.ldc = ldc;
     g.tiled = 0;
-    return t2sp::dispatch(g, cfg, false, (hipStream_t)stream);
+    return t2sp::dispatch(g, cfg, false, (hipStream_t)stream, workspace, workspace_bytes);
 }
 
 extern "C" int t2sp_sgemm_f32_tiled(const float *A, const float *B, float *C, int M, int N, int K,
                                     int64_t lda, int64_t ldb, int jjj, int iii, int jj, int ii,
-                                    const int64_t *strides6, int cfg, void *stream) {
+                                    const int64_t *strides6, int cfg, float *workspace,
+                                    size_t workspace_bytes, void *stream) {
     if (jjj <= 0 || iii <= 0 || jj <= 0 || ii <= 0 || !strides6) return T2SP_ERR_SHAPE;
     t2sp::GemmArgs g{};
     g.A = A; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K;
     g.lda = lda; g.ldb = ldb; g.ldc = 0;
     g.tiled = 1; g.t_jjj = jjj; g.t_iii = iii; g.t_jj = jj; g.t_ii = ii;
     for (int d = 0; d < 6; d++) g.s[d] = strides6[d];
-    return t2sp::dispatch(g, cfg, false, (hipStream_t)stream);
+    return t2sp::dispatch(g, cfg, false, (hipStream_t)stream, workspace, workspace_bytes);
 }
 
 extern "C" size_t t2sp_sgemm_ex_workspace_bytes(int transa, int M, int N, int K) {

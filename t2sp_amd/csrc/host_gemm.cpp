@@ -48,6 +48,9 @@ static int gemm_impl(halide_buffer_t *A, halide_buffer_t *B, halide_buffer_t *C,
     if ((err = da.input(A, sa, op))) return err;
     if ((err = db.input(B, sb, op))) return err;
     if ((err = dc.output(C, sc, op))) return err;
+    const size_t ws_bytes = K > 0 ? t2sp_sgemm_workspace_bytes(M, N, K) : 0;
+    float *ws = ws_bytes ? static_cast<float *>(pool().get(ws_bytes)) : nullptr;   // optional
+    struct PutWs { float *p; ~PutWs() { if (p) pool().put(p); } } put_ws{ws};
     KernelTimer timer;
     if (K == 0) {
         // an empty reduction leaves C = 0 (Z is initialised to 0 at k = 0, gemm.cpp:59)
@@ -58,10 +61,11 @@ static int gemm_impl(halide_buffer_t *A, halide_buffer_t *B, halide_buffer_t *C,
         for (int d = 0; d < 6; d++) s6[d] = C->dim[d].stride;
         err = t2sp_sgemm_f32_tiled(da.ptr(), db.ptr(), dc.ptr(), M, N, K, A->dim[1].stride,
                                    B->dim[1].stride, C->dim[0].extent, C->dim[1].extent,
-                                   C->dim[2].extent, C->dim[3].extent, s6, cfg, api_stream());
+                                   C->dim[2].extent, C->dim[3].extent, s6, cfg, ws, ws ? ws_bytes : 0,
+                                   api_stream());
     } else {
         err = t2sp_sgemm_f32(da.ptr(), db.ptr(), dc.ptr(), M, N, K, A->dim[1].stride,
-                             B->dim[1].stride, C->dim[1].stride, cfg, api_stream());
+                             B->dim[1].stride, C->dim[1].stride, cfg, ws, ws ? ws_bytes : 0, api_stream());
     }
     if (err) return report(err, op, "kernel launch failed");
     if ((err = timer.stop_and_sync(op))) return err;

@@ -120,8 +120,8 @@ def test_other_entries_reject_bad_arguments_without_a_device():
 
 def test_thin_layer_rejects_bad_shapes():
     L = t2sp_amd.lib()
-    assert L.t2sp_sgemm_f32(None, None, None, 0, 4, 4, 4, 4, 4, 0, None) == -8
-    assert L.t2sp_sgemm_f32(None, None, None, 4, 4, 4, 4, 4, 4, 12345, None) in (-8, -23)
+    assert L.t2sp_sgemm_f32(None, None, None, 0, 4, 4, 4, 4, 4, 0, None, 0, None) == -8
+    assert L.t2sp_sgemm_f32(None, None, None, 4, 4, 4, 4, 4, 4, 12345, None, 0, None) in (-8, -23)
     assert L.t2sp_fill_uniform_f32(None, -1, 0, None) == -8
     assert L.t2sp_fill_uniform_f32(None, 0, 0, None) == 0
     assert L.t2sp_conv2d_f32(None, None, None, 1, 1, 1, 0, 4, 3, 3, None, None, None, 0, None, 0, None) == -8

@@ -130,6 +130,39 @@ def test_padded_leading_dimensions(oracle):
     assert (Cp[:, N:] == keep).all()          # padding columns of C untouched
 
 
+@pytest.mark.parametrize("shape", [(1024, 1024, 1024), (500, 260, 4096), (64, 128, 8192)])
+def test_split_reduction_with_workspace(oracle, torch_cuda, shape):
+    """Few output tiles: with a workspace the thin layer splits the reduction over more workgroups.
+    Same tolerance as the unsplit product, and bit-identical from run to run (the partial planes
+    are summed in a fixed order)."""
+    torch = torch_cuda
+    M, N, K = shape
+    L = t2sp_amd.lib()
+    nbytes = L.t2sp_sgemm_workspace_bytes(M, N, K)
+    assert nbytes > 0
+    A = t2sp_amd.fill_uniform(torch.empty(M, K, device="cuda"), 21)
+    B = t2sp_amd.fill_uniform(torch.empty(K, N, device="cuda"), 22)
+    ws = torch.empty(nbytes // 4, device="cuda")
+    outs = []
+    for _ in range(2):
+        C = torch.full((M, N), float("nan"), device="cuda")
+        rc = L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, ws.data_ptr(), nbytes,
+                              None)
+        assert rc == 0
+        torch.cuda.synchronize()
+        outs.append(C.cpu().numpy())
+    assert (outs[0] == outs[1]).all()
+    err, mx = rel_fro(outs[0], oracle.gemm(A.cpu().numpy(), B.cpu().numpy()))
+    print("split %s rel_fro %.3e max_abs %.3e" % (shape, err, mx))
+    assert err <= TOL
+    # a workspace that is too small is ignored, not an error
+    C = torch.full((M, N), float("nan"), device="cuda")
+    assert L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, ws.data_ptr(), 16,
+                            None) == 0
+    torch.cuda.synchronize()
+    assert rel_fro(C.cpu().numpy(), outs[0])[0] <= TOL
+
+
 def test_empty_extents():
     C = np.full((16, 8), np.nan, np.float32)
     t2sp_amd.gemm(np.zeros((16, 0), np.float32), np.zeros((0, 8), np.float32), out=C)
