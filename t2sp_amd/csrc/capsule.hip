@@ -76,7 +76,7 @@ struct PoseKcLoader {
     }
     template <int S>
     __device__ __forceinline__ void fetch() {
-        const bool go = k0 + 2 * Cfg::BK <= g.KRED;
+        const bool go = KPAD || k0 + 2 * Cfg::BK <= g.KRED;
 #pragma unroll
         for (int i = 0; i < Cfg::A_VEC; i++) {
             KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
@@ -90,7 +90,7 @@ struct PoseKcLoader {
             }
             slot[i].advance(wp, go);
         }
-        k0 += (KPAD || go) ? Cfg::BK : 0;
+        k0 += go ? Cfg::BK : 0;
     }
     template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
@@ -129,7 +129,7 @@ struct PoseWeightRcLoader {
     }
     template <int S>
     __device__ __forceinline__ void fetch() {
-        const bool go = k0 + 2 * Cfg::BK <= g.KRED;
+        const bool go = KPAD || k0 + 2 * Cfg::BK <= g.KRED;
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
@@ -143,7 +143,7 @@ struct PoseWeightRcLoader {
             }
             slot[i].advance(wp, go);
         }
-        k0 += (KPAD || go) ? Cfg::BK : 0;
+        k0 += go ? Cfg::BK : 0;
     }
     template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
@@ -177,6 +177,116 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) capsule_kernel(const CapsuleArg
         drain<Cfg>(acc, [&](int row, int col, v4f v) { map.store(m0 + row, n0 + col, v); });
     } else {
         store_partial<Cfg>(acc, g.scratch, split, m0, n0, g.Mp, g.Np);
+    }
+}
+
+// Small batches: the benchmark shape has 196 tiles of 32 x 128 votes, fewer than the 256 CUs, and a
+// reduction that is split over workgroups pays for a second kernel and for the partial planes.
+// Here one workgroup of 8 waves owns one 32 x 128 tile and splits the reduction over its waves
+// instead.  No operand is shared between waves, so nothing is staged in LDS: a lane loads its pose
+// row (4 mk, 128 bits) and its weight rows (4 my each) straight into the MFMA operand registers,
+// two steps ahead of their use, and the only synchronisation is the final sum of the 8 partial
+// tiles through LDS (in wave order, so the result does not depend on timing).
+//   step = 2 pose rows q of the reduction (lanes 0-31: q, lanes 32-63: q+1) = 16 MFMAs
+constexpr int DIRECT_WAVES = 8;
+constexpr int DIRECT_RING = 3;            // operand register sets; loads run RING-1 steps ahead
+constexpr int DIRECT_RED_STRIDE = 69;     // float4 per accumulator register row in LDS (64 lanes, padded)
+constexpr int DIRECT_RED_HI = 36;         // offset of lanes 32-63 inside a row
+__global__ void __launch_bounds__(DIRECT_WAVES * 64) capsule_direct_kernel(const CapsuleArgs g) {
+    extern __shared__ __align__(16) float smem[];
+    constexpr int NW = DIRECT_WAVES, R = DIRECT_RING;
+    v4f *red = reinterpret_cast<v4f *>(smem);
+    int *tab_p = reinterpret_cast<int *>(smem + NW * 16 * DIRECT_RED_STRIDE * 4);
+    int *tab_w = tab_p + g.KH * g.KW;
+    fill_window_table(tab_p, g.KH, g.KW, (int)g.sp[2], (int)g.sp[3]);
+    fill_window_table(tab_w, g.KH, g.KW, (int)g.sw[2], (int)g.sw[3]);
+    __syncthreads();
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
+    const int tm = blockIdx.x / g.tiles_n, tn = blockIdx.x - tm * g.tiles_n;
+    const int m0 = tm * 32, n0 = tn * 128;
+
+    // pose rows [2*s0, qb) of the reduction belong to this wave
+    const int Q = g.KRED >> 2, steps = (Q + 1) >> 1;
+    const int s0 = (int)((int64_t)steps * wave / NW), s1 = (int)((int64_t)steps * (wave + 1) / NW);
+    const int qb = min(2 * s1, Q);
+    int qi = 2 * s0 + lhi;                 // pose row of this lane's next load
+
+    int row = m0 + l32;
+    if (row >= g.ROWS) row = 0;
+    const int mx = row % g.MX, pix = row / g.MX;
+    const int w = pix % g.OW, h = (pix / g.OW) % g.OH, n = pix / (g.OW * g.OH);
+    const int base_p = (int)(n * g.sp[0] + h * g.S * g.sp[2] + w * g.S * g.sp[3] + mx * g.sp[4]);
+    int co = (n0 >> 2) + l32;
+    if (co * 4 >= g.COLS) co = 0;
+    const int base_w = (int)(co * g.sw[0]);
+    const int mk_stride = (int)g.sw[4];
+
+    WindowParams wpp, wpw;
+    wpp.tab = tab_p; wpw.tab = tab_w;
+    wpp.win = wpw.win = g.KH * g.KW;
+    wpp.stride_c = (int)g.sp[1]; wpw.stride_c = (int)g.sw[1];
+    wpp.step_r = wpw.step_r = 2 % wpp.win;
+    wpp.step_coff = (2 / wpp.win) * wpp.stride_c;
+    wpw.step_coff = (2 / wpw.win) * wpw.stride_c;
+    WindowSlot slp, slw;
+    slp.init(wpp, min(qi, Q - 1));
+    slw.init(wpw, min(qi, Q - 1));
+
+    v4f ra[R], rb[R][4];
+    bool live[R];   // false: the set lies past the end of this wave's range and must add nothing
+    auto issue = [&](int d) {
+        live[d] = qi < qb;
+        ra[d] = *reinterpret_cast<const v4f *>(g.P + (uint32_t)(base_p + slp.offset()));
+        const float *pb = g.W + (uint32_t)(base_w + slw.offset());
+#pragma unroll
+        for (int j = 0; j < 4; j++) rb[d][j] = *reinterpret_cast<const v4f *>(pb + j * mk_stride);
+        const bool go = qi + 2 < Q;
+        slp.advance(wpp, go);
+        slw.advance(wpw, go);
+        qi += 2;
+    };
+    v16f acc[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[c][r] = 0.f;
+
+#pragma unroll
+    for (int d = 0; d < R - 1; d++) {
+        issue(d);
+        __builtin_amdgcn_sched_barrier(0);   // keep the sets in program order: waits count loads
+    }
+    const int iters = (s1 - s0 + R - 1) / R;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int d = 0; d < R; d++) {
+            issue((d + R - 1) % R);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float a = live[d] ? ra[d][j] : 0.f;
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                    acc[c] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, rb[d][j][c], acc[c], 0, 0, 0);
+            }
+            T2SP_INTERLEAVE(SG_VMEM_READ, 5, 3)
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // sum the 8 partial tiles in wave order
+    v4f *mine = red + wave * 16 * DIRECT_RED_STRIDE + lhi * DIRECT_RED_HI + l32;
+#pragma unroll
+    for (int r = 0; r < 16; r++)
+        mine[r * DIRECT_RED_STRIDE] = v4f{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+    __syncthreads();
+    CapsuleOutMap map{g.V, g.OH, g.OW, g.MX, g.ROWS, g.COLS, {g.sv[0], g.sv[1], g.sv[2], g.sv[3], g.sv[4]}};
+    for (int r = wave; r < 16; r += NW) {
+        const v4f *src = red + r * DIRECT_RED_STRIDE + lhi * DIRECT_RED_HI + l32;
+        v4f sum = src[0];
+#pragma unroll
+        for (int wv = 1; wv < NW; wv++) sum += src[wv * 16 * DIRECT_RED_STRIDE];
+        map.store(m0 + 8 * (r >> 2) + 4 * lhi + (r & 3), n0 + 4 * l32, sum);
     }
 }
 
@@ -217,6 +327,8 @@ using CapsS = TileCfg<64, 128, 16, 2, 1, STYLE_RC>;
 using CapsL = TileCfg<256, 256, 16, 4, 2, STYLE_RC>;
 using CapsW = TileCfg<32, 128, 16, 1, 1, STYLE_RC>;   // one wave per tile
 
+constexpr int DIRECT_MAX_TILES = 384;   // beyond this the LDS-tiled kernels win (operands shared)
+
 struct CapsulePlan {
     int cfg, splits, Mp, Np;
     size_t scratch_bytes;
@@ -224,6 +336,16 @@ struct CapsulePlan {
 
 static CapsulePlan plan_capsule(int rows, int cols, int kred, int cfg, int splits) {
     CapsulePlan p{};
+    if (cfg == T2SP_CFG_AUTO) {
+        const int64_t t32 = (int64_t)((rows + 31) / 32) * ((cols + 127) / 128);
+        if (t32 <= DIRECT_MAX_TILES) cfg = T2SP_CFG_DIRECT;
+    }
+    if (cfg == T2SP_CFG_DIRECT) {
+        p.cfg = cfg; p.splits = 1;
+        p.Mp = (rows + 31) / 32 * 32;
+        p.Np = (cols + 127) / 128 * 128;
+        return p;
+    }
     if (cfg == T2SP_CFG_AUTO) {
         const int64_t t128 = (int64_t)((rows + 127) / 128) * ((cols + 127) / 128);
         const int64_t t256 = (int64_t)((rows + 255) / 256) * ((cols + 255) / 256);
@@ -245,6 +367,17 @@ static CapsulePlan plan_capsule(int rows, int cols, int kred, int cfg, int split
     p.Np = (cols + bn - 1) / bn * bn;
     p.scratch_bytes = splits > 1 ? (size_t)splits * p.Mp * p.Np * sizeof(float) : 0;
     return p;
+}
+
+static int launch_capsule_direct(CapsuleArgs g, hipStream_t stream) {
+    g.tiles_m = g.Mp / 32;
+    g.tiles_n = g.Np / 128;
+    const size_t smem = (size_t)DIRECT_WAVES * 16 * DIRECT_RED_STRIDE * sizeof(v4f) + 2 * (size_t)g.KH * g.KW * sizeof(int);
+    if (smem > 160 * 1024) return T2SP_ERR_SHAPE;
+    if (hipFuncSetAttribute((const void *)capsule_direct_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+        return T2SP_ERR_LAUNCH;
+    hipLaunchKernelGGL(capsule_direct_kernel, dim3(g.tiles_m * g.tiles_n), dim3(DIRECT_WAVES * 64), smem, stream, g);
+    return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
 }
 
 template <class Cfg>
@@ -320,6 +453,7 @@ extern "C" int t2sp_capsule_f32(const float *P, const float *W, float *V, const 
     g.ROWS = (int)rows; g.COLS = (int)cols; g.KRED = (int)kred;
     g.splits = p.splits; g.Mp = p.Mp; g.Np = p.Np; g.scratch = workspace;
     switch (p.cfg) {
+        case T2SP_CFG_DIRECT: return launch_capsule_direct(g, (hipStream_t)stream);
         case T2SP_CFG_256x256: return launch_capsule<CapsL>(g, (hipStream_t)stream);
         case T2SP_CFG_128x128: return launch_capsule<CapsM>(g, (hipStream_t)stream);
         case T2SP_CFG_64x128: return launch_capsule<CapsS>(g, (hipStream_t)stream);

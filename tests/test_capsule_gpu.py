@@ -20,7 +20,7 @@ def test_constant_fixture_exact():
     assert V.shape == (2, 8, 7, 7, 4, 4) and (V == 1152).all()
 
 
-@pytest.mark.parametrize("cfg,splits", [(0, 0), (2, 1), (2, 3), (3, 2), (1, 2), (99, 0)])
+@pytest.mark.parametrize("cfg,splits", [(0, 0), (5, 0), (2, 1), (2, 3), (3, 2), (4, 2), (1, 2), (99, 0)])
 def test_tiny_constants_parity_golden_and_ure_order(oracle, cfg, splits):
     """The TINY sizes of capsule/const-parameters.h:43-52 with N=4 (capsule-run-fpga.cpp:37-39):
     16 -> 16 channels, 15x15 -> 7x7, against both reduction orders the reference uses."""
@@ -56,6 +56,17 @@ def test_oneapi_memory_layout_and_other_strides(oracle):
         Ps = oracle.fill_uniform((1, 4, iy, iy, 4, 4), 6)
         got = t2sp_amd.capsule(Ps, W[:, :4], stride=s)
         assert rel_fro(got, oracle.capsule(Ps, np.ascontiguousarray(W[:, :4]), stride=s))[0] <= TOL
+
+
+@pytest.mark.parametrize("ci,co,n", [(1, 3, 1), (3, 40, 2), (5, 8, 3), (7, 33, 1)])
+@pytest.mark.parametrize("cfg", [5, 2])
+def test_short_and_odd_reductions_ragged_columns(oracle, ci, co, n, cfg):
+    """Reductions of an odd number of pose rows (CI*9 odd), shorter than the number of waves
+    that share them, and vote columns that do not fill a 128-column tile."""
+    P, W = oracle.fill_uniform((n, ci, 9, 7, 4, 4), 30 + ci), oracle.fill_uniform((co, ci, 3, 3, 4, 4), 40 + co)
+    got = t2sp_amd.capsule(P, W, cfg=cfg, splits=1)
+    err, mx = rel_fro(got, oracle.capsule(P, W))
+    assert err <= TOL, (ci, co, n, cfg, err, mx)
 
 
 def test_other_pose_sizes_take_the_scalar_kernel(oracle):
