@@ -182,70 +182,73 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) capsule_kernel(const CapsuleArg
 
 // Small batches: the benchmark shape has 196 tiles of 32 x 128 votes, fewer than the 256 CUs, and a
 // reduction that is split over workgroups pays for a second kernel and for the partial planes.
-// Here one workgroup of 8 waves owns one 32 x 128 tile and splits the reduction over its waves
+// Here one workgroup of 4 waves owns one 32 x 128 tile and splits the reduction over its waves
 // instead.  No operand is shared between waves, so nothing is staged in LDS: a lane loads its pose
 // row (4 mk, 128 bits) and its weight rows (4 my each) straight into the MFMA operand registers,
-// two steps ahead of their use, and the only synchronisation is the final sum of the 8 partial
-// tiles through LDS (in wave order, so the result does not depend on timing).
+// ahead of their use, and the only synchronisation is the final sum of the partial tiles
+// through LDS (in wave order, so the result does not depend on timing).
 //   step = 2 pose rows q of the reduction (lanes 0-31: q, lanes 32-63: q+1) = 16 MFMAs
-constexpr int DIRECT_WAVES = 8;
+// The offsets of the pose rows q = (ci, kh, kw) are the same for all lanes up to a per-lane constant,
+// so their offsets are tabulated once per wave.
+constexpr int DIRECT_WAVES = 4;
 constexpr int DIRECT_RING = 3;            // operand register sets; loads run RING-1 steps ahead
 constexpr int DIRECT_RED_STRIDE = 69;     // float4 per accumulator register row in LDS (64 lanes, padded)
 constexpr int DIRECT_RED_HI = 36;         // offset of lanes 32-63 inside a row
-__global__ void __launch_bounds__(DIRECT_WAVES * 64) capsule_direct_kernel(const CapsuleArgs g) {
+
+template <int NW, int R>
+__global__ void __launch_bounds__(NW * 64) capsule_direct_kernel(const CapsuleArgs g, int tab_entries) {
     extern __shared__ __align__(16) float smem[];
-    constexpr int NW = DIRECT_WAVES, R = DIRECT_RING;
     v4f *red = reinterpret_cast<v4f *>(smem);
-    int *tab_p = reinterpret_cast<int *>(smem + NW * 16 * DIRECT_RED_STRIDE * 4);
-    int *tab_w = tab_p + g.KH * g.KW;
-    fill_window_table(tab_p, g.KH, g.KW, (int)g.sp[2], (int)g.sp[3]);
-    fill_window_table(tab_w, g.KH, g.KW, (int)g.sw[2], (int)g.sw[3]);
-    __syncthreads();
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
     const int tm = blockIdx.x / g.tiles_n, tn = blockIdx.x - tm * g.tiles_n;
     const int m0 = tm * 32, n0 = tn * 128;
 
-    // pose rows [2*s0, qb) of the reduction belong to this wave
+    // steps [s0, s1) = pose rows [2*s0, qb) of the reduction belong to this wave
     const int Q = g.KRED >> 2, steps = (Q + 1) >> 1;
     const int s0 = (int)((int64_t)steps * wave / NW), s1 = (int)((int64_t)steps * (wave + 1) / NW);
     const int qb = min(2 * s1, Q);
-    int qi = 2 * s0 + lhi;                 // pose row of this lane's next load
+    const int nsteps = s1 - s0;
 
+    // Byte offsets, in P and in W, of the wave's pose rows q = (ci, kh, kw), tabulated once in a
+    // wave-private piece of LDS (rows past the end repeat the last one): the walk over the
+    // reduction then costs one LDS read per step.  Written and read by this wave only.
+    uint2 *tab = reinterpret_cast<uint2 *>(smem + NW * 16 * DIRECT_RED_STRIDE * 4) + wave * tab_entries;
+    for (int i = lane; i < 2 * nsteps + 2 * R; i += 64) {
+        const int q = min(2 * s0 + i, Q - 1);
+        const int c = q / (g.KH * g.KW), r = q - c * (g.KH * g.KW);
+        const int kh = r / g.KW, kw = r - kh * g.KW;
+        tab[i] = uint2{4u * (uint32_t)(c * (int)g.sp[1] + kh * (int)g.sp[2] + kw * (int)g.sp[3]),
+                       4u * (uint32_t)(c * (int)g.sw[1] + kh * (int)g.sw[2] + kw * (int)g.sw[3])};
+    }
+
+    int co = (n0 >> 2) + l32;
+    if (co * 4 >= g.COLS) co = 0;
+    const uint32_t w_lane = 4u * (uint32_t)(co * (int)g.sw[0]);
+    const char *w_base[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) w_base[j] = reinterpret_cast<const char *>(g.W + j * g.sw[4]);
     int row = m0 + l32;
     if (row >= g.ROWS) row = 0;
     const int mx = row % g.MX, pix = row / g.MX;
-    const int w = pix % g.OW, h = (pix / g.OW) % g.OH, n = pix / (g.OW * g.OH);
-    const int base_p = (int)(n * g.sp[0] + h * g.S * g.sp[2] + w * g.S * g.sp[3] + mx * g.sp[4]);
-    int co = (n0 >> 2) + l32;
-    if (co * 4 >= g.COLS) co = 0;
-    const int base_w = (int)(co * g.sw[0]);
-    const int mk_stride = (int)g.sw[4];
-
-    WindowParams wpp, wpw;
-    wpp.tab = tab_p; wpw.tab = tab_w;
-    wpp.win = wpw.win = g.KH * g.KW;
-    wpp.stride_c = (int)g.sp[1]; wpw.stride_c = (int)g.sw[1];
-    wpp.step_r = wpw.step_r = 2 % wpp.win;
-    wpp.step_coff = (2 / wpp.win) * wpp.stride_c;
-    wpw.step_coff = (2 / wpw.win) * wpw.stride_c;
-    WindowSlot slp, slw;
-    slp.init(wpp, min(qi, Q - 1));
-    slw.init(wpw, min(qi, Q - 1));
+    const int w = pix % g.OW, hn = pix / g.OW, h = hn % g.OH, n = hn / g.OH;
+    const uint32_t p_lane =
+        4u * (uint32_t)(int)(n * g.sp[0] + h * g.S * g.sp[2] + w * g.S * g.sp[3] + mx * g.sp[4]);
+    const char *p_base = reinterpret_cast<const char *>(g.P);
 
     v4f ra[R], rb[R][4];
-    bool live[R];   // false: the set lies past the end of this wave's range and must add nothing
-    auto issue = [&](int d) {
-        live[d] = qi < qb;
-        ra[d] = *reinterpret_cast<const v4f *>(g.P + (uint32_t)(base_p + slp.offset()));
-        const float *pb = g.W + (uint32_t)(base_w + slw.offset());
-#pragma unroll
-        for (int j = 0; j < 4; j++) rb[d][j] = *reinterpret_cast<const v4f *>(pb + j * mk_stride);
-        const bool go = qi + 2 < Q;
-        slp.advance(wpp, go);
-        slw.advance(wpw, go);
-        qi += 2;
-    };
+    const uint2 *tab_lane = tab + lhi;
+    uint2 off = tab_lane[0];   // offsets of the next set to load; the one after is read meanwhile
+    int t_issue = 0;
+#define T2SP_DIRECT_ISSUE(d)                                                                       \
+    {                                                                                              \
+        const uint32_t op = p_lane + off.x, ow = w_lane + off.y;                                   \
+        t_issue++;                                                                                 \
+        off = tab_lane[2 * t_issue];                                                               \
+        _Pragma("unroll") for (int j = 0; j < 4; j++)                                              \
+            rb[d][j] = *reinterpret_cast<const v4f *>(w_base[j] + ow);                             \
+        ra[d] = *reinterpret_cast<const v4f *>(p_base + op);                                       \
+    }
     v16f acc[4];
 #pragma unroll
     for (int c = 0; c < 4; c++)
@@ -254,27 +257,43 @@ __global__ void __launch_bounds__(DIRECT_WAVES * 64) capsule_direct_kernel(const
 
 #pragma unroll
     for (int d = 0; d < R - 1; d++) {
-        issue(d);
+        T2SP_DIRECT_ISSUE(d)
         __builtin_amdgcn_sched_barrier(0);   // keep the sets in program order: waits count loads
     }
-    const int iters = (s1 - s0 + R - 1) / R;
-    for (int it = 0; it < iters; it++) {
+    // All but the last 1..R steps run unguarded; only the tail can hold rows past the end of the
+    // wave's range (the reduction may be an odd number of pose rows), which must add nothing.
+    const int main_iters = nsteps > 0 ? (nsteps - 1) / R : 0;
+    const int rem = nsteps - main_iters * R;
+    for (int it = 0; it < main_iters; it++) {
 #pragma unroll
         for (int d = 0; d < R; d++) {
-            issue((d + R - 1) % R);
+            T2SP_DIRECT_ISSUE((d + R - 1) % R)
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const float a = live[d] ? ra[d][j] : 0.f;
+            for (int j = 0; j < 4; j++)
 #pragma unroll
                 for (int c = 0; c < 4; c++)
-                    acc[c] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, rb[d][j][c], acc[c], 0, 0, 0);
-            }
+                    acc[c] = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[d][j], rb[d][j][c], acc[c], 0, 0, 0);
             T2SP_INTERLEAVE(SG_VMEM_READ, 5, 3)
             __builtin_amdgcn_sched_barrier(0);
         }
     }
+    T2SP_DIRECT_ISSUE(R - 1)
+#undef T2SP_DIRECT_ISSUE
+#pragma unroll
+    for (int d = 0; d < R; d++) {
+        if (d < rem) {
+            const bool live = 2 * (s0 + main_iters * R + d) + lhi < qb;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float a = live ? ra[d][j] : 0.f;
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                    acc[c] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, rb[d][j][c], acc[c], 0, 0, 0);
+            }
+        }
+    }
 
-    // sum the 8 partial tiles in wave order
+    // sum the partial tiles of the waves in wave order
     v4f *mine = red + wave * 16 * DIRECT_RED_STRIDE + lhi * DIRECT_RED_HI + l32;
 #pragma unroll
     for (int r = 0; r < 16; r++)
@@ -327,7 +346,8 @@ using CapsS = TileCfg<64, 128, 16, 2, 1, STYLE_RC>;
 using CapsL = TileCfg<256, 256, 16, 4, 2, STYLE_RC>;
 using CapsW = TileCfg<32, 128, 16, 1, 1, STYLE_RC>;   // one wave per tile
 
-constexpr int DIRECT_MAX_TILES = 384;   // beyond this the LDS-tiled kernels win (operands shared)
+constexpr int DIRECT_MAX_KRED = 16384;   // its per-wave offset tables must fit in LDS
+constexpr int DIRECT_MAX_TILES = 4096;  // beyond this the LDS-tiled kernels win (operands shared)
 
 struct CapsulePlan {
     int cfg, splits, Mp, Np;
@@ -338,7 +358,12 @@ static CapsulePlan plan_capsule(int rows, int cols, int kred, int cfg, int split
     CapsulePlan p{};
     if (cfg == T2SP_CFG_AUTO) {
         const int64_t t32 = (int64_t)((rows + 31) / 32) * ((cols + 127) / 128);
-        if (t32 <= DIRECT_MAX_TILES) cfg = T2SP_CFG_DIRECT;
+        // Measured on the benchmark's channel counts at batch 8..1024: with fewer than ~100 tiles the
+        // reduction has to be split over workgroups to fill the chip; between one and one and a half
+        // rounds of 256 tiles the second round is mostly empty; very large batches reuse operands
+        // better through the shared LDS tiles.
+        const bool rounds_ok = t32 <= 256 || t32 >= 384;
+        if (t32 >= 100 && t32 <= DIRECT_MAX_TILES && rounds_ok && kred <= DIRECT_MAX_KRED) cfg = T2SP_CFG_DIRECT;
     }
     if (cfg == T2SP_CFG_DIRECT) {
         p.cfg = cfg; p.splits = 1;
@@ -369,14 +394,25 @@ static CapsulePlan plan_capsule(int rows, int cols, int kred, int cfg, int split
     return p;
 }
 
+// LDS of the direct kernel: the partial tiles of its waves plus their offset tables.
+static int direct_tab_entries(int kred) {
+    const int steps = (kred / 4 + 1) / 2;
+    return 2 * ((steps + DIRECT_WAVES - 1) / DIRECT_WAVES) + 2 * DIRECT_RING + 2;
+}
+static size_t direct_smem_bytes(int kred) {
+    return (size_t)DIRECT_WAVES * (16 * DIRECT_RED_STRIDE * sizeof(v4f) + direct_tab_entries(kred) * sizeof(uint2));
+}
+
 static int launch_capsule_direct(CapsuleArgs g, hipStream_t stream) {
     g.tiles_m = g.Mp / 32;
     g.tiles_n = g.Np / 128;
-    const size_t smem = (size_t)DIRECT_WAVES * 16 * DIRECT_RED_STRIDE * sizeof(v4f) + 2 * (size_t)g.KH * g.KW * sizeof(int);
+    const size_t smem = direct_smem_bytes(g.KRED);
     if (smem > 160 * 1024) return T2SP_ERR_SHAPE;
-    if (hipFuncSetAttribute((const void *)capsule_direct_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+    auto kern = capsule_direct_kernel<DIRECT_WAVES, DIRECT_RING>;
+    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
-    hipLaunchKernelGGL(capsule_direct_kernel, dim3(g.tiles_m * g.tiles_n), dim3(DIRECT_WAVES * 64), smem, stream, g);
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(DIRECT_WAVES * 64), smem, stream, g,
+                       direct_tab_entries(g.KRED));
     return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
 }
 
@@ -401,7 +437,7 @@ static int launch_capsule(CapsuleArgs g, hipStream_t stream) {
 }  // namespace t2sp
 
 static bool capsule_fast(const int *d, const int64_t *sp6, const int64_t *sw6, const int64_t *sv6,
-                         const float *P, const float *W, const float *V) {
+                         const float *P, const float *W, const float *V, bool *byte_offsets_fit) {
     const int MY = d[9], MK = d[10];
     if (MY != 4 || MK != 4 || d[5] * d[6] > 4096) return false;
     // 32-bit element offsets: every tensor must span fewer than 2^31 elements
@@ -411,6 +447,7 @@ static bool capsule_fast(const int *d, const int64_t *sp6, const int64_t *sw6, c
     const int64_t span_w = (int64_t)(d[2] - 1) * sw6[0] + (int64_t)(d[1] - 1) * sw6[1] + (int64_t)(d[5] - 1) * sw6[2] +
                            (int64_t)(d[6] - 1) * sw6[3] + 3 * sw6[4] + 3;
     if (span_p >= INT32_MAX || span_w >= INT32_MAX) return false;
+    *byte_offsets_fit = span_p < (1 << 30) && span_w < (1 << 30);   // the direct kernel's 32-bit byte offsets
     if (sp6[5] != 1 || sw6[5] != 1 || sv6[5] != 1) return false;
     for (int i = 0; i < 5; i++)
         if (sp6[i] % 4 || sw6[i] % 4 || sv6[i] % 4) return false;
@@ -436,7 +473,8 @@ extern "C" int t2sp_capsule_f32(const float *P, const float *W, float *V, const 
     const int64_t rows = (int64_t)d[0] * d[3] * d[4] * d[8], cols = (int64_t)d[2] * 4,
                   kred = (int64_t)d[1] * d[5] * d[6] * 4;
     if (rows > INT32_MAX / 2 || cols > INT32_MAX / 2 || kred > INT32_MAX / 2) return T2SP_ERR_SHAPE;
-    if (cfg == T2SP_CFG_SCALAR || !capsule_fast(d, sp6, sw6, sv6, P, W, V)) {
+    bool byte_offsets_fit = false;
+    if (cfg == T2SP_CFG_SCALAR || !capsule_fast(d, sp6, sw6, sv6, P, W, V, &byte_offsets_fit)) {
         CapsuleGenericArgs a{P, W, V, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], d[8], d[9], d[10], {}, {}, {}};
         for (int i = 0; i < 6; i++) { a.sp[i] = sp6[i]; a.sw[i] = sw6[i]; a.sv[i] = sv6[i]; }
         const int64_t total = (int64_t)d[0] * d[2] * d[3] * d[4] * d[8] * d[9];
@@ -444,7 +482,9 @@ extern "C" int t2sp_capsule_f32(const float *P, const float *W, float *V, const 
         hipLaunchKernelGGL(capsule_scalar_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
         return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
     }
-    const CapsulePlan p = plan_capsule((int)rows, (int)cols, (int)kred, cfg, splits);
+    CapsulePlan p = plan_capsule((int)rows, (int)cols, (int)kred, cfg, splits);
+    if (p.cfg == T2SP_CFG_DIRECT && !(byte_offsets_fit && direct_smem_bytes((int)kred) <= 160 * 1024))
+        p = plan_capsule((int)rows, (int)cols, (int)kred, T2SP_CFG_128x128, 1);   // needs no workspace either
     if (p.scratch_bytes > workspace_bytes || (p.scratch_bytes && !workspace)) return T2SP_ERR_SHAPE;
     CapsuleArgs g{};
     g.P = P; g.W = W; g.V = V;
