@@ -69,6 +69,29 @@ int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, float alpha, 
                       int64_t ldcin, float *C, int64_t ldc, int cfg, float *workspace,
                       size_t workspace_bytes, void *stream);
 
+/* D = alpha * A * A^T + beta * Cin, fp32, A row-major N x K (K x N when trans is non-zero: it is
+ * then first re-laid into `workspace`, t2sp_ssyrk_workspace_bytes).  Only tiles on or above the
+ * diagonal are multiplied.  Flat form: C row-major N x N; `upper` selects the triangle of BLAS
+ * semantics; mirror = 0 writes that triangle only, 1 writes both triangles with Cin read from the
+ * `upper` triangle (a symmetric result, what the reference's ssyrk wrapper returns,
+ * t2s/peppers/blas/level3/syrk/release/s10/blas-syrk.cpp:75-86), 2 writes both with Cin read
+ * where C is written (the pipeline's own semantics, t2s/tests/performance/syrk/syrk.cpp:72).
+ * Cin may be NULL (beta ignored) or equal to C.  Folded form: the reference's 6-D output
+ * Out(jjj, iii, jj, ii, j, i) with block edge iii*ii (syrk-run-fpga.cpp:62, syrk.cpp:37-46);
+ * N must be an even number of blocks; with a workspace of t2sp_ssyrk_folded_workspace_bytes the
+ * matrix is first formed flat and then folded (several times faster than folding in the
+ * product's epilogue, which is what happens without one).  Replaces the device side of the reference's SYRK pipeline
+ * (t2s/tests/performance/syrk/syrk.cpp:59-72, syrk/a.cl). */
+size_t t2sp_ssyrk_workspace_bytes(int trans, int N, int K);
+size_t t2sp_ssyrk_folded_workspace_bytes(int trans, int N, int K);
+int t2sp_ssyrk_f32(int upper, int trans, int N, int K, float alpha, const float *A, int64_t lda, float beta,
+                   const float *Cin, int64_t ldcin, float *C, int64_t ldc, int mirror, int cfg,
+                   float *workspace, size_t workspace_bytes, void *stream);
+int t2sp_ssyrk_f32_folded(int trans, int N, int K, float alpha, const float *A, int64_t lda, float beta,
+                          const float *Cin, int64_t ldcin, float *Out, int iii, int ii,
+                          const int64_t *strides6, int cfg, float *workspace, size_t workspace_bytes,
+                          void *stream);
+
 /* O[n,co,h,w] = sum_{ci,kh,kw} I[n,ci,h+kh,w+kw] * W[co,ci,kh,kw], stride 1, valid
  * padding, fp32.  si4/sw4/so4 are element strides of the logical indices
  * (n,ci,h,w), (co,ci,kh,kw), (n,co,h,w); "w" is the innermost spatial axis (the

@@ -18,6 +18,10 @@
  *   oracle_capsule   golden loop  capsule/capsule-run-fpga.cpp:78-104, capsule-run-gpu.cpp:43-71,
  *                                 oneapi/src/oneapi-target-6-run.cpp:131-173 (kx -> ky -> mk -> ci);
  *                    URE order    capsule/capsule.cpp:28,60-66 (mk -> ci -> kx -> ky -> cii).
+ *   oracle_syrk      golden loop  t2s/tests/performance/syrk/syrk-run-fpga.cpp:84-90 and
+ *                                 t2s/peppers/blas/level3/syrk/release/s10/ssyrk-run-fpga.cpp:45-54
+ *                                 (golden = beta*c; golden += alpha*a*b over ascending k).  The folded
+ *                                 output layout (syrk.cpp:37-46) is restated in oracle.py.
  *   oracle_mttkrp    golden       t2s/tests/performance/util/util.h:498-515 (two-step: TTM over l
  *                                 into e(i,j,k), then d += e*b over k).  The reference's outer loop
  *                                 bound `i < K` (util.h:502) is only right when I == K; this
@@ -321,6 +325,27 @@ void oracle_mttkrp_literal(const float *a, const float *b, const float *c, float
                 dij += e * b[k + K * j];
             }
             d[i + I * j] = dij;
+        }
+}
+
+/* ------------------------------------------------------------------------- */
+/* D[i,j] = beta*C[i,j] + sum_k alpha*A[i,k]*A[j,k] for every (i, j), in the golden loop's order
+ * and grouping: "golden = beta * cc; golden += alpha * aa * bb" = (alpha*aa)*bb added one k at a
+ * time (syrk-run-fpga.cpp:84-90).  A is row-major N x K with row stride lda, C and D N x N with
+ * row strides ldc / ldd.  C is read at (i, j) itself, so it need not be symmetric.  Rows
+ * [row0, row0 + nrows). */
+void oracle_syrk(const float *A, const float *C, float *D, int64_t N, int64_t K, int64_t lda, int64_t ldc,
+                 int64_t ldd, float alpha, float beta, int64_t row0, int64_t nrows, int threads) {
+    set_threads(threads);
+#pragma omp parallel for schedule(static)
+    for (int64_t i = row0; i < row0 + nrows; i++)
+        for (int64_t j = 0; j < N; j++) {
+            float golden = beta * C[i * ldc + j];
+            for (int64_t k = 0; k < K; k++) {
+                const float t = alpha * A[i * lda + k];
+                golden += t * A[j * lda + k];
+            }
+            D[i * ldd + j] = golden;
         }
 }
 

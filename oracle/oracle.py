@@ -42,6 +42,8 @@ def lib():
         _lib.oracle_mttkrp.argtypes = [fp, fp, fp, fp, ip, ip, ip, ip, ip, i64, i64, ctypes.c_int,
                                        ctypes.c_int]
         _lib.oracle_mttkrp_literal.argtypes = [fp, fp, fp, fp] + [i64] * 6
+        _lib.oracle_syrk.argtypes = [fp, fp, fp] + [i64] * 5 + [ctypes.c_float, ctypes.c_float, i64, i64, ctypes.c_int]
+        _lib.oracle_syrk.restype = None
         _lib.oracle_max_threads.restype = ctypes.c_int
         for f in (_lib.oracle_fill_uniform, _lib.oracle_gemm, _lib.oracle_gemm_literal,
                   _lib.oracle_conv, _lib.oracle_capsule, _lib.oracle_mttkrp,
@@ -167,6 +169,71 @@ def mttkrp_literal(a, b, c, i_range=None):
     i0, i1 = (0, I) if i_range is None else i_range
     lib().oracle_mttkrp_literal(_p(a), _p(b), _p(c), _p(d), L, I, J, K, i0, i1)
     return d
+
+
+def syrk(A, C, alpha, beta, rows=None, threads=0):
+    """alpha * A @ A.T + beta * C in the golden loop's order (syrk-run-fpga.cpp:84-90), all N x N
+    elements (or the given (row0, nrows) rows)."""
+    A = np.ascontiguousarray(A)
+    C = np.ascontiguousarray(C)
+    N, K = A.shape
+    row0, nrows = (0, N) if rows is None else rows
+    D = np.zeros((nrows, N), dtype=np.float32)
+    lib().oracle_syrk(_p(A), _p(C), D.ctypes.data - row0 * N * 4, N, K, K, N, N, alpha, beta, row0, nrows, threads)
+    return D
+
+
+def syrk_fold(D, III, II, fill=np.nan):
+    """The folded output Out(jjj, iii, jj, ii, j, i) -- numpy shape (I, I+1, II, II, III, III) -- that
+    the SYRK pipeline leaves for the N x N result D, restated from the pipeline's own index
+    expressions (syrk.cpp:37-46,59-72,80-86): block rows i < I/2; bottom blocks (i >= j) hold
+    D[N-1-total_i, N-1-total_j], top blocks D[total_i, total_j - III*II].  Positions the pipeline
+    never writes keep `fill`."""
+    N = D.shape[0]
+    B = III * II
+    I = N // B
+    assert N == B * I and I % 2 == 0
+    out = np.full((I, I + 1, II, II, III, III), fill, dtype=np.float32)
+    for i in range(I // 2):
+        for j in range(I + 1):
+            for ii in range(II):
+                for jj in range(II):
+                    for iii in range(III):
+                        for jjj in range(III):
+                            ti = iii + III * ii + B * i
+                            tj = jjj + III * jj + B * j
+                            if i >= j:
+                                r, c = N - 1 - ti, N - 1 - tj
+                            else:
+                                r, c = ti, tj - B
+                            out[i, j, ii, jj, iii, jjj] = D[r, c]
+    return out
+
+
+def syrk_unfold_upper(out, III, II):
+    """The upper triangle (zeros below it) read back from a folded output the way the reference's BLAS
+    wrapper does (t2s/peppers/blas/level3/syrk/release/s10/blas-syrk.cpp:49-73) -- an index
+    mapping written independently of syrk_fold's."""
+    I = out.shape[0]
+    B = III * II
+    N = B * I
+    D = np.zeros((N, N), dtype=np.float32)
+    for i in range(I):
+        for j in range(I):
+            for ii in range(II):
+                for jj in range(II):
+                    for iii in range(III):
+                        for jjj in range(III):
+                            ti = iii + III * ii + B * i
+                            tj = jjj + III * jj + B * j
+                            if ti > tj:
+                                continue
+                            if i * 2 < I:
+                                D[ti, tj] = out[i, j + 1, ii, jj, iii, jjj]
+                            else:
+                                D[ti, tj] = out[I - i - 1, I - j - 1, II - ii - 1, II - jj - 1, III - iii - 1,
+                                                III - jjj - 1]
+    return D
 
 
 def max_threads():

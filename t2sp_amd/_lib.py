@@ -48,6 +48,18 @@ def _declare(L):
     L.t2sp_sgemm_ex_workspace_bytes.restype = ctypes.c_size_t
     L.t2sp_sgemm_ex_f32.argtypes = [i32, i32, i32, i32, i32, f32, vp, i64, vp, i64, f32, vp, i64, vp, i64, i32, vp,
                                     ctypes.c_size_t, vp]
+    L.syrk.argtypes = [i32, f32, f32, bp, bp, bp]
+    L.t2sp_syrk_with_cfg.argtypes = [i32, f32, f32, bp, bp, bp, i32]
+    L.syrk_ns.argtypes = [i32, f32, f32, bp, bp, bp]
+    L.syrk_ns.restype = ctypes.c_double
+    L.t2sp_ssyrk_workspace_bytes.argtypes = [i32, i32, i32]
+    L.t2sp_ssyrk_workspace_bytes.restype = ctypes.c_size_t
+    L.t2sp_ssyrk_folded_workspace_bytes.argtypes = [i32, i32, i32]
+    L.t2sp_ssyrk_folded_workspace_bytes.restype = ctypes.c_size_t
+    L.t2sp_ssyrk_f32.argtypes = [i32, i32, i32, i32, f32, vp, i64, f32, vp, i64, vp, i64, i32, i32, vp,
+                                 ctypes.c_size_t, vp]
+    L.t2sp_ssyrk_f32_folded.argtypes = [i32, i32, i32, f32, vp, i64, f32, vp, i64, vp, i32, i32,
+                                        ctypes.POINTER(i64), i32, vp, ctypes.c_size_t, vp]
     L.conv.argtypes = [bp, bp, bp]
     L.t2sp_conv_with_cfg.argtypes = [bp, bp, bp, i32]
     p64, p32 = ctypes.POINTER(i64), ctypes.POINTER(i32)

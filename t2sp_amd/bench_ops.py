@@ -102,7 +102,30 @@ def mttkrp_config5(torch, steps, warmup, peak):
                   note="includes the split-reduction kernel")
 
 
+def ssyrk_8192(torch, steps, warmup, peak):
+    """Not a BASELINE configuration: the SYRK pipeline (t2s/tests/performance/syrk) at the headline
+    GEMM size.  Only the tiles on or above the diagonal are multiplied; the rate counts the
+    N*(N+1)/2 distinct outputs (N*(N+1)*K flop).  The reference's own report counts 2*N*N*K
+    (syrk-run-fpga.cpp:99), given as `TFLOP/s_reference_count`."""
+    L = lib()
+    N = K = 8192
+    A = ops.fill_uniform(torch.empty(N, K, device="cuda"), 1)
+    C = ops.fill_uniform(torch.empty(N, N, device="cuda"), 2)
+    O = torch.empty(N, N, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        rc = L.t2sp_ssyrk_f32(1, 0, N, K, 1.5, A.data_ptr(), K, 0.5, C.data_ptr(), N, O.data_ptr(), N, 1, 0, None, 0, s)
+        assert rc == 0, rc
+
+    ms = _time(torch, launch, steps, warmup)
+    flop = float(N) * (N + 1) * K
+    return _entry(flop / ms / 1e9, peak, ms, workload="N=K=8192, both triangles written, alpha/beta epilogue",
+                  **{"TFLOP/s_reference_count": round(2.0 * N * N * K / ms / 1e9, 3)})
+
+
 def run_all(torch, steps, warmup, peak):
     return {"conv2d": conv_config3(torch, steps, warmup, peak),
             "capsule": capsule_config4(torch, steps, warmup, peak),
-            "mttkrp": mttkrp_config5(torch, steps, warmup, peak)}
+            "mttkrp": mttkrp_config5(torch, steps, warmup, peak),
+            "ssyrk_8192": ssyrk_8192(torch, steps, warmup, peak)}

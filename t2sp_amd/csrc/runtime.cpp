@@ -144,7 +144,7 @@ int Staged::input(const halide_buffer_t *b, const Span &s, const char *op) {
     return 0;
 }
 
-int Staged::output(halide_buffer_t *b, const Span &s, const char *op) {
+int Staged::output(halide_buffer_t *b, const Span &s, const char *op, bool partial) {
     span_ = s.span;
     out_ = b;
     const size_t bytes = (size_t)s.span * sizeof(float);
@@ -155,7 +155,7 @@ int Staged::output(halide_buffer_t *b, const Span &s, const char *op) {
     ptr_ = static_cast<float *>(pool().get(bytes));
     if (!ptr_) return report(halide_error_code_device_malloc_failed, op, "device allocation failed");
     pooled_ = true;
-    if (s.span != s.elements && bytes)
+    if ((partial || s.span != s.elements) && bytes)
         if (hipMemcpyAsync(ptr_, b->host, bytes, hipMemcpyHostToDevice, api_stream()) != hipSuccess)
             return report(halide_error_code_copy_to_device_failed, op, "host to device copy failed");
     return 0;

@@ -72,7 +72,8 @@ public:
     int input(const halide_buffer_t *b, const Span &s, const char *op);
     // Output: use b->device when present, else pool memory (pre-filled from the
     // host when the buffer is not dense, so that gaps keep their contents).
-    int output(halide_buffer_t *b, const Span &s, const char *op);
+    // `partial`: the kernels write only part of the buffer; the rest must keep what it holds.
+    int output(halide_buffer_t *b, const Span &s, const char *op, bool partial = false);
     // After the kernels: copy a pool-backed output down to the host, or mark a
     // caller-staged one device_dirty.
     int finish(const char *op);

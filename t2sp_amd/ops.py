@@ -77,6 +77,31 @@ def gemm_ex(opa, opb, alpha, beta, A, B, C=None, out=None, tiles=None):
     return out
 
 
+def syrk(A, C, alpha, beta, out=None, fold=None, opa=0, cfg=0):
+    """Out = alpha * A @ A.T + beta * C through the `syrk` entry point (include/syrk-interface.h).
+
+    A: (N, K) row-major, or (K, N) when opa; C: (N, N) or None (beta ignored).  With
+    fold=(III, II) the result is the reference's folded triangle, numpy shape
+    (I, I+1, II, II, III, III) of which rows i < I/2 are written
+    (t2s/tests/performance/syrk/syrk-run-fpga.cpp:62); a freshly allocated one is filled with NaN
+    first.  Otherwise the whole (N, N) matrix."""
+    N = A.shape[1] if opa else A.shape[0]
+    if out is None:
+        if fold is None:
+            out = _empty_like_kind(A, (N, N))
+        else:
+            III, II = fold
+            assert N % (III * II) == 0
+            I = N // (III * II)
+            out = _empty_like_kind(A, (I, I + 1, II, II, III, III))
+            out[...] = float("nan")
+    a, o = HalideBuffer.wrap(A), HalideBuffer.wrap(out)
+    c = HalideBuffer.wrap(C) if C is not None else None
+    _check("syrk", lib().t2sp_syrk_with_cfg(int(bool(opa)), float(alpha), float(beta), a.ref,
+                                             c.ref if c is not None else None, o.ref, int(cfg)))
+    return out
+
+
 def conv(I, W, out=None, cfg=0):
     """O = conv2d(I, W), stride 1, no padding, through the `conv` entry point
     (include/conv-interface.h).

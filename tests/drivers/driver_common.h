@@ -24,10 +24,13 @@ struct Rng {
 struct Check {
     long checked = 0, bad = 0;
     double worst = 0.0;
+    // absolute slack for outputs that cancel to nearly zero (the reference's drivers use positive
+    // inputs, where a purely relative bound is enough)
+    double slack = 1e-6;
     void one(float golden, float got) {
         checked++;
         const double err = std::fabs((double)golden - (double)got);
-        const double lim = 0.005 * std::fabs((double)golden) + 1e-6;
+        const double lim = 0.005 * std::fabs((double)golden) + slack;
         if (err > worst) worst = err;
         if (!(err <= lim)) {
             if (bad < 5) std::printf("mismatch: golden %.9g got %.9g\n", golden, got);

@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol():
     assert {"gemm", "GEMM", "t2sp_sgemm_f32", "t2sp_last_kernel_ns"} <= names
     # sgemm and the Roofline.h helpers have C++ linkage, like the reference's own headers: look their
     # mangled names up instead
-    mangled = {"sgemm": "_Z5sgemmcciiifPfiS_ifS_i", "DSPs": "_Z4DSPsv", "FMax": "_Z4FMaxv",
+    mangled = {"sgemm": "_Z5sgemmcciiifPfiS_ifS_i", "ssyrk": "_Z5ssyrkcciifPfifS_i", "DSPs": "_Z4DSPsv", "FMax": "_Z4FMaxv",
                "ExecTime": "_Z8ExecTimePKc", "roofline": "_Z8rooflineddddd"}
     missing = [n for n in sorted(names) if not hasattr(L, mangled.get(n, n))]
     assert not missing, missing

@@ -307,3 +307,58 @@ def test_mttkrp_single_k_is_gemm():
     B, C = o.fill_uniform((I, J, 1), 41), o.fill_uniform((J, R), 42)
     got = o.mttkrp(B, C, np.ones((1, R), np.float32))
     assert (got == o.gemm(B[:, :, 0], C)).all()
+
+
+# ---------------------------------------------------------------------------------------------
+# SYRK
+def test_syrk_integers_exact_and_step_by_step_order():
+    N, K = 24, 40
+    A, C = ints((N, K), -2, 3, 50), ints((N, N), -3, 4, 51)
+    want = 3 * (A.astype(np.int64) @ A.astype(np.int64).T) - 2 * C.astype(np.int64)
+    assert (o.syrk(A, C, 3.0, -2.0) == want).all()
+    # float data: the golden loop's own order and grouping, one float32 operation at a time
+    # (golden = beta*cc; golden += (alpha*aa)*bb for ascending k, syrk-run-fpga.cpp:84-90)
+    Ar, Cr = o.fill_uniform((5, 33), 52), o.fill_uniform((5, 5), 53)
+    alpha, beta = np.float32(1.7), np.float32(-0.3)
+    got = o.syrk(Ar, Cr, float(alpha), float(beta))
+    for i in range(5):
+        for j in range(5):
+            g = np.float32(beta * Cr[i, j])
+            for k in range(33):
+                g = np.float32(g + np.float32(np.float32(alpha * Ar[i, k]) * Ar[j, k]))
+            assert got[i, j] == g
+    exact = 1.7 * (Ar.astype(np.float64) @ Ar.astype(np.float64).T) - 0.3 * Cr
+    assert np.abs(got - exact).max() < 1e-5
+    assert (o.syrk(Ar, Cr, 1.7, -0.3, rows=(2, 2))[0:2] == got[2:4]).all()
+
+
+def test_syrk_constant_closed_form_and_symmetry():
+    N, K = 12, 17
+    assert (o.syrk(np.ones((N, K), np.float32), np.full((N, N), 2, np.float32), 2.0, 0.5) == 2 * K + 1).all()
+    A = o.fill_uniform((N, K), 54)
+    D = o.syrk(A, np.zeros((N, N), np.float32), 1.0, 0.0)
+    assert (D == D.T).all()            # every product a*b is commutative, order over k is the same
+
+
+@pytest.mark.parametrize("III,II,I", [(4, 4, 4), (2, 3, 2), (3, 1, 6)])
+def test_syrk_folded_layout_two_reference_mappings_agree(III, II, I):
+    """syrk_fold follows the pipeline's index expressions (syrk.cpp:37-46) and syrk_unfold_upper the
+    BLAS wrapper's read-back loop (blas-syrk.cpp:49-73).  They are written independently in the
+    reference; composing them must return the upper triangle, every folded position they share
+    is hit exactly once, and the positions the driver skips when validating
+    (syrk-run-fpga.cpp:74-75) are exactly the strictly-lower parts of the diagonal blocks plus
+    the unused corner blocks."""
+    N = III * II * I
+    D = np.arange(N * N, dtype=np.float32).reshape(N, N)            # every element distinct
+    F = o.syrk_fold(D, III, II)
+    assert F.shape == (I, I + 1, II, II, III, III)
+    assert np.isnan(F[I // 2:]).all() and not np.isnan(F[:I // 2]).any()
+    assert (o.syrk_unfold_upper(F, III, II) == np.triu(D)).all()
+    # all elements on or above the diagonal appear in the folded half, and none strictly below a
+    # diagonal block's own lower triangle
+    vals = F[:I // 2].ravel().astype(np.int64)
+    r, c = vals // N, vals % N
+    B = III * II
+    assert (c // B >= r // B).all()                                  # only blocks on/above the diagonal
+    assert len(set(vals.tolist())) == len(vals)                      # no element stored twice
+    assert len(vals) == (I // 2) * (I + 1) * B * B == (I * (I + 1) // 2) * B * B

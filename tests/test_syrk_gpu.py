@@ -1,0 +1,151 @@
+"""GPU parity tests of the SYRK path through `syrk` (include/syrk-interface.h), `ssyrk`
+(include/blas-syrk.h) and the thin layer (include/t2sp_hip.h).
+
+Bar: relative Frobenius error <= 1e-5 against the CPU oracle's golden loop
+(syrk-run-fpga.cpp:84-90) on the same seeded inputs; exact equality on small integers."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import t2sp_amd
+from conftest import rel_fro
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+# (III, II, I, K): the TINY and GPU constant sets of syrk/const-parameters.h:23-52, the S10 release
+# set of peppers/blas/level3/syrk/release/s10/const-parameters.h (N = 768, K = 1024), and the
+# large FPGA set's block edge 12*32 = 384 with two blocks (a block wider than any tile)
+SETS = [(4, 4, 4, 64), (32, 2, 8, 64), (12, 8, 8, 1024), (12, 32, 2, 128)]
+
+
+@pytest.mark.parametrize("III,II,I,K", SETS)
+@pytest.mark.parametrize("cfg", [0, 2, 3])
+def test_folded_output_parity(oracle, III, II, I, K, cfg):
+    N = III * II * I
+    A, C = oracle.fill_uniform((N, K), 51), oracle.fill_uniform((N, N), 52)    # C is not symmetric
+    alpha, beta = 1.5, -0.75
+    want = oracle.syrk_fold(oracle.syrk(A, C, alpha, beta), III, II)
+    got = t2sp_amd.syrk(A, C, alpha, beta, fold=(III, II), cfg=cfg)
+    written = ~np.isnan(want)
+    assert (np.isnan(got) == ~written).all()        # exactly the positions the pipeline writes
+    err, mx = rel_fro(got[written], want[written])
+    print("folded III %d II %d I %d cfg %d rel_fro %.3e max_abs %.3e" % (III, II, I, cfg, err, mx))
+    assert err <= TOL
+    # read back the way the reference's BLAS wrapper does: the upper triangle of the result
+    up = oracle.syrk_unfold_upper(got, III, II)
+    assert rel_fro(up, np.triu(oracle.syrk(A, C, alpha, beta)))[0] <= TOL
+
+
+@pytest.mark.parametrize("shape", [(64, 64), (512, 96), (100, 36), (130, 20), (33, 7), (1, 4), (300, 2048)])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 99])
+def test_flat_output_whole_matrix(oracle, shape, cfg):
+    """2-D Out: every element alpha*A*A^T + beta*C with C read in place (not symmetric)."""
+    N, K = shape
+    A, C = oracle.fill_uniform((N, K), 53), oracle.fill_uniform((N, N), 54)
+    got = t2sp_amd.syrk(A, C, 0.5, 2.0, cfg=cfg)
+    assert rel_fro(got, oracle.syrk(A, C, 0.5, 2.0))[0] <= TOL, (shape, cfg)
+    got0 = t2sp_amd.syrk(A, None, 2.0, 0.0, cfg=cfg)
+    assert rel_fro(got0, oracle.syrk(A, np.zeros((N, N), np.float32), 2.0, 0.0))[0] <= TOL
+    assert (got0 == got0.T).all()                 # one product serves both triangles
+
+
+def test_transposed_a_and_integers_exact(oracle):
+    rng = np.random.default_rng(5)
+    A = rng.integers(-2, 3, (192, 64)).astype(np.float32)
+    C = rng.integers(-3, 4, (192, 192)).astype(np.float32)
+    ref = 2 * (A.astype(np.int64) @ A.astype(np.int64).T) - 3 * C.astype(np.int64)
+    assert (t2sp_amd.syrk(A, C, 2.0, -3.0) == ref).all()
+    At = np.ascontiguousarray(A.T)
+    assert (t2sp_amd.syrk(At, C, 2.0, -3.0, opa=1) == ref).all()
+
+
+def test_device_buffers_in_place_thin_layer_blas_semantics(oracle):
+    """t2sp_ssyrk_f32 with mirror = 0 updates one triangle of C in place and leaves the other
+    alone; mirror = 1 returns the symmetric matrix built from that triangle."""
+    import torch
+    N, K = 384, 160
+    L = t2sp_amd.lib()
+    A = t2sp_amd.fill_uniform(torch.empty(N, K, device="cuda"), 61)
+    C0 = t2sp_amd.fill_uniform(torch.empty(N, N, device="cuda"), 62)
+    a, c0 = A.cpu().numpy(), C0.cpu().numpy()
+    for upper in (1, 0):
+        tri = np.triu if upper else np.tril
+        csym = tri(c0) + tri(c0, 1 if upper else -1).T
+        want = oracle.syrk(a, csym, 0.7, 1.3)
+        for mirror in (0, 1):
+            C = C0.clone()
+            rc = L.t2sp_ssyrk_f32(upper, 0, N, K, 0.7, A.data_ptr(), K, 1.3, C.data_ptr(), N, C.data_ptr(), N, mirror, 0,
+                                  None, 0, None)
+            assert rc == 0
+            torch.cuda.synchronize()
+            got = C.cpu().numpy()
+            assert rel_fro(tri(got), tri(want))[0] <= TOL
+            other = np.tril(got, -1) if upper else np.triu(got, 1)
+            if mirror:
+                assert rel_fro(got, want)[0] <= TOL and (got == got.T).all()
+            else:
+                assert (other == (np.tril(c0, -1) if upper else np.triu(c0, 1))).all()
+
+
+def test_full_size_sampled_rows_and_symmetry(oracle):
+    """N = K = 8192 on the device: sampled rows against the oracle, symmetry of the whole result."""
+    import torch
+    N = K = 8192
+    A = t2sp_amd.fill_uniform(torch.empty(N, K, device="cuda"), 71)
+    C = t2sp_amd.fill_uniform(torch.empty(N, N, device="cuda"), 72)
+    out = torch.full((N, N), float("nan"), device="cuda")
+    L = t2sp_amd.lib()
+    assert L.t2sp_ssyrk_f32(1, 0, N, K, 1.0, A.data_ptr(), K, 0.5, C.data_ptr(), N, out.data_ptr(), N, 1, 0, None, 0,
+                            None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, out.t())
+    a = A.cpu().numpy()
+    c = C.cpu().numpy()
+    csym = np.triu(c) + np.triu(c, 1).T
+    for row0 in (0, 4091, 8184):
+        want = oracle.syrk(a, csym, 1.0, 0.5, rows=(row0, 8))
+        err, mx = rel_fro(out[row0:row0 + 8].cpu().numpy(), want)
+        print("rows %d.. rel_fro %.3e max_abs %.3e" % (row0, err, mx))
+        assert err <= TOL
+
+
+def test_error_codes():
+    A = np.zeros((96, 16), np.float32)
+    C = np.zeros((96, 96), np.float32)
+    with pytest.raises(t2sp_amd.T2spError) as e:           # I = 3 is odd
+        t2sp_amd.syrk(A, C, 1.0, 1.0, out=np.zeros((3, 4, 4, 4, 8, 8), np.float32), fold=(8, 4))
+    assert e.value.code == -8
+    with pytest.raises(t2sp_amd.T2spError) as e:           # Out smaller than N x N
+        t2sp_amd.syrk(A, C, 1.0, 1.0, out=np.zeros((64, 64), np.float32))
+    assert e.value.code == -4
+
+
+@pytest.mark.parametrize("III,II,I,K", [(4, 4, 4, 64), (12, 32, 2, 128)])
+def test_thin_layer_folded_with_and_without_workspace(oracle, III, II, I, K):
+    """Without a workspace the folded addresses are formed in the product's epilogue; with one the
+    matrix is formed flat and folded by a second kernel.  Same bits either way."""
+    import torch
+    N = III * II * I
+    L = t2sp_amd.lib()
+    A = t2sp_amd.fill_uniform(torch.empty(N, K, device="cuda"), 81)
+    C = t2sp_amd.fill_uniform(torch.empty(N, N, device="cuda"), 82)
+    nbytes = L.t2sp_ssyrk_folded_workspace_bytes(0, N, K)
+    assert nbytes == N * N * 4
+    ws = torch.empty(nbytes // 4, device="cuda")
+    outs = []
+    for w, nb in ((None, 0), (ws.data_ptr(), nbytes)):
+        out = torch.full((I, I + 1, II, II, III, III), float("nan"), device="cuda")
+        st = out.stride()
+        s6 = (ctypes.c_int64 * 6)(st[5], st[4], st[3], st[2], st[1], st[0])
+        assert L.t2sp_ssyrk_f32_folded(0, N, K, 1.25, A.data_ptr(), K, -0.5, C.data_ptr(), N, out.data_ptr(), III, II,
+                                       s6, 0, w, nb, None) == 0
+        torch.cuda.synchronize()
+        outs.append(out.cpu().numpy())
+    want = oracle.syrk_fold(oracle.syrk(A.cpu().numpy(), C.cpu().numpy(), 1.25, -0.5), III, II)
+    written = ~np.isnan(want)
+    for got in outs:
+        assert (np.isnan(got) == ~written).all()
+        assert rel_fro(got[written], want[written])[0] <= TOL
+    assert (outs[0][written] == outs[1][written]).all()
