@@ -36,6 +36,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace t2sp {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
@@ -220,6 +222,13 @@ enum : int { SG_MFMA = 0x008, SG_VMEM_READ = 0x020, SG_DS_READ = 0x100, SG_DS_WR
         __builtin_amdgcn_sched_group_barrier(SG_MFMA, (mfma_between), 0);\
     }
 
+// Global loads a loader issues per k-tile beyond its tile's 128-bit slots (a loader that needs
+// some declares `static constexpr int EXTRA_VMEM`), so that the interleave places them too.
+template <class L, class = void>
+struct LoaderExtraVmem { static constexpr int value = 0; };
+template <class L>
+struct LoaderExtraVmem<L, std::void_t<decltype(L::EXTRA_VMEM)>> { static constexpr int value = L::EXTRA_VMEM; };
+
 // The pipelined mainloop.  ALoader/BLoader expose, for register slot S in {0,1},
 //   void fetch<S>()                 issue the global loads of the next k-tile into slot S
 //   void commit<S>(float *stage)    write slot S into an LDS stage
@@ -244,7 +253,8 @@ __device__ __forceinline__ void mainloop_body(Accum<Cfg> &acc, ALoader &la, BLoa
     float *b_nxt = smem + 2 * Cfg::A_STAGE + (CUR ^ 1) * Cfg::B_STAGE;
     constexpr int MFMA_PER_SLICE = 4 * Cfg::MT * Cfg::NT;
     constexpr int N_DS_READ = Cfg::MT + Cfg::NT;
-    constexpr int N_VMEM = Cfg::A_VEC + Cfg::B_VEC;
+    constexpr int N_DS_WRITE = Cfg::A_VEC + Cfg::B_VEC;
+    constexpr int N_VMEM = N_DS_WRITE + LoaderExtraVmem<ALoader>::value + LoaderExtraVmem<BLoader>::value;
     la.template fetch<S>();
     lb.template fetch<S>();
 #pragma unroll
@@ -255,13 +265,13 @@ __device__ __forceinline__ void mainloop_body(Accum<Cfg> &acc, ALoader &la, BLoa
     la.template commit<S ^ 1>(a_nxt);
     lb.template commit<S ^ 1>(b_nxt);
     {
-        constexpr int N_MEM = 2 * N_VMEM + (KK - 1) * N_DS_READ;
+        constexpr int N_MEM = N_VMEM + N_DS_WRITE + (KK - 1) * N_DS_READ;
         constexpr int TOTAL = (KK - 1) * MFMA_PER_SLICE;
         constexpr int GAP = TOTAL / N_MEM > 0 ? TOTAL / N_MEM : 1;
         T2SP_INTERLEAVE(SG_DS_READ, N_DS_READ, GAP)
         T2SP_INTERLEAVE(SG_VMEM_READ, N_VMEM, GAP)
         T2SP_INTERLEAVE(SG_DS_READ, (KK - 2) * N_DS_READ, GAP)
-        T2SP_INTERLEAVE(SG_DS_WRITE, N_VMEM, GAP)
+        T2SP_INTERLEAVE(SG_DS_WRITE, N_DS_WRITE, GAP)
     }
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();

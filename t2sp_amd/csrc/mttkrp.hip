@@ -41,32 +41,62 @@ struct MttkrpOutMap {
     }
 };
 
-// B tensor rows: slot (row i, 4 consecutive j) of reduction tile kt: k = kt / (J/BK).
-template <class Cfg>
+// Walk over the reduction tiles kt = k * (J/BK) + j0/BK, the same for every lane: j0 advances by BK
+// and wraps into the next k.  Kept as running counters (scalar unit) instead of a division per
+// tile.  A plain (non-EDGE) walk stops on the last tile of the tensor; what is fetched past the
+// end of a workgroup's range is never multiplied.
+struct KjWalk {
+    int kt, total, j0, k, J;
+    __device__ __forceinline__ KjWalk(int kt0, int K, int J_, int BK) : kt(kt0), total(K * (J_ / BK)), J(J_) {
+        const int t = kt0 < total ? kt0 : 0;
+        k = t / (J / BK);
+        j0 = (t - k * (J / BK)) * BK;
+    }
+    __device__ __forceinline__ bool inside() const { return kt < total; }
+    // returns true when k moved on
+    __device__ __forceinline__ bool next(int BK, bool edge) {
+        const bool go = edge ? true : kt + 1 < total;
+        kt += go ? 1 : 0;
+        j0 += go ? BK : 0;
+        const bool wrap = j0 >= J;
+        j0 = wrap ? 0 : j0;
+        k += wrap ? 1 : 0;
+        return wrap;
+    }
+};
+
+// B tensor rows: slot (row i, 4 consecutive j) of reduction tile (k, j0).
+template <class Cfg, bool EDGE>
 struct TensorKcLoader {
     const float *p[Cfg::A_VEC];
     const float *safe;
     bool ok[Cfg::A_VEC];
     v4f reg[2][Cfg::A_VEC];
-    int kt, tiles_per_k, total;
-    int64_t sb_k;
+    KjWalk w;
+    int64_t off, sb_k;    // off = k * sb_k + j0
     __device__ TensorKcLoader(const MttkrpArgs &g, int m0, int kt0)
-        : safe(g.B), kt(kt0), tiles_per_k(g.J / Cfg::BK), total(g.K * (g.J / Cfg::BK)), sb_k(g.sb_k) {
+        : safe(g.B), w(kt0, g.K, g.J, Cfg::BK), sb_k(g.sb_k) {
+        off = w.k * sb_k + w.j0;
 #pragma unroll
         for (int i = 0; i < Cfg::A_VEC; i++) {
             KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
-            ok[i] = m0 + s.row < g.I;
+            ok[i] = !EDGE || m0 + s.row < g.I;
             p[i] = g.B + (int64_t)(ok[i] ? m0 + s.row : 0) * g.sb_i + s.k;
         }
     }
     template <int S>
     __device__ __forceinline__ void fetch() {
-        const bool in = kt < total;
-        const int t = in ? kt : 0;
-        const int k = t / tiles_per_k, j0 = (t - k * tiles_per_k) * Cfg::BK;
+        const bool in = w.inside();
 #pragma unroll
-        for (int i = 0; i < Cfg::A_VEC; i++) reg[S][i] = load_or_zero(p[i] + k * sb_k + j0, ok[i] && in, safe);
-        kt++;
+        for (int i = 0; i < Cfg::A_VEC; i++) {
+            if (EDGE)
+                reg[S][i] = load_or_zero(p[i] + (in ? off : 0), ok[i] && in, safe);
+            else
+                reg[S][i] = *reinterpret_cast<const v4f *>(p[i] + off);
+        }
+        const int kt_before = w.kt;
+        const bool wrap = w.next(Cfg::BK, EDGE);
+        off += (w.kt != kt_before) ? (wrap ? sb_k - (w.J - Cfg::BK) : Cfg::BK) : 0;
     }
     template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
@@ -78,24 +108,26 @@ struct TensorKcLoader {
     }
 };
 
-// Khatri-Rao rows: slot (column r, 4 consecutive j) of reduction tile kt holds
+// Khatri-Rao rows: slot (column r, 4 consecutive j) of reduction tile (k, j0) holds
 // C[j..j+3, r] * D[k, r], formed in registers.
-template <class Cfg>
+template <class Cfg, bool EDGE>
 struct KhatriRaoKcLoader {
+    static constexpr int EXTRA_VMEM = Cfg::B_VEC;   // the D[k, r] factors
     const float *pc[Cfg::B_VEC];
     const float *pd[Cfg::B_VEC];
     const float *safe;
     bool ok[Cfg::B_VEC];
     v4f reg[2][Cfg::B_VEC];
     float dval[2][Cfg::B_VEC];
-    int kt, tiles_per_k, total;
-    int64_t sd_k;
+    KjWalk w;
+    int64_t koff, sd_k;   // koff = k * sd_k
     __device__ KhatriRaoKcLoader(const MttkrpArgs &g, int n0, int kt0)
-        : safe(g.C), kt(kt0), tiles_per_k(g.J / Cfg::BK), total(g.K * (g.J / Cfg::BK)), sd_k(g.sd_k) {
+        : safe(g.C), w(kt0, g.K, g.J, Cfg::BK), sd_k(g.sd_k) {
+        koff = w.k * sd_k;
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
-            ok[i] = n0 + s.row < g.R;
+            ok[i] = !EDGE || n0 + s.row < g.R;
             const int r = ok[i] ? n0 + s.row : 0;
             pc[i] = g.C + (int64_t)r * g.sc_r + s.k;
             pd[i] = g.D + (int64_t)r * g.sd_r;
@@ -103,15 +135,18 @@ struct KhatriRaoKcLoader {
     }
     template <int S>
     __device__ __forceinline__ void fetch() {
-        const bool in = kt < total;
-        const int t = in ? kt : 0;
-        const int k = t / tiles_per_k, j0 = (t - k * tiles_per_k) * Cfg::BK;
+        const bool in = w.inside();
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
-            reg[S][i] = load_or_zero(pc[i] + j0, ok[i] && in, safe);
-            dval[S][i] = pd[i][k * sd_k];
+            if (EDGE)
+                reg[S][i] = load_or_zero(pc[i] + (in ? w.j0 : 0), ok[i] && in, safe);
+            else
+                reg[S][i] = *reinterpret_cast<const v4f *>(pc[i] + w.j0);
+            dval[S][i] = pd[i][(!EDGE || in) ? koff : 0];
         }
-        kt++;
+        const int kt_before = w.kt;
+        const bool wrap = w.next(Cfg::BK, EDGE);
+        koff += (w.kt != kt_before && wrap) ? sd_k : 0;
     }
     template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
@@ -123,7 +158,7 @@ struct KhatriRaoKcLoader {
     }
 };
 
-template <class Cfg>
+template <class Cfg, bool EDGE>
 __global__ void __launch_bounds__(Cfg::NTHREADS) mttkrp_kernel(const MttkrpArgs g) {
     extern __shared__ __align__(16) float smem[];
     const int tile = blockIdx.x % (g.tiles_m * g.tiles_n), split = blockIdx.x / (g.tiles_m * g.tiles_n);
@@ -131,8 +166,8 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) mttkrp_kernel(const MttkrpArgs 
     const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
     int kt0, kt1;
     split_range(g.K * (g.J / Cfg::BK), g.splits, split, kt0, kt1);
-    TensorKcLoader<Cfg> la(g, m0, kt0);
-    KhatriRaoKcLoader<Cfg> lb(g, n0, kt0);
+    TensorKcLoader<Cfg, EDGE> la(g, m0, kt0);
+    KhatriRaoKcLoader<Cfg, EDGE> lb(g, n0, kt0);
     Accum<Cfg> acc;
     mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem);
     if (g.splits == 1) {
@@ -201,7 +236,9 @@ static int launch_mttkrp(MttkrpArgs g, hipStream_t stream) {
     g.tiles_m = g.Mp / Cfg::BM;
     g.tiles_n = g.Np / Cfg::BN;
     const size_t smem = Cfg::SMEM_FLOATS * sizeof(float);
-    auto kern = mttkrp_kernel<Cfg>;
+    // plain loaders need whole tiles and a reduction that ends on a pair of k-tiles
+    const bool edge = (g.I % Cfg::BM) || (g.R % Cfg::BN) || ((int64_t)g.K * (g.J / Cfg::BK)) % 2;
+    auto kern = edge ? mttkrp_kernel<Cfg, true> : mttkrp_kernel<Cfg, false>;
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * g.splits), dim3(Cfg::NTHREADS), smem, stream, g);
