@@ -92,6 +92,16 @@ int t2sp_ssyrk_f32_folded(int trans, int N, int K, float alpha, const float *A, 
                           const int64_t *strides6, int cfg, float *workspace, size_t workspace_bytes,
                           void *stream);
 
+/* O[i,k] = A[i,k] + x[i] * y[k], fp32, product and sum rounded separately; A row-major I x K, O
+ * flat row-major or the reference's 6-D tiled Out(kkk, iii, ii, kk, k, i) with element strides
+ * strides6 (t2s/tests/performance/ger/ger-run-fpga.cpp:60).  An HBM-bound stream (8 bytes and
+ * 2 flop per element).  Replaces the device side of the reference's GER pipeline
+ * (t2s/tests/performance/ger/ger.cpp:57-61). */
+int t2sp_sger_f32(const float *A, const float *x, const float *y, float *O, int I, int K, int64_t lda,
+                  int64_t ldo, void *stream);
+int t2sp_sger_f32_tiled(const float *A, const float *x, const float *y, float *O, int I, int K, int64_t lda,
+                        int kkk, int iii, int ii, int kk, const int64_t *strides6, void *stream);
+
 /* O[n,co,h,w] = sum_{ci,kh,kw} I[n,ci,h+kh,w+kw] * W[co,ci,kh,kw], stride 1, valid
  * padding, fp32.  si4/sw4/so4 are element strides of the logical indices
  * (n,ci,h,w), (co,ci,kh,kw), (n,co,h,w); "w" is the innermost spatial axis (the

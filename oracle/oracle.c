@@ -22,6 +22,8 @@
  *                                 t2s/peppers/blas/level3/syrk/release/s10/ssyrk-run-fpga.cpp:45-54
  *                                 (golden = beta*c; golden += alpha*a*b over ascending k).  The folded
  *                                 output layout (syrk.cpp:37-46) is restated in oracle.py.
+ *   oracle_ger       golden       t2s/tests/performance/ger/ger-run-fpga.cpp:71
+ *                                 (golden = a + x * y, product and sum rounded separately).
  *   oracle_mttkrp    golden       t2s/tests/performance/util/util.h:498-515 (two-step: TTM over l
  *                                 into e(i,j,k), then d += e*b over k).  The reference's outer loop
  *                                 bound `i < K` (util.h:502) is only right when I == K; this
@@ -346,6 +348,17 @@ void oracle_syrk(const float *A, const float *C, float *D, int64_t N, int64_t K,
                 golden += t * A[j * lda + k];
             }
             D[i * ldd + j] = golden;
+        }
+}
+
+/* O[i,k] = A[i,k] + x[i]*y[k] (ger-run-fpga.cpp:71); A and O dense row-major I x K. */
+void oracle_ger(const float *A, const float *x, const float *y, float *O, int64_t I, int64_t K, int threads) {
+    set_threads(threads);
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < I; i++)
+        for (int64_t k = 0; k < K; k++) {
+            const float p = x[i] * y[k];
+            O[i * K + k] = A[i * K + k] + p;
         }
 }
 

@@ -44,6 +44,8 @@ def lib():
         _lib.oracle_mttkrp_literal.argtypes = [fp, fp, fp, fp] + [i64] * 6
         _lib.oracle_syrk.argtypes = [fp, fp, fp] + [i64] * 5 + [ctypes.c_float, ctypes.c_float, i64, i64, ctypes.c_int]
         _lib.oracle_syrk.restype = None
+        _lib.oracle_ger.argtypes = [fp, fp, fp, fp, i64, i64, ctypes.c_int]
+        _lib.oracle_ger.restype = None
         _lib.oracle_max_threads.restype = ctypes.c_int
         for f in (_lib.oracle_fill_uniform, _lib.oracle_gemm, _lib.oracle_gemm_literal,
                   _lib.oracle_conv, _lib.oracle_capsule, _lib.oracle_mttkrp,
@@ -234,6 +236,24 @@ def syrk_unfold_upper(out, III, II):
                                 D[ti, tj] = out[I - i - 1, I - j - 1, II - ii - 1, II - jj - 1, III - iii - 1,
                                                 III - jjj - 1]
     return D
+
+
+def ger(A, x, y, threads=0):
+    """A + outer(x, y), product and sum rounded separately (ger-run-fpga.cpp:71)."""
+    A, x, y = np.ascontiguousarray(A), np.ascontiguousarray(x), np.ascontiguousarray(y)
+    I, K = A.shape
+    O = np.empty((I, K), dtype=np.float32)
+    lib().oracle_ger(_p(A), _p(x), _p(y), _p(O), I, K, threads)
+    return O
+
+
+def ger_tile(O, III, II, KKK, KK):
+    """The tiled output Out(kkk, iii, ii, kk, k, i) -- numpy shape (I, K, KK, II, III, KKK) -- of the
+    flat result O, by the pipeline's addresses total_i = iii + III*ii + III*II*i,
+    total_k = kkk + KKK*kk + KKK*KK*k (ger.cpp:37-39)."""
+    TI, TK = O.shape
+    I, K = TI // (III * II), TK // (KKK * KK)
+    return np.ascontiguousarray(O.reshape(I, II, III, K, KK, KKK).transpose(0, 3, 4, 1, 2, 5))
 
 
 def max_threads():

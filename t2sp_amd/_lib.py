@@ -60,6 +60,11 @@ def _declare(L):
                                  ctypes.c_size_t, vp]
     L.t2sp_ssyrk_f32_folded.argtypes = [i32, i32, i32, f32, vp, i64, f32, vp, i64, vp, i32, i32,
                                         ctypes.POINTER(i64), i32, vp, ctypes.c_size_t, vp]
+    L.ger.argtypes = [bp, bp, bp, bp]
+    L.ger_ns.argtypes = [bp, bp, bp, bp]
+    L.ger_ns.restype = ctypes.c_double
+    L.t2sp_sger_f32.argtypes = [vp, vp, vp, vp, i32, i32, i64, i64, vp]
+    L.t2sp_sger_f32_tiled.argtypes = [vp, vp, vp, vp, i32, i32, i64, i32, i32, i32, i32, ctypes.POINTER(i64), vp]
     L.conv.argtypes = [bp, bp, bp]
     L.t2sp_conv_with_cfg.argtypes = [bp, bp, bp, i32]
     p64, p32 = ctypes.POINTER(i64), ctypes.POINTER(i32)

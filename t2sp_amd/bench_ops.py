@@ -124,8 +124,31 @@ def ssyrk_8192(torch, steps, warmup, peak):
                   **{"TFLOP/s_reference_count": round(2.0 * N * N * K / ms / 1e9, 3)})
 
 
+def sger_8192(torch, steps, warmup, peak):
+    """Not a BASELINE configuration: the GER pipeline (t2s/tests/performance/ger) on an 8192 x 8192
+    matrix.  It moves 8 bytes per element (A in, Out out; x and y are negligible) for 2 flop, so its
+    roof is HBM bandwidth (8 TB/s), reported next to the flop rate."""
+    L = lib()
+    N = 8192
+    A = ops.fill_uniform(torch.empty(N, N, device="cuda"), 1)
+    x = ops.fill_uniform(torch.empty(N, device="cuda"), 2)
+    y = ops.fill_uniform(torch.empty(N, device="cuda"), 3)
+    O = torch.empty(N, N, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        rc = L.t2sp_sger_f32(A.data_ptr(), x.data_ptr(), y.data_ptr(), O.data_ptr(), N, N, N, N, s)
+        assert rc == 0, rc
+
+    ms = _time(torch, launch, steps, warmup)
+    nbytes = 8.0 * N * N + 8.0 * N
+    return _entry(2.0 * N * N / ms / 1e9, peak, ms, workload="I=K=8192, flat output",
+                  **{"bound": "hbm", "GB/s": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / 8000.0, 4)})
+
+
 def run_all(torch, steps, warmup, peak):
     return {"conv2d": conv_config3(torch, steps, warmup, peak),
             "capsule": capsule_config4(torch, steps, warmup, peak),
             "mttkrp": mttkrp_config5(torch, steps, warmup, peak),
-            "ssyrk_8192": ssyrk_8192(torch, steps, warmup, peak)}
+            "ssyrk_8192": ssyrk_8192(torch, steps, warmup, peak),
+            "sger_8192": sger_8192(torch, steps, warmup, peak)}

@@ -102,6 +102,25 @@ def syrk(A, C, alpha, beta, out=None, fold=None, opa=0, cfg=0):
     return out
 
 
+def ger(A, x, y, out=None, tiles=None):
+    """Out = A + outer(x, y) through the `ger` entry point (include/ger-interface.h).
+
+    A: (I, K) row-major, x: (I,), y: (K,).  With tiles=(III, II, KKK, KK) the result has the
+    reference's tiled layout Out(KKK, III, II, KK, K, I), numpy shape (I, K, KK, II, III, KKK)
+    (t2s/tests/performance/ger/ger-run-fpga.cpp:60); otherwise the flat (I, K) matrix."""
+    I, K = A.shape
+    if out is None:
+        if tiles is None:
+            out = _empty_like_kind(A, (I, K))
+        else:
+            III, II, KKK, KK = tiles
+            assert I % (III * II) == 0 and K % (KKK * KK) == 0
+            out = _empty_like_kind(A, (I // (III * II), K // (KKK * KK), KK, II, III, KKK))
+    a, xb, yb, o = (HalideBuffer.wrap(t) for t in (A, x, y, out))
+    _check("ger", lib().ger(a.ref, xb.ref, yb.ref, o.ref))
+    return out
+
+
 def conv(I, W, out=None, cfg=0):
     """O = conv2d(I, W), stride 1, no padding, through the `conv` entry point
     (include/conv-interface.h).

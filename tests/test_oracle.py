@@ -362,3 +362,27 @@ def test_syrk_folded_layout_two_reference_mappings_agree(III, II, I):
     assert (c // B >= r // B).all()                                  # only blocks on/above the diagonal
     assert len(set(vals.tolist())) == len(vals)                      # no element stored twice
     assert len(vals) == (I // 2) * (I + 1) * B * B == (I * (I + 1) // 2) * B * B
+
+
+# ---------------------------------------------------------------------------------------------
+# GER
+def test_ger_matches_separately_rounded_numpy_and_tiled_addresses():
+    I, K = 24, 40
+    A, x, y = o.fill_uniform((I, K), 60), o.fill_uniform((I,), 61), o.fill_uniform((K,), 62)
+    want = A + (x[:, None] * y[None, :]).astype(np.float32)      # two float32 roundings, as in the golden loop
+    got = o.ger(A, x, y)
+    assert (got == want).all()
+    Ai, xi, yi = ints((I, K), -9, 9, 63), ints((I,), -9, 9, 64), ints((K,), -9, 9, 65)
+    assert (o.ger(Ai, xi, yi) == Ai + np.outer(xi, yi)).all()
+    # tiled form: walk the output the way the reference's driver validates it (ger-run-fpga.cpp:63-73)
+    III, II, KKK, KK = 2, 3, 4, 2
+    Ot = o.ger_tile(got, III, II, KKK, KK)
+    assert Ot.shape == (I // (III * II), K // (KKK * KK), KK, II, III, KKK)
+    for i in range(Ot.shape[0]):
+        for k in range(Ot.shape[1]):
+            for ii in range(II):
+                for kk in range(KK):
+                    for iii in range(III):
+                        for kkk in range(KKK):
+                            ti, tk = iii + III * ii + III * II * i, kkk + KKK * kk + KKK * KK * k
+                            assert Ot[i, k, kk, ii, iii, kkk] == got[ti, tk]
