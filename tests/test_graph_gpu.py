@@ -1,0 +1,95 @@
+"""The thin layer only enqueues kernels on the stream it is given (no allocation, no memset, no
+synchronisation), so its calls can be recorded into a HIP graph.  Each graph is replayed several
+times with eager work and synchronisations in between, and every replay is compared with the
+eager result."""
+import ctypes
+
+import pytest
+
+import t2sp_amd
+
+pytestmark = pytest.mark.gpu
+i64 = ctypes.c_int64
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+    assert torch.cuda.is_available()
+    return torch
+
+
+def _replays_match(torch, graph, out, eager, refill):
+    for rep in range(3):
+        out.fill_(float("nan"))
+        refill(rep)                                   # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), "replay %d differs from the eager launch" % rep
+
+
+def test_sgemm_with_split_reduction_in_a_graph(torch_cuda):
+    torch = torch_cuda
+    L = t2sp_amd.lib()
+    M = N = K = 1024                                   # kernel + reduce kernel through the workspace
+    A = t2sp_amd.fill_uniform(torch.empty(M, K, device="cuda"), 1)
+    B = t2sp_amd.fill_uniform(torch.empty(K, N, device="cuda"), 2)
+    C = torch.empty(M, N, device="cuda")
+    nbytes = L.t2sp_sgemm_workspace_bytes(M, N, K)
+    ws = torch.empty(max(nbytes // 4, 1), device="cuda")
+    scratch = torch.empty(1 << 20, device="cuda")
+
+    def launch(stream):
+        assert L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, ws.data_ptr(), nbytes,
+                                stream) == 0
+
+    launch(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    eager = C.clone()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        launch(torch.cuda.current_stream().cuda_stream)
+    _replays_match(torch, g, C, eager, lambda rep: (ws.fill_(float(rep)), scratch.normal_()))
+
+
+def test_capsule_and_conv_in_one_graph(torch_cuda):
+    torch = torch_cuda
+    L = t2sp_amd.lib()
+    P = t2sp_amd.fill_uniform(torch.empty(8, 16, 15, 15, 4, 4, device="cuda"), 3)
+    W = t2sp_amd.fill_uniform(torch.empty(16, 16, 3, 3, 4, 4, device="cuda"), 4)
+    V = torch.empty(8, 16, 7, 7, 4, 4, device="cuda")
+    dims = (ctypes.c_int * 11)(8, 16, 16, 7, 7, 3, 3, 2, 4, 4, 4)
+    sp, sw, sv = ((i64 * 6)(*t.stride()) for t in (P, W, V))
+    cap_bytes = L.t2sp_capsule_workspace_bytes(dims, 0, 0)
+    cap_ws = torch.empty(max(cap_bytes // 4, 1), device="cuda")
+    I = t2sp_amd.fill_uniform(torch.empty(4, 32, 18, 18, device="cuda"), 5)
+    Wc = t2sp_amd.fill_uniform(torch.empty(64, 32, 3, 3, device="cuda"), 6)
+    O = torch.empty(4, 64, 16, 16, device="cuda")
+    si, swc, so = ((i64 * 4)(*t.stride()) for t in (I, Wc, O))
+    conv_bytes = L.t2sp_conv2d_workspace_bytes(4, 32, 64, 16, 16, 3, 3)
+    conv_ws = torch.empty(max(conv_bytes // 4, 1), device="cuda")
+    out = torch.empty(V.numel() + O.numel(), device="cuda")
+
+    def launch(stream):
+        assert L.t2sp_capsule_f32(P.data_ptr(), W.data_ptr(), V.data_ptr(), dims, sp, sw, sv, 0, 0, cap_ws.data_ptr(),
+                                  cap_bytes, stream) == 0
+        assert L.t2sp_conv2d_f32(I.data_ptr(), Wc.data_ptr(), O.data_ptr(), 4, 32, 64, 16, 16, 3, 3, si, swc, so, 0,
+                                 conv_ws.data_ptr(), conv_bytes, stream) == 0
+
+    launch(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    eager_v, eager_o = V.clone(), O.clone()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        launch(torch.cuda.current_stream().cuda_stream)
+    for rep in range(3):
+        V.fill_(float("nan"))
+        O.fill_(float("nan"))
+        cap_ws.fill_(float(rep))
+        conv_ws.fill_(float(rep))
+        out.normal_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(V, eager_v) and torch.equal(O, eager_o), "replay %d" % rep
