@@ -31,7 +31,7 @@ extern "C" {
 #define T2SP_CFG_128x128 2
 #define T2SP_CFG_64x128 3
 #define T2SP_CFG_32x128 4 /* one wavefront per tile: for problems with few outputs */
-#define T2SP_CFG_DIRECT 5 /* capsule only: a 32x128 tile per workgroup, reduction split over its waves */
+#define T2SP_CFG_DIRECT 5 /* small problems (sgemm, capsule): one small tile per workgroup, reduction split over its waves, operands global -> registers */
 #define T2SP_CFG_SCALAR 99
 
 #define T2SP_MAX_DIMS 10

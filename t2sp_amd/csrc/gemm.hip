@@ -112,6 +112,114 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) sgemm_kernel(const GemmArgs g) 
     }
 }
 
+// Small products: fewer 128 x 128 tiles than CUs.  One workgroup of 4 waves owns a 64 x 64 tile of
+// C and splits the reduction over its waves, so a 1024^2 output already gives every CU a tile and
+// nothing has to go through a workspace and a second kernel.  No operand is shared between the
+// waves, so nothing is staged in LDS: a lane loads its rows of A (4 consecutive k, 128 bits) and
+// its two columns of four k-rows of B (64 bits each) straight into the MFMA operand registers, two
+// steps (8 k each, 16 MFMAs) ahead of their use, from uniform base pointers that the scalar unit
+// advances plus a fixed 32-bit offset per lane.  The four partial tiles are summed through LDS in
+// wave order, so the result does not depend on timing.
+constexpr int GEMM_DIRECT_WAVES = 4;
+constexpr int GEMM_DIRECT_RING = 3;
+typedef float v2f __attribute__((ext_vector_type(2)));
+
+template <int NW, int R>
+__global__ void __launch_bounds__(NW * 64) sgemm_direct_kernel(const GemmArgs g) {
+    extern __shared__ __align__(16) float smem[];
+    v2f *red = reinterpret_cast<v2f *>(smem);            // [wave][mi][r][lane]
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
+    const int tm = blockIdx.x / g.tiles_n, tn = blockIdx.x - tm * g.tiles_n;
+    const int m0 = tm * 64, n0 = tn * 64;
+    const int steps = g.K >> 3;
+    const int s0 = (int)((int64_t)steps * wave / NW), s1 = (int)((int64_t)steps * (wave + 1) / NW);
+    const int nsteps = s1 - s0;
+
+    // per-lane byte offsets (rows / columns outside the matrix re-read valid ones; never stored)
+    uint32_t a_off[2];
+#pragma unroll
+    for (int mi = 0; mi < 2; mi++) {
+        const int row = min(m0 + mi * 32 + l32, g.M - 1);
+        a_off[mi] = 4u * (uint32_t)(row * (int)g.lda + 4 * lhi);
+    }
+    const int col = (n0 + 2 * l32 + 1 < g.N) ? n0 + 2 * l32 : 0;
+    const uint32_t b_off = 4u * (uint32_t)(4 * lhi * (int)g.ldb + col);
+    const char *a_base = reinterpret_cast<const char *>(g.A + 8 * s0);
+    const char *b_base = reinterpret_cast<const char *>(g.B + (int64_t)8 * s0 * g.ldb);
+    const int64_t b_row = 4 * g.ldb, b_step = 32 * g.ldb;   // bytes per k-row and per step
+    const int a_last = 32 * (steps - 1 - s0);              // byte offset of the last step (loads past it stay there)
+    int issued = 0;
+
+    v4f ra[R][2];
+    v2f rb[R][4];
+#define T2SP_GEMM_DIRECT_ISSUE(d)                                                                   \
+    {                                                                                               \
+        const int st = min(issued, steps - 1 - s0);                                                 \
+        const char *ap = a_base + 32 * st;                                                          \
+        const char *bp = b_base + (int64_t)st * b_step;                                             \
+        issued++;                                                                                   \
+        _Pragma("unroll") for (int j = 0; j < 4; j++)                                               \
+            rb[d][j] = *reinterpret_cast<const v2f *>(bp + j * b_row + b_off);                      \
+        _Pragma("unroll") for (int mi = 0; mi < 2; mi++)                                            \
+            ra[d][mi] = *reinterpret_cast<const v4f *>(ap + a_off[mi]);                             \
+    }
+#define T2SP_GEMM_DIRECT_MMA(d)                                                                     \
+    _Pragma("unroll") for (int j = 0; j < 4; j++)                                                   \
+        _Pragma("unroll") for (int mi = 0; mi < 2; mi++)                                            \
+            _Pragma("unroll") for (int c = 0; c < 2; c++)                                           \
+                acc[mi][c] = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[d][mi][j], rb[d][j][c], acc[mi][c], 0, 0, 0);
+    (void)a_last;
+    v16f acc[2][2];
+#pragma unroll
+    for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+        for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[mi][c][r] = 0.f;
+
+#pragma unroll
+    for (int d = 0; d < R - 1; d++) {
+        T2SP_GEMM_DIRECT_ISSUE(d)
+        __builtin_amdgcn_sched_barrier(0);   // keep the sets in program order: waits count loads
+    }
+    const int main_iters = nsteps > 0 ? (nsteps - 1) / R : 0;
+    const int rem = nsteps - main_iters * R;              // 1..R steps left for the tail (0: none at all)
+    for (int it = 0; it < main_iters; it++) {
+#pragma unroll
+        for (int d = 0; d < R; d++) {
+            T2SP_GEMM_DIRECT_ISSUE((d + R - 1) % R)
+            T2SP_GEMM_DIRECT_MMA(d)
+            T2SP_INTERLEAVE(SG_VMEM_READ, 6, 2)
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    T2SP_GEMM_DIRECT_ISSUE(R - 1)
+#pragma unroll
+    for (int d = 0; d < R; d++) {
+        if (d < rem) { T2SP_GEMM_DIRECT_MMA(d) }
+    }
+#undef T2SP_GEMM_DIRECT_ISSUE
+#undef T2SP_GEMM_DIRECT_MMA
+
+    // sum the partial tiles of the waves in wave order
+    v2f *mine = red + wave * 2 * 16 * 64 + lane;
+#pragma unroll
+    for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) mine[(mi * 16 + r) * 64] = v2f{acc[mi][0][r], acc[mi][1][r]};
+    __syncthreads();
+    for (int q = wave; q < 32; q += NW) {                 // q = mi * 16 + r
+        const v2f *src = red + q * 64 + lane;
+        v2f sum = src[0];
+#pragma unroll
+        for (int wv = 1; wv < NW; wv++) sum += src[wv * 2 * 16 * 64];
+        const int r = q & 15;
+        const int row = m0 + (q >> 4) * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3), cc = n0 + 2 * l32;
+        if (row < g.M && cc + 1 < g.N) *reinterpret_cast<v2f *>(g.C + (int64_t)row * g.ldc + cc) = sum;
+    }
+}
+
 // Fallback for shapes the vector loaders cannot take (K or N not a multiple
 // of 4, or operands not 16-byte aligned): one thread per output, sequential k.
 __global__ void sgemm_scalar_kernel(const GemmArgs g, int bt) {
@@ -186,9 +294,37 @@ static GemmPlan plan_gemm(int M, int N, int K) {
     return p;
 }
 
+// The direct kernel takes products whose 128 x 128 tiles would not fill the CUs (`forced`: any size
+// it can address), with K a multiple of 8, N even, 8-byte aligned B and C rows and 32-bit byte
+// offsets inside A and B.
+static bool gemm_direct_ok(const GemmArgs &g, bool forced) {
+    const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
+    const int64_t t64 = (int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64);
+    // below ~160 tiles of 64 x 64 the split over workgroups fills the chip better
+    if (!forced && (t128 >= 200 || t64 < 160 || g.K < 256)) return false;
+    return g.K % 8 == 0 && g.N % 2 == 0 && g.ldb % 2 == 0 && g.ldc % 2 == 0 && ((uintptr_t)g.B % 8 == 0) &&
+           ((uintptr_t)g.C % 8 == 0) && (int64_t)g.M * g.lda < (1 << 30) && (int64_t)g.K * g.ldb < (1 << 30) &&
+           t64 < (1 << 30);
+}
+
+static int launch_direct(GemmArgs g, hipStream_t stream) {
+    g.tiles_m = (g.M + 63) / 64;
+    g.tiles_n = (g.N + 63) / 64;
+    const size_t smem = (size_t)GEMM_DIRECT_WAVES * 2 * 16 * 64 * sizeof(v2f);
+    auto kern = sgemm_direct_kernel<GEMM_DIRECT_WAVES, GEMM_DIRECT_RING>;
+    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+        return T2SP_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(GEMM_DIRECT_WAVES * 64), smem, stream, g);
+    return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+}
+
 static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *workspace = nullptr,
                     size_t workspace_bytes = 0) {
     if (g.M <= 0 || g.N <= 0 || g.K <= 0) return T2SP_ERR_SHAPE;
+    if ((cfg == T2SP_CFG_AUTO || cfg == T2SP_CFG_DIRECT) && !bt && !g.scale && !g.tiled &&
+        g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && gemm_direct_ok(g, cfg == T2SP_CFG_DIRECT))
+        return launch_direct(g, stream);
+    if (cfg == T2SP_CFG_DIRECT) return T2SP_ERR_SHAPE;
     const bool vec_ok = g.K % 4 == 0 && (bt || g.N % 4 == 0) && g.lda % 4 == 0 && g.ldb % 4 == 0 &&
                         ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
                         ((uintptr_t)g.C % 16 == 0) && (g.tiled || g.ldc % 4 == 0) &&

@@ -163,6 +163,31 @@ def test_split_reduction_with_workspace(oracle, torch_cuda, shape):
     assert rel_fro(C.cpu().numpy(), outs[0])[0] <= TOL
 
 
+@pytest.mark.parametrize("shape", [(1024, 1024, 1024), (500, 260, 4096), (64, 128, 8192), (130, 66, 64), (1, 2, 8),
+                                   (512, 768, 640), (192, 64, 24)])
+def test_direct_kernel_small_products(oracle, torch_cuda, shape):
+    """The one-launch kernel for products with few tiles (a 64 x 64 tile per workgroup, reduction
+    split over its waves): forced through the thin layer, against the oracle, same bits twice."""
+    torch = torch_cuda
+    M, N, K = shape
+    L = t2sp_amd.lib()
+    A = t2sp_amd.fill_uniform(torch.empty(M, K, device="cuda"), 31)
+    B = t2sp_amd.fill_uniform(torch.empty(K, N, device="cuda"), 32)
+    outs = []
+    for _ in range(2):
+        C = torch.full((M, N), float("nan"), device="cuda")
+        assert L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 5, None, 0, None) == 0
+        torch.cuda.synchronize()
+        outs.append(C.cpu().numpy())
+    assert (outs[0] == outs[1]).all()
+    err, mx = rel_fro(outs[0], oracle.gemm(A.cpu().numpy(), B.cpu().numpy()))
+    print("direct %s rel_fro %.3e max_abs %.3e" % (shape, err, mx))
+    assert err <= TOL
+    # a reduction length it cannot take is refused, not mangled
+    assert L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K - 4 if K > 4 else 4, K, N, N, 5, None, 0,
+                            None) == -8
+
+
 def test_empty_extents():
     C = np.full((16, 8), np.nan, np.float32)
     t2sp_amd.gemm(np.zeros((16, 0), np.float32), np.zeros((0, 8), np.float32), out=C)
