@@ -160,6 +160,47 @@ void oracle_gemm_literal(const float *A, const float *B, float *C, int64_t M, in
         }
 }
 
+/* The SGEMM spec executed as one serial loop nest in the spec's own loop order, the way a host
+ * (CPU) target runs the merged UREs: loops i, j, k outermost, then kk, ii, jj, iii, jjj, kkk with
+ * kkk innermost (gemm.cpp:30 "#define P kkk, jjj, iii, jj, ii, kk, k, j, i", bounds :69-71), Z kept
+ * as one accumulator per output of the (i, j) block (Z = 0 at total_k = 0, then Z += X*Y,
+ * gemm.cpp:59-61).  Every output sums its products in ascending total_k, so the values equal
+ * oracle_gemm_literal's bit for bit; only the traversal (and so the time) differs.
+ * c6 = {KKK, JJJ, III, JJ, II, KK}; block rows [i0, i1) of the I = M / (III*II) blocks. */
+void oracle_gemm_ure(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K,
+                     const int64_t *c6, int64_t i0, int64_t i1) {
+    const int64_t KKK = c6[0], JJJ = c6[1], III = c6[2], JJ = c6[3], II = c6[4], KK = c6[5];
+    const int64_t J = N / (JJJ * JJ), KO = K / (KKK * KK);
+    (void)M;
+    float *z = (float *)malloc(sizeof(float) * II * JJ * III * JJJ);
+    for (int64_t i = i0; i < i1; i++)
+        for (int64_t j = 0; j < J; j++) {
+            for (int64_t t = 0; t < II * JJ * III * JJJ; t++) z[t] = 0.0f;
+            for (int64_t k = 0; k < KO; k++)
+                for (int64_t kk = 0; kk < KK; kk++)
+                    for (int64_t ii = 0; ii < II; ii++)
+                        for (int64_t jj = 0; jj < JJ; jj++)
+                            for (int64_t iii = 0; iii < III; iii++)
+                                for (int64_t jjj = 0; jjj < JJJ; jjj++) {
+                                    const int64_t ti = iii + III * ii + III * II * i;
+                                    const int64_t tj = jjj + JJJ * jj + JJJ * JJ * j;
+                                    float acc = z[((ii * JJ + jj) * III + iii) * JJJ + jjj];
+                                    for (int64_t kkk = 0; kkk < KKK; kkk++) {
+                                        const int64_t tk = kkk + KKK * kk + KKK * KK * k;
+                                        acc += A[ti * K + tk] * B[tk * N + tj];
+                                    }
+                                    z[((ii * JJ + jj) * III + iii) * JJJ + jjj] = acc;
+                                }
+            for (int64_t ii = 0; ii < II; ii++)
+                for (int64_t jj = 0; jj < JJ; jj++)
+                    for (int64_t iii = 0; iii < III; iii++)
+                        for (int64_t jjj = 0; jjj < JJJ; jjj++)
+                            C[(iii + III * ii + III * II * i) * N + jjj + JJJ * jj + JJJ * JJ * j] =
+                                z[((ii * JJ + jj) * III + iii) * JJJ + jjj];
+        }
+    free(z);
+}
+
 /* ------------------------------------------------------------------------- */
 /* O[n,co,y,x] = sum_{ci,kx,ky} I[n,ci,y*sy+ky,x*sx+kx] * W[co,ci,ky,kx].
  * Here "y" is the spatial axis the reference calls y (the innermost one in

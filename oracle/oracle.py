@@ -35,6 +35,8 @@ def lib():
         _lib.oracle_fill_uniform.argtypes = [fp, i64, ctypes.c_uint64]
         _lib.oracle_gemm.argtypes = [fp, fp, fp] + [i64] * 11 + [ctypes.c_int, ctypes.c_int]
         _lib.oracle_gemm_literal.argtypes = [fp, fp, fp] + [i64] * 5
+        _lib.oracle_gemm_ure.argtypes = [fp, fp, fp, i64, i64, i64, ip, i64, i64]
+        _lib.oracle_gemm_ure.restype = None
         _lib.oracle_conv.argtypes = [fp, fp, fp, ip, ip, ip, ip, i64, i64, i64, i64, ctypes.c_int,
                                      i64, ctypes.c_int, ctypes.c_int]
         _lib.oracle_capsule.argtypes = [fp, fp, fp, ip, ip, ip, ip, i64, i64, ctypes.c_int, i64,
@@ -99,6 +101,26 @@ def gemm_literal(A, B, rows=None):
     row0, nrows = (0, M) if rows is None else rows
     C = np.zeros((nrows, N), dtype=np.float32)
     lib().oracle_gemm_literal(_p(A), _p(B), C.ctypes.data - row0 * N * 4, M, N, K, row0, nrows)
+    return C
+
+
+GEMM_GPU_CONSTANTS = (8, 8, 16, 2, 4, 4)   # KKK, JJJ, III, JJ, II, KK (gemm/const-parameters.h:23-29)
+
+
+def gemm_ure(A, B, constants=GEMM_GPU_CONSTANTS, blocks=None):
+    """C = A @ B by the spec's own serial loop nest (gemm.cpp:30,57-71), block rows `blocks` =
+    (i0, i1) of M / (III*II); returns those rows of C."""
+    A = np.ascontiguousarray(A)
+    B = np.ascontiguousarray(B)
+    M, K = A.shape
+    N = B.shape[1]
+    KKK, JJJ, III, JJ, II, KK = constants
+    assert M % (III * II) == 0 and N % (JJJ * JJ) == 0 and K % (KKK * KK) == 0
+    i0, i1 = (0, M // (III * II)) if blocks is None else blocks
+    rows0, rows = i0 * III * II, (i1 - i0) * III * II
+    C = np.zeros((rows, N), dtype=np.float32)
+    c6 = _i64(constants)
+    lib().oracle_gemm_ure(_p(A), _p(B), C.ctypes.data - rows0 * N * 4, M, N, K, c6.ctypes.data, i0, i1)
     return C
 
 

@@ -386,3 +386,14 @@ def test_ger_matches_separately_rounded_numpy_and_tiled_addresses():
                         for kkk in range(KKK):
                             ti, tk = iii + III * ii + III * II * i, kkk + KKK * kk + KKK * KK * k
                             assert Ot[i, k, kk, ii, iii, kkk] == got[ti, tk]
+
+
+def test_gemm_ure_loop_nest_equals_golden_loop_bit_for_bit():
+    """The spec's serial loop nest (gemm.cpp:30,57-71) sums every output in ascending total_k, like the
+    golden loop: same bits, for the GPU and the TINY constant sets."""
+    for consts, (M, N, K) in (((8, 8, 16, 2, 4, 4), (128, 32, 64)), ((4, 4, 4, 4, 4, 4), (32, 48, 32))):
+        A, B = o.fill_uniform((M, K), 70), o.fill_uniform((K, N), 71)
+        assert (o.gemm_ure(A, B, consts) == o.gemm_literal(A, B)).all()
+        III, II = consts[2], consts[4]
+        part = o.gemm_ure(A, B, consts, blocks=(1, 2))
+        assert (part == o.gemm_literal(A, B)[III * II:2 * III * II]).all()
