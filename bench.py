@@ -40,6 +40,9 @@ def parse():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cfg", type=int, default=0,
+                    help="force a tile configuration of the headline SGEMM (T2SP_CFG_*: 1 = 256x256, 2 = 128x128, "
+                         "3 = 64x128); 0 lets the library choose.  For tile-choice profiles.")
     ap.add_argument("--no-others", action="store_true", help="skip the non-headline configurations")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -87,7 +90,7 @@ def time_launches(torch, launch, steps, warmup, min_warm_ms=0.0):
     return wall_ms, avg_ms, best
 
 
-def sgemm_case(torch, t2sp_amd, M, N, K, steps, warmup, seed=1, min_warm_ms=0.0):
+def sgemm_case(torch, t2sp_amd, M, N, K, steps, warmup, seed=1, min_warm_ms=0.0, cfg=0):
     L = t2sp_amd.lib()
     A = t2sp_amd.fill_uniform(torch.empty(M, K, device="cuda"), seed)
     B = t2sp_amd.fill_uniform(torch.empty(K, N, device="cuda"), seed + 1)
@@ -97,7 +100,7 @@ def sgemm_case(torch, t2sp_amd, M, N, K, steps, warmup, seed=1, min_warm_ms=0.0)
     ws = torch.empty(max(nbytes // 4, 1), device="cuda")
 
     def launch():
-        rc = L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, ws.data_ptr(), nbytes,
+        rc = L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, cfg, ws.data_ptr(), nbytes,
                               stream)
         if rc != 0:
             raise RuntimeError("t2sp_sgemm_f32 returned %d" % rc)
@@ -180,7 +183,7 @@ def main():
         del src, dst
 
     M = N = K = 8192
-    r = sgemm_case(torch, t2sp_amd, M, N, K, args.steps, args.warmup)
+    r = sgemm_case(torch, t2sp_amd, M, N, K, args.steps, args.warmup, cfg=args.cfg)
     tflops = r["flop"] / (r["wall_ms"] * 1e-3) / 1e12
     kernel_tflops = r["flop"] / (r["avg_ms"] * 1e-3) / 1e12
 
