@@ -159,7 +159,7 @@ def main():
     args = parse()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (every box has one GPU, "
-              "and the path shards without exchange: see DESIGN.md)" % args.gpus, file=sys.stderr)
+              "and the four operators shard by rows or batch without any exchange)" % args.gpus, file=sys.stderr)
         sys.exit(2)
     import numpy as np
     import torch

@@ -75,7 +75,7 @@ def capsule_config4(torch, steps, warmup, peak):
     ms = _time(torch, launch, max(steps, 200), max(warmup, 20))
     flop = 2.0 * N * CO * 49 * 16 * CI * 9 * 4
     return _entry(flop / ms / 1e9, peak, ms, workload="N=32 CI=CO=32 15x15->7x7 3x3 s2 4x4 poses (configs[3])",
-                  note="back-to-back launches; includes the split-reduction kernel")
+                  note="back-to-back launches of one kernel (no split-reduction pass at this shape)")
 
 
 def mttkrp_config5(torch, steps, warmup, peak):
