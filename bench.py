@@ -43,6 +43,10 @@ def parse():
     ap.add_argument("--cfg", type=int, default=0,
                     help="force a tile configuration of the headline SGEMM (T2SP_CFG_*: 1 = 256x256, 2 = 128x128, "
                          "3 = 64x128); 0 lets the library choose.  For tile-choice profiles.")
+    ap.add_argument("--capsule-cfg", type=int, default=0,
+                    help="force the capsule kernel (T2SP_CFG_*: 2 = 128x128 LDS tiles, 4 = one-wave tiles, 5 = direct) "
+                         "and --capsule-splits its reduction split; for kernel-choice profiles")
+    ap.add_argument("--capsule-splits", type=int, default=0)
     ap.add_argument("--no-others", action="store_true", help="skip the non-headline configurations")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -222,7 +226,8 @@ def main():
             del c
         try:
             from t2sp_amd import bench_ops
-            others.update(bench_ops.run_all(torch, max(5, args.steps // 2), 5, PEAK_FP32_MFMA_TFLOPS))
+            others.update(bench_ops.run_all(torch, max(5, args.steps // 2), 5, PEAK_FP32_MFMA_TFLOPS, args.capsule_cfg,
+                                            args.capsule_splits))
         except ImportError:
             pass
         out["others"] = others

@@ -56,7 +56,7 @@ def conv_config3(torch, steps, warmup, peak):
     return _entry(flop / ms / 1e9, peak, ms, workload="N=64 CI=CO=256 56x56 out 3x3 NCHW (configs[2])")
 
 
-def capsule_config4(torch, steps, warmup, peak):
+def capsule_config4(torch, steps, warmup, peak, cfg=0, splits=0):
     L = lib()
     N, CI, CO = 32, 32, 32
     P = ops.fill_uniform(torch.empty(N, CI, 15, 15, 4, 4, device="cuda"), 1)
@@ -64,18 +64,20 @@ def capsule_config4(torch, steps, warmup, peak):
     V = torch.empty(N, CO, 7, 7, 4, 4, device="cuda")
     dims = (ctypes.c_int * 11)(N, CI, CO, 7, 7, 3, 3, 2, 4, 4, 4)
     sp, sw, sv = ((i64 * 6)(*t.stride()) for t in (P, W, V))
-    nbytes = L.t2sp_capsule_workspace_bytes(dims, 0, 0)
+    nbytes = L.t2sp_capsule_workspace_bytes(dims, cfg, splits)
     ws = torch.empty(max(nbytes // 4, 1), device="cuda")
     s = torch.cuda.current_stream().cuda_stream
 
     def launch():
-        rc = L.t2sp_capsule_f32(P.data_ptr(), W.data_ptr(), V.data_ptr(), dims, sp, sw, sv, 0, 0, ws.data_ptr(), nbytes, s)
+        rc = L.t2sp_capsule_f32(P.data_ptr(), W.data_ptr(), V.data_ptr(), dims, sp, sw, sv, cfg, splits, ws.data_ptr(),
+                                nbytes, s)
         assert rc == 0, rc
 
     ms = _time(torch, launch, max(steps, 200), max(warmup, 20))
     flop = 2.0 * N * CO * 49 * 16 * CI * 9 * 4
     return _entry(flop / ms / 1e9, peak, ms, workload="N=32 CI=CO=32 15x15->7x7 3x3 s2 4x4 poses (configs[3])",
-                  note="back-to-back launches of one kernel (no split-reduction pass at this shape)")
+                  note="back-to-back launches; the library's own choice is one direct kernel without a split-reduction "
+                       "pass" if cfg == 0 else "forced cfg %d splits %d" % (cfg, splits))
 
 
 def mttkrp_config5(torch, steps, warmup, peak):
@@ -146,9 +148,9 @@ def sger_8192(torch, steps, warmup, peak):
                   **{"bound": "hbm", "GB/s": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / 8000.0, 4)})
 
 
-def run_all(torch, steps, warmup, peak):
+def run_all(torch, steps, warmup, peak, capsule_cfg=0, capsule_splits=0):
     return {"conv2d": conv_config3(torch, steps, warmup, peak),
-            "capsule": capsule_config4(torch, steps, warmup, peak),
+            "capsule": capsule_config4(torch, steps, warmup, peak, capsule_cfg, capsule_splits),
             "mttkrp": mttkrp_config5(torch, steps, warmup, peak),
             "ssyrk_8192": ssyrk_8192(torch, steps, warmup, peak),
             "sger_8192": sger_8192(torch, steps, warmup, peak)}
