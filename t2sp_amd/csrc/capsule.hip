@@ -309,6 +309,160 @@ __global__ void __launch_bounds__(NW * 64) capsule_direct_kernel(const CapsuleAr
     }
 }
 
+// The same idea on 16 x 16 MFMA tiles, for an even spread over the CUs.  With 32 x 128 tiles the
+// benchmark shape has 196 workgroups for 256 CUs; here a workgroup owns `rows_per_tile` vote rows
+// (whole pixels: a multiple of 4, up to 16*MB) by 32 columns, and the host picks rows_per_tile so
+// that the workgroups come to just under a multiple of 256 (252 tiles of 100 x 32 at the
+// benchmark shape).  v_mfma_f32_16x16x4_f32 takes per lane one float of X at (row l%16, k-slot
+// l/16) and of Y at (k-slot l/16, col l%16) and leaves D[4*(l/16) + r][l%16] in register r.  A step
+// is 4 pose rows of the reduction (16 k): lane group l/16 loads pose row 4*step + l/16 as 128 bits
+// (its 4 mk) per row block and uses element j in MFMA j, so the k-slots of MFMA j are the mk = j
+// entries of 4 consecutive pose rows; the weights are single floats W[(pose row, mk = j)][co, my].
+// The reduction is split over the 4 waves and summed through LDS in wave order, as above.
+constexpr int D16_WAVES = 4;
+constexpr int D16_RING = 3;
+constexpr int D16_MAX_MB = 8;
+typedef float v4f_acc __attribute__((ext_vector_type(4)));
+
+template <int MB, int NW, int R>
+__global__ void __launch_bounds__(NW * 64) capsule_direct16_kernel(const CapsuleArgs g, int rows_per_tile,
+                                                                   int tab_entries) {
+    extern __shared__ __align__(16) float smem[];
+    v4f *red = reinterpret_cast<v4f *>(smem);                                   // [wave][mb][nb][lane]
+    uint32_t *pix_p = reinterpret_cast<uint32_t *>(smem + NW * MB * 2 * 64 * 4);  // [4*MB] byte offsets in P
+    uint32_t *pix_v = pix_p + 4 * MB;                                            // [4*MB] byte offsets in V, ~0u: none
+    uint2 *tab_all = reinterpret_cast<uint2 *>(pix_v + 4 * MB);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
+    const int tm = blockIdx.x % g.tiles_m, tn = blockIdx.x / g.tiles_m;   // the column tiles of one row tile: same XCD
+    const int r0 = tm * rows_per_tile, n0 = tn * 32;
+
+    // pixels of this tile: offsets of (n, h, w) in P and in V
+    const int pix_total = g.ROWS >> 2, pix0 = r0 >> 2, pix_n = min(rows_per_tile >> 2, pix_total - pix0);
+    if (threadIdx.x < 4 * MB) {
+        const int t = threadIdx.x;
+        const int pix = pix0 + (t < pix_n ? t : 0);
+        const int w = pix % g.OW, hn = pix / g.OW, h = hn % g.OH, n = hn / g.OH;
+        pix_p[t] = 4u * (uint32_t)(int)(n * g.sp[0] + h * g.S * g.sp[2] + w * g.S * g.sp[3]);
+        pix_v[t] = t < pix_n ? 4u * (uint32_t)(int)(n * g.sv[0] + h * g.sv[2] + w * g.sv[3]) : ~0u;
+    }
+    // steps [s0, s1) of 4 pose rows each belong to this wave; byte offsets of its pose rows
+    const int Q = g.KRED >> 2, steps = (Q + 3) >> 2;
+    const int s0 = (int)((int64_t)steps * wave / NW), s1 = (int)((int64_t)steps * (wave + 1) / NW);
+    const int nsteps = s1 - s0;
+    uint2 *tab = tab_all + wave * tab_entries;
+    for (int i = lane; i < 4 * nsteps + 4 * R; i += 64) {
+        const int q = min(4 * s0 + i, Q - 1);
+        const int c = q / (g.KH * g.KW), r = q - c * (g.KH * g.KW);
+        const int kh = r / g.KW, kw = r - kh * g.KW;
+        tab[i] = uint2{4u * (uint32_t)(c * (int)g.sp[1] + kh * (int)g.sp[2] + kw * (int)g.sp[3]),
+                       4u * (uint32_t)(c * (int)g.sw[1] + kh * (int)g.sw[2] + kw * (int)g.sw[3])};
+    }
+    __syncthreads();
+
+    uint32_t p_lane[MB], w_lane[2], v_lane[2];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) p_lane[mb] = pix_p[4 * mb + (li >> 2)] + 4u * (uint32_t)((li & 3) * (int)g.sp[4]);
+    bool col_ok[2];
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++) {
+        const int col = n0 + 16 * nb + li;
+        col_ok[nb] = col < g.COLS;
+        const int co = col_ok[nb] ? col >> 2 : 0;
+        w_lane[nb] = 4u * (uint32_t)(co * (int)g.sw[0] + (li & 3));
+        v_lane[nb] = 4u * (uint32_t)(co * (int)g.sv[1] + (li & 3));
+    }
+    const char *p_base = reinterpret_cast<const char *>(g.P);
+    const char *w_base[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) w_base[j] = reinterpret_cast<const char *>(g.W + j * g.sw[4]);
+
+    v4f ra[R][MB];
+    float rb[R][2][4];
+    const uint2 *tab_lane = tab + lq;
+    uint2 off = tab_lane[0];
+    int t_issue = 0;
+#define T2SP_D16_ISSUE(d)                                                                          \
+    {                                                                                              \
+        const uint32_t op = off.x, ow = off.y;                                                     \
+        t_issue++;                                                                                 \
+        off = tab_lane[4 * t_issue];                                                               \
+        _Pragma("unroll") for (int nb = 0; nb < 2; nb++)                                           \
+            _Pragma("unroll") for (int j = 0; j < 4; j++)                                          \
+                rb[d][nb][j] = *reinterpret_cast<const float *>(w_base[j] + (w_lane[nb] + ow));    \
+        _Pragma("unroll") for (int mb = 0; mb < MB; mb++)                                          \
+            ra[d][mb] = *reinterpret_cast<const v4f *>(p_base + (p_lane[mb] + op));                \
+    }
+    v4f_acc acc[MB][2];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++) acc[mb][nb] = v4f_acc{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+    for (int d = 0; d < R - 1; d++) {
+        T2SP_D16_ISSUE(d)
+        __builtin_amdgcn_sched_barrier(0);   // keep the sets in program order: waits count loads
+    }
+    const int main_iters = nsteps > 0 ? (nsteps - 1) / R : 0;
+    const int rem = nsteps - main_iters * R;
+    for (int it = 0; it < main_iters; it++) {
+#pragma unroll
+        for (int d = 0; d < R; d++) {
+            T2SP_D16_ISSUE((d + R - 1) % R)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+                    for (int nb = 0; nb < 2; nb++)
+                        acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[d][mb][j], rb[d][nb][j], acc[mb][nb], 0, 0, 0);
+            T2SP_INTERLEAVE(SG_VMEM_READ, MB + 8, (8 * MB) / (MB + 8))
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    T2SP_D16_ISSUE(R - 1)
+#undef T2SP_D16_ISSUE
+#pragma unroll
+    for (int d = 0; d < R; d++) {
+        if (d < rem) {
+            const bool live = 4 * (s0 + main_iters * R + d) + lq < Q;   // pose rows past the end add nothing
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int mb = 0; mb < MB; mb++) {
+                    const float a = live ? ra[d][mb][j] : 0.f;
+#pragma unroll
+                    for (int nb = 0; nb < 2; nb++)
+                        acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, rb[d][nb][j], acc[mb][nb], 0, 0, 0);
+                }
+        }
+    }
+
+    // sum the partial tiles of the waves in wave order; register r of a lane is vote row mx = r of
+    // pixel 4*mb + l/16 of the tile, column l%16 of the block
+    v4f *mine = red + wave * MB * 2 * 64 + lane;
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++) mine[(mb * 2 + nb) * 64] = acc[mb][nb];
+    __syncthreads();
+    char *v_base = reinterpret_cast<char *>(g.V);
+    const uint32_t mx_stride = 4u * (uint32_t)(int)g.sv[4];
+    for (int pr = wave; pr < 2 * MB; pr += NW) {
+        const v4f *src = red + pr * 64 + lane;
+        v4f sum = src[0];
+#pragma unroll
+        for (int wv = 1; wv < NW; wv++) sum += src[wv * MB * 2 * 64];
+        const int mb = pr >> 1, nb = pr & 1;
+        const uint32_t pv = pix_v[4 * mb + lq];
+        if (pv != ~0u && col_ok[nb]) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) *reinterpret_cast<float *>(v_base + (pv + v_lane[nb] + r * mx_stride)) = sum[r];
+        }
+    }
+}
+
 // Any pose sizes and strides: one thread per vote element, reduction in (ci,kh,kw,mk) order.
 struct CapsuleGenericArgs {
     const float *P, *W;
@@ -354,7 +508,7 @@ struct CapsulePlan {
     size_t scratch_bytes;
 };
 
-static CapsulePlan plan_capsule(int rows, int cols, int kred, int cfg, int splits) {
+static CapsulePlan plan_capsule(int rows, int cols, int kred, int cfg, int splits, int mx = 0) {
     CapsulePlan p{};
     if (cfg == T2SP_CFG_AUTO) {
         const int64_t t32 = (int64_t)((rows + 31) / 32) * ((cols + 127) / 128);
@@ -363,9 +517,12 @@ static CapsulePlan plan_capsule(int rows, int cols, int kred, int cfg, int split
         // rounds of 256 tiles the second round is mostly empty; very large batches reuse operands
         // better through the shared LDS tiles.
         const bool rounds_ok = t32 <= 256 || t32 >= 384;
-        if (t32 >= 100 && t32 <= DIRECT_MAX_TILES && rounds_ok && kred <= DIRECT_MAX_KRED) cfg = T2SP_CFG_DIRECT;
+        // With 4-row poses the 16 x 16 form spreads any batch up to a few hundred evenly over the
+        // CUs and was the fastest kernel at every batch from 8 to 256 (13-131 us against 19-152 us).
+        if (mx == 4 && t32 <= DIRECT_MAX_TILES && kred <= DIRECT_MAX_KRED) cfg = T2SP_CFG_DIRECT16;
+        else if (t32 >= 100 && t32 <= DIRECT_MAX_TILES && rounds_ok && kred <= DIRECT_MAX_KRED) cfg = T2SP_CFG_DIRECT;
     }
-    if (cfg == T2SP_CFG_DIRECT) {
+    if (cfg == T2SP_CFG_DIRECT || cfg == T2SP_CFG_DIRECT16) {
         p.cfg = cfg; p.splits = 1;
         p.Mp = (rows + 31) / 32 * 32;
         p.Np = (cols + 127) / 128 * 128;
@@ -392,6 +549,61 @@ static CapsulePlan plan_capsule(int rows, int cols, int kred, int cfg, int split
     p.Np = (cols + bn - 1) / bn * bn;
     p.scratch_bytes = splits > 1 ? (size_t)splits * p.Mp * p.Np * sizeof(float) : 0;
     return p;
+}
+
+// The 16 x 16 form: rows per tile (a multiple of 4, at most 16 * D16_MAX_MB) such that the workgroups
+// fill whole rounds of 256 as evenly as possible.
+struct Direct16Plan {
+    int rows_per_tile, mb, tiles_m, tiles_n;
+};
+static Direct16Plan plan_direct16(int rows, int cols) {
+    Direct16Plan p{};
+    p.tiles_n = (cols + 31) / 32;
+    for (int rounds = 1;; rounds++) {
+        const int want_m = (rounds * 256) / p.tiles_n > 0 ? (rounds * 256) / p.tiles_n : 1;
+        int rpt = ((rows + want_m - 1) / want_m + 3) / 4 * 4;
+        if (rpt < 64) rpt = 64;
+        if (rpt <= 16 * D16_MAX_MB) {
+            p.rows_per_tile = rpt;
+            p.mb = (rpt + 15) / 16;
+            p.tiles_m = (rows + rpt - 1) / rpt;
+            return p;
+        }
+    }
+}
+static int direct16_tab_entries(int kred) {
+    const int steps = (kred / 4 + 3) / 4;
+    return 4 * ((steps + D16_WAVES - 1) / D16_WAVES) + 4 * D16_RING + 4;
+}
+static size_t direct16_smem_bytes(int mb, int kred) {
+    return (size_t)D16_WAVES * mb * 2 * 64 * sizeof(v4f) + 2 * 4 * mb * sizeof(uint32_t) +
+           (size_t)D16_WAVES * direct16_tab_entries(kred) * sizeof(uint2);
+}
+
+template <int MB>
+static int launch_direct16_mb(const CapsuleArgs &g, const Direct16Plan &p, hipStream_t stream) {
+    const size_t smem = direct16_smem_bytes(MB, g.KRED);
+    if (smem > 160 * 1024) return T2SP_ERR_SHAPE;
+    auto kern = capsule_direct16_kernel<MB, D16_WAVES, D16_RING>;
+    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+        return T2SP_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(D16_WAVES * 64), smem, stream, g, p.rows_per_tile,
+                       direct16_tab_entries(g.KRED));
+    return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+}
+
+static int launch_capsule_direct16(CapsuleArgs g, hipStream_t stream) {
+    const Direct16Plan p = plan_direct16(g.ROWS, g.COLS);
+    g.tiles_m = p.tiles_m;
+    g.tiles_n = p.tiles_n;
+    switch (p.mb) {
+        case 4: return launch_direct16_mb<4>(g, p, stream);
+        case 5: return launch_direct16_mb<5>(g, p, stream);
+        case 6: return launch_direct16_mb<6>(g, p, stream);
+        case 7: return launch_direct16_mb<7>(g, p, stream);
+        case 8: return launch_direct16_mb<8>(g, p, stream);
+        default: return T2SP_ERR_SHAPE;
+    }
 }
 
 // LDS of the direct kernel: the partial tiles of its waves plus their offset tables.
@@ -447,7 +659,10 @@ static bool capsule_fast(const int *d, const int64_t *sp6, const int64_t *sw6, c
     const int64_t span_w = (int64_t)(d[2] - 1) * sw6[0] + (int64_t)(d[1] - 1) * sw6[1] + (int64_t)(d[5] - 1) * sw6[2] +
                            (int64_t)(d[6] - 1) * sw6[3] + 3 * sw6[4] + 3;
     if (span_p >= INT32_MAX || span_w >= INT32_MAX) return false;
-    *byte_offsets_fit = span_p < (1 << 30) && span_w < (1 << 30);   // the direct kernel's 32-bit byte offsets
+    const int64_t span_v = (int64_t)(d[0] - 1) * sv6[0] + (int64_t)(d[2] - 1) * sv6[1] + (int64_t)(d[3] - 1) * sv6[2] +
+                           (int64_t)(d[4] - 1) * sv6[3] + (int64_t)(d[8] - 1) * sv6[4] + 3;
+    // the direct kernels' 32-bit byte offsets
+    *byte_offsets_fit = span_p < (1 << 30) && span_w < (1 << 30) && span_v < (1 << 30);
     if (sp6[5] != 1 || sw6[5] != 1 || sv6[5] != 1) return false;
     for (int i = 0; i < 5; i++)
         if (sp6[i] % 4 || sw6[i] % 4 || sv6[i] % 4) return false;
@@ -459,7 +674,7 @@ extern "C" size_t t2sp_capsule_workspace_bytes(const int *dims11, int cfg, int s
     if (!d) return 0;
     const int64_t rows = (int64_t)d[0] * d[3] * d[4] * d[8], cols = (int64_t)d[2] * 4, kred = (int64_t)d[1] * d[5] * d[6] * 4;
     if (rows <= 0 || rows > INT32_MAX || cols > INT32_MAX || kred > INT32_MAX) return 0;
-    return t2sp::plan_capsule((int)rows, (int)cols, (int)kred, cfg, splits).scratch_bytes;
+    return t2sp::plan_capsule((int)rows, (int)cols, (int)kred, cfg, splits, dims11[8]).scratch_bytes;
 }
 
 extern "C" int t2sp_capsule_f32(const float *P, const float *W, float *V, const int *dims11,
@@ -482,9 +697,12 @@ extern "C" int t2sp_capsule_f32(const float *P, const float *W, float *V, const 
         hipLaunchKernelGGL(capsule_scalar_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
         return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
     }
-    CapsulePlan p = plan_capsule((int)rows, (int)cols, (int)kred, cfg, splits);
+    CapsulePlan p = plan_capsule((int)rows, (int)cols, (int)kred, cfg, splits, d[8]);
     if (p.cfg == T2SP_CFG_DIRECT && !(byte_offsets_fit && direct_smem_bytes((int)kred) <= 160 * 1024))
         p = plan_capsule((int)rows, (int)cols, (int)kred, T2SP_CFG_128x128, 1);   // needs no workspace either
+    if (p.cfg == T2SP_CFG_DIRECT16 &&
+        !(byte_offsets_fit && d[8] == 4 && direct16_smem_bytes(D16_MAX_MB, (int)kred) <= 160 * 1024))
+        p = plan_capsule((int)rows, (int)cols, (int)kred, T2SP_CFG_128x128, 1);
     if (p.scratch_bytes > workspace_bytes || (p.scratch_bytes && !workspace)) return T2SP_ERR_SHAPE;
     CapsuleArgs g{};
     g.P = P; g.W = W; g.V = V;
@@ -494,6 +712,7 @@ extern "C" int t2sp_capsule_f32(const float *P, const float *W, float *V, const 
     g.splits = p.splits; g.Mp = p.Mp; g.Np = p.Np; g.scratch = workspace;
     switch (p.cfg) {
         case T2SP_CFG_DIRECT: return launch_capsule_direct(g, (hipStream_t)stream);
+        case T2SP_CFG_DIRECT16: return launch_capsule_direct16(g, (hipStream_t)stream);
         case T2SP_CFG_256x256: return launch_capsule<CapsL>(g, (hipStream_t)stream);
         case T2SP_CFG_128x128: return launch_capsule<CapsM>(g, (hipStream_t)stream);
         case T2SP_CFG_64x128: return launch_capsule<CapsS>(g, (hipStream_t)stream);

@@ -20,7 +20,7 @@ def test_constant_fixture_exact():
     assert V.shape == (2, 8, 7, 7, 4, 4) and (V == 1152).all()
 
 
-@pytest.mark.parametrize("cfg,splits", [(0, 0), (5, 0), (2, 1), (2, 3), (3, 2), (4, 2), (1, 2), (99, 0)])
+@pytest.mark.parametrize("cfg,splits", [(0, 0), (5, 0), (6, 0), (2, 1), (2, 3), (3, 2), (4, 2), (1, 2), (99, 0)])
 def test_tiny_constants_parity_golden_and_ure_order(oracle, cfg, splits):
     """The TINY sizes of capsule/const-parameters.h:43-52 with N=4 (capsule-run-fpga.cpp:37-39):
     16 -> 16 channels, 15x15 -> 7x7, against both reduction orders the reference uses."""
@@ -59,7 +59,7 @@ def test_oneapi_memory_layout_and_other_strides(oracle):
 
 
 @pytest.mark.parametrize("ci,co,n", [(1, 3, 1), (3, 40, 2), (5, 8, 3), (7, 33, 1)])
-@pytest.mark.parametrize("cfg", [5, 2])
+@pytest.mark.parametrize("cfg", [5, 6, 2])
 def test_short_and_odd_reductions_ragged_columns(oracle, ci, co, n, cfg):
     """Reductions of an odd number of pose rows (CI*9 odd), shorter than the number of waves
     that share them, and vote columns that do not fill a 128-column tile."""
@@ -74,6 +74,16 @@ def test_other_pose_sizes_take_the_scalar_kernel(oracle):
     assert rel_fro(t2sp_amd.capsule(P, W), oracle.capsule(P, W))[0] <= TOL
 
 
+@pytest.mark.parametrize("cfg", [5, 6])
+@pytest.mark.parametrize("n", [1, 5, 48])
+def test_direct_kernels_other_batches(oracle, cfg, n):
+    """Batches whose vote rows do not fill the last tile, through both direct kernels."""
+    P, W = oracle.fill_uniform((n, 8, 15, 15, 4, 4), 21), oracle.fill_uniform((12, 8, 3, 3, 4, 4), 22)
+    got = t2sp_amd.capsule(P, W, cfg=cfg)
+    err, mx = rel_fro(got, oracle.capsule(P, W))
+    assert err <= TOL, (cfg, n, err, mx)
+
+
 def test_config4_full_size(oracle):
     """BASELINE config 4: N=32, CI=CO=32, 15x15 -> 7x7, 3x3, stride 2, on the device, whole
     result against the oracle."""
@@ -83,6 +93,10 @@ def test_config4_full_size(oracle):
     V = t2sp_amd.capsule(P, W)
     torch.cuda.synchronize()
     ref = oracle.capsule(P.cpu().numpy(), W.cpu().numpy())
+    for cfg in (5, 6):          # both direct kernels at the full size, whichever the library prefers
+        Vc = t2sp_amd.capsule(P, W, cfg=cfg)
+        torch.cuda.synchronize()
+        assert rel_fro(Vc.cpu().numpy(), ref)[0] <= TOL, cfg
     err, mx = rel_fro(V.cpu().numpy(), ref)
     print("capsule full size rel_fro %.3e max_abs %.3e" % (err, mx))
     assert err <= TOL
