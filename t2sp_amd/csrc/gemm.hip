@@ -220,6 +220,131 @@ __global__ void __launch_bounds__(NW * 64) sgemm_direct_kernel(const GemmArgs g)
     }
 }
 
+// The same one-launch form on 16 x 16 MFMA tiles, for an even spread of any small product over the
+// CUs: a workgroup owns `rows_per_tile` rows (any number up to 16*MB) by 16*NB columns, and the host
+// picks the tile so that the workgroups fill rounds of 256 CUs with the least idle time.
+// v_mfma_f32_16x16x4_f32 takes per lane one float of A at (row l%16, k-slot l/16) and of B at
+// (k-slot l/16, col l%16) and leaves D[4*(l/16) + r][l%16] in register r.  A step is 16 k: lane
+// group l/16 loads A[row][16*step + 4*(l/16) ..+3] as 128 bits per row block and uses element j in
+// MFMA j; accumulator nb holds the columns congruent to nb modulo NB, so a lane loads the NB
+// adjacent floats B[16*step + 4*(l/16) + j][c0 + NB*(l%16) ..] with one load and later stores NB
+// adjacent outputs with one store.
+constexpr int GEMM_D16_WAVES = 4;
+constexpr int GEMM_D16_RING = 3;
+template <int NB> struct VecOf;
+template <> struct VecOf<2> { typedef float type __attribute__((ext_vector_type(2))); };
+template <> struct VecOf<4> { typedef float type __attribute__((ext_vector_type(4))); };
+
+template <int MB, int NB, int NW, int R>
+__global__ void __launch_bounds__(NW * 64) sgemm_direct16_kernel(const GemmArgs g, int rows_per_tile) {
+    typedef typename VecOf<NB>::type vnb;
+    extern __shared__ __align__(16) float smem[];
+    v4f *red = reinterpret_cast<v4f *>(smem);            // [wave][mb][nb][lane]
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
+    const int tm = blockIdx.x % g.tiles_m, tn = blockIdx.x / g.tiles_m;
+    const int m0 = tm * rows_per_tile, n0 = tn * 16 * NB;
+    const int m_end = min(m0 + rows_per_tile, g.M);
+    const int steps = g.K >> 4;
+    const int s0 = (int)((int64_t)steps * wave / NW), s1 = (int)((int64_t)steps * (wave + 1) / NW);
+    const int nsteps = s1 - s0;
+
+    uint32_t a_off[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+        const int row = min(m0 + 16 * mb + li, g.M - 1);
+        a_off[mb] = 4u * (uint32_t)(row * (int)g.lda + 4 * lq);
+    }
+    const int col = n0 + NB * li;
+    const bool col_ok = col + NB <= g.N;
+    const uint32_t b_off = 4u * (uint32_t)(4 * lq * (int)g.ldb + (col_ok ? col : 0));
+    const char *a_base = reinterpret_cast<const char *>(g.A + 16 * s0);
+    const char *b_base = reinterpret_cast<const char *>(g.B + (int64_t)16 * s0 * g.ldb);
+    const int64_t b_row = 4 * g.ldb, b_step = 64 * g.ldb;   // bytes per k-row and per step
+    int issued = 0;
+
+    v4f ra[R][MB];
+    vnb rb[R][4];
+#define T2SP_GEMM_D16_ISSUE(d)                                                                      \
+    {                                                                                               \
+        const int st = min(issued, steps - 1 - s0);                                                 \
+        const char *ap = a_base + 64 * st;                                                          \
+        const char *bp = b_base + (int64_t)st * b_step;                                             \
+        issued++;                                                                                   \
+        _Pragma("unroll") for (int j = 0; j < 4; j++)                                               \
+            rb[d][j] = *reinterpret_cast<const vnb *>(bp + j * b_row + b_off);                      \
+        _Pragma("unroll") for (int mb = 0; mb < MB; mb++)                                           \
+            ra[d][mb] = *reinterpret_cast<const v4f *>(ap + a_off[mb]);                             \
+    }
+#define T2SP_GEMM_D16_MMA(d)                                                                        \
+    _Pragma("unroll") for (int j = 0; j < 4; j++)                                                   \
+        _Pragma("unroll") for (int mb = 0; mb < MB; mb++)                                           \
+            _Pragma("unroll") for (int nb = 0; nb < NB; nb++)                                       \
+                acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[d][mb][j], rb[d][j][nb], acc[mb][nb], 0, 0, 0);
+    v4f acc[MB][NB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) acc[mb][nb] = v4f{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+    for (int d = 0; d < R - 1; d++) {
+        T2SP_GEMM_D16_ISSUE(d)
+        __builtin_amdgcn_sched_barrier(0);   // keep the sets in program order: waits count loads
+    }
+    const int main_iters = nsteps > 0 ? (nsteps - 1) / R : 0;
+    const int rem = nsteps - main_iters * R;
+    for (int it = 0; it < main_iters; it++) {
+#pragma unroll
+        for (int d = 0; d < R; d++) {
+            T2SP_GEMM_D16_ISSUE((d + R - 1) % R)
+            T2SP_GEMM_D16_MMA(d)
+            T2SP_INTERLEAVE(SG_VMEM_READ, MB + 4, (4 * MB * NB) / (MB + 4))
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    T2SP_GEMM_D16_ISSUE(R - 1)
+#pragma unroll
+    for (int d = 0; d < R; d++) {
+        if (d < rem) { T2SP_GEMM_D16_MMA(d) }
+    }
+#undef T2SP_GEMM_D16_ISSUE
+#undef T2SP_GEMM_D16_MMA
+
+    // sum the partial tiles of the waves in wave order
+    v4f *mine = red + wave * MB * NB * 64 + lane;
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) mine[(mb * NB + nb) * 64] = acc[mb][nb];
+    __syncthreads();
+    for (int mb = wave; mb < MB; mb += NW) {
+        v4f sum[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+            const v4f *src = red + (mb * NB + nb) * 64 + lane;
+            sum[nb] = src[0];
+#pragma unroll
+            for (int wv = 1; wv < NW; wv++) sum[nb] += src[wv * MB * NB * 64];
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int row = m0 + 16 * mb + 4 * lq + r;
+            vnb out;
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) out[nb] = sum[nb][r];
+            if (row < m_end && col_ok) {
+                if (!g.tiled) {
+                    *reinterpret_cast<vnb *>(g.C + (int64_t)row * g.ldc + col) = out;
+                } else {
+#pragma unroll
+                    for (int nb = 0; nb < NB; nb++) g.C[tiled_offset(g, row, col + nb)] = out[nb];
+                }
+            }
+        }
+    }
+}
+
 // Fallback for shapes the vector loaders cannot take (K or N not a multiple
 // of 4, or operands not 16-byte aligned): one thread per output, sequential k.
 __global__ void sgemm_scalar_kernel(const GemmArgs g, int bt) {
@@ -318,9 +443,74 @@ static int launch_direct(GemmArgs g, hipStream_t stream) {
     return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
 }
 
+// Tile of the 16 x 16 form for an M x N output: the candidate (MB, NB, rows_per_tile) with the least
+// estimated time = rounds of 256 workgroups x padded tile area x a penalty for narrow tiles (more
+// loads per MFMA).
+struct GemmD16Plan {
+    int mb, nb, rows_per_tile, tiles_m, tiles_n;
+    double cost;
+};
+static GemmD16Plan plan_gemm_d16(int M, int N) {
+    GemmD16Plan best{};
+    best.cost = 1e300;
+    for (int nb = 2; nb <= 4; nb += 2)
+        for (int mb = 2; mb <= 8; mb++) {
+            if (mb * nb > 24) continue;                           // accumulators + operand ring must fit
+            const int tiles_m = (M + 16 * mb - 1) / (16 * mb), tiles_n = (N + 16 * nb - 1) / (16 * nb);
+            const int rpt = (M + tiles_m - 1) / tiles_m;
+            const int64_t tiles = (int64_t)tiles_m * tiles_n;
+            const double loads_per_mfma = (double)(mb + 4) / (4.0 * mb * nb);
+            const double cost = (double)((tiles + 255) / 256) * (16.0 * mb) * (16.0 * nb) * (1.0 + 1.5 * loads_per_mfma);
+            if (cost < best.cost) best = GemmD16Plan{mb, nb, rpt, tiles_m, tiles_n, cost};
+        }
+    return best;
+}
+
+static bool gemm_d16_ok(const GemmArgs &g) {
+    return g.K % 16 == 0 && g.N % 4 == 0 && g.ldb % 4 == 0 && (g.tiled || g.ldc % 4 == 0) && g.lda % 4 == 0 &&
+           ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) && ((uintptr_t)g.C % 16 == 0) &&
+           (int64_t)g.M * g.lda < (1 << 30) && (int64_t)g.K * g.ldb < (1 << 30);
+}
+
+template <int MB, int NB>
+static int launch_d16_t(GemmArgs g, const GemmD16Plan &p, hipStream_t stream) {
+    g.tiles_m = p.tiles_m;
+    g.tiles_n = p.tiles_n;
+    const size_t smem = (size_t)GEMM_D16_WAVES * MB * NB * 64 * sizeof(v4f);
+    auto kern = sgemm_direct16_kernel<MB, NB, GEMM_D16_WAVES, GEMM_D16_RING>;
+    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+        return T2SP_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(GEMM_D16_WAVES * 64), smem, stream, g, p.rows_per_tile);
+    return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+}
+
+static int launch_d16(const GemmArgs &g, hipStream_t stream) {
+    const GemmD16Plan p = plan_gemm_d16(g.M, g.N);
+#define T2SP_D16_CASE(MBV, NBV) if (p.mb == MBV && p.nb == NBV) return launch_d16_t<MBV, NBV>(g, p, stream);
+    T2SP_D16_CASE(2, 2) T2SP_D16_CASE(3, 2) T2SP_D16_CASE(4, 2) T2SP_D16_CASE(5, 2) T2SP_D16_CASE(6, 2)
+    T2SP_D16_CASE(7, 2) T2SP_D16_CASE(8, 2) T2SP_D16_CASE(2, 4) T2SP_D16_CASE(3, 4) T2SP_D16_CASE(4, 4)
+    T2SP_D16_CASE(5, 4) T2SP_D16_CASE(6, 4)
+#undef T2SP_D16_CASE
+    return T2SP_ERR_SHAPE;
+}
+
 static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *workspace = nullptr,
                     size_t workspace_bytes = 0) {
     if (g.M <= 0 || g.N <= 0 || g.K <= 0) return T2SP_ERR_SHAPE;
+    if (cfg == T2SP_CFG_DIRECT16)
+        return (!bt && !g.scale && gemm_d16_ok(g)) ? launch_d16(g, stream) : T2SP_ERR_SHAPE;
+    if (cfg == T2SP_CFG_AUTO && !bt && !g.scale && gemm_d16_ok(g)) {
+        // Measured from 256^2 x 8192 to 3072^2 x 1024: the 16 x 16 form wins whenever 256 x 256 tiles
+        // would not fill the chip, except where 128 x 128 tiles do and the reduction is long enough to
+        // amortise their prologue, and for tiny outputs with a long reduction (too few tiles even at
+        // 32 x 32: the reduction has to be split over workgroups).
+        const int64_t t256 = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
+        const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
+        const GemmD16Plan p = plan_gemm_d16(g.M, g.N);
+        const bool tiled_better = t128 >= 200 && g.K >= 2048;
+        const bool too_few = (int64_t)p.tiles_m * p.tiles_n < 128 && g.K >= 4096;
+        if (t256 < 200 && !tiled_better && !too_few && g.K >= 64) return launch_d16(g, stream);
+    }
     if ((cfg == T2SP_CFG_AUTO || cfg == T2SP_CFG_DIRECT) && !bt && !g.scale && !g.tiled &&
         g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && gemm_direct_ok(g, cfg == T2SP_CFG_DIRECT))
         return launch_direct(g, stream);

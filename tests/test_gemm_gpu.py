@@ -188,6 +188,30 @@ def test_direct_kernel_small_products(oracle, torch_cuda, shape):
                             None) == -8
 
 
+@pytest.mark.parametrize("shape", [(1024, 1024, 1024), (500, 260, 4096), (64, 128, 8192), (130, 68, 64), (1, 4, 16),
+                                   (640, 512, 1024), (1536, 1536, 1536), (200, 36, 48), (97, 1000, 160)])
+def test_direct16_kernel_small_products(oracle, torch_cuda, shape):
+    """The one-launch kernel on 16 x 16 MFMA tiles, whose tile is chosen per problem to fill the CUs
+    evenly: forced through the thin layer, against the oracle, same bits twice."""
+    torch = torch_cuda
+    M, N, K = shape
+    L = t2sp_amd.lib()
+    A = t2sp_amd.fill_uniform(torch.empty(M, K, device="cuda"), 33)
+    B = t2sp_amd.fill_uniform(torch.empty(K, N, device="cuda"), 34)
+    outs = []
+    for _ in range(2):
+        C = torch.full((M, N), float("nan"), device="cuda")
+        assert L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 6, None, 0, None) == 0
+        torch.cuda.synchronize()
+        outs.append(C.cpu().numpy())
+    assert (outs[0] == outs[1]).all()
+    err, mx = rel_fro(outs[0], oracle.gemm(A.cpu().numpy(), B.cpu().numpy()))
+    print("direct16 %s rel_fro %.3e max_abs %.3e" % (shape, err, mx))
+    assert err <= TOL
+    assert L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K - 8 if K > 8 else 8, K, N, N, 6, None, 0,
+                            None) == -8
+
+
 def test_empty_extents():
     C = np.full((16, 8), np.nan, np.float32)
     t2sp_amd.gemm(np.zeros((16, 0), np.float32), np.zeros((0, 8), np.float32), out=C)
