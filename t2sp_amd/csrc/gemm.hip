@@ -334,6 +334,10 @@ __global__ void __launch_bounds__(NW * 64) sgemm_direct16_kernel(const GemmArgs 
 #pragma unroll
             for (int nb = 0; nb < NB; nb++) out[nb] = sum[nb][r];
             if (row < m_end && col_ok) {
+                if (g.scale) {
+                    out = out * g.alpha;
+                    if (g.beta != 0.f) out += *reinterpret_cast<const vnb *>(g.Cin + (int64_t)row * g.ldcin + col) * g.beta;
+                }
                 if (!g.tiled) {
                     *reinterpret_cast<vnb *>(g.C + (int64_t)row * g.ldc + col) = out;
                 } else {
@@ -469,7 +473,8 @@ static GemmD16Plan plan_gemm_d16(int M, int N) {
 static bool gemm_d16_ok(const GemmArgs &g) {
     return g.K % 16 == 0 && g.N % 4 == 0 && g.ldb % 4 == 0 && (g.tiled || g.ldc % 4 == 0) && g.lda % 4 == 0 &&
            ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) && ((uintptr_t)g.C % 16 == 0) &&
-           (int64_t)g.M * g.lda < (1 << 30) && (int64_t)g.K * g.ldb < (1 << 30);
+           (int64_t)g.M * g.lda < (1 << 30) && (int64_t)g.K * g.ldb < (1 << 30) &&
+           (!g.scale || (g.ldcin % 4 == 0 && (uintptr_t)g.Cin % 16 == 0));
 }
 
 template <int MB, int NB>
@@ -498,8 +503,8 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
                     size_t workspace_bytes = 0) {
     if (g.M <= 0 || g.N <= 0 || g.K <= 0) return T2SP_ERR_SHAPE;
     if (cfg == T2SP_CFG_DIRECT16)
-        return (!bt && !g.scale && gemm_d16_ok(g)) ? launch_d16(g, stream) : T2SP_ERR_SHAPE;
-    if (cfg == T2SP_CFG_AUTO && !bt && !g.scale && gemm_d16_ok(g)) {
+        return (!bt && gemm_d16_ok(g)) ? launch_d16(g, stream) : T2SP_ERR_SHAPE;
+    if (cfg == T2SP_CFG_AUTO && !bt && gemm_d16_ok(g)) {
         // Measured from 256^2 x 8192 to 3072^2 x 1024: the 16 x 16 form wins whenever 256 x 256 tiles
         // would not fill the chip, except where 128 x 128 tiles do and the reduction is long enough to
         // amortise their prologue, and for tiny outputs with a long reduction (too few tiles even at
