@@ -512,9 +512,13 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         const int64_t t256 = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
         const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
         const GemmD16Plan p = plan_gemm_d16(g.M, g.N);
-        const bool tiled_better = t128 >= 200 && g.K >= 2048;
+        // how much of the large tiles would hold outputs (a thin matrix leaves them mostly empty)
+        const double fill256 = (double)g.M * g.N / ((double)t256 * 65536.0);
+        const double fill128 = (double)g.M * g.N / ((double)t128 * 16384.0);
+        const bool big_tiles = t256 >= 200 && fill256 >= 0.6;
+        const bool tiled_better = t128 >= 200 && g.K >= 2048 && fill128 >= 0.6;
         const bool too_few = (int64_t)p.tiles_m * p.tiles_n < 128 && g.K >= 4096;
-        if (t256 < 200 && !tiled_better && !too_few && g.K >= 64) return launch_d16(g, stream);
+        if (!big_tiles && !tiled_better && !too_few && g.K >= 64) return launch_d16(g, stream);
     }
     if ((cfg == T2SP_CFG_AUTO || cfg == T2SP_CFG_DIRECT) && !bt && !g.scale && !g.tiled &&
         g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && gemm_direct_ok(g, cfg == T2SP_CFG_DIRECT))
