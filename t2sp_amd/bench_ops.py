@@ -104,13 +104,12 @@ def mttkrp_config5(torch, steps, warmup, peak):
                   note="includes the split-reduction kernel")
 
 
-def ssyrk_8192(torch, steps, warmup, peak):
+def ssyrk_case(torch, steps, warmup, peak, N, K, note):
     """Not a BASELINE configuration: the SYRK pipeline (t2s/tests/performance/syrk) at the headline
-    GEMM size.  Only the tiles on or above the diagonal are multiplied; the rate counts the
+    GEMM size and at the size the reference's BLAS release is built for.  Only the tiles on or above the diagonal are multiplied; the rate counts the
     N*(N+1)/2 distinct outputs (N*(N+1)*K flop).  The reference's own report counts 2*N*N*K
     (syrk-run-fpga.cpp:99), given as `TFLOP/s_reference_count`."""
     L = lib()
-    N = K = 8192
     A = ops.fill_uniform(torch.empty(N, K, device="cuda"), 1)
     C = ops.fill_uniform(torch.empty(N, N, device="cuda"), 2)
     O = torch.empty(N, N, device="cuda")
@@ -122,7 +121,7 @@ def ssyrk_8192(torch, steps, warmup, peak):
 
     ms = _time(torch, launch, steps, warmup)
     flop = float(N) * (N + 1) * K
-    return _entry(flop / ms / 1e9, peak, ms, workload="N=K=8192, both triangles written, alpha/beta epilogue",
+    return _entry(flop / ms / 1e9, peak, ms, workload="N=%d K=%d, both triangles written, alpha/beta epilogue%s" % (N, K, note),
                   **{"TFLOP/s_reference_count": round(2.0 * N * N * K / ms / 1e9, 3)})
 
 
@@ -152,5 +151,7 @@ def run_all(torch, steps, warmup, peak, capsule_cfg=0, capsule_splits=0):
     return {"conv2d": conv_config3(torch, steps, warmup, peak),
             "capsule": capsule_config4(torch, steps, warmup, peak, capsule_cfg, capsule_splits),
             "mttkrp": mttkrp_config5(torch, steps, warmup, peak),
-            "ssyrk_8192": ssyrk_8192(torch, steps, warmup, peak),
+            "ssyrk_8192": ssyrk_case(torch, steps, warmup, peak, 8192, 8192, ""),
+            "ssyrk_768x1024": ssyrk_case(torch, max(steps, 200), max(warmup, 20), peak, 768, 1024,
+                                         " (the size of peppers/blas/level3/syrk/release/s10)"),
             "sger_8192": sger_8192(torch, steps, warmup, peak)}

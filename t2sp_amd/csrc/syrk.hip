@@ -164,6 +164,194 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) ssyrk_kernel(const SyrkArgs g) 
     });
 }
 
+// Small N: few tiles for 256 CUs, and 1024-long reductions that a launch gap rivals.  One launch
+// on 16 x 16 MFMA tiles, like the small-product SGEMM kernel: a workgroup of 4 waves owns
+// `rows_per_tile` rows by 16*NB columns of the result, splits the reduction over its waves with
+// both operands loaded straight from A into MFMA operand registers (a step is 16 k: lane group
+// l/16 loads A[row][16*step + 4*(l/16) ..+3] for its row blocks and A[col][same k] for its column
+// blocks, element j feeding MFMA j), and sums the four partial tiles through LDS in wave order.
+// Only tiles that touch the upper triangle are launched; the host picks the tile shape so that they
+// fill rounds of 256 CUs evenly.  Only elements on or above the diagonal are stored, each with
+// its mirror image where the output form wants one.
+constexpr int SYRK_D16_WAVES = 4;
+constexpr int SYRK_D16_RING = 3;
+
+template <int MODE>
+__device__ __forceinline__ void syrk_store_upper(const SyrkArgs &g, int r, int c, float acc) {
+    if (c < r) return;
+    if constexpr (MODE == SYRK_FLAT_SYM) {
+        const bool want_upper = g.upper || g.mirror, want_lower = !g.upper || g.mirror;
+        const float v = syrk_value<MODE>(g, r, c, acc);
+        if (want_upper || r == c) g.C[(int64_t)r * g.ldc + c] = v;
+        if (want_lower && r != c) g.C[(int64_t)c * g.ldc + r] = v;
+    } else if constexpr (MODE == SYRK_FLAT_FULL) {
+        g.C[(int64_t)r * g.ldc + c] = syrk_value<MODE>(g, r, c, acc);
+        if (c > r) g.C[(int64_t)c * g.ldc + r] = syrk_value<MODE>(g, c, r, acc);
+    } else {
+        const int B = g.f_iii * g.f_ii;
+        g.C[syrk_folded_offset(g, r, c)] = syrk_value<MODE>(g, r, c, acc);
+        if (r / B == c / B && r != c) g.C[syrk_folded_offset(g, c, r)] = syrk_value<MODE>(g, c, r, acc);
+    }
+}
+
+template <int MB, int NB, int MODE, int NW, int R>
+__global__ void __launch_bounds__(NW * 64) ssyrk_direct16_kernel(const SyrkArgs g, int rows_per_tile, int tiles_m) {
+    extern __shared__ __align__(16) float smem[];
+    v4f *red = reinterpret_cast<v4f *>(smem);            // [wave][mb][nb][lane]
+    // workgroup id -> (row tile, column tile) over the tiles that touch the upper triangle only,
+    // row by row: launching the empty ones too and letting them exit leaves whole XCDs with little
+    // work, because the round-robin deal of ids to XCDs then lines up with the row tiles
+    int tm = 0, rest = blockIdx.x;
+    const int tiles_n = (g.N + 16 * NB - 1) / (16 * NB);
+    for (; tm < tiles_m; tm++) {
+        const int count = tiles_n - (tm * rows_per_tile) / (16 * NB);
+        if (rest < count) break;
+        rest -= count;
+    }
+    const int tn = (tm * rows_per_tile) / (16 * NB) + rest;
+    const int m0 = tm * rows_per_tile, n0 = tn * 16 * NB;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
+    const int m_end = min(m0 + rows_per_tile, g.N);
+    const int steps = g.K >> 4;
+    const int s0 = (int)((int64_t)steps * wave / NW), s1 = (int)((int64_t)steps * (wave + 1) / NW);
+    const int nsteps = s1 - s0;
+
+    uint32_t a_off[MB], b_off[NB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) a_off[mb] = 4u * (uint32_t)(min(m0 + 16 * mb + li, g.N - 1) * (int)g.lda + 4 * lq);
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) b_off[nb] = 4u * (uint32_t)(min(n0 + 16 * nb + li, g.N - 1) * (int)g.lda + 4 * lq);
+    const char *a_base = reinterpret_cast<const char *>(g.A + 16 * s0);
+    int issued = 0;
+
+    v4f ra[R][MB], rb[R][NB];
+#define T2SP_SYRK_D16_ISSUE(d)                                                                      \
+    {                                                                                               \
+        const char *ap = a_base + 64 * min(issued, steps - 1 - s0);                                 \
+        issued++;                                                                                   \
+        _Pragma("unroll") for (int nb = 0; nb < NB; nb++)                                           \
+            rb[d][nb] = *reinterpret_cast<const v4f *>(ap + b_off[nb]);                             \
+        _Pragma("unroll") for (int mb = 0; mb < MB; mb++)                                           \
+            ra[d][mb] = *reinterpret_cast<const v4f *>(ap + a_off[mb]);                             \
+    }
+#define T2SP_SYRK_D16_MMA(d)                                                                        \
+    _Pragma("unroll") for (int j = 0; j < 4; j++)                                                   \
+        _Pragma("unroll") for (int mb = 0; mb < MB; mb++)                                           \
+            _Pragma("unroll") for (int nb = 0; nb < NB; nb++)                                       \
+                acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[d][mb][j], rb[d][nb][j], acc[mb][nb], 0, 0, 0);
+    v4f acc[MB][NB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) acc[mb][nb] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int d = 0; d < R - 1; d++) {
+        T2SP_SYRK_D16_ISSUE(d)
+        __builtin_amdgcn_sched_barrier(0);   // keep the sets in program order: waits count loads
+    }
+    const int main_iters = nsteps > 0 ? (nsteps - 1) / R : 0;
+    const int rem = nsteps - main_iters * R;
+    for (int it = 0; it < main_iters; it++) {
+#pragma unroll
+        for (int d = 0; d < R; d++) {
+            T2SP_SYRK_D16_ISSUE((d + R - 1) % R)
+            T2SP_SYRK_D16_MMA(d)
+            T2SP_INTERLEAVE(SG_VMEM_READ, MB + NB, (4 * MB * NB) / (MB + NB))
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    T2SP_SYRK_D16_ISSUE(R - 1)
+#pragma unroll
+    for (int d = 0; d < R; d++) {
+        if (d < rem) { T2SP_SYRK_D16_MMA(d) }
+    }
+#undef T2SP_SYRK_D16_ISSUE
+#undef T2SP_SYRK_D16_MMA
+
+    v4f *mine = red + wave * MB * NB * 64 + lane;
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) mine[(mb * NB + nb) * 64] = acc[mb][nb];
+    __syncthreads();
+    for (int pr = wave; pr < MB * NB; pr += NW) {
+        const v4f *src = red + pr * 64 + lane;
+        v4f sum = src[0];
+#pragma unroll
+        for (int wv = 1; wv < NW; wv++) sum += src[wv * MB * NB * 64];
+        const int mb = pr / NB, nb = pr - mb * NB;
+        const int col = n0 + 16 * nb + li;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int row = m0 + 16 * mb + 4 * lq + r;
+            if (row < m_end && col < g.N) syrk_store_upper<MODE>(g, row, col, sum[r]);
+        }
+    }
+}
+
+// Tile shape of the 16 x 16 form for an N x N triangle: least estimated time = rounds of 256
+// workgroups (counting only tiles that touch the upper triangle) x (padded tile area x a penalty
+// for small tiles, which need more loads per MFMA, + a fixed cost per round).
+struct SyrkD16Plan {
+    int mb, nb, rows_per_tile, tiles_m, tiles_n;
+    double cost;
+    int64_t needed;
+};
+static SyrkD16Plan plan_syrk_d16(int N) {
+    SyrkD16Plan best{};
+    best.cost = 1e300;
+    for (int nb = 2; nb <= 4; nb++)
+        for (int mb = 2; mb <= 8; mb++) {
+            if (mb * nb > 24) continue;
+            const int tiles_m = (N + 16 * mb - 1) / (16 * mb), tiles_n = (N + 16 * nb - 1) / (16 * nb);
+            const int rpt = (N + tiles_m - 1) / tiles_m;
+            int64_t needed = 0;
+            for (int tm = 0; tm < tiles_m; tm++) {
+                const int first_tn = (tm * rpt) / (16 * nb);      // first column tile not entirely left of the rows
+                needed += tiles_n - first_tn;
+            }
+            const double loads_per_mfma = (double)(mb + nb) / (4.0 * mb * nb);
+            // + a fixed cost per round (prologue, exchange, store) worth about 1500 outputs of work
+            const double cost = (double)((needed + 255) / 256) * ((16.0 * mb) * (16.0 * nb) * (1.0 + 1.5 * loads_per_mfma) + 1500.0);
+            if (cost < best.cost) best = SyrkD16Plan{mb, nb, rpt, tiles_m, tiles_n, cost, needed};
+        }
+    return best;
+}
+
+template <int MB, int NB>
+static int launch_syrk_d16_t(const SyrkArgs &g, const SyrkD16Plan &p, hipStream_t stream) {
+    const size_t smem = (size_t)SYRK_D16_WAVES * MB * NB * 64 * sizeof(v4f);
+    void (*kern)(const SyrkArgs, int, int);
+    switch (g.mode) {
+        case SYRK_FLAT_SYM: kern = ssyrk_direct16_kernel<MB, NB, SYRK_FLAT_SYM, SYRK_D16_WAVES, SYRK_D16_RING>; break;
+        case SYRK_FLAT_FULL: kern = ssyrk_direct16_kernel<MB, NB, SYRK_FLAT_FULL, SYRK_D16_WAVES, SYRK_D16_RING>; break;
+        default: kern = ssyrk_direct16_kernel<MB, NB, SYRK_FOLDED, SYRK_D16_WAVES, SYRK_D16_RING>; break;
+    }
+    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+        return T2SP_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3((unsigned)p.needed), dim3(SYRK_D16_WAVES * 64), smem, stream, g, p.rows_per_tile,
+                       p.tiles_m);
+    return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+}
+
+static int launch_syrk_d16(const SyrkArgs &g, hipStream_t stream) {
+    const SyrkD16Plan p = plan_syrk_d16(g.N);
+#define T2SP_D16_CASE(MBV, NBV) if (p.mb == MBV && p.nb == NBV) return launch_syrk_d16_t<MBV, NBV>(g, p, stream);
+    T2SP_D16_CASE(2, 2) T2SP_D16_CASE(3, 2) T2SP_D16_CASE(4, 2) T2SP_D16_CASE(5, 2) T2SP_D16_CASE(6, 2)
+    T2SP_D16_CASE(7, 2) T2SP_D16_CASE(8, 2) T2SP_D16_CASE(2, 3) T2SP_D16_CASE(3, 3) T2SP_D16_CASE(4, 3)
+    T2SP_D16_CASE(5, 3) T2SP_D16_CASE(6, 3) T2SP_D16_CASE(7, 3) T2SP_D16_CASE(8, 3) T2SP_D16_CASE(2, 4)
+    T2SP_D16_CASE(3, 4) T2SP_D16_CASE(4, 4) T2SP_D16_CASE(5, 4) T2SP_D16_CASE(6, 4)
+#undef T2SP_D16_CASE
+    return T2SP_ERR_SHAPE;
+}
+
+constexpr int SYRK_D16_MAX_N = 5120;   // measured: from about 6144 on the LDS tiles' operand reuse wins
+
+static bool syrk_d16_ok(const SyrkArgs &g) {
+    return g.K % 16 == 0 && g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && (int64_t)g.N * g.lda < (1 << 30);
+}
+
 // Shapes the vector loaders cannot take: one thread per element on or above the diagonal.
 template <int MODE>
 __global__ void ssyrk_scalar_kernel(const SyrkArgs g) {
@@ -210,6 +398,8 @@ static int dispatch_syrk(SyrkArgs g, int trans, int cfg, float *workspace, size_
         g.A = workspace;
         g.lda = g.K;
     }
+    if (cfg == T2SP_CFG_DIRECT16) return syrk_d16_ok(g) ? launch_syrk_d16(g, stream) : T2SP_ERR_SHAPE;
+    if (cfg == T2SP_CFG_AUTO && g.N <= SYRK_D16_MAX_N && g.K >= 64 && syrk_d16_ok(g)) return launch_syrk_d16(g, stream);
     const bool out_ok = g.mode == SYRK_FOLDED ||
                         (g.ldc % 4 == 0 && (uintptr_t)g.C % 16 == 0 &&
                          (!g.Cin || (g.ldcin % 4 == 0 && (uintptr_t)g.Cin % 16 == 0)));
