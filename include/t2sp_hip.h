@@ -103,6 +103,32 @@ int t2sp_sger_f32(const float *A, const float *x, const float *y, float *O, int 
 int t2sp_sger_f32_tiled(const float *A, const float *x, const float *y, float *O, int I, int K, int64_t lda,
                         int kkk, int iii, int ii, int kk, const int64_t *strides6, void *stream);
 
+/* Out[i] = alpha * sum_{k<K} A[i,k] * x[i+k] + beta * y[i], fp32: the band matrix-vector product in
+ * the reference's row-packed band form (A row-major I x K holds the diagonals of row i, x spans
+ * I + K - 1 elements, t2s/tests/performance/gbmv3/gbmv3-run-fpga.cpp:69-77).  O is flat, or the
+ * reference's 3-D Out(iii, ii, i) with element strides strides3 (gbmv3.cpp:88).  HBM-bound (4 bytes
+ * and 2 flop per element of A).  Replaces the device side of the reference's GBMV pipeline
+ * (t2s/tests/performance/gbmv3/gbmv3.cpp:55-63). */
+int t2sp_sgbmv3_f32(float alpha, float beta, const float *A, const float *x, const float *y, float *O, int I,
+                    int K, int64_t lda, void *stream);
+int t2sp_sgbmv3_f32_tiled(float alpha, float beta, const float *A, const float *x, const float *y, float *O,
+                          int I, int K, int64_t lda, int iii, int ii, const int64_t *strides3, void *stream);
+
+/* Out = alpha * S * x + beta * y, fp32, S the symmetric N x N matrix whose triangle col <= row is
+ * stored in row-major A (elements above the diagonal are never read).  O is flat, or the
+ * reference's 3-D Out(kkk, kk, k) with element strides strides3
+ * (t2s/tests/performance/symv/symv-run-fpga.cpp:79).  HBM-bound: the triangle is read once.  With
+ * N % 4 == 0, lda % 4 == 0, 16-byte aligned A and x and a workspace of
+ * t2sp_ssymv_workspace_bytes(N) it runs on 128 x 128 blocks; otherwise (workspace may be NULL) a
+ * slow kernel without requirements.  Replaces the device side of the reference's SYMV pipeline
+ * (t2s/tests/performance/symv/symv.cpp:57-72). */
+size_t t2sp_ssymv_workspace_bytes(int N);
+int t2sp_ssymv_f32(float alpha, float beta, const float *A, const float *x, const float *y, float *O, int N,
+                   int64_t lda, float *workspace, size_t workspace_bytes, void *stream);
+int t2sp_ssymv_f32_tiled(float alpha, float beta, const float *A, const float *x, const float *y, float *O, int N,
+                         int64_t lda, int kkk, int kk, const int64_t *strides3, float *workspace,
+                         size_t workspace_bytes, void *stream);
+
 /* O[n,co,h,w] = sum_{ci,kh,kw} I[n,ci,h+kh,w+kw] * W[co,ci,kh,kw], stride 1, valid
  * padding, fp32.  si4/sw4/so4 are element strides of the logical indices
  * (n,ci,h,w), (co,ci,kh,kw), (n,co,h,w); "w" is the innermost spatial axis (the

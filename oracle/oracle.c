@@ -24,6 +24,18 @@
  *                                 output layout (syrk.cpp:37-46) is restated in oracle.py.
  *   oracle_ger       golden       t2s/tests/performance/ger/ger-run-fpga.cpp:71
  *                                 (golden = a + x * y, product and sum rounded separately).
+ *   oracle_gbmv3     URE order    t2s/tests/performance/gbmv3/gbmv3.cpp:55-63 (uZ over ascending
+ *                                 total_k of A(total_k, total_i) * X(total_i + total_k), then
+ *                                 Out = V*Alpha + Y*Beta); the driver's golden loop over the dense
+ *                                 band (gbmv3-run-fpga.cpp:108-114) visits the same terms in the
+ *                                 same order.
+ *   oracle_symv      golden       t2s/tests/performance/symv/symv-run-fpga.cpp:86-96 (ascending k over
+ *                                 the full symmetric matrix, then alpha*golden + beta*y); reads only
+ *                                 the triangle col <= row, the one the pipeline keeps (symv.cpp:65).
+ *                                 The pipeline's own UREs (symv.cpp:57-72) fix I = II = 4 by macro
+ *                                 and, past one block of II rows, add the elements above the
+ *                                 diagonal on top of the finished row sum; the driver never asserts
+ *                                 on them (symv-run-fpga.cpp:97-98), so the golden loop is the oracle.
  *   oracle_mttkrp    golden       t2s/tests/performance/util/util.h:498-515 (two-step: TTM over l
  *                                 into e(i,j,k), then d += e*b over k).  The reference's outer loop
  *                                 bound `i < K` (util.h:502) is only right when I == K; this
@@ -401,6 +413,50 @@ void oracle_ger(const float *A, const float *x, const float *y, float *O, int64_
             const float p = x[i] * y[k];
             O[i * K + k] = A[i * K + k] + p;
         }
+}
+
+/* Out[i] = alpha * sum_k A[i,k]*x[i+k] + beta*y[i] (gbmv3.cpp:55-63); A row-major I x K, leading
+ * dimension lda; x spans I + K - 1 elements. */
+void oracle_gbmv3(float alpha, float beta, const float *A, const float *x, const float *y, float *O, int64_t I,
+                  int64_t K, int64_t lda, int acc, int threads) {
+    set_threads(threads);
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < I; i++) {
+        if (acc == ORACLE_ACC_F64) {
+            double z = 0.0;
+            for (int64_t k = 0; k < K; k++) z += (double)A[i * lda + k] * (double)x[i + k];
+            O[i] = (float)(z * (double)alpha + (double)y[i] * (double)beta);
+        } else {
+            float z = 0.f;
+            for (int64_t k = 0; k < K; k++)
+                z = acc == ORACLE_ACC_F32_FMA ? fmaf(A[i * lda + k], x[i + k], z) : z + A[i * lda + k] * x[i + k];
+            const float t = z * alpha, u = y[i] * beta;
+            O[i] = t + u;
+        }
+    }
+}
+
+/* Out[i] = alpha * sum_k S[i,k]*x[k] + beta*y[i], S[i,k] = A[max(i,k)][min(i,k)]
+ * (symv-run-fpga.cpp:86-96); A row-major N x N, leading dimension lda. */
+void oracle_symv(float alpha, float beta, const float *A, const float *x, const float *y, float *O, int64_t N,
+                 int64_t lda, int acc, int threads) {
+    set_threads(threads);
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < N; i++) {
+        if (acc == ORACLE_ACC_F64) {
+            double z = 0.0;
+            for (int64_t k = 0; k < N; k++) z += (double)(k <= i ? A[i * lda + k] : A[k * lda + i]) * (double)x[k];
+            O[i] = (float)((double)alpha * z + (double)beta * (double)y[i]);
+        } else {
+            float z = 0.f;
+            for (int64_t k = 0; k < N; k++) {
+                const float a = k <= i ? A[i * lda + k] : A[k * lda + i];
+                z = acc == ORACLE_ACC_F32_FMA ? fmaf(a, x[k], z) : z + a * x[k];
+            }
+            const float t = alpha * z, u = beta * y[i];
+            O[i] = t + u;
+        }
+    }
 }
 
 int oracle_max_threads(void) { return omp_get_max_threads(); }

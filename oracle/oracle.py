@@ -48,6 +48,11 @@ def lib():
         _lib.oracle_syrk.restype = None
         _lib.oracle_ger.argtypes = [fp, fp, fp, fp, i64, i64, ctypes.c_int]
         _lib.oracle_ger.restype = None
+        f32 = ctypes.c_float
+        _lib.oracle_gbmv3.argtypes = [f32, f32, fp, fp, fp, fp, i64, i64, i64, ctypes.c_int, ctypes.c_int]
+        _lib.oracle_gbmv3.restype = None
+        _lib.oracle_symv.argtypes = [f32, f32, fp, fp, fp, fp, i64, i64, ctypes.c_int, ctypes.c_int]
+        _lib.oracle_symv.restype = None
         _lib.oracle_max_threads.restype = ctypes.c_int
         for f in (_lib.oracle_fill_uniform, _lib.oracle_gemm, _lib.oracle_gemm_literal,
                   _lib.oracle_conv, _lib.oracle_capsule, _lib.oracle_mttkrp,
@@ -276,6 +281,40 @@ def ger_tile(O, III, II, KKK, KK):
     TI, TK = O.shape
     I, K = TI // (III * II), TK // (KKK * KK)
     return np.ascontiguousarray(O.reshape(I, II, III, K, KK, KKK).transpose(0, 3, 4, 1, 2, 5))
+
+
+def gbmv3(A, x, y, alpha=1.0, beta=1.0, acc=ACC_F32, threads=0):
+    """alpha * sum_k A[i,k]*x[i+k] + beta*y[i] in ascending k (gbmv3.cpp:55-63).  A: (I, K) band rows,
+    x: at least I + K - 1 elements."""
+    A, x, y = np.ascontiguousarray(A), np.ascontiguousarray(x), np.ascontiguousarray(y)
+    I, K = A.shape
+    assert x.shape[0] >= I + K - 1 and y.shape[0] >= I
+    O = np.empty(I, dtype=np.float32)
+    lib().oracle_gbmv3(alpha, beta, _p(A), _p(x), _p(y), _p(O), I, K, K, acc, threads)
+    return O
+
+
+def gbmv3_pack(a, kl, ku, k_pad):
+    """The band rows the driver hands to the pipeline (gbmv3-run-fpga.cpp:69-77): row i of the
+    result holds a[i, j] at column kl - i + j for the j inside the band, zero elsewhere; k_pad >=
+    kl + 1 + ku is the padded row length (TOTAL_K)."""
+    TI, TJ = a.shape
+    band = np.zeros((TI, k_pad), dtype=np.float32)
+    for i in range(TI):
+        for j in range(max(0, i - kl), min(TJ, i + ku + 1)):
+            band[i, kl - i + j] = a[i, j]
+    return band
+
+
+def symv(A, x, y, alpha=1.0, beta=1.0, acc=ACC_F32, threads=0):
+    """alpha * S x + beta * y with S[i,k] = A[max(i,k), min(i,k)], ascending k
+    (symv-run-fpga.cpp:86-96); elements of A above the diagonal are not read."""
+    A, x, y = np.ascontiguousarray(A), np.ascontiguousarray(x), np.ascontiguousarray(y)
+    N = A.shape[0]
+    assert A.shape == (N, N) and x.shape[0] >= N and y.shape[0] >= N
+    O = np.empty(N, dtype=np.float32)
+    lib().oracle_symv(alpha, beta, _p(A), _p(x), _p(y), _p(O), N, N, acc, threads)
+    return O
 
 
 def max_threads():

@@ -65,6 +65,17 @@ def _declare(L):
     L.ger_ns.restype = ctypes.c_double
     L.t2sp_sger_f32.argtypes = [vp, vp, vp, vp, i32, i32, i64, i64, vp]
     L.t2sp_sger_f32_tiled.argtypes = [vp, vp, vp, vp, i32, i32, i64, i32, i32, i32, i32, ctypes.POINTER(i64), vp]
+    for name in ("gbmv3", "symv"):
+        getattr(L, name).argtypes = [f32, f32, bp, bp, bp, bp]
+        getattr(L, name + "_ns").argtypes = [f32, f32, bp, bp, bp, bp]
+        getattr(L, name + "_ns").restype = ctypes.c_double
+    L.t2sp_sgbmv3_f32.argtypes = [f32, f32, vp, vp, vp, vp, i32, i32, i64, vp]
+    L.t2sp_sgbmv3_f32_tiled.argtypes = [f32, f32, vp, vp, vp, vp, i32, i32, i64, i32, i32, ctypes.POINTER(i64), vp]
+    L.t2sp_ssymv_workspace_bytes.argtypes = [i32]
+    L.t2sp_ssymv_workspace_bytes.restype = ctypes.c_size_t
+    L.t2sp_ssymv_f32.argtypes = [f32, f32, vp, vp, vp, vp, i32, i64, vp, ctypes.c_size_t, vp]
+    L.t2sp_ssymv_f32_tiled.argtypes = [f32, f32, vp, vp, vp, vp, i32, i64, i32, i32, ctypes.POINTER(i64), vp,
+                                       ctypes.c_size_t, vp]
     L.conv.argtypes = [bp, bp, bp]
     L.t2sp_conv_with_cfg.argtypes = [bp, bp, bp, i32]
     p64, p32 = ctypes.POINTER(i64), ctypes.POINTER(i32)

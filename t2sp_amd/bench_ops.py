@@ -147,6 +147,53 @@ def sger_8192(torch, steps, warmup, peak):
                   **{"bound": "hbm", "GB/s": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / 8000.0, 4)})
 
 
+def sgbmv3_case(torch, steps, warmup, peak):
+    """Not a BASELINE configuration: the GBMV pipeline (t2s/tests/performance/gbmv3) with the band
+    width of gbmv3-run-fpga.cpp:29-30 (Ku = Kl = 511, rows padded to 1024) and 131072 rows, so that
+    the band (512 MiB) does not fit the caches.  4 bytes of A per 2 flop: the roof is HBM."""
+    L = lib()
+    I, K = 131072, 1024
+    A = ops.fill_uniform(torch.empty(I, K, device="cuda"), 1)
+    x = ops.fill_uniform(torch.empty(I + K - 1, device="cuda"), 2)
+    y = ops.fill_uniform(torch.empty(I, device="cuda"), 3)
+    O = torch.empty(I, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        rc = L.t2sp_sgbmv3_f32(1.5, 0.5, A.data_ptr(), x.data_ptr(), y.data_ptr(), O.data_ptr(), I, K, K, s)
+        assert rc == 0, rc
+
+    ms = _time(torch, launch, steps, warmup)
+    nbytes = 4.0 * I * K + 4.0 * (I + K - 1) + 8.0 * I
+    return _entry(2.0 * I * K / ms / 1e9, peak, ms, workload="131072 band rows of 1024, flat output",
+                  **{"bound": "hbm", "GB/s": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / 8000.0, 4)})
+
+
+def ssymv_case(torch, steps, warmup, peak):
+    """Not a BASELINE configuration: the SYMV pipeline (t2s/tests/performance/symv) on a 16384 x 16384
+    matrix.  Only the triangle col <= row is read (N*(N+1)/2 elements, 4 flop each): the roof is HBM."""
+    L = lib()
+    N = 16384
+    A = ops.fill_uniform(torch.empty(N, N, device="cuda"), 1)
+    x = ops.fill_uniform(torch.empty(N, device="cuda"), 2)
+    y = ops.fill_uniform(torch.empty(N, device="cuda"), 3)
+    O = torch.empty(N, device="cuda")
+    nbytes_ws = L.t2sp_ssymv_workspace_bytes(N)
+    ws = torch.empty(nbytes_ws // 4, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        rc = L.t2sp_ssymv_f32(1.5, 0.5, A.data_ptr(), x.data_ptr(), y.data_ptr(), O.data_ptr(), N, N, ws.data_ptr(),
+                              nbytes_ws, s)
+        assert rc == 0, rc
+
+    ms = _time(torch, launch, steps, warmup)
+    nbytes = 2.0 * N * (N + 1) + 12.0 * N
+    return _entry(2.0 * N * N / ms / 1e9, peak, ms, workload="N=16384, flat output",
+                  note="includes the kernel that adds the partial vectors",
+                  **{"bound": "hbm", "GB/s": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / 8000.0, 4)})
+
+
 def run_all(torch, steps, warmup, peak, capsule_cfg=0, capsule_splits=0):
     return {"conv2d": conv_config3(torch, steps, warmup, peak),
             "capsule": capsule_config4(torch, steps, warmup, peak, capsule_cfg, capsule_splits),
@@ -154,4 +201,6 @@ def run_all(torch, steps, warmup, peak, capsule_cfg=0, capsule_splits=0):
             "ssyrk_8192": ssyrk_case(torch, steps, warmup, peak, 8192, 8192, ""),
             "ssyrk_768x1024": ssyrk_case(torch, max(steps, 200), max(warmup, 20), peak, 768, 1024,
                                          " (the size of peppers/blas/level3/syrk/release/s10)"),
-            "sger_8192": sger_8192(torch, steps, warmup, peak)}
+            "sger_8192": sger_8192(torch, steps, warmup, peak),
+            "sgbmv3_131072x1024": sgbmv3_case(torch, steps, warmup, peak),
+            "ssymv_16384": ssymv_case(torch, steps, warmup, peak)}

@@ -1,0 +1,102 @@
+// gbmv.hip — SGBMV in the reference's "gbmv3" band form:
+//     Out[i] = Alpha * sum_{k < K} A[i,k] * X[i + k]  +  Beta * Y[i]
+//
+// Replaces the device pipeline of t2s/tests/performance/gbmv3/gbmv3.cpp:55-63 (uA = A(total_k,
+// total_i), uX = X(total_i + total_k), uZ the running sum over total_k, Out = V*Alpha + Y*Beta).
+// A is the band matrix stored by rows: row i holds its Kl + 1 + Ku diagonals, padded to K
+// (gbmv3-run-fpga.cpp:69-77), so the matching X entry slides by one per row.  X therefore spans
+// rows + K - 1 elements.  The output is a vector; the reference shapes it (III, II, I) with
+// total_i = iii + III*ii + III*II*i (gbmv3.cpp:38,88), which is the flat row index when dense.
+//
+// 2 flop per 4 bytes of A: the roofline is HBM.  One wave owns one row: each lane takes four
+// consecutive k per step with a 128-bit load of A (consecutive lanes, consecutive 16 bytes) and
+// a 4-byte-aligned 128-bit load of X (cache-resident: neighbouring rows read nearly the same
+// window).  Partial sums are combined in a fixed order (the four vector slots, then a butterfly
+// over the 64 lanes), so results do not depend on the launch.
+#include <hip/hip_runtime.h>
+#include "t2sp_hip.h"
+
+namespace t2sp {
+
+typedef float gbmv_v4f __attribute__((ext_vector_type(4)));
+typedef float gbmv_v4f_u __attribute__((ext_vector_type(4), aligned(4)));
+
+constexpr int GBMV_ROWS_PER_WG = 4;      // one wave per row
+
+struct GbmvArgs {
+    const float *A, *x, *y;
+    float *O;
+    int I, K;
+    int64_t lda;
+    float alpha, beta;
+    int t_iii, t_ii;                     // output tile extents (III, II); the rest is i
+    int64_t s[3];                        // element strides of Out(iii, ii, i)
+};
+
+__device__ __forceinline__ float gbmv_wave_sum(float v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+    return v;
+}
+
+template <bool VEC>
+__global__ void __launch_bounds__(64 * GBMV_ROWS_PER_WG) sgbmv3_kernel(const GbmvArgs g) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    for (int64_t i = (int64_t)blockIdx.x * GBMV_ROWS_PER_WG + wave; i < g.I; i += (int64_t)gridDim.x * GBMV_ROWS_PER_WG) {
+        const float *a = g.A + i * g.lda;
+        const float *x = g.x + i;
+        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+        if (VEC) {
+#pragma unroll 4
+            for (int k = lane * 4; k < g.K; k += 256) {
+                const gbmv_v4f av = *reinterpret_cast<const gbmv_v4f *>(a + k);
+                const gbmv_v4f_u xv = *reinterpret_cast<const gbmv_v4f_u *>(x + k);
+                s0 += av[0] * xv[0];
+                s1 += av[1] * xv[1];
+                s2 += av[2] * xv[2];
+                s3 += av[3] * xv[3];
+            }
+        } else {
+            for (int k = lane; k < g.K; k += 64) s0 += a[k] * x[k];
+        }
+        const float z = gbmv_wave_sum((s0 + s1) + (s2 + s3));
+        if (lane == 0) {
+            const int iii = (int)(i % g.t_iii);
+            const int64_t q = i / g.t_iii;
+            const int64_t off = iii * g.s[0] + (q % g.t_ii) * g.s[1] + (q / g.t_ii) * g.s[2];
+            g.O[off] = z * g.alpha + g.y[i] * g.beta;
+        }
+    }
+}
+
+static int launch_gbmv(const GbmvArgs &g, hipStream_t stream) {
+    if (g.I <= 0 || g.K <= 0 || g.t_iii <= 0 || g.t_ii <= 0) return T2SP_ERR_SHAPE;
+    const bool vec = g.K % 4 == 0 && g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.x % 4 == 0);
+    int64_t blocks = ((int64_t)g.I + GBMV_ROWS_PER_WG - 1) / GBMV_ROWS_PER_WG;
+    if (blocks > 256 * 32) blocks = 256 * 32;            // grid-stride beyond 32 workgroups per CU
+    auto kern = vec ? sgbmv3_kernel<true> : sgbmv3_kernel<false>;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(64 * GBMV_ROWS_PER_WG), 0, stream, g);
+    return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+}
+
+}  // namespace t2sp
+
+extern "C" int t2sp_sgbmv3_f32(float alpha, float beta, const float *A, const float *x, const float *y, float *O,
+                               int I, int K, int64_t lda, void *stream) {
+    t2sp::GbmvArgs g{};
+    g.A = A; g.x = x; g.y = y; g.O = O; g.I = I; g.K = K; g.lda = lda; g.alpha = alpha; g.beta = beta;
+    g.t_iii = I > 0 ? I : 1; g.t_ii = 1; g.s[0] = 1; g.s[1] = 0; g.s[2] = 0;
+    return t2sp::launch_gbmv(g, (hipStream_t)stream);
+}
+
+extern "C" int t2sp_sgbmv3_f32_tiled(float alpha, float beta, const float *A, const float *x, const float *y,
+                                     float *O, int I, int K, int64_t lda, int iii, int ii,
+                                     const int64_t *strides3, void *stream) {
+    if (iii <= 0 || ii <= 0 || !strides3) return T2SP_ERR_SHAPE;
+    t2sp::GbmvArgs g{};
+    g.A = A; g.x = x; g.y = y; g.O = O; g.I = I; g.K = K; g.lda = lda; g.alpha = alpha; g.beta = beta;
+    g.t_iii = iii; g.t_ii = ii;
+    for (int d = 0; d < 3; d++) g.s[d] = strides3[d];
+    return t2sp::launch_gbmv(g, (hipStream_t)stream);
+}

@@ -121,6 +121,41 @@ def ger(A, x, y, out=None, tiles=None):
     return out
 
 
+def _vector_out(like, n, tiles):
+    if tiles is None:
+        return _empty_like_kind(like, (n,))
+    inner, mid = tiles
+    assert n % (inner * mid) == 0
+    return _empty_like_kind(like, (n // (inner * mid), mid, inner))
+
+
+def gbmv3(A, x, y, alpha=1.0, beta=1.0, out=None, tiles=None):
+    """Out[i] = alpha * sum_k A[i,k] * x[i+k] + beta * y[i] through the `gbmv3` entry point
+    (include/gbmv3-interface.h).
+
+    A: (I, K), the band matrix packed by rows; x: at least I + K - 1 elements; y: (I,).  With
+    tiles=(III, II) the result has the reference's shape Out(III, II, I), numpy (I, II, III)
+    (t2s/tests/performance/gbmv3/gbmv3-run-fpga.cpp:98); otherwise a flat vector."""
+    if out is None:
+        out = _vector_out(A, A.shape[0], tiles)
+    a, xb, yb, o = (HalideBuffer.wrap(t) for t in (A, x, y, out))
+    _check("gbmv3", lib().gbmv3(float(alpha), float(beta), a.ref, xb.ref, yb.ref, o.ref))
+    return out
+
+
+def symv(A, x, y, alpha=1.0, beta=1.0, out=None, tiles=None):
+    """Out = alpha * S x + beta * y through the `symv` entry point (include/symv-interface.h), S the
+    symmetric matrix whose triangle col <= row is stored in the row-major (N, N) array A.
+
+    With tiles=(KKK, KK) the result has the reference's shape Out(KKK, KK, K), numpy (K, KK, KKK)
+    (t2s/tests/performance/symv/symv-run-fpga.cpp:79); otherwise a flat vector."""
+    if out is None:
+        out = _vector_out(A, A.shape[0], tiles)
+    a, xb, yb, o = (HalideBuffer.wrap(t) for t in (A, x, y, out))
+    _check("symv", lib().symv(float(alpha), float(beta), a.ref, xb.ref, yb.ref, o.ref))
+    return out
+
+
 def conv(I, W, out=None, cfg=0):
     """O = conv2d(I, W), stride 1, no padding, through the `conv` entry point
     (include/conv-interface.h).

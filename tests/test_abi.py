@@ -116,6 +116,14 @@ def test_other_entries_reject_bad_arguments_without_a_device():
     assert L.mttkrp(b.ref, _buf((7, 9)).ref, d.ref, a.ref) == -8
     assert L.mttkrp(b.ref, _buf((7, 4)).ref, d.ref, a.ref) == -4
     assert L.mttkrp(_buf((6, 8)).ref, c.ref, d.ref, a.ref) == -43
+    am, v23, v8 = _buf((8, 16)), _buf((23,)), _buf((8,))
+    assert L.gbmv3(1.0, 1.0, None, v23.ref, v8.ref, v8.ref) == -12
+    assert L.gbmv3(1.0, 1.0, am.ref, _buf((22,)).ref, v8.ref, v8.ref) == -4      # x spans I + K - 1
+    assert L.gbmv3(1.0, 1.0, am.ref, v23.ref, v8.ref, _buf((2, 8)).ref) == -43
+    sq = _buf((8, 8))
+    assert L.symv(1.0, 1.0, sq.ref, v8.ref, v8.ref, None) == -12
+    assert L.symv(1.0, 1.0, am.ref, v8.ref, v8.ref, v8.ref) == -8                # A not square
+    assert L.symv(1.0, 1.0, sq.ref, _buf((7,)).ref, v8.ref, v8.ref) == -4
 
 
 def test_thin_layer_rejects_bad_shapes():
@@ -128,6 +136,9 @@ def test_thin_layer_rejects_bad_shapes():
     assert L.t2sp_mttkrp_f32(None, None, None, None, 0, 4, 4, 4, None, None, None, None, 0, 0, None, 0, None) == -8
     assert L.t2sp_capsule_f32(None, None, None, None, None, None, None, 0, 0, None, 0, None) == -8
     assert L.t2sp_relayout_f32(None, None, 11, None, None, None, None) == -8
+    assert L.t2sp_sgbmv3_f32(1.0, 1.0, None, None, None, None, 0, 4, 4, None) == -8
+    assert L.t2sp_ssymv_f32(1.0, 1.0, None, None, None, None, 0, 4, None, 0, None) == -8
+    assert L.t2sp_ssymv_workspace_bytes(1000) == 8 * 8 * 128 * 4
     assert L.t2sp_mttkrp_workspace_bytes(512, 512, 512, 256, 1, 128) == 128 * 512 * 256 * 4
 
 

@@ -388,6 +388,84 @@ def test_ger_matches_separately_rounded_numpy_and_tiled_addresses():
                             assert Ot[i, k, kk, ii, iii, kkk] == got[ti, tk]
 
 
+# ---------------------------------------------------------------------------------------------
+# GBMV3 and SYMV
+def test_gbmv3_equals_dense_band_product_and_driver_fixture():
+    """The row-packed band form times the sliding x equals the dense band matrix times x
+    (gbmv3-run-fpga.cpp:55-77 builds one from the other), exactly for integers; the driver's own
+    index-valued fixture (a = i*TOTAL_J + j, x = j, y = i, gbmv3-run-fpga.cpp:57-67) with its golden
+    loop (:108-114)."""
+    TI = TJ = 24
+    kl, ku, kpad = 3, 5, 12
+    a = ints((TI, TJ), -4, 5, 80)
+    dense = np.zeros_like(a)
+    for i in range(TI):
+        for j in range(TJ):
+            if -kl <= j - i <= ku:
+                dense[i, j] = a[i, j]
+    band = o.gbmv3_pack(a, kl, ku, kpad)
+    xs, y = ints((TJ,), -4, 5, 81), ints((TI,), -4, 5, 82)
+    x = np.zeros(TI + kpad - 1, np.float32)
+    x[kl:kl + TJ] = xs                                  # the pipeline reads x[i + (kl - i + j)] = x[kl + j]
+    want = 2.0 * (dense.astype(np.float64) @ xs) - 3.0 * y
+    for acc in (o.ACC_F32, o.ACC_F32_FMA, o.ACC_F64):
+        assert (o.gbmv3(band, x, y, 2.0, -3.0, acc=acc) == want).all()
+    # a shifted x must change the answer (pins the i + k index)
+    assert not (o.gbmv3(band, np.roll(x, 1), y, 2.0, -3.0) == want).all()
+    # driver fixture, TINY constants: TOTAL_I = TOTAL_J = 8, Ku = Kl = 2, TOTAL_K = 8
+    T, K2 = 8, 2
+    a = np.zeros((T, T), np.float32)
+    for i in range(T):
+        for j in range(T):
+            if abs(j - i) <= K2:
+                a[i, j] = i * T + j
+    band = o.gbmv3_pack(a, K2, K2, 8)
+    x = np.zeros(T + 8 - 1, np.float32)
+    x[K2:K2 + T] = np.arange(T)
+    y = np.arange(T, dtype=np.float32)
+    golden = np.array([sum(a[i, j] * j for j in range(T) if abs(j - i) <= K2) * 1.0 + y[i] * 1.0 for i in range(T)])
+    assert (o.gbmv3(band, x, y, 1.0, 1.0) == golden).all()
+    # uniform data: float32 ascending-k sum restated in numpy
+    A, xr, yr = o.fill_uniform((5, 16), 83), o.fill_uniform((20,), 84), o.fill_uniform((5,), 85)
+    ref = np.empty(5, np.float32)
+    for i in range(5):
+        z = np.float32(0)
+        for k in range(16):
+            z = np.float32(z + np.float32(A[i, k] * xr[i + k]))
+        ref[i] = np.float32(np.float32(z * np.float32(0.5)) + np.float32(yr[i] * np.float32(1.5)))
+    assert (o.gbmv3(A, xr, yr, 0.5, 1.5) == ref).all()
+
+
+def test_symv_reads_one_triangle_and_equals_full_symmetric_product():
+    """Integer data: the result equals numpy's product with the symmetrised matrix in any
+    arithmetic; NaN above the diagonal must not reach the output (only col <= row is input);
+    a transposed read (col >= row) must fail the check."""
+    N = 37
+    L = np.tril(ints((N, N), -5, 6, 86))
+    S = L + np.tril(L, -1).T
+    x, y = ints((N,), -5, 6, 87), ints((N,), -5, 6, 88)
+    want = 3.0 * (S.astype(np.float64) @ x) + 2.0 * y
+    A = L.copy()
+    A[np.triu_indices(N, 1)] = np.nan
+    for acc in (o.ACC_F32, o.ACC_F32_FMA, o.ACC_F64):
+        assert (o.symv(A, x, y, 3.0, 2.0, acc=acc) == want).all()
+    U = np.ascontiguousarray(L.T)                      # same triangle stored on the other side
+    got_u = o.symv(U, x, y, 3.0, 2.0)
+    assert not (got_u == want).all()
+    # uniform data against the driver's golden loop restated with float32 numpy scalars
+    N = 9
+    Af = np.tril(o.fill_uniform((N, N), 89))
+    Sf = Af + np.tril(Af, -1).T
+    xf, yf = o.fill_uniform((N,), 90), o.fill_uniform((N,), 91)
+    ref = np.empty(N, np.float32)
+    for i in range(N):
+        g = np.float32(0)
+        for k in range(N):
+            g = np.float32(g + np.float32(Sf[i, k] * xf[k]))
+        ref[i] = np.float32(np.float32(np.float32(0.75) * g) + np.float32(np.float32(1.25) * yf[i]))
+    assert (o.symv(Af, xf, yf, 0.75, 1.25) == ref).all()
+
+
 def test_gemm_ure_loop_nest_equals_golden_loop_bit_for_bit():
     """The spec's serial loop nest (gemm.cpp:30,57-71) sums every output in ascending total_k, like the
     golden loop: same bits, for the GPU and the TINY constant sets."""
