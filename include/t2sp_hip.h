@@ -71,7 +71,10 @@ int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, float alpha, 
                       size_t workspace_bytes, void *stream);
 
 /* D = alpha * A * A^T + beta * Cin, fp32, A row-major N x K (K x N when trans is non-zero: it is
- * then first re-laid into `workspace`, t2sp_ssyrk_workspace_bytes).  Only tiles on or above the
+ * then first re-laid into `workspace`, which the transposed form requires).  For large N the
+ * workspace (t2sp_ssyrk_workspace_bytes; optional when trans is zero) also holds partial planes
+ * that let the last, partial round of 256 tiles split its reduction over all CUs (N = 8192: two
+ * full rounds + 16 tiles).  Only tiles on or above the
  * diagonal are multiplied.  Flat form: C row-major N x N; `upper` selects the triangle of BLAS
  * semantics; mirror = 0 writes that triangle only, 1 writes both triangles with Cin read from the
  * `upper` triangle (a symmetric result, what the reference's ssyrk wrapper returns,

@@ -113,10 +113,13 @@ def ssyrk_case(torch, steps, warmup, peak, N, K, note):
     A = ops.fill_uniform(torch.empty(N, K, device="cuda"), 1)
     C = ops.fill_uniform(torch.empty(N, N, device="cuda"), 2)
     O = torch.empty(N, N, device="cuda")
+    nbytes = L.t2sp_ssyrk_workspace_bytes(0, N, K)
+    ws = torch.empty(max(nbytes // 4, 1), device="cuda")
     s = torch.cuda.current_stream().cuda_stream
 
     def launch():
-        rc = L.t2sp_ssyrk_f32(1, 0, N, K, 1.5, A.data_ptr(), K, 0.5, C.data_ptr(), N, O.data_ptr(), N, 1, 0, None, 0, s)
+        rc = L.t2sp_ssyrk_f32(1, 0, N, K, 1.5, A.data_ptr(), K, 0.5, C.data_ptr(), N, O.data_ptr(), N, 1, 0,
+                              ws.data_ptr(), nbytes, s)
         assert rc == 0, rc
 
     ms = _time(torch, launch, steps, warmup)

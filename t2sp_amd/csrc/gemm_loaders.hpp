@@ -105,12 +105,13 @@ struct RowMajorKcLoaderB {
     bool row_ok[Cfg::B_VEC];
     v4f reg[2][Cfg::B_VEC];
     int k0, K;
-    __device__ RowMajorKcLoaderB(const float *B, int64_t ldb, int n0, int N, int K_) : safe(B), k0(0), K(K_) {
+    __device__ RowMajorKcLoaderB(const float *B, int64_t ldb, int n0, int N, int K_, int k_begin = 0)
+        : safe(B), k0(k_begin), K(K_) {
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
             row_ok[i] = !EDGE || (n0 + s.row < N);
-            p[i] = B + (int64_t)(n0 + (row_ok[i] ? s.row : 0)) * ldb + s.k;
+            p[i] = B + (int64_t)(n0 + (row_ok[i] ? s.row : 0)) * ldb + k_begin + s.k;
         }
     }
     template <int S>

@@ -16,6 +16,7 @@
 //     computes them.
 #include "mfma_core.hpp"
 #include "gemm_loaders.hpp"
+#include "splitk.hpp"
 #include "t2sp_hip.h"
 
 namespace t2sp {
@@ -36,6 +37,11 @@ struct SyrkArgs {
     int f_iii, f_ii, f_blocks;
     int64_t s[6];
     int tiles;            // tiles per side
+    // a launch covers `tile_count` tiles of the triangle's walking order starting at `tile_first`;
+    // with splits > 1 every tile goes to `splits` workgroups, each reducing a slice of k into its
+    // own plane of `scratch` (plane = tile_count tiles side by side, [tile][col][row])
+    int tile_first, tile_count, splits;
+    float *scratch;
 };
 
 // MODE FLAT_SYM reads Cin from the `upper` triangle only; the other modes where C is written.
@@ -87,15 +93,11 @@ __device__ __forceinline__ void syrk_store(const SyrkArgs &g, int r, int c, floa
     }
 }
 
-// Workgroup id -> tile (tm, tn), tn >= tm, of the T x T upper triangle.  Ids are dealt round-robin
-// to the 8 XCDs, so each XCD is first given one contiguous run of the order below; that order
-// walks the triangle in bands of 4 tile-rows, column by column inside a band, so the workgroups
-// resident on one XCD at a time share a few row panels and column panels of A in its L2.
-__device__ __forceinline__ void syrk_tile(int bid, int T, int &tm, int &tn) {
-    const int total = T * (T + 1) / 2;
-    constexpr int NXCD = 8, BAND = 4;
-    int pid = bid;
-    if (total % NXCD == 0) pid = (bid % NXCD) * (total / NXCD) + bid / NXCD;
+// Position `pid` of the walking order -> tile (tm, tn), tn >= tm, of the T x T upper triangle.
+// The order walks the triangle in bands of 4 tile-rows, column by column inside a band, so tiles
+// that are near each other in the order share row panels and column panels of A.
+__device__ __forceinline__ void syrk_tile_of(int pid, int T, int &tm, int &tn) {
+    constexpr int BAND = 4;
     int row0 = 0;
     for (;;) {
         const int h = min(BAND, T - row0);                     // rows in this band
@@ -119,12 +121,22 @@ __device__ __forceinline__ void syrk_tile(int bid, int T, int &tm, int &tn) {
     }
 }
 
+// Workgroup id of a launch over `count` positions starting at `first`.  Ids are dealt round-robin
+// to the 8 XCDs, so each XCD is first given one contiguous run of the order: the workgroups
+// resident on one XCD at a time then share a few panels of A in its L2.
+__device__ __forceinline__ void syrk_tile(int bid, int first, int count, int T, int &tm, int &tn) {
+    constexpr int NXCD = 8;
+    int pid = bid;
+    if (count % NXCD == 0) pid = (bid % NXCD) * (count / NXCD) + bid / NXCD;
+    syrk_tile_of(first + pid, T, tm, tn);
+}
+
 template <class Cfg, bool EDGE, int MODE>
 __global__ void __launch_bounds__(Cfg::NTHREADS) ssyrk_kernel(const SyrkArgs g) {
     static_assert(Cfg::BM == Cfg::BN && Cfg::BSTYLE == STYLE_KC, "square KC/KC tiles");
     extern __shared__ __align__(16) float smem[];
     int tm, tn;
-    syrk_tile(blockIdx.x, g.tiles, tm, tn);
+    syrk_tile(blockIdx.x, g.tile_first, g.tile_count, g.tiles, tm, tn);
     const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
     RowMajorKcLoader<Cfg, EDGE> la(g.A, g.lda, m0, g.N, g.K);
     RowMajorKcLoaderB<Cfg, EDGE> lb(g.A, g.lda, n0, g.N, g.K);
@@ -140,7 +152,7 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) ssyrk_kernel(const SyrkArgs g) 
             const int r = m0 + row, c = n0 + col;
             v4f up = v * g.alpha, lo = up;
             if (g.Cin) {
-                v4f cu, cl;
+                v4f cu = {0.f, 0.f, 0.f, 0.f}, cl = cu;
                 if (MODE == SYRK_FLAT_FULL || g.upper) {
 #pragma unroll
                     for (int e = 0; e < 4; e++) cu[e] = g.Cin[(int64_t)(r + e) * g.ldcin + c];
@@ -162,6 +174,52 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) ssyrk_kernel(const SyrkArgs g) 
 #pragma unroll
         for (int e = 0; e < 4; e++) syrk_store<MODE>(g, m0 + row + e, n0 + col, v[e], diag);
     });
+}
+
+// The tiles of the last, partial round of 256 workgroups: each tile's reduction is split over
+// `splits` workgroups so that the round still fills the CUs and lasts 1/splits as long.  Workgroup
+// id = split * tile_count + tile: neighbours work on neighbouring tiles over the same slice of k.
+template <class Cfg, bool EDGE>
+__global__ void __launch_bounds__(Cfg::NTHREADS) ssyrk_split_kernel(const SyrkArgs g) {
+    extern __shared__ __align__(16) float smem[];
+    const int split = blockIdx.x / g.tile_count, t = blockIdx.x - split * g.tile_count;
+    int tm, tn;
+    syrk_tile_of(g.tile_first + t, g.tiles, tm, tn);
+    const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
+    int kt0, kt1;
+    split_range((g.K + Cfg::BK - 1) / Cfg::BK, g.splits, split, kt0, kt1);
+    RowMajorKcLoader<Cfg, EDGE> la(g.A, g.lda, m0, g.N, g.K, kt0 * Cfg::BK);
+    RowMajorKcLoaderB<Cfg, EDGE> lb(g.A, g.lda, n0, g.N, g.K, kt0 * Cfg::BK);
+    Accum<Cfg> acc;
+    mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem);
+    store_partial<Cfg>(acc, g.scratch, split, 0, t * Cfg::BN, Cfg::BM, g.tile_count * Cfg::BN);
+}
+
+// Adds the planes of the split tiles in ascending order and stores each sum like the one-pass
+// epilogue.  One thread per four consecutive rows of one column of one tile.
+template <int B, int MODE>
+__global__ void __launch_bounds__(256) ssyrk_split_sum_kernel(const SyrkArgs g) {
+    const size_t plane = (size_t)g.tile_count * B * B;
+    const size_t groups = plane / 4;
+    for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < groups; q += (size_t)gridDim.x * blockDim.x) {
+        const float *p = g.scratch + q * 4;
+        v4f sum = *reinterpret_cast<const v4f *>(p);
+        int s = 1;
+        for (; s + 3 < g.splits; s += 4) {   // four loads in flight; the additions stay in ascending order
+            const v4f a = *reinterpret_cast<const v4f *>(p + (size_t)s * plane);
+            const v4f b = *reinterpret_cast<const v4f *>(p + (size_t)(s + 1) * plane);
+            const v4f c = *reinterpret_cast<const v4f *>(p + (size_t)(s + 2) * plane);
+            const v4f d = *reinterpret_cast<const v4f *>(p + (size_t)(s + 3) * plane);
+            sum = (((sum + a) + b) + c) + d;
+        }
+        for (; s < g.splits; s++) sum += *reinterpret_cast<const v4f *>(p + (size_t)s * plane);
+        const int colg = (int)(q / (B / 4)), row = (int)(q % (B / 4)) * 4;
+        const int t = colg / B, col = colg - t * B;
+        int tm, tn;
+        syrk_tile_of(g.tile_first + t, g.tiles, tm, tn);
+#pragma unroll
+        for (int e = 0; e < 4; e++) syrk_store<MODE>(g, tm * B + row + e, tn * B + col, sum[e], tm == tn);
+    }
 }
 
 // Small N: few tiles for 256 CUs, and 1024-long reductions that a launch gap rivals.  One launch
@@ -367,8 +425,32 @@ using SyrkL = TileCfg<256, 256, 16, 4, 2, STYLE_KC>;
 using SyrkM = TileCfg<128, 128, 16, 2, 2, STYLE_KC>;
 using SyrkS = TileCfg<64, 64, 16, 2, 1, STYLE_KC>;
 
+// How the last, partial round of 256 tiles is split: `tail` tiles, each over `splits` workgroups.
+struct SyrkTail {
+    int64_t total, tail;
+    int splits;
+    size_t scratch_bytes;
+};
+static SyrkTail plan_syrk_tail(int N, int K, int b, int bk) {
+    SyrkTail t{};
+    const int64_t side = (N + b - 1) / b;
+    t.total = side * (side + 1) / 2;
+    t.tail = t.total % 256;
+    t.splits = 1;
+    if (t.total > 256 && t.tail > 0 && t.tail <= 128) {
+        const int pairs = (K + 2 * bk - 1) / (2 * bk);
+        int s = (int)(256 / t.tail);
+        if (s > pairs / 8) s = pairs / 8;          // at least 8 pairs of k-tiles per workgroup
+        if (s > 32) s = 32;
+        if (s >= 2) t.splits = s;
+    }
+    if (t.splits == 1) t.tail = 0;
+    t.scratch_bytes = (size_t)t.tail * t.splits * b * b * sizeof(float);
+    return t;
+}
+
 template <class Cfg>
-static int launch_syrk(SyrkArgs g, hipStream_t stream) {
+static int launch_syrk(SyrkArgs g, hipStream_t stream, float *scratch = nullptr, size_t scratch_bytes = 0) {
     g.tiles = (g.N + Cfg::BM - 1) / Cfg::BM;
     const bool edge = (g.N % Cfg::BM) || (g.K % (2 * Cfg::BK));
     const size_t smem = Cfg::SMEM_FLOATS * sizeof(float);
@@ -380,8 +462,32 @@ static int launch_syrk(SyrkArgs g, hipStream_t stream) {
     }
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
-    const int64_t count = (int64_t)g.tiles * (g.tiles + 1) / 2;
-    hipLaunchKernelGGL(kern, dim3((unsigned)count), dim3(Cfg::NTHREADS), smem, stream, g);
+    SyrkTail tail = plan_syrk_tail(g.N, g.K, Cfg::BM, Cfg::BK);
+    if (!scratch || scratch_bytes < tail.scratch_bytes) tail.tail = 0;
+    g.tile_first = 0;
+    g.tile_count = (int)(tail.total - tail.tail);
+    g.splits = 1;
+    hipLaunchKernelGGL(kern, dim3((unsigned)g.tile_count), dim3(Cfg::NTHREADS), smem, stream, g);
+    if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
+    if (tail.tail == 0) return T2SP_OK;
+    g.tile_first = g.tile_count;
+    g.tile_count = (int)tail.tail;
+    g.splits = tail.splits;
+    g.scratch = scratch;
+    auto split_kern = edge ? ssyrk_split_kernel<Cfg, true> : ssyrk_split_kernel<Cfg, false>;
+    if (hipFuncSetAttribute((const void *)split_kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+        return T2SP_ERR_LAUNCH;
+    hipLaunchKernelGGL(split_kern, dim3((unsigned)(g.tile_count * g.splits)), dim3(Cfg::NTHREADS), smem, stream, g);
+    if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
+    void (*sum_kern)(const SyrkArgs);
+    switch (g.mode) {
+        case SYRK_FLAT_SYM: sum_kern = ssyrk_split_sum_kernel<Cfg::BM, SYRK_FLAT_SYM>; break;
+        case SYRK_FLAT_FULL: sum_kern = ssyrk_split_sum_kernel<Cfg::BM, SYRK_FLAT_FULL>; break;
+        default: sum_kern = ssyrk_split_sum_kernel<Cfg::BM, SYRK_FOLDED>; break;
+    }
+    const size_t groups = (size_t)g.tile_count * Cfg::BM * Cfg::BM / 4;
+    const size_t blocks = (groups + 255) / 256;
+    hipLaunchKernelGGL(sum_kern, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0, stream, g);
     return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
 }
 
@@ -390,13 +496,16 @@ static int dispatch_syrk(SyrkArgs g, int trans, int cfg, float *workspace, size_
     if (g.N <= 0 || g.K <= 0) return T2SP_ERR_SHAPE;
     if (trans) {
         // A is stored K x N: bring it to N x K first (the MFMA loaders want k contiguous)
-        if (!workspace || workspace_bytes < (size_t)g.N * g.K * sizeof(float)) return T2SP_ERR_SHAPE;
+        const size_t relaid = (size_t)g.N * g.K * sizeof(float);
+        if (!workspace || workspace_bytes < relaid) return T2SP_ERR_SHAPE;
         const int ext[2] = {g.K, g.N};
         const int64_t ss[2] = {g.lda, 1}, ds[2] = {1, g.K};
         const int rc = t2sp_relayout_f32(g.A, workspace, 2, ext, ss, ds, stream);
         if (rc != T2SP_OK) return rc;
         g.A = workspace;
         g.lda = g.K;
+        workspace += (size_t)g.N * g.K;      // what is left may hold the planes of a split last round
+        workspace_bytes -= relaid;
     }
     if (cfg == T2SP_CFG_DIRECT16) return syrk_d16_ok(g) ? launch_syrk_d16(g, stream) : T2SP_ERR_SHAPE;
     if (cfg == T2SP_CFG_AUTO && g.N <= SYRK_D16_MAX_N && g.K >= 64 && syrk_d16_ok(g)) return launch_syrk_d16(g, stream);
@@ -411,22 +520,26 @@ static int dispatch_syrk(SyrkArgs g, int trans, int cfg, float *workspace, size_
         return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
     }
     if (cfg == T2SP_CFG_AUTO) {
-        // Estimated time of each tile size: the largest number of tiles any of the 256 CUs gets,
+        // Estimated time of each tile size: the number of rounds of 256 tiles (a last round whose
+        // reduction is split over the CUs counts 1/splits, plus a little for adding the planes)
         // times the work of one tile over the fraction of the MFMA rate that tile size sustains
         // (measured: the 128 and 64 tiles run at about 0.93 and 0.78 of the 256 tile's rate, and
-        // their finer grain wastes less of the last round).
+        // their finer grain wastes less of an unsplit last round).
         auto cost = [&](int b, double eff) {
-            const int64_t t = (g.N + b - 1) / b, tiles = t * (t + 1) / 2;
-            return (double)((tiles + 255) / 256) * b * b / eff;
+            const SyrkTail t = plan_syrk_tail(g.N, g.K, b, 16);
+            const bool split = t.tail > 0 && workspace && workspace_bytes >= t.scratch_bytes;
+            const double rounds = split ? (double)((t.total - t.tail) / 256) + 1.0 / t.splits + 0.03
+                                        : (double)((t.total + 255) / 256);
+            return rounds * b * b / eff;
         };
         const double c256 = cost(256, 1.0), c128 = cost(128, 0.93), c64 = cost(64, 0.78);
         cfg = (c256 <= c128 && c256 <= c64) ? T2SP_CFG_256x256 : (c128 <= c64 ? T2SP_CFG_128x128 : T2SP_CFG_64x128);
     }
     switch (cfg) {
-        case T2SP_CFG_256x256: return launch_syrk<SyrkL>(g, stream);
-        case T2SP_CFG_128x128: return launch_syrk<SyrkM>(g, stream);
+        case T2SP_CFG_256x256: return launch_syrk<SyrkL>(g, stream, workspace, workspace_bytes);
+        case T2SP_CFG_128x128: return launch_syrk<SyrkM>(g, stream, workspace, workspace_bytes);
         case T2SP_CFG_64x128:
-        case T2SP_CFG_32x128: return launch_syrk<SyrkS>(g, stream);
+        case T2SP_CFG_32x128: return launch_syrk<SyrkS>(g, stream, workspace, workspace_bytes);
         default: return T2SP_ERR_SHAPE;
     }
 }
@@ -454,7 +567,15 @@ __global__ void __launch_bounds__(256) syrk_fold_kernel(const float *flat, float
 }  // namespace t2sp
 
 extern "C" size_t t2sp_ssyrk_workspace_bytes(int trans, int N, int K) {
-    return (trans && N > 0 && K > 0) ? (size_t)N * K * sizeof(float) : 0;
+    if (N <= 0 || K <= 0) return 0;
+    // the re-laid A of the transposed form (required), then room for the planes of a split last
+    // round with any of the tile sizes (optional: without it the last round runs unsplit)
+    size_t planes = 0;
+    for (int b : {256, 128, 64}) {
+        const t2sp::SyrkTail t = t2sp::plan_syrk_tail(N, K, b, 16);
+        if (t.scratch_bytes > planes) planes = t.scratch_bytes;
+    }
+    return (trans ? (size_t)N * K * sizeof(float) : 0) + planes;
 }
 
 extern "C" size_t t2sp_ssyrk_folded_workspace_bytes(int trans, int N, int K) {

@@ -113,6 +113,45 @@ def test_full_size_sampled_rows_and_symmetry(oracle):
         assert err <= TOL
 
 
+@pytest.mark.parametrize("N,K,cfg", [(6144, 1024, 0), (6144, 1024, 1), (6000, 1000, 1), (3328, 1024, 2), (8192, 2048, 0)])
+def test_split_last_round_equals_unsplit(oracle, N, K, cfg):
+    """With a workspace the tiles of the last, partial round of 256 split their reduction over the
+    CUs: the result must agree with the run without a workspace (same kernels, unsplit) and, on
+    sampled rows, with the oracle; for every output form, including C updated in place."""
+    import torch
+    L = t2sp_amd.lib()
+    A = t2sp_amd.fill_uniform(torch.empty(N, K, device="cuda"), 75)
+    C0 = t2sp_amd.fill_uniform(torch.empty(N, N, device="cuda"), 76)
+    nbytes = L.t2sp_ssyrk_workspace_bytes(0, N, K)
+    assert nbytes > 0
+    ws = torch.empty(nbytes // 4, device="cuda")
+    a, c0 = A.cpu().numpy(), C0.cpu().numpy()
+    csym = np.triu(c0) + np.triu(c0, 1).T
+    for mirror in (0, 1, 2):
+        outs = []
+        for w, nb in ((None, 0), (ws.data_ptr(), nbytes)):
+            C = C0.clone()
+            rc = L.t2sp_ssyrk_f32(1, 0, N, K, 0.7, A.data_ptr(), K, 1.3, C.data_ptr(), N, C.data_ptr(), N, mirror, cfg,
+                                  w, nb, None)
+            assert rc == 0
+            torch.cuda.synchronize()
+            outs.append(C)
+        plain, split = outs
+        assert not torch.isnan(split).any()
+        if mirror == 0:                                       # the lower triangle still holds C0 in both
+            assert torch.equal(torch.tril(plain, -1), torch.tril(split, -1))
+        diff = (plain - split).abs().max().item()
+        assert diff <= 4e-6 * plain.abs().max().item(), diff  # a few ulps of the largest (diagonal) sums
+        assert not torch.equal(plain, split)                  # the split path really ran (sums differ in the last bits)
+        want_src = csym if mirror < 2 else c0
+        for row0 in (0, N // 2 - 3, N - 8):
+            want = oracle.syrk(a, want_src, 0.7, 1.3, rows=(row0, 8))
+            got = split[row0:row0 + 8].cpu().numpy()
+            if mirror == 0:                                   # only the upper triangle is written
+                got, want = np.triu(got, row0), np.triu(want, row0)
+            assert rel_fro(got, want)[0] <= TOL
+
+
 def test_error_codes():
     A = np.zeros((96, 16), np.float32)
     C = np.zeros((96, 96), np.float32)
