@@ -32,6 +32,10 @@ struct GemmArgs {
     // reduction split over `splits` workgroups per tile (1 = none): partial planes in scratch
     int splits, Mp, Np;
     float *scratch;
+    // a launch covers `tile_count` positions of the tile walking order starting at `tile_first`;
+    // with `compact` the planes hold just those tiles side by side ([row][tile][col]) instead of
+    // the whole padded matrix
+    int tile_first, tile_count, compact;
 };
 
 __device__ __forceinline__ int64_t tiled_offset(const GemmArgs &g, int row, int col) {
@@ -50,17 +54,35 @@ __device__ __forceinline__ void gemm_store1(const GemmArgs &g, int r, int c, flo
         g.C[(int64_t)r * g.ldc + c] = v;
 }
 
-// Where the sum of the partial planes of a split reduction goes (plain C = A*B only).
+// Where the sum of the partial planes of a split reduction goes.
 struct GemmOutMap {
     GemmArgs g;
     __device__ __forceinline__ void store(int row, int col, v4f v) const {
         if (row >= g.M || col >= g.N) return;
+        if (g.scale) {
+            v = v * g.alpha;
+            if (g.beta != 0.f) v += *reinterpret_cast<const v4f *>(g.Cin + (int64_t)row * g.ldcin + col) * g.beta;
+        }
         if (!g.tiled) {
             *reinterpret_cast<v4f *>(g.C + (int64_t)row * g.ldc + col) = v;
+        } else if (g.s[0] == 1 && g.t_jjj % 4 == 0) {
+            *reinterpret_cast<v4f *>(g.C + tiled_offset(g, row, col)) = v;
         } else {
 #pragma unroll
             for (int e = 0; e < 4; e++) g.C[tiled_offset(g, row, col + e)] = v[e];
         }
+    }
+};
+
+// The same for compact planes: column `col` of a plane belongs to tile col / BN of the launch.
+template <int BM, int BN>
+struct GemmCompactMap {
+    GemmOutMap inner;
+    __device__ __forceinline__ void store(int row, int col, v4f v) const {
+        const int t = col / BN;
+        int tm, tn;
+        tile_of_position(inner.g.tile_first + t, inner.g.tiles_m, inner.g.tiles_n, inner.g.group_m, tm, tn);
+        inner.store(tm * BM + row, tn * BN + (col - t * BN), v);
     }
 };
 
@@ -71,7 +93,9 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) sgemm_kernel(const GemmArgs g) 
     extern __shared__ __align__(16) float smem[];
     const int tile = blockIdx.x / g.splits, split = blockIdx.x - tile * g.splits;
     int tm, tn;
-    tile_coords(tile, g.tiles_m, g.tiles_n, g.group_m, tm, tn);
+    // the workgroups of a split tile read different slices of k: no run per XCD to arrange
+    tile_of_position(g.tile_first + (g.compact ? tile : xcd_contiguous(tile, g.tile_count)), g.tiles_m, g.tiles_n,
+                     g.group_m, tm, tn);
     const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
     int kt0 = 0, kt1 = ktiles_even<Cfg>(g.K);
     if (g.splits > 1) split_range((g.K + Cfg::BK - 1) / Cfg::BK, g.splits, split, kt0, kt1);
@@ -90,7 +114,8 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) sgemm_kernel(const GemmArgs g) 
         RowMajorRcLoader<Cfg, EDGE> lb(g.B, g.ldb, n0, g.N, g.K, kt0 * Cfg::BK);
         mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem);
         if (g.splits > 1) {
-            store_partial<Cfg>(acc, g.scratch, split, m0, n0, g.Mp, g.Np);
+            if (g.compact) store_partial<Cfg>(acc, g.scratch, split, 0, tile * Cfg::BN, Cfg::BM, g.tile_count * Cfg::BN);
+            else store_partial<Cfg>(acc, g.scratch, split, m0, n0, g.Mp, g.Np);
             return;
         }
         drain<Cfg>(acc, [&](int row, int col, v4f v) {   // v = D[row][col..col+3]
@@ -361,8 +386,61 @@ __global__ void sgemm_scalar_kernel(const GemmArgs g, int bt) {
     gemm_store1(g, r, c, acc);
 }
 
+// A launch plan over the tile walking order: whole rounds of 256 workgroups first, then the
+// remaining tiles in up to two groups whose reduction is split so that each group again puts
+// about one workgroup on every CU and lasts 1/splits of a round (a remainder above 128 tiles
+// goes as 128 tiles split in two, then the rest).  Without this the last, partial round costs a
+// whole one: 576 tiles (6144^2 outputs in 256 x 256 tiles) would take 3 rounds instead of 2.25.
+struct GemmPhase {
+    int first, count, splits;
+};
+struct GemmPhases {
+    int n;
+    GemmPhase ph[4];
+    size_t scratch_bytes;     // the largest group's planes
+    double rounds;            // estimated duration in rounds of one unsplit tile
+};
+constexpr int GEMM_CUS = 256;
+constexpr double GEMM_SPLIT_OVERHEAD = 0.03;   // prologue, plane traffic and extra launches, in rounds of a K = 8192 tile
+
+static GemmPhases plan_phases(int64_t tiles, int K, int bk, int bm, int bn, bool allow_split) {
+    GemmPhases p{};
+    const int pairs = (K + 2 * bk - 1) / (2 * bk);
+    int64_t first = 0, rest = tiles;
+    const int64_t full = rest / GEMM_CUS * GEMM_CUS;
+    if (full == 0) allow_split = false;        // a single partial round: splitting it gains nothing
+    if (full > 0) {
+        p.ph[p.n++] = GemmPhase{0, (int)full, 1};
+        p.rounds += (double)(full / GEMM_CUS);
+        first = full;
+        rest -= full;
+    }
+    while (rest > 0) {
+        int64_t take = rest;
+        int s = (int)(GEMM_CUS / rest);
+        if (s < 2 && rest > GEMM_CUS / 2 && p.n < 2) { take = GEMM_CUS / 2; s = 2; }
+        if (s > pairs / 4) s = pairs / 4;      // at least 4 pairs of k-tiles per workgroup
+        if (s > 32) s = 32;
+        if (!allow_split || s < 2 || p.n == 3) { take = rest; s = 1; }
+        if (s == 1 && p.n > 0 && p.ph[p.n - 1].splits == 1) {
+            p.ph[p.n - 1].count += (int)take;  // no split: the tiles simply join the preceding launch
+        } else {
+            p.ph[p.n++] = GemmPhase{(int)first, (int)take, s};
+        }
+        p.rounds += s == 1 ? 1.0 : 1.0 / s + GEMM_SPLIT_OVERHEAD * 8192.0 / (K > 0 ? K : 1);
+        if (s > 1) {
+            const size_t bytes = (size_t)take * s * bm * bn * sizeof(float);
+            if (bytes > p.scratch_bytes) p.scratch_bytes = bytes;
+        }
+        first += take;
+        rest -= take;
+    }
+    return p;
+}
+
 template <class Cfg, bool BT>
-static int launch(GemmArgs g, hipStream_t stream, int splits = 1, float *scratch = nullptr) {
+static int launch(GemmArgs g, hipStream_t stream, int splits = 1, float *scratch = nullptr, size_t scratch_bytes = 0,
+                  bool phased = false) {
     g.tiles_m = (g.M + Cfg::BM - 1) / Cfg::BM;
     g.tiles_n = (g.N + Cfg::BN - 1) / Cfg::BN;
     g.splits = BT ? 1 : splits;
@@ -377,6 +455,29 @@ static int launch(GemmArgs g, hipStream_t stream, int splits = 1, float *scratch
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
+    const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+    if (!BT && phased && splits == 1) {
+        GemmPhases p = plan_phases(tiles, g.K, Cfg::BK, Cfg::BM, Cfg::BN, true);
+        if (scratch && scratch_bytes >= p.scratch_bytes) {
+            for (int i = 0; i < p.n; i++) {
+                g.tile_first = p.ph[i].first;
+                g.tile_count = p.ph[i].count;
+                g.splits = p.ph[i].splits;
+                g.compact = g.splits > 1;
+                hipLaunchKernelGGL(kern, dim3((unsigned)(g.tile_count * g.splits)), dim3(Cfg::NTHREADS), smem, stream, g);
+                if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
+                if (g.splits > 1) {
+                    GemmCompactMap<Cfg::BM, Cfg::BN> map{GemmOutMap{g}};
+                    if (launch_splitk_reduce<true>(scratch, g.splits, Cfg::BM, g.tile_count * Cfg::BN, map, stream) != hipSuccess)
+                        return T2SP_ERR_LAUNCH;
+                }
+            }
+            return T2SP_OK;
+        }
+    }
+    g.tile_first = 0;
+    g.tile_count = (int)tiles;
+    g.compact = 0;
     hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * g.splits), dim3(Cfg::NTHREADS), smem, stream, g);
     if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
     if (g.splits > 1) {
@@ -400,14 +501,23 @@ using GemmST = TileCfg<64, 64, 16, 2, 1, STYLE_KC>;
 // workspace; without one the product runs unsplit).
 struct GemmPlan {
     int cfg, splits;
+    bool phased;              // whole rounds, then the remaining tiles with a split reduction
     size_t scratch_bytes;
 };
 static GemmPlan plan_gemm(int M, int N, int K) {
     auto tiles = [&](int bm, int bn) { return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    GemmPlan p{T2SP_CFG_64x128, 1, 0};
-    if (tiles(256, 256) >= 200) p.cfg = T2SP_CFG_256x256;
-    else if (tiles(128, 128) >= 200) p.cfg = T2SP_CFG_128x128;
-    else {
+    GemmPlan p{T2SP_CFG_64x128, 1, false, 0};
+    if (tiles(256, 256) >= 200 || tiles(128, 128) >= 200) {
+        // estimated time = rounds x tile area / the fraction of the 256 x 256 tile's rate that the
+        // tile size sustains (measured: 0.94 for 128 x 128)
+        const GemmPhases l = plan_phases(tiles(256, 256), K, 16, 256, 256, true);
+        const GemmPhases m = plan_phases(tiles(128, 128), K, 16, 128, 128, true);
+        const double cl = l.rounds * 65536.0, cm = m.rounds * 16384.0 / 0.94;
+        const bool large = tiles(256, 256) >= 200 && cl <= cm;
+        p.cfg = large ? T2SP_CFG_256x256 : T2SP_CFG_128x128;
+        p.phased = true;
+        p.scratch_bytes = large ? l.scratch_bytes : m.scratch_bytes;
+    } else {
         const int bm = tiles(128, 128) >= 32 ? 128 : 64;
         p.cfg = bm == 128 ? T2SP_CFG_128x128 : T2SP_CFG_64x128;
         const int64_t t = tiles(bm, 128);
@@ -533,10 +643,19 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
     }
     int splits = 1;
+    bool phased = false;
     if (cfg == T2SP_CFG_AUTO) {
         const GemmPlan p = plan_gemm(g.M, g.N, g.K);
         cfg = p.cfg;
         if (!bt && !g.scale && p.splits > 1 && workspace && workspace_bytes >= p.scratch_bytes) splits = p.splits;
+        phased = !bt && p.phased && workspace && workspace_bytes >= p.scratch_bytes;
+        // without room for the planes the last round runs unsplit: then the finer tiles waste less of it
+        if (!bt && p.phased && !phased) {
+            const int64_t t256 = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
+            const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
+            const double cl = (double)((t256 + 255) / 256) * 65536.0, cm = (double)((t128 + 255) / 256) * 16384.0 / 0.94;
+            cfg = (t256 >= 200 && cl <= cm) ? T2SP_CFG_256x256 : T2SP_CFG_128x128;
+        }
     }
     if (bt) {
         switch (cfg) {
@@ -548,8 +667,8 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         }
     }
     switch (cfg) {
-        case T2SP_CFG_256x256: return launch<GemmL, false>(g, stream);
-        case T2SP_CFG_128x128: return launch<GemmM, false>(g, stream, splits, workspace);
+        case T2SP_CFG_256x256: return launch<GemmL, false>(g, stream, 1, workspace, workspace_bytes, phased);
+        case T2SP_CFG_128x128: return launch<GemmM, false>(g, stream, splits, workspace, workspace_bytes, phased);
         case T2SP_CFG_64x128: return launch<GemmS, false>(g, stream, splits, workspace);
         case T2SP_CFG_32x128: return launch<GemmW, false>(g, stream);
         default: return T2SP_ERR_SHAPE;

@@ -344,18 +344,11 @@ __device__ __forceinline__ void drain(const Accum<Cfg> &acc, Emit &&emit) {
     }
 }
 
-// Workgroup id -> tile coordinates.  Workgroups are dealt round-robin to the 8
-// XCDs (each with its own L2), so consecutive ids land on different L2s.  The
-// remap gives every XCD one contiguous run of tile ids, and inside a run tiles
-// are visited in bands of GROUP_M tile-rows, column by column, so that the ~32
-// workgroups resident on one XCD share a few row panels of X and column panels
-// of Y in that XCD's L2.
-__device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, int group_m,
-                                            int &tm, int &tn) {
-    const int total = tiles_m * tiles_n;
-    constexpr int NXCD = 8;
-    int pid = bid;
-    if (total % NXCD == 0) pid = (bid % NXCD) * (total / NXCD) + bid / NXCD;
+// Position `pid` of the walking order -> tile coordinates: tiles are visited in bands of group_m
+// tile-rows, column by column inside a band, so that tiles near each other in the order share a
+// few row panels of X and column panels of Y.
+__device__ __forceinline__ void tile_of_position(int pid, int tiles_m, int tiles_n, int group_m,
+                                                 int &tm, int &tn) {
     const int band = group_m * tiles_n;
     const int band_id = pid / band;
     const int first_m = band_id * group_m;
@@ -363,6 +356,21 @@ __device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, i
     const int in_band = pid - band_id * band;
     tm = first_m + in_band % rows;
     tn = in_band / rows;
+}
+
+// Workgroup ids are dealt round-robin to the 8 XCDs (each with its own L2), so consecutive ids
+// land on different L2s.  This remap gives every XCD one contiguous run of the `count` positions
+// a launch covers, so that the ~32 workgroups resident on one XCD are neighbours in the walking
+// order and share panels in that XCD's L2.
+__device__ __forceinline__ int xcd_contiguous(int bid, int count) {
+    constexpr int NXCD = 8;
+    return count % NXCD == 0 ? (bid % NXCD) * (count / NXCD) + bid / NXCD : bid;
+}
+
+// Workgroup id -> tile coordinates for a launch over all tiles.
+__device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, int group_m,
+                                            int &tm, int &tn) {
+    tile_of_position(xcd_contiguous(bid, tiles_m * tiles_n), tiles_m, tiles_n, group_m, tm, tn);
 }
 
 }  // namespace t2sp

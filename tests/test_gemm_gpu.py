@@ -163,6 +163,48 @@ def test_split_reduction_with_workspace(oracle, torch_cuda, shape):
     assert rel_fro(C.cpu().numpy(), outs[0])[0] <= TOL
 
 
+@pytest.mark.parametrize("shape", [(6144, 6144, 4096), (3072, 3072, 2048), (5120, 5120, 512), (4100, 4100, 1024),
+                                   (3000, 7000, 520), (6400, 6400, 256)])
+def test_partial_last_round_split_with_workspace(oracle, torch_cuda, shape):
+    """Tile counts that are not a multiple of 256: with a workspace the tiles left after the whole
+    rounds split their reduction.  The whole result against the run without a workspace, sampled
+    rows (the last rows are where the split tiles lie) against the oracle, same bits twice, and the
+    tiled output form through the same path."""
+    torch = torch_cuda
+    M, N, K = shape
+    L = t2sp_amd.lib()
+    nbytes = L.t2sp_sgemm_workspace_bytes(M, N, K)
+    assert nbytes > 0
+    A = t2sp_amd.fill_uniform(torch.empty(M, K, device="cuda"), 23)
+    B = t2sp_amd.fill_uniform(torch.empty(K, N, device="cuda"), 24)
+    ws = torch.empty(nbytes // 4, device="cuda")
+    outs = []
+    for w, nb in ((None, 0), (ws.data_ptr(), nbytes), (ws.data_ptr(), nbytes)):
+        C = torch.full((M, N), float("nan"), device="cuda")
+        assert L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, w, nb, None) == 0
+        torch.cuda.synchronize()
+        outs.append(C)
+    plain, split, again = outs
+    assert torch.equal(split, again)
+    assert not torch.isnan(split).any()
+    assert (plain - split).abs().max().item() <= 4e-6 * plain.abs().max().item() * 4
+    assert not torch.equal(plain, split)
+    a, b = A.cpu().numpy(), B.cpu().numpy()
+    rows = np.unique(np.concatenate([[0, M // 2, M - 1, M - 2, M - 130, M - 300], np.random.default_rng(1).integers(0, M, 8)]))
+    err, mx = rel_fro(split[rows].cpu().numpy(), oracle.gemm(a[rows], b))
+    print("phased %s rel_fro %.3e max_abs %.3e" % (shape, err, mx))
+    assert err <= TOL
+    if M % 64 == 0 and N % 16 == 0:
+        III, II, JJJ, JJ = 16, 4, 8, 2
+        T = torch.full((M // 64, N // 16, II, JJ, III, JJJ), float("nan"), device="cuda")
+        s6 = (ctypes.c_int64 * 6)(*reversed(T.stride()))
+        assert L.t2sp_sgemm_f32_tiled(A.data_ptr(), B.data_ptr(), T.data_ptr(), M, N, K, K, N, JJJ, III, JJ, II, s6, 0,
+                                      ws.data_ptr(), nbytes, None) == 0
+        torch.cuda.synchronize()
+        flat = T.permute(0, 2, 4, 1, 3, 5).reshape(M, N)          # (i, ii, iii, j, jj, jjj)
+        assert torch.equal(flat, split)
+
+
 @pytest.mark.parametrize("shape", [(1024, 1024, 1024), (500, 260, 4096), (64, 128, 8192), (130, 66, 64), (1, 2, 8),
                                    (512, 768, 640), (192, 64, 24)])
 def test_direct_kernel_small_products(oracle, torch_cuda, shape):
