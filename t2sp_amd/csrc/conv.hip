@@ -188,33 +188,71 @@ static int launch_conv(ConvArgs g, int p_begin, int p_end, int splits, float *sc
     return T2SP_OK;
 }
 
-// How the automatic configuration covers the pixels: whole rounds of 256x256 tiles up to
-// p_split, then 128x128 tiles whose reduction is split `splits` ways so that the remainder
-// also spreads over all CUs.
+// How the automatic configuration covers the pixels.  One workgroup of the larger tiles occupies
+// a CU, so tiles run in rounds of 256 (the CU count) and a partial last round would leave most
+// CUs idle for a whole tile time.  Stages, each over its own range of output pixels:
+//   * whole rounds of the tile size that multiplies fastest for this CO (256 x 256 at its full
+//     rate, 128 x 128 at 0.94 of it, 64 x 128 at 0.8, each scaled by how much of its rows CO
+//     fills), then whole rounds of 128 x 128 tiles over what is left;
+//   * the rest, fewer tiles than CUs: the tile size and reduction split with the least estimated
+//     time (MFMA time of one workgroup + moving the partial planes; a split needs the workspace,
+//     without it the rest runs unsplit).
+struct ConvStage {
+    int cfg, p_begin, p_end, splits;
+};
 struct ConvPlan {
-    bool two_phase;
-    int p_split, splits;
+    int n;
+    ConvStage st[4];
     size_t scratch_bytes;
 };
 static ConvPlan plan_conv(int CO, int P, int KRED) {
     constexpr int CUS = 256;
-    ConvPlan p{false, 0, 1, 0};
-    const int tiles_m = (CO + 255) / 256;
-    const int rounds = (int)(((int64_t)tiles_m * (P / 256)) / CUS);
-    if (CO >= 256 && CUS % tiles_m == 0 && rounds >= 1) {
-        p.two_phase = true;
-        p.p_split = rounds * (CUS / tiles_m) * 256;
-        const int rem_tiles = ((CO + 127) / 128) * ((P - p.p_split + 127) / 128);
-        if (rem_tiles > 0 && rem_tiles < 128) {
-            int s = CUS / rem_tiles;
-            const int pairs = ((KRED + 15) / 16 + 1) / 2;
-            if (s > pairs / 4) s = pairs / 4;
-            if (s > 8) s = 8;
-            if (s > 1) {
-                p.splits = s;
-                p.scratch_bytes = (size_t)s * ((CO + 127) / 128 * 128) * ((P - p.p_split + 127) / 128 * 128) * sizeof(float);
-            }
+    struct Cand { int cfg, bm, bn; double eff; };
+    const Cand all[3] = {{T2SP_CFG_256x256, 256, 256, 1.0}, {T2SP_CFG_128x128, 128, 128, 0.94}, {T2SP_CFG_64x128, 64, 128, 0.8}};
+    auto tiles_m = [&](const Cand &c) { return (CO + c.bm - 1) / c.bm; };
+    auto tiles = [&](const Cand &c, int p0) { return (int64_t)tiles_m(c) * ((P - p0 + c.bn - 1) / c.bn); };
+    auto value = [&](const Cand &c) { return c.eff * CO / (double)(tiles_m(c) * c.bm); };
+    int best = 0;
+    for (int i = 1; i < 3; i++)
+        if (value(all[i]) > value(all[best])) best = i;
+
+    ConvPlan p{};
+    int p0 = 0;
+    // whole rounds: the best tile size, then 128 x 128 if that is smaller
+    for (int i = best; i < 3 && p0 < P; i++) {
+        if (i != best && all[i].cfg != T2SP_CFG_128x128) break;
+        const Cand &c = all[i];
+        const int64_t rounds = tiles(c, p0) / CUS;
+        if (rounds < 1) continue;
+        const int64_t ptiles = rounds * CUS / tiles_m(c);
+        const int p1 = (int)(p0 + ptiles * c.bn < P ? p0 + ptiles * c.bn : P);
+        p.st[p.n++] = ConvStage{c.cfg, p0, p1, 1};
+        p0 = p1;
+    }
+    if (p0 >= P) return p;
+    // the rest
+    const int pairs = ((KRED + 15) / 16 + 1) / 2;
+    double best_time = 1e300;
+    ConvStage tail{all[best].cfg, p0, P, 1};
+    for (int i = best; i < 3; i++) {
+        const Cand &c = all[i];
+        const int64_t t = tiles(c, p0);
+        int smax = (int)(CUS / (t < 1 ? 1 : t));
+        if (smax > pairs / 4) smax = pairs / 4;
+        if (smax > 16) smax = 16;
+        if (smax < 1) smax = 1;
+        for (int sp = 1; sp <= smax; sp++) {
+            const double wg = 2.0 * c.bm * c.bn * KRED / (614e9 * c.eff) / sp;     // one workgroup's MFMA time
+            const double rounds = (double)((t * sp + CUS - 1) / CUS);
+            const double planes = sp > 1 ? (double)t * sp * c.bm * c.bn * 8.0 / 3e12 + 8e-6 : 0.0;
+            const double time = wg * rounds + planes;
+            if (time < best_time) { best_time = time; tail = ConvStage{c.cfg, p0, P, sp}; }
         }
+    }
+    p.st[p.n++] = tail;
+    if (tail.splits > 1) {
+        const Cand &c = all[tail.cfg == T2SP_CFG_256x256 ? 0 : tail.cfg == T2SP_CFG_128x128 ? 1 : 2];
+        p.scratch_bytes = (size_t)tail.splits * (tiles_m(c) * c.bm) * ((P - p0 + c.bn - 1) / c.bn * c.bn) * sizeof(float);
     }
     return p;
 }
@@ -269,18 +307,20 @@ extern "C" int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, 
         case T2SP_CFG_AUTO: break;
         default: return T2SP_ERR_SHAPE;
     }
-    // Automatic choice.  One 256x256 tile occupies a CU, so big tiles run in rounds of 256 (the
-    // CU count); a partial last round would leave most CUs idle for a whole tile time.  Whole
-    // rounds of big tiles are therefore launched first and the remaining pixels are covered with
-    // 128x128 tiles; when those are too few to occupy the CUs their reduction is split as well
-    // (needs the workspace; without it the remainder runs unsplit).
+    // Automatic choice: the stages of plan_conv; a split stage without room for its planes runs unsplit.
     const ConvPlan plan = plan_conv(CO, g.P, g.KRED);
-    if (plan.two_phase) {
-        const int rc = launch_conv<ConvL>(g, 0, plan.p_split, 1, nullptr, st);
+    for (int i = 0; i < plan.n; i++) {
+        const ConvStage &sg = plan.st[i];
+        const bool split = sg.splits > 1 && workspace && workspace_bytes >= plan.scratch_bytes;
+        const int sp = split ? sg.splits : 1;
+        float *scratch = split ? workspace : nullptr;
+        int rc;
+        switch (sg.cfg) {
+            case T2SP_CFG_256x256: rc = launch_conv<ConvL>(g, sg.p_begin, sg.p_end, sp, scratch, st); break;
+            case T2SP_CFG_128x128: rc = launch_conv<ConvM>(g, sg.p_begin, sg.p_end, sp, scratch, st); break;
+            default: rc = launch_conv<ConvS>(g, sg.p_begin, sg.p_end, sp, scratch, st); break;
+        }
         if (rc != T2SP_OK) return rc;
-        const bool split = plan.splits > 1 && workspace && workspace_bytes >= plan.scratch_bytes;
-        return launch_conv<ConvM>(g, plan.p_split, g.P, split ? plan.splits : 1, split ? workspace : nullptr, st);
     }
-    if ((int64_t)((CO + 127) / 128) * ((g.P + 127) / 128) >= 128) return launch_conv<ConvM>(g, 0, g.P, 1, nullptr, st);
-    return launch_conv<ConvS>(g, 0, g.P, 1, nullptr, st);
+    return T2SP_OK;
 }

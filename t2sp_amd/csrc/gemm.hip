@@ -647,7 +647,7 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
     if (cfg == T2SP_CFG_AUTO) {
         const GemmPlan p = plan_gemm(g.M, g.N, g.K);
         cfg = p.cfg;
-        if (!bt && !g.scale && p.splits > 1 && workspace && workspace_bytes >= p.scratch_bytes) splits = p.splits;
+        if (!bt && p.splits > 1 && workspace && workspace_bytes >= p.scratch_bytes) splits = p.splits;
         phased = !bt && p.phased && workspace && workspace_bytes >= p.scratch_bytes;
         // without room for the planes the last round runs unsplit: then the finer tiles waste less of it
         if (!bt && p.phased && !phased) {
@@ -706,8 +706,9 @@ extern "C" int t2sp_sgemm_f32_tiled(const float *A, const float *B, float *C, in
 }
 
 extern "C" size_t t2sp_sgemm_ex_workspace_bytes(int transa, int M, int N, int K) {
-    (void)N;
-    return (transa && M > 0 && K > 0) ? (size_t)M * K * sizeof(float) : 0;
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    // the re-laid A of the transposed form (required), then the planes of a split reduction (optional)
+    return (transa ? (size_t)M * K * sizeof(float) : 0) + t2sp::plan_gemm(M, N, K).scratch_bytes;
 }
 
 extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, float alpha, const float *A,
@@ -726,6 +727,8 @@ extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, fl
         if (rc != T2SP_OK) return rc;
         a = workspace;
         la = K;
+        workspace += (size_t)M * K;
+        workspace_bytes -= (size_t)M * K * sizeof(float);
     }
     t2sp::GemmArgs g{};
     g.A = a; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K;
@@ -733,5 +736,5 @@ extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, fl
     g.tiled = 0;
     g.scale = 1; g.alpha = alpha; g.beta = beta; g.Cin = Cin ? Cin : C; g.ldcin = Cin ? ldcin : ldc;
     if (!Cin) g.beta = 0.f;
-    return t2sp::dispatch(g, cfg, transb != 0, (hipStream_t)stream);
+    return t2sp::dispatch(g, cfg, transb != 0, (hipStream_t)stream, workspace, workspace_bytes);
 }

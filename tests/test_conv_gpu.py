@@ -58,6 +58,25 @@ def test_ragged_shapes(oracle, shape):
     assert rel_fro(run(I, W), oracle.conv(I, W))[0] <= TOL
 
 
+# (N, CI, CO, OY, OX): sizes at which the automatic plan takes, in turn: whole rounds of 128 x 128
+# tiles and a split rest; a rest only (one image); 64-row tiles for few output channels; two tile rows
+# of 256 with whole rounds of 128 x 128 and a split rest; whole rounds of 256 x 256 and a rest
+STAGE_SHAPES = [(4, 64, 256, 96, 96), (1, 64, 256, 56, 56), (8, 64, 64, 56, 56), (64, 64, 512, 12, 12),
+                (20, 64, 256, 60, 64)]
+
+
+@pytest.mark.parametrize("shape", STAGE_SHAPES)
+def test_plan_stages_integer_exact(oracle, shape):
+    """Every stage of the automatic plan (whole rounds of one or two tile sizes, then a rest with a
+    split reduction) on small-integer data, where any summation order is exact."""
+    N, CI, CO, OY, OX = shape
+    rng = np.random.default_rng(7)
+    I = rng.integers(-2, 3, (N, CI, OY + 2, OX + 2)).astype(np.float32)
+    W = rng.integers(-2, 3, (CO, CI, 3, 3)).astype(np.float32)
+    got = run(I, W)
+    assert (got == oracle.conv(I, W)).all()
+
+
 def test_strided_4d_buffers(oracle):
     """Padded rows / channels in I and O, and an input larger than the output needs."""
     N, CI, CO, OY, OX = 2, 8, 8, 8, 6
