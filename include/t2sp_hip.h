@@ -138,8 +138,10 @@ int t2sp_ssymv_f32_tiled(float alpha, float beta, const float *A, const float *x
  * (n,ci,h,w), (co,ci,kh,kw), (n,co,h,w); "w" is the innermost spatial axis (the
  * one the reference calls y).  Dense NCHW/OIHW with OW % 4 == 0 takes the
  * implicit-GEMM MFMA kernel, anything else a scalar kernel.  `workspace` (optional, may be
- * NULL; t2sp_conv2d_workspace_bytes gives its size) lets the last, partial round of tiles split
- * its reduction over all CUs.  Replaces the device
+ * NULL; t2sp_conv2d_workspace_bytes gives its size) holds the partial planes that let the tiles
+ * left after whole rounds of 256 split their reduction over all CUs, and, when CI*KH*KW is not a
+ * multiple of 4, the weights re-laid with zero-padded rows (without it such a shape takes the
+ * scalar kernel).  Replaces the device
  * side of the reference's conv pipeline (t2s/tests/performance/conv/conv.cpp:59-65,
  * conv/bitstream/a10/a.cl). */
 size_t t2sp_conv2d_workspace_bytes(int N, int CI, int CO, int OH, int OW, int KH, int KW);

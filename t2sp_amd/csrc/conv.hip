@@ -261,12 +261,30 @@ using ConvL = TileCfg<256, 256, 16, 4, 2, STYLE_RC>;
 using ConvM = TileCfg<128, 128, 16, 4, 1, STYLE_RC>;
 using ConvS = TileCfg<64, 128, 16, 2, 1, STYLE_RC>;
 
+// Weight rows whose length is not a multiple of 4 (3 input channels x 7 x 7 = 147) cannot be read
+// with 128-bit loads where they lie: they are first copied into rows padded with zeros to a
+// multiple of 4.  The reduction still ends at the true length; the pad only completes the last load.
+__global__ void __launch_bounds__(256) conv_pad_weights_kernel(const float *W, int64_t sw_o, float *dst, int CO,
+                                                               int kred, int kred_pad) {
+    const int64_t total = (int64_t)CO * kred_pad;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
+        const int co = (int)(t / kred_pad), k = (int)(t - (int64_t)co * kred_pad);
+        dst[t] = k < kred ? W[co * sw_o + k] : 0.f;
+    }
+}
+static size_t conv_padded_weight_bytes(int CO, int kred) {
+    if (kred % 4 == 0) return 0;
+    const size_t bytes = (size_t)CO * ((kred + 3) / 4 * 4) * sizeof(float);
+    return (bytes + 255) / 256 * 256;
+}
+
 }  // namespace t2sp
 
 extern "C" size_t t2sp_conv2d_workspace_bytes(int N, int CI, int CO, int OH, int OW, int KH, int KW) {
     if (N <= 0 || CI <= 0 || CO <= 0 || OH <= 0 || OW <= 0 || KH <= 0 || KW <= 0) return 0;
     if ((int64_t)N * OH * OW > INT32_MAX || (int64_t)CI * KH * KW > INT32_MAX) return 0;
-    return t2sp::plan_conv(CO, N * OH * OW, CI * KH * KW).scratch_bytes;
+    // padded weight rows when their length is not a multiple of 4, then the planes of a split rest
+    return t2sp::conv_padded_weight_bytes(CO, CI * KH * KW) + t2sp::plan_conv(CO, N * OH * OW, CI * KH * KW).scratch_bytes;
 }
 
 extern "C" int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, int CI, int CO,
@@ -279,14 +297,32 @@ extern "C" int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, 
     if ((int64_t)N * OH * OW > INT32_MAX || (int64_t)CI * KH * KW > INT32_MAX) return T2SP_ERR_SHAPE;
     const int64_t in_span = (int64_t)(N - 1) * si4[0] + (int64_t)(CI - 1) * si4[1] +
                             (int64_t)(OH + KH - 2) * si4[2] + (OW + KW - 2);
-    const bool fast = cfg != T2SP_CFG_SCALAR && si4[3] == 1 && so4[3] == 1 && sw4[3] == 1 &&
-                      sw4[2] == KW && sw4[1] == (int64_t)KH * KW && sw4[0] % 4 == 0 && OW % 4 == 0 &&
-                      (CI * KH * KW) % 4 == 0 && KH * KW <= 4096 && in_span < INT32_MAX &&
+    hipStream_t st = (hipStream_t)stream;
+    const int kred = CI * KH * KW;
+    const bool w_dense = sw4[3] == 1 && sw4[2] == KW && sw4[1] == (int64_t)KH * KW;
+    int64_t sw_o = sw4[0];
+    const float *W_given = W;
+    bool padded = false;
+    const size_t pad_bytes = conv_padded_weight_bytes(CO, kred);
+    if (cfg != T2SP_CFG_SCALAR && w_dense && pad_bytes && workspace && workspace_bytes >= pad_bytes &&
+        ((uintptr_t)workspace % 16 == 0)) {
+        const int kred_pad = (kred + 3) / 4 * 4;
+        const int64_t total = (int64_t)CO * kred_pad;
+        hipLaunchKernelGGL(conv_pad_weights_kernel, dim3((unsigned)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096)),
+                           dim3(256), 0, st, W, sw4[0], workspace, CO, kred, kred_pad);
+        if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
+        W = workspace;
+        sw_o = kred_pad;
+        padded = true;
+        workspace += pad_bytes / sizeof(float);
+        workspace_bytes -= pad_bytes;
+    }
+    const bool fast = cfg != T2SP_CFG_SCALAR && si4[3] == 1 && so4[3] == 1 && w_dense && sw_o % 4 == 0 && OW % 4 == 0 &&
+                      (kred % 4 == 0 || padded) && KH * KW <= 4096 && in_span < INT32_MAX &&
                       so4[0] % 4 == 0 && so4[1] % 4 == 0 && so4[2] % 4 == 0 &&
                       ((uintptr_t)W % 16 == 0) && ((uintptr_t)O % 16 == 0) && ((uintptr_t)I % 4 == 0);
-    hipStream_t st = (hipStream_t)stream;
     if (!fast) {
-        ConvGenericArgs a{I, W, O, N, CI, CO, OH, OW, KH, KW, {}, {}, {}};
+        ConvGenericArgs a{I, W_given, O, N, CI, CO, OH, OW, KH, KW, {}, {}, {}};
         for (int d = 0; d < 4; d++) { a.si[d] = si4[d]; a.sw[d] = sw4[d]; a.so[d] = so4[d]; }
         const int64_t total = (int64_t)N * CO * OH * OW;
         const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
@@ -297,7 +333,7 @@ extern "C" int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, 
     g.I = I; g.W = W; g.O = O;
     g.N = N; g.CI = CI; g.CO = CO; g.OH = OH; g.OW = OW; g.KH = KH; g.KW = KW;
     g.si_n = (int)si4[0]; g.si_c = (int)si4[1]; g.si_h = (int)si4[2];
-    g.sw_o = sw4[0];
+    g.sw_o = sw_o;
     g.so_n = so4[0]; g.so_c = so4[1]; g.so_h = so4[2];
     g.P = N * OH * OW; g.KRED = CI * KH * KW;
     switch (cfg) {

@@ -58,6 +58,22 @@ def test_ragged_shapes(oracle, shape):
     assert rel_fro(run(I, W), oracle.conv(I, W))[0] <= TOL
 
 
+@pytest.mark.parametrize("shape", [(2, 3, 64, 32, 36, 7, 7), (1, 5, 40, 8, 20, 3, 3), (3, 3, 16, 12, 12, 5, 5), (1, 1, 8, 8, 8, 3, 3)])
+def test_odd_reduction_length_takes_padded_weights(oracle, shape):
+    """CI*KY*KX not a multiple of 4 (first-layer shapes such as 3 x 7 x 7 = 147): the weights are
+    re-laid with zero-padded rows and the MFMA path runs; integer data, exact result, and the
+    weights left untouched."""
+    N, CI, CO, OY, OX, KY, KX = shape
+    rng = np.random.default_rng(11)
+    I = rng.integers(-2, 3, (N, CI, OY + KY - 1, OX + KX - 1)).astype(np.float32)
+    W = rng.integers(-2, 3, (CO, CI, KY, KX)).astype(np.float32)
+    W0 = W.copy()
+    assert (run(I, W) == oracle.conv(I, W)).all()
+    assert (W == W0).all()
+    If, Wf = oracle.fill_uniform(I.shape, 12), oracle.fill_uniform(W.shape, 13)
+    assert rel_fro(run(If, Wf), oracle.conv(If, Wf))[0] <= TOL
+
+
 # (N, CI, CO, OY, OX): sizes at which the automatic plan takes, in turn: whole rounds of 128 x 128
 # tiles and a split rest; a rest only (one image); 64-row tiles for few output channels; two tile rows
 # of 256 with whole rounds of 128 x 128 and a split rest; whole rounds of 256 x 256 and a rest
