@@ -386,6 +386,34 @@ __global__ void sgemm_scalar_kernel(const GemmArgs g, int bt) {
     gemm_store1(g, r, c, acc);
 }
 
+// Zero-padded copy of a row-major rows x cols matrix into rows_p x cols_p (leading dimension cols_p).
+__global__ void __launch_bounds__(256) gemm_pad_copy_kernel(const float *src, int64_t ld, float *dst, int rows, int cols,
+                                                            int rows_p, int cols_p) {
+    const int64_t total = (int64_t)rows_p * cols_p;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
+        const int r = (int)(t / cols_p), c = (int)(t - (int64_t)r * cols_p);
+        dst[t] = (r < rows && c < cols) ? src[(int64_t)r * ld + c] : 0.f;
+    }
+}
+
+// The product computed on padded operands goes to the caller's C, with the BLAS form's scaling.
+__global__ void __launch_bounds__(256) gemm_unpad_kernel(const float *src, int64_t ld, const GemmArgs g) {
+    const int64_t total = (int64_t)g.M * g.N;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
+        const int r = (int)(t / g.N), c = (int)(t - (int64_t)r * g.N);
+        gemm_store1(g, r, c, src[(int64_t)r * ld + c]);
+    }
+}
+
+static inline int64_t round_up4(int64_t v) { return (v + 3) / 4 * 4; }
+static inline size_t round_up256(size_t v) { return (v + 255) / 256 * 256; }
+// Bytes of the padded copies of A, B and C for a product the vector loaders cannot take as it lies.
+static size_t gemm_pad_bytes(int M, int N, int K, bool bt) {
+    const int64_t kp = round_up4(K), np = bt ? N : round_up4(N);
+    return round_up256((size_t)M * kp * sizeof(float)) + round_up256((size_t)(bt ? (int64_t)N * kp : kp * np) * sizeof(float)) +
+           round_up256((size_t)M * np * sizeof(float));
+}
+
 // A launch plan over the tile walking order: whole rounds of 256 workgroups first, then the
 // remaining tiles in up to two groups whose reduction is split so that each group again puts
 // about one workgroup on every CU and lasts 1/splits of a round (a remainder above 128 tiles
@@ -638,6 +666,32 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
                         ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
                         ((uintptr_t)g.C % 16 == 0) && (g.tiled || g.ldc % 4 == 0) &&
                         (!g.scale || (g.ldcin % 4 == 0 && (uintptr_t)g.Cin % 16 == 0));
+    if (cfg == T2SP_CFG_AUTO && !vec_ok && workspace && ((uintptr_t)workspace % 16 == 0) &&
+        workspace_bytes >= gemm_pad_bytes(g.M, g.N, g.K, bt)) {
+        // K or N not a multiple of 4, or rows that are not 16-byte aligned: multiply zero-padded,
+        // aligned copies instead (the reference's BLAS wrapper pads its operands to tile multiples
+        // in the same way, t2s/peppers/blas/level3/gemm/release/a10/blas-gemm.cpp:28-31) and
+        // copy the result out.  Moving the matrices twice costs little next to the product.
+        const int kp = (int)round_up4(g.K), np = bt ? g.N : (int)round_up4(g.N);
+        float *a2 = workspace;
+        float *b2 = a2 + round_up256((size_t)g.M * kp * sizeof(float)) / sizeof(float);
+        float *c2 = b2 + round_up256((size_t)(bt ? (int64_t)g.N * kp : (int64_t)kp * np) * sizeof(float)) / sizeof(float);
+        const size_t used = gemm_pad_bytes(g.M, g.N, g.K, bt);
+        auto blocks = [](int64_t n) { return dim3((unsigned)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192)); };
+        hipLaunchKernelGGL(gemm_pad_copy_kernel, blocks((int64_t)g.M * kp), dim3(256), 0, stream, g.A, g.lda, a2, g.M, g.K, g.M, kp);
+        if (bt)
+            hipLaunchKernelGGL(gemm_pad_copy_kernel, blocks((int64_t)g.N * kp), dim3(256), 0, stream, g.B, g.ldb, b2, g.N, g.K, g.N, kp);
+        else
+            hipLaunchKernelGGL(gemm_pad_copy_kernel, blocks((int64_t)kp * np), dim3(256), 0, stream, g.B, g.ldb, b2, g.K, g.N, kp, np);
+        if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
+        GemmArgs h{};
+        h.A = a2; h.B = b2; h.C = c2; h.M = g.M; h.N = np; h.K = kp;
+        h.lda = kp; h.ldb = bt ? kp : np; h.ldc = np;
+        const int rc = dispatch(h, T2SP_CFG_AUTO, bt, stream, workspace + used / sizeof(float), workspace_bytes - used);
+        if (rc != T2SP_OK) return rc;
+        hipLaunchKernelGGL(gemm_unpad_kernel, blocks((int64_t)g.M * g.N), dim3(256), 0, stream, c2, (int64_t)np, g);
+        return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+    }
     if (cfg == T2SP_CFG_SCALAR || !vec_ok) {
         hipLaunchKernelGGL(sgemm_scalar_kernel, dim3((g.N + 255) / 256, g.M), dim3(256), 0, stream, g, bt ? 1 : 0);
         return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
@@ -679,7 +733,10 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
 
 extern "C" size_t t2sp_sgemm_workspace_bytes(int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
-    return t2sp::plan_gemm(M, N, K).scratch_bytes;
+    if (K % 4 == 0 && N % 4 == 0) return t2sp::plan_gemm(M, N, K).scratch_bytes;
+    // padded copies of the operands, then the planes for the padded product
+    return t2sp::gemm_pad_bytes(M, N, K, false) +
+           t2sp::plan_gemm(M, (int)t2sp::round_up4(N), (int)t2sp::round_up4(K)).scratch_bytes;
 }
 
 extern "C" int t2sp_sgemm_f32(const float *A, const float *B, float *C, int M, int N, int K,
@@ -708,7 +765,10 @@ extern "C" int t2sp_sgemm_f32_tiled(const float *A, const float *B, float *C, in
 extern "C" size_t t2sp_sgemm_ex_workspace_bytes(int transa, int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     // the re-laid A of the transposed form (required), then the planes of a split reduction (optional)
-    return (transa ? (size_t)M * K * sizeof(float) : 0) + t2sp::plan_gemm(M, N, K).scratch_bytes;
+    const size_t pad_t = t2sp::gemm_pad_bytes(M, N, K, true), pad_n = t2sp::gemm_pad_bytes(M, N, K, false);
+    const size_t pad = (K % 4 || N % 4) ? (pad_t > pad_n ? pad_t : pad_n) : 0;
+    return t2sp::round_up256(transa ? (size_t)M * K * sizeof(float) : 0) + pad +
+           t2sp::plan_gemm(M, (int)t2sp::round_up4(N), (int)t2sp::round_up4(K)).scratch_bytes;
 }
 
 extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, float alpha, const float *A,
@@ -727,8 +787,9 @@ extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, fl
         if (rc != T2SP_OK) return rc;
         a = workspace;
         la = K;
-        workspace += (size_t)M * K;
-        workspace_bytes -= (size_t)M * K * sizeof(float);
+        const size_t relaid = t2sp::round_up256((size_t)M * K * sizeof(float));
+        workspace = relaid <= workspace_bytes ? workspace + relaid / sizeof(float) : nullptr;
+        workspace_bytes = relaid <= workspace_bytes ? workspace_bytes - relaid : 0;
     }
     t2sp::GemmArgs g{};
     g.A = a; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K;

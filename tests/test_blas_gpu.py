@@ -26,6 +26,28 @@ def test_alpha_beta_and_transposes(oracle, opa, opb, shape):
     assert rel_fro(t2sp_amd.gemm_ex(opa, opb, 1.0, 0.0, Aa, Bb), oracle.gemm(A, B))[0] <= TOL
 
 
+@pytest.mark.parametrize("opa,opb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("shape", [(1001, 1003, 1005), (640, 513, 2050), (77, 130, 257)])
+def test_odd_sizes_run_on_padded_copies(oracle, opa, opb, shape):
+    """K or N not a multiple of 4: the operands are multiplied as zero-padded, aligned copies (as the
+    reference's wrapper pads to tile multiples, blas-gemm.cpp:28-31); integer data, so the result is
+    exact whatever the order, with alpha, beta and C applied on the way out; inputs untouched."""
+    M, N, K = shape
+    rng = np.random.default_rng(5)
+    A = rng.integers(-2, 3, (M, K)).astype(np.float32)
+    B = rng.integers(-2, 3, (K, N)).astype(np.float32)
+    C = rng.integers(-4, 5, (M, N)).astype(np.float32)
+    ref = 2.0 * (A.astype(np.float64) @ B.astype(np.float64)) - 3.0 * C
+    Aa = np.ascontiguousarray(A.T) if opa else A
+    Bb = np.ascontiguousarray(B.T) if opb else B
+    keep = (Aa.copy(), Bb.copy(), C.copy())
+    got = t2sp_amd.gemm_ex(opa, opb, 2.0, -3.0, Aa, Bb, C)
+    assert (got == ref).all()
+    assert (Aa == keep[0]).all() and (Bb == keep[1]).all() and (C == keep[2]).all()
+    if not opa and not opb:
+        assert (t2sp_amd.gemm(A, B) == A.astype(np.float64) @ B.astype(np.float64)).all()
+
+
 def test_tiled_output_and_in_place_device(oracle):
     import torch
     M, N, K = 128, 96, 64
