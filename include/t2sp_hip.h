@@ -136,8 +136,9 @@ int t2sp_ssymv_f32_tiled(float alpha, float beta, const float *A, const float *x
 /* O[n,co,h,w] = sum_{ci,kh,kw} I[n,ci,h+kh,w+kw] * W[co,ci,kh,kw], stride 1, valid
  * padding, fp32.  si4/sw4/so4 are element strides of the logical indices
  * (n,ci,h,w), (co,ci,kh,kw), (n,co,h,w); "w" is the innermost spatial axis (the
- * one the reference calls y).  Dense NCHW/OIHW with OW % 4 == 0 takes the
- * implicit-GEMM MFMA kernel, anything else a scalar kernel.  `workspace` (optional, may be
+ * one the reference calls y).  Inputs and outputs with unit w stride, dense OIHW weights and
+ * OW >= 4 take the implicit-GEMM MFMA kernel (rows whose length is not a multiple of 4 are
+ * walked in groups of four whose last group overlaps its neighbour), anything else a scalar kernel.  `workspace` (optional, may be
  * NULL; t2sp_conv2d_workspace_bytes gives its size) holds the partial planes that let the tiles
  * left after whole rounds of 256 split their reduction over all CUs, and, when CI*KH*KW is not a
  * multiple of 4, the weights re-laid with zero-padded rows (without it such a shape takes the

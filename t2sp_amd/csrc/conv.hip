@@ -10,6 +10,10 @@
 //                 consecutive w of one (n,ci,h+kh) row, 4-byte aligned (kw shifts the start)
 //   * output   -> a lane ends up with 4 consecutive w of one (n,co,h) row: 128-bit stores
 // "w" is the innermost spatial axis of the buffers (the one the reference calls y).
+// Rows whose length OW is not a multiple of 4 (14 x 14, 7 x 7 maps) are walked in ceil(OW/4)
+// groups whose last one starts at OW-4: it overlaps its neighbour, the shared outputs are
+// computed twice to the same value, and every 128-bit access stays inside its row.  The pixel
+// index p then counts these groups ("padded" row length OWp = 4*ceil(OW/4)).
 #include "mfma_core.hpp"
 #include "gemm_loaders.hpp"
 #include "splitk.hpp"
@@ -26,7 +30,8 @@ struct ConvArgs {
     int si_n, si_c, si_h;       // input strides in elements (w stride is 1); the input spans < 2^31 elements
     int64_t sw_o;               // weight stride of co (ci,kh,kw are dense)
     int64_t so_n, so_c, so_h;   // output strides (w stride is 1)
-    int P, KRED;                // N*OH*OW, CI*KH*KW
+    int OWp;                    // OW rounded up to a multiple of 4: positions per row in the pixel index
+    int P, KRED;                // N*OH*OWp, CI*KH*KW
     int tiles_m, tiles_n, group_m;
     int p_begin;                // first output pixel this launch covers
     int splits;                 // workgroups per tile along the reduction (1 = none)
@@ -34,17 +39,24 @@ struct ConvArgs {
     float *scratch;
 };
 
+// Four outputs of one image row to memory; rows of a length that is not a multiple of 4 start
+// at any 4-byte boundary.
+__device__ __forceinline__ void conv_store4(float *dst, v4f v, bool ragged) {
+    if (ragged) *reinterpret_cast<v4f_u *>(dst) = v;
+    else *reinterpret_cast<v4f *>(dst) = v;
+}
+
 struct ConvOutMap {
     float *O;
-    int CO, P, OH, OW, p_begin;
+    int CO, P, OH, OW, OWp, p_begin;
     int64_t so_n, so_c, so_h;
     __device__ __forceinline__ void store(int row, int col, v4f v) const {
         const int p = p_begin + col;
         if (row >= CO || p >= P) return;
-        const int hw = OH * OW;
+        const int hw = OH * OWp;
         const int n = p / hw, rem = p - n * hw;
-        const int h = rem / OW, w = rem - h * OW;
-        *reinterpret_cast<v4f *>(O + n * so_n + row * so_c + h * so_h + w) = v;
+        const int h = rem / OWp, w = min(rem - h * OWp, OW - 4);
+        conv_store4(O + n * so_n + row * so_c + h * so_h + w, v, OW != OWp);
     }
 };
 
@@ -71,9 +83,9 @@ struct Im2colRcLoader {
             int p = p0 + s.col;
             col_ok[i] = !EDGE || p < g.P;
             if (!col_ok[i]) p = 0;
-            const int hw = g.OH * g.OW;
+            const int hw = g.OH * g.OWp;
             const int n = p / hw, rem = p - n * hw;
-            const int h = rem / g.OW, w = rem - h * g.OW;
+            const int h = rem / g.OWp, w = min(rem - h * g.OWp, g.OW - 4);
             base_off[i] = n * g.si_n + h * g.si_h + w;
             slot[i].init(wp, (k_begin + s.k < g.KRED) ? k_begin + s.k : 0);
         }
@@ -126,13 +138,14 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) conv_kernel(const ConvArgs g) {
         store_partial<Cfg>(acc, g.scratch, split, co0, p0 - g.p_begin, g.Mp, g.Np);
         return;
     }
-    const int hw = g.OH * g.OW;
+    const int hw = g.OH * g.OWp;
+    const bool ragged = g.OW != g.OWp;
     drain<Cfg>(acc, [&](int row, int col, v4f v) {
         const int co = co0 + row, p = p0 + col;
         if (EDGE && (co >= g.CO || p >= g.P)) return;
         const int n = p / hw, rem = p - n * hw;
-        const int h = rem / g.OW, w = rem - h * g.OW;
-        *reinterpret_cast<v4f *>(g.O + n * g.so_n + co * g.so_c + h * g.so_h + w) = v;
+        const int h = rem / g.OWp, w = min(rem - h * g.OWp, g.OW - 4);
+        conv_store4(g.O + n * g.so_n + co * g.so_c + h * g.so_h + w, v, ragged);
     });
 }
 
@@ -182,7 +195,7 @@ static int launch_conv(ConvArgs g, int p_begin, int p_end, int splits, float *sc
     hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * splits), dim3(Cfg::NTHREADS), smem, stream, g);
     if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
     if (splits > 1) {
-        ConvOutMap map{g.O, g.CO, g.P, g.OH, g.OW, p_begin, g.so_n, g.so_c, g.so_h};
+        ConvOutMap map{g.O, g.CO, g.P, g.OH, g.OW, g.OWp, p_begin, g.so_n, g.so_c, g.so_h};
         if (launch_splitk_reduce<true>(scratch, splits, g.Mp, g.Np, map, stream) != hipSuccess) return T2SP_ERR_LAUNCH;
     }
     return T2SP_OK;
@@ -284,7 +297,10 @@ extern "C" size_t t2sp_conv2d_workspace_bytes(int N, int CI, int CO, int OH, int
     if (N <= 0 || CI <= 0 || CO <= 0 || OH <= 0 || OW <= 0 || KH <= 0 || KW <= 0) return 0;
     if ((int64_t)N * OH * OW > INT32_MAX || (int64_t)CI * KH * KW > INT32_MAX) return 0;
     // padded weight rows when their length is not a multiple of 4, then the planes of a split rest
-    return t2sp::conv_padded_weight_bytes(CO, CI * KH * KW) + t2sp::plan_conv(CO, N * OH * OW, CI * KH * KW).scratch_bytes;
+    const int64_t owp = (OW + 3) / 4 * 4;
+    if ((int64_t)N * OH * owp > INT32_MAX) return 0;
+    return t2sp::conv_padded_weight_bytes(CO, CI * KH * KW) +
+           t2sp::plan_conv(CO, (int)(N * OH * owp), CI * KH * KW).scratch_bytes;
 }
 
 extern "C" int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, int CI, int CO,
@@ -317,10 +333,14 @@ extern "C" int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, 
         workspace += pad_bytes / sizeof(float);
         workspace_bytes -= pad_bytes;
     }
-    const bool fast = cfg != T2SP_CFG_SCALAR && si4[3] == 1 && so4[3] == 1 && w_dense && sw_o % 4 == 0 && OW % 4 == 0 &&
-                      (kred % 4 == 0 || padded) && KH * KW <= 4096 && in_span < INT32_MAX &&
-                      so4[0] % 4 == 0 && so4[1] % 4 == 0 && so4[2] % 4 == 0 &&
-                      ((uintptr_t)W % 16 == 0) && ((uintptr_t)O % 16 == 0) && ((uintptr_t)I % 4 == 0);
+    const int owp = (OW + 3) / 4 * 4;
+    const bool ragged = OW != owp;
+    // aligned 128-bit stores need rows that start on 16-byte boundaries; ragged rows use 4-byte aligned ones
+    const bool out_ok = so4[3] == 1 && (ragged ? ((uintptr_t)O % 4 == 0)
+                                                : (so4[0] % 4 == 0 && so4[1] % 4 == 0 && so4[2] % 4 == 0 && (uintptr_t)O % 16 == 0));
+    const bool fast = cfg != T2SP_CFG_SCALAR && si4[3] == 1 && out_ok && w_dense && sw_o % 4 == 0 && OW >= 4 &&
+                      (int64_t)N * OH * owp <= INT32_MAX && (kred % 4 == 0 || padded) && KH * KW <= 4096 &&
+                      in_span < INT32_MAX && ((uintptr_t)W % 16 == 0) && ((uintptr_t)I % 4 == 0);
     if (!fast) {
         ConvGenericArgs a{I, W_given, O, N, CI, CO, OH, OW, KH, KW, {}, {}, {}};
         for (int d = 0; d < 4; d++) { a.si[d] = si4[d]; a.sw[d] = sw4[d]; a.so[d] = so4[d]; }
@@ -335,7 +355,8 @@ extern "C" int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, 
     g.si_n = (int)si4[0]; g.si_c = (int)si4[1]; g.si_h = (int)si4[2];
     g.sw_o = sw_o;
     g.so_n = so4[0]; g.so_c = so4[1]; g.so_h = so4[2];
-    g.P = N * OH * OW; g.KRED = CI * KH * KW;
+    g.OWp = owp;
+    g.P = N * OH * owp; g.KRED = CI * KH * KW;
     switch (cfg) {
         case T2SP_CFG_256x256: return launch_conv<ConvL>(g, 0, g.P, 1, nullptr, st);
         case T2SP_CFG_128x128: return launch_conv<ConvM>(g, 0, g.P, 1, nullptr, st);

@@ -86,7 +86,7 @@ static int conv_impl(halide_buffer_t *I, halide_buffer_t *K, halide_buffer_t *O,
     const int64_t IW = OW + KW - 1, IH = OH + KH - 1;
     li.ext[0] = N; li.ext[1] = CI; li.ext[2] = IH; li.ext[3] = IW;
     lk.ext[0] = CO; lk.ext[1] = CI; lk.ext[2] = KH; lk.ext[3] = KW;
-    if (N * OH * OW > INT32_MAX || CI * KH * KW > INT32_MAX)
+    if (N * OH * ((OW + 3) / 4 * 4) > INT32_MAX || CI * KH * KW > INT32_MAX)
         return report(halide_error_code_buffer_extents_too_large, op, "problem too large for 32-bit tile indices");
 
     Staged di, dk, dout;
@@ -103,9 +103,12 @@ static int conv_impl(halide_buffer_t *I, halide_buffer_t *K, halide_buffer_t *O,
         float **p[3];
         ~Release() { for (auto q : p) if (*q) pool().put(*q); }
     } release{{&tmp_i, &tmp_k, &tmp_o}};
-    const bool out_direct = O->dimensions == 4 && od[0].stride == 1 && OW % 4 == 0 && od[1].stride % 4 == 0 &&
-                            od[2].stride % 4 == 0 && od[3].stride % 4 == 0 && ((uintptr_t)dout.ptr() % 16 == 0);
-    const bool fast_shape = OW % 4 == 0 && (CI * KH * KW) % 4 == 0;
+    // rows of a length that is not a multiple of 4 are stored with 4-byte aligned accesses, others
+    // need 16-byte aligned rows
+    const bool out_direct = O->dimensions == 4 && od[0].stride == 1 &&
+                            (OW % 4 != 0 || (od[1].stride % 4 == 0 && od[2].stride % 4 == 0 && od[3].stride % 4 == 0 &&
+                                             ((uintptr_t)dout.ptr() % 16 == 0)));
+    const bool fast_shape = OW >= 4;
     Logical4 ci4 = li, ck4 = lk;
     if (fast_shape && cfg != T2SP_CFG_SCALAR) {
         if (li.str[3] != 1) {

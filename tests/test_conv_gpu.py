@@ -74,6 +74,22 @@ def test_odd_reduction_length_takes_padded_weights(oracle, shape):
     assert rel_fro(run(If, Wf), oracle.conv(If, Wf))[0] <= TOL
 
 
+@pytest.mark.parametrize("shape", [(2, 16, 32, 9, 14, 3, 3), (3, 8, 24, 5, 7, 3, 3), (1, 16, 16, 6, 5, 1, 1), (2, 3, 8, 10, 13, 5, 5),
+                                   (16, 64, 256, 14, 14, 3, 3), (64, 32, 128, 7, 7, 3, 3)])
+def test_rows_not_a_multiple_of_four(oracle, shape):
+    """Innermost output extent 14, 7, 5, 13: rows are walked in groups of four whose last group
+    overlaps its neighbour; integer data (exact in any order) and uniform data, and twice the same bits."""
+    N, CI, CO, OX, OY, KX, KY = shape          # OY is the innermost extent
+    rng = np.random.default_rng(17)
+    I = rng.integers(-2, 3, (N, CI, OY + KY - 1, OX + KX - 1)).astype(np.float32)
+    W = rng.integers(-2, 3, (CO, CI, KY, KX)).astype(np.float32)
+    assert (run(I, W) == oracle.conv(I, W)).all()
+    If, Wf = oracle.fill_uniform(I.shape, 18), oracle.fill_uniform(W.shape, 19)
+    got = run(If, Wf)
+    assert rel_fro(got, oracle.conv(If, Wf))[0] <= TOL
+    assert (run(If, Wf) == got).all()
+
+
 # (N, CI, CO, OY, OX): sizes at which the automatic plan takes, in turn: whole rounds of 128 x 128
 # tiles and a split rest; a rest only (one image); 64-row tiles for few output channels; two tile rows
 # of 256 with whole rounds of 128 x 128 and a split rest; whole rounds of 256 x 256 and a rest
