@@ -105,7 +105,7 @@ def mttkrp_config5(torch, steps, warmup, peak):
 
 
 def ssyrk_case(torch, steps, warmup, peak, N, K, note):
-    """Not a BASELINE configuration: the SYRK pipeline (t2s/tests/performance/syrk) at the headline
+    """Not one of the headline benchmark configurations: the SYRK pipeline (t2s/tests/performance/syrk) at the headline
     GEMM size and at the size the reference's BLAS release is built for.  Only the tiles on or above the diagonal are multiplied; the rate counts the
     N*(N+1)/2 distinct outputs (N*(N+1)*K flop).  The reference's own report counts 2*N*N*K
     (syrk-run-fpga.cpp:99), given as `TFLOP/s_reference_count`."""
@@ -129,7 +129,7 @@ def ssyrk_case(torch, steps, warmup, peak, N, K, note):
 
 
 def sger_8192(torch, steps, warmup, peak):
-    """Not a BASELINE configuration: the GER pipeline (t2s/tests/performance/ger) on an 8192 x 8192
+    """Not one of the headline benchmark configurations: the GER pipeline (t2s/tests/performance/ger) on an 8192 x 8192
     matrix.  It moves 8 bytes per element (A in, Out out; x and y are negligible) for 2 flop, so its
     roof is HBM bandwidth (8 TB/s), reported next to the flop rate."""
     L = lib()
@@ -151,7 +151,7 @@ def sger_8192(torch, steps, warmup, peak):
 
 
 def sgbmv3_case(torch, steps, warmup, peak):
-    """Not a BASELINE configuration: the GBMV pipeline (t2s/tests/performance/gbmv3) with the band
+    """Not one of the headline benchmark configurations: the GBMV pipeline (t2s/tests/performance/gbmv3) with the band
     width of gbmv3-run-fpga.cpp:29-30 (Ku = Kl = 511, rows padded to 1024) and 131072 rows, so that
     the band (512 MiB) does not fit the caches.  4 bytes of A per 2 flop: the roof is HBM."""
     L = lib()
@@ -173,7 +173,7 @@ def sgbmv3_case(torch, steps, warmup, peak):
 
 
 def ssymv_case(torch, steps, warmup, peak):
-    """Not a BASELINE configuration: the SYMV pipeline (t2s/tests/performance/symv) on a 16384 x 16384
+    """Not one of the headline benchmark configurations: the SYMV pipeline (t2s/tests/performance/symv) on a 16384 x 16384
     matrix.  Only the triangle col <= row is read (N*(N+1)/2 elements, 4 flop each): the roof is HBM."""
     L = lib()
     N = 16384

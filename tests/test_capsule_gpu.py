@@ -85,7 +85,7 @@ def test_direct_kernels_other_batches(oracle, cfg, n):
 
 
 def test_config4_full_size(oracle):
-    """BASELINE config 4: N=32, CI=CO=32, 15x15 -> 7x7, 3x3, stride 2, on the device, whole
+    """benchmark configuration 4: N=32, CI=CO=32, 15x15 -> 7x7, 3x3, stride 2, on the device, whole
     result against the oracle."""
     import torch
     P = t2sp_amd.fill_uniform(torch.empty(32, 32, 15, 15, 4, 4, device="cuda"), 41)

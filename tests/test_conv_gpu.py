@@ -161,7 +161,7 @@ def test_packed_inputs_need_tiled_output():
 
 
 def test_config3_full_size_sampled_and_shift_property(oracle):
-    """BASELINE config 3 on the device: N=64, CI=CO=256, 56x56 output, 3x3.  The oracle checks two
+    """benchmark configuration 3 on the device: N=64, CI=CO=256, 56x56 output, 3x3.  The oracle checks two
     images x 24 channels; a one-hot kernel gives an exact shifted copy of the whole input."""
     import torch
     N, C, OH = 64, 256, 56

@@ -32,7 +32,7 @@ def detile(Ct):
 
 @pytest.mark.parametrize("cfg", CFGS)
 def test_config1_1024_cubed_seed0_host_buffers(oracle, cfg):
-    """BASELINE config 1: M=N=K=1024, uniform[-1,1) from seed 0, host buffers in and out."""
+    """benchmark configuration 1: M=N=K=1024, uniform[-1,1) from seed 0, host buffers in and out."""
     A, B = oracle.fill_uniform((1024, 1024), 0), oracle.fill_uniform((1024, 1024), 1)
     ref = oracle.gemm(A, B)
     C = t2sp_amd.gemm(A, B, cfg=cfg)
@@ -263,7 +263,7 @@ def test_empty_extents():
 
 @pytest.mark.parametrize("shape", [(8192, 8192, 8192), (4096, 16384, 2048), (16384, 4096, 8192)])
 def test_config2_full_size_sampled_rows_and_identity(oracle, torch_cuda, shape):
-    """BASELINE config 2 at full size, on the device.  The oracle checks 48 sampled rows;
+    """benchmark configuration 2 at full size, on the device.  The oracle checks 48 sampled rows;
     the whole result is covered by a size-independent property: A @ I == A exactly."""
     torch = torch_cuda
     M, N, K = shape

@@ -78,7 +78,7 @@ def test_thin_layer_takes_any_strides(oracle):
 
 
 def test_config5_full_size_sampled_rows_and_rank1(oracle):
-    """BASELINE config 5: I=J=K=512, R=256 on the device.  The oracle checks 24 sampled rows; a
+    """benchmark configuration 5: I=J=K=512, R=256 on the device.  The oracle checks 24 sampled rows; a
     rank-1 integer tensor gives an exact closed form for the whole result."""
     import torch
     I = J = K = 512
