@@ -204,6 +204,7 @@ __global__ void mttkrp_scalar_kernel(const MttkrpGenericArgs g) {
 using MttL = TileCfg<256, 256, 16, 4, 2, STYLE_KC>;   // 8 waves, 64x128 per wave
 using MttM = TileCfg<128, 128, 16, 2, 2, STYLE_KC>;   // 4 waves, 64x64 per wave
 using MttS = TileCfg<64, 64, 16, 2, 1, STYLE_KC>;     // 2 waves, 32x64 per wave
+using MttW = TileCfg<256, 64, 16, 4, 1, STYLE_KC>;    // 4 waves, 64x64 per wave: small ranks (hint id T2SP_CFG_32x128)
 
 struct MttkrpPlan {
     int cfg, splits, Mp, Np;
@@ -212,10 +213,21 @@ struct MttkrpPlan {
 
 static MttkrpPlan plan_mttkrp(int I, int J, int K, int R, int cfg, int splits) {
     MttkrpPlan p{};
-    if (cfg == T2SP_CFG_AUTO)
-        cfg = (I >= 256 && R >= 256) ? T2SP_CFG_256x256 : (I >= 128 && R >= 128) ? T2SP_CFG_128x128 : T2SP_CFG_64x128;
-    const int bm = cfg == T2SP_CFG_256x256 ? 256 : cfg == T2SP_CFG_128x128 ? 128 : 64;
-    const int bn = bm;
+    struct Cand { int cfg, bm, bn; double eff; };
+    // sustained fraction of the 256 x 256 tile's rate, measured
+    const Cand cands[4] = {{T2SP_CFG_256x256, 256, 256, 1.0}, {T2SP_CFG_128x128, 128, 128, 0.93},
+                           {T2SP_CFG_32x128, 256, 64, 0.85}, {T2SP_CFG_64x128, 64, 64, 0.7}};
+    if (cfg == T2SP_CFG_AUTO) {
+        // least padded work over sustained rate: a rank of 64 in 256-wide tiles would multiply 4x too much
+        double best = 1e300;
+        for (const Cand &c : cands) {
+            const double cost = (double)((I + c.bm - 1) / c.bm * c.bm) * ((R + c.bn - 1) / c.bn * c.bn) / c.eff;
+            if (cost < best) { best = cost; cfg = c.cfg; }
+        }
+    }
+    int bm = 64, bn = 64;
+    for (const Cand &c : cands)
+        if (c.cfg == cfg) { bm = c.bm; bn = c.bn; }
     const int tiles = ((I + bm - 1) / bm) * ((R + bn - 1) / bn);
     const int64_t ktiles = (int64_t)K * (J / 16);
     if (splits <= 0) {
@@ -292,6 +304,7 @@ extern "C" int t2sp_mttkrp_f32(const float *B, const float *C, const float *D, f
         case T2SP_CFG_256x256: return launch_mttkrp<MttL>(g, (hipStream_t)stream);
         case T2SP_CFG_128x128: return launch_mttkrp<MttM>(g, (hipStream_t)stream);
         case T2SP_CFG_64x128: return launch_mttkrp<MttS>(g, (hipStream_t)stream);
+        case T2SP_CFG_32x128: return launch_mttkrp<MttW>(g, (hipStream_t)stream);
         default: return T2SP_ERR_SHAPE;
     }
 }

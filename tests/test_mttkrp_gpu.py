@@ -17,13 +17,26 @@ def run(B, C, D, cfg=0, splits=0):
     return t2sp_amd.mttkrp(*t2sp_amd.mttkrp_reference_layout(B, C, D), cfg=cfg, splits=splits)
 
 
-@pytest.mark.parametrize("cfg,splits", [(0, 0), (1, 1), (1, 4), (2, 3), (3, 2), (99, 0)])
+@pytest.mark.parametrize("cfg,splits", [(0, 0), (1, 1), (1, 4), (2, 3), (3, 2), (4, 1), (4, 5), (99, 0)])
 def test_small_parity_two_step_order(oracle, cfg, splits):
     B, C, D = oracle.fill_uniform((256, 64, 24), 1), oracle.fill_uniform((64, 256), 2), oracle.fill_uniform((24, 256), 3)
     got = run(B, C, D, cfg, splits)
     err, mx = rel_fro(got, oracle.mttkrp(B, C, D))
     assert err <= TOL, (cfg, splits, err, mx)
     assert rel_fro(got, oracle.mttkrp(B, C, D, acc=oracle.ACC_F32_FMA))[0] <= TOL
+
+
+@pytest.mark.parametrize("R", [16, 64, 96, 128, 192])
+def test_small_ranks_pick_narrow_tiles(oracle, R):
+    """Ranks below the 256-wide tile: the automatic choice (a 256 x 64 tile for R <= 64) against the
+    oracle, integer data exact."""
+    B, C, D = oracle.fill_uniform((256, 32, 40), 21), oracle.fill_uniform((32, R), 22), oracle.fill_uniform((40, R), 23)
+    assert rel_fro(run(B, C, D), oracle.mttkrp(B, C, D))[0] <= TOL
+    rng = np.random.default_rng(3)
+    Bi = rng.integers(-2, 3, (256, 32, 40)).astype(np.float32)
+    Ci, Di = rng.integers(-2, 3, (32, R)).astype(np.float32), rng.integers(-2, 3, (40, R)).astype(np.float32)
+    want = np.einsum("ijk,jr,kr->ir", Bi.astype(np.float64), Ci, Di)
+    assert (run(Bi, Ci, Di) == want).all()
 
 
 def test_literal_reference_buffers(oracle):
