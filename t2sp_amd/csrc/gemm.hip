@@ -75,14 +75,22 @@ struct GemmOutMap {
 };
 
 // The same for compact planes: column `col` of a plane belongs to tile col / BN of the launch.
-template <int BM, int BN>
+// ALONG_COLS: v = D[row][col..col+3] (B row-major); else v = D[row..row+3][col] (B stored transposed).
+template <int BM, int BN, bool ALONG_COLS>
 struct GemmCompactMap {
     GemmOutMap inner;
     __device__ __forceinline__ void store(int row, int col, v4f v) const {
         const int t = col / BN;
         int tm, tn;
         tile_of_position(inner.g.tile_first + t, inner.g.tiles_m, inner.g.tiles_n, inner.g.group_m, tm, tn);
-        inner.store(tm * BM + row, tn * BN + (col - t * BN), v);
+        const int r = tm * BM + row, c = tn * BN + (col - t * BN);
+        if (ALONG_COLS) {
+            inner.store(r, c, v);
+        } else if (c < inner.g.N) {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (r + e < inner.g.M) gemm_store1(inner.g, r + e, c, v[e]);
+        }
     }
 };
 
@@ -102,8 +110,12 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) sgemm_kernel(const GemmArgs g) 
     RowMajorKcLoader<Cfg, EDGE> la(g.A, g.lda, m0, g.M, g.K, kt0 * Cfg::BK);
     Accum<Cfg> acc;
     if constexpr (BT) {
-        RowMajorKcLoaderB<Cfg, EDGE> lb(g.B, g.ldb, n0, g.N, g.K);
-        mainloop<Cfg>(acc, la, lb, ktiles_even<Cfg>(g.K), smem);
+        RowMajorKcLoaderB<Cfg, EDGE> lb(g.B, g.ldb, n0, g.N, g.K, kt0 * Cfg::BK);
+        mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem);
+        if (g.splits > 1) {   // only in compact form
+            store_partial<Cfg>(acc, g.scratch, split, 0, tile * Cfg::BN, Cfg::BM, g.tile_count * Cfg::BN);
+            return;
+        }
         drain<Cfg>(acc, [&](int row, int col, v4f v) {   // v = D[row..row+3][col]
             const int c = n0 + col;
             if (EDGE && c >= g.N) return;
@@ -484,7 +496,7 @@ static int launch(GemmArgs g, hipStream_t stream, int splits = 1, float *scratch
                             (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
     const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
-    if (!BT && phased && splits == 1) {
+    if (phased && splits == 1) {
         GemmPhases p = plan_phases(tiles, g.K, Cfg::BK, Cfg::BM, Cfg::BN, true);
         if (scratch && scratch_bytes >= p.scratch_bytes) {
             for (int i = 0; i < p.n; i++) {
@@ -495,8 +507,8 @@ static int launch(GemmArgs g, hipStream_t stream, int splits = 1, float *scratch
                 hipLaunchKernelGGL(kern, dim3((unsigned)(g.tile_count * g.splits)), dim3(Cfg::NTHREADS), smem, stream, g);
                 if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
                 if (g.splits > 1) {
-                    GemmCompactMap<Cfg::BM, Cfg::BN> map{GemmOutMap{g}};
-                    if (launch_splitk_reduce<true>(scratch, g.splits, Cfg::BM, g.tile_count * Cfg::BN, map, stream) != hipSuccess)
+                    GemmCompactMap<Cfg::BM, Cfg::BN, !BT> map{GemmOutMap{g}};
+                    if (launch_splitk_reduce<!BT>(scratch, g.splits, Cfg::BM, g.tile_count * Cfg::BN, map, stream) != hipSuccess)
                         return T2SP_ERR_LAUNCH;
                 }
             }
@@ -702,9 +714,9 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         const GemmPlan p = plan_gemm(g.M, g.N, g.K);
         cfg = p.cfg;
         if (!bt && p.splits > 1 && workspace && workspace_bytes >= p.scratch_bytes) splits = p.splits;
-        phased = !bt && p.phased && workspace && workspace_bytes >= p.scratch_bytes;
+        phased = p.phased && workspace && workspace_bytes >= p.scratch_bytes;
         // without room for the planes the last round runs unsplit: then the finer tiles waste less of it
-        if (!bt && p.phased && !phased) {
+        if (p.phased && !phased) {
             const int64_t t256 = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
             const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
             const double cl = (double)((t256 + 255) / 256) * 65536.0, cm = (double)((t128 + 255) / 256) * 16384.0 / 0.94;
@@ -713,8 +725,8 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
     }
     if (bt) {
         switch (cfg) {
-            case T2SP_CFG_256x256: return launch<GemmLT, true>(g, stream);
-            case T2SP_CFG_128x128: return launch<GemmMT, true>(g, stream);
+            case T2SP_CFG_256x256: return launch<GemmLT, true>(g, stream, 1, workspace, workspace_bytes, phased);
+            case T2SP_CFG_128x128: return launch<GemmMT, true>(g, stream, 1, workspace, workspace_bytes, phased);
             case T2SP_CFG_64x128:
             case T2SP_CFG_32x128: return launch<GemmST, true>(g, stream);
             default: return T2SP_ERR_SHAPE;

@@ -48,6 +48,39 @@ def test_odd_sizes_run_on_padded_copies(oracle, opa, opb, shape):
         assert (t2sp_amd.gemm(A, B) == A.astype(np.float64) @ B.astype(np.float64)).all()
 
 
+@pytest.mark.parametrize("shape", [(3072, 3072, 2048), (6144, 6144, 4096), (5120, 5120, 512)])
+def test_partial_last_round_split_both_forms_of_b(oracle, shape):
+    """Tile counts that are not a multiple of 256, B row-major and B stored transposed, with alpha,
+    beta and C updated in place: the tiles left after whole rounds split their reduction when the
+    workspace is there.  Against the run without a workspace and, on sampled rows, the oracle."""
+    import torch
+    M, N, K = shape
+    L = t2sp_amd.lib()
+    A = t2sp_amd.fill_uniform(torch.empty(M, K, device="cuda"), 31)
+    B = t2sp_amd.fill_uniform(torch.empty(K, N, device="cuda"), 32)
+    C0 = t2sp_amd.fill_uniform(torch.empty(M, N, device="cuda"), 33)
+    Bt = B.t().contiguous()
+    a, b, c0 = A.cpu().numpy(), B.cpu().numpy(), C0.cpu().numpy()
+    rows = np.unique(np.concatenate([[0, M - 1, M - 2, M - 130, M - 300], np.random.default_rng(2).integers(0, M, 6)]))
+    want = 1.5 * oracle.gemm(a[rows], b) - 0.5 * c0[rows]
+    for transb, Bd, ldb in ((0, B, N), (1, Bt, K)):
+        nbytes = L.t2sp_sgemm_ex_workspace_bytes(0, M, N, K)
+        assert nbytes > 0
+        ws = torch.empty(nbytes // 4, device="cuda")
+        outs = []
+        for w, nb in ((None, 0), (ws.data_ptr(), nbytes)):
+            C = C0.clone()
+            rc = L.t2sp_sgemm_ex_f32(0, transb, M, N, K, 1.5, A.data_ptr(), K, Bd.data_ptr(), ldb, -0.5, C.data_ptr(), N,
+                                     C.data_ptr(), N, 0, w, nb, None)
+            assert rc == 0
+            torch.cuda.synchronize()
+            outs.append(C)
+        plain, split = outs
+        assert (plain - split).abs().max().item() <= 1.6e-5 * plain.abs().max().item()
+        assert not torch.equal(plain, split)
+        assert rel_fro(split[rows].cpu().numpy(), want)[0] <= TOL
+
+
 def test_tiled_output_and_in_place_device(oracle):
     import torch
     M, N, K = 128, 96, 64
