@@ -118,13 +118,17 @@ static_assert(offsetof(halide_buffer_t, dim) == 40, "dim at 40");
  * Halide::Runtime::Buffer<float> (Halide/src/runtime/HalideBuffer.h:1050-1061:
  * raw_buffer() and the implicit conversion to halide_buffer_t*) for the subset
  * those drivers use: dense allocation, operator() element access, extents. */
+#include <cstring>
 #include <initializer_list>
+#include <new>
 #include <vector>
+extern "C" void *t2sp_host_malloc(size_t bytes);
+extern "C" void t2sp_host_free(void *p);
 namespace t2sp {
 template <typename T>
 class Buffer {
     static_assert(sizeof(T) == 4, "only 32-bit element types are used on this path");
-    std::vector<T> storage_;
+    T *storage_ = nullptr;           // from t2sp_host_malloc: page-locked when a device is present
     std::vector<halide_dimension_t> dims_;
     halide_buffer_t buf_;
 
@@ -138,10 +142,14 @@ class Buffer {
             dims_[d].flags = 0;
             stride *= ext[d];
         }
-        if (!external) storage_.assign((size_t)stride, T(0));
+        if (!external) {
+            storage_ = static_cast<T *>(t2sp_host_malloc((size_t)stride * sizeof(T) + 1));
+            if (!storage_) throw std::bad_alloc();
+            std::memset(storage_, 0, (size_t)stride * sizeof(T));
+        }
         buf_.device = 0;
         buf_.device_interface = nullptr;
-        buf_.host = (uint8_t *)(external ? external : storage_.data());
+        buf_.host = (uint8_t *)(external ? external : storage_);
         buf_.flags = 0;
         buf_.type.code = halide_type_float;
         buf_.type.bits = 32;
@@ -158,6 +166,7 @@ public:
         init(ext, 1 + (int)sizeof...(rest), nullptr);
     }
     Buffer(T *data, const std::vector<int> &ext) { init(ext.data(), (int)ext.size(), data); }
+    ~Buffer() { t2sp_host_free(storage_); }
     Buffer(const Buffer &) = delete;
     Buffer &operator=(const Buffer &) = delete;
 

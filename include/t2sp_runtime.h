@@ -2,6 +2,7 @@
  * entry points.  They stand in for pieces of t2s/src/AOT-OpenCL-Runtime.cpp. */
 #ifndef T2SP_RUNTIME_H
 #define T2SP_RUNTIME_H
+#include <stddef.h>
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -17,6 +18,13 @@ double t2sp_last_kernel_ns(void);
 /* Frees the cached device allocations the entry points keep between calls
  * (counterpart of halide_device_and_host_free, AOT-OpenCL-Runtime.cpp:280-295). */
 void t2sp_release(void);
+
+/* Host memory for operator arguments: page-locked when a device is present, so that the copies
+ * the entry points make run at the full rate of the link, and 64-byte aligned in every case.
+ * Counterpart of halide_malloc / halide_free (t2s/src/AOT-OpenCL-Runtime.cpp:56-72).
+ * t2sp_host_free takes NULL or a pointer t2sp_host_malloc returned. */
+void *t2sp_host_malloc(size_t bytes);
+void t2sp_host_free(void *p);
 
 /* Number of HIP devices visible; 0 when there is none. */
 int t2sp_device_count(void);

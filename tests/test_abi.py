@@ -146,3 +146,22 @@ def test_python_mirror_raises_with_code():
     with pytest.raises(t2sp_amd.T2spError) as e:
         t2sp_amd.gemm(np.zeros((8, 4), np.float32), np.zeros((5, 12), np.float32))
     assert e.value.code == -8
+
+
+def test_host_allocation_is_aligned_and_survives_views():
+    """t2sp_host_malloc without a device: ordinary 64-byte aligned memory; the numpy wrapper keeps it
+    alive for as long as any view exists."""
+    import gc
+    L = t2sp_amd.lib()
+    p = L.t2sp_host_malloc(1000)
+    assert p and p % 64 == 0
+    L.t2sp_host_free(p)
+    L.t2sp_host_free(None)
+    a = t2sp_amd.host_empty((4, 6))
+    assert a.dtype == np.float32 and a.shape == (4, 6) and a.ctypes.data % 64 == 0
+    a[...] = 3.0
+    v = a[2:, 1::2]
+    del a
+    gc.collect()
+    assert (v == 3.0).all()
+    assert t2sp_amd.host_empty((0, 5)).shape == (0, 5)
