@@ -133,6 +133,21 @@ int t2sp_ssymv_f32_tiled(float alpha, float beta, const float *A, const float *x
                          int64_t lda, int kkk, int kk, const int64_t *strides3, float *workspace,
                          size_t workspace_bytes, void *stream);
 
+/* PairHMM forward probabilities of every (haplotype, read) pair:
+ *   M(i,j) = alpha*M(i-1,j-1) + beta*(I(i-1,j-1) + D(i-1,j-1)),  I(i,j) = delta*M(i-1,j) + eta*I(i-1,j),
+ *   D(i,j) = zeta*M(i,j-1) + eta*D(i,j-1),  out = sum_j M(last,j) + I(last,j)
+ * with alpha/beta = the match or the gap value of read position i by whether R[i] == H[j]
+ * (t2s/tests/performance/pairhmm/pairhmm.cpp:72-91).  H: uint8, haplotype index contiguous,
+ * `h_stride` elements between positions; R and the seven float32 probability arrays: position
+ * contiguous, `r_stride` elements between reads.  O(hh, rr, h, r) with element strides so4
+ * (haplotype = h*hh_extent + hh, read = r*rr_extent + rr; pairhmm-run-fpga.cpp:112).
+ * read_len <= 256, hap_len >= 2.  Vector arithmetic along anti-diagonals, no MFMA; the unit of
+ * work is the cell (num_haps*hap_len*num_reads*read_len cells per call). */
+int t2sp_pairhmm_f32(const uint8_t *H, const uint8_t *R, const float *delta, const float *zeta, const float *eta,
+                     const float *alpha_match, const float *alpha_gap, const float *beta_match,
+                     const float *beta_gap, float *O, int num_haps, int hap_len, int num_reads, int read_len,
+                     int64_t h_stride, int64_t r_stride, int hh, int rr, const int64_t *so4, void *stream);
+
 /* O[n,co,h,w] = sum_{ci,kh,kw} I[n,ci,h+kh,w+kw] * W[co,ci,kh,kw], stride 1, valid
  * padding, fp32.  si4/sw4/so4 are element strides of the logical indices
  * (n,ci,h,w), (co,ci,kh,kw), (n,co,h,w); "w" is the innermost spatial axis (the

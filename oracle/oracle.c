@@ -36,6 +36,11 @@
  *                                 and, past one block of II rows, add the elements above the
  *                                 diagonal on top of the finished row sum; the driver never asserts
  *                                 on them (symv-run-fpga.cpp:97-98), so the golden loop is the oracle.
+ *   oracle_pairhmm   golden       t2s/tests/performance/pairhmm/pairhmm-run-fpga.cpp:125-147 (column by
+ *                                 column over j, rows i inside; golden += M + I on the last row in
+ *                                 ascending j), the recurrence of pairhmm.cpp:72-91.  Only two columns
+ *                                 are kept instead of the driver's full matrices; the arithmetic and
+ *                                 its order are the driver's.
  *   oracle_mttkrp    golden       t2s/tests/performance/util/util.h:498-515 (two-step: TTM over l
  *                                 into e(i,j,k), then d += e*b over k).  The reference's outer loop
  *                                 bound `i < K` (util.h:502) is only right when I == K; this
@@ -457,6 +462,61 @@ void oracle_symv(float alpha, float beta, const float *A, const float *x, const 
             O[i] = t + u;
         }
     }
+}
+
+/* out[r * num_haps + h] = forward probability of read r against haplotype h.
+ * H: [hap_len][num_haps] characters (haplotype index contiguous); R and the probabilities:
+ * [num_reads][read_len] (pairhmm-run-fpga.cpp:58-61).  acc = ORACLE_ACC_F32: products and sums
+ * rounded separately, as the driver's loop is written; ORACLE_ACC_F32_FMA: the first product of
+ * each expression fused into the sum (fmaf(alpha, M, beta*(I+D)) and likewise for I and D). */
+void oracle_pairhmm(const unsigned char *H, const unsigned char *R, const float *delta, const float *zeta,
+                    const float *eta, const float *am, const float *ag, const float *bm, const float *bg,
+                    float *out, int64_t num_haps, int64_t hap_len, int64_t num_reads, int64_t read_len, int acc,
+                    int threads) {
+    set_threads(threads);
+#pragma omp parallel for schedule(dynamic, 16) collapse(2)
+    for (int64_t r = 0; r < num_reads; r++)
+        for (int64_t h = 0; h < num_haps; h++) {
+            /* previous and current column of M, I, D: [2][3][read_len] */
+            float *col = (float *)malloc((size_t)6 * read_len * sizeof(float));
+            float *pM = col, *pI = col + read_len, *pD = col + 2 * read_len;
+            float *cM = col + 3 * read_len, *cI = col + 4 * read_len, *cD = col + 5 * read_len;
+            const int64_t q = r * read_len;
+            float golden = 0.0f;
+            for (int64_t j = 0; j < hap_len; j++) {
+                for (int64_t i = 0; i < read_len; i++) {
+                    if (j == 0) { cM[i] = 0.0f; cI[i] = 0.0f; cD[i] = 0.0f; }
+                    if (i == 0) { cM[0] = 0.0f; cI[0] = 0.0f; cD[0] = (float)(1.0 / (double)(hap_len - 1)); }
+                    if (j != 0 && i != 0) {
+                        const int match = R[q + i] == H[j * num_haps + h];
+                        const float alpha = match ? am[q + i] : ag[q + i], beta = match ? bm[q + i] : bg[q + i];
+                        if (acc == ORACLE_ACC_F32_FMA) {
+                            cM[i] = fmaf(alpha, pM[i - 1], beta * (pI[i - 1] + pD[i - 1]));
+                            cI[i] = fmaf(delta[q + i], cM[i - 1], eta[q + i] * cI[i - 1]);
+                            cD[i] = fmaf(zeta[q + i], pM[i], eta[q + i] * pD[i]);
+                        } else {
+                            const float t = pI[i - 1] + pD[i - 1];
+                            const float a1 = alpha * pM[i - 1], a2 = beta * t;
+                            cM[i] = a1 + a2;
+                            const float b1 = delta[q + i] * cM[i - 1], b2 = eta[q + i] * cI[i - 1];
+                            cI[i] = b1 + b2;
+                            const float c1 = zeta[q + i] * pM[i], c2 = eta[q + i] * pD[i];
+                            cD[i] = c1 + c2;
+                        }
+                    }
+                    if (i == read_len - 1 && j > 0) {
+                        const float u = cM[i] + cI[i];
+                        golden += u;
+                    }
+                }
+                float *t;
+                t = pM; pM = cM; cM = t;
+                t = pI; pI = cI; cI = t;
+                t = pD; pD = cD; cD = t;
+            }
+            out[r * num_haps + h] = golden;
+            free(col);
+        }
 }
 
 int oracle_max_threads(void) { return omp_get_max_threads(); }

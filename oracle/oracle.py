@@ -53,6 +53,9 @@ def lib():
         _lib.oracle_gbmv3.restype = None
         _lib.oracle_symv.argtypes = [f32, f32, fp, fp, fp, fp, i64, i64, ctypes.c_int, ctypes.c_int]
         _lib.oracle_symv.restype = None
+        up = ctypes.POINTER(ctypes.c_ubyte)
+        _lib.oracle_pairhmm.argtypes = [up, up] + [fp] * 8 + [i64] * 4 + [ctypes.c_int, ctypes.c_int]
+        _lib.oracle_pairhmm.restype = None
         _lib.oracle_max_threads.restype = ctypes.c_int
         for f in (_lib.oracle_fill_uniform, _lib.oracle_gemm, _lib.oracle_gemm_literal,
                   _lib.oracle_conv, _lib.oracle_capsule, _lib.oracle_mttkrp,
@@ -315,6 +318,57 @@ def symv(A, x, y, alpha=1.0, beta=1.0, acc=ACC_F32, threads=0):
     O = np.empty(N, dtype=np.float32)
     lib().oracle_symv(alpha, beta, _p(A), _p(x), _p(y), _p(O), N, N, acc, threads)
     return O
+
+
+def pairhmm(H, R, delta, zeta, eta, alpha_match, alpha_gap, beta_match, beta_gap, acc=ACC_F32, threads=0):
+    """Forward probability of every (read, haplotype) pair by the driver's golden loop
+    (pairhmm-run-fpga.cpp:125-147).  H: uint8 (HAP_LEN, NUM_HAPS) -- numpy order of the reference's
+    Buffer(NUM_HAPS, HAP_LEN); R: uint8 (NUM_READS, READ_LEN); the probabilities float32
+    (NUM_READS, READ_LEN).  Returns float32 (NUM_READS, NUM_HAPS)."""
+    H, R = np.ascontiguousarray(H, dtype=np.uint8), np.ascontiguousarray(R, dtype=np.uint8)
+    probs = [np.ascontiguousarray(p, dtype=np.float32) for p in (delta, zeta, eta, alpha_match, alpha_gap, beta_match, beta_gap)]
+    hap_len, num_haps = H.shape
+    num_reads, read_len = R.shape
+    assert all(p.shape == (num_reads, read_len) for p in probs) and hap_len >= 2
+    out = np.empty((num_reads, num_haps), dtype=np.float32)
+    up = ctypes.POINTER(ctypes.c_ubyte)
+    lib().oracle_pairhmm(H.ctypes.data_as(up), R.ctypes.data_as(up), *[_p(p) for p in probs], _p(out), num_haps, hap_len,
+                         num_reads, read_len, acc, threads)
+    return out
+
+
+def pairhmm_inputs(num_haps, hap_len, num_reads, read_len, seed):
+    """Inputs with non-trivial results: haplotypes over ACGT, every read a window of a haplotype with a
+    few substitutions, base qualities 10..40, gap-open qualities 40..45 and gap-continuation quality 10,
+    turned into probabilities the way the driver does (pairhmm-run-fpga.cpp:90-107: delta and zeta
+    = 10^(-q_open/10), eta = 10^(-q_cont/10), alpha = 1 - (delta + zeta), beta = 1 - eta,
+    *_match = x * (1 - e), *_gap = x * e / 3 with e = 10^(-q_base/10)).  Random letters and the
+    driver's qualities (65..90) give results that underflow to zero everywhere."""
+    rng = np.random.default_rng(seed)
+    letters = np.frombuffer(b"ACGT", dtype=np.uint8)
+    haps = letters[rng.integers(0, 4, (num_haps, hap_len))]
+    R = np.empty((num_reads, read_len), np.uint8)
+    for r in range(num_reads):
+        src = haps[rng.integers(0, num_haps)]
+        start = rng.integers(0, max(hap_len - read_len, 0) + 1)
+        window = src[start:start + read_len]
+        R[r, :len(window)] = window
+        if len(window) < read_len:
+            R[r, len(window):] = letters[rng.integers(0, 4, read_len - len(window))]
+        flips = rng.random(read_len) < 0.03
+        R[r, flips] = letters[rng.integers(0, 4, int(flips.sum()))]
+    f32 = np.float32
+    qb = rng.integers(10, 41, (num_reads, read_len))
+    qi, qd = rng.integers(40, 46, (num_reads, read_len)), rng.integers(40, 46, (num_reads, read_len))
+    e = (10.0 ** (-qb / 10.0)).astype(f32)
+    delta, zeta = (10.0 ** (-qi / 10.0)).astype(f32), (10.0 ** (-qd / 10.0)).astype(f32)
+    eta = np.full((num_reads, read_len), 10.0 ** (-10 / 10.0), f32)
+    alpha = (f32(1.0) - (delta + zeta)).astype(f32)
+    beta = (f32(1.0) - eta).astype(f32)
+    am, ag = (alpha * (f32(1.0) - e)).astype(f32), (alpha * e / f32(3.0)).astype(f32)
+    bm, bg = (beta * (f32(1.0) - e)).astype(f32), (beta * e / f32(3.0)).astype(f32)
+    H = np.ascontiguousarray(haps.T)                      # (hap_len, num_haps): haplotype index innermost
+    return H, R, delta, zeta, eta, am, ag, bm, bg
 
 
 def max_threads():

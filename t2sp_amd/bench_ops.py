@@ -197,6 +197,36 @@ def ssymv_case(torch, steps, warmup, peak):
                   **{"bound": "hbm", "GB/s": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / 8000.0, 4)})
 
 
+def pairhmm_case(torch, steps, warmup, peak):
+    """Not one of the headline benchmark configurations: the PairHMM pipeline (t2s/tests/performance/pairhmm) at the
+    size its README reports, 224 reads of 128 against 224 haplotypes of 384.  The unit of work is the
+    cell update (README: 41.8-47.9 GCups on the FPGAs).  No matrix product: a cell costs at least 10
+    vector instructions (3 fused multiply-adds, 3 multiplies, 1 add, 1 compare, 2 selects), so the
+    roof is the vector issue rate, 256 CUs x 64 lanes x 2.4 GHz = 39.3e12 lane-instructions/s."""
+    import numpy as np
+    L = lib()
+    num_haps, hap_len, num_reads, read_len = 224, 384, 224, 128
+    rng = np.random.default_rng(0)
+    H = torch.from_numpy(rng.integers(65, 69, (hap_len, num_haps)).astype(np.uint8)).cuda()
+    R = torch.from_numpy(rng.integers(65, 69, (num_reads, read_len)).astype(np.uint8)).cuda()
+    P = [ops.fill_uniform(torch.empty(num_reads, read_len, device="cuda"), 10 + i).abs_().mul_(0.5) for i in range(7)]
+    O = torch.empty(num_reads, num_haps, device="cuda")
+    so4 = (ctypes.c_int64 * 4)(1, num_haps, 0, 0)
+    s = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        rc = L.t2sp_pairhmm_f32(H.data_ptr(), R.data_ptr(), *[p.data_ptr() for p in P], O.data_ptr(), num_haps, hap_len,
+                                num_reads, read_len, num_haps, read_len, num_haps, num_reads, so4, s)
+        assert rc == 0, rc
+
+    ms = _time(torch, launch, steps, warmup)
+    cells = float(num_haps) * hap_len * num_reads * read_len
+    gcups = cells / ms / 1e6
+    return {"GCups": round(gcups, 1), "avg_launch_ms": round(ms, 5), "bound": "vector issue",
+            "frac_of_vector_issue_peak": round(gcups * 1e9 * 10 / 39.3e12, 4),
+            "workload": "224 reads x 128 against 224 haplotypes x 384 (the size of the reference's README)"}
+
+
 def run_all(torch, steps, warmup, peak, capsule_cfg=0, capsule_splits=0):
     return {"conv2d": conv_config3(torch, steps, warmup, peak),
             "capsule": capsule_config4(torch, steps, warmup, peak, capsule_cfg, capsule_splits),
@@ -206,4 +236,5 @@ def run_all(torch, steps, warmup, peak, capsule_cfg=0, capsule_splits=0):
                                          " (the size of peppers/blas/level3/syrk/release/s10)"),
             "sger_8192": sger_8192(torch, steps, warmup, peak),
             "sgbmv3_131072x1024": sgbmv3_case(torch, steps, warmup, peak),
-            "ssymv_16384": ssymv_case(torch, steps, warmup, peak)}
+            "ssymv_16384": ssymv_case(torch, steps, warmup, peak),
+            "pairhmm_224x224": pairhmm_case(torch, steps, warmup, peak)}

@@ -38,6 +38,7 @@ assert ctypes.sizeof(halide_dimension_t) == 16
 assert ctypes.sizeof(halide_buffer_t) == 56
 
 FLOAT32 = (2, 32, 1)
+UINT8 = (1, 8, 1)
 
 
 class HalideBuffer:
@@ -73,22 +74,26 @@ class HalideBuffer:
 
     @classmethod
     def from_numpy(cls, a):
-        """Host buffer over a float32 numpy array (any non-negative strides)."""
-        assert isinstance(a, np.ndarray) and a.dtype == np.float32
-        assert all(s % 4 == 0 for s in a.strides)
-        ext, st = cls._dims_of(a.shape, [s // 4 for s in a.strides])
+        """Host buffer over a float32 (or, for character data, uint8) numpy array with non-negative strides."""
+        assert isinstance(a, np.ndarray) and a.dtype in (np.float32, np.uint8)
+        size = a.dtype.itemsize
+        assert all(s % size == 0 for s in a.strides)
+        ext, st = cls._dims_of(a.shape, [s // size for s in a.strides])
         if a.size == 0:  # numpy gives empty arrays arbitrary strides; describe them densely
             st = [int(np.prod(ext[:d], dtype=np.int64)) if d else 1 for d in range(len(ext))]
             st = [max(x, 1) for x in st]
-        return cls(ext, st, host=a.ctypes.data, keep=a)
+        for d in range(len(ext)):            # size-1 axes carry no stride information
+            if ext[d] == 1:
+                st[d] = 1 if d == 0 else st[d - 1] * max(ext[d - 1], 1)
+        return cls(ext, st, host=a.ctypes.data, keep=a, type_=FLOAT32 if a.dtype == np.float32 else UINT8)
 
     @classmethod
     def from_torch(cls, t):
         """Device buffer over a float32 torch CUDA tensor (used in place, no copies)."""
         import torch
-        assert t.is_cuda and t.dtype == torch.float32
+        assert t.is_cuda and t.dtype in (torch.float32, torch.uint8)
         ext, st = cls._dims_of(t.shape, t.stride())
-        return cls(ext, st, device=t.data_ptr(), keep=t)
+        return cls(ext, st, device=t.data_ptr(), keep=t, type_=FLOAT32 if t.dtype == torch.float32 else UINT8)
 
     @classmethod
     def from_axes(cls, x, axes):

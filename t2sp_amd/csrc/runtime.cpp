@@ -25,14 +25,19 @@ int report(int code, const char *op, const char *what) {
 
 int check_buffer(const halide_buffer_t *b, const char *op, const char *name, int dims_a,
                  int dims_b, Span *span) {
+    return check_buffer_typed(b, op, name, dims_a, dims_b, span, halide_type_float, 32);
+}
+
+int check_buffer_typed(const halide_buffer_t *b, const char *op, const char *name, int dims_a,
+                       int dims_b, Span *span, int type_code, int type_bits) {
     char msg[160];
     if (!b) {
         snprintf(msg, sizeof msg, "buffer argument %s is NULL", name);
         return report(halide_error_code_buffer_argument_is_null, op, msg);
     }
-    if (b->type.code != halide_type_float || b->type.bits != 32 || b->type.lanes != 1) {
-        snprintf(msg, sizeof msg, "%s has type code %d bits %d lanes %d, expected float32", name,
-                 (int)b->type.code, (int)b->type.bits, (int)b->type.lanes);
+    if (b->type.code != type_code || b->type.bits != type_bits || b->type.lanes != 1) {
+        snprintf(msg, sizeof msg, "%s has type code %d bits %d lanes %d, expected code %d bits %d", name,
+                 (int)b->type.code, (int)b->type.bits, (int)b->type.lanes, type_code, type_bits);
         return report(halide_error_code_bad_type, op, msg);
     }
     if (b->dimensions != dims_a && b->dimensions != dims_b) {
@@ -126,9 +131,9 @@ Staged::~Staged() {
     if (pooled_ && ptr_) pool().put(ptr_);
 }
 
-int Staged::input(const halide_buffer_t *b, const Span &s, const char *op) {
+int Staged::input(const halide_buffer_t *b, const Span &s, const char *op, int element_bytes) {
     span_ = s.span;
-    const size_t bytes = (size_t)s.span * sizeof(float);
+    const size_t bytes = (size_t)s.span * element_bytes;
     if (b->device) {
         ptr_ = reinterpret_cast<float *>(b->device);
         if ((b->flags & halide_buffer_flag_host_dirty) && b->host && bytes)

@@ -44,6 +44,9 @@ struct Span {
 // (Halide/src/AddImageChecks.cpp:352-636).
 int check_buffer(const halide_buffer_t *b, const char *op, const char *name, int dims_a,
                  int dims_b, Span *span);
+// The same for another element type (halide_type_code_t and bits), e.g. the uint8 characters of PairHMM.
+int check_buffer_typed(const halide_buffer_t *b, const char *op, const char *name, int dims_a,
+                       int dims_b, Span *span, int type_code, int type_bits);
 
 class DevicePool {
 public:
@@ -69,7 +72,7 @@ public:
     ~Staged();
     // Input: use b->device when the caller staged it (copying the host data up
     // first when host_dirty is set), else copy the host span into pool memory.
-    int input(const halide_buffer_t *b, const Span &s, const char *op);
+    int input(const halide_buffer_t *b, const Span &s, const char *op, int element_bytes = 4);
     // Output: use b->device when present, else pool memory (pre-filled from the
     // host when the buffer is not dense, so that gaps keep their contents).
     // `partial`: the kernels write only part of the buffer; the rest must keep what it holds.

@@ -173,6 +173,27 @@ def symv(A, x, y, alpha=1.0, beta=1.0, out=None, tiles=None):
     return out
 
 
+def pairhmm(H, R, delta, zeta, eta, alpha_match, alpha_gap, beta_match, beta_gap, out=None, tiles=None):
+    """Forward probability of every (read, haplotype) pair through the `pairhmm` entry point
+    (include/pairhmm-interface.h).
+
+    H: uint8 (HAP_LEN, NUM_HAPS); R: uint8 (NUM_READS, READ_LEN); the seven probabilities float32
+    (NUM_READS, READ_LEN).  With tiles=(HH, RR) the result has the reference's shape
+    Out(HH, RR, OH, OR), numpy (OR, OH, RR, HH) (t2s/tests/performance/pairhmm/pairhmm-run-fpga.cpp:112);
+    otherwise (NUM_READS, NUM_HAPS)."""
+    num_haps, num_reads = H.shape[1], R.shape[0]
+    if out is None:
+        if tiles is None:
+            out = _empty_like_kind(delta, (num_reads, num_haps))
+        else:
+            HH, RR = tiles
+            assert num_haps % HH == 0 and num_reads % RR == 0
+            out = _empty_like_kind(delta, (num_reads // RR, num_haps // HH, RR, HH))
+    bufs = [HalideBuffer.wrap(t) for t in (H, R, delta, zeta, eta, alpha_match, alpha_gap, beta_match, beta_gap, out)]
+    _check("pairhmm", lib().pairhmm(*[b.ref for b in bufs]))
+    return out
+
+
 def conv(I, W, out=None, cfg=0):
     """O = conv2d(I, W), stride 1, no padding, through the `conv` entry point
     (include/conv-interface.h).

@@ -466,6 +466,75 @@ def test_symv_reads_one_triangle_and_equals_full_symmetric_product():
     assert (o.symv(Af, xf, yf, 0.75, 1.25) == ref).all()
 
 
+# ---------------------------------------------------------------------------------------------
+# PairHMM
+def _pairhmm_full_matrices(H, R, delta, zeta, eta, am, ag, bm, bg):
+    """The driver's golden loop with its full M, I, D matrices (pairhmm-run-fpga.cpp:120-147),
+    numpy float32 scalars."""
+    f = np.float32
+    hap_len, num_haps = H.shape
+    num_reads, read_len = R.shape
+    out = np.zeros((num_reads, num_haps), f)
+    for r in range(num_reads):
+        for h in range(num_haps):
+            M, I, D = (np.zeros((read_len, hap_len), f) for _ in range(3))
+            golden = f(0)
+            for j in range(hap_len):
+                for i in range(read_len):
+                    if j == 0:
+                        M[i, 0] = I[i, 0] = D[i, 0] = 0
+                    if i == 0:
+                        M[0, j] = I[0, j] = 0
+                        D[0, j] = f(1.0 / (hap_len - 1))
+                    if j != 0 and i != 0:
+                        match = R[r, i] == H[j, h]
+                        alpha, beta = (am[r, i], bm[r, i]) if match else (ag[r, i], bg[r, i])
+                        M[i, j] = f(f(alpha * M[i - 1, j - 1]) + f(beta * f(I[i - 1, j - 1] + D[i - 1, j - 1])))
+                        I[i, j] = f(f(delta[r, i] * M[i - 1, j]) + f(eta[r, i] * I[i - 1, j]))
+                        D[i, j] = f(f(zeta[r, i] * M[i, j - 1]) + f(eta[r, i] * D[i, j - 1]))
+                    if i == read_len - 1 and j > 0:
+                        golden = f(golden + f(M[i, j] + I[i, j]))
+            out[r, h] = golden
+    return out
+
+
+def test_pairhmm_equals_full_matrix_loop_and_closed_forms():
+    """(1) The two-column restatement equals the driver's full-matrix loop bit for bit on realistic
+    inputs.  (2) Closed forms in exact dyadic arithmetic that fix which neighbour each term reads:
+    with alpha = beta = zeta = 1/2, delta = eta = 0 and 65 haplotype positions, a read of 3 positions
+    gives 63/256 + 62/512 (the diagonal term enters from column 2, the D term from column 3); with
+    delta = 1/2 instead of zeta and 4 positions, 62/512 + 63/512 + 63/512 (two diagonal steps from column 3,
+    the I terms from column 2).  (3) With the match and
+    gap values equal the characters do not matter; with them different they do."""
+    inp = o.pairhmm_inputs(5, 23, 4, 9, 3)
+    got = o.pairhmm(*inp)
+    assert (got == _pairhmm_full_matrices(*inp)).all()
+    assert got.max() > 1e-6                                     # not everything underflows
+    fma = o.pairhmm(*inp, acc=o.ACC_F32_FMA)
+    assert np.linalg.norm(fma - got) <= 1e-6 * np.linalg.norm(got)
+
+    hap_len, half = 65, np.float32(0.5)
+    H = np.full((hap_len, 2), ord("A"), np.uint8)
+    def const(n, v):
+        return np.full((1, n), v, np.float32)
+    R3 = np.full((1, 3), ord("C"), np.uint8)
+    out = o.pairhmm(H, R3, const(3, 0), const(3, half), const(3, 0), const(3, half), const(3, half), const(3, half), const(3, half))
+    assert (out == np.float32(63 / 256 + 62 / 512)).all()
+    R4 = np.full((1, 4), ord("C"), np.uint8)
+    out = o.pairhmm(H, R4, const(4, half), const(4, 0), const(4, 0), const(4, half), const(4, half), const(4, half), const(4, half))
+    assert (out == np.float32(62 / 512 + 63 / 512 + 63 / 512)).all()
+    # two read positions, alpha = 0, beta = 1/2: every column from 1 on adds beta / 64
+    R2 = np.full((1, 2), ord("C"), np.uint8)
+    out = o.pairhmm(H, R2, const(2, 0), const(2, 0), const(2, half), const(2, 0), const(2, 0), const(2, half), const(2, half))
+    assert (out == half).all()
+
+    H2, R, delta, zeta, eta, am, ag, bm, bg = o.pairhmm_inputs(3, 20, 2, 8, 4)
+    same = o.pairhmm(H2, R, delta, zeta, eta, am, am, bm, bm)
+    other = o.pairhmm(np.roll(H2, 1, axis=0), R, delta, zeta, eta, am, am, bm, bm)
+    assert (same == other).all()
+    assert not (o.pairhmm(H2, R, delta, zeta, eta, am, ag, bm, bg) == o.pairhmm(np.roll(H2, 1, axis=0), R, delta, zeta, eta, am, ag, bm, bg)).all()
+
+
 def test_gemm_ure_loop_nest_equals_golden_loop_bit_for_bit():
     """The spec's serial loop nest (gemm.cpp:30,57-71) sums every output in ascending total_k, like the
     golden loop: same bits, for the GPU and the TINY constant sets."""
