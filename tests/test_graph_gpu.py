@@ -93,3 +93,63 @@ def test_capsule_and_conv_in_one_graph(torch_cuda):
         g.replay()
         torch.cuda.synchronize()
         assert torch.equal(V, eager_v) and torch.equal(O, eager_o), "replay %d" % rep
+
+
+def test_partial_round_sgemm_padded_sgemm_and_pairhmm_in_one_graph(torch_cuda):
+    """The multi-launch plans (whole rounds + split rest + sum kernel; padded copies of operands of
+    an odd size + product + copy out) and the PairHMM kernel, recorded together."""
+    import numpy as np
+    torch = torch_cuda
+    L = t2sp_amd.lib()
+    M = N = 3072
+    K = 2048                                           # 576 tiles of 128 x 128: two rounds + 64 split tiles
+    A = t2sp_amd.fill_uniform(torch.empty(M, K, device="cuda"), 11)
+    B = t2sp_amd.fill_uniform(torch.empty(K, N, device="cuda"), 12)
+    C = torch.empty(M, N, device="cuda")
+    nbytes = L.t2sp_sgemm_workspace_bytes(M, N, K)
+    assert nbytes > 0
+    ws = torch.empty(nbytes // 4, device="cuda")
+    Mo, No, Ko = 301, 203, 105
+    Ao = t2sp_amd.fill_uniform(torch.empty(Mo, Ko, device="cuda"), 13)
+    Bo = t2sp_amd.fill_uniform(torch.empty(Ko, No, device="cuda"), 14)
+    Co = torch.empty(Mo, No, device="cuda")
+    obytes = L.t2sp_sgemm_workspace_bytes(Mo, No, Ko)
+    assert obytes > 0
+    wso = torch.empty(obytes // 4, device="cuda")
+    rng = np.random.default_rng(5)
+    num_haps, hap_len, num_reads, read_len = 32, 60, 8, 40
+    H = torch.from_numpy(rng.integers(65, 69, (hap_len, num_haps)).astype(np.uint8)).cuda()
+    R = torch.from_numpy(rng.integers(65, 69, (num_reads, read_len)).astype(np.uint8)).cuda()
+    P = [t2sp_amd.fill_uniform(torch.empty(num_reads, read_len, device="cuda"), 20 + i).abs_() for i in range(7)]
+    O = torch.empty(num_reads, num_haps, device="cuda")
+    so4 = (i64 * 4)(1, num_haps, 0, 0)
+    out = torch.empty(C.numel() + Co.numel() + O.numel(), device="cuda")
+
+    def launch(stream):
+        assert L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, ws.data_ptr(), nbytes,
+                                stream) == 0
+        assert L.t2sp_sgemm_f32(Ao.data_ptr(), Bo.data_ptr(), Co.data_ptr(), Mo, No, Ko, Ko, No, No, 0, wso.data_ptr(),
+                                obytes, stream) == 0
+        assert L.t2sp_pairhmm_f32(H.data_ptr(), R.data_ptr(), *[p.data_ptr() for p in P], O.data_ptr(), num_haps, hap_len,
+                                  num_reads, read_len, num_haps, read_len, num_haps, num_reads, so4, stream) == 0
+
+    def gather():
+        out[:C.numel()] = C.reshape(-1)
+        out[C.numel():C.numel() + Co.numel()] = Co.reshape(-1)
+        out[C.numel() + Co.numel():] = O.reshape(-1)
+
+    launch(torch.cuda.current_stream().cuda_stream)
+    gather()
+    torch.cuda.synchronize()
+    eager = out.clone()
+    assert torch.allclose(Co, Ao @ Bo, rtol=1e-4, atol=1e-4)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        launch(torch.cuda.current_stream().cuda_stream)
+        gather()
+
+    def refill(rep):
+        C.fill_(float("nan")); Co.fill_(float("nan")); O.fill_(float("nan"))
+        ws.fill_(float(rep)); wso.fill_(float(rep))
+
+    _replays_match(torch, g, out, eager, refill)
