@@ -418,10 +418,21 @@ __global__ void __launch_bounds__(256) gemm_unpad_kernel(const float *src, int64
 }
 
 static inline int64_t round_up4(int64_t v) { return (v + 3) / 4 * 4; }
+// Padded reduction length: a whole number of k-tile pairs, so that the padded product runs the
+// unguarded loaders.
+static inline int64_t pad_k(int64_t k) { return (k + 31) / 32 * 32; }
+// A reduction that is not a whole number of k-tile pairs sends every tile through the guarded
+// loaders (about 12 % slower); from about 5000^3 on, padding K in copies of A and B costs less.
+static bool gemm_k_tail_worth_padding(int M, int N, int K) {
+    if (K % 32 == 0) return false;
+    const double guarded_loss = 0.12 * 2.0 * M * N * K / 150e12;
+    const double copies = 8.0 * ((double)M * K + (double)K * N + 2.0 * M * N) / 4e12;
+    return guarded_loss > 1.3 * copies;
+}
 static inline size_t round_up256(size_t v) { return (v + 255) / 256 * 256; }
 // Bytes of the padded copies of A, B and C for a product the vector loaders cannot take as it lies.
 static size_t gemm_pad_bytes(int M, int N, int K, bool bt) {
-    const int64_t kp = round_up4(K), np = bt ? N : round_up4(N);
+    const int64_t kp = pad_k(K), np = bt ? N : round_up4(N);
     return round_up256((size_t)M * kp * sizeof(float)) + round_up256((size_t)(bt ? (int64_t)N * kp : kp * np) * sizeof(float)) +
            round_up256((size_t)M * np * sizeof(float));
 }
@@ -678,13 +689,14 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
                         ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
                         ((uintptr_t)g.C % 16 == 0) && (g.tiled || g.ldc % 4 == 0) &&
                         (!g.scale || (g.ldcin % 4 == 0 && (uintptr_t)g.Cin % 16 == 0));
-    if (cfg == T2SP_CFG_AUTO && !vec_ok && workspace && ((uintptr_t)workspace % 16 == 0) &&
-        workspace_bytes >= gemm_pad_bytes(g.M, g.N, g.K, bt)) {
+    if (cfg == T2SP_CFG_AUTO && (!vec_ok || gemm_k_tail_worth_padding(g.M, g.N, g.K)) && workspace &&
+        ((uintptr_t)workspace % 16 == 0) && workspace_bytes >= gemm_pad_bytes(g.M, g.N, g.K, bt)) {
         // K or N not a multiple of 4, or rows that are not 16-byte aligned: multiply zero-padded,
         // aligned copies instead (the reference's BLAS wrapper pads its operands to tile multiples
         // in the same way, t2s/peppers/blas/level3/gemm/release/a10/blas-gemm.cpp:28-31) and
-        // copy the result out.  Moving the matrices twice costs little next to the product.
-        const int kp = (int)round_up4(g.K), np = bt ? g.N : (int)round_up4(g.N);
+        // copy the result out.  Moving the matrices twice costs little next to the product.  Large
+        // products whose K is not a whole number of k-tile pairs come here too.
+        const int kp = (int)pad_k(g.K), np = bt ? g.N : (int)round_up4(g.N);
         float *a2 = workspace;
         float *b2 = a2 + round_up256((size_t)g.M * kp * sizeof(float)) / sizeof(float);
         float *c2 = b2 + round_up256((size_t)(bt ? (int64_t)g.N * kp : (int64_t)kp * np) * sizeof(float)) / sizeof(float);
@@ -745,10 +757,10 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
 
 extern "C" size_t t2sp_sgemm_workspace_bytes(int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
-    if (K % 4 == 0 && N % 4 == 0) return t2sp::plan_gemm(M, N, K).scratch_bytes;
+    if (K % 4 == 0 && N % 4 == 0 && !t2sp::gemm_k_tail_worth_padding(M, N, K)) return t2sp::plan_gemm(M, N, K).scratch_bytes;
     // padded copies of the operands, then the planes for the padded product
     return t2sp::gemm_pad_bytes(M, N, K, false) +
-           t2sp::plan_gemm(M, (int)t2sp::round_up4(N), (int)t2sp::round_up4(K)).scratch_bytes;
+           t2sp::plan_gemm(M, (int)t2sp::round_up4(N), (int)t2sp::pad_k(K)).scratch_bytes;
 }
 
 extern "C" int t2sp_sgemm_f32(const float *A, const float *B, float *C, int M, int N, int K,
@@ -778,9 +790,10 @@ extern "C" size_t t2sp_sgemm_ex_workspace_bytes(int transa, int M, int N, int K)
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     // the re-laid A of the transposed form (required), then the planes of a split reduction (optional)
     const size_t pad_t = t2sp::gemm_pad_bytes(M, N, K, true), pad_n = t2sp::gemm_pad_bytes(M, N, K, false);
-    const size_t pad = (K % 4 || N % 4) ? (pad_t > pad_n ? pad_t : pad_n) : 0;
+    const bool padded = K % 4 || N % 4 || t2sp::gemm_k_tail_worth_padding(M, N, K);
+    const size_t pad = padded ? (pad_t > pad_n ? pad_t : pad_n) : 0;
     return t2sp::round_up256(transa ? (size_t)M * K * sizeof(float) : 0) + pad +
-           t2sp::plan_gemm(M, (int)t2sp::round_up4(N), (int)t2sp::round_up4(K)).scratch_bytes;
+           t2sp::plan_gemm(M, (int)t2sp::round_up4(N), (int)(padded ? t2sp::pad_k(K) : K)).scratch_bytes;
 }
 
 extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, float alpha, const float *A,

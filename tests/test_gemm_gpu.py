@@ -205,6 +205,30 @@ def test_partial_last_round_split_with_workspace(oracle, torch_cuda, shape):
         assert torch.equal(flat, split)
 
 
+def test_large_product_with_a_k_tail_runs_on_padded_copies(oracle, torch_cuda):
+    """K = 8200 is not a whole number of pairs of k-tiles: with a workspace the product runs on copies
+    of A and B padded to K = 8224 (all tiles through the unguarded loaders); sampled rows against the
+    oracle, and the whole result against the run without a workspace."""
+    torch = torch_cuda
+    M, N, K = 8192, 8192, 8200
+    L = t2sp_amd.lib()
+    nbytes = L.t2sp_sgemm_workspace_bytes(M, N, K)
+    assert nbytes >= 4 * (M * 8224 + 8224 * N + M * N)
+    A = t2sp_amd.fill_uniform(torch.empty(M, K, device="cuda"), 25)
+    B = t2sp_amd.fill_uniform(torch.empty(K, N, device="cuda"), 26)
+    ws = torch.empty(nbytes // 4, device="cuda")
+    outs = []
+    for w, nb in ((None, 0), (ws.data_ptr(), nbytes)):
+        C = torch.full((M, N), float("nan"), device="cuda")
+        assert L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, w, nb, None) == 0
+        torch.cuda.synchronize()
+        outs.append(C)
+    plain, padded = outs
+    assert (plain - padded).abs().max().item() <= 1.6e-5 * plain.abs().max().item()
+    rows = np.array([0, 1, 4095, 8191])
+    assert rel_fro(padded[rows].cpu().numpy(), oracle.gemm(A[rows].cpu().numpy(), B.cpu().numpy()))[0] <= TOL
+
+
 @pytest.mark.parametrize("shape", [(1024, 1024, 1024), (500, 260, 4096), (64, 128, 8192), (130, 66, 64), (1, 2, 8),
                                    (512, 768, 640), (192, 64, 24)])
 def test_direct_kernel_small_products(oracle, torch_cuda, shape):
