@@ -117,17 +117,20 @@ static_assert(offsetof(halide_buffer_t, dim) == 40, "dim at 40");
  * a(TOTAL_K, TOTAL_I); a(k, i) = ...; gemm(a, b, c);  It plays the role of
  * Halide::Runtime::Buffer<float> (Halide/src/runtime/HalideBuffer.h:1050-1061:
  * raw_buffer() and the implicit conversion to halide_buffer_t*) for the subset
- * those drivers use: dense allocation, operator() element access, extents. */
+ * those drivers use: dense allocation, operator() element access, extents.
+ * Element types: float, and unsigned char for the character buffers of pairhmm. */
 #include <cstring>
 #include <initializer_list>
 #include <new>
+#include <type_traits>
 #include <vector>
 extern "C" void *t2sp_host_malloc(size_t bytes);
 extern "C" void t2sp_host_free(void *p);
 namespace t2sp {
 template <typename T>
 class Buffer {
-    static_assert(sizeof(T) == 4, "only 32-bit element types are used on this path");
+    static_assert(std::is_same<T, float>::value || std::is_same<T, uint8_t>::value,
+                  "float (every operator) and unsigned char (the characters of pairhmm) are the element types of this path");
     T *storage_ = nullptr;           // from t2sp_host_malloc: page-locked when a device is present
     std::vector<halide_dimension_t> dims_;
     halide_buffer_t buf_;
@@ -151,8 +154,8 @@ class Buffer {
         buf_.device_interface = nullptr;
         buf_.host = (uint8_t *)(external ? external : storage_);
         buf_.flags = 0;
-        buf_.type.code = halide_type_float;
-        buf_.type.bits = 32;
+        buf_.type.code = std::is_same<T, float>::value ? halide_type_float : halide_type_uint;
+        buf_.type.bits = (uint8_t)(8 * sizeof(T));
         buf_.type.lanes = 1;
         buf_.dimensions = nd;
         buf_.dim = dims_.data();

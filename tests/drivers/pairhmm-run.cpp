@@ -4,37 +4,20 @@
 // pair against the golden loop with its full M, I, D matrices.  Reads are windows of the
 // haplotypes with a few substitutions and qualities of 10..45, so that the results are not all
 // underflow (the reference's random letters and qualities of 65..90 give zeros everywhere).
+#include <cmath>
 #include <vector>
 
 #include "pairhmm-interface.h"
 #include "driver_common.h"
 
 namespace {
-// t2sp::Buffer holds 32-bit elements; the characters go through plain halide_buffer_t views.
-struct Chars {
-    std::vector<uint8_t> data;
-    halide_dimension_t dims[2];
-    halide_buffer_t buf;
-    Chars(int e0, int e1) : data((size_t)e0 * e1) {
-        dims[0] = {0, e0, 1, 0};
-        dims[1] = {0, e1, e0, 0};
-        buf = halide_buffer_t{};
-        buf.host = data.data();
-        buf.type.code = halide_type_uint;
-        buf.type.bits = 8;
-        buf.type.lanes = 1;
-        buf.dimensions = 2;
-        buf.dim = dims;
-    }
-    uint8_t &operator()(int i0, int i1) { return data[(size_t)i1 * dims[0].extent + i0]; }
-};
 uint32_t pick(drv::Rng &r, uint32_t n) { return (uint32_t)((r.next() * 0.5f + 0.5f) * n) % n; }
 float ph2pr(int q) { return std::pow(10.0f, -q / 10.0f); }
 }  // namespace
 
 static int run(int HH, int RR, int OH, int OR, int READ_LEN, int HAP_LEN) {
     const int NUM_HAPS = OH * HH, NUM_READS = OR * RR;
-    Chars H(NUM_HAPS, HAP_LEN), R(READ_LEN, NUM_READS);
+    t2sp::Buffer<unsigned char> H(NUM_HAPS, HAP_LEN), R(READ_LEN, NUM_READS);
     t2sp::Buffer<float> delta(READ_LEN, NUM_READS), zeta(READ_LEN, NUM_READS), eta(READ_LEN, NUM_READS);
     t2sp::Buffer<float> alpha_match(READ_LEN, NUM_READS), alpha_gap(READ_LEN, NUM_READS);
     t2sp::Buffer<float> beta_match(READ_LEN, NUM_READS), beta_gap(READ_LEN, NUM_READS);
@@ -58,7 +41,7 @@ static int run(int HH, int RR, int OH, int OR, int READ_LEN, int HAP_LEN) {
         }
     }
     t2sp::Buffer<float> result(HH, RR, OH, OR);
-    if (int err = pairhmm(&H.buf, &R.buf, delta, zeta, eta, alpha_match, alpha_gap, beta_match, beta_gap, result)) {
+    if (int err = pairhmm(H, R, delta, zeta, eta, alpha_match, alpha_gap, beta_match, beta_gap, result)) {
         std::printf("pairhmm returned %d\n", err);
         return 1;
     }
