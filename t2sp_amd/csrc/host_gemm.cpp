@@ -16,6 +16,106 @@
 
 using namespace t2sp;
 
+// Large products on host buffers: the rows of A and C go through the device in panels, so that the
+// upload of the next panel and the download of the previous one overlap with the product of the
+// current one (the reference copies everything in, runs, copies everything out:
+// AOT-OpenCL-Runtime.cpp:402-441).  Three streams of default priority: copies in, kernels (the
+// library stream), copies out, chained by events.  Panels are whole multiples of 256 rows (and of
+// the tiled output's III * II), at least one full round of 256 tiles each.
+namespace {
+constexpr int MAX_PANELS = 8;
+struct PanelStreams {
+    hipStream_t in = nullptr, out = nullptr;
+    hipEvent_t up[MAX_PANELS], k0[MAX_PANELS], k1[MAX_PANELS];
+    bool ok = false;
+    PanelStreams() {
+        ok = hipStreamCreateWithFlags(&in, hipStreamNonBlocking) == hipSuccess &&
+             hipStreamCreateWithFlags(&out, hipStreamNonBlocking) == hipSuccess;
+        for (int i = 0; i < MAX_PANELS && ok; i++)
+            ok = hipEventCreate(&up[i]) == hipSuccess && hipEventCreate(&k0[i]) == hipSuccess &&
+                 hipEventCreate(&k1[i]) == hipSuccess;
+        if (!ok) (void)hipGetLastError();
+    }
+};
+PanelStreams &panel_streams() {
+    static PanelStreams s;
+    return s;
+}
+
+// Rows per panel, or 0 when the product should run in one piece.
+int panel_rows(int M, int N, int K, int64_t row_quantum) {
+    if ((double)M * N * K < 1e11 || N < 256) return 0;          // small: the copies are short anyway
+    int64_t q = 256;
+    while (q % row_quantum) q += 256;                           // a multiple of 256 and of III * II
+    const int64_t tiles_per_q = (q / 256) * ((N + 255) / 256);
+    int64_t rows = q * ((256 + tiles_per_q - 1) / tiles_per_q);  // at least one round of 256 tiles
+    while ((M + rows - 1) / rows > MAX_PANELS) rows += q;
+    return (M + rows - 1) / rows >= 2 ? (int)rows : 0;
+}
+}  // namespace
+
+static int gemm_panels(halide_buffer_t *A, halide_buffer_t *B, halide_buffer_t *C, int cfg, int rows, const Span &sb) {
+    static const char *op = "gemm";
+    PanelStreams &ps = panel_streams();
+    if (!ps.ok) return 1;                                       // caller falls back to the one-piece path
+    const int K = A->dim[0].extent, M = A->dim[1].extent, N = B->dim[0].extent;
+    const bool tiled = C->dimensions == 6;
+    const float *ha = reinterpret_cast<const float *>(A->host), *hb = reinterpret_cast<const float *>(B->host);
+    float *hc = reinterpret_cast<float *>(C->host);
+    float *da = static_cast<float *>(pool().get((size_t)M * K * sizeof(float)));
+    float *db = static_cast<float *>(pool().get((size_t)sb.span * sizeof(float)));
+    float *dc = static_cast<float *>(pool().get((size_t)M * N * sizeof(float)));
+    const size_t ws_bytes = t2sp_sgemm_workspace_bytes(rows, N, K);
+    float *ws = ws_bytes ? static_cast<float *>(pool().get(ws_bytes)) : nullptr;
+    struct Put { float *p[4]; ~Put() { for (float *q : p) if (q) pool().put(q); } } put{{da, db, dc, ws}};
+    if (!da || !db || !dc) return report(halide_error_code_device_malloc_failed, op, "device allocation failed");
+    const int panels = (M + rows - 1) / rows;
+    int err = 0;
+    auto fail = [&](int code, const char *what) {
+        (void)hipDeviceSynchronize();
+        (void)hipGetLastError();
+        return report(code, op, what);
+    };
+    if (hipMemcpyAsync(db, hb, (size_t)sb.span * sizeof(float), hipMemcpyHostToDevice, ps.in) != hipSuccess)
+        return fail(halide_error_code_copy_to_device_failed, "host to device copy failed");
+    for (int p = 0; p < panels; p++) {
+        const int r0 = p * rows, nr = M - r0 < rows ? M - r0 : rows;
+        if (hipMemcpyAsync(da + (size_t)r0 * K, ha + (size_t)r0 * K, (size_t)nr * K * sizeof(float), hipMemcpyHostToDevice,
+                           ps.in) != hipSuccess)
+            return fail(halide_error_code_copy_to_device_failed, "host to device copy failed");
+        (void)hipEventRecord(ps.up[p], ps.in);
+        (void)hipStreamWaitEvent(api_stream(), ps.up[p], 0);
+        (void)hipEventRecord(ps.k0[p], api_stream());
+        float *cp = dc + (size_t)r0 * N;                        // panel p of C: contiguous in both output forms
+        if (tiled) {
+            int64_t s6[6];
+            for (int d = 0; d < 6; d++) s6[d] = C->dim[d].stride;
+            err = t2sp_sgemm_f32_tiled(da + (size_t)r0 * K, db, cp, nr, N, K, K, B->dim[1].stride, C->dim[0].extent,
+                                       C->dim[1].extent, C->dim[2].extent, C->dim[3].extent, s6, cfg, ws,
+                                       ws ? ws_bytes : 0, api_stream());
+        } else {
+            err = t2sp_sgemm_f32(da + (size_t)r0 * K, db, cp, nr, N, K, K, B->dim[1].stride, N, cfg, ws,
+                                 ws ? ws_bytes : 0, api_stream());
+        }
+        if (err) return fail(err, "kernel launch failed");
+        (void)hipEventRecord(ps.k1[p], api_stream());
+        (void)hipStreamWaitEvent(ps.out, ps.k1[p], 0);
+        if (hipMemcpyAsync(hc + (size_t)r0 * N, cp, (size_t)nr * N * sizeof(float), hipMemcpyDeviceToHost, ps.out) != hipSuccess)
+            return fail(halide_error_code_copy_to_host_failed, "device to host copy failed");
+    }
+    if (hipStreamSynchronize(ps.out) != hipSuccess || hipStreamSynchronize(api_stream()) != hipSuccess ||
+        hipStreamSynchronize(ps.in) != hipSuccess)
+        return fail(halide_error_code_device_run_failed, "kernel execution failed");
+    double ns = 0.0;
+    for (int p = 0; p < panels; p++) {
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, ps.k0[p], ps.k1[p]) == hipSuccess) ns += (double)ms * 1e6;
+    }
+    publish_kernel_ns(ns, op);
+    C->flags &= ~(uint64_t)(halide_buffer_flag_device_dirty | halide_buffer_flag_host_dirty);
+    return 0;
+}
+
 static int gemm_impl(halide_buffer_t *A, halide_buffer_t *B, halide_buffer_t *C, int cfg) {
     static const char *op = "gemm";
     std::lock_guard<std::mutex> lock(api_mutex());
@@ -43,6 +143,19 @@ static int gemm_impl(halide_buffer_t *A, halide_buffer_t *B, halide_buffer_t *C,
     if (c_rows != M || c_cols != N)
         return report(halide_error_code_constraint_violated, op, "C extents must equal M x N");
     if (M == 0 || N == 0) return 0;
+
+    // host buffers, dense rows of A and a dense C: large products run in row panels
+    const bool host_only = !A->device && !B->device && !C->device && A->host && B->host && C->host;
+    if (host_only && cfg == T2SP_CFG_AUTO && K > 0 && A->dim[1].stride == K && sc.span == sc.elements &&
+        (tiled || C->dim[1].stride == N)) {
+        const int64_t quantum = tiled ? (int64_t)C->dim[1].extent * C->dim[3].extent : 1;
+        const bool tiled_dense = !tiled || (C->dim[5].stride == (int64_t)C->dim[4].stride * C->dim[4].extent);
+        const int rows = tiled_dense ? panel_rows(M, N, K, quantum) : 0;
+        if (rows > 0) {
+            const int rc = gemm_panels(A, B, C, cfg, rows, sb);
+            if (rc <= 0) return rc;                              // > 0: streams unavailable, run in one piece
+        }
+    }
 
     Staged da, db, dc;
     if ((err = da.input(A, sa, op))) return err;

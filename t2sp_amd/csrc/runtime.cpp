@@ -195,20 +195,23 @@ int KernelTimer::stop_and_sync(const char *op) {
         return report(halide_error_code_device_run_failed, op, "kernel execution failed");
     }
     float ms = 0.f;
-    if (hipEventElapsedTime(&ms, g_ev0, g_ev1) == hipSuccess) g_last_kernel_ns = (double)ms * 1e6;
+    if (hipEventElapsedTime(&ms, g_ev0, g_ev1) == hipSuccess) publish_kernel_ns((double)ms * 1e6, op);
+    return 0;
+}
+
+void publish_kernel_ns(double ns, const char *op) {
+    g_last_kernel_ns = ns;
     // Optional file in the reference's exec_time.txt format (AOT-OpenCL-Runtime.cpp:380-394):
     // overall ns on the first line, then "<kernel_name> <ns>" lines.  The reference's drivers ask
     // for "kernel_unloader", the last kernel of its pipeline, so that name is written too.
     if (const char *file = getenv("T2SP_EXEC_TIME_FILE")) {
         if (*file) {
             if (FILE *fp = fopen(file, "w")) {
-                const double ns = g_last_kernel_ns.load();
                 fprintf(fp, "%f\nkernel_%s %lf\nkernel_unloader %lf\n", ns, op, ns, ns);
                 fclose(fp);
             }
         }
     }
-    return 0;
 }
 
 }  // namespace t2sp

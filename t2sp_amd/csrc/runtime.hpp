@@ -93,6 +93,10 @@ private:
 // stream; the elapsed time of the last call is what t2sp_last_kernel_ns returns
 // (the counterpart of the "latest end - earliest start" figure the reference
 // writes to exec_time.txt, AOT-OpenCL-Runtime.cpp:358-396).
+// Records `ns` as the kernel time of the call that just ended (what t2sp_last_kernel_ns returns
+// and, when $T2SP_EXEC_TIME_FILE names a file, what is written there in the reference's format).
+void publish_kernel_ns(double ns, const char *op);
+
 class KernelTimer {
 public:
     KernelTimer();

@@ -205,6 +205,29 @@ def test_partial_last_round_split_with_workspace(oracle, torch_cuda, shape):
         assert torch.equal(flat, split)
 
 
+@pytest.mark.parametrize("pinned", [False, True])
+def test_large_host_product_runs_in_row_panels(oracle, pinned):
+    """Host buffers and a large product: the entry point moves the rows of A and C through the device in
+    panels (8192 rows = 2 panels here) so that copies and kernels overlap.  Flat and tiled output,
+    pageable and page-locked buffers; sampled rows against the oracle, the two forms against each other,
+    and the kernel time still reported."""
+    M, N, K = 8192, 4096, 4096
+    mk = t2sp_amd.host_empty if pinned else (lambda shape: np.empty(shape, np.float32))
+    A, B = mk((M, K)), mk((K, N))
+    A[...] = oracle.fill_uniform((M, K), 27)
+    B[...] = oracle.fill_uniform((K, N), 28)
+    C = mk((M, N))
+    C[...] = np.nan
+    t2sp_amd.gemm(A, B, out=C)
+    ns = t2sp_amd.last_kernel_ns()
+    assert 0.5e6 < ns < 20e6                                      # about 1.9 ms of kernels
+    rows = np.array([0, 1, 4095, 4096, 8191])
+    assert rel_fro(C[rows], oracle.gemm(A[rows], B))[0] <= TOL
+    assert np.isfinite(C).all()
+    tiled = t2sp_amd.gemm(A, B, tiles=(16, 4, 8, 2))
+    assert (detile(tiled) == C).all()
+
+
 def test_large_product_with_a_k_tail_runs_on_padded_copies(oracle, torch_cuda):
     """K = 8200 is not a whole number of pairs of k-tiles: with a workspace the product runs on copies
     of A and B padded to K = 8224 (all tiles through the unguarded loaders); sampled rows against the
