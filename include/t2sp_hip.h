@@ -75,7 +75,8 @@ int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, float alpha, 
  * then first re-laid into `workspace`, which the transposed form requires).  For large N the
  * workspace (t2sp_ssyrk_workspace_bytes; optional when trans is zero) also holds partial planes
  * that let the last, partial round of 256 tiles split its reduction over all CUs (N = 8192: two
- * full rounds + 16 tiles).  Only tiles on or above the
+ * full rounds + 16 tiles), and, when K is not a multiple of 4, a zero-padded copy of A (without
+ * it such a product takes the scalar kernel).  Only tiles on or above the
  * diagonal are multiplied.  Flat form: C row-major N x N; `upper` selects the triangle of BLAS
  * semantics; mirror = 0 writes that triangle only, 1 writes both triangles with Cin read from the
  * `upper` triangle (a symmetric result, what the reference's ssyrk wrapper returns,

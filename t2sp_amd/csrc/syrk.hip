@@ -23,6 +23,14 @@ namespace t2sp {
 
 enum : int { SYRK_FLAT_SYM = 0, SYRK_FLAT_FULL = 1, SYRK_FOLDED = 2 };
 
+// Zero-padded copy of a row-major rows x cols matrix into rows_p x cols_p (defined with the SGEMM kernels).
+__global__ void gemm_pad_copy_kernel(const float *src, int64_t ld, float *dst, int rows, int cols, int rows_p, int cols_p);
+// K padded so that every kernel of this file can read the copy: a whole number of k-tile pairs.
+static inline int syrk_pad_k(int K) { return (K + 31) / 32 * 32; }
+static inline size_t syrk_padded_a_bytes(int N, int K) {
+    return ((size_t)N * syrk_pad_k(K) * sizeof(float) + 255) / 256 * 256;
+}
+
 struct SyrkArgs {
     const float *A;
     int64_t lda;
@@ -507,6 +515,23 @@ static int dispatch_syrk(SyrkArgs g, int trans, int cfg, float *workspace, size_
         workspace += (size_t)g.N * g.K;      // what is left may hold the planes of a split last round
         workspace_bytes -= relaid;
     }
+    // A the 128-bit loaders cannot read where it lies (K or its leading dimension not a multiple of 4,
+    // unaligned): a zero-padded, aligned copy is multiplied instead, as the SGEMM path does
+    const bool a_ok = g.K % 4 == 0 && g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0);
+    if (!a_ok && cfg == T2SP_CFG_AUTO && workspace && ((uintptr_t)workspace % 16 == 0) &&
+        workspace_bytes >= syrk_padded_a_bytes(g.N, g.K)) {
+        const int kp = syrk_pad_k(g.K);
+        const int64_t total = (int64_t)g.N * kp;
+        hipLaunchKernelGGL(gemm_pad_copy_kernel, dim3((unsigned)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192)),
+                           dim3(256), 0, stream, g.A, g.lda, workspace, g.N, g.K, g.N, kp);
+        if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
+        g.A = workspace;
+        g.lda = kp;
+        g.K = kp;
+        const size_t used = syrk_padded_a_bytes(g.N, kp);
+        workspace += used / sizeof(float);
+        workspace_bytes -= used;
+    }
     if (cfg == T2SP_CFG_DIRECT16) return syrk_d16_ok(g) ? launch_syrk_d16(g, stream) : T2SP_ERR_SHAPE;
     if (cfg == T2SP_CFG_AUTO && g.N <= SYRK_D16_MAX_N && g.K >= 64 && syrk_d16_ok(g)) return launch_syrk_d16(g, stream);
     const bool out_ok = g.mode == SYRK_FOLDED ||
@@ -575,7 +600,8 @@ extern "C" size_t t2sp_ssyrk_workspace_bytes(int trans, int N, int K) {
         const t2sp::SyrkTail t = t2sp::plan_syrk_tail(N, K, b, 16);
         if (t.scratch_bytes > planes) planes = t.scratch_bytes;
     }
-    return (trans ? (size_t)N * K * sizeof(float) : 0) + planes;
+    // and, when K is not a multiple of 4, a zero-padded copy of A
+    return (trans ? (size_t)N * K * sizeof(float) : 0) + (K % 4 ? t2sp::syrk_padded_a_bytes(N, K) : 0) + planes;
 }
 
 extern "C" size_t t2sp_ssyrk_folded_workspace_bytes(int trans, int N, int K) {

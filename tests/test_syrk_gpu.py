@@ -152,6 +152,36 @@ def test_split_last_round_equals_unsplit(oracle, N, K, cfg):
             assert rel_fro(got, want)[0] <= TOL
 
 
+@pytest.mark.parametrize("N,K", [(768, 1001), (130, 77), (6144, 1030)])
+def test_odd_reduction_length_runs_on_a_padded_copy(oracle, N, K):
+    """K not a multiple of 4: A is multiplied as a zero-padded, aligned copy (workspace) instead of by
+    the one-thread-per-output kernel.  Integer data: exact whatever the order."""
+    import torch
+    rng = np.random.default_rng(9)
+    A = rng.integers(-2, 3, (N, K)).astype(np.float32)
+    C = rng.integers(-4, 5, (N, N)).astype(np.float32)
+    C = np.triu(C) + np.triu(C, 1).T
+    ref = 2.0 * (A.astype(np.float64) @ A.astype(np.float64).T) - 3.0 * C
+    L = t2sp_amd.lib()
+    Ad, Cd = torch.from_numpy(A).cuda(), torch.from_numpy(C).cuda()
+    out = torch.full((N, N), float("nan"), device="cuda")
+    nbytes = L.t2sp_ssyrk_workspace_bytes(0, N, K)
+    assert nbytes >= 4 * N * ((K + 31) // 32 * 32)
+    ws = torch.empty(nbytes // 4, device="cuda")
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for rep in range(2):
+        e0.record()
+        assert L.t2sp_ssyrk_f32(1, 0, N, K, 2.0, Ad.data_ptr(), K, -3.0, Cd.data_ptr(), N, out.data_ptr(), N, 1, 0,
+                                ws.data_ptr(), nbytes, None) == 0
+        e1.record()
+        torch.cuda.synchronize()
+    assert (out.cpu().numpy() == ref).all()
+    assert (torch.from_numpy(A).cuda() == Ad).all()
+    # far from the scalar kernel's time (N*N*K/2 multiply-adds at well under 1 TFLOP/s)
+    assert e0.elapsed_time(e1) < 1.0 + N * N * K / 1e10
+    assert (t2sp_amd.syrk(A, C, 2.0, -3.0) == ref).all()           # the host entry sizes its own workspace
+
+
 def test_error_codes():
     A = np.zeros((96, 16), np.float32)
     C = np.zeros((96, 96), np.float32)
