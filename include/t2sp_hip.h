@@ -183,7 +183,9 @@ int t2sp_capsule_f32(const float *P, const float *W, float *V, const int *dims11
 /* A[i,r] = sum_{j,k} B[i,j,k] * C[j,r] * D[k,r].  sb3/sc2/sd2/sa2 are element strides of
  * (i,j,k), (j,r), (k,r), (i,r).  The layout of the reference's golden helper (j contiguous in B
  * and C, i contiguous in A; t2s/tests/performance/util/util.h:498-515) takes the MFMA kernel,
- * anything else a scalar kernel.  Workspace as for t2sp_capsule_f32. */
+ * anything else a scalar kernel; with that orientation but J not a multiple of 16, I not a
+ * multiple of 4 or unaligned strides, zero-padded copies made in the workspace are multiplied
+ * instead.  Workspace as for t2sp_capsule_f32. */
 size_t t2sp_mttkrp_workspace_bytes(int I, int J, int K, int R, int cfg, int splits);
 int t2sp_mttkrp_f32(const float *B, const float *C, const float *D, float *A, int I, int J, int K,
                     int R, const int64_t *sb3, const int64_t *sc2, const int64_t *sd2,

@@ -271,11 +271,43 @@ static bool mttkrp_fast(int I, int J, const int64_t *sb3, const int64_t *sc2, co
            ((uintptr_t)C % 16 == 0) && ((uintptr_t)A % 16 == 0);
 }
 
+// Sizes the MFMA kernel cannot take as they lie (J not a multiple of 16, I not a multiple of 4,
+// strides or addresses that are not 16-byte aligned) run on zero-padded, aligned copies:
+// B' [K][Ip][Jp], C' [R][Jp] and a temporary A' [R][Ip].  Copying B moves it twice more; the
+// product itself reads it once and is bound by arithmetic, not by that traffic.
+__global__ void __launch_bounds__(256) mttkrp_pad_b_kernel(const float *B, int64_t s_i, int64_t s_k, float *dst, int I,
+                                                           int J, int K, int Ip, int Jp) {
+    const int64_t total = (int64_t)K * Ip * Jp;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
+        const int j = (int)(t % Jp);
+        const int64_t q = t / Jp;
+        const int i = (int)(q % Ip), k = (int)(q / Ip);
+        dst[t] = (i < I && j < J) ? B[k * s_k + i * s_i + j] : 0.f;
+    }
+}
+// rows x cols (column stride 1, row stride `ld`) <-> the padded rows_p x cols_p block, either way
+__global__ void __launch_bounds__(256) mttkrp_pad_2d_kernel(const float *src, int64_t ld_src, float *dst, int64_t ld_dst,
+                                                            int rows, int cols, int rows_d, int cols_d) {
+    const int64_t total = (int64_t)rows_d * cols_d;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
+        const int r = (int)(t / cols_d), c = (int)(t - (int64_t)r * cols_d);
+        dst[r * ld_dst + c] = (r < rows && c < cols) ? src[r * ld_src + c] : 0.f;
+    }
+}
+static inline size_t up256(size_t v) { return (v + 255) / 256 * 256; }
+static size_t mttkrp_pad_bytes(int I, int J, int K, int R) {
+    const size_t Ip = (I + 3) / 4 * 4, Jp = (J + 15) / 16 * 16;
+    return up256((size_t)K * Ip * Jp * sizeof(float)) + up256((size_t)R * Jp * sizeof(float)) + up256((size_t)R * Ip * sizeof(float));
+}
+
 }  // namespace t2sp
 
 extern "C" size_t t2sp_mttkrp_workspace_bytes(int I, int J, int K, int R, int cfg, int splits) {
     if (I <= 0 || J <= 0 || K <= 0 || R <= 0) return 0;
-    return t2sp::plan_mttkrp(I, J, K, R, cfg, splits).scratch_bytes;
+    if (J % 16 == 0 && I % 4 == 0) return t2sp::plan_mttkrp(I, J, K, R, cfg, splits).scratch_bytes;
+    // padded copies of B and C and a temporary result, then the planes of the padded product
+    return t2sp::mttkrp_pad_bytes(I, J, K, R) +
+           t2sp::plan_mttkrp((I + 3) / 4 * 4, (J + 15) / 16 * 16, K, R, cfg, splits).scratch_bytes;
 }
 
 extern "C" int t2sp_mttkrp_f32(const float *B, const float *C, const float *D, float *A, int I, int J,
@@ -285,7 +317,28 @@ extern "C" int t2sp_mttkrp_f32(const float *B, const float *C, const float *D, f
     using namespace t2sp;
     if (I <= 0 || J <= 0 || K <= 0 || R <= 0 || !sb3 || !sc2 || !sd2 || !sa2) return T2SP_ERR_SHAPE;
     if ((int64_t)K * J > INT32_MAX) return T2SP_ERR_SHAPE;
-    if (cfg == T2SP_CFG_SCALAR || !mttkrp_fast(I, J, sb3, sc2, sd2, sa2, B, C, A)) {
+    const bool fast = mttkrp_fast(I, J, sb3, sc2, sd2, sa2, B, C, A);
+    if (cfg == T2SP_CFG_AUTO && !fast && sb3[1] == 1 && sc2[0] == 1 && sa2[0] == 1 && workspace &&
+        ((uintptr_t)workspace % 16 == 0) && workspace_bytes >= mttkrp_pad_bytes(I, J, K, R) &&
+        (int64_t)K * ((J + 15) / 16 * 16) <= INT32_MAX) {
+        const int Ip = (I + 3) / 4 * 4, Jp = (J + 15) / 16 * 16;
+        float *b2 = workspace;
+        float *c2 = b2 + up256((size_t)K * Ip * Jp * sizeof(float)) / sizeof(float);
+        float *a2 = c2 + up256((size_t)R * Jp * sizeof(float)) / sizeof(float);
+        const size_t used = mttkrp_pad_bytes(I, J, K, R);
+        hipStream_t st = (hipStream_t)stream;
+        auto blocks = [](int64_t n) { return dim3((unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384)); };
+        hipLaunchKernelGGL(mttkrp_pad_b_kernel, blocks((int64_t)K * Ip * Jp), dim3(256), 0, st, B, sb3[0], sb3[2], b2, I, J, K, Ip, Jp);
+        hipLaunchKernelGGL(mttkrp_pad_2d_kernel, blocks((int64_t)R * Jp), dim3(256), 0, st, C, sc2[1], c2, (int64_t)Jp, R, J, R, Jp);
+        if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
+        const int64_t sb[3] = {Jp, 1, (int64_t)Ip * Jp}, sc[2] = {1, Jp}, sa[2] = {1, Ip};
+        const int rc = t2sp_mttkrp_f32(b2, c2, D, a2, Ip, Jp, K, R, sb, sc, sd2, sa, cfg, splits, workspace + used / sizeof(float),
+                                       workspace_bytes - used, stream);
+        if (rc != T2SP_OK) return rc;
+        hipLaunchKernelGGL(mttkrp_pad_2d_kernel, blocks((int64_t)R * I), dim3(256), 0, st, a2, (int64_t)Ip, A, sa2[1], R, I, R, I);
+        return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+    }
+    if (cfg == T2SP_CFG_SCALAR || !fast) {
         MttkrpGenericArgs a{B, C, D, A, I, J, K, R, {sb3[0], sb3[1], sb3[2]}, {sc2[0], sc2[1]},
                             {sd2[0], sd2[1]}, {sa2[0], sa2[1]}};
         const int64_t total = (int64_t)I * R;

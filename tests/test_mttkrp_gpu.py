@@ -39,6 +39,20 @@ def test_small_ranks_pick_narrow_tiles(oracle, R):
     assert (run(Bi, Ci, Di) == want).all()
 
 
+@pytest.mark.parametrize("shape", [(300, 200, 100, 64), (130, 50, 33, 20), (64, 24, 7, 256), (5, 3, 2, 1)])
+def test_sizes_off_the_vector_grid_run_on_padded_copies(oracle, shape):
+    """J not a multiple of 16 or I not a multiple of 4: B and C are multiplied as zero-padded copies.
+    Integer data, exact in any order; uniform data within the tolerance."""
+    I, J, K, R = shape
+    rng = np.random.default_rng(13)
+    B = rng.integers(-2, 3, (I, J, K)).astype(np.float32)
+    C, D = rng.integers(-2, 3, (J, R)).astype(np.float32), rng.integers(-2, 3, (K, R)).astype(np.float32)
+    want = np.einsum("ijk,jr,kr->ir", B.astype(np.float64), C, D)
+    assert (run(B, C, D) == want).all()
+    Bf, Cf, Df = oracle.fill_uniform((I, J, K), 31), oracle.fill_uniform((J, R), 32), oracle.fill_uniform((K, R), 33)
+    assert rel_fro(run(Bf, Cf, Df), oracle.mttkrp(Bf, Cf, Df))[0] <= TOL
+
+
 def test_literal_reference_buffers(oracle):
     """Buffers exactly as the helper takes them: a(l,i,k), c(l,j), b(k,j) -> d(i,j)."""
     L, I, J, K = 32, 12, 20, 6
