@@ -39,3 +39,10 @@ def test_hip_path_matches_the_fixtures():
     assert (np.isnan(folded) == ~written).all()
     assert rel_fro(folded[written], FIX["syrk_folded"][written])[0] <= TOL
     assert np.array_equal(t2sp_amd.ger(r["A"], r["x"], r["y"]), FIX["ger"])
+    b, v = mk.inputs("gbmv3"), mk.inputs("symv")
+    assert rel_fro(t2sp_amd.gbmv3(b["A"], b["x"], b["y"], 1.5, -0.5), FIX["gbmv3"])[0] <= TOL
+    assert rel_fro(t2sp_amd.symv(v["A"], v["x"], v["y"], 1.25, 0.75), FIX["symv"])[0] <= TOL
+    from oracle import oracle as o
+    ph = t2sp_amd.pairhmm(*o.pairhmm_inputs(**mk.PAIRHMM))
+    assert np.array_equal(ph, FIX["pairhmm_fused"])
+    assert rel_fro(ph, FIX["pairhmm"])[0] <= TOL
