@@ -68,11 +68,53 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *scratch
     }
 }
 
+// The same sum for a small plane under many splits (MTTKRP: 128 planes of 0.5 MB): one thread per
+// group would leave most of the chip idle, so WAYS threads share a group, thread w adding planes
+// w, w + WAYS, ... in ascending order, and the WAYS partial sums are then added in the order of w
+// through LDS.  Still a fixed order, so the result does not depend on the launch.
+template <bool ALONG_COLS, class OutMap, int WAYS>
+__global__ void __launch_bounds__(256) splitk_reduce_wide_kernel(const float *scratch, int S, int Mp, int Np,
+                                                                  const OutMap map) {
+    constexpr int GROUPS = 256 / WAYS;                  // groups per workgroup
+    __shared__ v4f part[WAYS][GROUPS];
+    const size_t plane = (size_t)Mp * Np;
+    const size_t groups = plane / 4;
+    const int way = threadIdx.x / GROUPS, slot = threadIdx.x % GROUPS;
+    const size_t g = (size_t)blockIdx.x * GROUPS + slot;
+    v4f sum = {0.f, 0.f, 0.f, 0.f};
+    if (g < groups) {
+        const float *p = scratch + g * 4;
+        for (int s = way; s < S; s += WAYS) sum += *reinterpret_cast<const v4f *>(p + (size_t)s * plane);
+    }
+    part[way][slot] = sum;
+    __syncthreads();
+    if (way != 0 || g >= groups) return;
+    v4f total = part[0][slot];
+#pragma unroll
+    for (int w = 1; w < WAYS; w++) total += part[w][slot];
+    int row, col;
+    if (ALONG_COLS) {
+        row = (int)(g / (Np / 4));
+        col = (int)(g % (Np / 4)) * 4;
+    } else {
+        col = (int)(g / (Mp / 4));
+        row = (int)(g % (Mp / 4)) * 4;
+    }
+    map.store(row, col, total);
+}
+
 template <bool ALONG_COLS, class OutMap>
 inline hipError_t launch_splitk_reduce(const float *scratch, int S, int Mp, int Np, const OutMap &map,
                                        hipStream_t stream) {
     const size_t groups = (size_t)Mp * Np / 4;
     size_t blocks = (groups + 255) / 256;
+    if (blocks < 512 && S >= 16) {
+        constexpr int WAYS = 8;
+        const size_t wide_blocks = (groups + 256 / WAYS - 1) / (256 / WAYS);
+        hipLaunchKernelGGL((splitk_reduce_wide_kernel<ALONG_COLS, OutMap, WAYS>), dim3((unsigned)wide_blocks), dim3(256), 0,
+                           stream, scratch, S, Mp, Np, map);
+        return hipGetLastError();
+    }
     if (blocks > 4096) blocks = 4096;
     hipLaunchKernelGGL((splitk_reduce_kernel<ALONG_COLS, OutMap>), dim3((unsigned)blocks), dim3(256), 0,
                        stream, scratch, S, Mp, Np, map);
