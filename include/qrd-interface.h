@@ -1,0 +1,32 @@
+/* qrd-interface.h — host interface of the batched QR factorisation pipeline.
+ *
+ * Same name and signature as the header the reference generates with
+ * Pipeline({QDeserializer, RDeserializer}).compile_to_host("qrd-interface", {a}, "qrd", ...)
+ * (t2s/tests/performance/qrd/qrd.cpp:105): the input, then the two outputs in the pipeline's order.
+ */
+#ifndef T2SP_QRD_INTERFACE_H
+#define T2SP_QRD_INTERFACE_H
+#include "t2sp_buffer.h"
+#include "t2sp_runtime.h"
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* A = Q * R for every matrix of the batch, by modified Gram-Schmidt (qrd.cpp:51-63).
+ *   a: float32 (J, K, BATCH): element (row k, column j) of matrix b, the column index innermost
+ *      (qrd.cpp:46-48);
+ *   Q: float32 (K, J, BATCH): column j of Q contiguous over k (the commented realize of qrd.cpp:100,
+ *      qrd-run-fpga.cpp:572-580);
+ *   R: float32 (J, I, BATCH) with I = J: row i contiguous over j, zeros left of the diagonal
+ *      (qrd-run-fpga.cpp:583-596).
+ * K, J <= 128 (the reference's pipeline is built for 128 x 128).  Returns 0 or a negative
+ * halide_error_code_t. */
+int qrd(struct halide_buffer_t *a, struct halide_buffer_t *Q, struct halide_buffer_t *R);
+
+/* qrd() that returns the kernel time in ns (negative error code on failure). */
+double qrd_ns(struct halide_buffer_t *a, struct halide_buffer_t *Q, struct halide_buffer_t *R);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

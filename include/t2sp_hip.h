@@ -149,6 +149,20 @@ int t2sp_pairhmm_f32(const uint8_t *H, const uint8_t *R, const float *delta, con
                      const float *beta_gap, float *O, int num_haps, int hap_len, int num_reads, int read_len,
                      int64_t h_stride, int64_t r_stride, int hh, int rr, const int64_t *so4, void *stream);
 
+/* QR factorisation of `batch` m x n matrices by modified Gram-Schmidt, column by column, every
+ * inner product summed over ascending k: R(i,i) = sqrt(X_i), R(i,j) = X_j / sqrt(X_i),
+ * Q(:,i) = t_i / sqrt(X_i), t_j -= (X_j / X_i) * t_i with X_j = <t_i, t_j>
+ * (t2s/tests/performance/qrd/qrd.cpp:51-63; the spec's fast_inverse_sqrt is an exact 1/sqrt here).
+ * A(k, j) at k*a_row_stride + j (the spec's a(j, k, b), qrd.cpp:46-48); Q(k, i) at i*q_col_stride + k
+ * (QDeserializer(k, j, b)); R(i, j) at i*r_row_stride + j, zero left of the diagonal
+ * (RDeserializer(j, i, b), qrd-run-fpga.cpp:583-596); the batch strides separate matrices.
+ * 1 <= m, n <= T2SP_QRD_MAX_DIM (the reference's pipeline is built for 128 x 128).  Vector
+ * arithmetic with the columns in registers, no MFMA; the unit of work is the matrix. */
+#define T2SP_QRD_MAX_DIM 128
+int t2sp_qrd_f32(const float *A, float *Q, float *R, int m, int n, int batch, int64_t a_row_stride,
+                 int64_t a_batch_stride, int64_t q_col_stride, int64_t q_batch_stride, int64_t r_row_stride,
+                 int64_t r_batch_stride, void *stream);
+
 /* O[n,co,h,w] = sum_{ci,kh,kw} I[n,ci,h+kh,w+kw] * W[co,ci,kh,kw], stride 1, valid
  * padding, fp32.  si4/sw4/so4 are element strides of the logical indices
  * (n,ci,h,w), (co,ci,kh,kw), (n,co,h,w); "w" is the innermost spatial axis (the

@@ -2,7 +2,7 @@
  *
  * A CPU restatement, in plain C, of the arithmetic the reference's dense
  * tensor pipelines compute (SGEMM, 2-D convolution, capsule convolution,
- * MTTKRP), used only as the checker for the HIP path and as the reported CPU
+ * MTTKRP, and the BLAS-2/3, PairHMM and QR pipelines next to them), used only as the checker for the HIP path and as the reported CPU
  * baseline.  Nothing in the shipped library links or calls this file.
  *
  * What each function follows in the reference:
@@ -41,6 +41,21 @@
  *                                 ascending j), the recurrence of pairhmm.cpp:72-91.  Only two columns
  *                                 are kept instead of the driver's full matrices; the arithmetic and
  *                                 its order are the driver's.
+ *   oracle_qrd       URE order    t2s/tests/performance/qrd/qrd.cpp:51-63: modified Gram-Schmidt by
+ *                                 columns.  X (the inner products of the pivot column with itself
+ *                                 and with every later column, ascending k, qrd.cpp:59), Xi and
+ *                                 irXi (qrd.cpp:60-61), S = irXi for the pivot and -X/Xi for the
+ *                                 others (qrd.cpp:62), the update vec_t = vec_a + S * vec_ai
+ *                                 (qrd.cpp:55), Q = the scaled pivot column (qrd.cpp:57) and
+ *                                 R = sqrt(Xi) on the diagonal, irXi * X right of it (qrd.cpp:63).
+ *                                 The spec runs the inner products of step i + 1 at the end of step
+ *                                 i (its index i starts at -1); the values and their order are the
+ *                                 same.  ONE DEVIATION: the spec's irXi is Halide's
+ *                                 fast_inverse_sqrt, an approximation whose bits depend on the
+ *                                 target; here it is 1 / sqrtf(x), both correctly rounded.  Parity
+ *                                 with the reference is therefore pinned to its driver's own
+ *                                 acceptance check (|Q*R - A| < 0.005, qrd-run-fpga.cpp:627-640) and
+ *                                 to the uniqueness of the factorisation, not to bits.
  *   oracle_mttkrp    golden       t2s/tests/performance/util/util.h:498-515 (two-step: TTM over l
  *                                 into e(i,j,k), then d += e*b over k).  The reference's outer loop
  *                                 bound `i < K` (util.h:502) is only right when I == K; this
@@ -64,6 +79,8 @@
  * (Halide/apps/cuda_mat_mul/runner.cpp:19-35), the CONSTANT capsule test
  * (correctness/multi-projection/capsule.cpp:75-102), 1x1-kernel/K=1 reductions
  * to GEMM, rank-1 closed forms for MTTKRP, and float64 einsum on random data.
+ * QRD: the driver's acceptance check on the driver's inputs, float64 numpy.linalg.qr (the
+ * factorisation is unique), exact triangular and Hadamard cases.
  * MTTKRP has no fixture, test or caller in the reference beyond util.h:498-515:
  * its parity is pinned only by that definition and by the mathematics.
  */
@@ -517,6 +534,57 @@ void oracle_pairhmm(const unsigned char *H, const unsigned char *R, const float 
             out[r * num_haps + h] = golden;
             free(col);
         }
+}
+
+/* QR factorisation of `batch` matrices by modified Gram-Schmidt (see the header for the
+ * reference lines).  A: [batch][m][n], element (k, j) at k*n + j (the spec's a(j, k, b), j
+ * innermost); Q: [batch][n][m], column i contiguous over k (QDeserializer(k, j, b)); R:
+ * [batch][n][n], row i contiguous over j, zero left of the diagonal as the driver fills it
+ * (qrd-run-fpga.cpp:583-596). */
+void oracle_qrd(const float *A, float *Q, float *R, int64_t m, int64_t n, int64_t batch, int acc, int threads) {
+    set_threads(threads);
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int64_t b = 0; b < batch; b++) {
+        float *t = (float *)malloc((size_t)(n * m + n) * sizeof(float));   /* columns, then X */
+        float *X = t + n * m;
+        const float *a = A + b * m * n;
+        float *q = Q + b * n * m, *r = R + b * n * n;
+        for (int64_t j = 0; j < n; j++)
+            for (int64_t k = 0; k < m; k++) t[j * m + k] = a[k * n + j];
+        for (int64_t i = 0; i < n; i++) {
+            const float *ti = t + i * m;
+            for (int64_t j = i; j < n; j++) {
+                const float *tj = t + j * m;
+                float x = 0.0f;
+                for (int64_t k = 0; k < m; k++) {
+                    if (acc == ORACLE_ACC_F32_FMA) {
+                        x = fmaf(ti[k], tj[k], x);
+                    } else {
+                        const float p = ti[k] * tj[k];
+                        x = x + p;
+                    }
+                }
+                X[j] = x;
+            }
+            const float xi = X[i];
+            const float ir = 1.0f / sqrtf(xi);
+            for (int64_t j = 0; j < n; j++) r[i * n + j] = j < i ? 0.0f : j == i ? sqrtf(xi) : ir * X[j];
+            for (int64_t k = 0; k < m; k++) q[i * m + k] = ir * ti[k];
+            for (int64_t j = i + 1; j < n; j++) {
+                float *tj = t + j * m;
+                const float s = -X[j] / xi;
+                for (int64_t k = 0; k < m; k++) {
+                    if (acc == ORACLE_ACC_F32_FMA) {
+                        tj[k] = fmaf(s, ti[k], tj[k]);
+                    } else {
+                        const float p = s * ti[k];
+                        tj[k] = tj[k] + p;
+                    }
+                }
+            }
+        }
+        free(t);
+    }
 }
 
 int oracle_max_threads(void) { return omp_get_max_threads(); }

@@ -56,6 +56,8 @@ def lib():
         up = ctypes.POINTER(ctypes.c_ubyte)
         _lib.oracle_pairhmm.argtypes = [up, up] + [fp] * 8 + [i64] * 4 + [ctypes.c_int, ctypes.c_int]
         _lib.oracle_pairhmm.restype = None
+        _lib.oracle_qrd.argtypes = [fp, fp, fp, i64, i64, i64, ctypes.c_int, ctypes.c_int]
+        _lib.oracle_qrd.restype = None
         _lib.oracle_max_threads.restype = ctypes.c_int
         for f in (_lib.oracle_fill_uniform, _lib.oracle_gemm, _lib.oracle_gemm_literal,
                   _lib.oracle_conv, _lib.oracle_capsule, _lib.oracle_mttkrp,
@@ -369,6 +371,29 @@ def pairhmm_inputs(num_haps, hap_len, num_reads, read_len, seed):
     bm, bg = (beta * (f32(1.0) - e)).astype(f32), (beta * e / f32(3.0)).astype(f32)
     H = np.ascontiguousarray(haps.T)                      # (hap_len, num_haps): haplotype index innermost
     return H, R, delta, zeta, eta, am, ag, bm, bg
+
+
+def qrd(A, acc=ACC_F32, threads=0):
+    """QR factorisation by modified Gram-Schmidt as the reference's UREs state it (qrd.cpp:51-63).
+    A: float32 (batch, m, n) -- numpy order of the reference's a(j, k, b).  Returns Q as float32
+    (batch, n, m) (numpy order of QDeserializer(k, j, b): Q[b, i] is column i) and R as float32
+    (batch, n, n) (numpy order of RDeserializer(j, i, b): R[b, i] is row i, zero left of the diagonal)."""
+    A = np.ascontiguousarray(A, dtype=np.float32)
+    batch, m, n = A.shape
+    Q = np.empty((batch, n, m), dtype=np.float32)
+    R = np.empty((batch, n, n), dtype=np.float32)
+    lib().oracle_qrd(_p(A), _p(Q), _p(R), m, n, batch, acc, threads)
+    return Q, R
+
+
+def qrd_driver_inputs(batch, m, n, seed=1138):
+    """The driver's inputs (qrd-run-fpga.cpp:108-123): srand(1138), then rand() % 9 + 1 as a float
+    for every element in b, k, j order.  Uses the C library's own rand(), as the driver does."""
+    libc = ctypes.CDLL(None)
+    libc.srand(ctypes.c_uint(seed))
+    libc.rand.restype = ctypes.c_int
+    vals = np.fromiter((libc.rand() % 9 + 1 for _ in range(batch * m * n)), dtype=np.float32, count=batch * m * n)
+    return vals.reshape(batch, m, n)
 
 
 def max_threads():

@@ -80,6 +80,10 @@ def _declare(L):
     L.pairhmm_ns.argtypes = [bp] * 10
     L.pairhmm_ns.restype = ctypes.c_double
     L.t2sp_pairhmm_f32.argtypes = [vp] * 10 + [i32] * 4 + [i64, i64, i32, i32, ctypes.POINTER(i64), vp]
+    L.qrd.argtypes = [bp] * 3
+    L.qrd_ns.argtypes = [bp] * 3
+    L.qrd_ns.restype = ctypes.c_double
+    L.t2sp_qrd_f32.argtypes = [vp, vp, vp, i32, i32, i32] + [i64] * 6 + [vp]
     L.t2sp_host_malloc.argtypes = [ctypes.c_size_t]
     L.t2sp_host_malloc.restype = ctypes.c_void_p
     L.t2sp_host_free.argtypes = [ctypes.c_void_p]

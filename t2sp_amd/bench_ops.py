@@ -227,6 +227,31 @@ def pairhmm_case(torch, steps, warmup, peak):
             "workload": "224 reads x 128 against 224 haplotypes x 384 (the size of the reference's README)"}
 
 
+def qrd_case(torch, steps, warmup, peak):
+    """Not one of the headline benchmark configurations: the batched QR pipeline (t2s/tests/performance/qrd) at the
+    size its README reports, 16384 matrices of 128 x 128 (23.3 K matrices/s on the FPGA).  The unit of work
+    is the matrix.  No matrix product: modified Gram-Schmidt takes m*n^2 fused multiply-adds per matrix
+    (one inner product and one update per pair of columns), so the roof is the vector issue rate,
+    256 CUs x 64 lanes x 2.4 GHz = 39.3e12 lane-instructions/s."""
+    L = lib()
+    batch, m, n = 16384, 128, 128
+    A = ops.fill_uniform(torch.empty(batch, m, n, device="cuda"), 1)
+    Q = torch.empty(batch, n, m, device="cuda")
+    R = torch.empty(batch, n, n, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        rc = L.t2sp_qrd_f32(A.data_ptr(), Q.data_ptr(), R.data_ptr(), m, n, batch, n, m * n, m, m * n, n, n * n, s)
+        assert rc == 0, rc
+
+    ms = _time(torch, launch, steps, warmup)
+    rate = batch / ms * 1e3
+    return {"Mmatrices/s": round(rate / 1e6, 3), "avg_launch_ms": round(ms, 5), "bound": "vector issue",
+            "frac_of_vector_issue_peak": round(rate * m * n * n / 39.3e12, 4),
+            "GB/s": round(rate * (m * n + n * m + n * n) * 4 / 1e9, 1),
+            "workload": "16384 matrices of 128 x 128 (the size of the reference's README)"}
+
+
 def run_all(torch, steps, warmup, peak, capsule_cfg=0, capsule_splits=0):
     return {"conv2d": conv_config3(torch, steps, warmup, peak),
             "capsule": capsule_config4(torch, steps, warmup, peak, capsule_cfg, capsule_splits),
@@ -237,4 +262,5 @@ def run_all(torch, steps, warmup, peak, capsule_cfg=0, capsule_splits=0):
             "sger_8192": sger_8192(torch, steps, warmup, peak),
             "sgbmv3_131072x1024": sgbmv3_case(torch, steps, warmup, peak),
             "ssymv_16384": ssymv_case(torch, steps, warmup, peak),
-            "pairhmm_224x224": pairhmm_case(torch, steps, warmup, peak)}
+            "pairhmm_224x224": pairhmm_case(torch, steps, warmup, peak),
+            "qrd_128x128_b16384": qrd_case(torch, steps, warmup, peak)}

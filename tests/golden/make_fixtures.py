@@ -4,7 +4,7 @@ and the outputs the CPU oracle gives for them in the reference's golden reductio
 Provenance: the reference stores no golden vectors for these operators -- its drivers recompute
 every expected value with naive loops at run time (gemm-run-fpga.cpp:74-86, conv-run-fpga.cpp:73-93,
 capsule-run-fpga.cpp:78-104, syrk-run-fpga.cpp:66-92, ger-run-fpga.cpp:63-73, gbmv3-run-fpga.cpp:108-114,
-symv-run-fpga.cpp:86-96, pairhmm-run-fpga.cpp:120-147, util.h:498-515).
+symv-run-fpga.cpp:86-96, pairhmm-run-fpga.cpp:120-147, qrd.cpp:51-63, util.h:498-515).
 These fixtures are therefore outputs of oracle/oracle.c, whose functions are pinned against the
 reference's closed forms and index mappings in tests/test_oracle.py.  They freeze those outputs so
 that a later change to the oracle or to a kernel cannot move both sides of a parity test at once.
@@ -31,6 +31,7 @@ CASES = {
     "gbmv3": dict(A=((12, 16), 1015), x=((27,), 1016), y=((12,), 1017)),
     "symv": dict(A=((20, 20), 1018), x=((20,), 1019), y=((20,), 1020)),
 }
+QRD = ((3, 24, 16), 1022)   # (batch, rows, columns), seed: uniform inputs
 PAIRHMM = dict(num_haps=6, hap_len=30, num_reads=5, read_len=20, seed=1021)   # inputs from oracle.pairhmm_inputs
 
 
@@ -53,6 +54,10 @@ def outputs():
         "symv": o.symv(*(inputs("symv")[k] for k in ("A", "x", "y")), 1.25, 0.75),
         "pairhmm": o.pairhmm(*o.pairhmm_inputs(**PAIRHMM)),
         "pairhmm_fused": o.pairhmm(*o.pairhmm_inputs(**PAIRHMM), acc=o.ACC_F32_FMA),
+        "qrd_q": o.qrd(o.fill_uniform(*QRD))[0],
+        "qrd_r": o.qrd(o.fill_uniform(*QRD))[1],
+        "qrd_q_fused": o.qrd(o.fill_uniform(*QRD), acc=o.ACC_F32_FMA)[0],
+        "qrd_r_fused": o.qrd(o.fill_uniform(*QRD), acc=o.ACC_F32_FMA)[1],
     }
 
 

@@ -124,6 +124,12 @@ def test_other_entries_reject_bad_arguments_without_a_device():
     assert L.symv(1.0, 1.0, sq.ref, v8.ref, v8.ref, None) == -12
     assert L.symv(1.0, 1.0, am.ref, v8.ref, v8.ref, v8.ref) == -8                # A not square
     assert L.symv(1.0, 1.0, sq.ref, _buf((7,)).ref, v8.ref, v8.ref) == -4
+    qa, qq, qr = _buf((2, 16, 8)), _buf((2, 8, 16)), _buf((2, 8, 8))            # numpy order of a(J, K, B), Q(K, J, B), R(J, J, B)
+    assert L.qrd(qa.ref, qq.ref, None) == -12
+    assert L.qrd(qa.ref, _buf((8, 16)).ref, qr.ref) == -43
+    assert L.qrd(qa.ref, _buf((2, 8, 15)).ref, qr.ref) == -8
+    assert L.qrd(qa.ref, qq.ref, _buf((2, 9, 8)).ref) == -4
+    assert L.qrd(_buf((1, 8, 129)).ref, _buf((1, 129, 8)).ref, _buf((1, 129, 129)).ref) == -8   # beyond 128 x 128
 
 
 def test_thin_layer_rejects_bad_shapes():
@@ -139,6 +145,9 @@ def test_thin_layer_rejects_bad_shapes():
     assert L.t2sp_sgbmv3_f32(1.0, 1.0, None, None, None, None, 0, 4, 4, None) == -8
     assert L.t2sp_ssymv_f32(1.0, 1.0, None, None, None, None, 0, 4, None, 0, None) == -8
     assert L.t2sp_ssymv_workspace_bytes(1000) == 8 * 8 * 128 * 4
+    assert L.t2sp_qrd_f32(None, None, None, 129, 8, 1, 8, 8 * 129, 129, 8 * 129, 8, 64, None) == -8
+    assert L.t2sp_qrd_f32(None, None, None, 16, 8, 1, 7, 128, 16, 128, 8, 64, None) == -8        # row stride below the row length
+    assert L.t2sp_qrd_f32(None, None, None, 16, 8, 0, 8, 128, 16, 128, 8, 64, None) == 0
     assert L.t2sp_mttkrp_workspace_bytes(512, 512, 512, 256, 1, 128) == 128 * 512 * 256 * 4
 
 

@@ -544,3 +544,60 @@ def test_gemm_ure_loop_nest_equals_golden_loop_bit_for_bit():
         III, II = consts[2], consts[4]
         part = o.gemm_ure(A, B, consts, blocks=(1, 2))
         assert (part == o.gemm_literal(A, B)[III * II:2 * III * II]).all()
+
+
+def _hadamard(n):
+    H = np.ones((1, 1), np.float32)
+    while H.shape[0] < n:
+        H = np.block([[H, H], [H, -H]])
+    return H
+
+
+def test_qrd_unique_factorisation_driver_check_and_closed_forms():
+    """Pins of the QR restatement.  (1) On the driver's own inputs (srand(1138), rand() % 9 + 1,
+    qrd-run-fpga.cpp:108-123) the driver's acceptance test holds: |Q R - A| < 0.005 element-wise
+    (qrd-run-fpga.cpp:627-640).  (2) A = Q R with orthonormal Q and a positive diagonal of R is unique:
+    float64 numpy.linalg.qr, signs normalised, agrees.  (3) Exact cases that fix the layouts and the
+    roles of sqrt and 1/sqrt: an upper-triangular A with powers of two on the diagonal gives Q = I and
+    R = A bit for bit (a transposed Q or R, or rows taken for columns, fails); 128 x 128 Hadamard columns
+    give R = sqrt(128) I with exact zeros elsewhere and Q = H / sqrt(128)."""
+    A = o.qrd_driver_inputs(3, 128, 128)
+    assert A.min() == 1 and A.max() == 9
+    for acc in (o.ACC_F32, o.ACC_F32_FMA):
+        Q, R = o.qrd(A, acc)
+        QR = np.einsum("bik,bij->bkj", Q.astype(np.float64), R.astype(np.float64))
+        assert np.abs(QR - A).max() < 0.005
+        assert (np.tril(R, -1) == 0).all() and (np.diagonal(R, axis1=1, axis2=2) > 0).all()
+        gram = np.einsum("bik,bjk->bij", Q.astype(np.float64), Q.astype(np.float64))
+        assert np.abs(gram - np.eye(128)).max() < 2e-4
+        for b in range(3):
+            q64, r64 = np.linalg.qr(A[b].astype(np.float64))
+            sign = np.sign(np.diag(r64))
+            assert np.abs(Q[b].T - q64 * sign).max() < 5e-5
+            assert np.abs(R[b] - (r64.T * sign).T).max() < 1e-4
+    Qa, Ra = o.qrd(A, o.ACC_F32)
+    Qf, Rf = o.qrd(A, o.ACC_F32_FMA)
+    assert np.linalg.norm(Qa - Qf) <= 1e-5 * np.linalg.norm(Qa) and np.linalg.norm(Ra - Rf) <= 1e-5 * np.linalg.norm(Ra)
+
+    rng = np.random.default_rng(5)
+    m, n = 12, 7                                      # rectangular: more rows than columns
+    U = np.triu(rng.integers(-3, 4, (m, n))).astype(np.float32)
+    U[np.arange(n), np.arange(n)] = 2.0 ** rng.integers(-2, 3, n)
+    Q, R = o.qrd(U[None])
+    assert Q.shape == (1, n, m) and R.shape == (1, n, n)
+    assert (Q[0] == np.eye(n, m, dtype=np.float32)).all()
+    assert (R[0] == U[:n]).all()
+
+    H = _hadamard(128)
+    Q, R = o.qrd(H[None])
+    root = np.sqrt(np.float32(128))
+    assert (R[0] == root * np.eye(128, dtype=np.float32)).all()
+    assert (Q[0].T == H * (np.float32(1) / root)).all()
+
+    # a rectangular random case against the unique factorisation, both layouts exercised
+    B = rng.standard_normal((2, 40, 17)).astype(np.float32)
+    Q, R = o.qrd(B)
+    for b in range(2):
+        q64, r64 = np.linalg.qr(B[b].astype(np.float64))
+        sign = np.sign(np.diag(r64))
+        assert np.abs(Q[b].T - q64 * sign).max() < 1e-5 and np.abs(R[b] - (r64.T * sign).T).max() < 1e-5
