@@ -195,9 +195,9 @@ __device__ __forceinline__ void qrd_wave(const QrdArgs &g, float (*pivot)[MR], f
         if (OWN && lane == p + 1) publish((i + 1) % 3, MR);
     };
 
-    // Two waves: while the pivots are in the first wave both take them from LDS, which costs a
-    // quarter of the vector-ALU slots of the register route but keeps the one LDS pipe of the CU
-    // busy; the first wave runs one step ahead and never waits for data.  Its barrier at the end of
+    // Two waves: while the pivots are in the first wave both take them from LDS, which needs less
+    // than half the vector-ALU time of the register route but loads the one LDS pipe of the CU;
+    // the first wave runs one step ahead and never waits for data.  Its barrier at the end of
     // step i pairs with the second wave's barrier before step i: by then column i, its squared
     // norm and column i + 1 are in their slots, and the first wave's next writes (the norm of
     // column i + 1, column i + 2) go to the two other slots of the three.
@@ -214,7 +214,7 @@ __device__ __forceinline__ void qrd_wave(const QrdArgs &g, float (*pivot)[MR], f
         }
         if (lane == 0) publish(64 % 3, MR / 2);
         for (int i = 64; i < g.n; i++) {
-            if (lane < 64) r[(int64_t)i * g.r_row + lane] = 0.f;          // the columns of the wave that has left
+            r[(int64_t)i * g.r_row + lane] = 0.f;                         // row i under the columns of the wave that has left
             __builtin_amdgcn_wave_barrier();                              // one wave: its LDS accesses stay in program order
             split_step(i, i - 64);
         }

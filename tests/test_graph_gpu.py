@@ -153,3 +153,35 @@ def test_partial_round_sgemm_padded_sgemm_and_pairhmm_in_one_graph(torch_cuda):
         ws.fill_(float(rep)); wso.fill_(float(rep))
 
     _replays_match(torch, g, out, eager, refill)
+
+
+def test_qrd_in_a_graph(torch_cuda):
+    """The QR kernel (two waves per matrix meeting at barriers, then one wave alone) replayed."""
+    torch = torch_cuda
+    L = t2sp_amd.lib()
+    batch, m, n = 40, 128, 128
+    A = t2sp_amd.fill_uniform(torch.empty(batch, m, n, device="cuda"), 31)
+    Q = torch.empty(batch, n, m, device="cuda")
+    R = torch.empty(batch, n, n, device="cuda")
+    out = torch.empty(Q.numel() + R.numel(), device="cuda")
+
+    def launch(stream):
+        assert L.t2sp_qrd_f32(A.data_ptr(), Q.data_ptr(), R.data_ptr(), m, n, batch, n, m * n, m, m * n, n, n * n, stream) == 0
+
+    def gather():
+        out[:Q.numel()] = Q.reshape(-1)
+        out[Q.numel():] = R.reshape(-1)
+
+    launch(torch.cuda.current_stream().cuda_stream)
+    gather()
+    torch.cuda.synchronize()
+    eager = out.clone()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        launch(torch.cuda.current_stream().cuda_stream)
+        gather()
+
+    def refill(rep):
+        Q.fill_(float("nan")); R.fill_(float("nan"))
+
+    _replays_match(torch, g, out, eager, refill)
