@@ -62,3 +62,17 @@ def test_syrk_and_mttkrp_random_shapes(oracle, seed):
         B, Cm, D = oracle.fill_uniform((I, J, K), 8), oracle.fill_uniform((J, R), 9), oracle.fill_uniform((K, R), 10)
         got = t2sp_amd.mttkrp(*t2sp_amd.mttkrp_reference_layout(B, Cm, D))
         assert rel_fro(got, oracle.mttkrp(B, Cm, D))[0] <= TOL, (I, J, K, R)
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_qrd_random_shapes(oracle, seed):
+    """Random row and column counts up to 128 (one wave or two per matrix, padded registers, vector
+    and scalar stores of Q): bit for bit against the oracle's fused variant."""
+    rnd = random.Random(400 + seed)
+    for _ in range(12):
+        n = rnd.randrange(1, 129)
+        m = rnd.randrange(n, 129)
+        A = oracle.fill_uniform((rnd.randrange(1, 5), m, n), 7 + seed)
+        Q, R = t2sp_amd.qrd(A)
+        Qf, Rf = oracle.qrd(A, acc=oracle.ACC_F32_FMA)
+        assert np.array_equal(Q, Qf, equal_nan=True) and np.array_equal(R, Rf, equal_nan=True), (m, n)
