@@ -311,8 +311,9 @@ __global__ void __launch_bounds__(NW * 64) capsule_direct_kernel(const CapsuleAr
 
 // The same idea on 16 x 16 MFMA tiles, for an even spread over the CUs.  With 32 x 128 tiles the
 // benchmark shape has 196 workgroups for 256 CUs; here a workgroup owns `rows_per_tile` vote rows
-// (whole pixels: a multiple of 4, up to 16*MB) by 32 columns, and the host picks rows_per_tile so
-// that the workgroups come to just under a multiple of 256 (252 tiles of 100 x 32 at the
+// (whole pixels: a multiple of 4, up to 16*MB) by NB blocks of 16 columns, and the host picks NB and
+// rows_per_tile so that the workgroups come to just under a multiple of 256 (see plan_direct16; 256
+// tiles of 196 x 16 at the
 // benchmark shape).  v_mfma_f32_16x16x4_f32 takes per lane one float of X at (row l%16, k-slot
 // l/16) and of Y at (k-slot l/16, col l%16) and leaves D[4*(l/16) + r][l%16] in register r.  A step
 // is 4 pose rows of the reduction (16 k): lane group l/16 loads pose row 4*step + l/16 as 128 bits
@@ -321,21 +322,22 @@ __global__ void __launch_bounds__(NW * 64) capsule_direct_kernel(const CapsuleAr
 // The reduction is split over the 4 waves and summed through LDS in wave order, as above.
 constexpr int D16_WAVES = 4;
 constexpr int D16_RING = 3;
-constexpr int D16_MAX_MB = 8;
+constexpr int D16_MAX_MB = 8;        // row blocks of 16 per workgroup with two column blocks
+constexpr int D16_MAX_MB_TALL = 13;  // with one
 typedef float v4f_acc __attribute__((ext_vector_type(4)));
 
-template <int MB, int NW, int R>
+template <int MB, int NB, int NW, int R>
 __global__ void __launch_bounds__(NW * 64) capsule_direct16_kernel(const CapsuleArgs g, int rows_per_tile,
                                                                    int tab_entries) {
     extern __shared__ __align__(16) float smem[];
     v4f *red = reinterpret_cast<v4f *>(smem);                                   // [wave][mb][nb][lane]
-    uint32_t *pix_p = reinterpret_cast<uint32_t *>(smem + NW * MB * 2 * 64 * 4);  // [4*MB] byte offsets in P
+    uint32_t *pix_p = reinterpret_cast<uint32_t *>(smem + NW * MB * NB * 64 * 4);  // [4*MB] byte offsets in P
     uint32_t *pix_v = pix_p + 4 * MB;                                            // [4*MB] byte offsets in V, ~0u: none
     uint2 *tab_all = reinterpret_cast<uint2 *>(pix_v + 4 * MB);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
     const int tm = blockIdx.x % g.tiles_m, tn = blockIdx.x / g.tiles_m;   // the column tiles of one row tile: same XCD
-    const int r0 = tm * rows_per_tile, n0 = tn * 32;
+    const int r0 = tm * rows_per_tile, n0 = tn * 16 * NB;
 
     // pixels of this tile: offsets of (n, h, w) in P and in V
     const int pix_total = g.ROWS >> 2, pix0 = r0 >> 2, pix_n = min(rows_per_tile >> 2, pix_total - pix0);
@@ -360,12 +362,12 @@ __global__ void __launch_bounds__(NW * 64) capsule_direct16_kernel(const Capsule
     }
     __syncthreads();
 
-    uint32_t p_lane[MB], w_lane[2], v_lane[2];
+    uint32_t p_lane[MB], w_lane[NB], v_lane[NB];
 #pragma unroll
     for (int mb = 0; mb < MB; mb++) p_lane[mb] = pix_p[4 * mb + (li >> 2)] + 4u * (uint32_t)((li & 3) * (int)g.sp[4]);
-    bool col_ok[2];
+    bool col_ok[NB];
 #pragma unroll
-    for (int nb = 0; nb < 2; nb++) {
+    for (int nb = 0; nb < NB; nb++) {
         const int col = n0 + 16 * nb + li;
         col_ok[nb] = col < g.COLS;
         const int co = col_ok[nb] ? col >> 2 : 0;
@@ -378,7 +380,7 @@ __global__ void __launch_bounds__(NW * 64) capsule_direct16_kernel(const Capsule
     for (int j = 0; j < 4; j++) w_base[j] = reinterpret_cast<const char *>(g.W + j * g.sw[4]);
 
     v4f ra[R][MB];
-    float rb[R][2][4];
+    float rb[R][NB][4];
     const uint2 *tab_lane = tab + lq;
     uint2 off = tab_lane[0];
     int t_issue = 0;
@@ -387,17 +389,17 @@ __global__ void __launch_bounds__(NW * 64) capsule_direct16_kernel(const Capsule
         const uint32_t op = off.x, ow = off.y;                                                     \
         t_issue++;                                                                                 \
         off = tab_lane[4 * t_issue];                                                               \
-        _Pragma("unroll") for (int nb = 0; nb < 2; nb++)                                           \
+        _Pragma("unroll") for (int nb = 0; nb < NB; nb++)                                          \
             _Pragma("unroll") for (int j = 0; j < 4; j++)                                          \
                 rb[d][nb][j] = *reinterpret_cast<const float *>(w_base[j] + (w_lane[nb] + ow));    \
         _Pragma("unroll") for (int mb = 0; mb < MB; mb++)                                          \
             ra[d][mb] = *reinterpret_cast<const v4f *>(p_base + (p_lane[mb] + op));                \
     }
-    v4f_acc acc[MB][2];
+    v4f_acc acc[MB][NB];
 #pragma unroll
     for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-        for (int nb = 0; nb < 2; nb++) acc[mb][nb] = v4f_acc{0.f, 0.f, 0.f, 0.f};
+        for (int nb = 0; nb < NB; nb++) acc[mb][nb] = v4f_acc{0.f, 0.f, 0.f, 0.f};
 
 #pragma unroll
     for (int d = 0; d < R - 1; d++) {
@@ -415,9 +417,9 @@ __global__ void __launch_bounds__(NW * 64) capsule_direct16_kernel(const Capsule
 #pragma unroll
                 for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-                    for (int nb = 0; nb < 2; nb++)
+                    for (int nb = 0; nb < NB; nb++)
                         acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[d][mb][j], rb[d][nb][j], acc[mb][nb], 0, 0, 0);
-            T2SP_INTERLEAVE(SG_VMEM_READ, MB + 8, (8 * MB) / (MB + 8))
+            T2SP_INTERLEAVE(SG_VMEM_READ, MB + 4 * NB, (4 * NB * MB) / (MB + 4 * NB))
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -433,7 +435,7 @@ __global__ void __launch_bounds__(NW * 64) capsule_direct16_kernel(const Capsule
                 for (int mb = 0; mb < MB; mb++) {
                     const float a = live ? ra[d][mb][j] : 0.f;
 #pragma unroll
-                    for (int nb = 0; nb < 2; nb++)
+                    for (int nb = 0; nb < NB; nb++)
                         acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, rb[d][nb][j], acc[mb][nb], 0, 0, 0);
                 }
         }
@@ -441,20 +443,20 @@ __global__ void __launch_bounds__(NW * 64) capsule_direct16_kernel(const Capsule
 
     // sum the partial tiles of the waves in wave order; register r of a lane is vote row mx = r of
     // pixel 4*mb + l/16 of the tile, column l%16 of the block
-    v4f *mine = red + wave * MB * 2 * 64 + lane;
+    v4f *mine = red + wave * MB * NB * 64 + lane;
 #pragma unroll
     for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-        for (int nb = 0; nb < 2; nb++) mine[(mb * 2 + nb) * 64] = acc[mb][nb];
+        for (int nb = 0; nb < NB; nb++) mine[(mb * NB + nb) * 64] = acc[mb][nb];
     __syncthreads();
     char *v_base = reinterpret_cast<char *>(g.V);
     const uint32_t mx_stride = 4u * (uint32_t)(int)g.sv[4];
-    for (int pr = wave; pr < 2 * MB; pr += NW) {
+    for (int pr = wave; pr < NB * MB; pr += NW) {
         const v4f *src = red + pr * 64 + lane;
         v4f sum = src[0];
 #pragma unroll
-        for (int wv = 1; wv < NW; wv++) sum += src[wv * MB * 2 * 64];
-        const int mb = pr >> 1, nb = pr & 1;
+        for (int wv = 1; wv < NW; wv++) sum += src[wv * MB * NB * 64];
+        const int mb = pr / NB, nb = pr % NB;
         const uint32_t pv = pix_v[4 * mb + lq];
         if (pv != ~0u && col_ok[nb]) {
 #pragma unroll
@@ -554,37 +556,50 @@ static CapsulePlan plan_capsule(int rows, int cols, int kred, int cfg, int split
 // The 16 x 16 form: rows per tile (a multiple of 4, at most 16 * D16_MAX_MB) such that the workgroups
 // fill whole rounds of 256 as evenly as possible.
 struct Direct16Plan {
-    int rows_per_tile, mb, tiles_m, tiles_n;
+    int rows_per_tile, mb, nb, tiles_m, tiles_n, rounds;
 };
-static Direct16Plan plan_direct16(int rows, int cols) {
+// Rows per tile for workgroups that are `nb` column blocks (of 16) wide and at most max_mb row
+// blocks tall, in as few rounds of 256 workgroups as that allows.
+static Direct16Plan plan_direct16_for(int rows, int cols, int nb, int max_mb) {
     Direct16Plan p{};
-    p.tiles_n = (cols + 31) / 32;
+    p.nb = nb;
+    p.tiles_n = (cols + 16 * nb - 1) / (16 * nb);
     for (int rounds = 1;; rounds++) {
         const int want_m = (rounds * 256) / p.tiles_n > 0 ? (rounds * 256) / p.tiles_n : 1;
         int rpt = ((rows + want_m - 1) / want_m + 3) / 4 * 4;
         if (rpt < 64) rpt = 64;
-        if (rpt <= 16 * D16_MAX_MB) {
+        if (rpt <= 16 * max_mb) {
             p.rows_per_tile = rpt;
             p.mb = (rpt + 15) / 16;
             p.tiles_m = (rows + rpt - 1) / rpt;
+            p.rounds = rounds;
             return p;
         }
     }
+}
+// Two column blocks per workgroup share every input load between them; one column block allows
+// taller tiles, which can land closer to an even split of the rows (196 rows = 13 blocks x 256
+// workgroups against 100 rows = 7 x 2 blocks x 252 at the benchmark shape).  The time goes with
+// rounds x MFMA blocks per workgroup.
+static Direct16Plan plan_direct16(int rows, int cols) {
+    const Direct16Plan wide = plan_direct16_for(rows, cols, 2, D16_MAX_MB);
+    const Direct16Plan tall = plan_direct16_for(rows, cols, 1, D16_MAX_MB_TALL);
+    return tall.rounds * tall.mb < wide.rounds * wide.mb * 2 ? tall : wide;
 }
 static int direct16_tab_entries(int kred) {
     const int steps = (kred / 4 + 3) / 4;
     return 4 * ((steps + D16_WAVES - 1) / D16_WAVES) + 4 * D16_RING + 4;
 }
-static size_t direct16_smem_bytes(int mb, int kred) {
-    return (size_t)D16_WAVES * mb * 2 * 64 * sizeof(v4f) + 2 * 4 * mb * sizeof(uint32_t) +
+static size_t direct16_smem_bytes(int mb, int nb, int kred) {
+    return (size_t)D16_WAVES * mb * nb * 64 * sizeof(v4f) + 2 * 4 * mb * sizeof(uint32_t) +
            (size_t)D16_WAVES * direct16_tab_entries(kred) * sizeof(uint2);
 }
 
-template <int MB>
+template <int MB, int NB>
 static int launch_direct16_mb(const CapsuleArgs &g, const Direct16Plan &p, hipStream_t stream) {
-    const size_t smem = direct16_smem_bytes(MB, g.KRED);
+    const size_t smem = direct16_smem_bytes(MB, NB, g.KRED);
     if (smem > 160 * 1024) return T2SP_ERR_SHAPE;
-    auto kern = capsule_direct16_kernel<MB, D16_WAVES, D16_RING>;
+    auto kern = capsule_direct16_kernel<MB, NB, D16_WAVES, D16_RING>;
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(D16_WAVES * 64), smem, stream, g, p.rows_per_tile,
@@ -596,12 +611,27 @@ static int launch_capsule_direct16(CapsuleArgs g, hipStream_t stream) {
     const Direct16Plan p = plan_direct16(g.ROWS, g.COLS);
     g.tiles_m = p.tiles_m;
     g.tiles_n = p.tiles_n;
+    if (p.nb == 2) {
+        switch (p.mb) {
+            case 4: return launch_direct16_mb<4, 2>(g, p, stream);
+            case 5: return launch_direct16_mb<5, 2>(g, p, stream);
+            case 6: return launch_direct16_mb<6, 2>(g, p, stream);
+            case 7: return launch_direct16_mb<7, 2>(g, p, stream);
+            case 8: return launch_direct16_mb<8, 2>(g, p, stream);
+            default: return T2SP_ERR_SHAPE;
+        }
+    }
     switch (p.mb) {
-        case 4: return launch_direct16_mb<4>(g, p, stream);
-        case 5: return launch_direct16_mb<5>(g, p, stream);
-        case 6: return launch_direct16_mb<6>(g, p, stream);
-        case 7: return launch_direct16_mb<7>(g, p, stream);
-        case 8: return launch_direct16_mb<8>(g, p, stream);
+        case 4: return launch_direct16_mb<4, 1>(g, p, stream);
+        case 5: return launch_direct16_mb<5, 1>(g, p, stream);
+        case 6: return launch_direct16_mb<6, 1>(g, p, stream);
+        case 7: return launch_direct16_mb<7, 1>(g, p, stream);
+        case 8: return launch_direct16_mb<8, 1>(g, p, stream);
+        case 9: return launch_direct16_mb<9, 1>(g, p, stream);
+        case 10: return launch_direct16_mb<10, 1>(g, p, stream);
+        case 11: return launch_direct16_mb<11, 1>(g, p, stream);
+        case 12: return launch_direct16_mb<12, 1>(g, p, stream);
+        case 13: return launch_direct16_mb<13, 1>(g, p, stream);
         default: return T2SP_ERR_SHAPE;
     }
 }
@@ -701,7 +731,7 @@ extern "C" int t2sp_capsule_f32(const float *P, const float *W, float *V, const 
     if (p.cfg == T2SP_CFG_DIRECT && !(byte_offsets_fit && direct_smem_bytes((int)kred) <= 160 * 1024))
         p = plan_capsule((int)rows, (int)cols, (int)kred, T2SP_CFG_128x128, 1);   // needs no workspace either
     if (p.cfg == T2SP_CFG_DIRECT16 &&
-        !(byte_offsets_fit && d[8] == 4 && direct16_smem_bytes(D16_MAX_MB, (int)kred) <= 160 * 1024))
+        !(byte_offsets_fit && d[8] == 4 && direct16_smem_bytes(D16_MAX_MB, 2, (int)kred) <= 160 * 1024))
         p = plan_capsule((int)rows, (int)cols, (int)kred, T2SP_CFG_128x128, 1);
     if (p.scratch_bytes > workspace_bytes || (p.scratch_bytes && !workspace)) return T2SP_ERR_SHAPE;
     CapsuleArgs g{};

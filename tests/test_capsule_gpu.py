@@ -69,6 +69,17 @@ def test_short_and_odd_reductions_ragged_columns(oracle, ci, co, n, cfg):
     assert err <= TOL, (ci, co, n, cfg, err, mx)
 
 
+@pytest.mark.parametrize("n,co", [(23, 32), (28, 32), (32, 16), (27, 20), (20, 32), (40, 64)])
+def test_direct16_tile_plans(oracle, n, co):
+    """Shapes that make the 16 x 16 direct kernel pick each of its tile forms: one column block and
+    9, 11 or 7 row blocks per workgroup (the second with ragged columns), two column blocks and 4 or
+    8 row blocks, in one round of workgroups and in two."""
+    P, W = oracle.fill_uniform((n, 6, 15, 15, 4, 4), 60 + n), oracle.fill_uniform((co, 6, 3, 3, 4, 4), 70 + co)
+    got = t2sp_amd.capsule(P, W, cfg=6)
+    err, mx = rel_fro(got, oracle.capsule(P, W))
+    assert err <= TOL, (n, co, err, mx)
+
+
 def test_other_pose_sizes_take_the_scalar_kernel(oracle):
     P, W = oracle.fill_uniform((1, 3, 5, 5, 2, 3), 7), oracle.fill_uniform((2, 3, 3, 3, 3, 5), 8)
     assert rel_fro(t2sp_amd.capsule(P, W), oracle.capsule(P, W))[0] <= TOL
