@@ -23,8 +23,9 @@
 // The first costs LDS time (one pipe per CU, and a one-lane store of 128 values is as slow as a
 // full one), the second two vector-ALU slots per value.  With two waves per matrix, both take
 // the pivots of the first 64 steps through LDS; the first wave never waits for the second and
-// leaves when its columns are finished, and the second takes the last 64 pivots from its own
-// registers.  Row i of R is stored as soon as step i knows it (lanes along the row).  A column
+// leaves when its columns are finished, and the second, then alone, splits each of the last 64
+// pivots between the two routes (rows 0..MR/2-1 through LDS, the rest from its own registers),
+// as does a matrix of at most 64 columns from the start.  Row i of R is stored as soon as step i knows it (lanes along the row).  A column
 // is final once it has been the pivot, so Q is written at the end: every lane scales its own
 // column and stores it (contiguous per lane).
 #include <hip/hip_runtime.h>
