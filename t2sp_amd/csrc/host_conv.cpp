@@ -31,6 +31,78 @@ bool dense_nchw(const Logical4 &t) {
 }
 }  // namespace
 
+// Large convolutions on dense host buffers: the images go through the device in panels, so that
+// the upload of the next panel and the download of the previous one overlap with the kernels of
+// the current one (streams and events of panel_streams()).  Images are independent, the weights go
+// up once.  A panel holds enough images for a full round of 256 output tiles; returns the images
+// per panel, or 0 when the convolution should run in one piece.
+static int conv_panel_images(int64_t N, int64_t CI, int64_t CO, int64_t OH, int64_t OW, int64_t KH, int64_t KW) {
+    if (2.0 * N * CO * OH * OW * CI * KH * KW < 5e10) return 0;        // small: the copies are short anyway
+    const double tiles_per_image = (double)(OH * OW) / 256.0 * (double)((CO + 255) / 256);
+    int64_t images = (int64_t)(256.0 / tiles_per_image) + 1;
+    int64_t panels = N / images;
+    if (panels > MAX_PANELS) panels = MAX_PANELS;
+    if (panels < 2) return 0;
+    return (int)((N + panels - 1) / panels);
+}
+
+static int conv_panels(halide_buffer_t *I, halide_buffer_t *K, halide_buffer_t *O, int images, int64_t N, int64_t CI,
+                       int64_t CO, int64_t OH, int64_t OW, int64_t KH, int64_t KW) {
+    static const char *op = "conv";
+    PanelStreams &ps = panel_streams();
+    if (!ps.ok) return 1;                                       // caller falls back to the one-piece path
+    const int64_t IH = OH + KH - 1, IW = OW + KW - 1;
+    const size_t image_in = (size_t)(CI * IH * IW), image_out = (size_t)(CO * OH * OW), k_elems = (size_t)(CO * CI * KH * KW);
+    const float *hi = reinterpret_cast<const float *>(I->host), *hk = reinterpret_cast<const float *>(K->host);
+    float *ho = reinterpret_cast<float *>(O->host);
+    float *di = static_cast<float *>(pool().get(N * image_in * sizeof(float)));
+    float *dk = static_cast<float *>(pool().get(k_elems * sizeof(float)));
+    float *dout = static_cast<float *>(pool().get(N * image_out * sizeof(float)));
+    const size_t ws_bytes = t2sp_conv2d_workspace_bytes(images, (int)CI, (int)CO, (int)OH, (int)OW, (int)KH, (int)KW);
+    float *ws = ws_bytes ? static_cast<float *>(pool().get(ws_bytes)) : nullptr;
+    struct Put { float *p[4]; ~Put() { for (float *q : p) if (q) pool().put(q); } } put{{di, dk, dout, ws}};
+    if (!di || !dk || !dout) return report(halide_error_code_device_malloc_failed, op, "device allocation failed");
+    auto fail = [&](int code, const char *what) {
+        (void)hipDeviceSynchronize();
+        (void)hipGetLastError();
+        return report(code, op, what);
+    };
+    const int64_t si4[4] = {(int64_t)image_in, IH * IW, IW, 1}, sk4[4] = {CI * KH * KW, KH * KW, KW, 1},
+                  so4[4] = {(int64_t)image_out, OH * OW, OW, 1};
+    if (hipMemcpyAsync(dk, hk, k_elems * sizeof(float), hipMemcpyHostToDevice, ps.in) != hipSuccess)
+        return fail(halide_error_code_copy_to_device_failed, "host to device copy failed");
+    const int panels = (int)((N + images - 1) / images);
+    for (int p = 0; p < panels; p++) {
+        const int64_t n0 = (int64_t)p * images, nn = N - n0 < images ? N - n0 : images;
+        if (hipMemcpyAsync(di + n0 * image_in, hi + n0 * image_in, nn * image_in * sizeof(float), hipMemcpyHostToDevice,
+                           ps.in) != hipSuccess)
+            return fail(halide_error_code_copy_to_device_failed, "host to device copy failed");
+        (void)hipEventRecord(ps.up[p], ps.in);
+        (void)hipStreamWaitEvent(api_stream(), ps.up[p], 0);
+        (void)hipEventRecord(ps.k0[p], api_stream());
+        const int err = t2sp_conv2d_f32(di + n0 * image_in, dk, dout + n0 * image_out, (int)nn, (int)CI, (int)CO, (int)OH,
+                                        (int)OW, (int)KH, (int)KW, si4, sk4, so4, T2SP_CFG_AUTO, ws, ws ? ws_bytes : 0,
+                                        api_stream());
+        if (err) return fail(err, "kernel launch failed");
+        (void)hipEventRecord(ps.k1[p], api_stream());
+        (void)hipStreamWaitEvent(ps.out, ps.k1[p], 0);
+        if (hipMemcpyAsync(ho + n0 * image_out, dout + n0 * image_out, nn * image_out * sizeof(float), hipMemcpyDeviceToHost,
+                           ps.out) != hipSuccess)
+            return fail(halide_error_code_copy_to_host_failed, "device to host copy failed");
+    }
+    if (hipStreamSynchronize(ps.out) != hipSuccess || hipStreamSynchronize(api_stream()) != hipSuccess ||
+        hipStreamSynchronize(ps.in) != hipSuccess)
+        return fail(halide_error_code_device_run_failed, "kernel execution failed");
+    double ns = 0.0;
+    for (int p = 0; p < panels; p++) {
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, ps.k0[p], ps.k1[p]) == hipSuccess) ns += (double)ms * 1e6;
+    }
+    publish_kernel_ns(ns, op);
+    O->flags &= ~(uint64_t)(halide_buffer_flag_device_dirty | halide_buffer_flag_host_dirty);
+    return 0;
+}
+
 static int conv_impl(halide_buffer_t *I, halide_buffer_t *K, halide_buffer_t *O, int cfg) {
     static const char *op = "conv";
     std::lock_guard<std::mutex> lock(api_mutex());
@@ -88,6 +160,18 @@ static int conv_impl(halide_buffer_t *I, halide_buffer_t *K, halide_buffer_t *O,
     lk.ext[0] = CO; lk.ext[1] = CI; lk.ext[2] = KH; lk.ext[3] = KW;
     if (N * OH * ((OW + 3) / 4 * 4) > INT32_MAX || CI * KH * KW > INT32_MAX)
         return report(halide_error_code_buffer_extents_too_large, op, "problem too large for 32-bit tile indices");
+
+    // dense NCHW / OIHW host buffers: large convolutions run in panels of images
+    const bool host_only = !I->device && !K->device && !O->device && I->host && K->host && O->host;
+    if (host_only && !packed && O->dimensions == 4 && cfg == T2SP_CFG_AUTO && OW >= 4 && dense_nchw(li) && dense_nchw(lk) &&
+        so.span == so.elements && od[0].stride == 1 && od[1].stride == OW && od[2].stride == OW * OH &&
+        od[3].stride == OW * OH * CO && (CI * IH * IW) % 4 == 0 && (CO * OH * OW) % 4 == 0) {
+        const int images = conv_panel_images(N, CI, CO, OH, OW, KH, KW);
+        if (images > 0) {
+            const int rc = conv_panels(I, K, O, images, N, CI, CO, OH, OW, KH, KW);
+            if (rc <= 0) return rc;                             // done, or failed with a code; 1 = no streams
+        }
+    }
 
     Staged di, dk, dout;
     if ((err = di.input(I, si, op))) return err;

@@ -19,29 +19,10 @@ using namespace t2sp;
 // Large products on host buffers: the rows of A and C go through the device in panels, so that the
 // upload of the next panel and the download of the previous one overlap with the product of the
 // current one (the reference copies everything in, runs, copies everything out:
-// AOT-OpenCL-Runtime.cpp:402-441).  Three streams of default priority: copies in, kernels (the
-// library stream), copies out, chained by events.  Panels are whole multiples of 256 rows (and of
-// the tiled output's III * II), at least one full round of 256 tiles each.
+// AOT-OpenCL-Runtime.cpp:402-441), on the three streams of panel_streams().  Panels are whole
+// multiples of 256 rows (and of the tiled output's III * II), at least one full round of 256 tiles
+// each.
 namespace {
-constexpr int MAX_PANELS = 8;
-struct PanelStreams {
-    hipStream_t in = nullptr, out = nullptr;
-    hipEvent_t up[MAX_PANELS], k0[MAX_PANELS], k1[MAX_PANELS];
-    bool ok = false;
-    PanelStreams() {
-        ok = hipStreamCreateWithFlags(&in, hipStreamNonBlocking) == hipSuccess &&
-             hipStreamCreateWithFlags(&out, hipStreamNonBlocking) == hipSuccess;
-        for (int i = 0; i < MAX_PANELS && ok; i++)
-            ok = hipEventCreate(&up[i]) == hipSuccess && hipEventCreate(&k0[i]) == hipSuccess &&
-                 hipEventCreate(&k1[i]) == hipSuccess;
-        if (!ok) (void)hipGetLastError();
-    }
-};
-PanelStreams &panel_streams() {
-    static PanelStreams s;
-    return s;
-}
-
 // Rows per panel, or 0 when the product should run in one piece.
 int panel_rows(int M, int N, int K, int64_t row_quantum) {
     if ((double)M * N * K < 1e11 || N < 256) return 0;          // small: the copies are short anyway

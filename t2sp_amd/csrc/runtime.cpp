@@ -180,6 +180,20 @@ int Staged::finish(const char *op) {
     return 0;
 }
 
+PanelStreams::PanelStreams() {
+    ok = hipStreamCreateWithFlags(&in, hipStreamNonBlocking) == hipSuccess &&
+         hipStreamCreateWithFlags(&out, hipStreamNonBlocking) == hipSuccess;
+    for (int i = 0; i < MAX_PANELS && ok; i++)
+        ok = hipEventCreate(&up[i]) == hipSuccess && hipEventCreate(&k0[i]) == hipSuccess &&
+             hipEventCreate(&k1[i]) == hipSuccess;
+    if (!ok) (void)hipGetLastError();
+}
+
+PanelStreams &panel_streams() {
+    static PanelStreams s;
+    return s;
+}
+
 KernelTimer::KernelTimer() {
     if (!g_ev0) {
         (void)hipEventCreate(&g_ev0);

@@ -97,6 +97,20 @@ private:
 // and, when $T2SP_EXEC_TIME_FILE names a file, what is written there in the reference's format).
 void publish_kernel_ns(double ns, const char *op);
 
+// Streams and events for operator entries that move large host buffers through the device in
+// panels: copies in, kernels (the library stream), copies out, chained by events so that the upload
+// of the next panel and the download of the previous one overlap with the kernels of the current
+// one (the reference copies everything in, runs, copies everything out:
+// AOT-OpenCL-Runtime.cpp:402-441).  Default priority, created on first use, kept for the process.
+constexpr int MAX_PANELS = 8;
+struct PanelStreams {
+    hipStream_t in = nullptr, out = nullptr;
+    hipEvent_t up[MAX_PANELS], k0[MAX_PANELS], k1[MAX_PANELS];
+    bool ok = false;
+    PanelStreams();
+};
+PanelStreams &panel_streams();
+
 class KernelTimer {
 public:
     KernelTimer();

@@ -179,3 +179,26 @@ def test_config3_full_size_sampled_and_shift_property(oracle):
     Wd = torch.zeros_like(W)
     Wd[torch.arange(C), torch.arange(C), 1, 2] = 1.0
     assert torch.equal(t2sp_amd.conv(I, Wd), I[:, :, 1:OH + 1, 2:OH + 2])
+
+
+def test_large_host_buffers_run_in_image_panels(oracle):
+    """Dense NCHW host buffers of a large convolution take the panel path of `conv` (images uploaded,
+    convolved and downloaded in two or more overlapping panels): same result as the one-piece path on
+    device buffers, and the oracle on the first and last image (one in each panel)."""
+    import torch
+    N, C, OH = 48, 192, 56
+    I = t2sp_amd.host_empty((N, C, OH + 2, OH + 2))
+    W = t2sp_amd.host_empty((C, C, 3, 3))
+    I[...] = oracle.fill_uniform(I.shape, 51)
+    W[...] = oracle.fill_uniform(W.shape, 52)
+    O = t2sp_amd.host_empty((N, C, OH, OH))
+    O[...] = np.nan
+    t2sp_amd.conv(I, W, out=O)
+    assert t2sp_amd.last_kernel_ns() > 0
+    Od = t2sp_amd.conv(torch.from_numpy(np.ascontiguousarray(I)).cuda(), torch.from_numpy(np.ascontiguousarray(W)).cuda())
+    assert rel_fro(O, Od.cpu().numpy())[0] <= 1e-6
+    cos = slice(40, 52)
+    In, Wn = I[[0, N - 1]].transpose(0, 1, 3, 2), W.transpose(0, 1, 3, 2)
+    ref = oracle.conv(np.ascontiguousarray(In), np.ascontiguousarray(Wn), co_range=(cos.start, cos.stop))[:, cos]
+    got = O[[0, N - 1]][:, cos].transpose(0, 1, 3, 2)
+    assert rel_fro(got, ref)[0] <= TOL
