@@ -120,3 +120,21 @@ def test_error_codes(oracle):
         t2sp_amd.qrd(A, out=(np.zeros((2, 8, 15), np.float32), np.zeros((2, 8, 8), np.float32)))
     assert e.value.code == -8
     assert t2sp_amd.lib().t2sp_qrd_f32(None, None, None, 200, 8, 1, 8, 1600, 200, 1600, 8, 64, None) != 0
+
+
+def test_large_host_batch_runs_in_panels(oracle):
+    """A dense host batch of 64 MB takes the panel path of `qrd` (matrices uploaded, factored and
+    downloaded in eight overlapping panels): bit for bit the one-piece result of device buffers."""
+    import torch
+    batch = 1030                                           # not a multiple of the panel count
+    A = t2sp_amd.host_empty((batch, 128, 128))
+    A[...] = oracle.fill_uniform(A.shape, 91)
+    Q, R = t2sp_amd.host_empty((batch, 128, 128)), t2sp_amd.host_empty((batch, 128, 128))
+    Q[...] = np.nan
+    R[...] = np.nan
+    t2sp_amd.qrd(A, out=(Q, R))
+    assert t2sp_amd.last_kernel_ns() > 0
+    Qd, Rd = t2sp_amd.qrd(torch.from_numpy(np.ascontiguousarray(A)).cuda())
+    assert np.array_equal(Q, Qd.cpu().numpy()) and np.array_equal(R, Rd.cpu().numpy())
+    Qf, Rf = oracle.qrd(A[[0, batch - 1]], acc=oracle.ACC_F32_FMA)
+    assert np.array_equal(Q[[0, batch - 1]], Qf) and np.array_equal(R[[0, batch - 1]], Rf)
