@@ -206,6 +206,21 @@ int t2sp_mttkrp_f32(const float *B, const float *C, const float *D, float *A, in
                     const int64_t *sa2, int cfg, int splits, float *workspace,
                     size_t workspace_bytes, void *stream);
 
+/* t2sp_mttkrp_f32 for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same arguments minus the workspace: the partial planes of the split reduction (and the padded
+ * copies of sizes off the vector grid) live in an array of T2SP_MTTKRP_NOALLOC_SCRATCH_BYTES that
+ * is part of the library's device image; each GPU the library runs on holds it until the process
+ * ends.  The benchmark size (I = J = K = 512, R = 256: 128 planes of 0.5 MB) fits exactly; a
+ * product that needs more returns T2SP_ERR_SHAPE with a message.  The call itself allocates and
+ * frees nothing.  All calls on one GPU share the array: calls that overlap on one GPU (different
+ * streams or threads) race; calls on one stream are ordered and safe.  Same results, bit for
+ * bit, as t2sp_mttkrp_f32 with a workspace. */
+#define T2SP_MTTKRP_NOALLOC_SCRATCH_BYTES (64u << 20)
+int t2sp_mttkrp_f32_noalloc(const float *B, const float *C, const float *D, float *A, int I, int J,
+                            int K, int R, const int64_t *sb3, const int64_t *sc2, const int64_t *sd2,
+                            const int64_t *sa2, int cfg, int splits, void *stream);
+
 /* dst[sum_d c_d*dst_strides[d]] = src[sum_d c_d*src_strides[d]] for every coordinate c of the
  * box `extents` (nd <= T2SP_MAX_DIMS, dimension 0 fastest).  Device-side replacement of the
  * host serializer/deserializer loops the reference's generated interface runs around its

@@ -106,6 +106,7 @@ def _declare(L):
     L.t2sp_mttkrp_workspace_bytes.argtypes = [i32, i32, i32, i32, i32, i32]
     L.t2sp_mttkrp_workspace_bytes.restype = sz
     L.t2sp_mttkrp_f32.argtypes = [vp, vp, vp, vp, i32, i32, i32, i32, p64, p64, p64, p64, i32, i32, vp, sz, vp]
+    L.t2sp_mttkrp_f32_noalloc.argtypes = [vp, vp, vp, vp, i32, i32, i32, i32, p64, p64, p64, p64, i32, i32, vp]
     L.t2sp_fill_uniform_f32.argtypes = [vp, i64, ctypes.c_uint64, vp]
     L.t2sp_last_kernel_ns.restype = ctypes.c_double
     L.t2sp_release.restype = None

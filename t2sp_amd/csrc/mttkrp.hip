@@ -17,6 +17,10 @@
 #include "splitk.hpp"
 #include "t2sp_hip.h"
 
+#include <stdio.h>
+
+#include <mutex>
+
 namespace t2sp {
 
 struct MttkrpArgs {
@@ -360,4 +364,65 @@ extern "C" int t2sp_mttkrp_f32(const float *B, const float *C, const float *D, f
         case T2SP_CFG_32x128: return launch_mttkrp<MttW>(g, (hipStream_t)stream);
         default: return T2SP_ERR_SHAPE;
     }
+}
+
+// ---- the entry point that allocates nothing -----------------------------------------------
+// For callers that cannot allocate device memory (code under HIP graph capture, serving loops,
+// harnesses that forbid it): t2sp_mttkrp_f32 with the partial planes of the split reduction in
+// a static device array instead of a caller's workspace.  The array's name is only a host-side
+// handle; its device address is looked up once per device and kept.
+namespace t2sp {
+static __device__ __align__(256) float scratch[T2SP_MTTKRP_NOALLOC_SCRATCH_BYTES / sizeof(float)];
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static float *g_scratch_ptr[NOALLOC_MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device (each device holds its own copy).
+static float *scratch_on_current_device() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= NOALLOC_MAX_DEVICES) return nullptr;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        float *p = nullptr;
+        if (hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    return g_scratch_ptr[dev];
+}
+}  // namespace t2sp
+
+extern "C" int t2sp_mttkrp_f32_noalloc(const float *B, const float *C, const float *D, float *A, int I, int J,
+                                       int K, int R, const int64_t *sb3, const int64_t *sc2,
+                                       const int64_t *sd2, const int64_t *sa2, int cfg, int splits,
+                                       void *stream) {
+    using namespace t2sp;
+    if (I <= 0 || J <= 0 || K <= 0 || R <= 0 || !sb3 || !sc2 || !sd2 || !sa2) return T2SP_ERR_SHAPE;
+    if ((int64_t)K * J > INT32_MAX) return T2SP_ERR_SHAPE;
+    // what the product needs beyond its operands: the planes of a split reduction and, for sizes
+    // off the vector grid, the zero-padded copies (the scalar kernel of other orientations needs nothing)
+    size_t need = 0;
+    if (cfg != T2SP_CFG_SCALAR) {
+        if (mttkrp_fast(I, J, sb3, sc2, sd2, sa2, B, C, A))
+            need = plan_mttkrp(I, J, K, R, cfg, splits).scratch_bytes;
+        else if (cfg == T2SP_CFG_AUTO && sb3[1] == 1 && sc2[0] == 1 && sa2[0] == 1)
+            need = mttkrp_pad_bytes(I, J, K, R) +
+                   plan_mttkrp((I + 3) / 4 * 4, (J + 15) / 16 * 16, K, R, cfg, splits).scratch_bytes;
+    }
+    if (need > T2SP_MTTKRP_NOALLOC_SCRATCH_BYTES) {
+        fprintf(stderr, "t2sp: mttkrp (no allocation): this product needs %zu bytes of scratch (partial planes of the "
+                        "split reduction, padded copies), the built-in array holds %zu\n", need,
+                (size_t)T2SP_MTTKRP_NOALLOC_SCRATCH_BYTES);
+        return T2SP_ERR_SHAPE;
+    }
+    float *ptr = scratch_on_current_device();
+    if (!ptr) {
+        fprintf(stderr, "t2sp: mttkrp (no allocation): the address of the built-in scratch is not available\n");
+        return T2SP_ERR_LAUNCH;
+    }
+    // every plane a launch reads has been written by the same launch's workgroups: nothing to clear
+    return t2sp_mttkrp_f32(B, C, D, A, I, J, K, R, sb3, sc2, sd2, sa2, cfg, splits, ptr,
+                           T2SP_MTTKRP_NOALLOC_SCRATCH_BYTES, stream);
 }
