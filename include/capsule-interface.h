@@ -20,8 +20,33 @@ extern "C" {
  *   V(MY, MX, CO, OY, OX, N)   as in correctness/multi-projection/capsule.cpp:77
  * S is recovered from the sizes: the largest S with S*(OY-1)+KY <= IY (2 in the reference).
  * 4x4 poses (MK = MY = 4) take the MFMA kernel; other pose sizes a scalar kernel.
+ *
+ * The reference's own call form (capsule-run-fpga.cpp:49-74) is accepted as well:
+ *   P(TOTAL_CI*MK*MX*NN, IY*IX*N)      element (ci + TOTAL_CI*mk + TOTAL_CI*MK*mx + TOTAL_CI*MK*MX*nn,
+ *                                               iy + IY*ix + IY*IX*n)              capsule.cpp:52
+ *   W(TOTAL_CO*MY, TOTAL_CI*KY*KX*MK)  element (co + TOTAL_CO*my,
+ *                                               cii + CII*ky + CII*KY*kx + CII*KY*KX*ci + TOTAL_CI*KY*KX*mk)   capsule.cpp:53
+ *   V(COOO, YYY_XXX, YY_XX, Y_X, MY, MX, COO, NN, CO, N)   the 10-D output of capsule-run-fpga.cpp:73, or
+ *   V(TOTAL_CO*MY*MX*NN, OY*OX*N)      the 2-D output of the GPU flow (capsule-run-gpu.cpp:38-39,67-69)
+ * with the constants the pipeline bakes for every target (capsule/const-parameters.h:22-28,
+ * capsule.cpp:38-41): OX = OY = 7, KX = KY = 3, MX = MY = MK = 4, stride 2, IX = IY = 15; extents
+ * that contradict them return -8.  Batch n_total = nn + NN*n and channel co_total =
+ * cooo + COOO*coo + COOO*COO*co are read from V, TOTAL_CI from P.  An output pixel is the linear
+ * index yyy_xxx + YYY_XXX*yy_xx + YYY_XXX*YY_XX*y_x = oy + OY*ox; designs that cover more than 49
+ * positions (50 with the A10 constants, 56 with the S10 ones) get zeros in the surplus, where
+ * the reference computes from memory past the image.  The pipeline's batch loop runs to
+ * P.extent.1 / (IY*IX*NN) (capsule.cpp:55), i.e. N/NN blocks when NN > 1; here all N blocks that
+ * P and V hold are computed.
+ * CII, which orders W's second dimension, is carried by no buffer: state it once with
+ * t2sp_capsule_design() (or the environment variable T2SP_CAPSULE_CII), as the reference picks its
+ * design at run time through $BITSTREAM.  Without it the packed form returns -8.
  * Device-resident buffers: see gemm-interface.h. */
 int capsule(struct halide_buffer_t *P, struct halide_buffer_t *W, struct halide_buffer_t *V);
+
+/* States the design constant CII (capsule/const-parameters.h:31-70: 4 for the GPU and TINY sets, 32
+ * for S10, 16 for A10) that the packed form of capsule() needs; 0 clears it.  Returns the previous
+ * value.  Process-wide; no counterpart in the reference, where CII is compiled into the pipeline. */
+int t2sp_capsule_design(int cii);
 
 /* capsule() with a forced tile configuration (T2SP_CFG_* of t2sp_hip.h) and number of
  * reduction splits (0 = automatic); no counterpart in the reference. */

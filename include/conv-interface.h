@@ -19,10 +19,21 @@ extern "C" {
  *                                         dense buffers are NCHW / OIHW memory with y as "W"
  *   I(CI*N, IY*IX),   K(CO*KX, CI*KY)     packed 2-D, as in conv-run-fpga.cpp:49-66
  *   O(OY, OX, CO, N)                      4-D, or
- *   O(COOO, YYY, XXX, COO, YY, XX, Y, X, CO, N)  the 10-D tiled output of conv-run-fpga.cpp:68
- * Packed inputs need the 10-D output (N, CO and the image size are read from it).
+ *   O(COOO, YYY, XXX, COO, YY, XX, Y, X, CO, N)  the 10-D tiled output of conv-run-fpga.cpp:68, or
+ *   O(CO*N, OY*OX)                        2-D, element (co + CO*n, oy + OY*ox): the output of the GPU
+ *                                         flow (conv-run-gpu.cpp:33-38,60-62)
+ * Packed inputs need the 10-D or the 2-D output (N, CO and the image size are read from it).  With
+ * the 2-D output the packed form bakes KX = KY = 3, as every design of the reference does
+ * (conv/const-parameters.h:22-23), and solves OY*OX and (OY+2)*(OX+2) for the map: unique when it
+ * is square (the reference's GPU design is 64 x 64); otherwise t2sp_conv_design() says which
+ * root is OY, and without it the call returns -8.
  * Device-resident buffers: see gemm-interface.h. */
 int conv(struct halide_buffer_t *I, struct halide_buffer_t *K, struct halide_buffer_t *O);
+
+/* States TOTAL_OY for packed inputs with the 2-D output when the map is not square (0 clears it;
+ * also read from the environment variable T2SP_CONV_TOTAL_OY).  Returns the previous value.  No
+ * counterpart in the reference, where the map size is compiled into the pipeline. */
+int t2sp_conv_design(int total_oy);
 
 /* conv() with a forced tile configuration (T2SP_CFG_* of t2sp_hip.h); no counterpart in
  * the reference. */

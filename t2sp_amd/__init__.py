@@ -7,7 +7,7 @@ arithmetic happens in the HIP kernels; there is no CPU fallback.
 """
 from ._lib import lib, lib_path, build  # noqa: F401
 from .buffer import HalideBuffer, halide_buffer_t, halide_dimension_t, halide_type_t  # noqa: F401
-from .ops import capsule, conv, gemm, gemm_ex, syrk, ger, gbmv3, symv, pairhmm, qrd, mttkrp, mttkrp_reference_layout, gemm_tiled_shape, fill_uniform, host_empty, last_kernel_ns, release, T2spError  # noqa: F401
+from .ops import capsule, capsule_packed, conv, gemm, gemm_ex, syrk, ger, gbmv3, symv, pairhmm, qrd, mttkrp, mttkrp_reference_layout, gemm_tiled_shape, fill_uniform, host_empty, last_kernel_ns, release, T2spError  # noqa: F401
 
 
 def smoke_more(check, oracle):

@@ -90,6 +90,7 @@ def _declare(L):
     L.t2sp_host_free.restype = None
     L.conv.argtypes = [bp, bp, bp]
     L.t2sp_conv_with_cfg.argtypes = [bp, bp, bp, i32]
+    L.t2sp_conv_design.argtypes = [i32]
     p64, p32 = ctypes.POINTER(i64), ctypes.POINTER(i32)
     L.t2sp_conv2d_f32.argtypes = [vp, vp, vp] + [i32] * 7 + [p64, p64, p64, i32, vp, ctypes.c_size_t, vp]
     L.t2sp_conv2d_workspace_bytes.argtypes = [i32] * 7
@@ -97,6 +98,7 @@ def _declare(L):
     L.t2sp_relayout_f32.argtypes = [vp, vp, i32, p32, p64, p64, vp]
     L.capsule.argtypes = [bp, bp, bp]
     L.t2sp_capsule_with_cfg.argtypes = [bp, bp, bp, i32, i32]
+    L.t2sp_capsule_design.argtypes = [i32]
     L.mttkrp.argtypes = [bp, bp, bp, bp]
     L.t2sp_mttkrp_with_cfg.argtypes = [bp, bp, bp, bp, i32, i32]
     sz = ctypes.c_size_t

@@ -9,18 +9,155 @@
 //   V(MY, MX, CO, OY, OX, N)     correctness/multi-projection/capsule.cpp:77
 // with V[n,co,y,x,mx,my] = sum P[n,ci,S*y+ky,S*x+kx,mx,mk] * W[co,ci,ky,kx,mk,my]; the stride S
 // (2 in the reference, capsule.cpp:40-41) is recovered from the image sizes.  Strides of every
-// dimension but the innermost are free.  The reference's packed 2-D form (capsule.cpp:51-55)
-// bakes OY, OX and S into the pipeline as compile-time constants that no buffer carries, so it
-// cannot be expressed through a buffers-only interface and is not accepted.
+// dimension but the innermost are free.
+//
+// The reference's own call (capsule-run-fpga.cpp:49-74) is accepted too:
+//   P(TOTAL_CI*MK*MX*NN, IY*IX*N), W(TOTAL_CO*MY, TOTAL_CI*KY*KX*MK)   packed 2-D, capsule.cpp:51-53
+//   V(COOO, YYY_XXX, YY_XX, Y_X, MY, MX, COO, NN, CO, N)                10-D, capsule-run-fpga.cpp:73
+//   V(TOTAL_CO*MY*MX*NN, OY*OX*N)                                       2-D, capsule-run-gpu.cpp:38-39,67-69
+// The pipeline bakes OX = OY = 7, KX = KY = 3, MX = MY = MK = 4 and the stride 2 for every target
+// (capsule/const-parameters.h:22-28, capsule.cpp:38-41); the packed form bakes the same values and
+// checks them against the extents.  NN, N and the split of TOTAL_CO come from V, TOTAL_CI from
+// P.  One design constant is carried by no buffer: CII, the inner block of input channels that
+// orders W's second dimension (cii + CII*ky + CII*KY*kx + CII*KY*KX*ci + TOTAL_CI*KY*KX*mk,
+// capsule.cpp:53).  It comes from t2sp_capsule_design() or $T2SP_CAPSULE_CII, as the reference
+// selects its design at run time through $BITSTREAM.  Packed operands are re-laid on the device
+// into the dense N-D form, the counterpart of the reference's host serializer loops.
 #include "capsule-interface.h"
 #include "runtime.hpp"
 #include "t2sp_hip.h"
 
+#include <stdlib.h>
+
+#include <atomic>
+
 using namespace t2sp;
+
+static std::atomic<int> g_capsule_cii{0};
+
+extern "C" int t2sp_capsule_design(int cii) { return g_capsule_cii.exchange(cii < 0 ? 0 : cii); }
+
+static int capsule_cii() {
+    int cii = g_capsule_cii.load();
+    if (cii <= 0)
+        if (const char *e = getenv("T2SP_CAPSULE_CII")) cii = atoi(e);
+    return cii;
+}
+
+// The reference's packed call form.  Called with the library lock held.
+static int capsule_packed(halide_buffer_t *P, halide_buffer_t *W, halide_buffer_t *V, int cfg, int splits) {
+    static const char *op = "capsule";
+    constexpr int64_t OYX = 7, KYX = 3, M = 4, S = 2, IYX = OYX * S + KYX - S;   // 15
+    Span sp, sw, sv;
+    int err;
+    if ((err = check_buffer(P, op, "P", 2, 2, &sp))) return err;
+    if ((err = check_buffer(W, op, "W", 2, 2, &sw))) return err;
+    if ((err = check_buffer(V, op, "V", 10, 2, &sv))) return err;
+    const halide_dimension_t *p = P->dim, *w = W->dim, *v = V->dim;
+    const bool tiled = V->dimensions == 10;
+    int64_t COOO = 1, COO = 1, CO = 1, NN, N, PIX = OYX * OYX, TCO;
+    if (w[0].extent % M)
+        return report(halide_error_code_constraint_violated, op, "W.extent.0 must be TOTAL_CO*MY with MY = 4");
+    TCO = w[0].extent / M;
+    if (tiled) {
+        COOO = v[0].extent; COO = v[6].extent; CO = v[8].extent; NN = v[7].extent; N = v[9].extent;
+        PIX = (int64_t)v[1].extent * v[2].extent * v[3].extent;
+        if (v[4].extent != M || v[5].extent != M)
+            return report(halide_error_code_constraint_violated, op, "V.extent.4 and V.extent.5 must be MY = MX = 4");
+        if (COOO * COO * CO != TCO)
+            return report(halide_error_code_constraint_violated, op, "W.extent.0 must be COOO*COO*CO*MY of V");
+    } else {
+        if (TCO == 0 || v[0].extent % (TCO * M * M) || v[1].extent % (OYX * OYX))
+            return report(halide_error_code_constraint_violated, op,
+                          "V must be (TOTAL_CO*MY*MX*NN, OY*OX*N) with OY = OX = 7, MY = MX = 4");
+        NN = TCO ? v[0].extent / (TCO * M * M) : 0;
+        N = v[1].extent / (OYX * OYX);
+    }
+    if (N == 0 || NN == 0 || TCO == 0 || PIX == 0) return 0;
+    if (p[0].extent % (M * M * NN))
+        return report(halide_error_code_constraint_violated, op, "P.extent.0 must be TOTAL_CI*MK*MX*NN with MK = MX = 4");
+    const int64_t TCI = p[0].extent / (M * M * NN);
+    if (TCI == 0) return report(halide_error_code_constraint_violated, op, "empty reduction extents");
+    if (w[1].extent != TCI * KYX * KYX * M)
+        return report(halide_error_code_constraint_violated, op, "W.extent.1 must be TOTAL_CI*KY*KX*MK with KY = KX = 3, MK = 4");
+    if (p[1].extent != IYX * IYX * N)
+        return report(halide_error_code_constraint_violated, op, "P.extent.1 must be IY*IX*N with IY = IX = 15");
+    const int64_t CII = capsule_cii();
+    if (CII <= 0)
+        return report(halide_error_code_constraint_violated, op,
+                      "the packed W is ordered by the design constant CII, which no buffer carries: "
+                      "call t2sp_capsule_design(CII) or set T2SP_CAPSULE_CII");
+    if (TCI % CII) return report(halide_error_code_constraint_violated, op, "TOTAL_CI is not a multiple of the design's CII");
+    const int64_t NT = NN * N, CIO = TCI / CII;
+    const int64_t p_elems = NT * TCI * IYX * IYX * M * M, w_elems = TCO * TCI * KYX * KYX * M * M,
+                  SLOTS = PIX > OYX * OYX ? PIX : OYX * OYX, v_elems = NT * TCO * SLOTS * M * M;
+    if (p_elems > INT32_MAX || v_elems > INT32_MAX)
+        return report(halide_error_code_buffer_extents_too_large, op, "problem too large for 32-bit offsets");
+
+    Staged dp, dw, dv;
+    if ((err = dp.input(P, sp, op))) return err;
+    if ((err = dw.input(W, sw, op))) return err;
+    if ((err = dv.output(V, sv, op))) return err;
+    float *tp = static_cast<float *>(pool().get(p_elems * sizeof(float)));
+    float *tw = static_cast<float *>(pool().get(w_elems * sizeof(float)));
+    float *tv = static_cast<float *>(pool().get(v_elems * sizeof(float)));
+    const int dims[11] = {(int)NT, (int)TCI, (int)TCO, (int)OYX, (int)OYX, (int)KYX, (int)KYX, (int)S, (int)M, (int)M, (int)M};
+    const size_t ws_bytes = t2sp_capsule_workspace_bytes(dims, cfg, splits);
+    float *ws = ws_bytes ? static_cast<float *>(pool().get(ws_bytes)) : nullptr;
+    struct Put { float *q[4]; ~Put() { for (float *x : q) if (x) pool().put(x); } } put{{tp, tw, tv, ws}};
+    if (!tp || !tw || !tv || (ws_bytes && !ws))
+        return report(halide_error_code_device_malloc_failed, op, "device allocation failed");
+    KernelTimer timer;
+    hipStream_t st = api_stream();
+    {   // P(ci + TCI*mk + TCI*MK*mx + TCI*MK*MX*nn, iy + IY*ix + IY*IX*n)  ->  dense [nn + NN*n][ci][ix][iy][mx][mk]
+        const int64_t s1 = p[1].stride, img = TCI * IYX * IYX * M * M;
+        const int ext[7] = {(int)M, (int)M, (int)IYX, (int)IYX, (int)TCI, (int)NN, (int)N};          // mk mx iy ix ci nn n
+        const int64_t ss[7] = {TCI, TCI * M, s1, IYX * s1, 1, TCI * M * M, IYX * IYX * s1};
+        const int64_t ds[7] = {1, M, M * M, M * M * IYX, M * M * IYX * IYX, img, NN * img};
+        if ((err = t2sp_relayout_f32(dp.ptr(), tp, 7, ext, ss, ds, st))) return report(err, op, "relayout failed");
+    }
+    {   // W(co + TCO*my, cii + CII*ky + CII*KY*kx + CII*KY*KX*ci + TCI*KY*KX*mk)  ->  dense [co][ci][kx][ky][mk][my]
+        const int64_t s1 = w[1].stride, win = KYX * KYX * M * M;
+        const int ext[7] = {(int)M, (int)M, (int)KYX, (int)KYX, (int)CII, (int)CIO, (int)TCO};       // my mk ky kx cii ci co
+        const int64_t ss[7] = {TCO, TCI * KYX * KYX * s1, CII * s1, CII * KYX * s1, s1, CII * KYX * KYX * s1, 1};
+        const int64_t ds[7] = {1, M, M * M, M * M * KYX, win, CII * win, TCI * win};
+        if ((err = t2sp_relayout_f32(dw.ptr(), tw, 7, ext, ss, ds, st))) return report(err, op, "relayout failed");
+    }
+    // votes: dense [n][co][pixel][mx][my] with pixel = oy + OY*ox, the pipeline's linear pixel index
+    // (capsule.cpp:38-39), and SLOTS >= 49 slots per (n, co).  The FPGA designs cover 50 or 56 positions for
+    // the 49 real ones (const-parameters.h:53-71) and compute them from memory past the image; here
+    // slots from 49 on are written as zeros.
+    if (PIX > OYX * OYX && hipMemsetAsync(tv, 0, v_elems * sizeof(float), st) != hipSuccess)
+        return report(halide_error_code_device_run_failed, op, "clearing the votes failed");
+    const int64_t sp6[6] = {TCI * IYX * IYX * M * M, IYX * IYX * M * M, IYX * M * M, M * M, M, 1};
+    const int64_t sw6[6] = {TCI * KYX * KYX * M * M, KYX * KYX * M * M, KYX * M * M, M * M, M, 1};
+    const int64_t sv6[6] = {TCO * SLOTS * M * M, SLOTS * M * M, OYX * M * M, M * M, M, 1};
+    err = t2sp_capsule_f32(tp, tw, tv, dims, sp6, sw6, sv6, cfg, splits, ws, ws_bytes, st);
+    if (err) return report(err, op, "kernel launch failed");
+    if (tiled) {
+        int ext[10];
+        int64_t ds[10];
+        for (int d = 0; d < 10; d++) { ext[d] = v[d].extent; ds[d] = v[d].stride; }
+        const int64_t px = M * M, cs = SLOTS * px;             // source strides of a pixel slot and a channel
+        const int64_t ss[10] = {cs, px, px * v[1].extent, px * v[1].extent * v[2].extent, 1, M,
+                                cs * COOO, cs * TCO, cs * COOO * COO, cs * TCO * NN};
+        if ((err = t2sp_relayout_f32(tv, dv.ptr(), 10, ext, ss, ds, st))) return report(err, op, "relayout failed");
+    } else {
+        // V(co + TCO*my + TCO*MY*mx + TCO*MY*MX*nn, oy + OY*ox + OY*OX*n)
+        const int64_t s1 = v[1].stride, px = M * M, cs = SLOTS * px;
+        const int ext[6] = {(int)TCO, (int)M, (int)M, (int)NN, (int)(OYX * OYX), (int)N};            // co my mx nn pixel n
+        const int64_t ss[6] = {cs, 1, M, cs * TCO, px, cs * TCO * NN};
+        const int64_t ds[6] = {1, TCO, TCO * M, TCO * M * M, s1, OYX * OYX * s1};
+        if ((err = t2sp_relayout_f32(tv, dv.ptr(), 6, ext, ss, ds, st))) return report(err, op, "relayout failed");
+    }
+    if ((err = timer.stop_and_sync(op))) return err;
+    return dv.finish(op);
+}
 
 static int capsule_impl(halide_buffer_t *P, halide_buffer_t *W, halide_buffer_t *V, int cfg, int splits) {
     static const char *op = "capsule";
     std::lock_guard<std::mutex> lock(api_mutex());
+    if (P && W && P->dimensions == 2 && W->dimensions == 2) return capsule_packed(P, W, V, cfg, splits);
     Span sp, sw, sv;
     int err;
     if ((err = check_buffer(P, op, "P", 6, 6, &sp))) return err;

@@ -8,8 +8,12 @@
 //   2-D  I(CI*N, IY*IX),   K(CO*KX, CI*KY)  (packed)             conv-run-fpga.cpp:49-66, conv.cpp:51-54
 //   O    4-D (OY, OX, CO, N), or the 10-D tiled
 //        (COOO, YYY, XXX, COO, YY, XX, Y, X, CO, N)              conv-run-fpga.cpp:68, conv.cpp:39-44
+//        or the 2-D (CO*N, OY*OX) of the GPU flow                conv-run-gpu.cpp:33-38,60-62
 // with  O[n,co,y,x] = sum_{ci,kx,ky} I[n,ci,y+ky,x+kx] * K[co,ci,ky,kx].  All sizes come from
-// the buffers; the packed form needs the 10-D output to recover N, CO and the image size.
+// the buffers.  Packed inputs with the 2-D output leave the kernel size open, so that pairing bakes
+// KX = KY = 3 as the reference does for every target (conv/const-parameters.h:22-23); OY and OX then
+// follow from OY*OX and (OY+2)*(OX+2), uniquely for square maps (the reference's GPU design is
+// 64 x 64); for other maps t2sp_conv_design(TOTAL_OY) or $T2SP_CONV_TOTAL_OY says which root is OY.
 // The 4-D form with dense I/K/O is the benchmark's NCHW/OIHW layout and goes to the MFMA
 // kernel directly; other forms are re-laid on the device first, which is what the
 // reference's host serializer/deserializer loops do on the CPU.
@@ -17,7 +21,16 @@
 #include "runtime.hpp"
 #include "t2sp_hip.h"
 
+#include <math.h>
+#include <stdlib.h>
+
+#include <atomic>
+
 using namespace t2sp;
+
+static std::atomic<int> g_conv_total_oy{0};
+
+extern "C" int t2sp_conv_design(int total_oy) { return g_conv_total_oy.exchange(total_oy < 0 ? 0 : total_oy); }
 
 namespace {
 struct Logical4 {
@@ -110,18 +123,55 @@ static int conv_impl(halide_buffer_t *I, halide_buffer_t *K, halide_buffer_t *O,
     int err;
     if ((err = check_buffer(I, op, "I", 4, 2, &si))) return err;
     if ((err = check_buffer(K, op, "K", 4, 2, &sk))) return err;
-    if ((err = check_buffer(O, op, "O", 4, 10, &so))) return err;
+    const bool flat_out = O && O->dimensions == 2;
+    if ((err = check_buffer(O, op, "O", flat_out ? 2 : 4, flat_out ? 2 : 10, &so))) return err;
     const bool packed = I->dimensions == 2;
     if ((K->dimensions == 2) != packed)
         return report(halide_error_code_bad_dimensions, op, "I and K must both be 4-D or both be packed 2-D");
-    if (packed && O->dimensions != 10)
-        return report(halide_error_code_bad_dimensions, op, "packed 2-D inputs need the 10-D tiled output");
+    if (packed && O->dimensions == 4)
+        return report(halide_error_code_bad_dimensions, op, "packed 2-D inputs need the 10-D tiled or the 2-D output");
 
     // Output: logical (n, co, h, w) with w = the reference's y (innermost), h = its x.
     int64_t N, CO, OH, OW;
     const halide_dimension_t *od = O->dim;
     if (O->dimensions == 4) {
         OW = od[0].extent; OH = od[1].extent; CO = od[2].extent; N = od[3].extent;
+    } else if (flat_out && !packed) {
+        // O(CO*N, OY*OX) with 4-D inputs: every size is in I and K
+        CO = K->dim[3].extent; N = I->dim[3].extent;
+        OW = (int64_t)I->dim[0].extent - K->dim[0].extent + 1; OH = (int64_t)I->dim[1].extent - K->dim[1].extent + 1;
+        if (OW < 0 || OH < 0)
+            return report(halide_error_code_access_out_of_bounds, op, "I is smaller than the kernel");
+        if (od[0].extent != CO * N || od[1].extent != OW * OH)
+            return report(halide_error_code_constraint_violated, op, "O must be (CO*N, OY*OX)");
+    } else if (flat_out) {
+        // O(CO*N, OY*OX) with packed inputs: KX = KY = 3 as in every design of the reference
+        constexpr int64_t KYX = 3;
+        if (K->dim[0].extent % KYX || K->dim[1].extent % KYX)
+            return report(halide_error_code_constraint_violated, op, "K must be (CO*KX, CI*KY) with KX = KY = 3");
+        CO = K->dim[0].extent / KYX;
+        const int64_t ci = K->dim[1].extent / KYX;
+        if (CO == 0 || ci == 0 || I->dim[0].extent % ci || od[0].extent % CO || od[0].extent / CO != I->dim[0].extent / ci)
+            return report(halide_error_code_constraint_violated, op, "I must be (CI*N, IY*IX) and O (CO*N, OY*OX) with one N");
+        N = od[0].extent / CO;
+        // OY*OX = a, (OY+2)*(OX+2) = b  ->  OY + OX = (b - a - 4)/2, the two sizes are the roots of t^2 - s t + a
+        const int64_t a = od[1].extent, b = I->dim[1].extent, s2 = b - a - (KYX - 1) * (KYX - 1);
+        const int64_t sum = s2 / (KYX - 1), disc = sum * sum - 4 * a;
+        const int64_t root = disc >= 0 ? (int64_t)llround(sqrt((double)disc)) : -1;
+        if (s2 < 0 || s2 % (KYX - 1) || root < 0 || root * root != disc || (sum + root) % 2)
+            return report(halide_error_code_constraint_violated, op, "no map OY x OX has O.extent.1 outputs and I.extent.1 inputs under a 3 x 3 kernel");
+        const int64_t big = (sum + root) / 2, small = (sum - root) / 2;
+        int hint = g_conv_total_oy.load();
+        if (hint <= 0)
+            if (const char *e = getenv("T2SP_CONV_TOTAL_OY")) hint = atoi(e);
+        if (big == small) {
+            OW = OH = big;
+        } else if (hint == big || hint == small) {
+            OW = hint; OH = hint == big ? small : big;
+        } else {
+            return report(halide_error_code_constraint_violated, op,
+                          "a map that is not square leaves OY and OX open: call t2sp_conv_design(TOTAL_OY) or set T2SP_CONV_TOTAL_OY");
+        }
     } else {
         CO = (int64_t)od[0].extent * od[3].extent * od[8].extent;
         OW = (int64_t)od[1].extent * od[4].extent * od[6].extent;
@@ -240,8 +290,15 @@ static int conv_impl(halide_buffer_t *I, halide_buffer_t *K, halide_buffer_t *O,
         int64_t ss[T2SP_MAX_DIMS], ds[T2SP_MAX_DIMS];
         const int nd = O->dimensions;
         for (int d = 0; d < nd; d++) { ext[d] = od[d].extent; ds[d] = od[d].stride; }
+        int rnd = nd;
         if (nd == 4) {
             ss[0] = so4[3]; ss[1] = so4[2]; ss[2] = so4[1]; ss[3] = so4[0];
+        } else if (nd == 2) {
+            // O(co + CO*n, oy + OY*ox): a box over (co, n, oy, ox)
+            rnd = 4;
+            ext[0] = (int)CO; ext[1] = (int)N; ext[2] = (int)OW; ext[3] = (int)OH;
+            ss[0] = so4[1]; ss[1] = so4[0]; ss[2] = so4[3]; ss[3] = so4[2];
+            ds[0] = 1; ds[1] = CO; ds[2] = od[1].stride; ds[3] = OW * (int64_t)od[1].stride;
         } else {
             const int64_t COOO = od[0].extent, YYY = od[1].extent, XXX = od[2].extent, COO = od[3].extent,
                           YY = od[4].extent, XX = od[5].extent;
@@ -250,7 +307,7 @@ static int conv_impl(halide_buffer_t *I, halide_buffer_t *K, halide_buffer_t *O,
             ss[2] = so4[2]; ss[5] = XXX * so4[2];  ss[7] = XXX * XX * so4[2];          // xxx, xx, x
             ss[9] = so4[0];                                                            // n
         }
-        if ((err = t2sp_relayout_f32(tmp_o, dout.ptr(), nd, ext, ss, ds, api_stream())))
+        if ((err = t2sp_relayout_f32(tmp_o, dout.ptr(), rnd, ext, ss, ds, api_stream())))
             return report(err, op, "relayout failed");
     }
     if ((err = timer.stop_and_sync(op))) return err;

@@ -253,6 +253,20 @@ def capsule(P, W, out=None, stride=2, cfg=0, splits=0):
     return out
 
 
+def capsule_packed(P2, W2, out, cii, cfg=0, splits=0):
+    """The reference's own call form of `capsule` (capsule-run-fpga.cpp:49-74): packed 2-D P and W and
+    the 10-D (or, GPU flow, 2-D) output, passed as arrays whose axes are the reversed Halide
+    dimensions.  `cii` is the design constant that orders W's second dimension."""
+    L = lib()
+    p, w, v = HalideBuffer.wrap(P2), HalideBuffer.wrap(W2), HalideBuffer.wrap(out)
+    previous = L.t2sp_capsule_design(int(cii))
+    try:
+        _check("capsule", L.t2sp_capsule_with_cfg(p.ref, w.ref, v.ref, int(cfg), int(splits)))
+    finally:
+        L.t2sp_capsule_design(previous)
+    return out
+
+
 def mttkrp_reference_layout(B, C, D):
     """Views of B (i,j,k), C (j,r), D (k,r) re-laid as the reference's golden helper stores them
     (t2s/tests/performance/util/util.h:498-515): j contiguous in B and C, k contiguous in D."""

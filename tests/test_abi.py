@@ -174,3 +174,27 @@ def test_host_allocation_is_aligned_and_survives_views():
     gc.collect()
     assert (v == 3.0).all()
     assert t2sp_amd.host_empty((0, 5)).shape == (0, 5)
+
+
+def test_packed_capsule_form_is_checked_without_a_device():
+    """The reference's packed call (capsule-run-fpga.cpp:49-74) with the TINY constants: extents are
+    checked against the baked OX = OY = 7, KX = KY = 3, 4 x 4 poses, and the design constant CII must
+    have been stated, all before any device work."""
+    L = t2sp_amd.lib()
+    TCI, TCO, NN, N = 16, 16, 1, 2
+    P, W = _buf((225 * N, TCI * 16 * NN)), _buf((TCI * 36, TCO * 4))
+    V = _buf((N, 1, NN, 4, 4, 4, 7, 1, 7, 4))
+    assert L.t2sp_capsule_design(0) == 0
+    os.environ.pop("T2SP_CAPSULE_CII", None)
+    assert L.capsule(P.ref, W.ref, V.ref) == -8                                  # CII not stated
+    assert L.t2sp_capsule_design(4) == 0
+    try:
+        assert L.capsule(P.ref, _buf((TCI * 36 - 4, TCO * 4)).ref, V.ref) == -8      # W rows != TOTAL_CI*KY*KX*MK
+        assert L.capsule(_buf((224 * N, TCI * 16)).ref, W.ref, V.ref) == -8          # P rows != IY*IX*N
+        assert L.capsule(P.ref, W.ref, _buf((N, 1, NN, 4, 4, 3, 7, 1, 7, 4)).ref) == -8   # MY != 4
+        assert L.capsule(P.ref, _buf((TCI * 36, TCO * 4 + 4)).ref, V.ref) == -8      # TOTAL_CO of W and V differ
+        assert L.capsule(P.ref, W.ref, _buf((2, 8, 4, 4, 4, 4)).ref) == -43          # 6-D V with packed inputs
+        assert L.t2sp_capsule_design(5) == 4
+        assert L.capsule(P.ref, W.ref, V.ref) == -8                                  # CII does not divide TOTAL_CI
+    finally:
+        L.t2sp_capsule_design(0)

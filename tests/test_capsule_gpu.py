@@ -113,3 +113,86 @@ def test_config4_full_size(oracle):
     assert err <= TOL
     V2 = t2sp_amd.capsule(P, W)
     assert torch.equal(V, V2)          # the split reduction is added in a fixed order
+
+
+# ---- the reference's own call form: packed 2-D P and W, 10-D or 2-D V (capsule-run-fpga.cpp:49-74) ----
+
+CAPSULE_DESIGNS = {   # capsule/const-parameters.h:31-70
+    "TINY": dict(CII=4, CI=4, COOO=4, COO=4, CO=1, YYY_XXX=7, YY_XX=1, Y_X=7, NN=1),
+    "GPU": dict(CII=4, CI=8, COOO=8, COO=1, CO=4, YYY_XXX=7, YY_XX=7, Y_X=1, NN=16),
+    "S10": dict(CII=32, CI=1, COOO=8, COO=4, CO=1, YYY_XXX=14, YY_XX=1, Y_X=4, NN=4),
+    "A10": dict(CII=16, CI=2, COOO=8, COO=4, CO=1, YYY_XXX=10, YY_XX=1, Y_X=5, NN=4),
+}
+
+
+def pack_capsule_inputs(P, W, NN, CII):
+    """Logical P (n_total,ci,y,x,mx,mk), W (co,ci,ky,kx,mk,my) -> the packed 2-D buffers, as numpy
+    arrays with reversed Halide dimensions: P2[iy + 15*ix + 225*n][ci + TCI*mk + TCI*4*mx + TCI*16*nn],
+    W2[cii + CII*ky + CII*3*kx + CII*9*ci + TCI*9*mk][co + TCO*my]  (capsule.cpp:52-53)."""
+    NT, TCI, IY, IX, MX, MK = P.shape
+    TCO = W.shape[0]
+    N = NT // NN
+    P2 = P.reshape(N, NN, TCI, IY, IX, MX, MK).transpose(0, 4, 3, 1, 5, 6, 2)        # n, ix, iy, nn, mx, mk, ci
+    P2 = np.ascontiguousarray(P2).reshape(N * IX * IY, NN * MX * MK * TCI)
+    W2 = W.reshape(TCO, TCI // CII, CII, 3, 3, 4, 4).transpose(5, 1, 4, 3, 2, 6, 0)   # mk, ci, kx, ky, cii, my, co
+    W2 = np.ascontiguousarray(W2).reshape(4 * TCI * 9, 4 * TCO)
+    return P2, W2
+
+
+def unpack_capsule_v10(V10):
+    """10-D V (numpy axes n, co, nn, coo, mx, my, y_x, yy_xx, yyy_xxx, cooo) -> logical (n_total, co_total,
+    y, x, mx, my) and the surplus pixel positions beyond 49."""
+    N, CO, NN, COO, MX, MY, YX1, YX2, YX3, COOO = V10.shape
+    t = V10.transpose(0, 2, 1, 3, 9, 6, 7, 8, 4, 5).reshape(N * NN, CO * COO * COOO, YX1 * YX2 * YX3, MX, MY)
+    votes = t[:, :, :49].reshape(N * NN, -1, 7, 7, MX, MY).transpose(0, 1, 3, 2, 4, 5)     # pixel = oy + 7*ox
+    return votes, t[:, :, 49:]
+
+
+@pytest.mark.parametrize("design,N", [("TINY", 4), ("GPU", 1), ("S10", 2), ("A10", 2)])
+def test_reference_packed_call_form(oracle, design, N):
+    """capsule(P, W, V) exactly as capsule-run-fpga.cpp:49-74 builds its buffers, for the four constant
+    sets of capsule/const-parameters.h, against the oracle in the golden order and in the pipeline's
+    own order; then the 2-D output of the GPU flow (capsule-run-gpu.cpp:38-39,67-69)."""
+    c = CAPSULE_DESIGNS[design]
+    TCI, TCO, NT = c["CII"] * c["CI"], c["COOO"] * c["COO"] * c["CO"], c["NN"] * N
+    P, W = oracle.fill_uniform((NT, TCI, 15, 15, 4, 4), 80), oracle.fill_uniform((TCO, TCI, 3, 3, 4, 4), 81)
+    ref = oracle.capsule(P, W)
+    P2, W2 = pack_capsule_inputs(P, W, c["NN"], c["CII"])
+    V10 = np.full((N, c["CO"], c["NN"], c["COO"], 4, 4, c["Y_X"], c["YY_XX"], c["YYY_XXX"], c["COOO"]), np.nan, np.float32)
+    t2sp_amd.capsule_packed(P2, W2, V10, c["CII"])
+    votes, surplus = unpack_capsule_v10(V10)
+    err, mx = rel_fro(votes, ref)
+    assert err <= TOL, (design, err, mx)
+    assert rel_fro(votes, oracle.capsule(P, W, order=oracle.ORDER_URE, cii=c["CII"]))[0] <= TOL
+    assert surplus.size == (c["YYY_XXX"] * c["YY_XX"] * c["Y_X"] - 49) * NT * TCO * 16 and (surplus == 0).all()
+    assert (votes == t2sp_amd.capsule(P, W)).all()               # same kernel, same bits as the N-D form
+    V2 = np.full((49 * N, TCO * 16 * c["NN"]), np.nan, np.float32)
+    t2sp_amd.capsule_packed(P2, W2, V2, c["CII"])
+    got = V2.reshape(N, 7, 7, c["NN"], 4, 4, TCO).transpose(0, 3, 6, 2, 1, 4, 5).reshape(NT, TCO, 7, 7, 4, 4)
+    assert (got == votes).all()
+
+
+def test_packed_form_needs_its_design_constant_and_consistent_extents(oracle):
+    c = CAPSULE_DESIGNS["TINY"]
+    P, W = oracle.fill_uniform((2, 16, 15, 15, 4, 4), 82), oracle.fill_uniform((16, 16, 3, 3, 4, 4), 83)
+    P2, W2 = pack_capsule_inputs(P, W, 1, 4)
+    V10 = np.zeros((2, 1, 1, 4, 4, 4, 7, 1, 7, 4), np.float32)
+    L = t2sp_amd.lib()
+    from t2sp_amd.buffer import HalideBuffer
+    p, w, v = HalideBuffer.wrap(P2), HalideBuffer.wrap(W2), HalideBuffer.wrap(V10)
+    assert L.t2sp_capsule_design(0) == 0
+    assert L.capsule(p.ref, w.ref, v.ref) == -8                  # CII not stated
+    with pytest.raises(t2sp_amd.T2spError) as e:                 # CII does not divide TOTAL_CI
+        t2sp_amd.capsule_packed(P2, W2, V10, 5)
+    assert e.value.code == -8
+    with pytest.raises(t2sp_amd.T2spError) as e:                 # W's rows contradict TOTAL_CI*KY*KX*MK
+        t2sp_amd.capsule_packed(P2, W2[:-4], V10, 4)
+    assert e.value.code == -8
+    with pytest.raises(t2sp_amd.T2spError) as e:                 # P's second extent is not IY*IX*N
+        t2sp_amd.capsule_packed(P2[:-15], W2, V10, 4)
+    assert e.value.code == -8
+    # a different CII is a different weight layout: the result must change
+    t2sp_amd.capsule_packed(P2, W2, V10, 4)
+    other = np.zeros_like(V10)
+    t2sp_amd.capsule_packed(P2, W2, other, 16)
+    assert not np.array_equal(other, V10)

@@ -154,6 +154,34 @@ def test_reference_packed_inputs_and_tiled_output(oracle, consts):
     assert (O10b == O10).all()
 
 
+@pytest.mark.parametrize("N,CI,CO,OY,OX", [(4, 16, 24, 8, 8), (2, 8, 8, 12, 5), (1, 256, 8, 64, 64)])
+def test_gpu_flow_flat_output(oracle, N, CI, CO, OY, OX):
+    """The 2-D output of the GPU flow, O(co + CO*n, oy + OY*ox) (conv-run-gpu.cpp:33-38,60-62), with
+    packed inputs (3 x 3 baked; the map that is not square needs TOTAL_OY stated) and with 4-D inputs."""
+    I, W = oracle.fill_uniform((N, CI, OY + 2, OX + 2), 12), oracle.fill_uniform((CO, CI, 3, 3), 13)
+    ref = oracle.conv(I, W)
+    Ip = np.ascontiguousarray(I.transpose(3, 2, 0, 1)).reshape((OX + 2) * (OY + 2), N * CI)
+    Kp = np.ascontiguousarray(W.transpose(2, 1, 3, 0)).reshape(3 * CI, 3 * CO)
+    L = t2sp_amd.lib()
+
+    def unflat(O2):
+        return O2.reshape(OX, OY, N, CO).transpose(2, 3, 1, 0)
+    O2 = np.full((OX * OY, N * CO), np.nan, np.float32)
+    if OY != OX:
+        with pytest.raises(t2sp_amd.T2spError) as e:
+            t2sp_amd.conv(Ip, Kp, out=O2)
+        assert e.value.code == -8 and np.isnan(O2).all()
+        assert L.t2sp_conv_design(OY) == 0
+    try:
+        t2sp_amd.conv(Ip, Kp, out=O2)
+    finally:
+        L.t2sp_conv_design(0)
+    assert rel_fro(unflat(O2), ref)[0] <= TOL
+    O2b = np.full_like(O2, np.nan)
+    t2sp_amd.conv(np.ascontiguousarray(I.transpose(0, 1, 3, 2)), np.ascontiguousarray(W.transpose(0, 1, 3, 2)), out=O2b)
+    assert (O2b == O2).all()
+
+
 def test_packed_inputs_need_tiled_output():
     with pytest.raises(t2sp_amd.T2spError) as e:
         t2sp_amd.conv(np.zeros((36, 8), np.float32), np.zeros((12, 12), np.float32), out=np.zeros((1, 4, 4, 4), np.float32))

@@ -12,7 +12,8 @@ BIN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "drivers", "bin")
 
 
 @pytest.mark.parametrize("name", ["gemm-run", "conv-run", "capsule-run", "mttkrp-run", "sgemm-run", "gemm-large-run",
-                                  "syrk-run", "ssyrk-run", "ger-run", "gbmv3-run", "symv-run", "pairhmm-run", "qrd-run"])
+                                  "syrk-run", "ssyrk-run", "ger-run", "gbmv3-run", "symv-run", "pairhmm-run", "qrd-run",
+                                  "capsule-packed-run-tiny", "capsule-packed-run-s10", "capsule-packed-run-a10"])
 def test_driver_prints_success(name, tmp_path):
     exe = os.path.join(BIN, name)
     assert os.path.exists(exe), "build the drivers first: make -C tests/drivers"
