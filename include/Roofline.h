@@ -10,9 +10,11 @@
  *                    or from the file named by $T2SP_EXEC_TIME_FILE when that is set (the entry
  *                    points write that file in the reference's format: first line the overall
  *                    ns, then one "<kernel_name> <ns>" line).
- *   roofline(...)    prints "GFlops: ..." like the reference and writes roofline.txt (the point
- *                    and both roofs) and roofline.svg into the current directory instead of
- *                    shelling out to matplotlib (Roofline.py:24-56).  Units as in the reference:
+ *   roofline(...)    prints "GFlops: ..." like the reference and writes roofline.png (the file the
+ *                    reference's drivers check for, gemm-run-fpga.cpp:101-104: both roofs and
+ *                    the point, rasterised here instead of shelling out to matplotlib,
+ *                    Roofline.py:24-56), plus roofline.svg (the same picture with its labels)
+ *                    and roofline.txt (the numbers) into the current directory.  Units as in the reference:
  *                    mem_bandwidth in GB/s, compute_roof in MFLOP/s (it is divided by 1000 for
  *                    the plot, Roofline.py:33), number_ops in flop, exec_time in ns.
  *   DSPs(), FMax()   the reference multiplies 2*DSPs()*FMax() for the compute roof; here

@@ -25,8 +25,15 @@ int t2sp_gemm_ex(int opa, int opb, float alpha, float beta, struct halide_buffer
                  struct halide_buffer_t *C, struct halide_buffer_t *O);
 #ifdef __cplusplus
 }
-/* The reference's pipeline entry gemm(opa, opb, alpha, beta, A, B, C, O) (blas-gemm.cpp:47) as a
- * C++ overload next to the 3-argument gemm() of gemm-interface.h. */
+/* The reference's pipeline entry gemm(opa, opb, alpha, beta, A, B, C, O) (blas-gemm.cpp:29) as a
+ * C++ overload next to the 3-argument gemm() of gemm-interface.h, so that the reference's
+ * blas-gemm.cpp compiles against these headers unchanged.  The same entry with C linkage, the
+ * symbol the generated gemm-interface.cpp of that release defines, is exported by
+ * libt2sp_blas_gemm.so (one library cannot hold two C functions called gemm): declared as
+ *   extern "C" int gemm(int32_t opa, int32_t opb, float alpha, float beta, halide_buffer_t *A,
+ *                       halide_buffer_t *B, halide_buffer_t *C, halide_buffer_t *O);
+ * O may cover more than M x N (the wrapper rounds it up to whole tiles, blas-gemm.cpp:10-12); the
+ * surplus is written as zeros. */
 inline int gemm(bool opa, bool opb, float alpha, float beta, struct halide_buffer_t *A, struct halide_buffer_t *B,
                 struct halide_buffer_t *C, struct halide_buffer_t *O) {
     return t2sp_gemm_ex(opa, opb, alpha, beta, A, B, C, O);

@@ -43,6 +43,11 @@ extern "C" {
  * Device-resident buffers: see gemm-interface.h. */
 int capsule(struct halide_buffer_t *P, struct halide_buffer_t *W, struct halide_buffer_t *V);
 
+/* The argv form Halide declares next to every generated entry
+ * (Halide/src/CodeGen_C.cpp:1828-1833, the default ExternalPlusMetadata linkage): args[i] is the
+ * i-th argument, a buffer argument being the halide_buffer_t* itself. */
+int capsule_argv(void **args);
+
 /* States the design constant CII (capsule/const-parameters.h:31-70: 4 for the GPU and TINY sets, 32
  * for S10, 16 for A10) that the packed form of capsule() needs; 0 clears it.  Returns the previous
  * value.  Process-wide; no counterpart in the reference, where CII is compiled into the pipeline. */

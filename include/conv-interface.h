@@ -30,6 +30,11 @@ extern "C" {
  * Device-resident buffers: see gemm-interface.h. */
 int conv(struct halide_buffer_t *I, struct halide_buffer_t *K, struct halide_buffer_t *O);
 
+/* The argv form Halide declares next to every generated entry
+ * (Halide/src/CodeGen_C.cpp:1828-1833, the default ExternalPlusMetadata linkage): args[i] is the
+ * i-th argument, a buffer argument being the halide_buffer_t* itself. */
+int conv_argv(void **args);
+
 /* States TOTAL_OY for packed inputs with the 2-D output when the map is not square (0 clears it;
  * also read from the environment variable T2SP_CONV_TOTAL_OY).  Returns the previous value.  No
  * counterpart in the reference, where the map size is compiled into the pipeline. */

@@ -27,10 +27,22 @@ int gemm(struct halide_buffer_t *A, struct halide_buffer_t *B, struct halide_buf
  * (t2s/tests/correctness/aot/gemm-generate.cpp:176, gemm-run.cpp:62). */
 int GEMM(struct halide_buffer_t *A, struct halide_buffer_t *B, struct halide_buffer_t *C);
 
+/* The argv form Halide declares next to every generated entry
+ * (Halide/src/CodeGen_C.cpp:1828-1833, the default ExternalPlusMetadata linkage): args[i] is the
+ * i-th argument, a buffer argument being the halide_buffer_t* itself. */
+int gemm_argv(void **args);
+int GEMM_argv(void **args);
+
 /* gemm() with a forced tile configuration (T2SP_CFG_* of t2sp_hip.h);
  * for benchmarks and tests, no counterpart in the reference. */
 int t2sp_gemm_with_cfg(struct halide_buffer_t *A, struct halide_buffer_t *B,
                        struct halide_buffer_t *C, int cfg);
+
+/* The number of rows per panel gemm(A, B, C) would move through the device at a time (large
+ * products on dense host buffers overlap their copies with the kernels), 0 = one piece.  For
+ * tests of that choice; no counterpart in the reference. */
+int t2sp_gemm_panel_rows(const struct halide_buffer_t *A, const struct halide_buffer_t *B,
+                         const struct halide_buffer_t *C);
 
 /* gemm() that returns the kernel time in ns (negative error code on failure), like the oneAPI
  * flavour of the reference's entry (t2s/tests/performance/oneapi/src/oneapi-target-4-run.cpp:99). */

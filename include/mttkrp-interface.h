@@ -19,6 +19,11 @@ extern "C" {
 int mttkrp(struct halide_buffer_t *B, struct halide_buffer_t *C, struct halide_buffer_t *D,
            struct halide_buffer_t *A);
 
+/* The argv form Halide declares next to every generated entry
+ * (Halide/src/CodeGen_C.cpp:1828-1833): args[i] is the i-th argument, a buffer argument being the
+ * halide_buffer_t* itself. */
+int mttkrp_argv(void **args);
+
 /* mttkrp() with a forced tile configuration (T2SP_CFG_* of t2sp_hip.h) and number of
  * reduction splits (0 = automatic); no counterpart in the reference. */
 int t2sp_mttkrp_with_cfg(struct halide_buffer_t *B, struct halide_buffer_t *C,

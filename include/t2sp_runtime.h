@@ -7,8 +7,10 @@
 extern "C" {
 #endif
 
-/* GPU time, in nanoseconds, of the kernels of the most recent operator call
- * (hipEvent bracket on the library stream).  Counterpart of the
+/* GPU time, in nanoseconds, of the kernels of the most recent operator call made by the
+ * calling thread (hipEvent bracket on the library stream); for a thread that has made none, of
+ * the most recent call in the process.  Callers on several threads are serialised by the
+ * library and each reads its own call's time.  Counterpart of the
  * "latest end - earliest start" figure the reference writes to exec_time.txt
  * (t2s/src/AOT-OpenCL-Runtime.cpp:358-396) and reads back with ExecTime()
  * (t2s/src/Roofline.cpp:113-140), and of the value the oneAPI-flavour entry

@@ -33,7 +33,10 @@ extern "C" int t2sp_gemm_ex(int opa, int opb, float alpha, float beta, halide_bu
     const int64_t o_cols = tiled ? (int64_t)O->dim[0].extent * O->dim[2].extent * O->dim[4].extent : O->dim[0].extent;
     const int64_t o_rows = tiled ? (int64_t)O->dim[1].extent * O->dim[3].extent * O->dim[5].extent : O->dim[1].extent;
     if (o_rows < M || o_cols < N) return report(halide_error_code_access_out_of_bounds, op, "O is smaller than M x N");
-    if (o_rows != M || o_cols != N) return report(halide_error_code_constraint_violated, op, "O extents must equal M x N");
+    // a tiled O may be larger than M x N: the reference's wrapper rounds it up to whole tiles
+    // (blas-gemm.cpp:10-12,32) and reads back only the M x N part; the surplus is written as zeros
+    if (!tiled && (o_rows != M || o_cols != N))
+        return report(halide_error_code_constraint_violated, op, "O extents must equal M x N");
     if (C && (C->dim[0].extent < N || C->dim[1].extent < M))
         return report(halide_error_code_access_out_of_bounds, op, "C is smaller than M x N");
     if (M == 0 || N == 0) return 0;
@@ -50,10 +53,13 @@ extern "C" int t2sp_gemm_ex(int opa, int opb, float alpha, float beta, halide_bu
     float *tmp_o = nullptr, *ws = nullptr;
     struct Release { float **a, **b; ~Release() { if (*a) pool().put(*a); if (*b) pool().put(*b); } } rel{&tmp_o, &ws};
     if (tiled) {
-        tmp_o = static_cast<float *>(pool().get((size_t)M * N * sizeof(float)));
+        tmp_o = static_cast<float *>(pool().get((size_t)o_rows * o_cols * sizeof(float)));
         if (!tmp_o) return report(halide_error_code_device_malloc_failed, op, "device allocation failed");
         flat = tmp_o;
-        ldo = N;
+        ldo = o_cols;
+        if ((o_rows != M || o_cols != N) &&
+            hipMemsetAsync(tmp_o, 0, (size_t)o_rows * o_cols * sizeof(float), api_stream()) != hipSuccess)
+            return report(halide_error_code_device_run_failed, op, "clearing the padded output failed");
     }
     const size_t ws_bytes = t2sp_sgemm_ex_workspace_bytes(opa, M, N, K);
     if (ws_bytes) {
@@ -70,7 +76,7 @@ extern "C" int t2sp_gemm_ex(int opa, int opb, float alpha, float beta, halide_bu
         const halide_dimension_t *d = O->dim;
         const int ext[6] = {d[0].extent, d[1].extent, d[2].extent, d[3].extent, d[4].extent, d[5].extent};
         const int64_t JJJ = d[0].extent, III = d[1].extent, JJ = d[2].extent, II = d[3].extent;
-        const int64_t ss[6] = {1, N, JJJ, III * N, JJJ * JJ, III * II * N};   // jjj, iii, jj, ii, j, i in the flat matrix
+        const int64_t ss[6] = {1, ldo, JJJ, III * ldo, JJJ * JJ, III * II * ldo};   // jjj, iii, jj, ii, j, i in the flat matrix
         const int64_t ds[6] = {d[0].stride, d[1].stride, d[2].stride, d[3].stride, d[4].stride, d[5].stride};
         if ((err = t2sp_relayout_f32(tmp_o, dout.ptr(), 6, ext, ss, ds, api_stream()))) return report(err, op, "relayout failed");
     }

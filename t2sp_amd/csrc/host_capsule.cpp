@@ -211,6 +211,13 @@ extern "C" int capsule(halide_buffer_t *P, halide_buffer_t *W, halide_buffer_t *
     return capsule_impl(P, W, V, T2SP_CFG_AUTO, 0);
 }
 
+// The argv form Halide declares next to every generated entry (Halide/src/CodeGen_C.cpp:1828-1833):
+// one pointer per argument, a buffer argument being the halide_buffer_t* itself.
+extern "C" int capsule_argv(void **args) {
+    if (!args) return halide_error_code_buffer_argument_is_null;
+    return capsule_impl(static_cast<halide_buffer_t *>(args[0]), static_cast<halide_buffer_t *>(args[1]), static_cast<halide_buffer_t *>(args[2]), T2SP_CFG_AUTO, 0);
+}
+
 extern "C" int t2sp_capsule_with_cfg(halide_buffer_t *P, halide_buffer_t *W, halide_buffer_t *V, int cfg, int splits) {
     return capsule_impl(P, W, V, cfg, splits);
 }
@@ -219,6 +226,6 @@ extern "C" int t2sp_capsule_with_cfg(halide_buffer_t *P, halide_buffer_t *W, hal
 // (double exec_time = capsule(device_selector, ...), t2s/src/CodeGen_OneAPI_Dev.cpp:3554-3617); this is
 // that form: the time on success, the negative error code otherwise.
 extern "C" double capsule_ns(halide_buffer_t *P, halide_buffer_t *W, halide_buffer_t *V) {
-    const int rc = capsule(P, W, V);
+    const int rc = capsule_impl(P, W, V, T2SP_CFG_AUTO, 0);
     return rc == 0 ? t2sp_last_kernel_ns() : (double)rc;
 }

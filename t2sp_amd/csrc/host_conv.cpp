@@ -318,6 +318,13 @@ extern "C" int conv(halide_buffer_t *I, halide_buffer_t *K, halide_buffer_t *O) 
     return conv_impl(I, K, O, T2SP_CFG_AUTO);
 }
 
+// The argv form Halide declares next to every generated entry (Halide/src/CodeGen_C.cpp:1828-1833):
+// one pointer per argument, a buffer argument being the halide_buffer_t* itself.
+extern "C" int conv_argv(void **args) {
+    if (!args) return halide_error_code_buffer_argument_is_null;
+    return conv_impl(static_cast<halide_buffer_t *>(args[0]), static_cast<halide_buffer_t *>(args[1]), static_cast<halide_buffer_t *>(args[2]), T2SP_CFG_AUTO);
+}
+
 extern "C" int t2sp_conv_with_cfg(halide_buffer_t *I, halide_buffer_t *K, halide_buffer_t *O, int cfg) {
     return conv_impl(I, K, O, cfg);
 }
@@ -326,6 +333,6 @@ extern "C" int t2sp_conv_with_cfg(halide_buffer_t *I, halide_buffer_t *K, halide
 // (double exec_time = conv(device_selector, ...), t2s/src/CodeGen_OneAPI_Dev.cpp:3554-3617); this is
 // that form: the time on success, the negative error code otherwise.
 extern "C" double conv_ns(halide_buffer_t *I, halide_buffer_t *K, halide_buffer_t *O) {
-    const int rc = conv(I, K, O);
+    const int rc = conv_impl(I, K, O, T2SP_CFG_AUTO);
     return rc == 0 ? t2sp_last_kernel_ns() : (double)rc;
 }

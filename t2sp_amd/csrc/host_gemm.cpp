@@ -97,6 +97,42 @@ static int gemm_panels(halide_buffer_t *A, halide_buffer_t *B, halide_buffer_t *
     return 0;
 }
 
+// Rows per panel when gemm(A, B, C) may run in row panels, else 0.  gemm_panels() takes panel p of C
+// to be the contiguous slice that starts r0*N elements into the buffer and hands the kernel C's own
+// strides relative to that slice, which holds only for a flat row-major C and for a tiled C whose
+// six dimensions are dense in their canonical order (i outermost: stride N*III*II); a dense C with
+// permuted strides runs in one piece instead.
+static int gemm_panel_rows(const halide_buffer_t *A, const halide_buffer_t *B, const halide_buffer_t *C, const Span &sc) {
+    const int K = A->dim[0].extent, M = A->dim[1].extent, N = B->dim[0].extent;
+    const bool host_only = !A->device && !B->device && !C->device && A->host && B->host && C->host;
+    if (!host_only || K <= 0 || A->dim[1].stride != K || sc.span != sc.elements) return 0;
+    int64_t quantum = 1;
+    if (C->dimensions == 6) {
+        int64_t dense = 1;
+        for (int d = 0; d < 6; d++) {
+            if (C->dim[d].stride != dense) return 0;
+            dense *= C->dim[d].extent;
+        }
+        quantum = (int64_t)C->dim[1].extent * C->dim[3].extent;
+    } else if (C->dim[1].stride != N) {
+        return 0;
+    }
+    return panel_rows(M, N, K, quantum);
+}
+
+// The gate above, for tests: the number of rows per panel gemm(A, B, C) would use, 0 = one piece.
+extern "C" int t2sp_gemm_panel_rows(const halide_buffer_t *A, const halide_buffer_t *B, const halide_buffer_t *C) {
+    if (!A || !B || !C || A->dimensions != 2 || B->dimensions != 2 || (C->dimensions != 2 && C->dimensions != 6) ||
+        !A->dim || !B->dim || !C->dim)
+        return 0;
+    Span sc{1, 1};
+    for (int d = 0; d < C->dimensions; d++) {
+        sc.elements *= C->dim[d].extent;
+        sc.span += (int64_t)(C->dim[d].extent > 0 ? C->dim[d].extent - 1 : 0) * C->dim[d].stride;
+    }
+    return gemm_panel_rows(A, B, C, sc);
+}
+
 static int gemm_impl(halide_buffer_t *A, halide_buffer_t *B, halide_buffer_t *C, int cfg) {
     static const char *op = "gemm";
     std::lock_guard<std::mutex> lock(api_mutex());
@@ -125,13 +161,9 @@ static int gemm_impl(halide_buffer_t *A, halide_buffer_t *B, halide_buffer_t *C,
         return report(halide_error_code_constraint_violated, op, "C extents must equal M x N");
     if (M == 0 || N == 0) return 0;
 
-    // host buffers, dense rows of A and a dense C: large products run in row panels
-    const bool host_only = !A->device && !B->device && !C->device && A->host && B->host && C->host;
-    if (host_only && cfg == T2SP_CFG_AUTO && K > 0 && A->dim[1].stride == K && sc.span == sc.elements &&
-        (tiled || C->dim[1].stride == N)) {
-        const int64_t quantum = tiled ? (int64_t)C->dim[1].extent * C->dim[3].extent : 1;
-        const bool tiled_dense = !tiled || (C->dim[5].stride == (int64_t)C->dim[4].stride * C->dim[4].extent);
-        const int rows = tiled_dense ? panel_rows(M, N, K, quantum) : 0;
+    // host buffers, dense rows of A and a dense C in canonical order: large products run in row panels
+    {
+        const int rows = cfg == T2SP_CFG_AUTO ? gemm_panel_rows(A, B, C, sc) : 0;
         if (rows > 0) {
             const int rc = gemm_panels(A, B, C, cfg, rows, sb);
             if (rc <= 0) return rc;                              // > 0: streams unavailable, run in one piece
@@ -176,6 +208,15 @@ extern "C" int GEMM(halide_buffer_t *A, halide_buffer_t *B, halide_buffer_t *C) 
     return gemm_impl(A, B, C, T2SP_CFG_AUTO);
 }
 
+// The argv form Halide declares next to every generated entry (Halide/src/CodeGen_C.cpp:1828-1833):
+// one pointer per argument, a buffer argument being the halide_buffer_t* itself.
+extern "C" int gemm_argv(void **args) {
+    if (!args) return halide_error_code_buffer_argument_is_null;
+    return gemm_impl(static_cast<halide_buffer_t *>(args[0]), static_cast<halide_buffer_t *>(args[1]),
+                     static_cast<halide_buffer_t *>(args[2]), T2SP_CFG_AUTO);
+}
+extern "C" int GEMM_argv(void **args) { return gemm_argv(args); }
+
 extern "C" int t2sp_gemm_with_cfg(halide_buffer_t *A, halide_buffer_t *B, halide_buffer_t *C, int cfg) {
     return gemm_impl(A, B, C, cfg);
 }
@@ -184,6 +225,6 @@ extern "C" int t2sp_gemm_with_cfg(halide_buffer_t *A, halide_buffer_t *B, halide
 // (double exec_time = gemm(device_selector, ...), t2s/src/CodeGen_OneAPI_Dev.cpp:3554-3617); this is
 // that form: the time on success, the negative error code otherwise.
 extern "C" double gemm_ns(halide_buffer_t *A, halide_buffer_t *B, halide_buffer_t *C) {
-    const int rc = gemm(A, B, C);
+    const int rc = gemm_impl(A, B, C, T2SP_CFG_AUTO);
     return rc == 0 ? t2sp_last_kernel_ns() : (double)rc;
 }

@@ -73,6 +73,14 @@ extern "C" int mttkrp(halide_buffer_t *B, halide_buffer_t *C, halide_buffer_t *D
     return mttkrp_impl(B, C, D, A, T2SP_CFG_AUTO, 0);
 }
 
+// The argv form Halide declares next to every generated entry (Halide/src/CodeGen_C.cpp:1828-1833):
+// one pointer per argument, a buffer argument being the halide_buffer_t* itself.
+extern "C" int mttkrp_argv(void **args) {
+    if (!args) return halide_error_code_buffer_argument_is_null;
+    return mttkrp_impl(static_cast<halide_buffer_t *>(args[0]), static_cast<halide_buffer_t *>(args[1]),
+                       static_cast<halide_buffer_t *>(args[2]), static_cast<halide_buffer_t *>(args[3]), T2SP_CFG_AUTO, 0);
+}
+
 extern "C" int t2sp_mttkrp_with_cfg(halide_buffer_t *B, halide_buffer_t *C, halide_buffer_t *D,
                                     halide_buffer_t *A, int cfg, int splits) {
     return mttkrp_impl(B, C, D, A, cfg, splits);
@@ -82,6 +90,6 @@ extern "C" int t2sp_mttkrp_with_cfg(halide_buffer_t *B, halide_buffer_t *C, hali
 // (double exec_time = mttkrp(device_selector, ...), t2s/src/CodeGen_OneAPI_Dev.cpp:3554-3617); this is
 // that form: the time on success, the negative error code otherwise.
 extern "C" double mttkrp_ns(halide_buffer_t *B, halide_buffer_t *C, halide_buffer_t *D, halide_buffer_t *A) {
-    const int rc = mttkrp(B, C, D, A);
+    const int rc = mttkrp_impl(B, C, D, A, T2SP_CFG_AUTO, 0);
     return rc == 0 ? t2sp_last_kernel_ns() : (double)rc;
 }

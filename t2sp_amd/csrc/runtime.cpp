@@ -15,7 +15,12 @@ std::mutex &api_mutex() {
 // queued on it (for example a framework that filled a pre-staged device buffer).
 hipStream_t api_stream() { return nullptr; }
 
+// Kernel time of the last call: per calling thread (an entry point runs in its caller's thread and
+// publishes while it holds the library lock, so a second thread's call cannot overwrite what the
+// first is about to read), with the process-wide latest as the answer for a thread that has made
+// no call itself.
 static std::atomic<double> g_last_kernel_ns{0.0};
+static thread_local double tl_last_kernel_ns = -1.0;
 static hipEvent_t g_ev0 = nullptr, g_ev1 = nullptr;
 
 int report(int code, const char *op, const char *what) {
@@ -215,6 +220,7 @@ int KernelTimer::stop_and_sync(const char *op) {
 
 void publish_kernel_ns(double ns, const char *op) {
     g_last_kernel_ns = ns;
+    tl_last_kernel_ns = ns;
     // Optional file in the reference's exec_time.txt format (AOT-OpenCL-Runtime.cpp:380-394):
     // overall ns on the first line, then "<kernel_name> <ns>" lines.  The reference's drivers ask
     // for "kernel_unloader", the last kernel of its pipeline, so that name is written too.
@@ -230,7 +236,9 @@ void publish_kernel_ns(double ns, const char *op) {
 
 }  // namespace t2sp
 
-extern "C" double t2sp_last_kernel_ns(void) { return t2sp::g_last_kernel_ns.load(); }
+extern "C" double t2sp_last_kernel_ns(void) {
+    return t2sp::tl_last_kernel_ns >= 0.0 ? t2sp::tl_last_kernel_ns : t2sp::g_last_kernel_ns.load();
+}
 
 extern "C" void t2sp_release(void) {
     std::lock_guard<std::mutex> lock(t2sp::api_mutex());

@@ -198,3 +198,115 @@ def test_packed_capsule_form_is_checked_without_a_device():
         assert L.capsule(P.ref, W.ref, V.ref) == -8                                  # CII does not divide TOTAL_CI
     finally:
         L.t2sp_capsule_design(0)
+
+
+def test_argv_entries_take_one_pointer_per_argument():
+    """`<fn>_argv(void **args)` next to each entry (Halide/src/CodeGen_C.cpp:1828-1833): the same
+    argument checks run behind it, so a NULL buffer comes back as -12 and bad dimensions as -43."""
+    L = t2sp_amd.lib()
+    a, b, c = _buf((8, 4)), _buf((4, 12)), _buf((8, 12))
+
+    def argv(*bufs):
+        return (ctypes.c_void_p * len(bufs))(*[ctypes.cast(x.ref, ctypes.c_void_p) if x is not None else None for x in bufs])
+    for name in ("gemm_argv", "GEMM_argv"):
+        fn = getattr(L, name)
+        fn.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+        assert fn(argv(a, b, None)) == -12
+        assert fn(argv(_buf((2, 8, 4)), b, c)) == -43
+        assert fn(argv(a, _buf((5, 12)), c)) == -8
+        assert fn(None) == -12
+    for name, n in (("conv_argv", 3), ("capsule_argv", 3), ("mttkrp_argv", 4)):
+        fn = getattr(L, name)
+        fn.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+        assert fn(argv(*([None] + [a] * (n - 1)))) == -12
+        assert fn(None) == -12
+
+
+def test_row_panels_only_for_canonically_dense_outputs():
+    """gemm() moves large host products through the device in row panels and takes panel p of C to be
+    the contiguous slice r0*N elements in; that holds for a flat C and for a tiled C whose six
+    dimensions are dense in their own order, not for a dense C with permuted strides."""
+    L = t2sp_amd.lib()
+    L.t2sp_gemm_panel_rows.argtypes = [ctypes.POINTER(halide_buffer_t)] * 3
+    M = N = K = 8192
+    JJJ, III, JJ, II = 8, 16, 2, 4
+    J, I = N // (JJJ * JJ), M // (III * II)
+    one = np.zeros(1, np.float32)                               # extents and strides only; never dereferenced
+
+    def buf(ext, strides):
+        return HalideBuffer(ext, strides, host=one.ctypes.data, keep=one)
+    a, b = buf([K, M], [1, K]), buf([N, K], [1, N])
+    flat = buf([N, M], [1, N])
+    assert L.t2sp_gemm_panel_rows(a.ref, b.ref, flat.ref) >= 256
+    assert L.t2sp_gemm_panel_rows(a.ref, b.ref, buf([N, M], [1, N + 8]).ref) == 0          # padded rows
+    ext = [JJJ, III, JJ, II, J, I]
+    dense = [1, JJJ, JJJ * III, JJJ * III * JJ, JJJ * III * JJ * II, JJJ * III * JJ * II * J]
+    rows = L.t2sp_gemm_panel_rows(a.ref, b.ref, buf(ext, dense).ref)
+    assert rows >= 256 and rows % (III * II) == 0
+    # dense but permuted: s0=1, s2=JJJ, s4=JJJ*JJ, s5=N, s1=N*I, s3=N*I*III (every element has a place,
+    # span == elements, and the old check s5 == s4*J also held)
+    permuted = [1, N * I, JJJ, N * I * III, JJJ * JJ, N]
+    assert 1 + sum((e - 1) * s for e, s in zip(ext, permuted)) == M * N
+    assert L.t2sp_gemm_panel_rows(a.ref, b.ref, buf(ext, permuted).ref) == 0
+    small = buf([256, 256], [1, 256])
+    assert L.t2sp_gemm_panel_rows(small.ref, small.ref, small.ref) == 0                     # short copies: one piece
+    dev = buf([N, M], [1, N])
+    dev.struct.device = 1
+    assert L.t2sp_gemm_panel_rows(a.ref, b.ref, dev.ref) == 0                               # device-resident
+
+
+def test_roofline_writes_a_png_the_reference_drivers_can_open(tmp_path):
+    """roofline() must leave roofline.png behind (every LARGE branch of the reference's drivers checks
+    for it, gemm-run-fpga.cpp:101-104).  Decoded here with zlib: signature, chunk CRCs, size, and the
+    pixel of the measured point."""
+    import struct
+    import zlib
+    L = t2sp_amd.lib()
+    fn = L._Z8rooflineddddd
+    fn.argtypes = [ctypes.c_double] * 5
+    fn.restype = None
+    cwd = os.getcwd()
+    os.chdir(tmp_path)
+    try:
+        fn(8000.0, 157.3e6, 1.0995e12, 805e6, 7.28e6)          # GB/s, MFLOP/s, flop, bytes, ns
+    finally:
+        os.chdir(cwd)
+    d = (tmp_path / "roofline.png").read_bytes()
+    assert d[:8] == b"\x89PNG\r\n\x1a\n"
+    off, idat, seen = 8, b"", []
+    while off < len(d):
+        n, = struct.unpack(">I", d[off:off + 4])
+        kind, body = d[off + 4:off + 8], d[off + 8:off + 8 + n]
+        assert zlib.crc32(kind + body) == struct.unpack(">I", d[off + 8 + n:off + 12 + n])[0]
+        seen.append(kind)
+        if kind == b"IHDR":
+            w, h, depth, colour = struct.unpack(">IIBB", body[:10])
+        if kind == b"IDAT":
+            idat += body
+        off += 12 + n
+    assert seen[0] == b"IHDR" and seen[-1] == b"IEND" and (depth, colour) == (8, 2)
+    raw = zlib.decompress(idat)
+    assert len(raw) == h * (1 + 3 * w)
+    rows = np.frombuffer(raw, np.uint8).reshape(h, 1 + 3 * w)
+    assert (rows[:, 0] == 0).all()
+    img = rows[:, 1:].reshape(h, w, 3)
+    # the point: x = ops/bytes of xmax = 1.5*x, y = 151 of ymax = 2*157.3 TFLOP/s, drawn in steel blue
+    x = int(50 + (w - 70) / 1.5)
+    y = int(h - 40 - (h - 60) * (1.0995e12 / 7.28e6) / (2 * 157.3e3))
+    assert tuple(img[y, x]) == (0x46, 0x82, 0xB4)
+    assert (tmp_path / "roofline.txt").exists() and (tmp_path / "roofline.svg").exists()
+
+
+def test_blas_library_exports_the_eight_argument_gemm():
+    """libt2sp_blas_gemm.so holds the reference's 8-argument gemm(opa, opb, alpha, beta, A, B, C, O)
+    (blas-gemm.cpp:29) under its C name; argument checks answer without a device."""
+    path = os.path.join(os.path.dirname(t2sp_amd.lib_path()), "libt2sp_blas_gemm.so")
+    assert os.path.exists(path), "make -C t2sp_amd/csrc builds it"
+    B = ctypes.CDLL(path)
+    bp = ctypes.POINTER(halide_buffer_t)
+    B.gemm.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_float, ctypes.c_float, bp, bp, bp, bp]
+    a, b, c = _buf((8, 4)), _buf((4, 12)), _buf((8, 12))
+    assert B.gemm(0, 0, 1.0, 0.0, a.ref, b.ref, c.ref, None) == -12
+    assert B.gemm(0, 0, 1.0, 0.0, a.ref, _buf((5, 12)).ref, c.ref, c.ref) == -8
+    assert B.gemm(0, 0, 1.0, 0.0, a.ref, b.ref, c.ref, _buf((4, 12)).ref) == -4
+    assert hasattr(B, "gemm_argv")

@@ -93,3 +93,35 @@ def test_tiled_output_and_in_place_device(oracle):
     t2sp_amd.gemm_ex(0, 0, 2.0, 0.5, Ad, Bd, Cd, out=Cd)       # c = alpha*a*b + beta*c in place
     torch.cuda.synchronize()
     assert (Cd.cpu().numpy() == flat).all()
+
+
+def test_eight_argument_gemm_as_the_reference_wrapper_calls_it(oracle):
+    """libt2sp_blas_gemm.so: gemm(opa, opb, alpha, beta, A, B, C, O) under its C name, called the way
+    blas-gemm.cpp:10-29 calls it: m, n not multiples of the tile, O(JJJ, III, JJ, II, J, I) rounded up
+    to whole tiles, the M x N part read back (blas-gemm.cpp:31-41), the surplus zero."""
+    import ctypes
+    import os
+    from t2sp_amd.buffer import HalideBuffer, halide_buffer_t
+    Bl = ctypes.CDLL(os.path.join(os.path.dirname(t2sp_amd.lib_path()), "libt2sp_blas_gemm.so"))
+    bp = ctypes.POINTER(halide_buffer_t)
+    Bl.gemm.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_float, ctypes.c_float, bp, bp, bp, bp]
+    m, n, k = 100, 60, 72
+    III, II, JJJ, JJ = 16, 4, 8, 2                              # 64 x 16 tiles: O covers 128 x 64
+    I, J = -(-m // (III * II)), -(-n // (JJJ * JJ))
+    A, B, C = oracle.fill_uniform((m, k), 41), oracle.fill_uniform((k, n), 42), oracle.fill_uniform((m, n), 43)
+    O = np.full((I, J, II, JJ, III, JJJ), np.nan, np.float32)
+    a, b, c, o = (HalideBuffer.from_numpy(x) for x in (A, B, C, O))
+    assert Bl.gemm(0, 0, 2.0, 0.5, a.ref, b.ref, c.ref, o.ref) == 0
+    full = O.transpose(0, 2, 4, 1, 3, 5).reshape(I * II * III, J * JJ * JJJ)      # (i, ii, iii), (j, jj, jjj)
+    ref = 2.0 * oracle.gemm(A, B, acc=oracle.ACC_F64).astype(np.float64) + 0.5 * C
+    assert rel_fro(full[:m, :n], ref)[0] <= TOL
+    assert (full[m:] == 0).all() and (full[:, n:] == 0).all()
+    # the argv form of the same entry: scalars by address, buffers as themselves
+    Bl.gemm_argv.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+    O2 = np.full_like(O, np.nan)
+    o2 = HalideBuffer.from_numpy(O2)
+    sc = (ctypes.c_int32(0), ctypes.c_int32(0), ctypes.c_float(2.0), ctypes.c_float(0.5))
+    args = (ctypes.c_void_p * 8)(*[ctypes.cast(ctypes.pointer(x), ctypes.c_void_p) for x in sc],
+                                 *[ctypes.cast(x.ref, ctypes.c_void_p) for x in (a, b, c, o2)])
+    assert Bl.gemm_argv(args) == 0
+    assert (O2 == O).all()
