@@ -13,9 +13,12 @@ printed:
                   this host on a bounded sample of the same workload
   parity          relative Frobenius / max-abs error of this run's result against
                   the CPU oracle on sampled rows
-  others          the remaining benchmark configurations (SGEMM sweep; conv,
-                  capsule, MTTKRP once built), each with its own TFLOP/s and
-                  fraction of peak
+  others          the remaining benchmark configurations (SGEMM sweep and 1024^3,
+                  conv, capsule, MTTKRP), each with its own TFLOP/s, fraction of
+                  peak, parity against the oracle and (the four named
+                  configurations) its own cpu_baseline; then the kernels of the
+                  next rows
+  end_to_end      gemm() on host buffers, copies included (never `value`)
 """
 import argparse
 import json
@@ -28,10 +31,28 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3   # 256 CU x 256 flop/clk/CU x 2.4 GHz
 PEAK_HBM_GBS = 8000.0
-# Bytes the L2s fetch from / write to the fabric per SGEMM 8192^3 launch: rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE (two runs of this script with --calibrate-copy), each scaled by what the same counter reads
-# for the 256 MiB calibration copy (x1.999 and x1.000); summary in profiles/all_kernels_hbm_traffic_pmc.md.
-SGEMM_8192_TRAFFIC_BYTES = 3.49e9
+# Bytes the L2s fetch from / write to the fabric per SGEMM 8192^3 launch come from a tracked summary of two
+# rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter
+# reads for the 256 MiB calibration copy of --calibrate-copy); `python -m t2sp_amd.pmc_summary` writes it.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "sgemm_8192_hbm_traffic.txt")
+
+
+def load_traffic():
+    """(bytes per launch, description) from the tracked counter summary, or (None, reason)."""
+    try:
+        fields = {}
+        for line in open(TRAFFIC_FILE):
+            line = line.strip()
+            if line and not line.startswith("#"):
+                key, _, val = line.partition(" ")
+                fields[key] = val.strip()
+        return float(fields["traffic_bytes"]), (
+            "bytes per launch, L2<->fabric, read from profiles/%s: rocprofv3 FETCH_SIZE %s KiB x %s + WRITE_SIZE %s KiB x %s "
+            "(scales from a 256 MiB copy kernel); algorithmic 8.05e8" % (
+                os.path.basename(TRAFFIC_FILE), fields.get("fetch_kib_raw"), fields.get("fetch_scale"),
+                fields.get("write_kib_raw"), fields.get("write_scale")))
+    except (OSError, KeyError, ValueError) as e:
+        return None, "no counter summary at profiles/%s (%s)" % (os.path.basename(TRAFFIC_FILE), type(e).__name__)
 
 
 def parse():
@@ -159,6 +180,116 @@ def cpu_baseline_gemm(oracle, M, N, K, budget_s):
     }
 
 
+def parity_of(got, ref, what):
+    import numpy as np
+    got, ref = np.asarray(got, np.float64), np.asarray(ref, np.float64)
+    return {"rel_frobenius": float(np.linalg.norm(got - ref) / max(np.linalg.norm(ref), 1e-300)),
+            "max_abs": float(np.abs(got - ref).max()), "checked": what}
+
+
+def cpu_baseline_sgemm_1024(oracle, A, B):
+    """configs[0] is the size that runs on the CPU path in full: the golden loop (gemm-run-fpga.cpp:74-86),
+    scalar accumulator, i,j,k order, one thread, every output."""
+    t0 = time.perf_counter()
+    oracle.gemm_literal(A, B)
+    dt = time.perf_counter() - t0
+    return {"value": round(2.0 * 1024 ** 3 / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": "golden loop (i,j,k order, scalar accumulator), the full 1024^3 problem, single thread, %.1f s" % dt}
+
+
+def check_conv(oracle, tensors, cpu_seconds):
+    """configs[2]: parity on two images x 24 output channels; CPU: the golden loop order (ci -> kx -> ky per
+    output, conv-run-fpga.cpp:73-93), one thread, on a declared sample of output channels of one image."""
+    I, W, O = tensors
+    N, CO = I.shape[0], W.shape[0]
+    imgs, cos = [0, N - 1], slice(100, 124)
+    In, Wn = I[imgs].cpu().numpy(), W.cpu().numpy()
+    # device layout [n][c][h][w] with w = the reference's y: the oracle indexes (n, ci, y, x)
+    ref = oracle.conv(In.transpose(0, 1, 3, 2), Wn.transpose(0, 1, 3, 2), co_range=(cos.start, cos.stop))[:, cos]
+    got = O[imgs][:, cos].cpu().numpy().transpose(0, 1, 3, 2)
+    out = {"parity": parity_of(got, ref, "images 0 and %d, output channels 100-123, against the CPU oracle (golden order)" % (N - 1))}
+    if cpu_seconds:
+        one, Wt = In[:1].transpose(0, 1, 3, 2), Wn.transpose(0, 1, 3, 2)
+        t0 = time.perf_counter()
+        oracle.conv(one, Wt, co_range=(0, 4), threads=1)
+        per_co = (time.perf_counter() - t0) / 4
+        n_co = int(max(4, min(CO, cpu_seconds / max(per_co, 1e-6))))
+        t0 = time.perf_counter()
+        oracle.conv(one, Wt, co_range=(0, n_co), threads=1)
+        dt = time.perf_counter() - t0
+        flop = 2.0 * n_co * O.shape[2] * O.shape[3] * I.shape[1] * 9
+        out["cpu_baseline"] = {"value": round(flop / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                               "sample": "sampled: golden order per output, single thread, %d of %d output channels of 1 of %d "
+                                         "images, %.1f s; extrapolated full problem: %.0f s" % (n_co, CO, N, dt, dt * CO / n_co * N)}
+    return out
+
+
+def check_capsule(oracle, tensors, cpu_seconds):
+    """configs[3]: parity on every vote; CPU: the golden loop order (kx -> ky -> mk -> ci per vote,
+    capsule-run-fpga.cpp:78-104), one thread, the full problem."""
+    P, W, V = tensors
+    Pn, Wn = P.cpu().numpy(), W.cpu().numpy()
+    # device layout P [n][ci][h][w][mx][mk] with w = the reference's y: the oracle indexes (n, ci, y, x, mx, mk)
+    Pt, Wt = Pn.transpose(0, 1, 3, 2, 4, 5), Wn.transpose(0, 1, 3, 2, 4, 5)
+    t0 = time.perf_counter()
+    ref = oracle.capsule(Pt, Wt, threads=1)
+    dt = time.perf_counter() - t0
+    out = {"parity": parity_of(V.cpu().numpy().transpose(0, 1, 3, 2, 4, 5), ref, "all %d votes against the CPU oracle (golden order)" % ref.size)}
+    if cpu_seconds:
+        flop = 2.0 * ref.size * Pn.shape[1] * 9 * 4
+        out["cpu_baseline"] = {"value": round(flop / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                               "sample": "golden order per vote, single thread, the full problem, %.1f s" % dt}
+    return out
+
+
+def check_mttkrp(oracle, tensors, cpu_seconds):
+    """configs[4]: parity on sampled rows i; CPU: the helper's two-step order (util.h:498-515), one thread,
+    on a declared sample of rows i."""
+    import numpy as np
+    B, C, D, A = tensors                                          # views indexed (i,j,k), (j,r), (k,r), (i,r)
+    I = B.shape[0]
+    rows = [0, 1, I // 2, I - 1]
+    Bn, Cn, Dn = B.cpu().numpy(), C.cpu().numpy(), D.cpu().numpy()
+    An = A.cpu().numpy()
+    ref = np.stack([oracle.mttkrp(Bn, Cn, Dn, i_range=(r, r + 1))[r] for r in rows])
+    out = {"parity": parity_of(An[rows], ref, "rows i = %s against the CPU oracle (the helper's two-step order)" % rows)}
+    if cpu_seconds:
+        t0 = time.perf_counter()
+        oracle.mttkrp(Bn, Cn, Dn, i_range=(0, 1), threads=1)
+        per_row = time.perf_counter() - t0
+        n_rows = int(max(1, min(I, cpu_seconds / max(per_row, 1e-6))))
+        t0 = time.perf_counter()
+        oracle.mttkrp(Bn, Cn, Dn, i_range=(0, n_rows), threads=1)
+        dt = time.perf_counter() - t0
+        flop = n_rows * (2.0 * B.shape[1] * B.shape[2] * C.shape[1])
+        out["cpu_baseline"] = {"value": round(flop / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                               "sample": "sampled: two-step order of util.h:498-515, single thread, %d of %d rows i, %.1f s; "
+                                         "extrapolated full problem: %.0f s" % (n_rows, I, dt, dt * I / n_rows)}
+    return out
+
+
+def end_to_end_gemm(torch, t2sp_amd, M, N, K):
+    """The drop-in entry on host buffers: gemm(A, B, C) with page-locked host memory (t2sp_host_malloc),
+    copies in, kernels and copies out included.  Never `value`: the link, not the kernel, bounds it."""
+    A, B, C = t2sp_amd.host_empty((M, K)), t2sp_amd.host_empty((K, N)), t2sp_amd.host_empty((M, N))
+    A[:] = 0.5
+    B[:] = 0.25
+    t2sp_amd.gemm(A, B, out=C)
+    best, kernel = 1e30, 0.0
+    for _ in range(3):
+        t0 = time.perf_counter()
+        t2sp_amd.gemm(A, B, out=C)
+        dt = time.perf_counter() - t0
+        if dt < best:
+            best, kernel = dt, t2sp_amd.last_kernel_ns() * 1e-9
+    ok = bool((C[::1023, ::1023] == 0.125 * K).all())
+    t2sp_amd.release()
+    return {"entry": "gemm(A, B, C) on page-locked host buffers, %dx%dx%d" % (M, N, K), "ms": round(best * 1e3, 3),
+            "TFLOP/s": round(2.0 * M * N * K / best / 1e12, 2), "kernel_ms": round(kernel * 1e3, 3),
+            "host_bytes_moved": 4 * (M * K + K * N + M * N), "result_ok": ok,
+            "note": "PCIe-inclusive; rows of A and C move in panels so that copies overlap the kernels"}
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -173,6 +304,7 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     t2sp_amd.lib()
+    from oracle import oracle          # the CPU checker: parity and cpu_baseline legs only, never timed as the product
 
     if args.calibrate_copy:
         import ctypes
@@ -191,6 +323,7 @@ def main():
     tflops = r["flop"] / (r["wall_ms"] * 1e-3) / 1e12
     kernel_tflops = r["flop"] / (r["avg_ms"] * 1e-3) / 1e12
 
+    traffic, traffic_note = load_traffic()
     out = {
         "metric": "fp32 TFLOPS + % of fp32-MFMA peak, SGEMM 8192^3 on 1 MI355X",
         "value": round(tflops, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -200,13 +333,12 @@ def main():
                    "entry": "t2sp_sgemm_f32", "inputs": "resident in HBM"},
         "pct_of_peak": round(100.0 * tflops / PEAK_FP32_MFMA_TFLOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 3), "peak": PEAK_FP32_MFMA_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(kernel_tflops / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": SGEMM_8192_TRAFFIC_BYTES,
-                     "traffic_note": "bytes per launch, L2<->fabric, from rocprofv3 FETCH_SIZE+WRITE_SIZE scaled by a copy kernel; algorithmic 8.05e8",
+                     "unit": "TFLOP/s", "frac": round(kernel_tflops / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": traffic,
+                     "traffic_note": traffic_note,
                      "kernel": "sgemm_kernel<256x256x16>", "avg_launch_ms": round(r["avg_ms"], 4),
                      "best_launch_ms": round(r["min_ms"], 4), "flop_per_launch": r["flop"]},
     }
 
-    from oracle import oracle
     rows = np.unique(np.concatenate([[0, M - 1], np.random.default_rng(0).integers(0, M, 30)]))
     idx = torch.as_tensor(rows, device="cuda")
     ref = oracle.gemm(r["A"][idx].cpu().numpy(), r["B"].cpu().numpy())
@@ -218,19 +350,36 @@ def main():
 
     if not args.no_others:
         others = {}
-        for (m, n, k) in [(4096, 16384, 2048), (16384, 4096, 8192), (1024, 1024, 1024)]:
+        for (m, n, k) in [(4096, 16384, 2048), (16384, 4096, 8192)]:
             c = sgemm_case(torch, t2sp_amd, m, n, k, max(5, args.steps // 2), 5, min_warm_ms=100.0)
             tf = c["flop"] / (c["avg_ms"] * 1e-3) / 1e12
             others["sgemm_%dx%dx%d" % (m, n, k)] = {"TFLOP/s": round(tf, 3), "frac_of_peak": round(tf / PEAK_FP32_MFMA_TFLOPS, 4),
-                                                    "avg_launch_ms": round(c["avg_ms"], 4)}
+                                                    "avg_launch_ms": round(c["avg_ms"], 4),
+                                                    "parity": parity_of(c["C"][:24].cpu().numpy(),
+                                                                        oracle.gemm(c["A"][:24].cpu().numpy(), c["B"].cpu().numpy()),
+                                                                        "rows 0-23 against the CPU oracle (golden order)")}
             del c
-        try:
-            from t2sp_amd import bench_ops
-            others.update(bench_ops.run_all(torch, max(5, args.steps // 2), 5, PEAK_FP32_MFMA_TFLOPS, args.capsule_cfg,
-                                            args.capsule_splits))
-        except ImportError:
-            pass
+        # configs[0]: SGEMM 1024^3 from seed 0, whole result against the oracle, golden loop timed in full
+        c = sgemm_case(torch, t2sp_amd, 1024, 1024, 1024, max(200, args.steps), 20, seed=0, min_warm_ms=100.0)
+        tf = c["flop"] / (c["avg_ms"] * 1e-3) / 1e12
+        e = {"TFLOP/s": round(tf, 3), "frac_of_peak": round(tf / PEAK_FP32_MFMA_TFLOPS, 4), "avg_launch_ms": round(c["avg_ms"], 5),
+             "workload": "M=N=K=1024, seeds 0,1 (configs[0])"}
+        A1, B1 = c["A"].cpu().numpy(), c["B"].cpu().numpy()
+        e["parity"] = parity_of(c["C"].cpu().numpy(), oracle.gemm(A1, B1), "all 1024 x 1024 outputs against the CPU oracle (golden order)")
+        if not args.no_cpu:
+            e["cpu_baseline"] = cpu_baseline_sgemm_1024(oracle, A1, B1)
+        others["sgemm_1024x1024x1024"] = e
+        del c
+        from t2sp_amd import bench_ops
+        more = bench_ops.run_all(torch, max(5, args.steps // 2), 5, PEAK_FP32_MFMA_TFLOPS, args.capsule_cfg, args.capsule_splits)
+        for name, check in (("conv2d", check_conv), ("capsule", check_capsule), ("mttkrp", check_mttkrp)):
+            tensors = more[name].pop("_tensors")
+            more[name].update(check(oracle, tensors, None if args.no_cpu else args.cpu_seconds / 4))
+            del tensors
+        others.update(more)
         out["others"] = others
+        if not args.no_cpu:
+            out["end_to_end"] = end_to_end_gemm(torch, t2sp_amd, M, N, K)
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_gemm(oracle, M, N, K, args.cpu_seconds)

@@ -1,5 +1,7 @@
-"""Timed launches of the non-headline benchmark configurations (conv, capsule, MTTKRP),
-used by bench.py's `others` block.  Inputs are synthetic, seeded, resident in HBM."""
+"""Timed launches of the non-headline benchmark configurations (conv, capsule, MTTKRP) and of the
+kernels of the next rows, used by bench.py's `others` block.  Inputs are synthetic, seeded, resident
+in HBM.  The three benchmark configurations hand their device tensors back under "_tensors" so that
+the caller can check the result of the timed launches; bench.py removes that key before printing."""
 import ctypes
 
 from . import ops
@@ -53,7 +55,9 @@ def conv_config3(torch, steps, warmup, peak):
 
     ms = _time(torch, launch, steps, warmup)
     flop = 2.0 * N * CO * OH * OW * CI * 9
-    return _entry(flop / ms / 1e9, peak, ms, workload="N=64 CI=CO=256 56x56 out 3x3 NCHW (configs[2])")
+    e = _entry(flop / ms / 1e9, peak, ms, workload="N=64 CI=CO=256 56x56 out 3x3 NCHW, seeds 1,2 (configs[2])")
+    e["_tensors"] = (I, W, O)
+    return e
 
 
 def capsule_config4(torch, steps, warmup, peak, cfg=0, splits=0):
@@ -75,9 +79,11 @@ def capsule_config4(torch, steps, warmup, peak, cfg=0, splits=0):
 
     ms = _time(torch, launch, max(steps, 200), max(warmup, 20))
     flop = 2.0 * N * CO * 49 * 16 * CI * 9 * 4
-    return _entry(flop / ms / 1e9, peak, ms, workload="N=32 CI=CO=32 15x15->7x7 3x3 s2 4x4 poses (configs[3])",
-                  note="back-to-back launches; the library's own choice is one direct kernel without a split-reduction "
-                       "pass" if cfg == 0 else "forced cfg %d splits %d" % (cfg, splits))
+    e = _entry(flop / ms / 1e9, peak, ms, workload="N=32 CI=CO=32 15x15->7x7 3x3 s2 4x4 poses, seeds 1,2 (configs[3])",
+               note="back-to-back launches; the library's own choice is one direct kernel without a split-reduction "
+                    "pass" if cfg == 0 else "forced cfg %d splits %d" % (cfg, splits))
+    e["_tensors"] = (P, W, V)
+    return e
 
 
 def mttkrp_config5(torch, steps, warmup, peak):
@@ -100,8 +106,10 @@ def mttkrp_config5(torch, steps, warmup, peak):
 
     ms = _time(torch, launch, steps, warmup)
     flop = 2.0 * I * J * K * R + J * K * R
-    return _entry(flop / ms / 1e9, peak, ms, workload="I=J=K=512 R=256, helper layout (configs[4])",
-                  note="includes the split-reduction kernel")
+    e = _entry(flop / ms / 1e9, peak, ms, workload="I=J=K=512 R=256, helper layout, seeds 1,2,3 (configs[4])",
+               note="includes the split-reduction kernel")
+    e["_tensors"] = (B, C, D, A)
+    return e
 
 
 def ssyrk_case(torch, steps, warmup, peak, N, K, note):
