@@ -313,76 +313,53 @@ __global__ void __launch_bounds__(NW * 64) capsule_direct_kernel(const CapsuleAr
 // benchmark shape has 196 workgroups for 256 CUs; here a workgroup owns `rows_per_tile` vote rows
 // (whole pixels: a multiple of 4, up to 16*MB) by NB blocks of 16 columns, and the host picks NB and
 // rows_per_tile so that the workgroups come to just under a multiple of 256 (see plan_direct16; 256
-// tiles of 196 x 16 at the
-// benchmark shape).  v_mfma_f32_16x16x4_f32 takes per lane one float of X at (row l%16, k-slot
-// l/16) and of Y at (k-slot l/16, col l%16) and leaves D[4*(l/16) + r][l%16] in register r.  A step
-// is 4 pose rows of the reduction (16 k): lane group l/16 loads pose row 4*step + l/16 as 128 bits
-// (its 4 mk) per row block and uses element j in MFMA j, so the k-slots of MFMA j are the mk = j
-// entries of 4 consecutive pose rows; the weights are single floats W[(pose row, mk = j)][co, my].
-// The reduction is split over the 4 waves and summed through LDS in wave order, as above.
-constexpr int D16_WAVES = 4;
-constexpr int D16_RING = 3;
+// tiles of 196 x 16 at the benchmark shape).  v_mfma_f32_16x16x4_f32 takes per lane one float of X
+// at (row l%16, k-slot l/16) and of Y at (k-slot l/16, col l%16) and leaves D[4*(l/16) + r][l%16] in
+// register r.  A step is 4 pose rows of the reduction (16 k): lane group l/16 loads pose row
+// 4*step + l/16 as 128 bits (its 4 mk) per row block and uses element j in MFMA j, so the k-slots of
+// MFMA j are the mk = j entries of 4 consecutive pose rows; the weights are single floats
+// W[(pose row, mk = j)][co, my].
+//
+// A workgroup has D16_WAVES * D16_ROWSPLIT waves, two per SIMD: wave (kq, rh) takes share kq of the
+// reduction and share rh of the row blocks, so the two waves of a SIMD, (kq, 0) and (kq, 1), split
+// what one wave would do and either can issue MFMAs while the other waits for its operands (one
+// wave per SIMD left the matrix pipe idle for a third of the kernel: 20.3 -> 18.7 us at the
+// benchmark shape), and one register set of operands ahead is enough with two (18.3 us).  The
+// per-pixel offsets of the tile and, per share of the reduction, the offsets of its pose rows are
+// tabulated in LDS first, by all waves together.  The partial tiles of the D16_WAVES shares are summed through LDS in the order
+// of kq, as above, so the result does not depend on timing.
+constexpr int D16_WAVES = 4;         // shares of the reduction
+constexpr int D16_ROWSPLIT = 2;      // shares of the row blocks = waves per SIMD
+constexpr int D16_RING = 2;          // operand register sets
 constexpr int D16_MAX_MB = 8;        // row blocks of 16 per workgroup with two column blocks
 constexpr int D16_MAX_MB_TALL = 13;  // with one
 typedef float v4f_acc __attribute__((ext_vector_type(4)));
 
-template <int MB, int NB, int NW, int R>
-__global__ void __launch_bounds__(NW * 64) capsule_direct16_kernel(const CapsuleArgs g, int rows_per_tile,
-                                                                   int tab_entries) {
-    extern __shared__ __align__(16) float smem[];
-    v4f *red = reinterpret_cast<v4f *>(smem);                                   // [wave][mb][nb][lane]
-    uint32_t *pix_p = reinterpret_cast<uint32_t *>(smem + NW * MB * NB * 64 * 4);  // [4*MB] byte offsets in P
-    uint32_t *pix_v = pix_p + 4 * MB;                                            // [4*MB] byte offsets in V, ~0u: none
-    uint2 *tab_all = reinterpret_cast<uint2 *>(pix_v + 4 * MB);
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+template <int MBW, int NB>
+__device__ __forceinline__ void direct16_wave(const CapsuleArgs &g, int mb0, int nsteps, int s0, int n0, const uint32_t *pix_p,
+                                              const uint2 *tab, v4f *red_kq) {
+    constexpr int R = D16_RING;
     const int lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
-    const int tm = blockIdx.x % g.tiles_m, tn = blockIdx.x / g.tiles_m;   // the column tiles of one row tile: same XCD
-    const int r0 = tm * rows_per_tile, n0 = tn * 16 * NB;
-
-    // pixels of this tile: offsets of (n, h, w) in P and in V
-    const int pix_total = g.ROWS >> 2, pix0 = r0 >> 2, pix_n = min(rows_per_tile >> 2, pix_total - pix0);
-    if (threadIdx.x < 4 * MB) {
-        const int t = threadIdx.x;
-        const int pix = pix0 + (t < pix_n ? t : 0);
-        const int w = pix % g.OW, hn = pix / g.OW, h = hn % g.OH, n = hn / g.OH;
-        pix_p[t] = 4u * (uint32_t)(int)(n * g.sp[0] + h * g.S * g.sp[2] + w * g.S * g.sp[3]);
-        pix_v[t] = t < pix_n ? 4u * (uint32_t)(int)(n * g.sv[0] + h * g.sv[2] + w * g.sv[3]) : ~0u;
-    }
-    // steps [s0, s1) of 4 pose rows each belong to this wave; byte offsets of its pose rows
-    const int Q = g.KRED >> 2, steps = (Q + 3) >> 2;
-    const int s0 = (int)((int64_t)steps * wave / NW), s1 = (int)((int64_t)steps * (wave + 1) / NW);
-    const int nsteps = s1 - s0;
-    uint2 *tab = tab_all + wave * tab_entries;
-    for (int i = lane; i < 4 * nsteps + 4 * R; i += 64) {
-        const int q = min(4 * s0 + i, Q - 1);
-        const int c = q / (g.KH * g.KW), r = q - c * (g.KH * g.KW);
-        const int kh = r / g.KW, kw = r - kh * g.KW;
-        tab[i] = uint2{4u * (uint32_t)(c * (int)g.sp[1] + kh * (int)g.sp[2] + kw * (int)g.sp[3]),
-                       4u * (uint32_t)(c * (int)g.sw[1] + kh * (int)g.sw[2] + kw * (int)g.sw[3])};
-    }
-    __syncthreads();
-
-    uint32_t p_lane[MB], w_lane[NB], v_lane[NB];
+    const int Q = g.KRED >> 2;
+    uint32_t p_lane[MBW], w_lane[NB];
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++) p_lane[mb] = pix_p[4 * mb + (li >> 2)] + 4u * (uint32_t)((li & 3) * (int)g.sp[4]);
-    bool col_ok[NB];
+    for (int mb = 0; mb < MBW; mb++)
+        p_lane[mb] = pix_p[4 * (mb0 + mb) + (li >> 2)] + 4u * (uint32_t)((li & 3) * (int)g.sp[4]);
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) {
         const int col = n0 + 16 * nb + li;
-        col_ok[nb] = col < g.COLS;
-        const int co = col_ok[nb] ? col >> 2 : 0;
+        const int co = col < g.COLS ? col >> 2 : 0;
         w_lane[nb] = 4u * (uint32_t)(co * (int)g.sw[0] + (li & 3));
-        v_lane[nb] = 4u * (uint32_t)(co * (int)g.sv[1] + (li & 3));
     }
     const char *p_base = reinterpret_cast<const char *>(g.P);
     const char *w_base[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) w_base[j] = reinterpret_cast<const char *>(g.W + j * g.sw[4]);
 
-    v4f ra[R][MB];
+    v4f ra[R][MBW];
     float rb[R][NB][4];
     const uint2 *tab_lane = tab + lq;
-    uint2 off = tab_lane[0];
+    uint2 off = tab_lane[0];   // offsets of the next set to load; the one after is read meanwhile
     int t_issue = 0;
 #define T2SP_D16_ISSUE(d)                                                                          \
     {                                                                                              \
@@ -392,20 +369,20 @@ __global__ void __launch_bounds__(NW * 64) capsule_direct16_kernel(const Capsule
         _Pragma("unroll") for (int nb = 0; nb < NB; nb++)                                          \
             _Pragma("unroll") for (int j = 0; j < 4; j++)                                          \
                 rb[d][nb][j] = *reinterpret_cast<const float *>(w_base[j] + (w_lane[nb] + ow));    \
-        _Pragma("unroll") for (int mb = 0; mb < MB; mb++)                                          \
+        _Pragma("unroll") for (int mb = 0; mb < MBW; mb++)                                         \
             ra[d][mb] = *reinterpret_cast<const v4f *>(p_base + (p_lane[mb] + op));                \
     }
-    v4f_acc acc[MB][NB];
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) acc[mb][nb] = v4f_acc{0.f, 0.f, 0.f, 0.f};
-
 #pragma unroll
     for (int d = 0; d < R - 1; d++) {
         T2SP_D16_ISSUE(d)
         __builtin_amdgcn_sched_barrier(0);   // keep the sets in program order: waits count loads
     }
+
+    v4f_acc acc[MBW][NB];
+#pragma unroll
+    for (int mb = 0; mb < MBW; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) acc[mb][nb] = v4f_acc{0.f, 0.f, 0.f, 0.f};
     const int main_iters = nsteps > 0 ? (nsteps - 1) / R : 0;
     const int rem = nsteps - main_iters * R;
     for (int it = 0; it < main_iters; it++) {
@@ -415,11 +392,11 @@ __global__ void __launch_bounds__(NW * 64) capsule_direct16_kernel(const Capsule
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
-                for (int mb = 0; mb < MB; mb++)
+                for (int mb = 0; mb < MBW; mb++)
 #pragma unroll
                     for (int nb = 0; nb < NB; nb++)
                         acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[d][mb][j], rb[d][nb][j], acc[mb][nb], 0, 0, 0);
-            T2SP_INTERLEAVE(SG_VMEM_READ, MB + 4 * NB, (4 * NB * MB) / (MB + 4 * NB))
+            T2SP_INTERLEAVE(SG_VMEM_READ, MBW + 4 * NB, (4 * NB * MBW) / (MBW + 4 * NB))
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -432,7 +409,7 @@ __global__ void __launch_bounds__(NW * 64) capsule_direct16_kernel(const Capsule
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
-                for (int mb = 0; mb < MB; mb++) {
+                for (int mb = 0; mb < MBW; mb++) {
                     const float a = live ? ra[d][mb][j] : 0.f;
 #pragma unroll
                     for (int nb = 0; nb < NB; nb++)
@@ -440,27 +417,75 @@ __global__ void __launch_bounds__(NW * 64) capsule_direct16_kernel(const Capsule
                 }
         }
     }
-
-    // sum the partial tiles of the waves in wave order; register r of a lane is vote row mx = r of
-    // pixel 4*mb + l/16 of the tile, column l%16 of the block
-    v4f *mine = red + wave * MB * NB * 64 + lane;
+    // register r of a lane is vote row mx = r of pixel 4*mb + l/16 of the tile, column l%16 of the block
+    v4f *mine = red_kq + mb0 * NB * 64 + lane;
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++)
+    for (int mb = 0; mb < MBW; mb++)
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) mine[(mb * NB + nb) * 64] = acc[mb][nb];
+}
+
+template <int MB, int NB>
+__global__ void __launch_bounds__(D16_WAVES * D16_ROWSPLIT * 64)
+    capsule_direct16_kernel(const CapsuleArgs g, int rows_per_tile, int tab_entries) {
+    static_assert(MB >= D16_ROWSPLIT, "a row block per wave at least");
+    constexpr int NW = D16_WAVES, RS = D16_ROWSPLIT, R = D16_RING;
+    extern __shared__ __align__(16) float smem[];
+    v4f *red = reinterpret_cast<v4f *>(smem);                                   // [kq][mb][nb][lane]
+    uint32_t *pix_p = reinterpret_cast<uint32_t *>(smem + NW * MB * NB * 64 * 4);  // [4*MB] byte offsets in P
+    uint32_t *pix_v = pix_p + 4 * MB;                                            // [4*MB] byte offsets in V, ~0u: none
+    uint2 *tab_all = reinterpret_cast<uint2 *>(pix_v + 4 * MB);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int kq = wave % NW, rh = wave / NW;          // waves w and w + NW run on the same SIMD
+    const int lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
+    const int tm = blockIdx.x % g.tiles_m, tn = blockIdx.x / g.tiles_m;   // the column tiles of one row tile: same XCD
+    const int r0 = tm * rows_per_tile, n0 = tn * 16 * NB;
+
+    // pixels of this tile: offsets of (n, h, w) in P and in V (the last wave's job: it has no table
+    // entries of its own to fill, see below)
+    const int pix_total = g.ROWS >> 2, pix0 = r0 >> 2, pix_n = min(rows_per_tile >> 2, pix_total - pix0);
+    if (wave == NW * RS - 1 && lane < 4 * MB) {
+        const int t = lane;
+        const int pix = pix0 + (t < pix_n ? t : 0);
+        const int w = pix % g.OW, hn = pix / g.OW, h = hn % g.OH, n = hn / g.OH;
+        pix_p[t] = 4u * (uint32_t)(int)(n * g.sp[0] + h * g.S * g.sp[2] + w * g.S * g.sp[3]);
+        pix_v[t] = t < pix_n ? 4u * (uint32_t)(int)(n * g.sv[0] + h * g.sv[2] + w * g.sv[3]) : ~0u;
+    }
+    // steps [s0, s1) of 4 pose rows each belong to share kq; byte offsets of its pose rows, filled
+    // by the first wave of the pair (rows past the end repeat the last one)
+    const int Q = g.KRED >> 2, steps = (Q + 3) >> 2;
+    const int s0 = (int)((int64_t)steps * kq / NW), s1 = (int)((int64_t)steps * (kq + 1) / NW);
+    const int nsteps = s1 - s0;
+    uint2 *tab = tab_all + kq * tab_entries;
+    if (rh == 0)
+        for (int i = lane; i < 4 * nsteps + 4 * R; i += 64) {
+            const int q = min(4 * s0 + i, Q - 1);
+            const int c = q / (g.KH * g.KW), r = q - c * (g.KH * g.KW);
+            const int kh = r / g.KW, kw = r - kh * g.KW;
+            tab[i] = uint2{4u * (uint32_t)(c * (int)g.sp[1] + kh * (int)g.sp[2] + kw * (int)g.sp[3]),
+                           4u * (uint32_t)(c * (int)g.sw[1] + kh * (int)g.sw[2] + kw * (int)g.sw[3])};
+        }
+    __syncthreads();
+    v4f *red_kq = red + kq * MB * NB * 64;
+    // row blocks [0, MB/2) belong to row share 0, the rest to share 1
+    constexpr int CUT = MB / RS;
+    if (rh == 0) direct16_wave<CUT, NB>(g, 0, nsteps, s0, n0, pix_p, tab, red_kq);
+    else direct16_wave<MB - CUT, NB>(g, CUT, nsteps, s0, n0, pix_p, tab, red_kq);
     __syncthreads();
     char *v_base = reinterpret_cast<char *>(g.V);
     const uint32_t mx_stride = 4u * (uint32_t)(int)g.sv[4];
-    for (int pr = wave; pr < NB * MB; pr += NW) {
+    for (int pr = wave; pr < NB * MB; pr += RS * NW) {
         const v4f *src = red + pr * 64 + lane;
         v4f sum = src[0];
 #pragma unroll
         for (int wv = 1; wv < NW; wv++) sum += src[wv * MB * NB * 64];
         const int mb = pr / NB, nb = pr % NB;
         const uint32_t pv = pix_v[4 * mb + lq];
-        if (pv != ~0u && col_ok[nb]) {
+        const int col = n0 + 16 * nb + li;
+        if (pv != ~0u && col < g.COLS) {
+            const uint32_t v_lane = 4u * (uint32_t)((col >> 2) * (int)g.sv[1] + (li & 3));
 #pragma unroll
-            for (int r = 0; r < 4; r++) *reinterpret_cast<float *>(v_base + (pv + v_lane[nb] + r * mx_stride)) = sum[r];
+            for (int r = 0; r < 4; r++) *reinterpret_cast<float *>(v_base + (pv + v_lane + r * mx_stride)) = sum[r];
         }
     }
 }
@@ -588,7 +613,7 @@ static Direct16Plan plan_direct16(int rows, int cols) {
 }
 static int direct16_tab_entries(int kred) {
     const int steps = (kred / 4 + 3) / 4;
-    return 4 * ((steps + D16_WAVES - 1) / D16_WAVES) + 4 * D16_RING + 4;
+    return 4 * ((steps + D16_WAVES - 1) / D16_WAVES) + 4 * D16_RING + 8;
 }
 static size_t direct16_smem_bytes(int mb, int nb, int kred) {
     return (size_t)D16_WAVES * mb * nb * 64 * sizeof(v4f) + 2 * 4 * mb * sizeof(uint32_t) +
@@ -599,11 +624,11 @@ template <int MB, int NB>
 static int launch_direct16_mb(const CapsuleArgs &g, const Direct16Plan &p, hipStream_t stream) {
     const size_t smem = direct16_smem_bytes(MB, NB, g.KRED);
     if (smem > 160 * 1024) return T2SP_ERR_SHAPE;
-    auto kern = capsule_direct16_kernel<MB, NB, D16_WAVES, D16_RING>;
+    auto kern = capsule_direct16_kernel<MB, NB>;
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(D16_WAVES * 64), smem, stream, g, p.rows_per_tile,
-                       direct16_tab_entries(g.KRED));
+    hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(D16_WAVES * D16_ROWSPLIT * 64), smem, stream, g,
+                       p.rows_per_tile, direct16_tab_entries(g.KRED));
     return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
 }
 

@@ -266,61 +266,71 @@ __global__ void __launch_bounds__(NW * 64) sgemm_direct_kernel(const GemmArgs g)
 // MFMA j; accumulator nb holds the columns congruent to nb modulo NB, so a lane loads the NB
 // adjacent floats B[16*step + 4*(l/16) + j][c0 + NB*(l%16) ..] with one load and later stores NB
 // adjacent outputs with one store.
-constexpr int GEMM_D16_WAVES = 4;
-constexpr int GEMM_D16_RING = 3;
+// Two waves per SIMD (the row blocks split between them, as in the capsule kernel of this form) were
+// measured and are slower here: 20.8 against 19.0 us at 1024^3, because both waves load the same B.
+constexpr int GEMM_D16_WAVES = 4;      // shares of the reduction, one wave each
+constexpr int GEMM_D16_RING = 3;       // operand register sets; loads run RING-1 steps ahead
 template <int NB> struct VecOf;
 template <> struct VecOf<2> { typedef float type __attribute__((ext_vector_type(2))); };
 template <> struct VecOf<4> { typedef float type __attribute__((ext_vector_type(4))); };
 
-template <int MB, int NB, int NW, int R>
-__global__ void __launch_bounds__(NW * 64) sgemm_direct16_kernel(const GemmArgs g, int rows_per_tile) {
+// Timeline stamps of this kernel (100 MHz wall clock, one set per wave), compiled in only by
+// `make trace-lib`; python -m t2sp_amd.d16_timeline reads them back.
+#ifdef T2SP_D16_TRACE
+__device__ long long g_d16_trace[4096 * 8 * 8];
+#define T2SP_TRACE_STAMP(i) \
+    if ((threadIdx.x & 63) == 0 && blockIdx.x < 4096) g_d16_trace[(blockIdx.x * 8 + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64();
+#else
+#define T2SP_TRACE_STAMP(i)
+#endif
+// Row blocks [mb0, mb0 + MBW) of the tile over steps [s0, s0 + nsteps) of 16 k, partial result to red_kq.
+template <int MBW, int NB>
+__device__ __forceinline__ void sgemm_d16_wave(const GemmArgs &g, int mb0, int m0, int n0, int s0, int nsteps, int steps,
+                                               v4f *red_kq) {
     typedef typename VecOf<NB>::type vnb;
-    extern __shared__ __align__(16) float smem[];
-    v4f *red = reinterpret_cast<v4f *>(smem);            // [wave][mb][nb][lane]
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    constexpr int R = GEMM_D16_RING;
     const int lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
-    const int tm = blockIdx.x % g.tiles_m, tn = blockIdx.x / g.tiles_m;
-    const int m0 = tm * rows_per_tile, n0 = tn * 16 * NB;
-    const int m_end = min(m0 + rows_per_tile, g.M);
-    const int steps = g.K >> 4;
-    const int s0 = (int)((int64_t)steps * wave / NW), s1 = (int)((int64_t)steps * (wave + 1) / NW);
-    const int nsteps = s1 - s0;
-
-    uint32_t a_off[MB];
+    T2SP_TRACE_STAMP(0)
+    uint32_t a_off[MBW];
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++) {
-        const int row = min(m0 + 16 * mb + li, g.M - 1);
+    for (int mb = 0; mb < MBW; mb++) {
+        const int row = min(m0 + 16 * (mb0 + mb) + li, g.M - 1);
         a_off[mb] = 4u * (uint32_t)(row * (int)g.lda + 4 * lq);
     }
     const int col = n0 + NB * li;
     const bool col_ok = col + NB <= g.N;
-    const uint32_t b_off = 4u * (uint32_t)(4 * lq * (int)g.ldb + (col_ok ? col : 0));
+    // Loads take a scalar base and a 32-bit byte offset per lane (the offsets are below 2^32, see
+    // gemm_d16_ok): a 64-bit address per lane doubles the address traffic of every load, and that
+    // traffic holds up the wave's MFMA issue.  The step's part of the offset is added in 32 bits
+    // inside the loop, which keeps the compiler from hoisting a 64-bit lane address out of it.
+    uint32_t b_off[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) b_off[j] = 4u * (uint32_t)((4 * lq + j) * (int)g.ldb + (col_ok ? col : 0));
     const char *a_base = reinterpret_cast<const char *>(g.A + 16 * s0);
     const char *b_base = reinterpret_cast<const char *>(g.B + (int64_t)16 * s0 * g.ldb);
-    const int64_t b_row = 4 * g.ldb, b_step = 64 * g.ldb;   // bytes per k-row and per step
+    const uint32_t b_step = 64u * (uint32_t)g.ldb;         // bytes per step of 16 k-rows
     int issued = 0;
 
-    v4f ra[R][MB];
+    v4f ra[R][MBW];
     vnb rb[R][4];
 #define T2SP_GEMM_D16_ISSUE(d)                                                                      \
     {                                                                                               \
         const int st = min(issued, steps - 1 - s0);                                                 \
-        const char *ap = a_base + 64 * st;                                                          \
-        const char *bp = b_base + (int64_t)st * b_step;                                             \
+        const uint32_t ao = 64u * (uint32_t)st, bo = (uint32_t)st * b_step;                         \
         issued++;                                                                                   \
         _Pragma("unroll") for (int j = 0; j < 4; j++)                                               \
-            rb[d][j] = *reinterpret_cast<const vnb *>(bp + j * b_row + b_off);                      \
-        _Pragma("unroll") for (int mb = 0; mb < MB; mb++)                                           \
-            ra[d][mb] = *reinterpret_cast<const v4f *>(ap + a_off[mb]);                             \
+            rb[d][j] = *reinterpret_cast<const vnb *>(b_base + (b_off[j] + bo));                    \
+        _Pragma("unroll") for (int mb = 0; mb < MBW; mb++)                                          \
+            ra[d][mb] = *reinterpret_cast<const v4f *>(a_base + (a_off[mb] + ao));                  \
     }
 #define T2SP_GEMM_D16_MMA(d)                                                                        \
     _Pragma("unroll") for (int j = 0; j < 4; j++)                                                   \
-        _Pragma("unroll") for (int mb = 0; mb < MB; mb++)                                           \
+        _Pragma("unroll") for (int mb = 0; mb < MBW; mb++)                                          \
             _Pragma("unroll") for (int nb = 0; nb < NB; nb++)                                       \
                 acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[d][mb][j], rb[d][j][nb], acc[mb][nb], 0, 0, 0);
-    v4f acc[MB][NB];
+    v4f acc[MBW][NB];
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++)
+    for (int mb = 0; mb < MBW; mb++)
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) acc[mb][nb] = v4f{0.f, 0.f, 0.f, 0.f};
 
@@ -331,15 +341,20 @@ __global__ void __launch_bounds__(NW * 64) sgemm_direct16_kernel(const GemmArgs 
     }
     const int main_iters = nsteps > 0 ? (nsteps - 1) / R : 0;
     const int rem = nsteps - main_iters * R;
+    T2SP_TRACE_STAMP(1)
     for (int it = 0; it < main_iters; it++) {
 #pragma unroll
         for (int d = 0; d < R; d++) {
             T2SP_GEMM_D16_ISSUE((d + R - 1) % R)
             T2SP_GEMM_D16_MMA(d)
-            T2SP_INTERLEAVE(SG_VMEM_READ, MB + 4, (4 * MB * NB) / (MB + 4))
+            T2SP_INTERLEAVE(SG_VMEM_READ, MBW + 4, (4 * MBW * NB) / (MBW + 4))
             __builtin_amdgcn_sched_barrier(0);
+#ifdef T2SP_D16_TRACE
+            if (it == 0 && d == 0) { T2SP_TRACE_STAMP(2) }
+#endif
         }
     }
+    T2SP_TRACE_STAMP(3)
     T2SP_GEMM_D16_ISSUE(R - 1)
 #pragma unroll
     for (int d = 0; d < R; d++) {
@@ -347,14 +362,33 @@ __global__ void __launch_bounds__(NW * 64) sgemm_direct16_kernel(const GemmArgs 
     }
 #undef T2SP_GEMM_D16_ISSUE
 #undef T2SP_GEMM_D16_MMA
-
-    // sum the partial tiles of the waves in wave order
-    v4f *mine = red + wave * MB * NB * 64 + lane;
+    T2SP_TRACE_STAMP(4)
+    v4f *mine = red_kq + mb0 * NB * 64 + lane;
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++)
+    for (int mb = 0; mb < MBW; mb++)
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) mine[(mb * NB + nb) * 64] = acc[mb][nb];
+}
+
+template <int MB, int NB>
+__global__ void __launch_bounds__(GEMM_D16_WAVES * 64) sgemm_direct16_kernel(const GemmArgs g, int rows_per_tile) {
+    typedef typename VecOf<NB>::type vnb;
+    constexpr int NW = GEMM_D16_WAVES;
+    extern __shared__ __align__(16) float smem[];
+    v4f *red = reinterpret_cast<v4f *>(smem);            // [wave][mb][nb][lane]
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
+    const int tm = blockIdx.x % g.tiles_m, tn = blockIdx.x / g.tiles_m;
+    const int m0 = tm * rows_per_tile, n0 = tn * 16 * NB;
+    const int m_end = min(m0 + rows_per_tile, g.M);
+    const int steps = g.K >> 4;
+    const int s0 = (int)((int64_t)steps * wave / NW), s1 = (int)((int64_t)steps * (wave + 1) / NW);
+    sgemm_d16_wave<MB, NB>(g, 0, m0, n0, s0, s1 - s0, steps, red + wave * MB * NB * 64);
     __syncthreads();
+    T2SP_TRACE_STAMP(5)
+    // sum the partial tiles of the waves in wave order
+    const int col = n0 + NB * li;
+    const bool col_ok = col + NB <= g.N;
     for (int mb = wave; mb < MB; mb += NW) {
         v4f sum[NB];
 #pragma unroll
@@ -384,7 +418,15 @@ __global__ void __launch_bounds__(NW * 64) sgemm_direct16_kernel(const GemmArgs 
             }
         }
     }
+    T2SP_TRACE_STAMP(6)
 }
+#ifdef T2SP_D16_TRACE
+}  // namespace t2sp
+extern "C" int t2sp_d16_trace(long long *host, int n) {
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(t2sp::g_d16_trace), (size_t)n * 8);
+}
+namespace t2sp {
+#endif
 
 // Fallback for shapes the vector loaders cannot take (K or N not a multiple
 // of 4, or operands not 16-byte aligned): one thread per output, sequential k.
@@ -643,7 +685,7 @@ static int launch_d16_t(GemmArgs g, const GemmD16Plan &p, hipStream_t stream) {
     g.tiles_m = p.tiles_m;
     g.tiles_n = p.tiles_n;
     const size_t smem = (size_t)GEMM_D16_WAVES * MB * NB * 64 * sizeof(v4f);
-    auto kern = sgemm_direct16_kernel<MB, NB, GEMM_D16_WAVES, GEMM_D16_RING>;
+    auto kern = sgemm_direct16_kernel<MB, NB>;
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(GEMM_D16_WAVES * 64), smem, stream, g, p.rows_per_tile);
@@ -677,7 +719,7 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         const double fill256 = (double)g.M * g.N / ((double)t256 * 65536.0);
         const double fill128 = (double)g.M * g.N / ((double)t128 * 16384.0);
         const bool big_tiles = t256 >= 200 && fill256 >= 0.6;
-        const bool tiled_better = t128 >= 200 && g.K >= 2048 && fill128 >= 0.6;
+        const bool tiled_better = t128 >= 500 && g.K >= 2048 && fill128 >= 0.6;   // 2304^3, 2560^3: the 16 x 16 form is 7-11 % ahead
         const bool too_few = (int64_t)p.tiles_m * p.tiles_n < 128 && g.K >= 4096;
         if (!big_tiles && !tiled_better && !too_few && g.K >= 64) return launch_d16(g, stream);
     }
