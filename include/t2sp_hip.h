@@ -221,6 +221,21 @@ int t2sp_mttkrp_f32_noalloc(const float *B, const float *C, const float *D, floa
                             int K, int R, const int64_t *sb3, const int64_t *sc2, const int64_t *sd2,
                             const int64_t *sa2, int cfg, int splits, void *stream);
 
+/* What the launch planners decide, for tests (they plan for t2sp_machine_cus() compute units, see
+ * t2sp_runtime.h; no device is needed).  No counterpart in the reference.
+ *   t2sp_sgemm_plan: number of launches of the LDS-tiled kernels, the tile edge (256 / 128, 0 = the
+ *     product takes another kernel) and (first tile, tiles, splits of the reduction) per launch;
+ *   t2sp_conv2d_plan: number of stages and (T2SP_CFG_*, first pixel, end pixel, splits) per stage
+ *     for CO output channels, P output pixels and a reduction of KRED;
+ *   t2sp_ssyrk_plan: (tiles of the triangle, tiles of the last round that are split, splits) for
+ *     tiles of edge b;
+ *   t2sp_capsule_direct16_plan: (rows per tile, row blocks, column blocks, tiles along rows, tiles
+ *     along columns, rounds of workgroups) of the 16 x 16 direct form for rows x cols votes. */
+int t2sp_sgemm_plan(int M, int N, int K, int *tile_edge, int *phases12);
+int t2sp_conv2d_plan(int CO, int P, int KRED, int *stages16);
+int t2sp_ssyrk_plan(int N, int K, int b, int *total_tail_splits);
+int t2sp_capsule_direct16_plan(int rows, int cols, int *out6);
+
 /* dst[sum_d c_d*dst_strides[d]] = src[sum_d c_d*src_strides[d]] for every coordinate c of the
  * box `extents` (nd <= T2SP_MAX_DIMS, dimension 0 fastest).  Device-side replacement of the
  * host serializer/deserializer loops the reference's generated interface runs around its

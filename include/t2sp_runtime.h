@@ -28,6 +28,15 @@ void t2sp_release(void);
 void *t2sp_host_malloc(size_t bytes);
 void t2sp_host_free(void *p);
 
+/* The machine the launch planners size rounds of workgroups and the die-aware tile order for:
+ * compute units and dies (XCDs) of the current device, asked of it on first use (256 and 8 on a
+ * full MI355X; a partition reports less).  t2sp_set_machine states them instead (cus <= 0: ask the
+ * device again; xcds <= 0: derive from cus).  No counterpart in the reference, whose designs are
+ * sized at synthesis time. */
+int t2sp_machine_cus(void);
+int t2sp_machine_xcds(void);
+void t2sp_set_machine(int cus, int xcds);
+
 /* Number of HIP devices visible; 0 when there is none. */
 int t2sp_device_count(void);
 

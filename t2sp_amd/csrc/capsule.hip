@@ -14,6 +14,7 @@
 #include "mfma_core.hpp"
 #include "splitk.hpp"
 #include "t2sp_hip.h"
+#include "machine.hpp"
 
 namespace t2sp {
 
@@ -543,11 +544,12 @@ static CapsulePlan plan_capsule(int rows, int cols, int kred, int cfg, int split
         // reduction has to be split over workgroups to fill the chip; between one and one and a half
         // rounds of 256 tiles the second round is mostly empty; very large batches reuse operands
         // better through the shared LDS tiles.
-        const bool rounds_ok = t32 <= 256 || t32 >= 384;
+        const int cus = machine().cus;
+        const bool rounds_ok = t32 <= cus || t32 >= cus + cus / 2;
         // With 4-row poses the 16 x 16 form spreads any batch up to a few hundred evenly over the
         // CUs and was the fastest kernel at every batch from 8 to 256 (13-131 us against 19-152 us).
         if (mx == 4 && t32 <= DIRECT_MAX_TILES && kred <= DIRECT_MAX_KRED) cfg = T2SP_CFG_DIRECT16;
-        else if (t32 >= 100 && t32 <= DIRECT_MAX_TILES && rounds_ok && kred <= DIRECT_MAX_KRED) cfg = T2SP_CFG_DIRECT;
+        else if (t32 >= cus * 25 / 64 && t32 <= DIRECT_MAX_TILES && rounds_ok && kred <= DIRECT_MAX_KRED) cfg = T2SP_CFG_DIRECT;
     }
     if (cfg == T2SP_CFG_DIRECT || cfg == T2SP_CFG_DIRECT16) {
         p.cfg = cfg; p.splits = 1;
@@ -558,15 +560,16 @@ static CapsulePlan plan_capsule(int rows, int cols, int kred, int cfg, int split
     if (cfg == T2SP_CFG_AUTO) {
         const int64_t t128 = (int64_t)((rows + 127) / 128) * ((cols + 127) / 128);
         const int64_t t256 = (int64_t)((rows + 255) / 256) * ((cols + 255) / 256);
-        cfg = (t256 >= 200 && cols > 128) ? T2SP_CFG_256x256 : (t128 >= 24 ? T2SP_CFG_128x128 : T2SP_CFG_64x128);
+        cfg = (t256 >= machine().cus * 25 / 32 && cols > 128) ? T2SP_CFG_256x256 : (t128 >= 24 ? T2SP_CFG_128x128 : T2SP_CFG_64x128);
     }
     const int bm = cfg == T2SP_CFG_256x256 ? 256 : cfg == T2SP_CFG_128x128 ? 128 : cfg == T2SP_CFG_64x128 ? 64 : 32;
     const int bn = cfg == T2SP_CFG_256x256 ? 256 : 128;
     const int tiles = ((rows + bm - 1) / bm) * ((cols + bn - 1) / bn);
     const int ktiles = (kred + 15) / 16;
     if (splits <= 0) {
-        // fill the 256 CUs about once, keep at least 8 k-tiles per split
-        splits = tiles >= 200 ? 1 : (256 + tiles / 2) / tiles;
+        // fill the CUs about once, keep at least 8 k-tiles per split
+        const int cus = machine().cus;
+        splits = tiles >= cus * 25 / 32 ? 1 : (cus + tiles / 2) / tiles;
         if (splits > ktiles / 8) splits = ktiles / 8;
         if (splits < 1) splits = 1;
     }
@@ -589,8 +592,9 @@ static Direct16Plan plan_direct16_for(int rows, int cols, int nb, int max_mb) {
     Direct16Plan p{};
     p.nb = nb;
     p.tiles_n = (cols + 16 * nb - 1) / (16 * nb);
+    const int cus = machine().cus;
     for (int rounds = 1;; rounds++) {
-        const int want_m = (rounds * 256) / p.tiles_n > 0 ? (rounds * 256) / p.tiles_n : 1;
+        const int want_m = (rounds * cus) / p.tiles_n > 0 ? (rounds * cus) / p.tiles_n : 1;
         int rpt = ((rows + want_m - 1) / want_m + 3) / 4 * 4;
         if (rpt < 64) rpt = 64;
         if (rpt <= 16 * max_mb) {
@@ -722,6 +726,16 @@ static bool capsule_fast(const int *d, const int64_t *sp6, const int64_t *sw6, c
     for (int i = 0; i < 5; i++)
         if (sp6[i] % 4 || sw6[i] % 4 || sv6[i] % 4) return false;
     return ((uintptr_t)P % 16 == 0) && ((uintptr_t)W % 16 == 0) && ((uintptr_t)V % 16 == 0);
+}
+
+// The tile of the 16 x 16 direct form for rows x cols votes on the current machine(): rows per
+// tile, row blocks, column blocks, tiles along rows and columns, rounds of workgroups.  For tests
+// of the planner.
+extern "C" int t2sp_capsule_direct16_plan(int rows, int cols, int *out6) {
+    if (rows <= 0 || cols <= 0 || !out6) return 0;
+    const t2sp::Direct16Plan p = t2sp::plan_direct16(rows, cols);
+    out6[0] = p.rows_per_tile; out6[1] = p.mb; out6[2] = p.nb; out6[3] = p.tiles_m; out6[4] = p.tiles_n; out6[5] = p.rounds;
+    return 1;
 }
 
 extern "C" size_t t2sp_capsule_workspace_bytes(const int *dims11, int cfg, int splits) {

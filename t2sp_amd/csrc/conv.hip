@@ -18,6 +18,7 @@
 #include "gemm_loaders.hpp"
 #include "splitk.hpp"
 #include "t2sp_hip.h"
+#include "machine.hpp"
 
 namespace t2sp {
 
@@ -33,6 +34,7 @@ struct ConvArgs {
     int OWp;                    // OW rounded up to a multiple of 4: positions per row in the pixel index
     int P, KRED;                // N*OH*OWp, CI*KH*KW
     int tiles_m, tiles_n, group_m;
+    int nxcd;                   // dies the workgroup ids are dealt to (tile order)
     int p_begin;                // first output pixel this launch covers
     int splits;                 // workgroups per tile along the reduction (1 = none)
     int Mp, Np;                 // padded extents of one partial plane (CO, pixels of this launch)
@@ -126,7 +128,7 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) conv_kernel(const ConvArgs g) {
     __syncthreads();
     const int tile = blockIdx.x / g.splits, split = blockIdx.x - tile * g.splits;
     int tm, tn;
-    tile_coords(tile, g.tiles_m, g.tiles_n, g.group_m, tm, tn);
+    tile_coords(tile, g.tiles_m, g.tiles_n, g.group_m, g.nxcd, tm, tn);
     const int co0 = tm * Cfg::BM, p0 = g.p_begin + tn * Cfg::BN;
     int kt0 = 0, kt1 = ktiles_even<Cfg>(g.KRED);
     if (g.splits > 1) split_range((g.KRED + Cfg::BK - 1) / Cfg::BK, g.splits, split, kt0, kt1);
@@ -181,6 +183,7 @@ static int launch_conv(ConvArgs g, int p_begin, int p_end, int splits, float *sc
     g.p_begin = p_begin;
     g.tiles_m = (g.CO + Cfg::BM - 1) / Cfg::BM;
     g.tiles_n = (p_end - p_begin + Cfg::BN - 1) / Cfg::BN;
+    g.nxcd = machine().xcds;
     g.group_m = g.tiles_m;   // all output channels of a pixel tile run together: the input tile is shared in L2
     g.splits = splits;
     g.Mp = g.tiles_m * Cfg::BM;
@@ -219,7 +222,7 @@ struct ConvPlan {
     size_t scratch_bytes;
 };
 static ConvPlan plan_conv(int CO, int P, int KRED) {
-    constexpr int CUS = 256;
+    const int CUS = machine().cus;
     struct Cand { int cfg, bm, bn; double eff; };
     const Cand all[3] = {{T2SP_CFG_256x256, 256, 256, 1.0}, {T2SP_CFG_128x128, 128, 128, 0.94}, {T2SP_CFG_64x128, 64, 128, 0.8}};
     auto tiles_m = [&](const Cand &c) { return (CO + c.bm - 1) / c.bm; };
@@ -255,7 +258,7 @@ static ConvPlan plan_conv(int CO, int P, int KRED) {
         if (smax > 16) smax = 16;
         if (smax < 1) smax = 1;
         for (int sp = 1; sp <= smax; sp++) {
-            const double wg = 2.0 * c.bm * c.bn * KRED / (614e9 * c.eff) / sp;     // one workgroup's MFMA time
+            const double wg = 2.0 * c.bm * c.bn * KRED / (614e9 * c.eff) / sp;     // one workgroup's MFMA time (256 flop/clk at 2.4 GHz)
             const double rounds = (double)((t * sp + CUS - 1) / CUS);
             const double planes = sp > 1 ? (double)t * sp * c.bm * c.bn * 8.0 / 3e12 + 8e-6 : 0.0;
             const double time = wg * rounds + planes;
@@ -292,6 +295,19 @@ static size_t conv_padded_weight_bytes(int CO, int kred) {
 }
 
 }  // namespace t2sp
+
+// The launch plan of the implicit-GEMM kernels on the current machine(): stages over ranges of output
+// pixels as (tile configuration, first pixel, end pixel, splits of the reduction) quadruples; P is
+// the number of output pixels N*OH*round_up4(OW).  For tests of the planner.
+extern "C" int t2sp_conv2d_plan(int CO, int P, int KRED, int *stages16) {
+    if (CO <= 0 || P <= 0 || KRED <= 0 || !stages16) return 0;
+    const t2sp::ConvPlan p = t2sp::plan_conv(CO, P, KRED);
+    for (int i = 0; i < p.n; i++) {
+        stages16[4 * i] = p.st[i].cfg; stages16[4 * i + 1] = p.st[i].p_begin;
+        stages16[4 * i + 2] = p.st[i].p_end; stages16[4 * i + 3] = p.st[i].splits;
+    }
+    return p.n;
+}
 
 extern "C" size_t t2sp_conv2d_workspace_bytes(int N, int CI, int CO, int OH, int OW, int KH, int KW) {
     if (N <= 0 || CI <= 0 || CO <= 0 || OH <= 0 || OW <= 0 || KH <= 0 || KW <= 0) return 0;

@@ -10,6 +10,7 @@
 #include "gemm_loaders.hpp"
 #include "splitk.hpp"
 #include "t2sp_hip.h"
+#include "machine.hpp"
 
 namespace t2sp {
 
@@ -24,6 +25,7 @@ struct GemmArgs {
     int tiled, t_jjj, t_iii, t_jj, t_ii;
     int64_t s[6];
     int tiles_m, tiles_n, group_m;
+    int nxcd;                 // dies the workgroup ids are dealt to (tile order)
     // C = alpha * A*B + beta * Cin (Cin read through ldcin); scale == 0 means plain C = A*B
     int scale;
     float alpha, beta;
@@ -102,7 +104,7 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) sgemm_kernel(const GemmArgs g) 
     const int tile = blockIdx.x / g.splits, split = blockIdx.x - tile * g.splits;
     int tm, tn;
     // the workgroups of a split tile read different slices of k: no run per XCD to arrange
-    tile_of_position(g.tile_first + (g.compact ? tile : xcd_contiguous(tile, g.tile_count)), g.tiles_m, g.tiles_n,
+    tile_of_position(g.tile_first + (g.compact ? tile : xcd_contiguous(tile, g.tile_count, g.nxcd)), g.tiles_m, g.tiles_n,
                      g.group_m, tm, tn);
     const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
     int kt0 = 0, kt1 = ktiles_even<Cfg>(g.K);
@@ -493,10 +495,10 @@ struct GemmPhases {
     size_t scratch_bytes;     // the largest group's planes
     double rounds;            // estimated duration in rounds of one unsplit tile
 };
-constexpr int GEMM_CUS = 256;
 constexpr double GEMM_SPLIT_OVERHEAD = 0.03;   // prologue, plane traffic and extra launches, in rounds of a K = 8192 tile
 
 static GemmPhases plan_phases(int64_t tiles, int K, int bk, int bm, int bn, bool allow_split) {
+    const int GEMM_CUS = machine().cus;      // a tile occupies a CU: rounds of this many
     GemmPhases p{};
     const int pairs = (K + 2 * bk - 1) / (2 * bk);
     int64_t first = 0, rest = tiles;
@@ -542,6 +544,7 @@ static int launch(GemmArgs g, hipStream_t stream, int splits = 1, float *scratch
     g.scratch = scratch;
     // bands of about sqrt(32) tile-rows keep a XCD's resident tiles near-square
     g.group_m = g.tiles_m >= 4 ? 4 : g.tiles_m;
+    g.nxcd = machine().xcds;
     const bool edge = (g.M % Cfg::BM) || (g.N % Cfg::BN) || (g.K % (2 * Cfg::BK));
     const size_t smem = Cfg::SMEM_FLOATS * sizeof(float);
     auto kern = edge ? sgemm_kernel<Cfg, true, BT> : sgemm_kernel<Cfg, false, BT>;
@@ -600,13 +603,14 @@ struct GemmPlan {
 static GemmPlan plan_gemm(int M, int N, int K) {
     auto tiles = [&](int bm, int bn) { return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
     GemmPlan p{T2SP_CFG_64x128, 1, false, 0};
-    if (tiles(256, 256) >= 200 || tiles(128, 128) >= 200) {
+    const int cus = machine().cus, nearly_full = cus * 25 / 32;   // 200 of 256: enough tiles to be worth whole rounds
+    if (tiles(256, 256) >= nearly_full || tiles(128, 128) >= nearly_full) {
         // estimated time = rounds x tile area / the fraction of the 256 x 256 tile's rate that the
         // tile size sustains (measured: 0.94 for 128 x 128)
         const GemmPhases l = plan_phases(tiles(256, 256), K, 16, 256, 256, true);
         const GemmPhases m = plan_phases(tiles(128, 128), K, 16, 128, 128, true);
         const double cl = l.rounds * 65536.0, cm = m.rounds * 16384.0 / 0.94;
-        const bool large = tiles(256, 256) >= 200 && cl <= cm;
+        const bool large = tiles(256, 256) >= nearly_full && cl <= cm;
         p.cfg = large ? T2SP_CFG_256x256 : T2SP_CFG_128x128;
         p.phased = true;
         p.scratch_bytes = large ? l.scratch_bytes : m.scratch_bytes;
@@ -615,7 +619,7 @@ static GemmPlan plan_gemm(int M, int N, int K) {
         p.cfg = bm == 128 ? T2SP_CFG_128x128 : T2SP_CFG_64x128;
         const int64_t t = tiles(bm, 128);
         const int pairs = ((K + 15) / 16 + 1) / 2;
-        int s = (int)((256 + t / 2) / t);
+        int s = (int)((cus + t / 2) / t);
         if (s > pairs / 4) s = pairs / 4;
         if (s > 16) s = 16;
         if (s > 1) {
@@ -633,7 +637,8 @@ static bool gemm_direct_ok(const GemmArgs &g, bool forced) {
     const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
     const int64_t t64 = (int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64);
     // below ~160 tiles of 64 x 64 the split over workgroups fills the chip better
-    if (!forced && (t128 >= 200 || t64 < 160 || g.K < 256)) return false;
+    const int cus = machine().cus;
+    if (!forced && (t128 >= cus * 25 / 32 || t64 < cus * 5 / 8 || g.K < 256)) return false;
     return g.K % 8 == 0 && g.N % 2 == 0 && g.ldb % 2 == 0 && g.ldc % 2 == 0 && ((uintptr_t)g.B % 8 == 0) &&
            ((uintptr_t)g.C % 8 == 0) && (int64_t)g.M * g.lda < (1 << 30) && (int64_t)g.K * g.ldb < (1 << 30) &&
            t64 < (1 << 30);
@@ -658,6 +663,7 @@ struct GemmD16Plan {
     double cost;
 };
 static GemmD16Plan plan_gemm_d16(int M, int N) {
+    const int cus = machine().cus;
     GemmD16Plan best{};
     best.cost = 1e300;
     for (int nb = 2; nb <= 4; nb += 2)
@@ -667,7 +673,7 @@ static GemmD16Plan plan_gemm_d16(int M, int N) {
             const int rpt = (M + tiles_m - 1) / tiles_m;
             const int64_t tiles = (int64_t)tiles_m * tiles_n;
             const double loads_per_mfma = (double)(mb + 4) / (4.0 * mb * nb);
-            const double cost = (double)((tiles + 255) / 256) * (16.0 * mb) * (16.0 * nb) * (1.0 + 1.5 * loads_per_mfma);
+            const double cost = (double)((tiles + cus - 1) / cus) * (16.0 * mb) * (16.0 * nb) * (1.0 + 1.5 * loads_per_mfma);
             if (cost < best.cost) best = GemmD16Plan{mb, nb, rpt, tiles_m, tiles_n, cost};
         }
     return best;
@@ -718,9 +724,10 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         // how much of the large tiles would hold outputs (a thin matrix leaves them mostly empty)
         const double fill256 = (double)g.M * g.N / ((double)t256 * 65536.0);
         const double fill128 = (double)g.M * g.N / ((double)t128 * 16384.0);
-        const bool big_tiles = t256 >= 200 && fill256 >= 0.6;
-        const bool tiled_better = t128 >= 500 && g.K >= 2048 && fill128 >= 0.6;   // 2304^3, 2560^3: the 16 x 16 form is 7-11 % ahead
-        const bool too_few = (int64_t)p.tiles_m * p.tiles_n < 128 && g.K >= 4096;
+        const int cus = machine().cus;
+        const bool big_tiles = t256 >= cus * 25 / 32 && fill256 >= 0.6;
+        const bool tiled_better = t128 >= 2 * cus - cus / 16 && g.K >= 2048 && fill128 >= 0.6;   // 2304^3, 2560^3: the 16 x 16 form is 7-11 % ahead
+        const bool too_few = (int64_t)p.tiles_m * p.tiles_n < cus / 2 && g.K >= 4096;
         if (!big_tiles && !tiled_better && !too_few && g.K >= 64) return launch_d16(g, stream);
     }
     if ((cfg == T2SP_CFG_AUTO || cfg == T2SP_CFG_DIRECT) && !bt && !g.scale && !g.tiled &&
@@ -773,8 +780,9 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         if (p.phased && !phased) {
             const int64_t t256 = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
             const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
-            const double cl = (double)((t256 + 255) / 256) * 65536.0, cm = (double)((t128 + 255) / 256) * 16384.0 / 0.94;
-            cfg = (t256 >= 200 && cl <= cm) ? T2SP_CFG_256x256 : T2SP_CFG_128x128;
+            const int cus = machine().cus;
+            const double cl = (double)((t256 + cus - 1) / cus) * 65536.0, cm = (double)((t128 + cus - 1) / cus) * 16384.0 / 0.94;
+            cfg = (t256 >= cus * 25 / 32 && cl <= cm) ? T2SP_CFG_256x256 : T2SP_CFG_128x128;
         }
     }
     if (bt) {
@@ -796,6 +804,24 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
 }
 
 }  // namespace t2sp
+
+// The launch plan of the LDS-tiled kernels for an M x N x K product on the current machine(): tile
+// edge (256 or 128; 0 when the product would not take whole rounds of these tiles) and the launches
+// as (first tile, tiles, splits of the reduction) triples.  For tests of the planner.
+extern "C" int t2sp_sgemm_plan(int M, int N, int K, int *tile_edge, int *phases12) {
+    if (M <= 0 || N <= 0 || K <= 0 || !tile_edge || !phases12) return 0;
+    const t2sp::GemmPlan p = t2sp::plan_gemm(M, N, K);
+    *tile_edge = 0;
+    if (!p.phased) return 0;
+    const int b = p.cfg == T2SP_CFG_256x256 ? 256 : 128;
+    *tile_edge = b;
+    const int64_t tiles = (int64_t)((M + b - 1) / b) * ((N + b - 1) / b);
+    const t2sp::GemmPhases ph = t2sp::plan_phases(tiles, K, 16, b, b, true);
+    for (int i = 0; i < ph.n; i++) {
+        phases12[3 * i] = ph.ph[i].first; phases12[3 * i + 1] = ph.ph[i].count; phases12[3 * i + 2] = ph.ph[i].splits;
+    }
+    return ph.n;
+}
 
 extern "C" size_t t2sp_sgemm_workspace_bytes(int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;

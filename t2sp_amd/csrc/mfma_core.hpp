@@ -358,19 +358,18 @@ __device__ __forceinline__ void tile_of_position(int pid, int tiles_m, int tiles
     tn = in_band / rows;
 }
 
-// Workgroup ids are dealt round-robin to the 8 XCDs (each with its own L2), so consecutive ids
-// land on different L2s.  This remap gives every XCD one contiguous run of the `count` positions
-// a launch covers, so that the ~32 workgroups resident on one XCD are neighbours in the walking
-// order and share panels in that XCD's L2.
-__device__ __forceinline__ int xcd_contiguous(int bid, int count) {
-    constexpr int NXCD = 8;
-    return count % NXCD == 0 ? (bid % NXCD) * (count / NXCD) + bid / NXCD : bid;
+// Workgroup ids are dealt round-robin to the `nxcd` XCDs (each with its own L2), so consecutive
+// ids land on different L2s.  This remap gives every XCD one contiguous run of the `count`
+// positions a launch covers, so that the ~32 workgroups resident on one XCD are neighbours in the
+// walking order and share panels in that XCD's L2.
+__device__ __forceinline__ int xcd_contiguous(int bid, int count, int nxcd) {
+    return (nxcd > 1 && count % nxcd == 0) ? (bid % nxcd) * (count / nxcd) + bid / nxcd : bid;
 }
 
 // Workgroup id -> tile coordinates for a launch over all tiles.
-__device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, int group_m,
+__device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, int group_m, int nxcd,
                                             int &tm, int &tn) {
-    tile_of_position(xcd_contiguous(bid, tiles_m * tiles_n), tiles_m, tiles_n, group_m, tm, tn);
+    tile_of_position(xcd_contiguous(bid, tiles_m * tiles_n, nxcd), tiles_m, tiles_n, group_m, tm, tn);
 }
 
 }  // namespace t2sp

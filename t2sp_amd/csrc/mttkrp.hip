@@ -16,6 +16,7 @@
 #include "mfma_core.hpp"
 #include "splitk.hpp"
 #include "t2sp_hip.h"
+#include "machine.hpp"
 
 #include <stdio.h>
 
@@ -235,7 +236,8 @@ static MttkrpPlan plan_mttkrp(int I, int J, int K, int R, int cfg, int splits) {
     const int tiles = ((I + bm - 1) / bm) * ((R + bn - 1) / bn);
     const int64_t ktiles = (int64_t)K * (J / 16);
     if (splits <= 0) {
-        splits = tiles >= 200 ? 1 : (256 + tiles / 2) / tiles;
+        const int cus = machine().cus;
+        splits = tiles >= cus * 25 / 32 ? 1 : (cus + tiles / 2) / tiles;
         if (splits > ktiles / 16) splits = (int)(ktiles / 16);
         if (splits < 1) splits = 1;
     }

@@ -1,5 +1,6 @@
 // runtime.cpp — see runtime.hpp.
 #include "runtime.hpp"
+#include "machine.hpp"
 
 #include <atomic>
 #include <stdlib.h>
@@ -235,6 +236,42 @@ void publish_kernel_ns(double ns, const char *op) {
 }
 
 }  // namespace t2sp
+
+namespace t2sp {
+static std::atomic<int> g_machine_cus{0}, g_machine_xcds{0};
+
+int xcds_for(int cus) {
+    for (int x = 8; x > 1; x /= 2)
+        if (cus % x == 0 && cus / x >= 20 && cus / x <= 40) return x;
+    return 1;
+}
+
+Machine machine() {
+    int cus = g_machine_cus.load(), xcds = g_machine_xcds.load();
+    if (cus <= 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) {
+            cus = prop.multiProcessorCount;
+        } else {
+            (void)hipGetLastError();
+            cus = 256;                     // no device: plan for a full MI355X
+        }
+        xcds = xcds_for(cus);
+        g_machine_cus = cus;
+        g_machine_xcds = xcds;
+    }
+    return Machine{cus, xcds > 0 ? xcds : xcds_for(cus)};
+}
+}  // namespace t2sp
+
+extern "C" void t2sp_set_machine(int cus, int xcds) {
+    t2sp::g_machine_cus = cus > 0 ? cus : 0;
+    t2sp::g_machine_xcds = cus > 0 ? (xcds > 0 ? xcds : t2sp::xcds_for(cus)) : 0;
+}
+
+extern "C" int t2sp_machine_cus(void) { return t2sp::machine().cus; }
+extern "C" int t2sp_machine_xcds(void) { return t2sp::machine().xcds; }
 
 extern "C" double t2sp_last_kernel_ns(void) {
     return t2sp::tl_last_kernel_ns >= 0.0 ? t2sp::tl_last_kernel_ns : t2sp::g_last_kernel_ns.load();

@@ -18,6 +18,7 @@
 #include "gemm_loaders.hpp"
 #include "splitk.hpp"
 #include "t2sp_hip.h"
+#include "machine.hpp"
 
 namespace t2sp {
 
@@ -50,6 +51,7 @@ struct SyrkArgs {
     // own plane of `scratch` (plane = tile_count tiles side by side, [tile][col][row])
     int tile_first, tile_count, splits;
     float *scratch;
+    int nxcd;             // dies the workgroup ids are dealt to (tile order)
 };
 
 // MODE FLAT_SYM reads Cin from the `upper` triangle only; the other modes where C is written.
@@ -130,13 +132,10 @@ __device__ __forceinline__ void syrk_tile_of(int pid, int T, int &tm, int &tn) {
 }
 
 // Workgroup id of a launch over `count` positions starting at `first`.  Ids are dealt round-robin
-// to the 8 XCDs, so each XCD is first given one contiguous run of the order: the workgroups
+// to the XCDs, so each XCD is first given one contiguous run of the order: the workgroups
 // resident on one XCD at a time then share a few panels of A in its L2.
-__device__ __forceinline__ void syrk_tile(int bid, int first, int count, int T, int &tm, int &tn) {
-    constexpr int NXCD = 8;
-    int pid = bid;
-    if (count % NXCD == 0) pid = (bid % NXCD) * (count / NXCD) + bid / NXCD;
-    syrk_tile_of(first + pid, T, tm, tn);
+__device__ __forceinline__ void syrk_tile(int bid, int first, int count, int T, int nxcd, int &tm, int &tn) {
+    syrk_tile_of(first + xcd_contiguous(bid, count, nxcd), T, tm, tn);
 }
 
 template <class Cfg, bool EDGE, int MODE>
@@ -144,7 +143,7 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) ssyrk_kernel(const SyrkArgs g) 
     static_assert(Cfg::BM == Cfg::BN && Cfg::BSTYLE == STYLE_KC, "square KC/KC tiles");
     extern __shared__ __align__(16) float smem[];
     int tm, tn;
-    syrk_tile(blockIdx.x, g.tile_first, g.tile_count, g.tiles, tm, tn);
+    syrk_tile(blockIdx.x, g.tile_first, g.tile_count, g.tiles, g.nxcd, tm, tn);
     const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
     RowMajorKcLoader<Cfg, EDGE> la(g.A, g.lda, m0, g.N, g.K);
     RowMajorKcLoaderB<Cfg, EDGE> lb(g.A, g.lda, n0, g.N, g.K);
@@ -294,12 +293,13 @@ __global__ void __launch_bounds__(NW * 64) ssyrk_direct16_kernel(const SyrkArgs 
     v4f ra[R][MB], rb[R][NB];
 #define T2SP_SYRK_D16_ISSUE(d)                                                                      \
     {                                                                                               \
-        const char *ap = a_base + 64 * min(issued, steps - 1 - s0);                                 \
+        /* scalar base + 32-bit lane offset, the step added in 32 bits: see sgemm_d16_wave */      \
+        const uint32_t ao = 64u * (uint32_t)min(issued, steps - 1 - s0);                            \
         issued++;                                                                                   \
         _Pragma("unroll") for (int nb = 0; nb < NB; nb++)                                           \
-            rb[d][nb] = *reinterpret_cast<const v4f *>(ap + b_off[nb]);                             \
+            rb[d][nb] = *reinterpret_cast<const v4f *>(a_base + (b_off[nb] + ao));                  \
         _Pragma("unroll") for (int mb = 0; mb < MB; mb++)                                           \
-            ra[d][mb] = *reinterpret_cast<const v4f *>(ap + a_off[mb]);                             \
+            ra[d][mb] = *reinterpret_cast<const v4f *>(a_base + (a_off[mb] + ao));                  \
     }
 #define T2SP_SYRK_D16_MMA(d)                                                                        \
     _Pragma("unroll") for (int j = 0; j < 4; j++)                                                   \
@@ -365,6 +365,7 @@ struct SyrkD16Plan {
     int64_t needed;
 };
 static SyrkD16Plan plan_syrk_d16(int N) {
+    const int cus = machine().cus;
     SyrkD16Plan best{};
     best.cost = 1e300;
     for (int nb = 2; nb <= 4; nb++)
@@ -379,7 +380,7 @@ static SyrkD16Plan plan_syrk_d16(int N) {
             }
             const double loads_per_mfma = (double)(mb + nb) / (4.0 * mb * nb);
             // + a fixed cost per round (prologue, exchange, store) worth about 1500 outputs of work
-            const double cost = (double)((needed + 255) / 256) * ((16.0 * mb) * (16.0 * nb) * (1.0 + 1.5 * loads_per_mfma) + 1500.0);
+            const double cost = (double)((needed + cus - 1) / cus) * ((16.0 * mb) * (16.0 * nb) * (1.0 + 1.5 * loads_per_mfma) + 1500.0);
             if (cost < best.cost) best = SyrkD16Plan{mb, nb, rpt, tiles_m, tiles_n, cost, needed};
         }
     return best;
@@ -433,7 +434,7 @@ using SyrkL = TileCfg<256, 256, 16, 4, 2, STYLE_KC>;
 using SyrkM = TileCfg<128, 128, 16, 2, 2, STYLE_KC>;
 using SyrkS = TileCfg<64, 64, 16, 2, 1, STYLE_KC>;
 
-// How the last, partial round of 256 tiles is split: `tail` tiles, each over `splits` workgroups.
+// How the last, partial round of tiles (one per CU) is split: `tail` tiles, each over `splits` workgroups.
 struct SyrkTail {
     int64_t total, tail;
     int splits;
@@ -441,13 +442,14 @@ struct SyrkTail {
 };
 static SyrkTail plan_syrk_tail(int N, int K, int b, int bk) {
     SyrkTail t{};
+    const int cus = machine().cus;
     const int64_t side = (N + b - 1) / b;
     t.total = side * (side + 1) / 2;
-    t.tail = t.total % 256;
+    t.tail = t.total % cus;
     t.splits = 1;
-    if (t.total > 256 && t.tail > 0 && t.tail <= 128) {
+    if (t.total > cus && t.tail > 0 && t.tail <= cus / 2) {
         const int pairs = (K + 2 * bk - 1) / (2 * bk);
-        int s = (int)(256 / t.tail);
+        int s = (int)(cus / t.tail);
         if (s > pairs / 8) s = pairs / 8;          // at least 8 pairs of k-tiles per workgroup
         if (s > 32) s = 32;
         if (s >= 2) t.splits = s;
@@ -460,6 +462,7 @@ static SyrkTail plan_syrk_tail(int N, int K, int b, int bk) {
 template <class Cfg>
 static int launch_syrk(SyrkArgs g, hipStream_t stream, float *scratch = nullptr, size_t scratch_bytes = 0) {
     g.tiles = (g.N + Cfg::BM - 1) / Cfg::BM;
+    g.nxcd = machine().xcds;
     const bool edge = (g.N % Cfg::BM) || (g.K % (2 * Cfg::BK));
     const size_t smem = Cfg::SMEM_FLOATS * sizeof(float);
     void (*kern)(const SyrkArgs);
@@ -553,8 +556,9 @@ static int dispatch_syrk(SyrkArgs g, int trans, int cfg, float *workspace, size_
         auto cost = [&](int b, double eff) {
             const SyrkTail t = plan_syrk_tail(g.N, g.K, b, 16);
             const bool split = t.tail > 0 && workspace && workspace_bytes >= t.scratch_bytes;
-            const double rounds = split ? (double)((t.total - t.tail) / 256) + 1.0 / t.splits + 0.03
-                                        : (double)((t.total + 255) / 256);
+            const int cus = machine().cus;
+            const double rounds = split ? (double)((t.total - t.tail) / cus) + 1.0 / t.splits + 0.03
+                                        : (double)((t.total + cus - 1) / cus);
             return rounds * b * b / eff;
         };
         const double c256 = cost(256, 1.0), c128 = cost(128, 0.93), c64 = cost(64, 0.78);
@@ -590,6 +594,15 @@ __global__ void __launch_bounds__(256) syrk_fold_kernel(const float *flat, float
 }
 
 }  // namespace t2sp
+
+// How SYRK with tiles of edge b splits its last, partial round on the current machine(): tiles of
+// the triangle, tiles of the tail that is split, splits per tail tile.  For tests of the planner.
+extern "C" int t2sp_ssyrk_plan(int N, int K, int b, int *total_tail_splits) {
+    if (N <= 0 || K <= 0 || b <= 0 || !total_tail_splits) return 0;
+    const t2sp::SyrkTail t = t2sp::plan_syrk_tail(N, K, b, 16);
+    total_tail_splits[0] = (int)t.total; total_tail_splits[1] = (int)t.tail; total_tail_splits[2] = t.splits;
+    return 1;
+}
 
 extern "C" size_t t2sp_ssyrk_workspace_bytes(int trans, int N, int K) {
     if (N <= 0 || K <= 0) return 0;

@@ -1,0 +1,107 @@
+"""CPU checks of the launch planners: they size rounds of workgroups by the number of compute units
+the machine reports (a full MI355X has 256 in 8 dies; its partitions and other parts of the family
+have 64, 128, 304, ...), not by a constant.  The planners run on the host, so no device is needed:
+`t2sp_set_machine` states the machine and the `*_plan` calls of include/t2sp_hip.h return what would
+be launched."""
+import ctypes
+
+import pytest
+
+import t2sp_amd
+
+CUS = [64, 128, 256, 304]
+
+
+@pytest.fixture
+def lib():
+    L = t2sp_amd.lib()
+    i32p = ctypes.POINTER(ctypes.c_int)
+    L.t2sp_set_machine.argtypes = [ctypes.c_int, ctypes.c_int]
+    L.t2sp_set_machine.restype = None
+    L.t2sp_sgemm_plan.argtypes = [ctypes.c_int] * 3 + [i32p, i32p]
+    L.t2sp_conv2d_plan.argtypes = [ctypes.c_int] * 3 + [i32p]
+    L.t2sp_ssyrk_plan.argtypes = [ctypes.c_int] * 3 + [i32p]
+    L.t2sp_capsule_direct16_plan.argtypes = [ctypes.c_int] * 2 + [i32p]
+    yield L
+    L.t2sp_set_machine(0, 0)          # back to asking the device
+
+
+@pytest.mark.parametrize("cus,xcds", [(64, 2), (128, 4), (256, 8), (304, 8), (32, 1), (38, 1), (152, 4), (76, 2)])
+def test_dies_follow_from_the_compute_units(lib, cus, xcds):
+    lib.t2sp_set_machine(cus, 0)
+    assert (lib.t2sp_machine_cus(), lib.t2sp_machine_xcds()) == (cus, xcds)
+    lib.t2sp_set_machine(cus, 3)
+    assert lib.t2sp_machine_xcds() == 3
+
+
+@pytest.mark.parametrize("cus", CUS)
+@pytest.mark.parametrize("shape", [(8192, 8192, 8192), (6144, 6144, 6144), (5120, 5120, 2048), (4096, 16384, 2048),
+                                   (10240, 10240, 1024), (7168, 7168, 7168)])
+def test_sgemm_launches_whole_rounds_then_a_split_rest(lib, cus, shape):
+    lib.t2sp_set_machine(cus, 0)
+    M, N, K = shape
+    edge, ph = ctypes.c_int(0), (ctypes.c_int * 12)()
+    n = lib.t2sp_sgemm_plan(M, N, K, ctypes.byref(edge), ph)
+    assert n >= 1 and edge.value in (128, 256)
+    tiles = -(-M // edge.value) * -(-N // edge.value)
+    phases = [(ph[3 * i], ph[3 * i + 1], ph[3 * i + 2]) for i in range(n)]
+    covered = 0
+    for i, (first, count, splits) in enumerate(phases):
+        assert first == covered and count > 0 and splits >= 1
+        covered += count
+        if splits > 1:
+            assert count * splits <= cus            # a split rest is at most one round of workgroups
+        elif i == 0 and tiles >= cus and n > 1:
+            assert count % cus == 0                 # the unsplit part is whole rounds
+    assert covered == tiles
+    if tiles % cus and tiles > cus and K >= 1024:
+        assert any(s > 1 for _, _, s in phases), (cus, phases)
+
+
+@pytest.mark.parametrize("cus", CUS)
+def test_conv_stages_are_whole_rounds_until_the_rest(lib, cus):
+    """The benchmark convolution: CO = 256, 64 x 56 x 56 output pixels, reduction 2304."""
+    lib.t2sp_set_machine(cus, 0)
+    CO, P, KRED = 256, 64 * 56 * 56, 2304
+    st = (ctypes.c_int * 16)()
+    n = lib.t2sp_conv2d_plan(CO, P, KRED, st)
+    assert n >= 1
+    edge = {1: (256, 256), 2: (128, 128), 3: (64, 128)}
+    p = 0
+    for i in range(n):
+        cfg, p0, p1, splits = st[4 * i], st[4 * i + 1], st[4 * i + 2], st[4 * i + 3]
+        bm, bn = edge[cfg]
+        assert p0 == p and p1 > p0
+        tiles = -(-CO // bm) * -(-(p1 - p0) // bn)
+        if i < n - 1:
+            assert splits == 1 and tiles % cus == 0, (cus, i, tiles)
+        p = p1
+    assert p == P
+
+
+@pytest.mark.parametrize("cus", CUS)
+def test_syrk_splits_only_a_small_last_round(lib, cus):
+    lib.t2sp_set_machine(cus, 0)
+    out = (ctypes.c_int * 3)()
+    for N in (4096, 8192, 12288):
+        assert lib.t2sp_ssyrk_plan(N, 8192, 256, out) == 1
+        total, tail, splits = out[0], out[1], out[2]
+        side = N // 256
+        assert total == side * (side + 1) // 2
+        if splits > 1:
+            assert tail == total % cus and 0 < tail <= cus // 2 and tail * splits <= cus
+        else:
+            assert tail == 0
+
+
+@pytest.mark.parametrize("cus", CUS)
+def test_capsule_direct_tiles_fill_rounds_of_the_machine(lib, cus):
+    """The benchmark capsule layer: 32 x 49 pixels x 4 rows = 6272 vote rows by 128 columns."""
+    lib.t2sp_set_machine(cus, 0)
+    out = (ctypes.c_int * 6)()
+    assert lib.t2sp_capsule_direct16_plan(6272, 128, out) == 1
+    rpt, mb, nb, tiles_m, tiles_n, rounds = list(out)
+    assert rpt % 4 == 0 and mb == -(-rpt // 16) and tiles_m == -(-6272 // rpt) and tiles_n == -(-128 // (16 * nb))
+    groups = tiles_m * tiles_n
+    assert (rounds - 1) * cus < groups <= rounds * cus
+    assert groups > rounds * cus * 0.9              # the last round is nearly full
