@@ -60,9 +60,11 @@ int t2sp_sgemm_f32_tiled(const float *A, const float *B, float *C, int M, int N,
 
 /* BLAS form, row-major: C = alpha * op(A) * op(B) + beta * Cin with op(X) = X or X^T (transa /
  * transb non-zero: A stored K x M, B stored N x K).  Cin may be NULL (beta is then ignored) or
- * equal to C (in place).  A transposed A is first re-laid into `workspace` (required then; the
- * rest of t2sp_sgemm_ex_workspace_bytes is optional room for the planes of a split reduction,
- * as in t2sp_sgemm_f32); B^T runs natively.  Device side of the reference's 8-argument
+ * equal to C (in place).  Every form but A^T * B^T reads both operands as they lie: B^T through
+ * k-contiguous tiles, A^T (with M, N and the leading dimensions multiples of 4 and 16-byte
+ * aligned pointers) through row-contiguous ones, for any K.  Otherwise a transposed A is first
+ * re-laid into `workspace`, which is required then; the rest of t2sp_sgemm_ex_workspace_bytes is
+ * optional room for the planes of a split reduction, as in t2sp_sgemm_f32.  Device side of the reference's 8-argument
  * gemm(opa, opb, alpha, beta, A, B, C, O) pipeline behind its BLAS wrapper
  * (t2s/peppers/blas/level3/gemm/release/a10/blas-gemm.cpp:28-47). */
 size_t t2sp_sgemm_ex_workspace_bytes(int transa, int M, int N, int K);

@@ -135,7 +135,7 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) conv_kernel(const ConvArgs g) {
     RowMajorKcLoader<Cfg, EDGE> la(g.W, g.sw_o, co0, g.CO, g.KRED, kt0 * Cfg::BK);
     Im2colRcLoader<Cfg, EDGE> lb(g, p0, tab, kt0 * Cfg::BK);
     Accum<Cfg> acc;
-    mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem);
+    mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem, tail_from_for<Cfg>(g.KRED - kt0 * Cfg::BK));
     if (g.splits > 1) {
         store_partial<Cfg>(acc, g.scratch, split, co0, p0 - g.p_begin, g.Mp, g.Np);
         return;

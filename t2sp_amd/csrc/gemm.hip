@@ -38,6 +38,8 @@ struct GemmArgs {
     // with `compact` the planes hold just those tiles side by side ([row][tile][col]) instead of
     // the whole padded matrix
     int tile_first, tile_count, compact;
+    // A is stored transposed (K x M, lda >= M): taken as it lies by the kernels whose X tile is RC
+    int at;
 };
 
 __device__ __forceinline__ int64_t tiled_offset(const GemmArgs &g, int row, int col) {
@@ -98,6 +100,8 @@ struct GemmCompactMap {
 
 // BT = false: B is row-major K x N (columns contiguous, RC tile).
 // BT = true:  B is stored transposed, N x K with k contiguous (KC tile): C = A * B^T.
+// A is row-major M x K (KC tile) unless the tile's X style is RC: then it is stored transposed,
+// K x M with the rows of the product contiguous: C = A^T * B.
 template <class Cfg, bool EDGE, bool BT>
 __global__ void __launch_bounds__(Cfg::NTHREADS) sgemm_kernel(const GemmArgs g) {
     extern __shared__ __align__(16) float smem[];
@@ -109,11 +113,13 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) sgemm_kernel(const GemmArgs g) 
     const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
     int kt0 = 0, kt1 = ktiles_even<Cfg>(g.K);
     if (g.splits > 1) split_range((g.K + Cfg::BK - 1) / Cfg::BK, g.splits, split, kt0, kt1);
-    RowMajorKcLoader<Cfg, EDGE> la(g.A, g.lda, m0, g.M, g.K, kt0 * Cfg::BK);
+    using ALoader = std::conditional_t<Cfg::ASTYLE == STYLE_RC, RowMajorRcLoaderA<Cfg, EDGE>, RowMajorKcLoader<Cfg, EDGE>>;
+    ALoader la(g.A, g.lda, m0, g.M, g.K, kt0 * Cfg::BK);
     Accum<Cfg> acc;
+    const int tail_from = tail_from_for<Cfg>(g.K - kt0 * Cfg::BK);
     if constexpr (BT) {
         RowMajorKcLoaderB<Cfg, EDGE> lb(g.B, g.ldb, n0, g.N, g.K, kt0 * Cfg::BK);
-        mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem);
+        mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem, tail_from);
         if (g.splits > 1) {   // only in compact form
             store_partial<Cfg>(acc, g.scratch, split, 0, tile * Cfg::BN, Cfg::BM, g.tile_count * Cfg::BN);
             return;
@@ -126,7 +132,7 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) sgemm_kernel(const GemmArgs g) 
         });
     } else {
         RowMajorRcLoader<Cfg, EDGE> lb(g.B, g.ldb, n0, g.N, g.K, kt0 * Cfg::BK);
-        mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem);
+        mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem, tail_from);
         if (g.splits > 1) {
             if (g.compact) store_partial<Cfg>(acc, g.scratch, split, 0, tile * Cfg::BN, Cfg::BM, g.tile_count * Cfg::BN);
             else store_partial<Cfg>(acc, g.scratch, split, m0, n0, g.Mp, g.Np);
@@ -462,17 +468,8 @@ __global__ void __launch_bounds__(256) gemm_unpad_kernel(const float *src, int64
 }
 
 static inline int64_t round_up4(int64_t v) { return (v + 3) / 4 * 4; }
-// Padded reduction length: a whole number of k-tile pairs, so that the padded product runs the
-// unguarded loaders.
+// Padded reduction length of the zero-padded copies (a whole number of k-tile pairs).
 static inline int64_t pad_k(int64_t k) { return (k + 31) / 32 * 32; }
-// A reduction that is not a whole number of k-tile pairs sends every tile through the guarded
-// loaders (about 12 % slower); from about 5000^3 on, padding K in copies of A and B costs less.
-static bool gemm_k_tail_worth_padding(int M, int N, int K) {
-    if (K % 32 == 0) return false;
-    const double guarded_loss = 0.12 * 2.0 * M * N * K / 150e12;
-    const double copies = 8.0 * ((double)M * K + (double)K * N + 2.0 * M * N) / 4e12;
-    return guarded_loss > 1.3 * copies;
-}
 static inline size_t round_up256(size_t v) { return (v + 255) / 256 * 256; }
 // Bytes of the padded copies of A, B and C for a product the vector loaders cannot take as it lies.
 static size_t gemm_pad_bytes(int M, int N, int K, bool bt) {
@@ -590,6 +587,8 @@ using GemmW = TileCfg<32, 128, 16, 1, 1, STYLE_RC>;   // 1 wave per tile
 using GemmLT = TileCfg<256, 256, 16, 4, 2, STYLE_KC>;  // B^T forms: both operands k-contiguous
 using GemmMT = TileCfg<128, 128, 16, 2, 2, STYLE_KC>;
 using GemmST = TileCfg<64, 64, 16, 2, 1, STYLE_KC>;
+using GemmLA = TileCfg<256, 256, 16, 4, 2, STYLE_RC, STYLE_RC>;  // A^T forms: both operands as they lie, 64x128 per wave
+using GemmMA = TileCfg<128, 128, 16, 2, 1, STYLE_RC, STYLE_RC>;  // 2 waves
 
 // Tile configuration and reduction split for a plain product.  Large problems take 256x256
 // tiles; when those would leave CUs idle the tile shrinks, and when even 128x128 tiles are fewer
@@ -711,6 +710,26 @@ static int launch_d16(const GemmArgs &g, hipStream_t stream) {
 static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *workspace = nullptr,
                     size_t workspace_bytes = 0) {
     if (g.M <= 0 || g.N <= 0 || g.K <= 0) return T2SP_ERR_SHAPE;
+    if (g.at) {
+        // A^T * B with both operands as they lie (the caller has checked the alignment the 128-bit
+        // loads need).  Any K: k is the row index of both operands.
+        if (bt || cfg != T2SP_CFG_AUTO) return T2SP_ERR_SHAPE;
+        const GemmPlan p = plan_gemm(g.M, g.N, g.K);
+        if (p.phased) {
+            const bool phased = workspace && workspace_bytes >= p.scratch_bytes;
+            if (p.cfg == T2SP_CFG_256x256) return launch<GemmLA, false>(g, stream, 1, workspace, workspace_bytes, phased);
+            return launch<GemmMA, false>(g, stream, 1, workspace, workspace_bytes, phased);
+        }
+        // too few tiles for whole rounds: 128 x 128 tiles with the reduction split over workgroups
+        const int64_t t = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
+        const int pairs = ((g.K + 15) / 16 + 1) / 2;
+        int sp = (int)((machine().cus + t / 2) / t);
+        if (sp > pairs / 4) sp = pairs / 4;
+        if (sp > 16) sp = 16;
+        const size_t need = (size_t)sp * ((g.M + 127) / 128 * 128) * ((g.N + 127) / 128 * 128) * sizeof(float);
+        if (sp < 2 || !workspace || workspace_bytes < need) sp = 1;
+        return launch<GemmMA, false>(g, stream, sp, workspace);
+    }
     if (cfg == T2SP_CFG_DIRECT16)
         return (!bt && gemm_d16_ok(g)) ? launch_d16(g, stream) : T2SP_ERR_SHAPE;
     if (cfg == T2SP_CFG_AUTO && !bt && gemm_d16_ok(g)) {
@@ -738,13 +757,14 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
                         ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
                         ((uintptr_t)g.C % 16 == 0) && (g.tiled || g.ldc % 4 == 0) &&
                         (!g.scale || (g.ldcin % 4 == 0 && (uintptr_t)g.Cin % 16 == 0));
-    if (cfg == T2SP_CFG_AUTO && (!vec_ok || gemm_k_tail_worth_padding(g.M, g.N, g.K)) && workspace &&
+    if (cfg == T2SP_CFG_AUTO && !vec_ok && workspace &&
         ((uintptr_t)workspace % 16 == 0) && workspace_bytes >= gemm_pad_bytes(g.M, g.N, g.K, bt)) {
         // K or N not a multiple of 4, or rows that are not 16-byte aligned: multiply zero-padded,
         // aligned copies instead (the reference's BLAS wrapper pads its operands to tile multiples
         // in the same way, t2s/peppers/blas/level3/gemm/release/a10/blas-gemm.cpp:28-31) and
-        // copy the result out.  Moving the matrices twice costs little next to the product.  Large
-        // products whose K is not a whole number of k-tile pairs come here too.
+        // copy the result out.  Moving the matrices twice costs little next to the product.  (A K or
+        // M, N that is merely not a multiple of the tile needs none of this: the guarded kernels
+        // run at the rate of the unguarded ones.)
         const int kp = (int)pad_k(g.K), np = bt ? g.N : (int)round_up4(g.N);
         float *a2 = workspace;
         float *b2 = a2 + round_up256((size_t)g.M * kp * sizeof(float)) / sizeof(float);
@@ -825,7 +845,7 @@ extern "C" int t2sp_sgemm_plan(int M, int N, int K, int *tile_edge, int *phases1
 
 extern "C" size_t t2sp_sgemm_workspace_bytes(int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
-    if (K % 4 == 0 && N % 4 == 0 && !t2sp::gemm_k_tail_worth_padding(M, N, K)) return t2sp::plan_gemm(M, N, K).scratch_bytes;
+    if (K % 4 == 0 && N % 4 == 0) return t2sp::plan_gemm(M, N, K).scratch_bytes;
     // padded copies of the operands, then the planes for the padded product
     return t2sp::gemm_pad_bytes(M, N, K, false) +
            t2sp::plan_gemm(M, (int)t2sp::round_up4(N), (int)t2sp::pad_k(K)).scratch_bytes;
@@ -858,7 +878,7 @@ extern "C" size_t t2sp_sgemm_ex_workspace_bytes(int transa, int M, int N, int K)
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     // the re-laid A of the transposed form (required), then the planes of a split reduction (optional)
     const size_t pad_t = t2sp::gemm_pad_bytes(M, N, K, true), pad_n = t2sp::gemm_pad_bytes(M, N, K, false);
-    const bool padded = K % 4 || N % 4 || t2sp::gemm_k_tail_worth_padding(M, N, K);
+    const bool padded = K % 4 || N % 4;
     const size_t pad = padded ? (pad_t > pad_n ? pad_t : pad_n) : 0;
     return t2sp::round_up256(transa ? (size_t)M * K * sizeof(float) : 0) + pad +
            t2sp::plan_gemm(M, (int)t2sp::round_up4(N), (int)(padded ? t2sp::pad_k(K) : K)).scratch_bytes;
@@ -871,8 +891,20 @@ extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, fl
     if (M <= 0 || N <= 0 || K <= 0) return T2SP_ERR_SHAPE;
     const float *a = A;
     int64_t la = lda;
-    if (transa) {
-        // A is stored K x M: bring it to M x K first (the MFMA loaders want k contiguous in A)
+    auto aligned16 = [](const void *p) { return ((uintptr_t)p & 15) == 0; };
+    // A stored K x M is taken as it lies when B is not transposed too and rows of all operands
+    // can be read and written 128 bits at a time
+    const bool at_possible = transa && !transb && cfg == T2SP_CFG_AUTO && M % 4 == 0 && N % 4 == 0 && lda % 4 == 0 &&
+                             ldb % 4 == 0 && ldc % 4 == 0 && aligned16(A) && aligned16(B) && aligned16(C) &&
+                             (!Cin || (ldcin % 4 == 0 && aligned16(Cin)));
+    // Products too small for rounds of 256 x 256 tiles run faster on the kernels that want k
+    // contiguous in A (the 16 x 16 form above all), even after a pass that re-lays A: take that
+    // route when the caller has given the room for it.
+    const int64_t t256 = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
+    const bool room = workspace && workspace_bytes >= (size_t)M * K * sizeof(float);
+    const bool native_at = at_possible && (t256 >= t2sp::machine().cus * 25 / 32 || !room);
+    if (transa && !native_at) {
+        // A is stored K x M: bring it to M x K first (the loaders of the other kernels want k contiguous in A)
         if (!workspace || workspace_bytes < (size_t)M * K * sizeof(float)) return T2SP_ERR_SHAPE;
         const int ext[2] = {K, M};
         const int64_t ss[2] = {lda, 1}, ds[2] = {1, K};
@@ -888,6 +920,7 @@ extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, fl
     g.A = a; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K;
     g.lda = la; g.ldb = ldb; g.ldc = ldc;
     g.tiled = 0;
+    g.at = native_at ? 1 : 0;
     g.scale = 1; g.alpha = alpha; g.beta = beta; g.Cin = Cin ? Cin : C; g.ldcin = Cin ? ldcin : ldc;
     if (!Cin) g.beta = 0.f;
     return t2sp::dispatch(g, cfg, transb != 0, (hipStream_t)stream, workspace, workspace_bytes);

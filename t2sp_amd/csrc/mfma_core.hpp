@@ -32,6 +32,12 @@
 //       a 128-column group holds the columns congruent to c mod 4.  After the
 //       loop a lane therefore owns 4 consecutive columns of each row it holds
 //       and the epilogue stores 128 bits at a time.
+// X may be an RC tile too ([k][row], row contiguous: a matrix stored transposed, rows contiguous
+// in memory).  The two MFMA operands have the same lane layout, so the same trick applies, with
+// 64 bits per read: a lane reads 2 consecutive ROWS of k-row j + 4*(l/32) and feeds them to two
+// accumulator tiles, so tile c of a 64-row group holds the rows congruent to c mod 2.  (A 64-bit
+// read serves half a wave per cycle, so the two halves, 4 k-rows apart, never collide on a bank
+// and the tile needs no padding.)
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -45,23 +51,27 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 
 enum : int { STYLE_KC = 0, STYLE_RC = 1 };
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int BSTYLE_>
+typedef float v2f __attribute__((ext_vector_type(2)));
+
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int BSTYLE_, int ASTYLE_ = STYLE_KC>
 struct TileCfg {
-    static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, BSTYLE = BSTYLE_;
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, BSTYLE = BSTYLE_, ASTYLE = ASTYLE_;
     static constexpr int NTHREADS = WM * WN * 64;
     static constexpr int TM = BM / WM;          // rows per wave
     static constexpr int TN = BN / WN;          // cols per wave
     static constexpr int MT = TM / 32;          // 32-row accumulator tiles per wave
     static constexpr int NT = TN / 32;          // 32-col accumulator tiles per wave
-    static constexpr int LDA = BK + 4;          // floats per row of a KC tile
+    static constexpr int LDA = (ASTYLE == STYLE_RC) ? BM : BK + 4;   // floats per row of the X tile
     static constexpr int LDB = (BSTYLE == STYLE_RC) ? BN : BK + 4;
-    static constexpr int A_STAGE = BM * LDA;    // floats
+    static constexpr int A_STAGE = (ASTYLE == STYLE_RC) ? BK * LDA : BM * LDA;    // floats
+    static constexpr int A_READS = (ASTYLE == STYLE_RC) ? 4 * (MT / 2) : MT;      // LDS reads of X per k-slice
     static constexpr int B_STAGE = (BSTYLE == STYLE_RC) ? BK * LDB : BN * LDB;
     static constexpr int SMEM_FLOATS = 2 * (A_STAGE + B_STAGE);
     static constexpr int A_VEC = BM * BK / 4 / NTHREADS;  // float4 per thread per k-tile
     static constexpr int B_VEC = BN * BK / 4 / NTHREADS;
     static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be a multiple of 32x32");
     static_assert(BSTYLE == STYLE_KC || TN % 128 == 0, "RC wave tiles are 128-column groups");
+    static_assert(ASTYLE == STYLE_KC || (TM % 64 == 0 && BSTYLE == STYLE_RC), "RC X tiles: 64-row groups, with RC Y tiles");
     static_assert(BK % 16 == 0, "BK must be a multiple of 16 (an even number of k-slices of 8)");
     static_assert(A_VEC * 4 * NTHREADS == BM * BK && A_VEC >= 1, "A tile must split evenly");
     static_assert(B_VEC * 4 * NTHREADS == BN * BK && B_VEC >= 1, "B tile must split evenly");
@@ -168,10 +178,22 @@ __device__ __forceinline__ void load_frag(Frag<Cfg> &f, const float *__restrict_
                                           const float *__restrict__ Bs, int kk, int wm, int wn,
                                           int lane) {
     const int l32 = lane & 31, lhi = lane >> 5;
-    const float *a_base = As + (wm * Cfg::TM + l32) * Cfg::LDA + 4 * lhi + kk * 8;
+    if constexpr (Cfg::ASTYLE == STYLE_RC) {
 #pragma unroll
-    for (int mi = 0; mi < Cfg::MT; mi++)
-        f.a[mi] = *reinterpret_cast<const v4f *>(a_base + mi * 32 * Cfg::LDA);
+        for (int g = 0; g < Cfg::MT / 2; g++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const v2f two = *reinterpret_cast<const v2f *>(As + (kk * 8 + j + 4 * lhi) * Cfg::LDA + wm * Cfg::TM +
+                                                               g * 64 + 2 * l32);
+                f.a[2 * g][j] = two[0];
+                f.a[2 * g + 1][j] = two[1];
+            }
+    } else {
+        const float *a_base = As + (wm * Cfg::TM + l32) * Cfg::LDA + 4 * lhi + kk * 8;
+#pragma unroll
+        for (int mi = 0; mi < Cfg::MT; mi++)
+            f.a[mi] = *reinterpret_cast<const v4f *>(a_base + mi * 32 * Cfg::LDA);
+    }
     if constexpr (Cfg::BSTYLE == STYLE_RC) {
 #pragma unroll
         for (int g = 0; g < Cfg::NT / 4; g++)
@@ -229,6 +251,30 @@ struct LoaderExtraVmem { static constexpr int value = 0; };
 template <class L>
 struct LoaderExtraVmem<L, std::void_t<decltype(L::EXTRA_VMEM)>> { static constexpr int value = L::EXTRA_VMEM; };
 
+// A loader whose guarded fetch costs issue time may offer two forms: fetch<S>() without the guard
+// on the reduction index, and fetch_tail<S>() with it (it then declares
+// `static constexpr bool HAS_TAIL_FETCH = true`).  The mainloop uses the first while the tile being
+// fetched is known to lie wholly inside the reduction and the second for the last few k-tiles.
+template <class L, class = void>
+struct LoaderHasTail { static constexpr bool value = false; };
+template <class L>
+struct LoaderHasTail<L, std::void_t<decltype(L::HAS_TAIL_FETCH)>> { static constexpr bool value = L::HAS_TAIL_FETCH; };
+template <int S, bool TAIL, class L>
+__device__ __forceinline__ void loader_fetch(L &l) {
+    if constexpr (TAIL && LoaderHasTail<L>::value)
+        l.template fetch_tail<S>();
+    else
+        l.template fetch<S>();
+}
+// First k-tile (even) whose loop body must use the guarded fetch, for a reduction of `k_len`
+// elements seen from the loader's first k: the body of tile t fetches tile t + 2, and a pair of
+// bodies t, t + 1 may run unguarded while tiles t + 2 and t + 3 are whole.
+template <class Cfg>
+__device__ __host__ inline int tail_from_for(int k_len) {
+    const int whole = k_len / Cfg::BK;
+    return whole >= 4 ? 2 * (whole / 2) - 2 : 0;
+}
+
 // The pipelined mainloop.  ALoader/BLoader expose, for register slot S in {0,1},
 //   void fetch<S>()                 issue the global loads of the next k-tile into slot S
 //   void commit<S>(float *stage)    write slot S into an LDS stage
@@ -242,7 +288,7 @@ struct LoaderExtraVmem<L, std::void_t<decltype(L::EXTRA_VMEM)>> { static constex
 //     first fragments of tile t+1 are read while the last slice of tile t is multiplied;
 //   * loads and stores are interleaved one by one between MFMAs: a wave issues in order, so a
 //     burst of memory instructions that backs up in the address path would starve the MFMA pipe.
-template <class Cfg, int S, class ALoader, class BLoader>
+template <class Cfg, int S, bool TAIL, class ALoader, class BLoader>
 __device__ __forceinline__ void mainloop_body(Accum<Cfg> &acc, ALoader &la, BLoader &lb,
                                               Frag<Cfg> (&frag)[2], float *smem, int wm, int wn,
                                               int lane) {
@@ -252,11 +298,11 @@ __device__ __forceinline__ void mainloop_body(Accum<Cfg> &acc, ALoader &la, BLoa
     float *b_cur = smem + 2 * Cfg::A_STAGE + CUR * Cfg::B_STAGE;
     float *b_nxt = smem + 2 * Cfg::A_STAGE + (CUR ^ 1) * Cfg::B_STAGE;
     constexpr int MFMA_PER_SLICE = 4 * Cfg::MT * Cfg::NT;
-    constexpr int N_DS_READ = Cfg::MT + Cfg::NT;
+    constexpr int N_DS_READ = Cfg::A_READS + Cfg::NT;
     constexpr int N_DS_WRITE = Cfg::A_VEC + Cfg::B_VEC;
     constexpr int N_VMEM = N_DS_WRITE + LoaderExtraVmem<ALoader>::value + LoaderExtraVmem<BLoader>::value;
-    la.template fetch<S>();
-    lb.template fetch<S>();
+    loader_fetch<S, TAIL>(la);
+    loader_fetch<S, TAIL>(lb);
 #pragma unroll
     for (int kk = 0; kk < KK - 1; kk++) {
         load_frag<Cfg>(frag[(kk + 1) & 1], a_cur, b_cur, kk + 1, wm, wn, lane);
@@ -284,25 +330,36 @@ __device__ __forceinline__ void mainloop_body(Accum<Cfg> &acc, ALoader &la, BLoa
 
 // `ktiles` must be even (callers round the reduction up to a pair of k-tiles; loaders return
 // zeros, or re-read valid data that is never multiplied, for tiles past the end).  fetch() is
-// called for two tiles past the last one and commit() for one.
+// called for two tiles past the last one and commit() for one.  `tail_from` (even; see
+// tail_from_for) only matters to loaders with a guarded and an unguarded fetch: bodies of tiles
+// below it use the unguarded one.
 template <class Cfg, class ALoader, class BLoader>
 __device__ __forceinline__ void mainloop(Accum<Cfg> &acc, ALoader &la, BLoader &lb, int ktiles,
-                                         float *smem) {
+                                         float *smem, int tail_from = 0) {
+    constexpr bool TAILS = LoaderHasTail<ALoader>::value || LoaderHasTail<BLoader>::value;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
     acc.clear();
-    la.template fetch<0>();
-    lb.template fetch<0>();
+    loader_fetch<0, TAILS>(la);
+    loader_fetch<0, TAILS>(lb);
     la.template commit<0>(smem);
     lb.template commit<0>(smem + 2 * Cfg::A_STAGE);
-    la.template fetch<1>();
-    lb.template fetch<1>();
+    loader_fetch<1, TAILS>(la);
+    loader_fetch<1, TAILS>(lb);
     __syncthreads();
     Frag<Cfg> frag[2];
     load_frag<Cfg>(frag[0], smem, smem + 2 * Cfg::A_STAGE, 0, wm, wn, lane);
-    for (int kt = 0; kt < ktiles; kt += 2) {
-        mainloop_body<Cfg, 0>(acc, la, lb, frag, smem, wm, wn, lane);
-        mainloop_body<Cfg, 1>(acc, la, lb, frag, smem, wm, wn, lane);
+    int kt = 0;
+    if constexpr (TAILS) {
+        const int plain_end = tail_from < ktiles ? tail_from : ktiles;
+        for (; kt < plain_end; kt += 2) {
+            mainloop_body<Cfg, 0, false>(acc, la, lb, frag, smem, wm, wn, lane);
+            mainloop_body<Cfg, 1, false>(acc, la, lb, frag, smem, wm, wn, lane);
+        }
+    }
+    for (; kt < ktiles; kt += 2) {
+        mainloop_body<Cfg, 0, TAILS>(acc, la, lb, frag, smem, wm, wn, lane);
+        mainloop_body<Cfg, 1, TAILS>(acc, la, lb, frag, smem, wm, wn, lane);
     }
 }
 
@@ -323,7 +380,9 @@ __device__ __forceinline__ void drain(const Accum<Cfg> &acc, Emit &&emit) {
             for (int g = 0; g < Cfg::NT / 4; g++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
-                    const int row = wm * Cfg::TM + mi * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+                    const int in_tile = 8 * (r >> 2) + 4 * lhi + (r & 3);
+                    const int row = Cfg::ASTYLE == STYLE_RC ? wm * Cfg::TM + (mi / 2) * 64 + 2 * in_tile + (mi & 1)
+                                                            : wm * Cfg::TM + mi * 32 + in_tile;
                     const int col = wn * Cfg::TN + g * 128 + 4 * l32;
                     v4f v = {acc.t[mi][g * 4 + 0][r], acc.t[mi][g * 4 + 1][r],
                              acc.t[mi][g * 4 + 2][r], acc.t[mi][g * 4 + 3][r]};

@@ -148,7 +148,7 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) ssyrk_kernel(const SyrkArgs g) 
     RowMajorKcLoader<Cfg, EDGE> la(g.A, g.lda, m0, g.N, g.K);
     RowMajorKcLoaderB<Cfg, EDGE> lb(g.A, g.lda, n0, g.N, g.K);
     Accum<Cfg> acc;
-    mainloop<Cfg>(acc, la, lb, ktiles_even<Cfg>(g.K), smem);
+    mainloop<Cfg>(acc, la, lb, ktiles_even<Cfg>(g.K), smem, tail_from_for<Cfg>(g.K));
     const bool diag = tm == tn;
     if (MODE != SYRK_FOLDED && !EDGE && !diag) {
         // whole tile strictly above the diagonal: four rows of one column per lane go out as four
@@ -198,7 +198,7 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) ssyrk_split_kernel(const SyrkAr
     RowMajorKcLoader<Cfg, EDGE> la(g.A, g.lda, m0, g.N, g.K, kt0 * Cfg::BK);
     RowMajorKcLoaderB<Cfg, EDGE> lb(g.A, g.lda, n0, g.N, g.K, kt0 * Cfg::BK);
     Accum<Cfg> acc;
-    mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem);
+    mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem, tail_from_for<Cfg>(g.K - kt0 * Cfg::BK));
     store_partial<Cfg>(acc, g.scratch, split, 0, t * Cfg::BN, Cfg::BM, g.tile_count * Cfg::BN);
 }
 

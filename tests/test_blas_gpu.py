@@ -81,6 +81,65 @@ def test_partial_last_round_split_both_forms_of_b(oracle, shape):
         assert rel_fro(split[rows].cpu().numpy(), want)[0] <= TOL
 
 
+@pytest.mark.parametrize("shape", [(256, 256, 64), (128, 128, 37), (260, 132, 101), (516, 772, 5), (2304, 2052, 333),
+                                   (4096, 4352, 520), (4100, 4100, 70)])
+def test_transposed_a_as_it_lies_without_workspace(shape):
+    """A stored K x M (opa of blas-gemm.cpp:28-47) with no workspace: the row-contiguous loader reads
+    it in place, any K, M and N ragged against the tiles.  Integer data, so every order of the sum
+    gives the same floats; alpha, beta and C applied; then with the workspace (small products re-lay
+    A and take the k-contiguous kernels): same values."""
+    import torch
+    M, N, K = shape
+    L = t2sp_amd.lib()
+    g = torch.Generator(device="cpu").manual_seed(M + N + K)
+    At = torch.randint(-2, 3, (K, M), generator=g).float().cuda()
+    B = torch.randint(-2, 3, (K, N), generator=g).float().cuda()
+    C0 = torch.randint(-4, 5, (M, N), generator=g).float().cuda()
+    ref = 2.0 * (At.double().t() @ B.double()) - 3.0 * C0.double()
+    nbytes = L.t2sp_sgemm_ex_workspace_bytes(1, M, N, K)
+    ws = torch.empty(max(nbytes // 4, 1), device="cuda")
+    for w, nb in ((None, 0), (ws.data_ptr(), nbytes)):
+        C = torch.full((M, N), float("nan"), device="cuda")
+        rc = L.t2sp_sgemm_ex_f32(1, 0, M, N, K, 2.0, At.data_ptr(), M, B.data_ptr(), N, -3.0, C0.data_ptr(), N,
+                                 C.data_ptr(), N, 0, w, nb, None)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert torch.equal(C.double(), ref)
+    # rows of A that are not 16-byte aligned cannot be read that way: the workspace is required then
+    if M % 4 == 0:
+        Atp = torch.zeros(K, M + 2, device="cuda")
+        C = torch.empty(M, N, device="cuda")
+        rc = L.t2sp_sgemm_ex_f32(1, 0, M, N, K, 1.0, Atp.data_ptr(), M + 2, B.data_ptr(), N, 0.0, None, 0, C.data_ptr(), N, 0,
+                                 None, 0, None)
+        assert rc != 0
+
+
+@pytest.mark.parametrize("K", [4, 20, 36, 60, 64, 68, 100, 132, 1000, 4104])
+@pytest.mark.parametrize("MN", [(256, 256), (260, 132), (1024, 1028), (3000, 2000)])
+def test_reduction_tails_and_ragged_tiles_exact(K, MN):
+    """K that is not a whole number of pairs of k-tiles, M and N that are not whole tiles: the guarded
+    kernels only guard the last k-tiles (rows and columns outside the matrix are read from inside it
+    and never stored).  Integer data: exact.  Both forms of B; a canary frame around C stays."""
+    import torch
+    M, N = MN
+    L = t2sp_amd.lib()
+    g = torch.Generator(device="cpu").manual_seed(K * 7 + M)
+    A = torch.randint(-2, 3, (M, K), generator=g).float().cuda()
+    B = torch.randint(-2, 3, (K, N), generator=g).float().cuda()
+    ref = A.double() @ B.double()
+    Bt = B.t().contiguous()
+    for transb, Bd, ldb in ((0, B, N), (1, Bt, K)):
+        frame = torch.full((M + 2, N + 8), 7.0, device="cuda")
+        C = frame[1:M + 1, 4:N + 4]
+        rc = L.t2sp_sgemm_ex_f32(0, transb, M, N, K, 1.0, A.data_ptr(), K, Bd.data_ptr(), ldb, 0.0, None, 0, C.data_ptr(),
+                                 N + 8, 0, None, 0, None)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert torch.equal(C.double(), ref)
+        frame[1:M + 1, 4:N + 4] = 7.0
+        assert (frame == 7.0).all()
+
+
 def test_tiled_output_and_in_place_device(oracle):
     import torch
     M, N, K = 128, 96, 64
