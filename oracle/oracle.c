@@ -119,8 +119,16 @@ void oracle_fill_uniform(float *x, int64_t n, uint64_t seed) {
     }
 }
 
+/* threads > 0: that many; otherwise what the process started with (a call that asked for fewer
+ * must not narrow the calls after it). */
+static int initial_threads(void) {
+    static int initial = 0;
+    if (!initial) initial = omp_get_max_threads();
+    return initial;
+}
 static void set_threads(int threads) {
-    if (threads > 0) omp_set_num_threads(threads);
+    const int all = initial_threads();
+    omp_set_num_threads(threads > 0 ? threads : all);
 }
 
 /* acc[j] (op)= a * b[j*sb] for j in [0,n): one reduction step applied to a
@@ -587,4 +595,4 @@ void oracle_qrd(const float *A, float *Q, float *R, int64_t m, int64_t n, int64_
     }
 }
 
-int oracle_max_threads(void) { return omp_get_max_threads(); }
+int oracle_max_threads(void) { return initial_threads(); }

@@ -260,8 +260,24 @@ def qrd_case(torch, steps, warmup, peak):
             "workload": "16384 matrices of 128 x 128 (the size of the reference's README)"}
 
 
+def launch_floor(torch):
+    """Interval between back-to-back launches of a kernel that does next to nothing (64 floats filled, one
+    workgroup): what every launch costs on this box before its first wave runs and after its last one ends.
+    The one-launch kernels of the two small benchmark configurations (18-19 us) carry it in full."""
+    L = lib()
+    t = torch.empty(64, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        L.t2sp_fill_uniform_f32(t.data_ptr(), 64, ctypes.c_uint64(1), s)
+
+    ms = _time(torch, launch, 5000, 500)
+    return {"us_per_launch": round(ms * 1e3, 3), "workload": "5000 back-to-back launches of a one-workgroup fill kernel"}
+
+
 def run_all(torch, steps, warmup, peak, capsule_cfg=0, capsule_splits=0):
-    return {"conv2d": conv_config3(torch, steps, warmup, peak),
+    return {"launch_floor": launch_floor(torch),
+            "conv2d": conv_config3(torch, steps, warmup, peak),
             "capsule": capsule_config4(torch, steps, warmup, peak, capsule_cfg, capsule_splits),
             "mttkrp": mttkrp_config5(torch, steps, warmup, peak),
             "ssyrk_8192": ssyrk_case(torch, steps, warmup, peak, 8192, 8192, ""),
