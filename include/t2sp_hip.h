@@ -223,6 +223,11 @@ int t2sp_mttkrp_f32_noalloc(const float *B, const float *C, const float *D, floa
                             int K, int R, const int64_t *sb3, const int64_t *sc2, const int64_t *sd2,
                             const int64_t *sa2, int cfg, int splits, void *stream);
 
+/* The LDS-tiled kernels fetch two k-tiles (16 deep) ahead; bodies of tiles below the returned
+ * (even) index fetch without a guard on k, so tiles index + 2 and index + 3 must be whole for
+ * every index below it.  For tests. */
+int t2sp_sgemm_tail_from(int k_len);
+
 /* What the launch planners decide, for tests (they plan for t2sp_machine_cus() compute units, see
  * t2sp_runtime.h; no device is needed).  No counterpart in the reference.
  *   t2sp_sgemm_plan: number of launches of the LDS-tiled kernels, the tile edge (256 / 128, 0 = the

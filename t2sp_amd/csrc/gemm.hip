@@ -843,6 +843,10 @@ extern "C" int t2sp_sgemm_plan(int M, int N, int K, int *tile_edge, int *phases1
     return ph.n;
 }
 
+// First k-tile (16 deep) of a workgroup's loop whose fetches are guarded, for a reduction of k_len
+// elements seen from the workgroup's first k.  For tests of the index arithmetic.
+extern "C" int t2sp_sgemm_tail_from(int k_len) { return t2sp::tail_from_for<t2sp::GemmL>(k_len); }
+
 extern "C" size_t t2sp_sgemm_workspace_bytes(int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     if (K % 4 == 0 && N % 4 == 0) return t2sp::plan_gemm(M, N, K).scratch_bytes;

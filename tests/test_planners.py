@@ -105,3 +105,20 @@ def test_capsule_direct_tiles_fill_rounds_of_the_machine(lib, cus):
     groups = tiles_m * tiles_n
     assert (rounds - 1) * cus < groups <= rounds * cus
     assert groups > rounds * cus * 0.9              # the last round is nearly full
+
+
+def test_unguarded_loop_bodies_only_fetch_whole_k_tiles():
+    """The body of k-tile t fetches tile t + 2 (16 deep) without a guard when t is below
+    t2sp_sgemm_tail_from(k_len): every such fetch must end inside the reduction, for any length;
+    and from 64 on all but the last two pairs of tiles are unguarded."""
+    L = t2sp_amd.lib()
+    L.t2sp_sgemm_tail_from.argtypes = [ctypes.c_int]
+    for k_len in list(range(0, 600)) + [8192, 8196, 8200, 8220, 8223, 100000, 100001]:
+        t = L.t2sp_sgemm_tail_from(k_len)
+        assert t >= 0 and t % 2 == 0
+        if t > 0:
+            # the last unguarded pair of bodies is (t - 2, t - 1): it fetches tiles t and t + 1
+            assert (t + 2) * 16 <= k_len
+        tiles = -(-k_len // 16)
+        if k_len >= 64:
+            assert t >= tiles - 5
