@@ -75,23 +75,32 @@ struct PoseKcLoader {
             slot[i].init(wp, q);
         }
     }
+    // KPAD: reduction rows past KRED must read as zero, which only the last k-tiles can reach:
+    // fetch_tail guards them, fetch does not (see tail_from_for).
+    static constexpr bool HAS_TAIL_FETCH = KPAD;
     template <int S>
     __device__ __forceinline__ void fetch() {
         const bool go = KPAD || k0 + 2 * Cfg::BK <= g.KRED;
 #pragma unroll
         for (int i = 0; i < Cfg::A_VEC; i++) {
-            KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
             const uint32_t off = (uint32_t)(base_off[i] + slot[i].offset());
-            if (KPAD) {
-                const bool ok = k0 + s.k < g.KRED;
-                const v4f v = *reinterpret_cast<const v4f *>(g.P + (ok ? off : 0u));
-                reg[S][i] = ok ? v : v4f{0.f, 0.f, 0.f, 0.f};
-            } else {
-                reg[S][i] = *reinterpret_cast<const v4f *>(g.P + off);
-            }
+            reg[S][i] = *reinterpret_cast<const v4f *>(g.P + off);
             slot[i].advance(wp, go);
         }
         k0 += go ? Cfg::BK : 0;
+    }
+    template <int S>
+    __device__ __forceinline__ void fetch_tail() {
+#pragma unroll
+        for (int i = 0; i < Cfg::A_VEC; i++) {
+            KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
+            const uint32_t off = (uint32_t)(base_off[i] + slot[i].offset());
+            const bool ok = k0 + s.k < g.KRED;
+            const v4f v = *reinterpret_cast<const v4f *>(g.P + (ok ? off : 0u));
+            reg[S][i] = ok ? v : v4f{0.f, 0.f, 0.f, 0.f};
+            slot[i].advance(wp, true);
+        }
+        k0 += Cfg::BK;
     }
     template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
@@ -128,23 +137,30 @@ struct PoseWeightRcLoader {
             slot[i].init(wp, q);
         }
     }
+    static constexpr bool HAS_TAIL_FETCH = KPAD;   // as in PoseKcLoader
     template <int S>
     __device__ __forceinline__ void fetch() {
         const bool go = KPAD || k0 + 2 * Cfg::BK <= g.KRED;
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
-            RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
             const uint32_t off = (uint32_t)(base_off[i] + slot[i].offset());
-            if (KPAD) {
-                const bool ok = k0 + s.k < g.KRED;
-                const v4f v = *reinterpret_cast<const v4f *>(g.W + (ok ? off : 0u));
-                reg[S][i] = ok ? v : v4f{0.f, 0.f, 0.f, 0.f};
-            } else {
-                reg[S][i] = *reinterpret_cast<const v4f *>(g.W + off);
-            }
+            reg[S][i] = *reinterpret_cast<const v4f *>(g.W + off);
             slot[i].advance(wp, go);
         }
         k0 += go ? Cfg::BK : 0;
+    }
+    template <int S>
+    __device__ __forceinline__ void fetch_tail() {
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
+            const uint32_t off = (uint32_t)(base_off[i] + slot[i].offset());
+            const bool ok = k0 + s.k < g.KRED;
+            const v4f v = *reinterpret_cast<const v4f *>(g.W + (ok ? off : 0u));
+            reg[S][i] = ok ? v : v4f{0.f, 0.f, 0.f, 0.f};
+            slot[i].advance(wp, true);
+        }
+        k0 += Cfg::BK;
     }
     template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
@@ -172,7 +188,7 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) capsule_kernel(const CapsuleArg
     PoseKcLoader<Cfg, KPAD> la(g, m0, kt0 * Cfg::BK, tab_p);
     PoseWeightRcLoader<Cfg, KPAD> lb(g, n0, kt0 * Cfg::BK, tab_w);
     Accum<Cfg> acc;
-    mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem);
+    mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem, tail_from_for<Cfg>(g.KRED - kt0 * Cfg::BK));
     if (g.splits == 1) {
         CapsuleOutMap map{g.V, g.OH, g.OW, g.MX, g.ROWS, g.COLS, {g.sv[0], g.sv[1], g.sv[2], g.sv[3], g.sv[4]}};
         drain<Cfg>(acc, [&](int row, int col, v4f v) { map.store(m0 + row, n0 + col, v); });

@@ -67,7 +67,6 @@ struct ConvOutMap {
 template <class Cfg, bool EDGE>
 struct Im2colRcLoader {
     int base_off[Cfg::B_VEC];        // pixel part of the element offset (n, h, w), fixed for the block
-    bool col_ok[Cfg::B_VEC];
     WindowSlot slot[Cfg::B_VEC];     // window part of the reduction row this slot loads next
     v4f reg[2][Cfg::B_VEC];
     int k0;                          // first reduction row of the tile fetched next
@@ -83,8 +82,7 @@ struct Im2colRcLoader {
         for (int i = 0; i < Cfg::B_VEC; i++) {
             RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
             int p = p0 + s.col;
-            col_ok[i] = !EDGE || p < g.P;
-            if (!col_ok[i]) p = 0;
+            if (EDGE && p >= g.P) p = 0;
             const int hw = g.OH * g.OWp;
             const int n = p / hw, rem = p - n * hw;
             const int h = rem / g.OWp, w = min(rem - h * g.OWp, g.OW - 4);
@@ -92,23 +90,33 @@ struct Im2colRcLoader {
             slot[i].init(wp, (k_begin + s.k < g.KRED) ? k_begin + s.k : 0);
         }
     }
+    // EDGE: pixels past the end of the launch read pixel 0 instead (they only feed outputs that are
+    // never stored); only reduction rows past KRED must read as zero, which only the last k-tiles
+    // can reach: fetch_tail guards them, fetch does not (see tail_from_for).
+    static constexpr bool HAS_TAIL_FETCH = EDGE;
     template <int S>
     __device__ __forceinline__ void fetch() {
         const bool go = EDGE || k0 + 2 * Cfg::BK <= g.KRED;
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
-            RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
             const uint32_t off = (uint32_t)(base_off[i] + slot[i].offset());
-            if (EDGE) {
-                const bool ok = col_ok[i] && k0 + s.k < g.KRED;
-                const v4f_u v = *reinterpret_cast<const v4f_u *>(g.I + (ok ? off : 0u));
-                reg[S][i] = ok ? (v4f)v : v4f{0.f, 0.f, 0.f, 0.f};
-            } else {
-                reg[S][i] = *reinterpret_cast<const v4f_u *>(g.I + off);
-            }
+            reg[S][i] = *reinterpret_cast<const v4f_u *>(g.I + off);
             slot[i].advance(wp, go);
         }
         k0 += go ? Cfg::BK : 0;
+    }
+    template <int S>
+    __device__ __forceinline__ void fetch_tail() {
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
+            const uint32_t off = (uint32_t)(base_off[i] + slot[i].offset());
+            const bool ok = k0 + s.k < g.KRED;
+            const v4f_u v = *reinterpret_cast<const v4f_u *>(g.I + (ok ? off : 0u));
+            reg[S][i] = ok ? (v4f)v : v4f{0.f, 0.f, 0.f, 0.f};
+            slot[i].advance(wp, true);
+        }
+        k0 += Cfg::BK;
     }
     template <int S>
     __device__ __forceinline__ void commit(float *stage) const {

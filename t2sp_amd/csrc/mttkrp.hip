@@ -75,7 +75,6 @@ template <class Cfg, bool EDGE>
 struct TensorKcLoader {
     const float *p[Cfg::A_VEC];
     const float *safe;
-    bool ok[Cfg::A_VEC];
     v4f reg[2][Cfg::A_VEC];
     KjWalk w;
     int64_t off, sb_k;    // off = k * sb_k + j0
@@ -85,23 +84,29 @@ struct TensorKcLoader {
 #pragma unroll
         for (int i = 0; i < Cfg::A_VEC; i++) {
             KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
-            ok[i] = !EDGE || m0 + s.row < g.I;
-            p[i] = g.B + (int64_t)(ok[i] ? m0 + s.row : 0) * g.sb_i + s.k;
+            const bool ok = !EDGE || m0 + s.row < g.I;
+            p[i] = g.B + (int64_t)(ok ? m0 + s.row : 0) * g.sb_i + s.k;
         }
     }
+    // EDGE: a row past I reads row 0 instead (it only feeds outputs that are never stored); only a
+    // tile past the end of the reduction must read as zero, which only the last fetches of a
+    // workgroup can reach: fetch_tail guards them, fetch does not (see tail_from_for).
+    static constexpr bool HAS_TAIL_FETCH = EDGE;
     template <int S>
     __device__ __forceinline__ void fetch() {
-        const bool in = w.inside();
 #pragma unroll
-        for (int i = 0; i < Cfg::A_VEC; i++) {
-            if (EDGE)
-                reg[S][i] = load_or_zero(p[i] + (in ? off : 0), ok[i] && in, safe);
-            else
-                reg[S][i] = *reinterpret_cast<const v4f *>(p[i] + off);
-        }
+        for (int i = 0; i < Cfg::A_VEC; i++) reg[S][i] = *reinterpret_cast<const v4f *>(p[i] + off);
         const int kt_before = w.kt;
         const bool wrap = w.next(Cfg::BK, EDGE);
         off += (w.kt != kt_before) ? (wrap ? sb_k - (w.J - Cfg::BK) : Cfg::BK) : 0;
+    }
+    template <int S>
+    __device__ __forceinline__ void fetch_tail() {
+        const bool in = w.inside();
+#pragma unroll
+        for (int i = 0; i < Cfg::A_VEC; i++) reg[S][i] = load_or_zero(p[i] + (in ? off : 0), in, safe);
+        const bool wrap = w.next(Cfg::BK, true);
+        off += wrap ? sb_k - (w.J - Cfg::BK) : Cfg::BK;
     }
     template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
@@ -121,7 +126,6 @@ struct KhatriRaoKcLoader {
     const float *pc[Cfg::B_VEC];
     const float *pd[Cfg::B_VEC];
     const float *safe;
-    bool ok[Cfg::B_VEC];
     v4f reg[2][Cfg::B_VEC];
     float dval[2][Cfg::B_VEC];
     KjWalk w;
@@ -132,26 +136,33 @@ struct KhatriRaoKcLoader {
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
-            ok[i] = !EDGE || n0 + s.row < g.R;
-            const int r = ok[i] ? n0 + s.row : 0;
+            const int r = (!EDGE || n0 + s.row < g.R) ? n0 + s.row : 0;
             pc[i] = g.C + (int64_t)r * g.sc_r + s.k;
             pd[i] = g.D + (int64_t)r * g.sd_r;
         }
     }
+    static constexpr bool HAS_TAIL_FETCH = EDGE;   // as in TensorKcLoader; a column past R reads column 0
     template <int S>
     __device__ __forceinline__ void fetch() {
-        const bool in = w.inside();
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
-            if (EDGE)
-                reg[S][i] = load_or_zero(pc[i] + (in ? w.j0 : 0), ok[i] && in, safe);
-            else
-                reg[S][i] = *reinterpret_cast<const v4f *>(pc[i] + w.j0);
-            dval[S][i] = pd[i][(!EDGE || in) ? koff : 0];
+            reg[S][i] = *reinterpret_cast<const v4f *>(pc[i] + w.j0);
+            dval[S][i] = pd[i][koff];
         }
         const int kt_before = w.kt;
         const bool wrap = w.next(Cfg::BK, EDGE);
         koff += (w.kt != kt_before && wrap) ? sd_k : 0;
+    }
+    template <int S>
+    __device__ __forceinline__ void fetch_tail() {
+        const bool in = w.inside();
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            reg[S][i] = load_or_zero(pc[i] + (in ? w.j0 : 0), in, safe);
+            dval[S][i] = pd[i][in ? koff : 0];
+        }
+        const bool wrap = w.next(Cfg::BK, true);
+        koff += wrap ? sd_k : 0;
     }
     template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
@@ -174,7 +185,7 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) mttkrp_kernel(const MttkrpArgs 
     TensorKcLoader<Cfg, EDGE> la(g, m0, kt0);
     KhatriRaoKcLoader<Cfg, EDGE> lb(g, n0, kt0);
     Accum<Cfg> acc;
-    mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem);
+    mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem, tail_from_for<Cfg>((g.K * (g.J / Cfg::BK) - kt0) * Cfg::BK));
     if (g.splits == 1) {
         MttkrpOutMap map{g.A, g.I, g.R, g.sa_r};
         drain<Cfg>(acc, [&](int row, int col, v4f v) { map.store(m0 + row, n0 + col, v); });

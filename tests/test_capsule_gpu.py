@@ -69,6 +69,21 @@ def test_short_and_odd_reductions_ragged_columns(oracle, ci, co, n, cfg):
     assert err <= TOL, (ci, co, n, cfg, err, mx)
 
 
+@pytest.mark.parametrize("ci", [1, 2, 3, 5, 9, 17])
+@pytest.mark.parametrize("cfg,splits", [(2, 1), (3, 1), (4, 1), (2, 2), (1, 1)])
+def test_lds_tile_kernels_reduction_tails_exact(ci, cfg, splits):
+    """The LDS-tiled kernels with reductions of CI * 36 = 36 .. 612 rows, none a whole number of pairs of
+    16-row tiles (guarded fetches only for the last tiles; with a split, per slice).  Integer data: exact
+    against the float64 einsum."""
+    rng = np.random.default_rng(ci)
+    P = rng.integers(-2, 3, (3, ci, 9, 7, 4, 4)).astype(np.float32)
+    W = rng.integers(-2, 3, (20, ci, 3, 3, 4, 4)).astype(np.float32)
+    win = np.lib.stride_tricks.sliding_window_view(P, (3, 3), axis=(2, 3))[:, :, ::2, ::2]    # n c h w mx mk kh kw
+    want = np.einsum("nchwxkab,ocabky->nohwxy", win.astype(np.float64), W.astype(np.float64))
+    got = t2sp_amd.capsule(P, W, cfg=cfg, splits=splits)
+    assert (got == want).all()
+
+
 @pytest.mark.parametrize("n,co", [(23, 32), (28, 32), (32, 16), (27, 20), (20, 32), (40, 64)])
 def test_direct16_tile_plans(oracle, n, co):
     """Shapes that make the 16 x 16 direct kernel pick each of its tile forms: one column block and

@@ -58,6 +58,20 @@ def test_ragged_shapes(oracle, shape):
     assert rel_fro(run(I, W), oracle.conv(I, W))[0] <= TOL
 
 
+@pytest.mark.parametrize("CI", [4, 8, 12, 20, 36, 68])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3])
+def test_reduction_tails_guarded_only_in_the_last_tiles_exact(cfg, CI):
+    """Reductions of CI * 9 = 36 .. 612 rows, none a whole number of pairs of 16-row tiles, so the
+    loop of unguarded fetches is empty, one pair long or many; 70 output channels and 3 * 9 * 12
+    pixels leave ragged tiles on both sides.  Integer data: exact against the float64 convolution."""
+    import torch
+    g = torch.Generator().manual_seed(CI)
+    I = torch.randint(-2, 3, (3, CI, 11, 14), generator=g).float().numpy()
+    W = torch.randint(-2, 3, (70, CI, 3, 3), generator=g).float().numpy()
+    want = torch.nn.functional.conv2d(torch.from_numpy(I).double(), torch.from_numpy(W).double()).numpy()
+    assert (run(I, W, cfg=cfg) == want).all()
+
+
 @pytest.mark.parametrize("shape", [(2, 3, 64, 32, 36, 7, 7), (1, 5, 40, 8, 20, 3, 3), (3, 3, 16, 12, 12, 5, 5), (1, 1, 8, 8, 8, 3, 3)])
 def test_odd_reduction_length_takes_padded_weights(oracle, shape):
     """CI*KY*KX not a multiple of 4 (first-layer shapes such as 3 x 7 x 7 = 147): the weights are

@@ -91,6 +91,21 @@ def test_ragged_sizes_and_layout_rule(oracle):
     assert e.value.code == -8
 
 
+@pytest.mark.parametrize("shape", [(100, 16, 1, 20), (100, 16, 3, 20), (260, 32, 3, 70), (40, 48, 5, 300), (300, 64, 9, 36)])
+@pytest.mark.parametrize("cfg,splits", [(0, 0), (1, 1), (2, 1), (3, 1), (4, 1), (2, 3)])
+def test_ragged_tiles_and_odd_tile_counts_exact(shape, cfg, splits):
+    """I and R that leave ragged tiles (rows and columns outside read from inside and are never stored)
+    and reductions of 1 to 36 tiles of 16, odd and even (tiles past the end read as zero, guarded only in
+    the last fetches).  Integer data: exact against the float64 einsum."""
+    I, J, K, R = shape
+    rng = np.random.default_rng(I + J + K + R)
+    B = np.ascontiguousarray(rng.integers(-2, 3, (K, I, J)).astype(np.float32)).transpose(1, 2, 0)    # [k][i][j] in memory
+    C = rng.integers(-2, 3, (J, R)).astype(np.float32)
+    D = rng.integers(-2, 3, (K, R)).astype(np.float32)
+    want = np.einsum("ijk,jr,kr->ir", B.astype(np.float64), C.astype(np.float64), D.astype(np.float64))
+    assert (run(B, C, D, cfg=cfg, splits=splits) == want).all()
+
+
 def test_thin_layer_takes_any_strides(oracle):
     import torch
     B, C, D = oracle.fill_uniform((24, 10, 6), 15), oracle.fill_uniform((10, 8), 16), oracle.fill_uniform((6, 8), 17)
