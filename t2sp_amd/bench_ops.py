@@ -311,8 +311,30 @@ def launch_floor(torch):
     return {"us_per_launch": round(ms * 1e3, 3), "workload": "5000 back-to-back launches of a one-workgroup fill kernel"}
 
 
+def copy_rate(torch):
+    """What a plain device-to-device copy of 256 MiB reaches on this box (torch's copy kernel; read + write
+    bytes per second): the measured ceiling next to the nominal 8 TB/s that `frac_of_hbm_peak` of the three
+    matrix-vector entries is quoted against."""
+    n = 64 << 20
+    src, dst = torch.empty(n, device="cuda"), torch.empty(n, device="cuda")
+    ms = _time(torch, lambda: dst.copy_(src), 20, 5)
+    gbs = 8.0 * n / ms / 1e6
+    return {"GB/s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / 8000.0, 4), "avg_launch_ms": round(ms, 5),
+            "workload": "device copy of 64 Mi floats (256 MiB read, 256 MiB written)"}
+
+
 def run_all(torch, steps, warmup, peak, capsule_cfg=0, capsule_splits=0):
+    out = _run_all(torch, steps, warmup, peak, capsule_cfg, capsule_splits)
+    ceiling = out["hbm_copy_rate"]["GB/s"]
+    for v in out.values():
+        if v.get("bound") == "hbm":
+            v["frac_of_measured_copy_rate"] = round(v["GB/s"] / ceiling, 4)
+    return out
+
+
+def _run_all(torch, steps, warmup, peak, capsule_cfg=0, capsule_splits=0):
     return {"launch_floor": launch_floor(torch),
+            "hbm_copy_rate": copy_rate(torch),
             "conv2d": conv_config3(torch, steps, warmup, peak),
             "capsule": capsule_config4(torch, steps, warmup, peak, capsule_cfg, capsule_splits),
             "mttkrp": mttkrp_config5(torch, steps, warmup, peak),
