@@ -246,9 +246,11 @@ static ConvPlan plan_conv(int CO, int P, int KRED) {
     for (int i = best; i < 3 && p0 < P; i++) {
         if (i != best && all[i].cfg != T2SP_CFG_128x128) break;
         const Cand &c = all[i];
-        const int64_t rounds = tiles(c, p0) / CUS;
+        // a round puts a wave on every SIMD: one workgroup per CU, two of the 2-wave ones
+        const int64_t per_round = (int64_t)CUS * (c.bm == 64 ? 2 : 1);
+        const int64_t rounds = tiles(c, p0) / per_round;
         if (rounds < 1) continue;
-        const int64_t ptiles = rounds * CUS / tiles_m(c);
+        const int64_t ptiles = rounds * per_round / tiles_m(c);
         const int p1 = (int)(p0 + ptiles * c.bn < P ? p0 + ptiles * c.bn : P);
         p.st[p.n++] = ConvStage{c.cfg, p0, p1, 1};
         p0 = p1;
@@ -261,15 +263,19 @@ static ConvPlan plan_conv(int CO, int P, int KRED) {
     for (int i = best; i < 3; i++) {
         const Cand &c = all[i];
         const int64_t t = tiles(c, p0);
-        int smax = (int)(CUS / (t < 1 ? 1 : t));
-        if (smax > pairs / 4) smax = pairs / 4;
+        const int waves = c.bm == 256 ? 8 : c.bm == 128 ? 4 : 2;      // per workgroup
+        int smax = pairs / 4;
         if (smax > 16) smax = 16;
         if (smax < 1) smax = 1;
         for (int sp = 1; sp <= smax; sp++) {
+            // Workgroups spread evenly over the CUs; a CU needs a wave on each of its four SIMDs to
+            // multiply at its full rate, so one 2-wave workgroup alone on a CU runs at half of it
+            // (several small workgroups share a CU: their LDS tiles and registers fit).
+            const int64_t per_cu = (t * sp + CUS - 1) / CUS;
+            const double busy = per_cu * waves >= 4 ? 1.0 : per_cu * waves / 4.0;
             const double wg = 2.0 * c.bm * c.bn * KRED / (614e9 * c.eff) / sp;     // one workgroup's MFMA time (256 flop/clk at 2.4 GHz)
-            const double rounds = (double)((t * sp + CUS - 1) / CUS);
             const double planes = sp > 1 ? (double)t * sp * c.bm * c.bn * 8.0 / 3e12 + 8e-6 : 0.0;
-            const double time = wg * rounds + planes;
+            const double time = wg * (double)per_cu / busy + planes;
             if (time < best_time) { best_time = time; tail = ConvStage{c.cfg, p0, P, sp}; }
         }
     }
