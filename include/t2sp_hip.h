@@ -32,7 +32,7 @@ extern "C" {
 #define T2SP_CFG_64x128 3
 #define T2SP_CFG_32x128 4 /* sgemm: one wavefront per tile, for problems with few outputs; mttkrp: the 256x64 tile for small ranks */
 #define T2SP_CFG_DIRECT 5 /* small problems (sgemm, capsule): one small tile per workgroup, reduction split over its waves, operands global -> registers */
-#define T2SP_CFG_DIRECT16 6 /* capsule: the direct form on 16x16 MFMA tiles, rows and column blocks per workgroup chosen to fill the CUs evenly */
+#define T2SP_CFG_DIRECT16 6 /* sgemm, conv, capsule: the direct form on 16x16 MFMA tiles, rows (and column blocks) per workgroup chosen to fill the CUs evenly */
 #define T2SP_CFG_SCALAR 99
 
 #define T2SP_MAX_DIMS 10
@@ -240,6 +240,10 @@ int t2sp_sgemm_tail_from(int k_len);
  *     along columns, rounds of workgroups) of the 16 x 16 direct form for rows x cols votes. */
 int t2sp_sgemm_plan(int M, int N, int K, int *tile_edge, int *phases12);
 int t2sp_conv2d_plan(int CO, int P, int KRED, int *stages16);
+/* The one-launch 16 x 16 form of the convolution: (row blocks, rows per tile, tiles along CO, tiles
+ * along the pixels) and the estimated seconds of that form and of the staged plan above; returns 1
+ * when the automatic choice takes the 16 x 16 form (given operands it can address). */
+int t2sp_conv2d_direct16_plan(int CO, int P, int KRED, int *out4, double *times2);
 int t2sp_ssyrk_plan(int N, int K, int b, int *total_tail_splits);
 int t2sp_capsule_direct16_plan(int rows, int cols, int *out6);
 

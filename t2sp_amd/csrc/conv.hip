@@ -212,6 +212,188 @@ static int launch_conv(ConvArgs g, int p_begin, int p_end, int splits, float *sc
     return T2SP_OK;
 }
 
+// Small convolutions: too few 128 x 128 tiles for the CUs.  The one-launch form of the small SGEMM
+// (gemm.hip, sgemm_direct16_kernel) with the im2col operand: a workgroup of 4 waves owns
+// `rows_per_tile` output channels (up to 16 * MB) by 64 pixel positions (16 groups of four along
+// w), splits the reduction over its waves and sums the four partial tiles through LDS in wave
+// order; nothing is staged in LDS but a table of the element offset of every reduction row
+// (ci, kh, kw), built once per workgroup.  Per step of 16 reduction rows a lane loads, straight
+// into MFMA operand registers (v_mfma_f32_16x16x4_f32, see gemm.hip for the lane layouts), 4
+// consecutive k of its weight rows (128 bits each) and the four pixels of its group for each of
+// its 4 reduction rows (4-byte aligned 128-bit loads), from scalar bases + 32-bit lane offsets.
+constexpr int CONV_D16_WAVES = 4;
+constexpr int CONV_D16_RING = 3;
+constexpr int CONV_D16_MAX_KRED = 8192;      // the offset table: 32 KB of LDS
+
+template <int MB>
+__global__ void __launch_bounds__(CONV_D16_WAVES * 64) conv_direct16_kernel(const ConvArgs g, int rows_per_tile) {
+    constexpr int NW = CONV_D16_WAVES, R = CONV_D16_RING, NB = 4;
+    extern __shared__ __align__(16) float smem[];
+    v4f *red = reinterpret_cast<v4f *>(smem);                                   // [wave][mb][nb][lane]
+    int *tab = reinterpret_cast<int *>(smem + NW * MB * NB * 64 * 4);           // [KRED] byte offsets
+    {
+        const int win = g.KH * g.KW;
+        for (int k = threadIdx.x; k < g.KRED; k += NW * 64) {
+            const int ci = k / win, r = k - ci * win;
+            const int kh = r / g.KW, kw = r - kh * g.KW;
+            tab[k] = 4 * (ci * g.si_c + kh * g.si_h + kw);
+        }
+    }
+    __syncthreads();
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
+    const int tm = blockIdx.x % g.tiles_m, tn = blockIdx.x / g.tiles_m;
+    const int m0 = tm * rows_per_tile, n0 = tn * 64;
+    const int m_end = min(m0 + rows_per_tile, g.CO);
+    const int steps = g.KRED >> 4;
+    const int s0 = (int)((int64_t)steps * wave / NW), s1 = (int)((int64_t)steps * (wave + 1) / NW);
+    const int nsteps = s1 - s0;
+
+    uint32_t a_off[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) a_off[mb] = 4u * (uint32_t)(min(m0 + 16 * mb + li, g.CO - 1) * (int)g.sw_o + 4 * lq);
+    // this lane's group of four pixels; a group past the end reads group 0 and is never stored
+    const int p = n0 + 4 * li;
+    const bool p_ok = p < g.P;
+    const int pp = p_ok ? p : 0;
+    const int hw = g.OH * g.OWp;
+    const int n = pp / hw, rem = pp - n * hw;
+    const int h = rem / g.OWp, w = min(rem - h * g.OWp, g.OW - 4);
+    const uint32_t b_off = 4u * (uint32_t)(n * g.si_n + h * g.si_h + w);
+    const char *a_base = reinterpret_cast<const char *>(g.W + 16 * s0);
+    const char *b_base = reinterpret_cast<const char *>(g.I);
+    const int *my_tab = tab + 16 * s0 + 4 * lq;
+    int issued = 0;
+
+    v4f ra[R][MB];
+    v4f rb[R][4];
+    typedef int v4i __attribute__((ext_vector_type(4)));
+    v4i tcur = *reinterpret_cast<const v4i *>(my_tab);      // offsets of this lane's 4 reduction rows of the next step issued
+#define T2SP_CONV_D16_ISSUE(d)                                                                      \
+    {                                                                                               \
+        const int st = min(issued, steps - 1 - s0);                                                 \
+        const int st_next = min(issued + 1, steps - 1 - s0);                                        \
+        const uint32_t ao = 64u * (uint32_t)st;                                                     \
+        issued++;                                                                                   \
+        _Pragma("unroll") for (int j = 0; j < 4; j++)                                               \
+            rb[d][j] = *reinterpret_cast<const v4f_u *>(b_base + (b_off + (uint32_t)tcur[j]));      \
+        _Pragma("unroll") for (int mb = 0; mb < MB; mb++)                                           \
+            ra[d][mb] = *reinterpret_cast<const v4f *>(a_base + (a_off[mb] + ao));                  \
+        tcur = *reinterpret_cast<const v4i *>(my_tab + 16 * st_next);                               \
+    }
+#define T2SP_CONV_D16_MMA(d)                                                                        \
+    _Pragma("unroll") for (int j = 0; j < 4; j++)                                                   \
+        _Pragma("unroll") for (int mb = 0; mb < MB; mb++)                                           \
+            _Pragma("unroll") for (int nb = 0; nb < NB; nb++)                                       \
+                acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[d][mb][j], rb[d][j][nb], acc[mb][nb], 0, 0, 0);
+    v4f acc[MB][NB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) acc[mb][nb] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int d = 0; d < R - 1; d++) {
+        T2SP_CONV_D16_ISSUE(d)
+        __builtin_amdgcn_sched_barrier(0);   // keep the sets in program order: waits count loads
+    }
+    const int main_iters = nsteps > 0 ? (nsteps - 1) / R : 0;
+    const int left = nsteps - main_iters * R;
+    for (int it = 0; it < main_iters; it++) {
+#pragma unroll
+        for (int d = 0; d < R; d++) {
+            T2SP_CONV_D16_ISSUE((d + R - 1) % R)
+            T2SP_CONV_D16_MMA(d)
+            T2SP_INTERLEAVE(SG_VMEM_READ, MB + 4, (4 * MB * NB) / (MB + 4))
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    T2SP_CONV_D16_ISSUE(R - 1)
+#pragma unroll
+    for (int d = 0; d < R; d++) {
+        if (d < left) { T2SP_CONV_D16_MMA(d) }
+    }
+#undef T2SP_CONV_D16_ISSUE
+#undef T2SP_CONV_D16_MMA
+
+    v4f *mine = red + wave * MB * NB * 64 + lane;
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) mine[(mb * NB + nb) * 64] = acc[mb][nb];
+    __syncthreads();
+    // sum the partial tiles of the waves in wave order; a lane ends up with its four pixels of 4 channels
+    const bool ragged = g.OW != g.OWp;
+    float *o_base = g.O + n * g.so_n + h * g.so_h + w;
+    for (int mb = wave; mb < MB; mb += NW) {
+        v4f sum[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+            const v4f *src = red + (mb * NB + nb) * 64 + lane;
+            sum[nb] = src[0];
+#pragma unroll
+            for (int wv = 1; wv < NW; wv++) sum[nb] += src[wv * MB * NB * 64];
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int co = m0 + 16 * mb + 4 * lq + r;
+            const v4f out = {sum[0][r], sum[1][r], sum[2][r], sum[3][r]};
+            if (co < m_end && p_ok) conv_store4(o_base + co * g.so_c, out, ragged);
+        }
+    }
+}
+
+// Rows per tile of the 16 x 16 form: the split of CO into tiles of up to 16 * mb rows that fills
+// rounds of CUs with the least estimated time (as plan_gemm_d16 in gemm.hip, columns fixed at 64).
+struct ConvD16Plan {
+    int mb, rows_per_tile, tiles_m, tiles_n;
+    double time;       // estimated seconds
+};
+static ConvD16Plan plan_conv_d16(int CO, int P, int KRED) {
+    const int cus = machine().cus;
+    ConvD16Plan best{};
+    best.time = 1e300;
+    const int tiles_n = (P + 63) / 64;
+    for (int mb = 1; mb <= 6; mb++) {
+        const int tiles_m = (CO + 16 * mb - 1) / (16 * mb);
+        const int rpt = (CO + tiles_m - 1) / tiles_m;
+        const int64_t tiles = (int64_t)tiles_m * tiles_n;
+        const double loads_per_mfma = (double)(mb + 4) / (4.0 * mb * 4);
+        // a workgroup alone on its CU: 4 waves at the rate of this form (measured: 0.92 of the MFMA
+        // rate at 4 x 4 blocks, less with fewer MFMAs per load) + launch, first loads, exchange
+        // (5 and 6 row blocks run 6 % under that: their operand ring leaves the registers little room)
+        const double wg = 2.0 * (16.0 * mb) * 64.0 * KRED / 614e9 * (1.0 + 1.5 * loads_per_mfma) / 1.09 * (mb >= 5 ? 1.06 : 1.0);
+        const double time = (double)((tiles + cus - 1) / cus) * (wg + 2.5e-6) + 3e-6;
+        if (time < best.time) best = ConvD16Plan{mb, rpt, tiles_m, tiles_n, time};
+    }
+    return best;
+}
+
+struct ConvPlan;
+static bool conv_prefers_d16(int CO, int P, int KRED, const ConvPlan &lds);
+
+template <int MB>
+static int launch_conv_d16_t(ConvArgs g, const ConvD16Plan &p, hipStream_t stream) {
+    g.tiles_m = p.tiles_m;
+    g.tiles_n = p.tiles_n;
+    const size_t smem = (size_t)CONV_D16_WAVES * MB * 4 * 64 * sizeof(v4f) + (size_t)g.KRED * sizeof(int);
+    auto kern = conv_direct16_kernel<MB>;
+    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+        return T2SP_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(CONV_D16_WAVES * 64), smem, stream, g, p.rows_per_tile);
+    return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+}
+static int launch_conv_d16(const ConvArgs &g, hipStream_t stream) {
+    const ConvD16Plan p = plan_conv_d16(g.CO, g.P, g.KRED);
+    switch (p.mb) {
+        case 1: return launch_conv_d16_t<1>(g, p, stream);
+        case 2: return launch_conv_d16_t<2>(g, p, stream);
+        case 3: return launch_conv_d16_t<3>(g, p, stream);
+        case 4: return launch_conv_d16_t<4>(g, p, stream);
+        case 5: return launch_conv_d16_t<5>(g, p, stream);
+        default: return launch_conv_d16_t<6>(g, p, stream);
+    }
+}
+
 // How the automatic configuration covers the pixels.  One workgroup of the larger tiles occupies
 // a CU, so tiles run in rounds of 256 (the CU count) and a partial last round would leave most
 // CUs idle for a whole tile time.  Stages, each over its own range of output pixels:
@@ -228,7 +410,9 @@ struct ConvPlan {
     int n;
     ConvStage st[4];
     size_t scratch_bytes;
+    double time;                // estimated seconds (MFMA time at the sustained rate + planes + launches)
 };
+constexpr double CONV_SUSTAINED = 0.92;     // of the MFMA peak, what the 256 x 256 tile reaches on the benchmark shape
 static ConvPlan plan_conv(int CO, int P, int KRED) {
     const int CUS = machine().cus;
     struct Cand { int cfg, bm, bn; double eff; };
@@ -253,6 +437,7 @@ static ConvPlan plan_conv(int CO, int P, int KRED) {
         const int64_t ptiles = rounds * per_round / tiles_m(c);
         const int p1 = (int)(p0 + ptiles * c.bn < P ? p0 + ptiles * c.bn : P);
         p.st[p.n++] = ConvStage{c.cfg, p0, p1, 1};
+        p.time += (double)rounds * (c.bm == 64 ? 2.0 : 1.0) * 2.0 * c.bm * c.bn * KRED / (614e9 * c.eff * CONV_SUSTAINED) + 3e-6;
         p0 = p1;
     }
     if (p0 >= P) return p;
@@ -273,18 +458,26 @@ static ConvPlan plan_conv(int CO, int P, int KRED) {
             // (several small workgroups share a CU: their LDS tiles and registers fit).
             const int64_t per_cu = (t * sp + CUS - 1) / CUS;
             const double busy = per_cu * waves >= 4 ? 1.0 : per_cu * waves / 4.0;
-            const double wg = 2.0 * c.bm * c.bn * KRED / (614e9 * c.eff) / sp;     // one workgroup's MFMA time (256 flop/clk at 2.4 GHz)
+            const double wg = 2.0 * c.bm * c.bn * KRED / (614e9 * c.eff * CONV_SUSTAINED) / sp;     // one workgroup's MFMA time (256 flop/clk at 2.4 GHz)
             const double planes = sp > 1 ? (double)t * sp * c.bm * c.bn * 8.0 / 3e12 + 8e-6 : 0.0;
             const double time = wg * (double)per_cu / busy + planes;
             if (time < best_time) { best_time = time; tail = ConvStage{c.cfg, p0, P, sp}; }
         }
     }
     p.st[p.n++] = tail;
+    p.time += best_time + 3e-6;
     if (tail.splits > 1) {
         const Cand &c = all[tail.cfg == T2SP_CFG_256x256 ? 0 : tail.cfg == T2SP_CFG_128x128 ? 1 : 2];
         p.scratch_bytes = (size_t)tail.splits * (tiles_m(c) * c.bm) * ((P - p0 + c.bn - 1) / c.bn * c.bn) * sizeof(float);
     }
     return p;
+}
+
+// Short reductions (1 x 1 kernels over few channels) leave the 16 x 16 form nothing to amortise its
+// set-up and its narrow stores with; from 288 reduction rows on (3 x 3 over 32 channels) the estimates decide.
+static bool conv_prefers_d16(int CO, int P, int KRED, const ConvPlan &lds) {
+    // within 3 % the staged plan is taken: over many rounds it tends to beat its estimate, the 16 x 16 form not
+    return KRED >= 288 && plan_conv_d16(CO, P, KRED).time < 0.97 * lds.time;
 }
 
 using ConvL = TileCfg<256, 256, 16, 4, 2, STYLE_RC>;
@@ -321,6 +514,15 @@ extern "C" int t2sp_conv2d_plan(int CO, int P, int KRED, int *stages16) {
         stages16[4 * i + 2] = p.st[i].p_end; stages16[4 * i + 3] = p.st[i].splits;
     }
     return p.n;
+}
+
+extern "C" int t2sp_conv2d_direct16_plan(int CO, int P, int KRED, int *out4, double *times2) {
+    if (CO <= 0 || P <= 0 || KRED <= 0 || !out4 || !times2) return 0;
+    const t2sp::ConvD16Plan d = t2sp::plan_conv_d16(CO, P, KRED);
+    const t2sp::ConvPlan l = t2sp::plan_conv(CO, P, KRED);
+    out4[0] = d.mb; out4[1] = d.rows_per_tile; out4[2] = d.tiles_m; out4[3] = d.tiles_n;
+    times2[0] = d.time; times2[1] = l.time;
+    return KRED % 16 == 0 && KRED <= t2sp::CONV_D16_MAX_KRED && t2sp::conv_prefers_d16(CO, P, KRED, l) ? 1 : 0;
 }
 
 extern "C" size_t t2sp_conv2d_workspace_bytes(int N, int CI, int CO, int OH, int OW, int KH, int KW) {
@@ -387,6 +589,11 @@ extern "C" int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, 
     g.so_n = so4[0]; g.so_c = so4[1]; g.so_h = so4[2];
     g.OWp = owp;
     g.P = N * OH * owp; g.KRED = CI * KH * KW;
+    // the 16 x 16 form: reductions of whole steps of 16 whose offset table fits, byte offsets in 32 bits,
+    // weight rows that start on 16-byte boundaries
+    const bool d16_ok = g.KRED % 16 == 0 && g.KRED <= CONV_D16_MAX_KRED && in_span < (1 << 30) &&
+                        (int64_t)CO * sw_o < (1 << 30);
+    if (cfg == T2SP_CFG_DIRECT16) return d16_ok ? launch_conv_d16(g, st) : T2SP_ERR_SHAPE;
     switch (cfg) {
         case T2SP_CFG_256x256: return launch_conv<ConvL>(g, 0, g.P, 1, nullptr, st);
         case T2SP_CFG_128x128: return launch_conv<ConvM>(g, 0, g.P, 1, nullptr, st);
@@ -394,8 +601,12 @@ extern "C" int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, 
         case T2SP_CFG_AUTO: break;
         default: return T2SP_ERR_SHAPE;
     }
-    // Automatic choice: the stages of plan_conv; a split stage without room for its planes runs unsplit.
+    // Automatic choice: the one-launch 16 x 16 form when its estimate is the lower one (small and
+    // middle-sized convolutions with a reduction long enough to amortise its set-up; measured from
+    // 7 x 7 to 56 x 56 maps, 64 to 1024 channels), else the stages of plan_conv; a split stage
+    // without room for its planes runs unsplit.
     const ConvPlan plan = plan_conv(CO, g.P, g.KRED);
+    if (d16_ok && conv_prefers_d16(CO, g.P, g.KRED, plan)) return launch_conv_d16(g, st);
     for (int i = 0; i < plan.n; i++) {
         const ConvStage &sg = plan.st[i];
         const bool split = sg.splits > 1 && workspace && workspace_bytes >= plan.scratch_bytes;

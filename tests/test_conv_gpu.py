@@ -58,6 +58,39 @@ def test_ragged_shapes(oracle, shape):
     assert rel_fro(run(I, W), oracle.conv(I, W))[0] <= TOL
 
 
+@pytest.mark.parametrize("shape", [(3, 16, 70, 9, 12), (1, 32, 40, 7, 7), (2, 48, 16, 14, 14), (5, 64, 100, 8, 20), (2, 16, 200, 30, 30),
+                                   (1, 112, 24, 5, 6), (4, 32, 33, 4, 4)])
+def test_one_launch_16x16_form_exact(shape):
+    """The direct kernel on 16 x 16 MFMA tiles, forced: reductions of 9 to 63 steps of 16 split over four
+    waves (some waves get none), channel counts that leave ragged tiles of every row-block count, maps whose
+    rows are not multiples of 4 (overlapping last group), pixel counts that end inside a tile.  Integer data:
+    exact against the float64 convolution; the same bits twice; and the automatic choice gives the same
+    values whichever kernel it takes."""
+    import torch
+    N, CI, CO, OH, OW = shape
+    g = torch.Generator().manual_seed(CI * CO)
+    I = torch.randint(-2, 3, (N, CI, OH + 2, OW + 2), generator=g).float().numpy()
+    W = torch.randint(-2, 3, (CO, CI, 3, 3), generator=g).float().numpy()
+    want = torch.nn.functional.conv2d(torch.from_numpy(I).double(), torch.from_numpy(W).double()).numpy()
+    got = run(I, W, cfg=6)
+    assert (got == want).all()
+    assert (run(I, W, cfg=6) == got).all()
+    assert (run(I, W, cfg=0) == want).all()
+    # 1 x 1 kernels: the reduction is the channels alone
+    W1 = torch.randint(-2, 3, (CO, CI, 1, 1), generator=g).float().numpy()
+    want1 = torch.nn.functional.conv2d(torch.from_numpy(I).double(), torch.from_numpy(W1).double()).numpy()
+    assert (run(I, W1, cfg=6) == want1).all()
+
+
+def test_one_launch_16x16_form_refuses_what_it_cannot_address():
+    """A reduction that is not a whole number of steps of 16 has no 16 x 16 form: forcing it is an error,
+    the automatic choice takes another kernel."""
+    I, W = np.ones((1, 5, 8, 8), np.float32), np.ones((8, 5, 3, 3), np.float32)
+    with pytest.raises(t2sp_amd.T2spError):
+        run(I, W, cfg=6)
+    assert (run(I, W) == 45.0).all()
+
+
 @pytest.mark.parametrize("CI", [4, 8, 12, 20, 36, 68])
 @pytest.mark.parametrize("cfg", [0, 1, 2, 3])
 def test_reduction_tails_guarded_only_in_the_last_tiles_exact(cfg, CI):

@@ -99,6 +99,30 @@ def test_conv_never_leaves_half_of_a_cu_idle_when_a_split_fills_it(lib, cus):
             assert per_cu * waves[cfg] >= 4, (cus, CO, P, KRED, cfg, splits)
 
 
+def test_conv_takes_the_one_launch_form_for_small_convolutions_only(lib):
+    """On the full machine: the benchmark convolution and other many-round shapes keep the staged LDS-tile
+    plan, small and middle-sized ones with a reduction of at least 288 rows take the 16 x 16 form, short
+    reductions (1 x 1 kernels over 64 channels) never do; its tiles cover CO with at most 6 row blocks."""
+    lib.t2sp_set_machine(256, 8)
+    lib.t2sp_conv2d_direct16_plan.argtypes = [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_void_p]
+    out, times = (ctypes.c_int * 4)(), (ctypes.c_double * 2)()
+
+    def takes(N, CI, CO, OH, OW, KH=3):
+        P, K = N * OH * ((OW + 3) // 4 * 4), CI * KH * KH
+        r = lib.t2sp_conv2d_direct16_plan(CO, P, K, out, times)
+        mb, rpt, tm, tn = out
+        assert 1 <= mb <= 6 and rpt <= 16 * mb and tm * rpt >= CO and tn * 64 >= P
+        assert times[0] > 0 and times[1] > 0
+        return r
+
+    assert not takes(64, 256, 256, 56, 56)
+    assert not takes(64, 512, 512, 28, 28)
+    assert not takes(64, 64, 256, 56, 56, 1)
+    for shape in ((32, 64, 64, 30, 30), (8, 256, 256, 14, 14), (16, 144, 144, 28, 28), (4, 128, 128, 28, 28), (1, 256, 256, 56, 56)):
+        assert takes(*shape), shape
+    lib.t2sp_set_machine(0, 0)
+
+
 @pytest.mark.parametrize("cus", CUS)
 def test_syrk_splits_only_a_small_last_round(lib, cus):
     lib.t2sp_set_machine(cus, 0)
