@@ -291,9 +291,18 @@ __device__ long long g_d16_trace[4096 * 8 * 8];
 #else
 #define T2SP_TRACE_STAMP(i)
 #endif
+// What the loop of the 16 x 16 form needs of the arguments.  The kernel takes these as leading
+// scalar parameters, which the dispatcher preloads into scalar registers before the first wave
+// starts (the build sets -amdgpu-kernarg-preload-count): a wave that has to fetch them from the
+// argument buffer, which lives in host memory, waits about a microsecond before it can issue its
+// first load, and for a product of 14 us that wait is not hidden by anything.
+struct GemmHot {
+    const float *A, *B;
+    int M, N, lda, ldb;
+};
 // Row blocks [mb0, mb0 + MBW) of the tile over steps [s0, s0 + nsteps) of 16 k, partial result to red_kq.
 template <int MBW, int NB>
-__device__ __forceinline__ void sgemm_d16_wave(const GemmArgs &g, int mb0, int m0, int n0, int s0, int nsteps, int steps,
+__device__ __forceinline__ void sgemm_d16_wave(const GemmHot &g, int mb0, int m0, int n0, int s0, int nsteps, int steps,
                                                v4f *red_kq) {
     typedef typename VecOf<NB>::type vnb;
     constexpr int R = GEMM_D16_RING;
@@ -379,24 +388,27 @@ __device__ __forceinline__ void sgemm_d16_wave(const GemmArgs &g, int mb0, int m
 }
 
 template <int MB, int NB>
-__global__ void __launch_bounds__(GEMM_D16_WAVES * 64) sgemm_direct16_kernel(const GemmArgs g, int rows_per_tile) {
+__global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
+    sgemm_direct16_kernel(const float *A, const float *B, int M, int N, int K, int lda, int ldb, int tiles_m, int rows_per_tile,
+                          const GemmArgs g) {
     typedef typename VecOf<NB>::type vnb;
     constexpr int NW = GEMM_D16_WAVES;
     extern __shared__ __align__(16) float smem[];
     v4f *red = reinterpret_cast<v4f *>(smem);            // [wave][mb][nb][lane]
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
-    const int tm = blockIdx.x % g.tiles_m, tn = blockIdx.x / g.tiles_m;
+    const int tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
     const int m0 = tm * rows_per_tile, n0 = tn * 16 * NB;
-    const int m_end = min(m0 + rows_per_tile, g.M);
-    const int steps = g.K >> 4;
+    const int m_end = min(m0 + rows_per_tile, M);
+    const int steps = K >> 4;
     const int s0 = (int)((int64_t)steps * wave / NW), s1 = (int)((int64_t)steps * (wave + 1) / NW);
-    sgemm_d16_wave<MB, NB>(g, 0, m0, n0, s0, s1 - s0, steps, red + wave * MB * NB * 64);
+    const GemmHot hot{A, B, M, N, lda, ldb};
+    sgemm_d16_wave<MB, NB>(hot, 0, m0, n0, s0, s1 - s0, steps, red + wave * MB * NB * 64);
     __syncthreads();
     T2SP_TRACE_STAMP(5)
     // sum the partial tiles of the waves in wave order
     const int col = n0 + NB * li;
-    const bool col_ok = col + NB <= g.N;
+    const bool col_ok = col + NB <= N;
     for (int mb = wave; mb < MB; mb += NW) {
         v4f sum[NB];
 #pragma unroll
@@ -693,7 +705,8 @@ static int launch_d16_t(GemmArgs g, const GemmD16Plan &p, hipStream_t stream) {
     auto kern = sgemm_direct16_kernel<MB, NB>;
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(GEMM_D16_WAVES * 64), smem, stream, g, p.rows_per_tile);
+    hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(GEMM_D16_WAVES * 64), smem, stream, g.A, g.B, g.M, g.N, g.K,
+                       (int)g.lda, (int)g.ldb, p.tiles_m, p.rows_per_tile, g);
     return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
 }
 
