@@ -82,6 +82,32 @@ def test_one_launch_16x16_form_exact(shape):
     assert (run(I, W1, cfg=6) == want1).all()
 
 
+def test_one_launch_16x16_form_on_views_of_larger_buffers():
+    """The thin layer with the 16 x 16 form forced on strided operands: the input a window of a larger
+    tensor (rows, channels and images further apart than their extents, first element not 16-byte aligned),
+    the output a window too (canary frame untouched), weights with padded rows.  Integer data: exact."""
+    import ctypes
+    import torch
+    L = t2sp_amd.lib()
+    N, CI, CO, OH, OW = 3, 32, 40, 9, 13
+    g = torch.Generator().manual_seed(7)
+    big_i = torch.randint(-2, 3, (N + 1, CI + 2, OH + 5, OW + 9), generator=g).float().cuda()
+    I = big_i[1:, 1:CI + 1, 2:OH + 4, 3:OW + 5]
+    big_w = torch.randint(-2, 3, (CO, CI * 9 + 4), generator=g).float().cuda()
+    W = big_w[:, :CI * 9].view(CO, CI * 9).as_strided((CO, CI, 3, 3), (CI * 9 + 4, 9, 3, 1))
+    frame = torch.full((N, CO + 1, OH + 2, OW + 3), 7.0, device="cuda")
+    O = frame[:, 1:, 1:OH + 1, 2:OW + 2]
+    i64 = ctypes.c_int64
+    si, sw, so = ((i64 * 4)(*t.stride()) for t in (I, W, O))
+    rc = L.t2sp_conv2d_f32(I.data_ptr(), W.data_ptr(), O.data_ptr(), N, CI, CO, OH, OW, 3, 3, si, sw, so, 6, None, 0, None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    want = torch.nn.functional.conv2d(I.double(), W.double())
+    assert torch.equal(O.double(), want)
+    O.fill_(7.0)
+    assert (frame == 7.0).all()
+
+
 def test_one_launch_16x16_form_refuses_what_it_cannot_address():
     """A reduction that is not a whole number of steps of 16 has no 16 x 16 form: forcing it is an error,
     the automatic choice takes another kernel."""
