@@ -412,6 +412,7 @@ struct ConvPlan {
     size_t scratch_bytes;
     double time;                // estimated seconds (MFMA time at the sustained rate + planes + launches)
 };
+constexpr int CONV_SHORT_KRED = 288;        // reductions up to this length take one launch of small tiles
 constexpr double CONV_SUSTAINED = 0.92;     // of the MFMA peak, what the 256 x 256 tile reaches on the benchmark shape
 static ConvPlan plan_conv(int CO, int P, int KRED) {
     const int CUS = machine().cus;
@@ -426,6 +427,18 @@ static ConvPlan plan_conv(int CO, int P, int KRED) {
 
     ConvPlan p{};
     int p0 = 0;
+    // Short reductions (1 x 1 kernels over up to 288 channels, 3 x 3 over up to 32): a tile is mostly its
+    // loads and its stores, rounds are short and several small workgroups share a CU, so one launch of
+    // small tiles flows better than rounds of large ones followed by a rest (measured at 64 to 512
+    // output channels: 8 to 25 % faster).
+    if (KRED <= CONV_SHORT_KRED) {
+        const Cand &c = CO <= 64 ? all[2] : all[1];
+        p.st[p.n++] = ConvStage{c.cfg, 0, P, 1};
+        const int64_t per_round = (int64_t)CUS * (c.bm == 64 ? 2 : 1);
+        p.time = (double)((tiles(c, 0) + per_round - 1) / per_round) * (c.bm == 64 ? 2.0 : 1.0) * 2.0 * c.bm * c.bn * KRED /
+                     (614e9 * c.eff * CONV_SUSTAINED) + 3e-6;
+        return p;
+    }
     // whole rounds: the best tile size, then 128 x 128 if that is smaller
     for (int i = best; i < 3 && p0 < P; i++) {
         if (i != best && all[i].cfg != T2SP_CFG_128x128) break;
@@ -474,10 +487,10 @@ static ConvPlan plan_conv(int CO, int P, int KRED) {
 }
 
 // Short reductions (1 x 1 kernels over few channels) leave the 16 x 16 form nothing to amortise its
-// set-up and its narrow stores with; from 288 reduction rows on (3 x 3 over 32 channels) the estimates decide.
+// set-up and its narrow stores with; above 288 reduction rows (3 x 3 over 32 channels) the estimates decide.
 static bool conv_prefers_d16(int CO, int P, int KRED, const ConvPlan &lds) {
     // within 3 % the staged plan is taken: over many rounds it tends to beat its estimate, the 16 x 16 form not
-    return KRED >= 288 && plan_conv_d16(CO, P, KRED).time < 0.97 * lds.time;
+    return KRED > CONV_SHORT_KRED && plan_conv_d16(CO, P, KRED).time < 0.97 * lds.time;
 }
 
 using ConvL = TileCfg<256, 256, 16, 4, 2, STYLE_RC>;
