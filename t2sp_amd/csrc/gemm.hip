@@ -440,6 +440,101 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     }
     T2SP_TRACE_STAMP(6)
 }
+// The same form for B stored transposed (N x K, k contiguous: C = A * B^T, the layout of a weight
+// matrix): both operands are read as A is above, 4 consecutive k of one row (of A) or column (of
+// the product) per lane and 128-bit load, element j feeding MFMA j; accumulator block nb holds the
+// 16 adjacent columns n0 + 16 nb .., so a lane ends with four rows of one column per block and
+// stores them one by one (16 lanes side by side: 64 contiguous bytes per row).
+template <int MB, int NB>
+__global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
+    sgemm_direct16_bt_kernel(const float *A, const float *B, int M, int N, int K, int lda, int ldb, int tiles_m, int rows_per_tile,
+                             const GemmArgs g) {
+    constexpr int NW = GEMM_D16_WAVES, R = GEMM_D16_RING;
+    extern __shared__ __align__(16) float smem[];
+    v4f *red = reinterpret_cast<v4f *>(smem);            // [wave][mb][nb][lane]
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
+    const int tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
+    const int m0 = tm * rows_per_tile, n0 = tn * 16 * NB;
+    const int m_end = min(m0 + rows_per_tile, M);
+    const int steps = K >> 4;
+    const int s0 = (int)((int64_t)steps * wave / NW), s1 = (int)((int64_t)steps * (wave + 1) / NW);
+    const int nsteps = s1 - s0;
+
+    uint32_t a_off[MB], b_off[NB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) a_off[mb] = 4u * (uint32_t)(min(m0 + 16 * mb + li, M - 1) * lda + 4 * lq);
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) b_off[nb] = 4u * (uint32_t)(min(n0 + 16 * nb + li, N - 1) * ldb + 4 * lq);
+    const char *a_base = reinterpret_cast<const char *>(A + 16 * s0);
+    const char *b_base = reinterpret_cast<const char *>(B + 16 * s0);
+    int issued = 0;
+
+    v4f ra[R][MB], rb[R][NB];
+#define T2SP_GEMM_D16BT_ISSUE(d)                                                                    \
+    {                                                                                               \
+        const uint32_t ko = 64u * (uint32_t)min(issued, steps - 1 - s0);                            \
+        issued++;                                                                                   \
+        _Pragma("unroll") for (int nb = 0; nb < NB; nb++)                                           \
+            rb[d][nb] = *reinterpret_cast<const v4f *>(b_base + (b_off[nb] + ko));                  \
+        _Pragma("unroll") for (int mb = 0; mb < MB; mb++)                                           \
+            ra[d][mb] = *reinterpret_cast<const v4f *>(a_base + (a_off[mb] + ko));                  \
+    }
+#define T2SP_GEMM_D16BT_MMA(d)                                                                      \
+    _Pragma("unroll") for (int j = 0; j < 4; j++)                                                   \
+        _Pragma("unroll") for (int mb = 0; mb < MB; mb++)                                           \
+            _Pragma("unroll") for (int nb = 0; nb < NB; nb++)                                       \
+                acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[d][mb][j], rb[d][nb][j], acc[mb][nb], 0, 0, 0);
+    v4f acc[MB][NB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) acc[mb][nb] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int d = 0; d < R - 1; d++) {
+        T2SP_GEMM_D16BT_ISSUE(d)
+        __builtin_amdgcn_sched_barrier(0);   // keep the sets in program order: waits count loads
+    }
+    const int main_iters = nsteps > 0 ? (nsteps - 1) / R : 0;
+    const int rem = nsteps - main_iters * R;
+    for (int it = 0; it < main_iters; it++) {
+#pragma unroll
+        for (int d = 0; d < R; d++) {
+            T2SP_GEMM_D16BT_ISSUE((d + R - 1) % R)
+            T2SP_GEMM_D16BT_MMA(d)
+            T2SP_INTERLEAVE(SG_VMEM_READ, MB + NB, (4 * MB * NB) / (MB + NB))
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    T2SP_GEMM_D16BT_ISSUE(R - 1)
+#pragma unroll
+    for (int d = 0; d < R; d++) {
+        if (d < rem) { T2SP_GEMM_D16BT_MMA(d) }
+    }
+#undef T2SP_GEMM_D16BT_ISSUE
+#undef T2SP_GEMM_D16BT_MMA
+
+    v4f *mine = red + wave * MB * NB * 64 + lane;
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) mine[(mb * NB + nb) * 64] = acc[mb][nb];
+    __syncthreads();
+    for (int pr = wave; pr < MB * NB; pr += NW) {        // sum the partial blocks of the waves in wave order
+        const v4f *src = red + pr * 64 + lane;
+        v4f sum = src[0];
+#pragma unroll
+        for (int wv = 1; wv < NW; wv++) sum += src[wv * MB * NB * 64];
+        const int mb = pr / NB, nb = pr - mb * NB;
+        const int col = n0 + 16 * nb + li;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int row = m0 + 16 * mb + 4 * lq + r;
+            if (row < m_end && col < N) gemm_store1(g, row, col, sum[r]);
+        }
+    }
+}
+
 #ifdef T2SP_D16_TRACE
 }  // namespace t2sp
 extern "C" int t2sp_d16_trace(long long *host, int n) {
@@ -720,6 +815,50 @@ static int launch_d16(const GemmArgs &g, hipStream_t stream) {
     return T2SP_ERR_SHAPE;
 }
 
+// Tile of the 16 x 16 form for B stored transposed: up to 8 row blocks by 2 to 4 column blocks of 16.
+static GemmD16Plan plan_gemm_d16_bt(int M, int N) {
+    const int cus = machine().cus;
+    GemmD16Plan best{};
+    best.cost = 1e300;
+    for (int nb = 2; nb <= 4; nb++)
+        for (int mb = 2; mb <= 8; mb++) {
+            if (mb * nb > 24) continue;
+            const int tiles_m = (M + 16 * mb - 1) / (16 * mb), tiles_n = (N + 16 * nb - 1) / (16 * nb);
+            const int rpt = (M + tiles_m - 1) / tiles_m;
+            const int64_t tiles = (int64_t)tiles_m * tiles_n;
+            const double loads_per_mfma = (double)(mb + nb) / (4.0 * mb * nb);
+            const double cost = (double)((tiles + cus - 1) / cus) * (16.0 * mb) * (16.0 * nb) * (1.0 + 1.5 * loads_per_mfma);
+            if (cost < best.cost) best = GemmD16Plan{mb, nb, rpt, tiles_m, tiles_n, cost};
+        }
+    return best;
+}
+static bool gemm_d16_bt_ok(const GemmArgs &g) {
+    return g.K % 16 == 0 && g.lda % 4 == 0 && g.ldb % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
+           (int64_t)g.M * g.lda < (1 << 30) && (int64_t)g.N * g.ldb < (1 << 30);
+}
+template <int MB, int NB>
+static int launch_d16_bt_t(GemmArgs g, const GemmD16Plan &p, hipStream_t stream) {
+    g.tiles_m = p.tiles_m;
+    g.tiles_n = p.tiles_n;
+    const size_t smem = (size_t)GEMM_D16_WAVES * MB * NB * 64 * sizeof(v4f);
+    auto kern = sgemm_direct16_bt_kernel<MB, NB>;
+    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+        return T2SP_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(GEMM_D16_WAVES * 64), smem, stream, g.A, g.B, g.M, g.N, g.K,
+                       (int)g.lda, (int)g.ldb, p.tiles_m, p.rows_per_tile, g);
+    return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+}
+static int launch_d16_bt(const GemmArgs &g, hipStream_t stream) {
+    const GemmD16Plan p = plan_gemm_d16_bt(g.M, g.N);
+#define T2SP_D16_CASE(MBV, NBV) if (p.mb == MBV && p.nb == NBV) return launch_d16_bt_t<MBV, NBV>(g, p, stream);
+    T2SP_D16_CASE(2, 2) T2SP_D16_CASE(3, 2) T2SP_D16_CASE(4, 2) T2SP_D16_CASE(5, 2) T2SP_D16_CASE(6, 2)
+    T2SP_D16_CASE(7, 2) T2SP_D16_CASE(8, 2) T2SP_D16_CASE(2, 3) T2SP_D16_CASE(3, 3) T2SP_D16_CASE(4, 3)
+    T2SP_D16_CASE(5, 3) T2SP_D16_CASE(6, 3) T2SP_D16_CASE(7, 3) T2SP_D16_CASE(8, 3) T2SP_D16_CASE(2, 4)
+    T2SP_D16_CASE(3, 4) T2SP_D16_CASE(4, 4) T2SP_D16_CASE(5, 4) T2SP_D16_CASE(6, 4)
+#undef T2SP_D16_CASE
+    return T2SP_ERR_SHAPE;
+}
+
 static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *workspace = nullptr,
                     size_t workspace_bytes = 0) {
     if (g.M <= 0 || g.N <= 0 || g.K <= 0) return T2SP_ERR_SHAPE;
@@ -743,9 +882,11 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         if (sp < 2 || !workspace || workspace_bytes < need) sp = 1;
         return launch<GemmMA, false>(g, stream, sp, workspace);
     }
-    if (cfg == T2SP_CFG_DIRECT16)
-        return (!bt && gemm_d16_ok(g)) ? launch_d16(g, stream) : T2SP_ERR_SHAPE;
-    if (cfg == T2SP_CFG_AUTO && !bt && gemm_d16_ok(g)) {
+    if (cfg == T2SP_CFG_DIRECT16) {
+        if (bt) return gemm_d16_bt_ok(g) ? launch_d16_bt(g, stream) : T2SP_ERR_SHAPE;
+        return gemm_d16_ok(g) ? launch_d16(g, stream) : T2SP_ERR_SHAPE;
+    }
+    if (cfg == T2SP_CFG_AUTO && (bt ? gemm_d16_bt_ok(g) : gemm_d16_ok(g))) {
         // Measured from 256^2 x 8192 to 3072^2 x 1024: the 16 x 16 form wins whenever 256 x 256 tiles
         // would not fill the chip, except where 128 x 128 tiles do and the reduction is long enough to
         // amortise their prologue, and for tiny outputs with a long reduction (too few tiles even at
@@ -758,9 +899,12 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         const double fill128 = (double)g.M * g.N / ((double)t128 * 16384.0);
         const int cus = machine().cus;
         const bool big_tiles = t256 >= cus * 25 / 32 && fill256 >= 0.6;
-        const bool tiled_better = t128 >= 2 * cus - cus / 16 && g.K >= 2048 && fill128 >= 0.6;   // 2304^3, 2560^3: the 16 x 16 form is 7-11 % ahead
+        // 2304^3, 2560^3: the 16 x 16 form is 7-11 % ahead.  With B transposed it stores element by element and
+        // whole rounds of 128 x 128 tiles are 4-10 % ahead of it (1024 x 4096 x 512, 2048^3, 4096 x 1024 x 1024).
+        const bool tiled_better = (t128 >= 2 * cus - cus / 16 && g.K >= 2048 && fill128 >= 0.6) ||
+                                  (bt && t128 % cus == 0 && fill128 >= 0.9);
         const bool too_few = (int64_t)p.tiles_m * p.tiles_n < cus / 2 && g.K >= 4096;
-        if (!big_tiles && !tiled_better && !too_few && g.K >= 64) return launch_d16(g, stream);
+        if (!big_tiles && !tiled_better && !too_few && g.K >= 64) return bt ? launch_d16_bt(g, stream) : launch_d16(g, stream);
     }
     if ((cfg == T2SP_CFG_AUTO || cfg == T2SP_CFG_DIRECT) && !bt && !g.scale && !g.tiled &&
         g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && gemm_direct_ok(g, cfg == T2SP_CFG_DIRECT))

@@ -140,6 +140,32 @@ def test_reduction_tails_and_ragged_tiles_exact(K, MN):
         assert (frame == 7.0).all()
 
 
+@pytest.mark.parametrize("shape", [(512, 512, 512), (1000, 260, 96), (260, 1000, 64), (1536, 1100, 176), (33, 47, 80), (2052, 1028, 128)])
+def test_transposed_b_one_launch_form_exact(shape):
+    """B stored N x K (the layout of a weight matrix): small and middle-sized products take the one-launch
+    16 x 16 form, forced here and through the automatic choice; ragged rows and columns (any N), alpha, beta
+    and C in place, a canary frame around C.  Integer data: exact."""
+    import torch
+    M, N, K = shape
+    L = t2sp_amd.lib()
+    g = torch.Generator().manual_seed(M * 3 + N)
+    A = torch.randint(-2, 3, (M, K), generator=g).float().cuda()
+    Bt = torch.randint(-2, 3, (N, K), generator=g).float().cuda()
+    C0 = torch.randint(-4, 5, (M, N), generator=g).float().cuda()
+    want = 2.0 * (A.double() @ Bt.double().t()) - 3.0 * C0.double()
+    for cfg in (6, 0):
+        frame = torch.full((M + 2, N + 8), 7.0, device="cuda")
+        C = frame[1:M + 1, 4:N + 4]
+        C.copy_(C0)
+        rc = L.t2sp_sgemm_ex_f32(0, 1, M, N, K, 2.0, A.data_ptr(), K, Bt.data_ptr(), K, -3.0, C.data_ptr(), N + 8, C.data_ptr(), N + 8,
+                                 cfg, None, 0, None)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert torch.equal(C.double(), want)
+        C.fill_(7.0)
+        assert (frame == 7.0).all()
+
+
 def test_tiled_output_and_in_place_device(oracle):
     import torch
     M, N, K = 128, 96, 64
