@@ -62,7 +62,8 @@ int t2sp_sgemm_f32_tiled(const float *A, const float *B, float *C, int M, int N,
  * transb non-zero: A stored K x M, B stored N x K).  Cin may be NULL (beta is then ignored) or
  * equal to C (in place).  Every form but A^T * B^T reads both operands as they lie: B^T through
  * k-contiguous tiles, A^T (with M, N and the leading dimensions multiples of 4 and 16-byte
- * aligned pointers) through row-contiguous ones, for any K.  Otherwise a transposed A is first
+ * aligned pointers) through row-contiguous ones, for any K; small and middle-sized products of
+ * each form have a one-launch kernel of their own (T2SP_CFG_DIRECT16 forces it).  Otherwise a transposed A is first
  * re-laid into `workspace`, which is required then; the rest of t2sp_sgemm_ex_workspace_bytes is
  * optional room for the planes of a split reduction, as in t2sp_sgemm_f32.  Device side of the reference's 8-argument
  * gemm(opa, opb, alpha, beta, A, B, C, O) pipeline behind its BLAS wrapper

@@ -535,6 +535,117 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     }
 }
 
+// And for A stored transposed (K x M, the rows of the product contiguous: C = A^T * B): both
+// operands are read as B is in the first form, four adjacent rows (of A^T: four adjacent m) or
+// columns of one k-row per lane and 128-bit load, so row block mb holds the rows congruent to mb
+// modulo 4 and column block nb the columns congruent to nb modulo 4 of the 64 x 64 tile; a lane
+// ends with four adjacent columns of each of its rows and stores 128 bits at a time.
+template <int MB>
+__global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
+    sgemm_direct16_at_kernel(const float *A, const float *B, int M, int N, int K, int lda, int ldb, int tiles_m, const GemmArgs g) {
+    constexpr int NW = GEMM_D16_WAVES, R = GEMM_D16_RING, NB = 4;
+    extern __shared__ __align__(16) float smem[];
+    v4f *red = reinterpret_cast<v4f *>(smem);            // [wave][mb][nb][lane]
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
+    const int tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
+    const int m0 = tm * 16 * MB, n0 = tn * 64;
+    const int steps = K >> 4;
+    const int s0 = (int)((int64_t)steps * wave / NW), s1 = (int)((int64_t)steps * (wave + 1) / NW);
+    const int nsteps = s1 - s0;
+
+    // a lane's MB adjacent rows (MB = 4: one 128-bit load; MB = 2: 64 bits) and 4 adjacent columns
+    typedef typename VecOf<MB>::type vmb;
+    const int row = m0 + MB * li, col = n0 + 4 * li;
+    const bool row_ok = row + MB <= M, col_ok = col + 4 <= N;
+    uint32_t a_off[4], b_off[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        a_off[j] = 4u * (uint32_t)((4 * lq + j) * lda + (row_ok ? row : 0));
+        b_off[j] = 4u * (uint32_t)((4 * lq + j) * ldb + (col_ok ? col : 0));
+    }
+    const char *a_base = reinterpret_cast<const char *>(A + (int64_t)16 * s0 * lda);
+    const char *b_base = reinterpret_cast<const char *>(B + (int64_t)16 * s0 * ldb);
+    const uint32_t a_step = 64u * (uint32_t)lda, b_step = 64u * (uint32_t)ldb;
+    int issued = 0;
+
+    vmb ra[R][4];
+    v4f rb[R][4];
+#define T2SP_GEMM_D16AT_ISSUE(d)                                                                    \
+    {                                                                                               \
+        const uint32_t st = (uint32_t)min(issued, steps - 1 - s0);                                  \
+        issued++;                                                                                   \
+        _Pragma("unroll") for (int j = 0; j < 4; j++)                                               \
+            rb[d][j] = *reinterpret_cast<const v4f *>(b_base + (b_off[j] + st * b_step));           \
+        _Pragma("unroll") for (int j = 0; j < 4; j++)                                               \
+            ra[d][j] = *reinterpret_cast<const vmb *>(a_base + (a_off[j] + st * a_step));           \
+    }
+#define T2SP_GEMM_D16AT_MMA(d)                                                                      \
+    _Pragma("unroll") for (int j = 0; j < 4; j++)                                                   \
+        _Pragma("unroll") for (int mb = 0; mb < MB; mb++)                                           \
+            _Pragma("unroll") for (int nb = 0; nb < NB; nb++)                                       \
+                acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[d][j][mb], rb[d][j][nb], acc[mb][nb], 0, 0, 0);
+    v4f acc[MB][NB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) acc[mb][nb] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int d = 0; d < R - 1; d++) {
+        T2SP_GEMM_D16AT_ISSUE(d)
+        __builtin_amdgcn_sched_barrier(0);   // keep the sets in program order: waits count loads
+    }
+    const int main_iters = nsteps > 0 ? (nsteps - 1) / R : 0;
+    const int rem = nsteps - main_iters * R;
+    for (int it = 0; it < main_iters; it++) {
+#pragma unroll
+        for (int d = 0; d < R; d++) {
+            T2SP_GEMM_D16AT_ISSUE((d + R - 1) % R)
+            T2SP_GEMM_D16AT_MMA(d)
+            T2SP_INTERLEAVE(SG_VMEM_READ, 8, (4 * MB * NB) / 8)
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    T2SP_GEMM_D16AT_ISSUE(R - 1)
+#pragma unroll
+    for (int d = 0; d < R; d++) {
+        if (d < rem) { T2SP_GEMM_D16AT_MMA(d) }
+    }
+#undef T2SP_GEMM_D16AT_ISSUE
+#undef T2SP_GEMM_D16AT_MMA
+
+    v4f *mine = red + wave * MB * NB * 64 + lane;
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) mine[(mb * NB + nb) * 64] = acc[mb][nb];
+    __syncthreads();
+    // sum the partial tiles of the waves in wave order; block (mb, nb), register r of lane (li, lq) is
+    // row m0 + MB * (4 lq + r) + mb, column n0 + 4 li + nb
+    for (int mb = wave; mb < MB; mb += NW) {
+        v4f sum[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+            const v4f *src = red + (mb * NB + nb) * 64 + lane;
+            sum[nb] = src[0];
+#pragma unroll
+            for (int wv = 1; wv < NW; wv++) sum[nb] += src[wv * MB * NB * 64];
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int orow = m0 + MB * (4 * lq + r) + mb;
+            v4f out = {sum[0][r], sum[1][r], sum[2][r], sum[3][r]};
+            if (orow < M && col_ok) {
+                if (g.scale) {
+                    out = out * g.alpha;
+                    if (g.beta != 0.f) out += *reinterpret_cast<const v4f *>(g.Cin + (int64_t)orow * g.ldcin + col) * g.beta;
+                }
+                *reinterpret_cast<v4f *>(g.C + (int64_t)orow * g.ldc + col) = out;
+            }
+        }
+    }
+}
+
 #ifdef T2SP_D16_TRACE
 }  // namespace t2sp
 extern "C" int t2sp_d16_trace(long long *host, int n) {
@@ -859,13 +970,45 @@ static int launch_d16_bt(const GemmArgs &g, hipStream_t stream) {
     return T2SP_ERR_SHAPE;
 }
 
+// The 16 x 16 form for A stored transposed: tiles of 64 (or 32) rows by 64 columns.
+static bool gemm_d16_at_ok(const GemmArgs &g) {
+    return g.K % 16 == 0 && g.M % 4 == 0 && g.N % 4 == 0 && g.lda % 4 == 0 && g.ldb % 4 == 0 && g.ldc % 4 == 0 && !g.tiled &&
+           ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) && ((uintptr_t)g.C % 16 == 0) &&
+           (int64_t)g.K * g.lda < (1 << 30) && (int64_t)g.K * g.ldb < (1 << 30) &&
+           (!g.scale || (g.ldcin % 4 == 0 && (uintptr_t)g.Cin % 16 == 0));
+}
+static int launch_d16_at(GemmArgs g, hipStream_t stream) {
+    const int cus = machine().cus;
+    const int64_t t64 = (int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64), t32 = (int64_t)((g.M + 31) / 32) * ((g.N + 63) / 64);
+    // 32-row tiles when they fill the CUs and 64-row tiles would leave most of them idle
+    const bool narrow = t64 < cus / 2 && t32 <= cus;
+    const int mb = narrow ? 2 : 4;
+    g.tiles_m = (g.M + 16 * mb - 1) / (16 * mb);
+    g.tiles_n = (g.N + 63) / 64;
+    const size_t smem = (size_t)GEMM_D16_WAVES * mb * 4 * 64 * sizeof(v4f);
+    auto kern = narrow ? sgemm_direct16_at_kernel<2> : sgemm_direct16_at_kernel<4>;
+    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+        return T2SP_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(GEMM_D16_WAVES * 64), smem, stream, g.A, g.B, g.M, g.N, g.K, (int)g.lda,
+                       (int)g.ldb, g.tiles_m, g);
+    return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+}
+
 static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *workspace = nullptr,
                     size_t workspace_bytes = 0) {
     if (g.M <= 0 || g.N <= 0 || g.K <= 0) return T2SP_ERR_SHAPE;
     if (g.at) {
         // A^T * B with both operands as they lie (the caller has checked the alignment the 128-bit
         // loads need).  Any K: k is the row index of both operands.
-        if (bt || cfg != T2SP_CFG_AUTO) return T2SP_ERR_SHAPE;
+        if (bt || (cfg != T2SP_CFG_AUTO && cfg != T2SP_CFG_DIRECT16)) return T2SP_ERR_SHAPE;
+        if (cfg == T2SP_CFG_DIRECT16) return gemm_d16_at_ok(g) ? launch_d16_at(g, stream) : T2SP_ERR_SHAPE;
+        {
+            // small and middle-sized products: the one-launch form, as for the other layouts
+            const int64_t t256 = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
+            const int64_t t64 = (int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64);
+            const int cus = machine().cus;
+            if (gemm_d16_at_ok(g) && t256 < cus * 25 / 32 && g.K >= 64 && !(t64 < cus / 8 && g.K >= 4096)) return launch_d16_at(g, stream);
+        }
         const GemmPlan p = plan_gemm(g.M, g.N, g.K);
         if (p.phased) {
             const bool phased = workspace && workspace_bytes >= p.scratch_bytes;
@@ -1055,7 +1198,7 @@ extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, fl
     auto aligned16 = [](const void *p) { return ((uintptr_t)p & 15) == 0; };
     // A stored K x M is taken as it lies when B is not transposed too and rows of all operands
     // can be read and written 128 bits at a time
-    const bool at_possible = transa && !transb && cfg == T2SP_CFG_AUTO && M % 4 == 0 && N % 4 == 0 && lda % 4 == 0 &&
+    const bool at_possible = transa && !transb && (cfg == T2SP_CFG_AUTO || cfg == T2SP_CFG_DIRECT16) && M % 4 == 0 && N % 4 == 0 && lda % 4 == 0 &&
                              ldb % 4 == 0 && ldc % 4 == 0 && aligned16(A) && aligned16(B) && aligned16(C) &&
                              (!Cin || (ldcin % 4 == 0 && aligned16(Cin)));
     // Products too small for rounds of 256 x 256 tiles run faster on the kernels that want k
@@ -1063,7 +1206,10 @@ extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, fl
     // route when the caller has given the room for it.
     const int64_t t256 = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
     const bool room = workspace && workspace_bytes >= (size_t)M * K * sizeof(float);
-    const bool native_at = at_possible && (t256 >= t2sp::machine().cus * 25 / 32 || !room);
+    // (now that the 16 x 16 form reads a transposed A as it lies, the re-laying route is only left for
+    // operands it cannot address)
+    const bool native_at = at_possible && (cfg == T2SP_CFG_AUTO || cfg == T2SP_CFG_DIRECT16);
+    (void)t256; (void)room;
     if (transa && !native_at) {
         // A is stored K x M: bring it to M x K first (the loaders of the other kernels want k contiguous in A)
         if (!workspace || workspace_bytes < (size_t)M * K * sizeof(float)) return T2SP_ERR_SHAPE;

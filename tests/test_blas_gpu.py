@@ -82,7 +82,9 @@ def test_partial_last_round_split_both_forms_of_b(oracle, shape):
 
 
 @pytest.mark.parametrize("shape", [(256, 256, 64), (128, 128, 37), (260, 132, 101), (516, 772, 5), (2304, 2052, 333),
-                                   (4096, 4352, 520), (4100, 4100, 70)])
+                                   (4096, 4352, 520), (4100, 4100, 70),
+                                   # reductions of whole steps of 16: the one-launch 16 x 16 form, 64-row and 32-row tiles
+                                   (260, 132, 96), (516, 772, 16), (2304, 2052, 336), (36, 68, 64), (512, 512, 256), (1028, 260, 1024)])
 def test_transposed_a_as_it_lies_without_workspace(shape):
     """A stored K x M (opa of blas-gemm.cpp:28-47) with no workspace: the row-contiguous loader reads
     it in place, any K, M and N ragged against the tiles.  Integer data, so every order of the sum
