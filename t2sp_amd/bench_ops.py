@@ -311,6 +311,44 @@ def launch_floor(torch):
     return {"us_per_launch": round(ms * 1e3, 3), "workload": "5000 back-to-back launches of a one-workgroup fill kernel"}
 
 
+def conv_small(torch, steps, warmup, peak):
+    """A convolution too small for rounds of LDS tiles (a 14 x 14 layer at batch 32): the one-launch 16 x 16 form."""
+    L = lib()
+    N, CI, CO, OH, OW = 32, 256, 256, 14, 14
+    I = ops.fill_uniform(torch.empty(N, CI, OH + 2, OW + 2, device="cuda"), 1)
+    W = ops.fill_uniform(torch.empty(CO, CI, 3, 3, device="cuda"), 2)
+    O = torch.empty(N, CO, OH, OW, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    si, sw, so = ((i64 * 4)(*t.stride()) for t in (I, W, O))
+
+    def launch():
+        rc = L.t2sp_conv2d_f32(I.data_ptr(), W.data_ptr(), O.data_ptr(), N, CI, CO, OH, OW, 3, 3, si, sw, so, 0, None, 0, s)
+        assert rc == 0, rc
+
+    ms = _time(torch, launch, max(steps, 100), max(warmup, 10))
+    flop = 2.0 * N * CO * OH * OW * CI * 9
+    return _entry(flop / ms / 1e9, peak, ms, workload="N=32 CI=CO=256 14x14 out 3x3 NCHW, no workspace")
+
+
+def sgemm_transposed_1024(torch, steps, warmup, peak, transa, transb):
+    """The BLAS form at 1024^3 with one operand stored transposed (B^T: the layout of a weight matrix), no workspace."""
+    L = lib()
+    n = 1024
+    A = ops.fill_uniform(torch.empty(n, n, device="cuda"), 1)
+    B = ops.fill_uniform(torch.empty(n, n, device="cuda"), 2)
+    C = torch.empty(n, n, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        rc = L.t2sp_sgemm_ex_f32(transa, transb, n, n, n, 1.0, A.data_ptr(), n, B.data_ptr(), n, 0.0, None, 0, C.data_ptr(), n, 0,
+                                 None, 0, s)
+        assert rc == 0, rc
+
+    ms = _time(torch, launch, max(steps, 200), max(warmup, 20))
+    return _entry(2.0 * n ** 3 / ms / 1e9, peak, ms,
+                  workload="C = %s * %s, M=N=K=1024, one launch" % ("A^T" if transa else "A", "B^T" if transb else "B"))
+
+
 def copy_rate(torch):
     """What a plain device-to-device copy of 256 MiB reaches on this box (torch's copy kernel; read + write
     bytes per second): the measured ceiling next to the nominal 8 TB/s that `frac_of_hbm_peak` of the three
@@ -336,6 +374,9 @@ def _run_all(torch, steps, warmup, peak, capsule_cfg=0, capsule_splits=0):
     return {"launch_floor": launch_floor(torch),
             "hbm_copy_rate": copy_rate(torch),
             "conv2d": conv_config3(torch, steps, warmup, peak),
+            "conv2d_n32_256ch_14x14": conv_small(torch, steps, warmup, peak),
+            "sgemm_1024_b_transposed": sgemm_transposed_1024(torch, steps, warmup, peak, 0, 1),
+            "sgemm_1024_a_transposed": sgemm_transposed_1024(torch, steps, warmup, peak, 1, 0),
             "capsule": capsule_config4(torch, steps, warmup, peak, capsule_cfg, capsule_splits),
             "mttkrp": mttkrp_config5(torch, steps, warmup, peak),
             "ssyrk_8192": ssyrk_case(torch, steps, warmup, peak, 8192, 8192, ""),
