@@ -236,7 +236,7 @@ __global__ void __launch_bounds__(CONV_D16_WAVES * 64) conv_direct16_kernel(cons
         for (int k = threadIdx.x; k < g.KRED; k += NW * 64) {
             const int ci = k / win, r = k - ci * win;
             const int kh = r / g.KW, kw = r - kh * g.KW;
-            tab[k] = 4 * (ci * g.si_c + kh * g.si_h + kw);
+            tab[k] = (int)(4u * (uint32_t)(ci * g.si_c + kh * g.si_h + kw));     // below 2^32 (checked on the host), used as unsigned
         }
     }
     __syncthreads();

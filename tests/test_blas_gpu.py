@@ -168,6 +168,35 @@ def test_transposed_b_one_launch_form_exact(shape):
         assert (frame == 7.0).all()
 
 
+@pytest.mark.parametrize("form", ["NN", "NT", "TN"])
+def test_one_launch_forms_byte_offsets_above_two_gib(form):
+    """Rows 56 MB apart (a leading dimension of 14 million) put the last rows of an operand more than 2^31
+    bytes from its start: the 32-bit lane offsets of the 16 x 16 forms must still reach them.  Integer data."""
+    import torch
+    L = t2sp_amd.lib()
+    M, N, K, ld = 64, 128, 64, 14_000_000
+    g = torch.Generator().manual_seed(11)
+    A = torch.randint(-2, 3, (M, K), generator=g).float().cuda()
+    B = torch.randint(-2, 3, (K, N), generator=g).float().cuda()
+    want = A.double() @ B.double()
+    big = torch.zeros(63 * ld + 128, device="cuda")               # 3.5 GB
+    transa, transb, a_ptr, lda, b_ptr, ldb = 0, 0, A.data_ptr(), K, B.data_ptr(), N
+    if form == "NN":      # A's rows far apart
+        view = big.as_strided((M, K), (ld, 1)); view.copy_(A); a_ptr, lda = view.data_ptr(), ld
+    elif form == "NT":    # B stored N x K with its rows far apart (only 64 of them fit the allocation)
+        N = 64
+        B = B[:, :N].contiguous(); want = A.double() @ B.double()
+        view = big.as_strided((N, K), (ld, 1)); view.copy_(B.t()); transb, b_ptr, ldb = 1, view.data_ptr(), ld
+    else:                 # A stored K x M with its k-rows far apart
+        view = big.as_strided((K, M), (ld, 1)); view.copy_(A.t()); transa, a_ptr, lda = 1, view.data_ptr(), ld
+    C = torch.full((M, N), float("nan"), device="cuda")
+    rc = L.t2sp_sgemm_ex_f32(transa, transb, M, N, K, 1.0, a_ptr, lda, b_ptr, ldb, 0.0, None, 0, C.data_ptr(), N, 6, None, 0, None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(C.double(), want)
+    del big
+
+
 def test_tiled_output_and_in_place_device(oracle):
     import torch
     M, N, K = 128, 96, 64

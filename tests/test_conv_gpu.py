@@ -108,6 +108,32 @@ def test_one_launch_16x16_form_on_views_of_larger_buffers():
     assert (frame == 7.0).all()
 
 
+def test_one_launch_16x16_form_byte_offsets_above_two_gib():
+    """Two images 3.6 GB apart inside one allocation: the kernel's 32-bit byte offsets reach past 2^31.
+    Integer data: exact."""
+    import ctypes
+    import torch
+    L = t2sp_amd.lib()
+    N, CI, CO, OH, OW = 2, 16, 32, 6, 8
+    gap = 900_000_000                                    # elements between the two images
+    per_image = CI * (OH + 2) * (OW + 2)
+    buf = torch.zeros(gap + per_image, device="cuda")
+    g = torch.Generator().manual_seed(3)
+    imgs = torch.randint(-2, 3, (N, CI, OH + 2, OW + 2), generator=g).float().cuda()
+    I = buf.as_strided((N, CI, OH + 2, OW + 2), (gap, (OH + 2) * (OW + 2), OW + 2, 1))
+    I.copy_(imgs)
+    W = torch.randint(-2, 3, (CO, CI, 3, 3), generator=g).float().cuda()
+    O = torch.full((N, CO, OH, OW), float("nan"), device="cuda")
+    i64 = ctypes.c_int64
+    si, sw, so = ((i64 * 4)(*t.stride()) for t in (I, W, O))
+    for cfg in (6, 0):
+        O.fill_(float("nan"))
+        assert L.t2sp_conv2d_f32(I.data_ptr(), W.data_ptr(), O.data_ptr(), N, CI, CO, OH, OW, 3, 3, si, sw, so, cfg, None, 0, None) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(O.double(), torch.nn.functional.conv2d(imgs.double(), W.double()))
+    del buf
+
+
 def test_one_launch_16x16_form_refuses_what_it_cannot_address():
     """A reduction that is not a whole number of steps of 16 has no 16 x 16 form: forcing it is an error,
     the automatic choice takes another kernel."""
