@@ -443,15 +443,14 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
 // The same form for B stored transposed (N x K, k contiguous: C = A * B^T, the layout of a weight
 // matrix): both operands are read as A is above, 4 consecutive k of one row (of A) or column (of
 // the product) per lane and 128-bit load, element j feeding MFMA j; accumulator block nb holds the
-// 16 adjacent columns n0 + 16 nb .., so a lane ends with four rows of one column per block and
-// stores them one by one (16 lanes side by side: 64 contiguous bytes per row).
+// 16 adjacent columns n0 + 16 nb ..; the exchange through LDS that sums the waves' partial tiles
+// also turns a lane's four rows of one column into four adjacent columns of one row.
 template <int MB, int NB>
 __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     sgemm_direct16_bt_kernel(const float *A, const float *B, int M, int N, int K, int lda, int ldb, int tiles_m, int rows_per_tile,
                              const GemmArgs g) {
     constexpr int NW = GEMM_D16_WAVES, R = GEMM_D16_RING;
     extern __shared__ __align__(16) float smem[];
-    v4f *red = reinterpret_cast<v4f *>(smem);            // [wave][mb][nb][lane]
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
     const int tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
@@ -514,23 +513,42 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
 #undef T2SP_GEMM_D16BT_ISSUE
 #undef T2SP_GEMM_D16BT_MMA
 
-    v4f *mine = red + wave * MB * NB * 64 + lane;
+    // A lane holds four rows of one column of each block; the partial blocks go to LDS row by row
+    // ([wave][block][row][column], one float per lane and store) so that they come back as four
+    // adjacent columns of one row per lane: 128-bit reads, and 128-bit stores to C where its rows allow.
+    // (row rho of a block starts at float 16 rho + 16 (rho / 4): the four row groups a store instruction
+    // writes then fall into four different sets of banks)
+    constexpr int BLK = 16 * 16 + 4 * 16;
+    float *mine = smem + wave * MB * NB * BLK + (4 * lq) * 16 + 16 * lq + li;
 #pragma unroll
     for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++) mine[(mb * NB + nb) * 64] = acc[mb][nb];
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) mine[(mb * NB + nb) * BLK + r * 16] = acc[mb][nb][r];
     __syncthreads();
+    const int orow = lane >> 2, ocol = (lane & 3) * 4;              // this lane's row and first column inside a block
+    const bool vec_ok = !g.tiled && g.ldc % 4 == 0 && ((uintptr_t)g.C % 16 == 0) &&
+                        (!g.scale || g.beta == 0.f || (g.ldcin % 4 == 0 && ((uintptr_t)g.Cin % 16 == 0)));
     for (int pr = wave; pr < MB * NB; pr += NW) {        // sum the partial blocks of the waves in wave order
-        const v4f *src = red + pr * 64 + lane;
+        const v4f *src = reinterpret_cast<const v4f *>(smem + pr * BLK + orow * 16 + 16 * (orow >> 2) + ocol);
         v4f sum = src[0];
 #pragma unroll
-        for (int wv = 1; wv < NW; wv++) sum += src[wv * MB * NB * 64];
+        for (int wv = 1; wv < NW; wv++) sum += src[wv * MB * NB * (BLK / 4)];
         const int mb = pr / NB, nb = pr - mb * NB;
-        const int col = n0 + 16 * nb + li;
+        const int row = m0 + 16 * mb + orow, col = n0 + 16 * nb + ocol;
+        if (row >= m_end) continue;
+        if (vec_ok && col + 4 <= N) {
+            v4f out = sum;
+            if (g.scale) {
+                out = out * g.alpha;
+                if (g.beta != 0.f) out += *reinterpret_cast<const v4f *>(g.Cin + (int64_t)row * g.ldcin + col) * g.beta;
+            }
+            *reinterpret_cast<v4f *>(g.C + (int64_t)row * g.ldc + col) = out;
+        } else {
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const int row = m0 + 16 * mb + 4 * lq + r;
-            if (row < m_end && col < N) gemm_store1(g, row, col, sum[r]);
+            for (int e = 0; e < 4; e++)
+                if (col + e < N) gemm_store1(g, row, col + e, sum[e]);
         }
     }
 }
@@ -951,7 +969,7 @@ template <int MB, int NB>
 static int launch_d16_bt_t(GemmArgs g, const GemmD16Plan &p, hipStream_t stream) {
     g.tiles_m = p.tiles_m;
     g.tiles_n = p.tiles_n;
-    const size_t smem = (size_t)GEMM_D16_WAVES * MB * NB * 64 * sizeof(v4f);
+    const size_t smem = (size_t)GEMM_D16_WAVES * MB * NB * (16 * 16 + 4 * 16) * sizeof(float);
     auto kern = sgemm_direct16_bt_kernel<MB, NB>;
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
