@@ -241,20 +241,33 @@ __global__ void __launch_bounds__(256) ssyrk_split_sum_kernel(const SyrkArgs g) 
 constexpr int SYRK_D16_WAVES = 4;
 constexpr int SYRK_D16_RING = 3;
 
+// The value of C the element (r, c), c >= r, is combined with (0 when there is none): what
+// syrk_value reads at (r, c).
 template <int MODE>
-__device__ __forceinline__ void syrk_store_upper(const SyrkArgs &g, int r, int c, float acc) {
+__device__ __forceinline__ float syrk_cin_upper(const SyrkArgs &g, int r, int c) {
+    if (!g.Cin) return 0.f;
+    int rr = r, cc = c;
+    if (MODE == SYRK_FLAT_SYM && !g.upper) { rr = c; cc = r; }
+    return g.Cin[(int64_t)rr * g.ldcin + cc];
+}
+
+// Element (r, c) of the 16 x 16 form, `cin` already read by syrk_cin_upper.
+template <int MODE>
+__device__ __forceinline__ void syrk_store_upper(const SyrkArgs &g, int r, int c, float acc, float cin,
+                                                 bool skip_mirror) {
     if (c < r) return;
+    float v = g.alpha * acc;
+    if (g.Cin) v += g.beta * cin;
     if constexpr (MODE == SYRK_FLAT_SYM) {
         const bool want_upper = g.upper || g.mirror, want_lower = !g.upper || g.mirror;
-        const float v = syrk_value<MODE>(g, r, c, acc);
         if (want_upper || r == c) g.C[(int64_t)r * g.ldc + c] = v;
-        if (want_lower && r != c) g.C[(int64_t)c * g.ldc + r] = v;
+        if (want_lower && r != c && !skip_mirror) g.C[(int64_t)c * g.ldc + r] = v;
     } else if constexpr (MODE == SYRK_FLAT_FULL) {
-        g.C[(int64_t)r * g.ldc + c] = syrk_value<MODE>(g, r, c, acc);
+        g.C[(int64_t)r * g.ldc + c] = v;
         if (c > r) g.C[(int64_t)c * g.ldc + r] = syrk_value<MODE>(g, c, r, acc);
     } else {
         const int B = g.f_iii * g.f_ii;
-        g.C[syrk_folded_offset(g, r, c)] = syrk_value<MODE>(g, r, c, acc);
+        g.C[syrk_folded_offset(g, r, c)] = v;
         if (r / B == c / B && r != c) g.C[syrk_folded_offset(g, c, r)] = syrk_value<MODE>(g, c, r, acc);
     }
 }
@@ -335,23 +348,57 @@ __global__ void __launch_bounds__(NW * 64) ssyrk_direct16_kernel(const SyrkArgs 
 #undef T2SP_SYRK_D16_ISSUE
 #undef T2SP_SYRK_D16_MMA
 
+    // The values of C this wave's blocks are combined with are requested before the exchange, so
+    // that their latency passes behind it (an element is read and written by its own workgroup
+    // only, so C may still be updated in place).
+    constexpr int PER_WAVE = (MB * NB + NW - 1) / NW;
+    float cin[PER_WAVE][4];
+#pragma unroll
+    for (int it = 0; it < PER_WAVE; it++) {
+        const int pr = wave + it * NW;
+        const int mb = pr / NB, nb = pr - mb * NB;
+        const int col = n0 + 16 * nb + li;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int row = m0 + 16 * mb + 4 * lq + r;
+            cin[it][r] = (pr < MB * NB && row < m_end && col < g.N && col >= row) ? syrk_cin_upper<MODE>(g, row, col) : 0.f;
+        }
+    }
     v4f *mine = red + wave * MB * NB * 64 + lane;
 #pragma unroll
     for (int mb = 0; mb < MB; mb++)
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) mine[(mb * NB + nb) * 64] = acc[mb][nb];
     __syncthreads();
-    for (int pr = wave; pr < MB * NB; pr += NW) {
+    // the mirror image of a lane's four rows of one column is four consecutive floats of one row
+    const bool mirror_rows = MODE == SYRK_FLAT_SYM && (!g.upper || g.mirror) && (m0 & 3) == 0 && (g.ldc & 3) == 0 &&
+                             ((uintptr_t)g.C & 15) == 0;
+#pragma unroll
+    for (int it = 0; it < PER_WAVE; it++) {
+        const int pr = wave + it * NW;
+        if (pr >= MB * NB) break;
         const v4f *src = red + pr * 64 + lane;
         v4f sum = src[0];
 #pragma unroll
         for (int wv = 1; wv < NW; wv++) sum += src[wv * MB * NB * 64];
         const int mb = pr / NB, nb = pr - mb * NB;
         const int col = n0 + 16 * nb + li;
+        const int row0 = m0 + 16 * mb + 4 * lq;
+        // all four elements strictly above the diagonal and inside the matrix: one 128-bit store
+        const bool vec = mirror_rows && col < g.N && row0 + 3 < m_end && col > row0 + 3;
+        if (vec) {
+            v4f v;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                v[r] = g.alpha * sum[r];
+                if (g.Cin) v[r] += g.beta * cin[it][r];
+            }
+            *reinterpret_cast<v4f *>(g.C + (int64_t)col * g.ldc + row0) = v;
+        }
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            const int row = m0 + 16 * mb + 4 * lq + r;
-            if (row < m_end && col < g.N) syrk_store_upper<MODE>(g, row, col, sum[r]);
+            const int row = row0 + r;
+            if (row < m_end && col < g.N) syrk_store_upper<MODE>(g, row, col, sum[r], cin[it][r], vec);
         }
     }
 }
