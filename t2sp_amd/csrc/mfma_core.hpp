@@ -266,6 +266,24 @@ __device__ __forceinline__ void loader_fetch(L &l) {
     else
         l.template fetch<S>();
 }
+// LDS reads a loader issues per k-tile in fetch (`static constexpr int EXTRA_DS_READ`).
+template <class L, class = void>
+struct LoaderExtraDsRead { static constexpr int value = 0; };
+template <class L>
+struct LoaderExtraDsRead<L, std::void_t<decltype(L::EXTRA_DS_READ)>> { static constexpr int value = L::EXTRA_DS_READ; };
+
+// A loader may ask to be called after every two fetches (`static constexpr bool HAS_PAIR_HOOK =
+// true` and `void after_pair()`): between the bodies of two pairs of k-tiles, where a branch that
+// is the same for every thread of the workgroup costs nothing, rather than inside a body, whose
+// one basic block the interleave above relies on.  The hook may use __syncthreads().
+template <class L, class = void>
+struct LoaderHasPairHook { static constexpr bool value = false; };
+template <class L>
+struct LoaderHasPairHook<L, std::void_t<decltype(L::HAS_PAIR_HOOK)>> { static constexpr bool value = L::HAS_PAIR_HOOK; };
+template <class L>
+__device__ __forceinline__ void loader_after_pair(L &l) {
+    if constexpr (LoaderHasPairHook<L>::value) l.after_pair();
+}
 // First k-tile (even) whose loop body must use the guarded fetch, for a reduction of `k_len`
 // elements seen from the loader's first k: the body of tile t fetches tile t + 2, and a pair of
 // bodies t, t + 1 may run unguarded while tiles t + 2 and t + 3 are whole.
@@ -299,6 +317,7 @@ __device__ __forceinline__ void mainloop_body(Accum<Cfg> &acc, ALoader &la, BLoa
     float *b_nxt = smem + 2 * Cfg::A_STAGE + (CUR ^ 1) * Cfg::B_STAGE;
     constexpr int MFMA_PER_SLICE = 4 * Cfg::MT * Cfg::NT;
     constexpr int N_DS_READ = Cfg::A_READS + Cfg::NT;
+    constexpr int N_DS_EXTRA = LoaderExtraDsRead<ALoader>::value + LoaderExtraDsRead<BLoader>::value;
     constexpr int N_DS_WRITE = Cfg::A_VEC + Cfg::B_VEC;
     constexpr int N_VMEM = N_DS_WRITE + LoaderExtraVmem<ALoader>::value + LoaderExtraVmem<BLoader>::value;
     loader_fetch<S, TAIL>(la);
@@ -311,12 +330,12 @@ __device__ __forceinline__ void mainloop_body(Accum<Cfg> &acc, ALoader &la, BLoa
     la.template commit<S ^ 1>(a_nxt);
     lb.template commit<S ^ 1>(b_nxt);
     {
-        constexpr int N_MEM = N_VMEM + N_DS_WRITE + (KK - 1) * N_DS_READ;
+        constexpr int N_MEM = N_VMEM + N_DS_WRITE + (KK - 1) * N_DS_READ + N_DS_EXTRA;
         constexpr int TOTAL = (KK - 1) * MFMA_PER_SLICE;
         constexpr int GAP = TOTAL / N_MEM > 0 ? TOTAL / N_MEM : 1;
         T2SP_INTERLEAVE(SG_DS_READ, N_DS_READ, GAP)
         T2SP_INTERLEAVE(SG_VMEM_READ, N_VMEM, GAP)
-        T2SP_INTERLEAVE(SG_DS_READ, (KK - 2) * N_DS_READ, GAP)
+        T2SP_INTERLEAVE(SG_DS_READ, (KK - 2) * N_DS_READ + N_DS_EXTRA, GAP)
         T2SP_INTERLEAVE(SG_DS_WRITE, N_DS_WRITE, GAP)
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -346,6 +365,8 @@ __device__ __forceinline__ void mainloop(Accum<Cfg> &acc, ALoader &la, BLoader &
     lb.template commit<0>(smem + 2 * Cfg::A_STAGE);
     loader_fetch<1, TAILS>(la);
     loader_fetch<1, TAILS>(lb);
+    loader_after_pair(la);
+    loader_after_pair(lb);
     __syncthreads();
     Frag<Cfg> frag[2];
     load_frag<Cfg>(frag[0], smem, smem + 2 * Cfg::A_STAGE, 0, wm, wn, lane);
@@ -355,11 +376,15 @@ __device__ __forceinline__ void mainloop(Accum<Cfg> &acc, ALoader &la, BLoader &
         for (; kt < plain_end; kt += 2) {
             mainloop_body<Cfg, 0, false>(acc, la, lb, frag, smem, wm, wn, lane);
             mainloop_body<Cfg, 1, false>(acc, la, lb, frag, smem, wm, wn, lane);
+            loader_after_pair(la);
+            loader_after_pair(lb);
         }
     }
     for (; kt < ktiles; kt += 2) {
         mainloop_body<Cfg, 0, TAILS>(acc, la, lb, frag, smem, wm, wn, lane);
         mainloop_body<Cfg, 1, TAILS>(acc, la, lb, frag, smem, wm, wn, lane);
+        loader_after_pair(la);
+        loader_after_pair(lb);
     }
 }
 

@@ -60,12 +60,12 @@ struct KjWalk {
     __device__ __forceinline__ bool inside() const { return kt < total; }
     // returns true when k moved on
     __device__ __forceinline__ bool next(int BK, bool edge) {
-        const bool go = edge ? true : kt + 1 < total;
-        kt += go ? 1 : 0;
-        j0 += go ? BK : 0;
-        const bool wrap = j0 >= J;
-        j0 = wrap ? 0 : j0;
-        k += wrap ? 1 : 0;
+        const bool go = edge || kt + 1 < total;
+        kt = go ? kt + 1 : kt;
+        const int j1 = go ? j0 + BK : j0;
+        const bool wrap = j1 >= J;
+        j0 = wrap ? 0 : j1;
+        k = wrap ? k + 1 : k;
         return wrap;
     }
 };
@@ -120,49 +120,82 @@ struct TensorKcLoader {
 
 // Khatri-Rao rows: slot (column r, 4 consecutive j) of reduction tile (k, j0) holds
 // C[j..j+3, r] * D[k, r], formed in registers.
+// The factors D[k, r] of the tile's BN columns come from a window of D_WIN consecutive k kept in
+// LDS.  Read from memory with every tile they cost as many cache-line requests as the tile's two
+// operands together when D is stored with k contiguous (the reference's helper layout): one line
+// per column.  The window is filled by the whole workgroup, 64 bytes per column at a time in that
+// layout, before the loop and again in after_pair() (which the mainloop calls between pairs of
+// k-tiles) whenever one of the next two fetches could leave it.
 template <class Cfg, bool EDGE>
 struct KhatriRaoKcLoader {
-    static constexpr int EXTRA_VMEM = Cfg::B_VEC;   // the D[k, r] factors
+    static constexpr int D_WIN = 16;
+    static constexpr int D_LD = Cfg::BN + 1;            // kk-major rows, padded: fills and reads without bank conflicts
+    static constexpr int D_FLOATS = D_WIN * D_LD;
+    static constexpr int EXTRA_DS_READ = Cfg::B_VEC;    // the D[k, r] factors
+    static constexpr bool HAS_PAIR_HOOK = true;
     const float *pc[Cfg::B_VEC];
-    const float *pd[Cfg::B_VEC];
+    int dslot[Cfg::B_VEC];                              // the slot's column within the tile
     const float *safe;
     v4f reg[2][Cfg::B_VEC];
     float dval[2][Cfg::B_VEC];
     KjWalk w;
-    int64_t koff, sd_k;   // koff = k * sd_k
-    __device__ KhatriRaoKcLoader(const MttkrpArgs &g, int n0, int kt0)
-        : safe(g.C), w(kt0, g.K, g.J, Cfg::BK), sd_k(g.sd_k) {
-        koff = w.k * sd_k;
+    const float *D;
+    int64_t sd_k, sd_r;
+    float *dl;                                          // the window: dl[kk * D_LD + column]
+    int kwin, k_last, n0, R;
+    __device__ KhatriRaoKcLoader(const MttkrpArgs &g, int n0_, int kt0, float *window)
+        : safe(g.C), w(kt0, g.K, g.J, Cfg::BK), D(g.D), sd_k(g.sd_k), sd_r(g.sd_r), dl(window), k_last(g.K - 1),
+          n0(n0_), R(g.R) {
+        kwin = w.k;
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
             const int r = (!EDGE || n0 + s.row < g.R) ? n0 + s.row : 0;
             pc[i] = g.C + (int64_t)r * g.sc_r + s.k;
-            pd[i] = g.D + (int64_t)r * g.sd_r;
+            dslot[i] = s.row;
+        }
+    }
+    // Every thread of the workgroup: D[kwin .. kwin + D_WIN) x the tile's columns -> LDS.  Rows past
+    // the end of D repeat the last one and columns past R the first (they only meet tiles that read
+    // as zero or feed outputs that are never stored).
+    __device__ __forceinline__ void fill_window() {
+        for (int e = threadIdx.x; e < Cfg::BN * D_WIN; e += Cfg::NTHREADS) {
+            const int kk = e % D_WIN, col = e / D_WIN;
+            const int r = (!EDGE || n0 + col < R) ? n0 + col : 0;
+            const int k = min(kwin + kk, k_last);
+            dl[kk * D_LD + col] = D[k * sd_k + r * sd_r];
+        }
+    }
+    __device__ __forceinline__ void after_pair() {
+        // the next two fetches are at k or k + 1; the same for every thread of the workgroup
+        if (w.k + 2 > kwin + D_WIN) {
+            __syncthreads();            // every wave has read the factors of its last fetch
+            kwin = w.k;
+            fill_window();
+            __syncthreads();
         }
     }
     static constexpr bool HAS_TAIL_FETCH = EDGE;   // as in TensorKcLoader; a column past R reads column 0
     template <int S>
     __device__ __forceinline__ void fetch() {
+        const float *row = dl + (w.k - kwin) * D_LD;
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             reg[S][i] = *reinterpret_cast<const v4f *>(pc[i] + w.j0);
-            dval[S][i] = pd[i][koff];
+            dval[S][i] = row[dslot[i]];
         }
-        const int kt_before = w.kt;
-        const bool wrap = w.next(Cfg::BK, EDGE);
-        koff += (w.kt != kt_before && wrap) ? sd_k : 0;
+        w.next(Cfg::BK, EDGE);
     }
     template <int S>
     __device__ __forceinline__ void fetch_tail() {
         const bool in = w.inside();
+        const float *row = dl + (w.k - kwin) * D_LD;
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             reg[S][i] = load_or_zero(pc[i] + (in ? w.j0 : 0), in, safe);
-            dval[S][i] = pd[i][in ? koff : 0];
+            dval[S][i] = row[dslot[i]];
         }
-        const bool wrap = w.next(Cfg::BK, true);
-        koff += wrap ? sd_k : 0;
+        w.next(Cfg::BK, true);
     }
     template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
@@ -183,7 +216,9 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) mttkrp_kernel(const MttkrpArgs 
     int kt0, kt1;
     split_range(g.K * (g.J / Cfg::BK), g.splits, split, kt0, kt1);
     TensorKcLoader<Cfg, EDGE> la(g, m0, kt0);
-    KhatriRaoKcLoader<Cfg, EDGE> lb(g, n0, kt0);
+    KhatriRaoKcLoader<Cfg, EDGE> lb(g, n0, kt0, smem + Cfg::SMEM_FLOATS);
+    lb.fill_window();
+    __syncthreads();
     Accum<Cfg> acc;
     mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem, tail_from_for<Cfg>((g.K * (g.J / Cfg::BK) - kt0) * Cfg::BK));
     if (g.splits == 1) {
@@ -264,7 +299,7 @@ template <class Cfg>
 static int launch_mttkrp(MttkrpArgs g, hipStream_t stream) {
     g.tiles_m = g.Mp / Cfg::BM;
     g.tiles_n = g.Np / Cfg::BN;
-    const size_t smem = Cfg::SMEM_FLOATS * sizeof(float);
+    const size_t smem = (Cfg::SMEM_FLOATS + KhatriRaoKcLoader<Cfg, false>::D_FLOATS) * sizeof(float);
     // plain loaders need whole tiles and a reduction that ends on a pair of k-tiles
     const bool edge = (g.I % Cfg::BM) || (g.R % Cfg::BN) || ((int64_t)g.K * (g.J / Cfg::BK)) % 2;
     auto kern = edge ? mttkrp_kernel<Cfg, true> : mttkrp_kernel<Cfg, false>;
