@@ -128,6 +128,98 @@ struct Im2colRcLoader {
     }
 };
 
+// The same operand for tiles 256 pixels wide: a k-row of the tile is then 64 slots, one wave, so the
+// window position (ci, kh, kw) of a slot is the same for every lane of its wave.  It is walked with
+// counters in scalar registers (no table, no vector arithmetic): a lane keeps the address of its
+// pixel and adds the wave's offset ci * si_c + kh * si_h + kw to it, one vector instruction per
+// load as for a plain matrix.  (The per-lane walk above costs about ten per load, which the MFMA
+// pipe pays for: a wave issues them in the cycles it would issue MFMAs in.)
+template <class Cfg, bool EDGE>
+struct Im2colWaveRowLoader {
+    static_assert((Cfg::BN / 4) % 64 == 0 && Cfg::BN / 4 == 64, "a k-row of the tile must be one wave");
+    static constexpr int ROWS_APART = Cfg::NTHREADS / 64;   // k-rows between a thread's slots
+    const float *pix[Cfg::B_VEC];    // the lane's input pixel (n, h, w) at ci = kh = kw = 0
+    int kh[Cfg::B_VEC], kw[Cfg::B_VEC];
+    uint32_t off[Cfg::B_VEC];        // ci * si_c + kh * si_h + kw of the row this slot loads next
+    v4f reg[2][Cfg::B_VEC];
+    int k0;                          // first reduction row of the tile fetched next
+    int KH, KW, KRED;
+    int step_kh, step_kw;            // a k-tile of BK rows moves the window position by these,
+    uint32_t step_off;               // and the offset by this, before carries
+    uint32_t carry_w, carry_h;       // offset corrections when kw, kh wrap
+    int wave_k;                      // the k-row of slot 0 within a tile
+    __device__ Im2colWaveRowLoader(const ConvArgs &g, int p0, const int *, int k_begin)
+        : k0(k_begin), KH(g.KH), KW(g.KW), KRED(g.KRED) {
+        const int win = g.KH * g.KW;
+        const int dr = Cfg::BK % win;
+        step_kh = dr / g.KW;
+        step_kw = dr - step_kh * g.KW;
+        step_off = (uint32_t)((Cfg::BK / win) * g.si_c + step_kh * g.si_h + step_kw);
+        carry_w = (uint32_t)(g.si_h - g.KW);
+        carry_h = (uint32_t)(g.si_c - g.KH * g.si_h);
+        wave_k = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
+            int p = p0 + s.col;
+            if (EDGE && p >= g.P) p = 0;
+            const int hw = g.OH * g.OWp;
+            const int n = p / hw, rem = p - n * hw;
+            const int h = rem / g.OWp, w = min(rem - h * g.OWp, g.OW - 4);
+            pix[i] = g.I + (n * g.si_n + h * g.si_h + w);
+            const int row = wave_k + i * ROWS_APART;
+            const int q = (k_begin + row < g.KRED) ? k_begin + row : 0;
+            const int c = q / win, r = q - c * win;
+            kh[i] = r / g.KW;
+            kw[i] = r - kh[i] * g.KW;
+            off[i] = (uint32_t)(c * g.si_c + kh[i] * g.si_h + kw[i]);
+        }
+    }
+    __device__ __forceinline__ void advance(int i, bool go) {
+        const int w1 = kw[i] + step_kw;
+        const bool cw = w1 >= KW;
+        const int h1 = cw ? kh[i] + step_kh + 1 : kh[i] + step_kh;
+        const bool ch = h1 >= KH;
+        const uint32_t o1 = off[i] + step_off, o2 = cw ? o1 + carry_w : o1, o3 = ch ? o2 + carry_h : o2;
+        kw[i] = go ? (cw ? w1 - KW : w1) : kw[i];
+        kh[i] = go ? (ch ? h1 - KH : h1) : kh[i];
+        off[i] = go ? o3 : off[i];
+    }
+    static constexpr bool HAS_TAIL_FETCH = EDGE;   // as in Im2colRcLoader
+    template <int S>
+    __device__ __forceinline__ void fetch() {
+        const bool go = EDGE || k0 + 2 * Cfg::BK <= KRED;
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            reg[S][i] = *reinterpret_cast<const v4f_u *>(pix[i] + off[i]);
+            advance(i, go);
+        }
+        k0 += go ? Cfg::BK : 0;
+    }
+    template <int S>
+    __device__ __forceinline__ void fetch_tail() {
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            const bool ok = k0 + wave_k + i * ROWS_APART < KRED;
+            const v4f_u v = *reinterpret_cast<const v4f_u *>(pix[i] + (ok ? off[i] : 0u));
+            reg[S][i] = ok ? (v4f)v : v4f{0.f, 0.f, 0.f, 0.f};
+            advance(i, true);
+        }
+        k0 += Cfg::BK;
+    }
+    template <int S>
+    __device__ __forceinline__ void commit(float *stage) const {
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
+            *reinterpret_cast<v4f *>(stage + s.k * Cfg::LDB + s.col) = reg[S][i];
+        }
+    }
+};
+
+template <class Cfg, bool EDGE>
+using Im2colLoaderFor = std::conditional_t<Cfg::BN == 256, Im2colWaveRowLoader<Cfg, EDGE>, Im2colRcLoader<Cfg, EDGE>>;
+
 template <class Cfg, bool EDGE>
 __global__ void __launch_bounds__(Cfg::NTHREADS) conv_kernel(const ConvArgs g) {
     extern __shared__ __align__(16) float smem[];
@@ -141,7 +233,7 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) conv_kernel(const ConvArgs g) {
     int kt0 = 0, kt1 = ktiles_even<Cfg>(g.KRED);
     if (g.splits > 1) split_range((g.KRED + Cfg::BK - 1) / Cfg::BK, g.splits, split, kt0, kt1);
     RowMajorKcLoader<Cfg, EDGE> la(g.W, g.sw_o, co0, g.CO, g.KRED, kt0 * Cfg::BK);
-    Im2colRcLoader<Cfg, EDGE> lb(g, p0, tab, kt0 * Cfg::BK);
+    Im2colLoaderFor<Cfg, EDGE> lb(g, p0, tab, kt0 * Cfg::BK);
     Accum<Cfg> acc;
     mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem, tail_from_for<Cfg>(g.KRED - kt0 * Cfg::BK));
     if (g.splits > 1) {
