@@ -300,8 +300,27 @@ struct GemmHot {
     const float *A, *B;
     int M, N, lda, ldb;
 };
+// Buffer loads: the address is a descriptor's base (scalar registers) + a 32-bit lane offset + a
+// 32-bit scalar offset, so a loop that moves the scalar offset needs no vector instruction per
+// load.  The descriptor covers 4 GiB from `base` without a range check that could bite.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t whole_buffer(const void *base) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, -1, 0x00020000);
+}
+template <class V>
+__device__ __forceinline__ V buffer_load(__amdgpu_buffer_rsrc_t rsrc, uint32_t lane_off, uint32_t scalar_off) {
+    if constexpr (sizeof(V) == 16) {
+        typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+        const u4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)lane_off, (int)scalar_off, 0);
+        return __builtin_bit_cast(V, v);
+    } else {
+        static_assert(sizeof(V) == 8, "128- or 64-bit loads");
+        typedef unsigned int u2 __attribute__((ext_vector_type(2)));
+        const u2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)lane_off, (int)scalar_off, 0);
+        return __builtin_bit_cast(V, v);
+    }
+}
 // Row blocks [mb0, mb0 + MBW) of the tile over steps [s0, s0 + nsteps) of 16 k, partial result to red_kq.
-template <int MBW, int NB>
+template <int MBW, int NB, bool BUF>
 __device__ __forceinline__ void sgemm_d16_wave(const GemmHot &g, int mb0, int m0, int n0, int s0, int nsteps, int steps,
                                                v4f *red_kq) {
     typedef typename VecOf<NB>::type vnb;
@@ -320,12 +339,18 @@ __device__ __forceinline__ void sgemm_d16_wave(const GemmHot &g, int mb0, int m0
     // gemm_d16_ok): a 64-bit address per lane doubles the address traffic of every load, and that
     // traffic holds up the wave's MFMA issue.  The step's part of the offset is added in 32 bits
     // inside the loop, which keeps the compiler from hoisting a 64-bit lane address out of it.
+    // BUF: buffer loads instead, which take the step's part as a scalar offset, so the loop has no
+    // vector instruction but its MFMAs.  Measured: 3 to 9 % faster where a launch gives a CU one
+    // workgroup (one wave per SIMD: nothing else issues in the cycles the additions take;
+    // 1024^3 18.5 -> 17.8 us), up to 4 % slower where two workgroups share a CU and the reduction
+    // is long (1536^3, 2048^3), so the host picks it for launches of one round and for short reductions.
     uint32_t b_off[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) b_off[j] = 4u * (uint32_t)((4 * lq + j) * (int)g.ldb + (col_ok ? col : 0));
     const char *a_base = reinterpret_cast<const char *>(g.A + 16 * s0);
     const char *b_base = reinterpret_cast<const char *>(g.B + (int64_t)16 * s0 * g.ldb);
     const uint32_t b_step = 64u * (uint32_t)g.ldb;         // bytes per step of 16 k-rows
+    const __amdgpu_buffer_rsrc_t a_rsrc = whole_buffer(a_base), b_rsrc = whole_buffer(b_base);
     int issued = 0;
 
     v4f ra[R][MBW];
@@ -336,9 +361,11 @@ __device__ __forceinline__ void sgemm_d16_wave(const GemmHot &g, int mb0, int m0
         const uint32_t ao = 64u * (uint32_t)st, bo = (uint32_t)st * b_step;                         \
         issued++;                                                                                   \
         _Pragma("unroll") for (int j = 0; j < 4; j++)                                               \
-            rb[d][j] = *reinterpret_cast<const vnb *>(b_base + (b_off[j] + bo));                    \
+            rb[d][j] = BUF ? buffer_load<vnb>(b_rsrc, b_off[j], bo)                                 \
+                           : *reinterpret_cast<const vnb *>(b_base + (b_off[j] + bo));              \
         _Pragma("unroll") for (int mb = 0; mb < MBW; mb++)                                          \
-            ra[d][mb] = *reinterpret_cast<const v4f *>(a_base + (a_off[mb] + ao));                  \
+            ra[d][mb] = BUF ? buffer_load<v4f>(a_rsrc, a_off[mb], ao)                               \
+                            : *reinterpret_cast<const v4f *>(a_base + (a_off[mb] + ao));            \
     }
 #define T2SP_GEMM_D16_MMA(d)                                                                        \
     _Pragma("unroll") for (int j = 0; j < 4; j++)                                                   \
@@ -387,7 +414,7 @@ __device__ __forceinline__ void sgemm_d16_wave(const GemmHot &g, int mb0, int m0
         for (int nb = 0; nb < NB; nb++) mine[(mb * NB + nb) * 64] = acc[mb][nb];
 }
 
-template <int MB, int NB>
+template <int MB, int NB, bool BUF>
 __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     sgemm_direct16_kernel(const float *A, const float *B, int M, int N, int K, int lda, int ldb, int tiles_m, int rows_per_tile,
                           const GemmArgs g) {
@@ -403,7 +430,7 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     const int steps = K >> 4;
     const int s0 = (int)((int64_t)steps * wave / NW), s1 = (int)((int64_t)steps * (wave + 1) / NW);
     const GemmHot hot{A, B, M, N, lda, ldb};
-    sgemm_d16_wave<MB, NB>(hot, 0, m0, n0, s0, s1 - s0, steps, red + wave * MB * NB * 64);
+    sgemm_d16_wave<MB, NB, BUF>(hot, 0, m0, n0, s0, s1 - s0, steps, red + wave * MB * NB * 64);
     __syncthreads();
     T2SP_TRACE_STAMP(5)
     // sum the partial tiles of the waves in wave order
@@ -926,7 +953,11 @@ static int launch_d16_t(GemmArgs g, const GemmD16Plan &p, hipStream_t stream) {
     g.tiles_m = p.tiles_m;
     g.tiles_n = p.tiles_n;
     const size_t smem = (size_t)GEMM_D16_WAVES * MB * NB * 64 * sizeof(v4f);
-    auto kern = sgemm_direct16_kernel<MB, NB>;
+    // one workgroup per CU at most, or a short reduction: the form whose loop has no vector arithmetic
+    // (see sgemm_d16_wave; measured with several rounds: 2048 x 1024 x 512 20.7 -> 18.8 us,
+    // 3072 x 1024 x 1024 53.7 -> 51.9 us, but 1536^3 54.2 -> 56.2 us)
+    const bool buf = p.tiles_m * p.tiles_n <= machine().cus || g.K <= 1024;
+    auto kern = buf ? sgemm_direct16_kernel<MB, NB, true> : sgemm_direct16_kernel<MB, NB, false>;
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(GEMM_D16_WAVES * 64), smem, stream, g.A, g.B, g.M, g.N, g.K,
