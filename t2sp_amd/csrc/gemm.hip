@@ -300,25 +300,6 @@ struct GemmHot {
     const float *A, *B;
     int M, N, lda, ldb;
 };
-// Buffer loads: the address is a descriptor's base (scalar registers) + a 32-bit lane offset + a
-// 32-bit scalar offset, so a loop that moves the scalar offset needs no vector instruction per
-// load.  The descriptor covers 4 GiB from `base` without a range check that could bite.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t whole_buffer(const void *base) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, -1, 0x00020000);
-}
-template <class V>
-__device__ __forceinline__ V buffer_load(__amdgpu_buffer_rsrc_t rsrc, uint32_t lane_off, uint32_t scalar_off) {
-    if constexpr (sizeof(V) == 16) {
-        typedef unsigned int u4 __attribute__((ext_vector_type(4)));
-        const u4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)lane_off, (int)scalar_off, 0);
-        return __builtin_bit_cast(V, v);
-    } else {
-        static_assert(sizeof(V) == 8, "128- or 64-bit loads");
-        typedef unsigned int u2 __attribute__((ext_vector_type(2)));
-        const u2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)lane_off, (int)scalar_off, 0);
-        return __builtin_bit_cast(V, v);
-    }
-}
 // Row blocks [mb0, mb0 + MBW) of the tile over steps [s0, s0 + nsteps) of 16 k, partial result to red_kq.
 template <int MBW, int NB, bool BUF>
 __device__ __forceinline__ void sgemm_d16_wave(const GemmHot &g, int mb0, int m0, int n0, int s0, int nsteps, int steps,
@@ -344,6 +325,8 @@ __device__ __forceinline__ void sgemm_d16_wave(const GemmHot &g, int mb0, int m0
     // workgroup (one wave per SIMD: nothing else issues in the cycles the additions take;
     // 1024^3 18.5 -> 17.8 us), up to 4 % slower where two workgroups share a CU and the reduction
     // is long (1536^3, 2048^3), so the host picks it for launches of one round and for short reductions.
+    // The form for A^T gains as much (1024^3 18.2 -> 17.3 us); the one for B^T gains nothing and the
+    // SYRK kernel of this form, whose two operands are one matrix, loses 4 %: they keep plain loads.
     uint32_t b_off[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) b_off[j] = 4u * (uint32_t)((4 * lq + j) * (int)g.ldb + (col_ok ? col : 0));
@@ -585,7 +568,7 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
 // columns of one k-row per lane and 128-bit load, so row block mb holds the rows congruent to mb
 // modulo 4 and column block nb the columns congruent to nb modulo 4 of the 64 x 64 tile; a lane
 // ends with four adjacent columns of each of its rows and stores 128 bits at a time.
-template <int MB>
+template <int MB, bool BUF>
 __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     sgemm_direct16_at_kernel(const float *A, const float *B, int M, int N, int K, int lda, int ldb, int tiles_m, const GemmArgs g) {
     constexpr int NW = GEMM_D16_WAVES, R = GEMM_D16_RING, NB = 4;
@@ -612,6 +595,7 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     const char *a_base = reinterpret_cast<const char *>(A + (int64_t)16 * s0 * lda);
     const char *b_base = reinterpret_cast<const char *>(B + (int64_t)16 * s0 * ldb);
     const uint32_t a_step = 64u * (uint32_t)lda, b_step = 64u * (uint32_t)ldb;
+    const __amdgpu_buffer_rsrc_t a_rsrc = whole_buffer(a_base), b_rsrc = whole_buffer(b_base);   // BUF: see sgemm_d16_wave
     int issued = 0;
 
     vmb ra[R][4];
@@ -621,9 +605,11 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
         const uint32_t st = (uint32_t)min(issued, steps - 1 - s0);                                  \
         issued++;                                                                                   \
         _Pragma("unroll") for (int j = 0; j < 4; j++)                                               \
-            rb[d][j] = *reinterpret_cast<const v4f *>(b_base + (b_off[j] + st * b_step));           \
+            rb[d][j] = BUF ? buffer_load<v4f>(b_rsrc, b_off[j], st * b_step)                        \
+                           : *reinterpret_cast<const v4f *>(b_base + (b_off[j] + st * b_step));     \
         _Pragma("unroll") for (int j = 0; j < 4; j++)                                               \
-            ra[d][j] = *reinterpret_cast<const vmb *>(a_base + (a_off[j] + st * a_step));           \
+            ra[d][j] = BUF ? buffer_load<vmb>(a_rsrc, a_off[j], st * a_step)                        \
+                           : *reinterpret_cast<const vmb *>(a_base + (a_off[j] + st * a_step));     \
     }
 #define T2SP_GEMM_D16AT_MMA(d)                                                                      \
     _Pragma("unroll") for (int j = 0; j < 4; j++)                                                   \
@@ -1035,7 +1021,9 @@ static int launch_d16_at(GemmArgs g, hipStream_t stream) {
     g.tiles_m = (g.M + 16 * mb - 1) / (16 * mb);
     g.tiles_n = (g.N + 63) / 64;
     const size_t smem = (size_t)GEMM_D16_WAVES * mb * 4 * 64 * sizeof(v4f);
-    auto kern = narrow ? sgemm_direct16_at_kernel<2> : sgemm_direct16_at_kernel<4>;
+    const bool buf = g.tiles_m * g.tiles_n <= cus || g.K <= 1024;   // as in launch_d16_t
+    auto kern = narrow ? (buf ? sgemm_direct16_at_kernel<2, true> : sgemm_direct16_at_kernel<2, false>)
+                       : (buf ? sgemm_direct16_at_kernel<4, true> : sgemm_direct16_at_kernel<4, false>);
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(GEMM_D16_WAVES * 64), smem, stream, g.A, g.B, g.M, g.N, g.K, (int)g.lda,

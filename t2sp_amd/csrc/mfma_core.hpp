@@ -85,6 +85,25 @@ __device__ __forceinline__ V load_or_zero(const float *ptr, bool valid, const fl
     return valid ? v : V{0.f, 0.f, 0.f, 0.f};
 }
 
+// Buffer loads: the address is a descriptor's base (scalar registers) + a 32-bit lane offset + a
+// 32-bit scalar offset, so a loop that moves the scalar offset needs no vector instruction per
+// load.  The descriptor covers 4 GiB from `base` without a range check that could bite.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t whole_buffer(const void *base) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, -1, 0x00020000);
+}
+template <class V>
+__device__ __forceinline__ V buffer_load(__amdgpu_buffer_rsrc_t rsrc, uint32_t lane_off, uint32_t scalar_off) {
+    if constexpr (sizeof(V) == 16) {
+        typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+        const u4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)lane_off, (int)scalar_off, 0);
+        return __builtin_bit_cast(V, v);
+    } else {
+        static_assert(sizeof(V) == 8, "128- or 64-bit loads");
+        typedef unsigned int u2 __attribute__((ext_vector_type(2)));
+        const u2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)lane_off, (int)scalar_off, 0);
+        return __builtin_bit_cast(V, v);
+    }
+}
 // Division-free, multiply-free walk over a reduction index q = c * WIN + r, r = kh * KW + kw,
 // that advances by a fixed step per k-tile (convolution windows).  The element offset of q is
 //     c * stride_c + tab[r],   tab[r] = (r / KW) * stride_h + (r % KW) * stride_w,
