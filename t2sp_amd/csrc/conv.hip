@@ -675,7 +675,7 @@ extern "C" int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, 
     // aligned 128-bit stores need rows that start on 16-byte boundaries; ragged rows use 4-byte aligned ones
     const bool out_ok = so4[3] == 1 && (ragged ? ((uintptr_t)O % 4 == 0)
                                                 : (so4[0] % 4 == 0 && so4[1] % 4 == 0 && so4[2] % 4 == 0 && (uintptr_t)O % 16 == 0));
-    const bool fast = cfg != T2SP_CFG_SCALAR && si4[3] == 1 && out_ok && w_dense && sw_o % 4 == 0 && OW >= 4 &&
+    const bool fast = cfg != T2SP_CFG_SCALAR && si4[3] == 1 && out_ok && w_dense && sw_o % 4 == 0 && sw_o < t2sp::LOADER_MAX_LD && OW >= 4 &&
                       (int64_t)N * OH * owp <= INT32_MAX && (kred % 4 == 0 || padded) && KH * KW <= 4096 &&
                       in_span < INT32_MAX && ((uintptr_t)W % 16 == 0) && ((uintptr_t)I % 4 == 0);
     if (!fast) {

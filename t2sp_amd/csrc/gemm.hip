@@ -1038,7 +1038,8 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         // A^T * B with both operands as they lie (the caller has checked the alignment the 128-bit
         // loads need).  Any K: k is the row index of both operands.
         if (bt || (cfg != T2SP_CFG_AUTO && cfg != T2SP_CFG_DIRECT16)) return T2SP_ERR_SHAPE;
-        if (cfg == T2SP_CFG_DIRECT16) return gemm_d16_at_ok(g) ? launch_d16_at(g, stream) : T2SP_ERR_SHAPE;
+        if (cfg == T2SP_CFG_DIRECT16 || g.lda >= LOADER_MAX_LD || g.ldb >= LOADER_MAX_LD)
+            return gemm_d16_at_ok(g) ? launch_d16_at(g, stream) : T2SP_ERR_SHAPE;
         {
             // small and middle-sized products: the one-launch form, as for the other layouts
             const int64_t t256 = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
@@ -1090,7 +1091,9 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && gemm_direct_ok(g, cfg == T2SP_CFG_DIRECT))
         return launch_direct(g, stream);
     if (cfg == T2SP_CFG_DIRECT) return T2SP_ERR_SHAPE;
+    // (the loaders address a tile with 32-bit offsets: leading dimensions below LOADER_MAX_LD)
     const bool vec_ok = g.K % 4 == 0 && (bt || g.N % 4 == 0) && g.lda % 4 == 0 && g.ldb % 4 == 0 &&
+                        g.lda < LOADER_MAX_LD && g.ldb < LOADER_MAX_LD &&
                         ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
                         ((uintptr_t)g.C % 16 == 0) && (g.tiled || g.ldc % 4 == 0) &&
                         (!g.scale || (g.ldcin % 4 == 0 && (uintptr_t)g.Cin % 16 == 0));
@@ -1245,7 +1248,10 @@ extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, fl
     const bool room = workspace && workspace_bytes >= (size_t)M * K * sizeof(float);
     // (now that the 16 x 16 form reads a transposed A as it lies, the re-laying route is only left for
     // operands it cannot address)
-    const bool native_at = at_possible && (cfg == T2SP_CFG_AUTO || cfg == T2SP_CFG_DIRECT16);
+    // (rows too far apart for the LDS-tile loaders' 32-bit offsets: only the 16 x 16 form, where it reaches)
+    const bool at_far = lda >= t2sp::LOADER_MAX_LD || ldb >= t2sp::LOADER_MAX_LD;
+    const bool at_far_ok = K % 16 == 0 && (int64_t)K * lda < (1 << 30) && (int64_t)K * ldb < (1 << 30);
+    const bool native_at = at_possible && (cfg == T2SP_CFG_AUTO || cfg == T2SP_CFG_DIRECT16) && (!at_far || at_far_ok);
     (void)t256; (void)room;
     if (transa && !native_at) {
         // A is stored K x M: bring it to M x K first (the loaders of the other kernels want k contiguous in A)

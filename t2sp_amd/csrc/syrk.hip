@@ -567,7 +567,7 @@ static int dispatch_syrk(SyrkArgs g, int trans, int cfg, float *workspace, size_
     }
     // A the 128-bit loaders cannot read where it lies (K or its leading dimension not a multiple of 4,
     // unaligned): a zero-padded, aligned copy is multiplied instead, as the SGEMM path does
-    const bool a_ok = g.K % 4 == 0 && g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0);
+    const bool a_ok = g.K % 4 == 0 && g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && g.lda < LOADER_MAX_LD;
     if (!a_ok && cfg == T2SP_CFG_AUTO && workspace && ((uintptr_t)workspace % 16 == 0) &&
         workspace_bytes >= syrk_padded_a_bytes(g.N, g.K)) {
         const int kp = syrk_pad_k(g.K);
@@ -587,7 +587,7 @@ static int dispatch_syrk(SyrkArgs g, int trans, int cfg, float *workspace, size_
     const bool out_ok = g.mode == SYRK_FOLDED ||
                         (g.ldc % 4 == 0 && (uintptr_t)g.C % 16 == 0 &&
                          (!g.Cin || (g.ldcin % 4 == 0 && (uintptr_t)g.Cin % 16 == 0)));
-    const bool vec_ok = out_ok && g.K % 4 == 0 && g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0);
+    const bool vec_ok = out_ok && g.K % 4 == 0 && g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && g.lda < LOADER_MAX_LD;
     if (cfg == T2SP_CFG_SCALAR || !vec_ok) {
         auto kern = g.mode == SYRK_FLAT_SYM ? ssyrk_scalar_kernel<SYRK_FLAT_SYM>
                     : g.mode == SYRK_FLAT_FULL ? ssyrk_scalar_kernel<SYRK_FLAT_FULL> : ssyrk_scalar_kernel<SYRK_FOLDED>;

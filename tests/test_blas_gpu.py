@@ -241,3 +241,34 @@ def test_eight_argument_gemm_as_the_reference_wrapper_calls_it(oracle):
                                  *[ctypes.cast(x.ref, ctypes.c_void_p) for x in (a, b, c, o2)])
     assert Bl.gemm_argv(args) == 0
     assert (O2 == O).all()
+
+
+@pytest.mark.parametrize("form,cfg", [("NN", 1), ("NN", 2), ("NT", 1), ("TN", 0), ("NN-far", 0)])
+def test_lds_tile_loaders_rows_far_apart(form, cfg):
+    """The LDS-tile loaders address a tile with one pointer for all lanes and a 32-bit byte offset per
+    lane: with rows 15.6 MB apart (a leading dimension of 3.9 million) the last rows of a 256-row tile
+    lie just under 2^32 bytes from its first, beyond what a signed offset reaches.  A leading dimension
+    of 2^22 or more ("NN-far") is beyond them: the call still succeeds on another kernel.  Integer data."""
+    import torch
+    L = t2sp_amd.lib()
+    M, N, K = 256, 256, 64
+    ld = 5_000_000 if form == "NN-far" else 3_900_000
+    g = torch.Generator().manual_seed(5)
+    A = torch.randint(-2, 3, (M, K), generator=g).float().cuda()
+    B = torch.randint(-2, 3, (K, N), generator=g).float().cuda()
+    want = A.double() @ B.double()
+    rows = K if form == "TN" else 256
+    big = torch.zeros((rows - 1) * ld + 256, device="cuda")        # up to 5.1 GB
+    transa, transb, a_ptr, lda, b_ptr, ldb = 0, 0, A.data_ptr(), K, B.data_ptr(), N
+    if form.startswith("NN"):
+        view = big.as_strided((M, K), (ld, 1)); view.copy_(A); a_ptr, lda = view.data_ptr(), ld
+    elif form == "NT":
+        view = big.as_strided((N, K), (ld, 1)); view.copy_(B.t()); transb, b_ptr, ldb = 1, view.data_ptr(), ld
+    else:
+        view = big.as_strided((K, M), (ld, 1)); view.copy_(A.t()); transa, a_ptr, lda = 1, view.data_ptr(), ld
+    C = torch.full((M, N), float("nan"), device="cuda")
+    rc = L.t2sp_sgemm_ex_f32(transa, transb, M, N, K, 1.0, a_ptr, lda, b_ptr, ldb, 0.0, None, 0, C.data_ptr(), N, cfg, None, 0, None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(C.double(), want)
+    del big
