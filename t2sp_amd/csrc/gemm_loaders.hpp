@@ -20,8 +20,6 @@
 
 namespace t2sp {
 
-constexpr int64_t LOADER_MAX_LD = (int64_t)1 << 22;   // 255 rows * ld * 4 bytes < 2^32
-
 // Slots whose rows are rows of a row-major matrix with k contiguous (an A operand, or a B operand
 // stored transposed): VEC slots per thread of a tile of `rows` starting at row0.
 template <class Cfg, bool EDGE, int VEC>

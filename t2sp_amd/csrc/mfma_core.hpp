@@ -104,6 +104,10 @@ __device__ __forceinline__ V buffer_load(__amdgpu_buffer_rsrc_t rsrc, uint32_t l
         return __builtin_bit_cast(V, v);
     }
 }
+// Loaders that reach the rows of a tile with 32-bit byte offsets from its first row take leading
+// dimensions below this: 255 rows * ld * 4 bytes < 2^32.  The hosts check it.
+constexpr int64_t LOADER_MAX_LD = (int64_t)1 << 22;
+
 // Division-free, multiply-free walk over a reduction index q = c * WIN + r, r = kh * KW + kw,
 // that advances by a fixed step per k-tile (convolution windows).  The element offset of q is
 //     c * stride_c + tab[r],   tab[r] = (r / KW) * stride_h + (r % KW) * stride_w,

@@ -73,19 +73,20 @@ struct KjWalk {
 // B tensor rows: slot (row i, 4 consecutive j) of reduction tile (k, j0).
 template <class Cfg, bool EDGE>
 struct TensorKcLoader {
-    const float *p[Cfg::A_VEC];
+    const char *base;            // row m0 of the tile at (k, j0): the same for every lane (see gemm_loaders.hpp)
+    uint32_t off[Cfg::A_VEC];    // the slot's (row, j) from there, bytes
     const float *safe;
     v4f reg[2][Cfg::A_VEC];
     KjWalk w;
-    int64_t off, sb_k;    // off = k * sb_k + j0
+    int64_t sb_k;
     __device__ TensorKcLoader(const MttkrpArgs &g, int m0, int kt0)
         : safe(g.B), w(kt0, g.K, g.J, Cfg::BK), sb_k(g.sb_k) {
-        off = w.k * sb_k + w.j0;
+        base = reinterpret_cast<const char *>(g.B + (int64_t)m0 * g.sb_i + w.k * sb_k + w.j0);
 #pragma unroll
         for (int i = 0; i < Cfg::A_VEC; i++) {
             KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
             const bool ok = !EDGE || m0 + s.row < g.I;
-            p[i] = g.B + (int64_t)(ok ? m0 + s.row : 0) * g.sb_i + s.k;
+            off[i] = 4u * (uint32_t)((ok ? s.row : 0) * (int)g.sb_i + s.k);
         }
     }
     // EDGE: a row past I reads row 0 instead (it only feeds outputs that are never stored); only a
@@ -94,19 +95,22 @@ struct TensorKcLoader {
     static constexpr bool HAS_TAIL_FETCH = EDGE;
     template <int S>
     __device__ __forceinline__ void fetch() {
+        const __amdgpu_buffer_rsrc_t rsrc = whole_buffer(base);
 #pragma unroll
-        for (int i = 0; i < Cfg::A_VEC; i++) reg[S][i] = *reinterpret_cast<const v4f *>(p[i] + off);
+        for (int i = 0; i < Cfg::A_VEC; i++) reg[S][i] = buffer_load<v4f>(rsrc, off[i], 0u);
         const int kt_before = w.kt;
         const bool wrap = w.next(Cfg::BK, EDGE);
-        off += (w.kt != kt_before) ? (wrap ? sb_k - (w.J - Cfg::BK) : Cfg::BK) : 0;
+        const int64_t step = wrap ? sb_k - (w.J - Cfg::BK) : (int64_t)Cfg::BK;
+        base += w.kt != kt_before ? 4 * step : 0;
     }
     template <int S>
     __device__ __forceinline__ void fetch_tail() {
         const bool in = w.inside();
 #pragma unroll
-        for (int i = 0; i < Cfg::A_VEC; i++) reg[S][i] = load_or_zero(p[i] + (in ? off : 0), in, safe);
+        for (int i = 0; i < Cfg::A_VEC; i++)
+            reg[S][i] = load_or_zero(reinterpret_cast<const float *>(base + off[i]), in, safe);
         const bool wrap = w.next(Cfg::BK, true);
-        off += wrap ? sb_k - (w.J - Cfg::BK) : Cfg::BK;
+        base += 4 * (wrap ? sb_k - (w.J - Cfg::BK) : (int64_t)Cfg::BK);
     }
     template <int S>
     __device__ __forceinline__ void commit(float *stage) const {
@@ -133,7 +137,8 @@ struct KhatriRaoKcLoader {
     static constexpr int D_FLOATS = D_WIN * D_LD;
     static constexpr int EXTRA_DS_READ = Cfg::B_VEC;    // the D[k, r] factors
     static constexpr bool HAS_PAIR_HOOK = true;
-    const float *pc[Cfg::B_VEC];
+    const char *cbase;                                  // column n0 of C at j = 0, the same for every lane
+    uint32_t coff[Cfg::B_VEC];                          // the slot's (column, j) from there, bytes
     int dslot[Cfg::B_VEC];                              // the slot's column within the tile
     const float *safe;
     v4f reg[2][Cfg::B_VEC];
@@ -147,11 +152,12 @@ struct KhatriRaoKcLoader {
         : safe(g.C), w(kt0, g.K, g.J, Cfg::BK), D(g.D), sd_k(g.sd_k), sd_r(g.sd_r), dl(window), k_last(g.K - 1),
           n0(n0_), R(g.R) {
         kwin = w.k;
+        cbase = reinterpret_cast<const char *>(g.C + (int64_t)n0 * g.sc_r);
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             KcSlot<Cfg::BK> s(threadIdx.x + i * Cfg::NTHREADS);
-            const int r = (!EDGE || n0 + s.row < g.R) ? n0 + s.row : 0;
-            pc[i] = g.C + (int64_t)r * g.sc_r + s.k;
+            const int r = (!EDGE || n0 + s.row < g.R) ? s.row : 0;       // a column past R reads the tile's first
+            coff[i] = 4u * (uint32_t)(r * (int)g.sc_r + s.k);
             dslot[i] = s.row;
         }
     }
@@ -175,13 +181,14 @@ struct KhatriRaoKcLoader {
             __syncthreads();
         }
     }
-    static constexpr bool HAS_TAIL_FETCH = EDGE;   // as in TensorKcLoader; a column past R reads column 0
+    static constexpr bool HAS_TAIL_FETCH = EDGE;   // as in TensorKcLoader
     template <int S>
     __device__ __forceinline__ void fetch() {
         const float *row = dl + (w.k - kwin) * D_LD;
+        const __amdgpu_buffer_rsrc_t rsrc = whole_buffer(cbase);
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
-            reg[S][i] = *reinterpret_cast<const v4f *>(pc[i] + w.j0);
+            reg[S][i] = buffer_load<v4f>(rsrc, coff[i], 4u * (uint32_t)w.j0);
             dval[S][i] = row[dslot[i]];
         }
         w.next(Cfg::BK, EDGE);
@@ -192,7 +199,7 @@ struct KhatriRaoKcLoader {
         const float *row = dl + (w.k - kwin) * D_LD;
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
-            reg[S][i] = load_or_zero(pc[i] + (in ? w.j0 : 0), in, safe);
+            reg[S][i] = load_or_zero(reinterpret_cast<const float *>(cbase + coff[i]) + (in ? w.j0 : 0), in, safe);
             dval[S][i] = row[dslot[i]];
         }
         w.next(Cfg::BK, true);
@@ -318,7 +325,9 @@ static int launch_mttkrp(MttkrpArgs g, hipStream_t stream) {
 static bool mttkrp_fast(int I, int J, const int64_t *sb3, const int64_t *sc2, const int64_t *sd2,
                         const int64_t *sa2, const float *B, const float *C, const float *A) {
     (void)sd2;
+    // (the loaders reach a tile's rows with 32-bit offsets: see LOADER_MAX_LD, and j within a row of C likewise)
     return J % 16 == 0 && I % 4 == 0 && sb3[1] == 1 && sc2[0] == 1 && sa2[0] == 1 && sb3[0] % 4 == 0 &&
+           sb3[0] < LOADER_MAX_LD && sc2[1] < LOADER_MAX_LD && J < LOADER_MAX_LD &&
            sb3[2] % 4 == 0 && sc2[1] % 4 == 0 && sa2[1] % 4 == 0 && ((uintptr_t)B % 16 == 0) &&
            ((uintptr_t)C % 16 == 0) && ((uintptr_t)A % 16 == 0);
 }
