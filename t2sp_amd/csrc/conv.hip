@@ -37,6 +37,7 @@ struct ConvArgs {
     int nxcd;                   // dies the workgroup ids are dealt to (tile order)
     int p_begin;                // first output pixel this launch covers
     int splits;                 // workgroups per tile along the reduction (1 = none)
+    int wide_input;             // the input spans 2^30 elements or more: lanes need more than 32-bit byte offsets
     int Mp, Np;                 // padded extents of one partial plane (CO, pixels of this launch)
     float *scratch;
 };
@@ -130,15 +131,18 @@ struct Im2colRcLoader {
 
 // The same operand for tiles 256 pixels wide: a k-row of the tile is then 64 slots, one wave, so the
 // window position (ci, kh, kw) of a slot is the same for every lane of its wave.  It is walked with
-// counters in scalar registers (no table, no vector arithmetic): a lane keeps the address of its
-// pixel and adds the wave's offset ci * si_c + kh * si_h + kw to it, one vector instruction per
-// load as for a plain matrix.  (The per-lane walk above costs about ten per load, which the MFMA
-// pipe pays for: a wave issues them in the cycles it would issue MFMAs in.)
+// counters in scalar registers (no table, no vector arithmetic): a lane keeps the 32-bit offset of
+// its pixel from the tile's first and the wave's offset ci * si_c + kh * si_h + kw goes into the
+// buffer load as its scalar offset (see gemm_loaders.hpp).  (The per-lane walk above costs about
+// ten vector instructions per load, which the MFMA pipe pays for: a wave issues them in the cycles
+// it would issue MFMAs in.)  For inputs that span less than 2^30 elements (4 GiB); larger ones
+// take the loader above.
 template <class Cfg, bool EDGE>
 struct Im2colWaveRowLoader {
     static_assert((Cfg::BN / 4) % 64 == 0 && Cfg::BN / 4 == 64, "a k-row of the tile must be one wave");
     static constexpr int ROWS_APART = Cfg::NTHREADS / 64;   // k-rows between a thread's slots
-    const float *pix[Cfg::B_VEC];    // the lane's input pixel (n, h, w) at ci = kh = kw = 0
+    const char *input;               // the input tensor (the same for every lane)
+    uint32_t pix[Cfg::B_VEC];        // the lane's pixels (n, h, w) at ci = kh = kw = 0 from there, bytes
     int kh[Cfg::B_VEC], kw[Cfg::B_VEC];
     uint32_t off[Cfg::B_VEC];        // ci * si_c + kh * si_h + kw of the row this slot loads next
     v4f reg[2][Cfg::B_VEC];
@@ -158,15 +162,16 @@ struct Im2colWaveRowLoader {
         carry_w = (uint32_t)(g.si_h - g.KW);
         carry_h = (uint32_t)(g.si_c - g.KH * g.si_h);
         wave_k = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        const int hw = g.OH * g.OWp;
+        input = reinterpret_cast<const char *>(g.I);
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             RcSlot<Cfg::BN> s(threadIdx.x + i * Cfg::NTHREADS);
             int p = p0 + s.col;
             if (EDGE && p >= g.P) p = 0;
-            const int hw = g.OH * g.OWp;
             const int n = p / hw, rem = p - n * hw;
             const int h = rem / g.OWp, w = min(rem - h * g.OWp, g.OW - 4);
-            pix[i] = g.I + (n * g.si_n + h * g.si_h + w);
+            pix[i] = 4u * (uint32_t)(n * g.si_n + h * g.si_h + w);
             const int row = wave_k + i * ROWS_APART;
             const int q = (k_begin + row < g.KRED) ? k_begin + row : 0;
             const int c = q / win, r = q - c * win;
@@ -189,20 +194,22 @@ struct Im2colWaveRowLoader {
     template <int S>
     __device__ __forceinline__ void fetch() {
         const bool go = EDGE || k0 + 2 * Cfg::BK <= KRED;
+        const __amdgpu_buffer_rsrc_t rsrc = whole_buffer(input);
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
-            reg[S][i] = *reinterpret_cast<const v4f_u *>(pix[i] + off[i]);
+            reg[S][i] = buffer_load<v4f>(rsrc, pix[i], 4u * off[i]);
             advance(i, go);
         }
         k0 += go ? Cfg::BK : 0;
     }
     template <int S>
     __device__ __forceinline__ void fetch_tail() {
+        const __amdgpu_buffer_rsrc_t rsrc = whole_buffer(input);
 #pragma unroll
         for (int i = 0; i < Cfg::B_VEC; i++) {
             const bool ok = k0 + wave_k + i * ROWS_APART < KRED;
-            const v4f_u v = *reinterpret_cast<const v4f_u *>(pix[i] + (ok ? off[i] : 0u));
-            reg[S][i] = ok ? (v4f)v : v4f{0.f, 0.f, 0.f, 0.f};
+            const v4f v = buffer_load<v4f>(rsrc, pix[i], ok ? 4u * off[i] : 0u);
+            reg[S][i] = ok ? v : v4f{0.f, 0.f, 0.f, 0.f};
             advance(i, true);
         }
         k0 += Cfg::BK;
@@ -217,10 +224,10 @@ struct Im2colWaveRowLoader {
     }
 };
 
-template <class Cfg, bool EDGE>
-using Im2colLoaderFor = std::conditional_t<Cfg::BN == 256, Im2colWaveRowLoader<Cfg, EDGE>, Im2colRcLoader<Cfg, EDGE>>;
+template <class Cfg, bool EDGE, bool WIDE>
+using Im2colLoaderFor = std::conditional_t<Cfg::BN == 256 && !WIDE, Im2colWaveRowLoader<Cfg, EDGE>, Im2colRcLoader<Cfg, EDGE>>;
 
-template <class Cfg, bool EDGE>
+template <class Cfg, bool EDGE, bool WIDE>
 __global__ void __launch_bounds__(Cfg::NTHREADS) conv_kernel(const ConvArgs g) {
     extern __shared__ __align__(16) float smem[];
     int *tab = reinterpret_cast<int *>(smem + Cfg::SMEM_FLOATS);
@@ -233,7 +240,7 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) conv_kernel(const ConvArgs g) {
     int kt0 = 0, kt1 = ktiles_even<Cfg>(g.KRED);
     if (g.splits > 1) split_range((g.KRED + Cfg::BK - 1) / Cfg::BK, g.splits, split, kt0, kt1);
     RowMajorKcLoader<Cfg, EDGE> la(g.W, g.sw_o, co0, g.CO, g.KRED, kt0 * Cfg::BK);
-    Im2colLoaderFor<Cfg, EDGE> lb(g, p0, tab, kt0 * Cfg::BK);
+    Im2colLoaderFor<Cfg, EDGE, WIDE> lb(g, p0, tab, kt0 * Cfg::BK);
     Accum<Cfg> acc;
     mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem, tail_from_for<Cfg>(g.KRED - kt0 * Cfg::BK));
     if (g.splits > 1) {
@@ -291,7 +298,10 @@ static int launch_conv(ConvArgs g, int p_begin, int p_end, int splits, float *sc
     g.scratch = scratch;
     const bool edge = (g.CO % Cfg::BM) || ((p_end - p_begin) % Cfg::BN) || (g.KRED % (2 * Cfg::BK));
     const size_t smem = Cfg::SMEM_FLOATS * sizeof(float) + (size_t)g.KH * g.KW * sizeof(int);
-    auto kern = edge ? conv_kernel<Cfg, true> : conv_kernel<Cfg, false>;
+    void (*kern)(const ConvArgs) = edge ? conv_kernel<Cfg, true, false> : conv_kernel<Cfg, false, false>;
+    if constexpr (Cfg::BN == 256) {
+        if (g.wide_input) kern = edge ? conv_kernel<Cfg, true, true> : conv_kernel<Cfg, false, true>;
+    }
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
@@ -675,7 +685,7 @@ extern "C" int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, 
     // aligned 128-bit stores need rows that start on 16-byte boundaries; ragged rows use 4-byte aligned ones
     const bool out_ok = so4[3] == 1 && (ragged ? ((uintptr_t)O % 4 == 0)
                                                 : (so4[0] % 4 == 0 && so4[1] % 4 == 0 && so4[2] % 4 == 0 && (uintptr_t)O % 16 == 0));
-    const bool fast = cfg != T2SP_CFG_SCALAR && si4[3] == 1 && out_ok && w_dense && sw_o % 4 == 0 && sw_o < t2sp::LOADER_MAX_LD && OW >= 4 &&
+    const bool fast = cfg != T2SP_CFG_SCALAR && si4[3] == 1 && out_ok && w_dense && sw_o % 4 == 0 && sw_o < t2sp::LOADER_MAX_LD && si4[0] >= 0 && si4[1] >= 0 && si4[2] >= 0 && OW >= 4 &&
                       (int64_t)N * OH * owp <= INT32_MAX && (kred % 4 == 0 || padded) && KH * KW <= 4096 &&
                       in_span < INT32_MAX && ((uintptr_t)W % 16 == 0) && ((uintptr_t)I % 4 == 0);
     if (!fast) {
@@ -694,6 +704,7 @@ extern "C" int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, 
     g.so_n = so4[0]; g.so_c = so4[1]; g.so_h = so4[2];
     g.OWp = owp;
     g.P = N * OH * owp; g.KRED = CI * KH * KW;
+    g.wide_input = in_span >= (1 << 30);
     // the 16 x 16 form: reductions of whole steps of 16 whose offset table fits, byte offsets in 32 bits,
     // weight rows that start on 16-byte boundaries
     const bool d16_ok = g.KRED % 16 == 0 && g.KRED <= CONV_D16_MAX_KRED && in_span < (1 << 30) &&

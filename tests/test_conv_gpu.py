@@ -134,6 +134,34 @@ def test_one_launch_16x16_form_byte_offsets_above_two_gib():
     del buf
 
 
+@pytest.mark.parametrize("gap", [1_000_000_000, 1_200_000_000])
+def test_lds_tile_kernels_reach_images_gigabytes_apart(gap):
+    """Two images 4.0 and 4.8 GB apart inside one allocation, every tile size forced: below 2^30 elements
+    the 256-pixel tiles address the input with 32-bit byte offsets that come close to 2^32, above it
+    they take the loader that keeps wider offsets.  Integer data: exact."""
+    import ctypes
+    import torch
+    L = t2sp_amd.lib()
+    N, CI, CO, OH, OW = 2, 8, 48, 10, 16
+    per_image = CI * (OH + 2) * (OW + 2)
+    buf = torch.zeros(gap + per_image, device="cuda")
+    g = torch.Generator().manual_seed(4)
+    imgs = torch.randint(-2, 3, (N, CI, OH + 2, OW + 2), generator=g).float().cuda()
+    I = buf.as_strided((N, CI, OH + 2, OW + 2), (gap, (OH + 2) * (OW + 2), OW + 2, 1))
+    I.copy_(imgs)
+    W = torch.randint(-2, 3, (CO, CI, 3, 3), generator=g).float().cuda()
+    O = torch.full((N, CO, OH, OW), float("nan"), device="cuda")
+    want = torch.nn.functional.conv2d(imgs.double(), W.double())
+    i64 = ctypes.c_int64
+    si, sw, so = ((i64 * 4)(*t.stride()) for t in (I, W, O))
+    for cfg in (1, 2, 3, 0):
+        O.fill_(float("nan"))
+        assert L.t2sp_conv2d_f32(I.data_ptr(), W.data_ptr(), O.data_ptr(), N, CI, CO, OH, OW, 3, 3, si, sw, so, cfg, None, 0, None) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(O.double(), want), cfg
+    del buf
+
+
 def test_one_launch_16x16_form_refuses_what_it_cannot_address():
     """A reduction that is not a whole number of steps of 16 has no 16 x 16 form: forcing it is an error,
     the automatic choice takes another kernel."""
