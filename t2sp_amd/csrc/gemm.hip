@@ -916,12 +916,17 @@ static GemmD16Plan plan_gemm_d16(int M, int N) {
     best.cost = 1e300;
     for (int nb = 2; nb <= 4; nb += 2)
         for (int mb = 2; mb <= 8; mb++) {
-            if (mb * nb > 24) continue;                           // accumulators + operand ring must fit
+            if (mb * nb > 32) continue;                           // accumulators + operand ring must fit
             const int tiles_m = (M + 16 * mb - 1) / (16 * mb), tiles_n = (N + 16 * nb - 1) / (16 * nb);
             const int rpt = (M + tiles_m - 1) / tiles_m;
             const int64_t tiles = (int64_t)tiles_m * tiles_n;
             const double loads_per_mfma = (double)(mb + 4) / (4.0 * mb * nb);
-            const double cost = (double)((tiles + cus - 1) / cus) * (16.0 * mb) * (16.0 * nb) * (1.0 + 1.5 * loads_per_mfma);
+            // tiles of more than 24 blocks leave room for one workgroup per CU only (registers, and the LDS of the
+            // exchange), so a wave has its SIMD to itself and nothing covers its waits: measured 4 to 8 % slower at
+            // equal work (2048^3, 2304^3, 2048 x 1024 x 512), and 14 % faster where they save a round (1280^3:
+            // 240 tiles of 112 x 64 instead of 320 of 80 x 64, 42.9 -> 36.7 us)
+            const double alone = mb * nb > 24 ? 1.1 : 1.0;
+            const double cost = (double)((tiles + cus - 1) / cus) * (16.0 * mb) * (16.0 * nb) * (1.0 + 1.5 * loads_per_mfma) * alone;
             if (cost < best.cost) best = GemmD16Plan{mb, nb, rpt, tiles_m, tiles_n, cost};
         }
     return best;
@@ -956,7 +961,7 @@ static int launch_d16(const GemmArgs &g, hipStream_t stream) {
 #define T2SP_D16_CASE(MBV, NBV) if (p.mb == MBV && p.nb == NBV) return launch_d16_t<MBV, NBV>(g, p, stream);
     T2SP_D16_CASE(2, 2) T2SP_D16_CASE(3, 2) T2SP_D16_CASE(4, 2) T2SP_D16_CASE(5, 2) T2SP_D16_CASE(6, 2)
     T2SP_D16_CASE(7, 2) T2SP_D16_CASE(8, 2) T2SP_D16_CASE(2, 4) T2SP_D16_CASE(3, 4) T2SP_D16_CASE(4, 4)
-    T2SP_D16_CASE(5, 4) T2SP_D16_CASE(6, 4)
+    T2SP_D16_CASE(5, 4) T2SP_D16_CASE(6, 4) T2SP_D16_CASE(7, 4) T2SP_D16_CASE(8, 4)
 #undef T2SP_D16_CASE
     return T2SP_ERR_SHAPE;
 }
