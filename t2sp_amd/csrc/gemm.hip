@@ -407,11 +407,15 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     v4f *red = reinterpret_cast<v4f *>(smem);            // [wave][mb][nb][lane]
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
-    const int tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
+    // a grid of tiles_m x tiles_n: no division on the way to the first loads (every instruction before
+    // them is fetched through a cold instruction cache at each launch)
+    const int tm = blockIdx.x, tn = blockIdx.y;
+    (void)tiles_m;
     const int m0 = tm * rows_per_tile, n0 = tn * 16 * NB;
     const int m_end = min(m0 + rows_per_tile, M);
     const int steps = K >> 4;
-    const int s0 = (int)((int64_t)steps * wave / NW), s1 = (int)((int64_t)steps * (wave + 1) / NW);
+    static_assert(NW == 4, "shares of the reduction by shifts");
+    const int s0 = (steps * wave) >> 2, s1 = (steps * (wave + 1)) >> 2;
     const GemmHot hot{A, B, M, N, lda, ldb};
     sgemm_d16_wave<MB, NB, BUF>(hot, 0, m0, n0, s0, s1 - s0, steps, red + wave * MB * NB * 64);
     __syncthreads();
@@ -951,7 +955,8 @@ static int launch_d16_t(GemmArgs g, const GemmD16Plan &p, hipStream_t stream) {
     auto kern = buf ? sgemm_direct16_kernel<MB, NB, true> : sgemm_direct16_kernel<MB, NB, false>;
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(GEMM_D16_WAVES * 64), smem, stream, g.A, g.B, g.M, g.N, g.K,
+    if (p.tiles_n > 65535) return T2SP_ERR_SHAPE;
+    hipLaunchKernelGGL(kern, dim3(p.tiles_m, p.tiles_n), dim3(GEMM_D16_WAVES * 64), smem, stream, g.A, g.B, g.M, g.N, g.K,
                        (int)g.lda, (int)g.ldb, p.tiles_m, p.rows_per_tile, g);
     return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
 }
