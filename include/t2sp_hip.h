@@ -42,7 +42,9 @@ extern "C" {
  * kernels of t2s/tests/performance/gemm/bitstream/a10/a.cl:67-770 launched by
  * halide_opencl_wait_for_kernels_finish (t2s/src/AOT-OpenCL-Runtime.cpp:312-397).
  * `workspace` is optional (NULL allowed): products with fewer output tiles than CUs use it
- * (t2sp_sgemm_workspace_bytes) to split the reduction over more workgroups. */
+ * (t2sp_sgemm_workspace_bytes) to split the reduction over more workgroups: the last, partial
+ * round of the large tiles, and outputs of a few small tiles with a long reduction
+ * (256 x 256 x 16384: 34 us with it, 88 us without). */
 size_t t2sp_sgemm_workspace_bytes(int M, int N, int K);
 int t2sp_sgemm_f32(const float *A, const float *B, float *C, int M, int N, int K, int64_t lda,
                    int64_t ldb, int64_t ldc, int cfg, float *workspace, size_t workspace_bytes,

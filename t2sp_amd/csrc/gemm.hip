@@ -399,7 +399,7 @@ __device__ __forceinline__ void sgemm_d16_wave(const GemmHot &g, int mb0, int m0
 
 template <int MB, int NB, bool BUF>
 __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
-    sgemm_direct16_kernel(const float *A, const float *B, int M, int N, int K, int lda, int ldb, int tiles_m, int rows_per_tile,
+    sgemm_direct16_kernel(const float *A, const float *B, int M, int N, int K, int lda, int ldb, int split_shift, int rows_per_tile,
                           const GemmArgs g) {
     typedef typename VecOf<NB>::type vnb;
     constexpr int NW = GEMM_D16_WAVES;
@@ -410,12 +410,14 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     // a grid of tiles_m x tiles_n: no division on the way to the first loads (every instruction before
     // them is fetched through a cold instruction cache at each launch)
     const int tm = blockIdx.x, tn = blockIdx.y;
-    (void)tiles_m;
     const int m0 = tm * rows_per_tile, n0 = tn * 16 * NB;
     const int m_end = min(m0 + rows_per_tile, M);
     const int steps = K >> 4;
+    // blockIdx.z: the workgroup's share of the reduction when it is split over 2^split_shift
+    // workgroups per tile (tiny outputs with a long reduction); its waves split that share again
     static_assert(NW == 4, "shares of the reduction by shifts");
-    const int s0 = (steps * wave) >> 2, s1 = (steps * (wave + 1)) >> 2;
+    const int z0 = (int)(((int64_t)steps * blockIdx.z) >> split_shift), z1 = (int)(((int64_t)steps * (blockIdx.z + 1)) >> split_shift);
+    const int s0 = z0 + (((z1 - z0) * wave) >> 2), s1 = z0 + (((z1 - z0) * (wave + 1)) >> 2);
     const GemmHot hot{A, B, M, N, lda, ldb};
     sgemm_d16_wave<MB, NB, BUF>(hot, 0, m0, n0, s0, s1 - s0, steps, red + wave * MB * NB * 64);
     __syncthreads();
@@ -439,6 +441,11 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
 #pragma unroll
             for (int nb = 0; nb < NB; nb++) out[nb] = sum[nb][r];
             if (row < m_end && col_ok) {
+                if (split_shift) {
+                    // a partial sum: plane blockIdx.z of the workspace, M x N; the kernel that adds the planes scales and stores
+                    *reinterpret_cast<vnb *>(g.scratch + ((int64_t)blockIdx.z * M + row) * N + col) = out;
+                    continue;
+                }
                 if (g.scale) {
                     out = out * g.alpha;
                     if (g.beta != 0.f) out += *reinterpret_cast<const vnb *>(g.Cin + (int64_t)row * g.ldcin + col) * g.beta;
@@ -936,6 +943,38 @@ static GemmD16Plan plan_gemm_d16(int M, int N) {
     return best;
 }
 
+// Tiny outputs with a long reduction: the tiles of the plan above leave most CUs idle, so each goes
+// to 2^shift workgroups that each reduce a share of k into a plane of the workspace, and a second
+// kernel adds the planes in order.  As many shares as fit one round of workgroups and leave each
+// workgroup 32 steps of 16 k (8 per wave) or more; not at all where the time saved would not pay
+// for the second launch.  Measured with every tile and split forced (256 x 256 x 16384,
+// 128 x 128 x 4096, 64 x 64 x 65536, ...): the small tiles of the plan above, split this way, are
+// within a few per cent of the best choice everywhere, and larger tiles with deeper splits are not
+// better: a step costs its MFMAs or its loads whichever is longer, and with few tiles the time is
+// that of one workgroup.
+struct GemmD16Split {
+    int shift;                 // 0: no split
+    size_t scratch_bytes;
+};
+static GemmD16Split plan_gemm_d16_split(int M, int N, int K, const GemmD16Plan &p) {
+    const int cus = machine().cus;
+    const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+    GemmD16Split r{0, 0};
+    if (tiles <= 0 || tiles > cus / 2 || K % 16) return r;
+    const int steps = K / 16;
+    int shift = 0;
+    while (shift < 5 && (tiles << (shift + 1)) <= cus && (steps >> (shift + 1)) >= 32) shift++;
+    if (!shift) return r;
+    // a step of the tile: its MFMAs (16 x 16 x 4, 32 cycles each) or its loads (measured 0.345 us for 32 x 32)
+    const double mfma_us = 4.0 * p.mb * p.nb * 32.0 / 2400.0 * 1.03, load_us = (p.mb + 4) * 0.0575;
+    const double step_us = mfma_us > load_us ? mfma_us : load_us;
+    const double saved_us = (steps / 4.0) * step_us * (1.0 - 1.0 / (1 << shift));
+    if (saved_us < 8.0) return r;                                         // the second launch and its pass over the planes
+    r.shift = shift;
+    r.scratch_bytes = ((size_t)M * N << shift) * sizeof(float);
+    return r;
+}
+
 static bool gemm_d16_ok(const GemmArgs &g) {
     return g.K % 16 == 0 && g.N % 4 == 0 && g.ldb % 4 == 0 && (g.tiled || g.ldc % 4 == 0) && g.lda % 4 == 0 &&
            ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) && ((uintptr_t)g.C % 16 == 0) &&
@@ -944,9 +983,10 @@ static bool gemm_d16_ok(const GemmArgs &g) {
 }
 
 template <int MB, int NB>
-static int launch_d16_t(GemmArgs g, const GemmD16Plan &p, hipStream_t stream) {
+static int launch_d16_t(GemmArgs g, const GemmD16Plan &p, hipStream_t stream, int split_shift = 0, float *scratch = nullptr) {
     g.tiles_m = p.tiles_m;
     g.tiles_n = p.tiles_n;
+    g.scratch = scratch;
     const size_t smem = (size_t)GEMM_D16_WAVES * MB * NB * 64 * sizeof(v4f);
     // one workgroup per CU at most, or a short reduction: the form whose loop has no vector arithmetic
     // (see sgemm_d16_wave; measured with several rounds: 2048 x 1024 x 512 20.7 -> 18.8 us,
@@ -956,14 +996,22 @@ static int launch_d16_t(GemmArgs g, const GemmD16Plan &p, hipStream_t stream) {
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
     if (p.tiles_n > 65535) return T2SP_ERR_SHAPE;
-    hipLaunchKernelGGL(kern, dim3(p.tiles_m, p.tiles_n), dim3(GEMM_D16_WAVES * 64), smem, stream, g.A, g.B, g.M, g.N, g.K,
-                       (int)g.lda, (int)g.ldb, p.tiles_m, p.rows_per_tile, g);
-    return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3(p.tiles_m, p.tiles_n, 1 << split_shift), dim3(GEMM_D16_WAVES * 64), smem, stream, g.A, g.B, g.M,
+                       g.N, g.K, (int)g.lda, (int)g.ldb, split_shift, p.rows_per_tile, g);
+    if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
+    if (split_shift) {
+        GemmOutMap map{g};
+        if (launch_splitk_reduce<true>(scratch, 1 << split_shift, g.M, g.N, map, stream) != hipSuccess) return T2SP_ERR_LAUNCH;
+    }
+    return T2SP_OK;
 }
 
-static int launch_d16(const GemmArgs &g, hipStream_t stream) {
+static int launch_d16(const GemmArgs &g, hipStream_t stream, float *workspace = nullptr, size_t workspace_bytes = 0) {
     const GemmD16Plan p = plan_gemm_d16(g.M, g.N);
-#define T2SP_D16_CASE(MBV, NBV) if (p.mb == MBV && p.nb == NBV) return launch_d16_t<MBV, NBV>(g, p, stream);
+    GemmD16Split sp = plan_gemm_d16_split(g.M, g.N, g.K, p);
+    if (!workspace || workspace_bytes < sp.scratch_bytes || ((uintptr_t)workspace % 16)) sp.shift = 0;
+    const int shift = sp.shift;
+#define T2SP_D16_CASE(MBV, NBV) if (p.mb == MBV && p.nb == NBV) return launch_d16_t<MBV, NBV>(g, p, stream, shift, workspace);
     T2SP_D16_CASE(2, 2) T2SP_D16_CASE(3, 2) T2SP_D16_CASE(4, 2) T2SP_D16_CASE(5, 2) T2SP_D16_CASE(6, 2)
     T2SP_D16_CASE(7, 2) T2SP_D16_CASE(8, 2) T2SP_D16_CASE(2, 4) T2SP_D16_CASE(3, 4) T2SP_D16_CASE(4, 4)
     T2SP_D16_CASE(5, 4) T2SP_D16_CASE(6, 4) T2SP_D16_CASE(7, 4) T2SP_D16_CASE(8, 4)
@@ -1075,7 +1123,7 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
     }
     if (cfg == T2SP_CFG_DIRECT16) {
         if (bt) return gemm_d16_bt_ok(g) ? launch_d16_bt(g, stream) : T2SP_ERR_SHAPE;
-        return gemm_d16_ok(g) ? launch_d16(g, stream) : T2SP_ERR_SHAPE;
+        return gemm_d16_ok(g) ? launch_d16(g, stream, workspace, workspace_bytes) : T2SP_ERR_SHAPE;
     }
     if (cfg == T2SP_CFG_AUTO && (bt ? gemm_d16_bt_ok(g) : gemm_d16_ok(g))) {
         // Measured from 256^2 x 8192 to 3072^2 x 1024: the 16 x 16 form wins whenever 256 x 256 tiles
@@ -1094,8 +1142,15 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         // whole rounds of 128 x 128 tiles are 4-10 % ahead of it (1024 x 4096 x 512, 2048^3, 4096 x 1024 x 1024).
         const bool tiled_better = (t128 >= 2 * cus - cus / 16 && g.K >= 2048 && fill128 >= 0.6) ||
                                   (bt && t128 % cus == 0 && fill128 >= 0.9);
-        const bool too_few = (int64_t)p.tiles_m * p.tiles_n < cus / 2 && g.K >= 4096;
-        if (!big_tiles && !tiled_better && !too_few && g.K >= 64) return bt ? launch_d16_bt(g, stream) : launch_d16(g, stream);
+        // (with room for the planes the 16 x 16 form splits such a reduction over workgroups itself)
+        const GemmD16Split sp = plan_gemm_d16_split(g.M, g.N, g.K, p);
+        const bool can_split = !bt && sp.shift && workspace && workspace_bytes >= sp.scratch_bytes && ((uintptr_t)workspace % 16 == 0);
+        // (without it, and without room for the planes of the LDS tiles' split either, it still has more tiles to
+        // spread over the CUs than they have)
+        const bool lds_split = workspace && workspace_bytes >= plan_gemm(g.M, g.N, g.K).scratch_bytes;
+        const bool too_few = (int64_t)p.tiles_m * p.tiles_n < cus / 2 && g.K >= 4096 && !can_split && lds_split;
+        if (!big_tiles && !tiled_better && !too_few && g.K >= 64)
+            return bt ? launch_d16_bt(g, stream) : launch_d16(g, stream, workspace, workspace_bytes);
     }
     if ((cfg == T2SP_CFG_AUTO || cfg == T2SP_CFG_DIRECT) && !bt && !g.scale && !g.tiled &&
         g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && gemm_direct_ok(g, cfg == T2SP_CFG_DIRECT))
@@ -1199,7 +1254,11 @@ extern "C" int t2sp_sgemm_tail_from(int k_len) { return t2sp::tail_from_for<t2sp
 
 extern "C" size_t t2sp_sgemm_workspace_bytes(int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
-    if (K % 4 == 0 && N % 4 == 0) return t2sp::plan_gemm(M, N, K).scratch_bytes;
+    if (K % 4 == 0 && N % 4 == 0) {
+        const size_t tiled = t2sp::plan_gemm(M, N, K).scratch_bytes;
+        const size_t one_launch = t2sp::plan_gemm_d16_split(M, N, K, t2sp::plan_gemm_d16(M, N)).scratch_bytes;
+        return tiled > one_launch ? tiled : one_launch;
+    }
     // padded copies of the operands, then the planes for the padded product
     return t2sp::gemm_pad_bytes(M, N, K, false) +
            t2sp::plan_gemm(M, (int)t2sp::round_up4(N), (int)t2sp::pad_k(K)).scratch_bytes;

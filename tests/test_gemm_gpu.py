@@ -308,6 +308,43 @@ def test_direct16_kernel_small_products(oracle, torch_cuda, shape):
                             None) == -8
 
 
+@pytest.mark.parametrize("shape", [(256, 256, 16384), (128, 128, 4096), (100, 132, 4096), (64, 64, 32768), (40, 520, 2048)])
+def test_tiny_outputs_split_their_reduction_over_workgroups(oracle, torch_cuda, shape):
+    """Outputs of a few tiles with a long reduction: given the workspace the library asks for, every tile
+    goes to several workgroups that reduce a share of k each, and a second kernel adds their planes; the
+    same call without a workspace runs unsplit.  Integer data: both exact, also through the BLAS form
+    with alpha, beta and a tiled output; uniform data against the oracle."""
+    torch = torch_cuda
+    import ctypes
+    M, N, K = shape
+    L = t2sp_amd.lib()
+    L.t2sp_sgemm_workspace_bytes.restype = ctypes.c_size_t
+    nbytes = L.t2sp_sgemm_workspace_bytes(M, N, K)
+    assert nbytes >= 2 * M * N * 4                     # at least two planes
+    ws = torch.empty(nbytes // 4, device="cuda")
+    g = torch.Generator().manual_seed(M + K)
+    A = torch.randint(-2, 3, (M, K), generator=g).float().cuda()
+    B = torch.randint(-2, 3, (K, N), generator=g).float().cuda()
+    C0 = torch.randint(-4, 5, (M, N), generator=g).float().cuda()
+    want = A.double() @ B.double()
+    for w, nb in ((ws.data_ptr(), nbytes), (None, 0)):
+        C = torch.full((M, N), float("nan"), device="cuda")
+        assert L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, w, nb, None) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(C.double(), want)
+        C.copy_(C0)
+        assert L.t2sp_sgemm_ex_f32(0, 0, M, N, K, 2.0, A.data_ptr(), K, B.data_ptr(), N, -3.0, C.data_ptr(), N, C.data_ptr(), N,
+                                   0, w, nb, None) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(C.double(), 2.0 * want - 3.0 * C0.double())
+    Au = t2sp_amd.fill_uniform(torch.empty(M, K, device="cuda"), 31)
+    Bu = t2sp_amd.fill_uniform(torch.empty(K, N, device="cuda"), 32)
+    C = torch.empty(M, N, device="cuda")
+    assert L.t2sp_sgemm_f32(Au.data_ptr(), Bu.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, ws.data_ptr(), nbytes, None) == 0
+    torch.cuda.synchronize()
+    assert rel_fro(C.cpu().numpy(), oracle.gemm(Au.cpu().numpy(), Bu.cpu().numpy()))[0] <= TOL
+
+
 def test_empty_extents():
     C = np.full((16, 8), np.nan, np.float32)
     t2sp_amd.gemm(np.zeros((16, 0), np.float32), np.zeros((0, 8), np.float32), out=C)
