@@ -286,8 +286,11 @@ template <> struct VecOf<4> { typedef float type __attribute__((ext_vector_type(
 // `make trace-lib`; python -m t2sp_amd.d16_timeline reads them back.
 #ifdef T2SP_D16_TRACE
 __device__ long long g_d16_trace[4096 * 8 * 8];
-#define T2SP_TRACE_STAMP(i) \
-    if ((threadIdx.x & 63) == 0 && blockIdx.x < 4096) g_d16_trace[(blockIdx.x * 8 + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64();
+#define T2SP_TRACE_STAMP(i)                                                                          \
+    {                                                                                                \
+        const unsigned wg = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);          \
+        if ((threadIdx.x & 63) == 0 && wg < 4096) g_d16_trace[(wg * 8 + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64(); \
+    }
 #else
 #define T2SP_TRACE_STAMP(i)
 #endif
