@@ -349,6 +349,30 @@ def sgemm_transposed_1024(torch, steps, warmup, peak, transa, transb):
                   workload="C = %s * %s, M=N=K=1024, one launch" % ("A^T" if transa else "A", "B^T" if transb else "B"))
 
 
+def sgemm_tiny_output(torch, steps, warmup, peak):
+    """An output of 64 small tiles with a long reduction: with the workspace the library asks for, the reduction is
+    split over the workgroups of one launch and a second kernel adds the planes."""
+    import ctypes
+    L = lib()
+    L.t2sp_sgemm_workspace_bytes.restype = ctypes.c_size_t
+    M = N = 256
+    K = 16384
+    A = ops.fill_uniform(torch.empty(M, K, device="cuda"), 1)
+    B = ops.fill_uniform(torch.empty(K, N, device="cuda"), 2)
+    C = torch.empty(M, N, device="cuda")
+    nbytes = L.t2sp_sgemm_workspace_bytes(M, N, K)
+    ws = torch.empty(max(nbytes // 4, 1), device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        rc = L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, ws.data_ptr(), nbytes, s)
+        assert rc == 0, rc
+
+    ms = _time(torch, launch, max(steps, 200), max(warmup, 20))
+    return _entry(2.0 * M * N * K / ms / 1e9, peak, ms,
+                  workload="C = A * B, M=N=256, K=16384, reduction split over workgroups, planes summed by a second kernel")
+
+
 def copy_rate(torch):
     """What a plain device-to-device copy of 256 MiB reaches on this box (torch's copy kernel; read + write
     bytes per second): the measured ceiling next to the nominal 8 TB/s that `frac_of_hbm_peak` of the three
@@ -377,6 +401,7 @@ def _run_all(torch, steps, warmup, peak, capsule_cfg=0, capsule_splits=0):
             "conv2d_n32_256ch_14x14": conv_small(torch, steps, warmup, peak),
             "sgemm_1024_b_transposed": sgemm_transposed_1024(torch, steps, warmup, peak, 0, 1),
             "sgemm_1024_a_transposed": sgemm_transposed_1024(torch, steps, warmup, peak, 1, 0),
+            "sgemm_256x256x16384": sgemm_tiny_output(torch, steps, warmup, peak),
             "capsule": capsule_config4(torch, steps, warmup, peak, capsule_cfg, capsule_splits),
             "mttkrp": mttkrp_config5(torch, steps, warmup, peak),
             "ssyrk_8192": ssyrk_case(torch, steps, warmup, peak, 8192, 8192, ""),
