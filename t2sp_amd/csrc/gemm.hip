@@ -423,12 +423,31 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     const int s0 = z0 + (((z1 - z0) * wave) >> 2), s1 = z0 + (((z1 - z0) * (wave + 1)) >> 2);
     const GemmHot hot{A, B, M, N, lda, ldb};
     sgemm_d16_wave<MB, NB, BUF>(hot, 0, m0, n0, s0, s1 - s0, steps, red + wave * MB * NB * 64);
+    const int col = n0 + NB * li;
+    const bool col_ok = col + NB <= N;
+    // beta * Cin: requested before the exchange, so that its latency passes behind it (an element is read
+    // and written by its own workgroup only, so C may be updated in place)
+    constexpr int PER_WAVE = (MB + NW - 1) / NW;
+    vnb cin[PER_WAVE][4];
+    const bool with_cin = g.scale && g.beta != 0.f && !split_shift;
+    if (with_cin) {
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; i++) {
+            const int mb = wave + i * NW;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int row = m0 + 16 * mb + 4 * lq + r;
+                if (mb < MB && row < m_end && col_ok) cin[i][r] = *reinterpret_cast<const vnb *>(g.Cin + (int64_t)row * g.ldcin + col);
+            }
+        }
+    }
     __syncthreads();
     T2SP_TRACE_STAMP(5)
     // sum the partial tiles of the waves in wave order
-    const int col = n0 + NB * li;
-    const bool col_ok = col + NB <= N;
-    for (int mb = wave; mb < MB; mb += NW) {
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; i++) {
+        const int mb = wave + i * NW;
+        if (mb >= MB) break;
         v4f sum[NB];
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) {
@@ -451,7 +470,7 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
                 }
                 if (g.scale) {
                     out = out * g.alpha;
-                    if (g.beta != 0.f) out += *reinterpret_cast<const vnb *>(g.Cin + (int64_t)row * g.ldcin + col) * g.beta;
+                    if (g.beta != 0.f) out += cin[i][r] * g.beta;
                 }
                 if (!g.tiled) {
                     *reinterpret_cast<vnb *>(g.C + (int64_t)row * g.ldc + col) = out;
