@@ -569,11 +569,27 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
         for (int nb = 0; nb < NB; nb++)
 #pragma unroll
             for (int r = 0; r < 4; r++) mine[(mb * NB + nb) * BLK + r * 16] = acc[mb][nb][r];
-    __syncthreads();
     const int orow = lane >> 2, ocol = (lane & 3) * 4;              // this lane's row and first column inside a block
     const bool vec_ok = !g.tiled && g.ldc % 4 == 0 && ((uintptr_t)g.C % 16 == 0) &&
                         (!g.scale || g.beta == 0.f || (g.ldcin % 4 == 0 && ((uintptr_t)g.Cin % 16 == 0)));
-    for (int pr = wave; pr < MB * NB; pr += NW) {        // sum the partial blocks of the waves in wave order
+    // beta * Cin of this wave's blocks: requested before the exchange (see sgemm_direct16_kernel)
+    constexpr int PER_WAVE = (MB * NB + NW - 1) / NW;
+    v4f cin[PER_WAVE];
+    const bool with_cin = vec_ok && g.scale && g.beta != 0.f;
+    if (with_cin) {
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; i++) {
+            const int pr = wave + i * NW;
+            const int mb = pr / NB, nb = pr - mb * NB;
+            const int row = m0 + 16 * mb + orow, col = n0 + 16 * nb + ocol;
+            if (pr < MB * NB && row < m_end && col + 4 <= N) cin[i] = *reinterpret_cast<const v4f *>(g.Cin + (int64_t)row * g.ldcin + col);
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; i++) {                 // sum the partial blocks of the waves in wave order
+        const int pr = wave + i * NW;
+        if (pr >= MB * NB) break;
         const v4f *src = reinterpret_cast<const v4f *>(smem + pr * BLK + orow * 16 + 16 * (orow >> 2) + ocol);
         v4f sum = src[0];
 #pragma unroll
@@ -585,7 +601,7 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
             v4f out = sum;
             if (g.scale) {
                 out = out * g.alpha;
-                if (g.beta != 0.f) out += *reinterpret_cast<const v4f *>(g.Cin + (int64_t)row * g.ldcin + col) * g.beta;
+                if (g.beta != 0.f) out += cin[i] * g.beta;
             }
             *reinterpret_cast<v4f *>(g.C + (int64_t)row * g.ldc + col) = out;
         } else {
@@ -683,9 +699,20 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     for (int mb = 0; mb < MB; mb++)
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) mine[(mb * NB + nb) * 64] = acc[mb][nb];
+    // block (mb, nb), register r of lane (li, lq) is row m0 + MB * (4 lq + r) + mb, column n0 + 4 li + nb.
+    // beta * Cin is requested before the exchange (see sgemm_direct16_kernel); MB <= NW: one row block per wave
+    static_assert(MB <= NW, "a wave sums one row block");
+    v4f cin[4];
+    const bool with_cin = g.scale && g.beta != 0.f && wave < MB;
+    if (with_cin) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int orow = m0 + MB * (4 * lq + r) + wave;
+            if (orow < M && col_ok) cin[r] = *reinterpret_cast<const v4f *>(g.Cin + (int64_t)orow * g.ldcin + col);
+        }
+    }
     __syncthreads();
-    // sum the partial tiles of the waves in wave order; block (mb, nb), register r of lane (li, lq) is
-    // row m0 + MB * (4 lq + r) + mb, column n0 + 4 li + nb
+    // sum the partial tiles of the waves in wave order
     for (int mb = wave; mb < MB; mb += NW) {
         v4f sum[NB];
 #pragma unroll
@@ -702,7 +729,7 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
             if (orow < M && col_ok) {
                 if (g.scale) {
                     out = out * g.alpha;
-                    if (g.beta != 0.f) out += *reinterpret_cast<const v4f *>(g.Cin + (int64_t)orow * g.ldcin + col) * g.beta;
+                    if (g.beta != 0.f) out += cin[r] * g.beta;
                 }
                 *reinterpret_cast<v4f *>(g.C + (int64_t)orow * g.ldc + col) = out;
             }
