@@ -327,7 +327,7 @@ constexpr int CONV_D16_WAVES = 4;
 constexpr int CONV_D16_RING = 3;
 constexpr int CONV_D16_MAX_KRED = 8192;      // the offset table: 32 KB of LDS
 
-template <int MB>
+template <int MB, bool BUF>
 __global__ void __launch_bounds__(CONV_D16_WAVES * 64) conv_direct16_kernel(const ConvArgs g, int rows_per_tile) {
     constexpr int NW = CONV_D16_WAVES, R = CONV_D16_RING, NB = 4;
     extern __shared__ __align__(16) float smem[];
@@ -365,6 +365,8 @@ __global__ void __launch_bounds__(CONV_D16_WAVES * 64) conv_direct16_kernel(cons
     const char *a_base = reinterpret_cast<const char *>(g.W + 16 * s0);
     const char *b_base = reinterpret_cast<const char *>(g.I);
     const int *my_tab = tab + 16 * s0 + 4 * lq;
+    // BUF: the weights through buffer loads, their step as the scalar offset (see sgemm_d16_wave in gemm.hip)
+    const __amdgpu_buffer_rsrc_t a_rsrc = whole_buffer(a_base);
     int issued = 0;
 
     v4f ra[R][MB];
@@ -380,7 +382,8 @@ __global__ void __launch_bounds__(CONV_D16_WAVES * 64) conv_direct16_kernel(cons
         _Pragma("unroll") for (int j = 0; j < 4; j++)                                               \
             rb[d][j] = *reinterpret_cast<const v4f_u *>(b_base + (b_off + (uint32_t)tcur[j]));      \
         _Pragma("unroll") for (int mb = 0; mb < MB; mb++)                                           \
-            ra[d][mb] = *reinterpret_cast<const v4f *>(a_base + (a_off[mb] + ao));                  \
+            ra[d][mb] = BUF ? buffer_load<v4f>(a_rsrc, a_off[mb], ao)                               \
+                            : *reinterpret_cast<const v4f *>(a_base + (a_off[mb] + ao));            \
         tcur = *reinterpret_cast<const v4i *>(my_tab + 16 * st_next);                               \
     }
 #define T2SP_CONV_D16_MMA(d)                                                                        \
@@ -478,7 +481,8 @@ static int launch_conv_d16_t(ConvArgs g, const ConvD16Plan &p, hipStream_t strea
     g.tiles_m = p.tiles_m;
     g.tiles_n = p.tiles_n;
     const size_t smem = (size_t)CONV_D16_WAVES * MB * 4 * 64 * sizeof(v4f) + (size_t)g.KRED * sizeof(int);
-    auto kern = conv_direct16_kernel<MB>;
+    const bool buf = (int64_t)p.tiles_m * p.tiles_n <= machine().cus || g.KRED <= 1024;   // as for the SGEMM of this form
+    auto kern = buf ? conv_direct16_kernel<MB, true> : conv_direct16_kernel<MB, false>;
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(CONV_D16_WAVES * 64), smem, stream, g, p.rows_per_tile);
