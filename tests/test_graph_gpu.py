@@ -34,9 +34,10 @@ def replays_equal(torch, launch_on, out):
     return True
 
 
-@pytest.mark.parametrize("shape", [(1024, 1024, 512), (3072, 3072, 256), (2304, 2560, 192), (516, 260, 100)])
+@pytest.mark.parametrize("shape", [(1024, 1024, 512), (3072, 3072, 256), (2304, 2560, 192), (516, 260, 100), (128, 192, 4096)])
 def test_sgemm_in_a_graph(shape):
-    """The 16 x 16 form, whole rounds followed by split tiles with their sum kernel, ragged tiles."""
+    """The 16 x 16 form, whole rounds followed by split tiles with their sum kernel, ragged tiles, a tiny output
+    whose reduction the 16 x 16 form splits over workgroups."""
     import torch
     L = t2sp_amd.lib()
     M, N, K = shape
