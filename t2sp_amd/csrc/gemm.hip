@@ -1342,8 +1342,10 @@ extern "C" size_t t2sp_sgemm_ex_workspace_bytes(int transa, int M, int N, int K)
     const size_t pad_t = t2sp::gemm_pad_bytes(M, N, K, true), pad_n = t2sp::gemm_pad_bytes(M, N, K, false);
     const bool padded = K % 4 || N % 4;
     const size_t pad = padded ? (pad_t > pad_n ? pad_t : pad_n) : 0;
-    return t2sp::round_up256(transa ? (size_t)M * K * sizeof(float) : 0) + pad +
-           t2sp::plan_gemm(M, (int)t2sp::round_up4(N), (int)(padded ? t2sp::pad_k(K) : K)).scratch_bytes;
+    const int n4 = (int)t2sp::round_up4(N), k4 = (int)(padded ? t2sp::pad_k(K) : K);
+    const size_t tiled = t2sp::plan_gemm(M, n4, k4).scratch_bytes;
+    const size_t one_launch = t2sp::plan_gemm_d16_split(M, n4, k4, t2sp::plan_gemm_d16(M, n4)).scratch_bytes;
+    return t2sp::round_up256(transa ? (size_t)M * K * sizeof(float) : 0) + pad + (tiled > one_launch ? tiled : one_launch);
 }
 
 extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, float alpha, const float *A,

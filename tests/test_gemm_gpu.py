@@ -319,8 +319,10 @@ def test_tiny_outputs_split_their_reduction_over_workgroups(oracle, torch_cuda, 
     M, N, K = shape
     L = t2sp_amd.lib()
     L.t2sp_sgemm_workspace_bytes.restype = ctypes.c_size_t
+    L.t2sp_sgemm_ex_workspace_bytes.restype = ctypes.c_size_t
     nbytes = L.t2sp_sgemm_workspace_bytes(M, N, K)
     assert nbytes >= 2 * M * N * 4                     # at least two planes
+    assert L.t2sp_sgemm_ex_workspace_bytes(0, M, N, K) >= nbytes
     ws = torch.empty(nbytes // 4, device="cuda")
     g = torch.Generator().manual_seed(M + K)
     A = torch.randint(-2, 3, (M, K), generator=g).float().cuda()
