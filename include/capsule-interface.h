@@ -48,6 +48,13 @@ int capsule(struct halide_buffer_t *P, struct halide_buffer_t *W, struct halide_
  * i-th argument, a buffer argument being the halide_buffer_t* itself. */
 int capsule_argv(void **args);
 
+/* The argument table Halide declares next to every generated entry
+ * (Halide/src/CodeGen_C.cpp:1830-1833; struct halide_filter_metadata_t,
+ * Halide/src/runtime/HalideRuntime.h:1653-1675): name, kind, rank and element type of each
+ * argument in call order, the entry's name, and "hip-gfx950" as the target.  The arguments are
+ * listed with the ranks of the FPGA flow (2, 2, 10; capsule-run-fpga.cpp:49-73); capsule() also takes the other forms above. */
+const struct halide_filter_metadata_t *capsule_metadata(void);
+
 /* States the design constant CII (capsule/const-parameters.h:31-70: 4 for the GPU and TINY sets, 32
  * for S10, 16 for A10) that the packed form of capsule() needs; 0 clears it.  Returns the previous
  * value.  Process-wide; no counterpart in the reference, where CII is compiled into the pipeline. */

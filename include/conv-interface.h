@@ -35,6 +35,13 @@ int conv(struct halide_buffer_t *I, struct halide_buffer_t *K, struct halide_buf
  * i-th argument, a buffer argument being the halide_buffer_t* itself. */
 int conv_argv(void **args);
 
+/* The argument table Halide declares next to every generated entry
+ * (Halide/src/CodeGen_C.cpp:1830-1833; struct halide_filter_metadata_t,
+ * Halide/src/runtime/HalideRuntime.h:1653-1675): name, kind, rank and element type of each
+ * argument in call order, the entry's name, and "hip-gfx950" as the target.  The arguments are
+ * listed with the ranks of the FPGA flow (2, 2, 10; conv-run-fpga.cpp:49-68); conv() also takes the other forms above. */
+const struct halide_filter_metadata_t *conv_metadata(void);
+
 /* States TOTAL_OY for packed inputs with the 2-D output when the map is not square (0 clears it;
  * also read from the environment variable T2SP_CONV_TOTAL_OY).  Returns the previous value.  No
  * counterpart in the reference, where the map size is compiled into the pipeline. */

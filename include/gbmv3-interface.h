@@ -25,6 +25,14 @@ int gbmv3(float Alpha, float Beta, struct halide_buffer_t *A, struct halide_buff
 double gbmv3_ns(float Alpha, float Beta, struct halide_buffer_t *A, struct halide_buffer_t *X,
                 struct halide_buffer_t *Y, struct halide_buffer_t *Out);
 
+/* The argv form and the argument table that Halide declares next to every generated entry
+ * (Halide/src/CodeGen_C.cpp:1828-1833; the generated header the reference ships,
+ * t2s/peppers/blas/level3/syrk/release/s10/syrk-interface.h:14-18): args[i] points at the i-th
+ * scalar argument or is the i-th halide_buffer_t* itself; the table lists name, kind, rank (of the
+ * FPGA flow's buffers) and element type of each argument in call order. */
+int gbmv3_argv(void **args);
+const struct halide_filter_metadata_t *gbmv3_metadata(void);
+
 #ifdef __cplusplus
 }
 #endif

@@ -24,6 +24,12 @@ int mttkrp(struct halide_buffer_t *B, struct halide_buffer_t *C, struct halide_b
  * halide_buffer_t* itself. */
 int mttkrp_argv(void **args);
 
+/* The argument table Halide declares next to every generated entry
+ * (Halide/src/CodeGen_C.cpp:1830-1833; struct halide_filter_metadata_t,
+ * Halide/src/runtime/HalideRuntime.h:1653-1675): name, kind, rank and element type of each
+ * argument in call order, the entry's name, and "hip-gfx950" as the target.   */
+const struct halide_filter_metadata_t *mttkrp_metadata(void);
+
 /* mttkrp() with a forced tile configuration (T2SP_CFG_* of t2sp_hip.h) and number of
  * reduction splits (0 = automatic); no counterpart in the reference. */
 int t2sp_mttkrp_with_cfg(struct halide_buffer_t *B, struct halide_buffer_t *C,

@@ -32,6 +32,14 @@ double pairhmm_ns(struct halide_buffer_t *H, struct halide_buffer_t *R, struct h
                   struct halide_buffer_t *alpha_gap, struct halide_buffer_t *beta_match,
                   struct halide_buffer_t *beta_gap, struct halide_buffer_t *Out);
 
+/* The argv form and the argument table that Halide declares next to every generated entry
+ * (Halide/src/CodeGen_C.cpp:1828-1833; the generated header the reference ships,
+ * t2s/peppers/blas/level3/syrk/release/s10/syrk-interface.h:14-18): args[i] points at the i-th
+ * scalar argument or is the i-th halide_buffer_t* itself; the table lists name, kind, rank (of the
+ * FPGA flow's buffers) and element type of each argument in call order. */
+int pairhmm_argv(void **args);
+const struct halide_filter_metadata_t *pairhmm_metadata(void);
+
 #ifdef __cplusplus
 }
 #endif

@@ -26,6 +26,14 @@ int qrd(struct halide_buffer_t *a, struct halide_buffer_t *Q, struct halide_buff
 /* qrd() that returns the kernel time in ns (negative error code on failure). */
 double qrd_ns(struct halide_buffer_t *a, struct halide_buffer_t *Q, struct halide_buffer_t *R);
 
+/* The argv form and the argument table that Halide declares next to every generated entry
+ * (Halide/src/CodeGen_C.cpp:1828-1833; the generated header the reference ships,
+ * t2s/peppers/blas/level3/syrk/release/s10/syrk-interface.h:14-18): args[i] points at the i-th
+ * scalar argument or is the i-th halide_buffer_t* itself; the table lists name, kind, rank (of the
+ * FPGA flow's buffers) and element type of each argument in call order. */
+int qrd_argv(void **args);
+const struct halide_filter_metadata_t *qrd_metadata(void);
+
 #ifdef __cplusplus
 }
 #endif

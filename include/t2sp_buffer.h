@@ -7,10 +7,14 @@
  *   halide_buffer_t     Halide/src/runtime/HalideRuntime.h:1392-1418
  *   buffer flags        Halide/src/runtime/HalideRuntime.h:1384-1385
  *   error codes         Halide/src/runtime/HalideRuntime.h:957-1143
- * A caller that already includes the reference's HalideRuntime.h (for example
- * through HalideBuffer.h) must define T2SP_USE_HALIDE_RUNTIME before this
- * header; the struct definitions below are then skipped and only the helper
- * functions are declared against Halide's own types.
+ *   filter metadata     Halide/src/runtime/HalideRuntime.h:1603-1675
+ * When the reference's own HalideRuntime.h is on the include path (a driver that
+ * uses Halide::Runtime::Buffer from HalideBuffer.h has it there), that header is
+ * included here instead and the definitions below are skipped, exactly as the
+ * generated <op>-interface.h brings in the Halide types before it declares the
+ * entry (Halide/src/CodeGen_C.cpp:327, t2s/src/AOT-OpenCL-Runtime.h:20-31).  This
+ * happens by itself where the compiler has __has_include; defining
+ * T2SP_USE_HALIDE_RUNTIME forces it, T2SP_NO_HALIDE_RUNTIME forbids it.
  *
  * Layout facts checked by the static asserts at the bottom:
  *   sizeof(halide_type_t) == 4, sizeof(halide_dimension_t) == 16,
@@ -24,7 +28,15 @@
 #include <stddef.h>
 #include <stdint.h>
 
-#ifndef T2SP_USE_HALIDE_RUNTIME
+#if !defined(T2SP_USE_HALIDE_RUNTIME) && !defined(T2SP_NO_HALIDE_RUNTIME) && defined(__has_include)
+#if __has_include("HalideRuntime.h")
+#define T2SP_USE_HALIDE_RUNTIME 1
+#endif
+#endif
+
+#ifdef T2SP_USE_HALIDE_RUNTIME
+#include "HalideRuntime.h"
+#else
 
 #ifdef __cplusplus
 extern "C" {
@@ -94,6 +106,32 @@ enum halide_error_code_t {
     halide_error_code_bad_dimensions = -43
 };
 
+/* What <fn>_metadata() returns: one record per argument of the entry. */
+enum halide_argument_kind_t {
+    halide_argument_kind_input_scalar = 0,
+    halide_argument_kind_input_buffer = 1,
+    halide_argument_kind_output_buffer = 2
+};
+
+struct halide_scalar_value_t;
+
+struct halide_filter_argument_t {
+    const char *name;
+    int32_t kind;       /* halide_argument_kind_t */
+    int32_t dimensions; /* 0 for scalars */
+    struct halide_type_t type;
+    const struct halide_scalar_value_t *scalar_def, *scalar_min, *scalar_max, *scalar_estimate; /* NULL for buffers */
+    int64_t const *const *buffer_estimates;                                                   /* may be NULL */
+};
+
+struct halide_filter_metadata_t {
+    int32_t version; /* 1 */
+    int32_t num_arguments;
+    const struct halide_filter_argument_t *arguments;
+    const char *target; /* what the entry was built for */
+    const char *name;   /* the entry's name */
+};
+
 #ifdef __cplusplus
 } /* extern "C" */
 #endif
@@ -109,6 +147,9 @@ static_assert(offsetof(halide_buffer_t, flags) == 24, "flags at 24");
 static_assert(offsetof(halide_buffer_t, type) == 32, "type at 32");
 static_assert(offsetof(halide_buffer_t, dimensions) == 36, "dimensions at 36");
 static_assert(offsetof(halide_buffer_t, dim) == 40, "dim at 40");
+static_assert(sizeof(struct halide_filter_argument_t) == 64, "halide_filter_argument_t must be 64 bytes");
+static_assert(offsetof(struct halide_filter_argument_t, type) == 16, "argument type at 16");
+static_assert(sizeof(struct halide_filter_metadata_t) == 32, "halide_filter_metadata_t must be 32 bytes");
 #endif
 
 #ifdef __cplusplus

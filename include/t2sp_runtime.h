@@ -2,8 +2,20 @@
  * entry points.  They stand in for pieces of t2s/src/AOT-OpenCL-Runtime.cpp. */
 #ifndef T2SP_RUNTIME_H
 #define T2SP_RUNTIME_H
+/* The C headers (and <iostream> in C++) that the reference's generated <op>-interface.h brings in
+ * through AOT-OpenCL-Runtime.h (t2s/src/AOT-OpenCL-Runtime.h:22-31, included by the generated
+ * header: Halide/src/CodeGen_C.cpp:327).  The reference's drivers rely on them: conv-run-fpga.cpp
+ * and capsule-run-fpga.cpp call fabs() and include no <math.h> of their own. */
+#include <assert.h>
+#include <float.h>
+#include <limits.h>
+#include <math.h>
 #include <stddef.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
 #ifdef __cplusplus
+#include <iostream>
 extern "C" {
 #endif
 

@@ -29,3 +29,33 @@ extern "C" int gemm_argv(void **args) {
                         static_cast<halide_buffer_t *>(args[5]), static_cast<halide_buffer_t *>(args[6]),
                         static_cast<halide_buffer_t *>(args[7]));
 }
+
+// The argument table of the 8-argument entry (Halide/src/CodeGen_C.cpp:1830-1833).  The release
+// ships no specification for it; the scalar names are those of the SYRK pipeline of the same family
+// (Param<int> OpA, Param<float> Alpha, Beta: t2s/tests/performance/syrk/syrk.cpp:56-57).
+extern "C" const halide_filter_metadata_t *gemm_metadata(void) {
+    static halide_filter_argument_t args[8];
+    static halide_filter_metadata_t meta;
+    static const bool once = [] {
+        const char *names[8] = {"OpA", "OpB", "Alpha", "Beta", "A", "B", "C", "deserializer"};
+        for (int i = 0; i < 8; i++) {
+            args[i].name = names[i];
+            args[i].kind = i < 4 ? halide_argument_kind_input_scalar
+                                 : i < 7 ? halide_argument_kind_input_buffer : halide_argument_kind_output_buffer;
+            args[i].dimensions = i < 4 ? 0 : i < 7 ? 2 : 6;
+            args[i].type.code = i < 2 ? halide_type_int : halide_type_float;
+            args[i].type.bits = 32;
+            args[i].type.lanes = 1;
+            args[i].scalar_def = args[i].scalar_min = args[i].scalar_max = args[i].scalar_estimate = nullptr;
+            args[i].buffer_estimates = nullptr;
+        }
+        meta.version = 1;
+        meta.num_arguments = 8;
+        meta.arguments = args;
+        meta.target = "hip-gfx950";
+        meta.name = "gemm";
+        return true;
+    }();
+    (void)once;
+    return &meta;
+}

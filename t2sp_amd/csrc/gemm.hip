@@ -284,16 +284,6 @@ template <> struct VecOf<4> { typedef float type __attribute__((ext_vector_type(
 
 // Timeline stamps of this kernel (100 MHz wall clock, one set per wave), compiled in only by
 // `make trace-lib`; python -m t2sp_amd.d16_timeline reads them back.
-#ifdef T2SP_D16_TRACE
-__device__ long long g_d16_trace[4096 * 8 * 8];
-#define T2SP_TRACE_STAMP(i)                                                                          \
-    {                                                                                                \
-        const unsigned wg = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);          \
-        if ((threadIdx.x & 63) == 0 && wg < 4096) g_d16_trace[(wg * 8 + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64(); \
-    }
-#else
-#define T2SP_TRACE_STAMP(i)
-#endif
 // What the loop of the 16 x 16 form needs of the arguments.  The kernel takes these as leading
 // scalar parameters, which the dispatcher preloads into scalar registers before the first wave
 // starts (the build sets -amdgpu-kernarg-preload-count): a wave that has to fetch them from the
@@ -310,7 +300,6 @@ __device__ __forceinline__ void sgemm_d16_wave(const GemmHot &g, int mb0, int m0
     typedef typename VecOf<NB>::type vnb;
     constexpr int R = GEMM_D16_RING;
     const int lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
-    T2SP_TRACE_STAMP(0)
     uint32_t a_off[MBW];
 #pragma unroll
     for (int mb = 0; mb < MBW; mb++) {
@@ -371,7 +360,6 @@ __device__ __forceinline__ void sgemm_d16_wave(const GemmHot &g, int mb0, int m0
     }
     const int main_iters = nsteps > 0 ? (nsteps - 1) / R : 0;
     const int rem = nsteps - main_iters * R;
-    T2SP_TRACE_STAMP(1)
     for (int it = 0; it < main_iters; it++) {
 #pragma unroll
         for (int d = 0; d < R; d++) {
@@ -379,12 +367,8 @@ __device__ __forceinline__ void sgemm_d16_wave(const GemmHot &g, int mb0, int m0
             T2SP_GEMM_D16_MMA(d)
             T2SP_INTERLEAVE(SG_VMEM_READ, MBW + 4, (4 * MBW * NB) / (MBW + 4))
             __builtin_amdgcn_sched_barrier(0);
-#ifdef T2SP_D16_TRACE
-            if (it == 0 && d == 0) { T2SP_TRACE_STAMP(2) }
-#endif
         }
     }
-    T2SP_TRACE_STAMP(3)
     T2SP_GEMM_D16_ISSUE(R - 1)
 #pragma unroll
     for (int d = 0; d < R; d++) {
@@ -392,7 +376,6 @@ __device__ __forceinline__ void sgemm_d16_wave(const GemmHot &g, int mb0, int m0
     }
 #undef T2SP_GEMM_D16_ISSUE
 #undef T2SP_GEMM_D16_MMA
-    T2SP_TRACE_STAMP(4)
     v4f *mine = red_kq + mb0 * NB * 64 + lane;
 #pragma unroll
     for (int mb = 0; mb < MBW; mb++)
@@ -442,7 +425,6 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
         }
     }
     __syncthreads();
-    T2SP_TRACE_STAMP(5)
     // sum the partial tiles of the waves in wave order
 #pragma unroll
     for (int i = 0; i < PER_WAVE; i++) {
@@ -481,7 +463,6 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
             }
         }
     }
-    T2SP_TRACE_STAMP(6)
 }
 // The same form for B stored transposed (N x K, k contiguous: C = A * B^T, the layout of a weight
 // matrix): both operands are read as A is above, 4 consecutive k of one row (of A) or column (of
@@ -737,13 +718,6 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     }
 }
 
-#ifdef T2SP_D16_TRACE
-}  // namespace t2sp
-extern "C" int t2sp_d16_trace(long long *host, int n) {
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(t2sp::g_d16_trace), (size_t)n * 8);
-}
-namespace t2sp {
-#endif
 
 // Fallback for shapes the vector loaders cannot take (K or N not a multiple
 // of 4, or operands not 16-byte aligned): one thread per output, sequential k.

@@ -22,7 +22,7 @@ def declared_symbols():
     for h in glob.glob(os.path.join(ROOT, "include", "*.h")):
         text = re.sub(r"/\*.*?\*/", "", open(h).read(), flags=re.S)
         text = re.sub(r"//[^\n]*", "", text)
-        for m in re.finditer(r"^(?:int|double|void|size_t)\s+(\w+)\s*\(", text, flags=re.M):
+        for m in re.finditer(r"^(?:int|double|void|size_t|const struct halide_filter_metadata_t \*)\s*(\w+)\s*\(", text, flags=re.M):
             names.add(m.group(1))
     return names
 
@@ -310,3 +310,70 @@ def test_blas_library_exports_the_eight_argument_gemm():
     assert B.gemm(0, 0, 1.0, 0.0, a.ref, _buf((5, 12)).ref, c.ref, c.ref) == -8
     assert B.gemm(0, 0, 1.0, 0.0, a.ref, b.ref, c.ref, _buf((4, 12)).ref) == -4
     assert hasattr(B, "gemm_argv")
+
+
+class _FilterArgument(ctypes.Structure):
+    _fields_ = [("name", ctypes.c_char_p), ("kind", ctypes.c_int32), ("dimensions", ctypes.c_int32),
+                ("code", ctypes.c_uint8), ("bits", ctypes.c_uint8), ("lanes", ctypes.c_uint16),
+                ("scalar_def", ctypes.c_void_p), ("scalar_min", ctypes.c_void_p), ("scalar_max", ctypes.c_void_p),
+                ("scalar_estimate", ctypes.c_void_p), ("buffer_estimates", ctypes.c_void_p)]
+
+
+class _FilterMetadata(ctypes.Structure):
+    _fields_ = [("version", ctypes.c_int32), ("num_arguments", ctypes.c_int32),
+                ("arguments", ctypes.POINTER(_FilterArgument)), ("target", ctypes.c_char_p), ("name", ctypes.c_char_p)]
+
+
+def _metadata(L, fn):
+    f = getattr(L, fn + "_metadata")
+    f.restype = ctypes.POINTER(_FilterMetadata)
+    f.argtypes = []
+    m = f().contents
+    assert m.version == 1 and m.name == fn.encode() and m.target
+    return [(a.name.decode(), a.kind, a.dimensions, a.code, a.bits, a.lanes)
+            for a in (m.arguments[i] for i in range(m.num_arguments))]
+
+
+def test_metadata_tables_describe_the_entries():
+    """<fn>_metadata() (Halide/src/CodeGen_C.cpp:1830-1833, struct at HalideRuntime.h:1634-1675): the layout
+    ctypes reads is Halide's (64-byte argument records), kinds 0/1/2 = scalar/input/output, type code 2 = float."""
+    assert ctypes.sizeof(_FilterArgument) == 64 and ctypes.sizeof(_FilterMetadata) == 32
+    L = t2sp_amd.lib()
+    F = (2, 32, 1)
+    assert _metadata(L, "gemm") == [("A", 1, 2, *F), ("B", 1, 2, *F), ("deserializer", 2, 6, *F)]
+    assert [a[1:] for a in _metadata(L, "GEMM")] == [(1, 2, *F), (1, 2, *F), (2, 6, *F)]
+    assert _metadata(L, "conv") == [("I", 1, 2, *F), ("K", 1, 2, *F), ("deserializer", 2, 10, *F)]
+    assert _metadata(L, "capsule") == [("P", 1, 2, *F), ("W", 1, 2, *F), ("deserializer", 2, 10, *F)]
+    assert _metadata(L, "mttkrp") == [("B", 1, 3, *F), ("C", 1, 2, *F), ("D", 1, 2, *F), ("A", 2, 2, *F)]
+    # the generated header the reference ships: syrk(int32_t _OpA, float _Alpha, float _Beta, A, C, deserializer)
+    # (t2s/peppers/blas/level3/syrk/release/s10/syrk-interface.h:12)
+    assert _metadata(L, "syrk") == [("OpA", 0, 0, 0, 32, 1), ("Alpha", 0, 0, *F), ("Beta", 0, 0, *F), ("A", 1, 2, *F),
+                                    ("C", 1, 2, *F), ("deserializer", 2, 6, *F)]
+    ph = _metadata(L, "pairhmm")
+    assert len(ph) == 10 and ph[0][3:] == (1, 8, 1) and ph[1][3:] == (1, 8, 1) and ph[9][1:3] == (2, 4)
+    assert [a[1] for a in _metadata(L, "qrd")] == [1, 2, 2]
+    for fn in ("ger", "gbmv3", "symv"):
+        m = _metadata(L, fn)
+        assert m[-1][0] == "deserializer" and m[-1][1] == 2 and all(a[1] != 2 for a in m[:-1])
+    # every table has an argv form that takes as many pointers
+    for fn in ("gemm", "GEMM", "conv", "capsule", "mttkrp", "syrk", "ger", "gbmv3", "symv", "pairhmm", "qrd"):
+        assert hasattr(L, fn + "_argv")
+    # the 8-argument pipeline entry of the BLAS release lives in a library of its own
+    B = ctypes.CDLL(os.path.join(ROOT, "t2sp_amd", "libt2sp_blas_gemm.so"))
+    m8 = _metadata(B, "gemm")
+    assert [a[1] for a in m8] == [0, 0, 0, 0, 1, 1, 1, 2] and m8[0][3:] == (0, 32, 1) and m8[2][3:] == F
+
+
+def test_argv_forms_of_scalar_entries_reject_null_buffers():
+    """syrk_argv / gbmv3_argv unpack pointers to scalars and buffers themselves; a NULL buffer comes back as -12
+    from the entry's own checks, before any device work."""
+    L = t2sp_amd.lib()
+    opa, alpha, beta = ctypes.c_int32(0), ctypes.c_float(1.0), ctypes.c_float(0.0)
+    args = (ctypes.c_void_p * 6)(ctypes.addressof(opa), ctypes.addressof(alpha), ctypes.addressof(beta), None, None, None)
+    L.syrk_argv.argtypes = [ctypes.c_void_p]
+    assert L.syrk_argv(args) == -12
+    args = (ctypes.c_void_p * 6)(ctypes.addressof(alpha), ctypes.addressof(beta), None, None, None, None)
+    L.gbmv3_argv.argtypes = [ctypes.c_void_p]
+    assert L.gbmv3_argv(args) == -12
+    L.qrd_argv.argtypes = [ctypes.c_void_p]
+    assert L.qrd_argv(None) == -12
