@@ -57,7 +57,9 @@ const struct halide_filter_metadata_t *capsule_metadata(void);
 
 /* States the design constant CII (capsule/const-parameters.h:31-70: 4 for the GPU and TINY sets, 32
  * for S10, 16 for A10) that the packed form of capsule() needs; 0 clears it.  Returns the previous
- * value.  Process-wide; no counterpart in the reference, where CII is compiled into the pipeline. */
+ * value.  The value belongs to the calling thread (threads that run different designs do not disturb
+ * each other); a thread that has stated none uses the one stated last by any thread, then the
+ * environment.  No counterpart in the reference, where CII is compiled into the pipeline. */
 int t2sp_capsule_design(int cii);
 
 /* capsule() with a forced tile configuration (T2SP_CFG_* of t2sp_hip.h) and number of

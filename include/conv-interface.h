@@ -43,8 +43,10 @@ int conv_argv(void **args);
 const struct halide_filter_metadata_t *conv_metadata(void);
 
 /* States TOTAL_OY for packed inputs with the 2-D output when the map is not square (0 clears it;
- * also read from the environment variable T2SP_CONV_TOTAL_OY).  Returns the previous value.  No
- * counterpart in the reference, where the map size is compiled into the pipeline. */
+ * also read from the environment variable T2SP_CONV_TOTAL_OY).  Returns the previous value.  The
+ * value belongs to the calling thread; a thread that has stated none uses the one stated last by
+ * any thread, then the environment.  No counterpart in the reference, where the map size is
+ * compiled into the pipeline. */
 int t2sp_conv_design(int total_oy);
 
 /* conv() with a forced tile configuration (T2SP_CFG_* of t2sp_hip.h); no counterpart in

@@ -38,7 +38,8 @@ extern "C" {
 #define T2SP_MAX_DIMS 10
 
 /* C[i,j] = sum_k A[i,k] * B[k,j], fp32, row-major with leading dimensions in
- * elements.  Replaces the device side of the reference's SGEMM pipeline: the
+ * elements, which must not be negative here and in the BLAS, SYRK and MTTKRP forms below
+ * (T2SP_ERR_SHAPE; MTTKRP takes its slow kernel for strides that step backwards).  Replaces the device side of the reference's SGEMM pipeline: the
  * kernels of t2s/tests/performance/gemm/bitstream/a10/a.cl:67-770 launched by
  * halide_opencl_wait_for_kernels_finish (t2s/src/AOT-OpenCL-Runtime.cpp:312-397).
  * `workspace` is optional (NULL allowed): products with fewer output tiles than CUs use it
@@ -66,7 +67,9 @@ int t2sp_sgemm_f32_tiled(const float *A, const float *B, float *C, int M, int N,
  * k-contiguous tiles, A^T (with M, N and the leading dimensions multiples of 4 and 16-byte
  * aligned pointers) through row-contiguous ones, for any K; small and middle-sized products of
  * each form have a one-launch kernel of their own (T2SP_CFG_DIRECT16 forces it).  Otherwise a transposed A is first
- * re-laid into `workspace`, which is required then; the rest of t2sp_sgemm_ex_workspace_bytes is
+ * re-laid into `workspace` when there is room for it (M * K floats) and read as it lies by a
+ * one-thread-per-output kernel when there is not (slow, like every shape the 128-bit loaders cannot
+ * take without a workspace); the rest of t2sp_sgemm_ex_workspace_bytes is
  * optional room for the planes of a split reduction, as in t2sp_sgemm_f32.  Device side of the reference's 8-argument
  * gemm(opa, opb, alpha, beta, A, B, C, O) pipeline behind its BLAS wrapper
  * (t2s/peppers/blas/level3/gemm/release/a10/blas-gemm.cpp:28-47). */
@@ -219,8 +222,10 @@ int t2sp_mttkrp_f32(const float *B, const float *C, const float *D, float *A, in
  * ends.  The benchmark size (I = J = K = 512, R = 256: 128 planes of 0.5 MB) fits exactly; a
  * product that needs more returns T2SP_ERR_SHAPE with a message.  The call itself allocates and
  * frees nothing.  All calls on one GPU share the array: calls that overlap on one GPU (different
- * streams or threads) race; calls on one stream are ordered and safe.  Same results, bit for
- * bit, as t2sp_mttkrp_f32 with a workspace. */
+ * streams or threads) race; calls on one stream are ordered and safe.  The first call on a device
+ * looks the array's address up (hipGetSymbolAddress, which may load the code object) and must
+ * therefore be made outside stream capture; later calls on that device only enqueue kernels.  Same
+ * results, bit for bit, as t2sp_mttkrp_f32 with a workspace. */
 #define T2SP_MTTKRP_NOALLOC_SCRATCH_BYTES (64u << 20)
 int t2sp_mttkrp_f32_noalloc(const float *B, const float *C, const float *D, float *A, int I, int J,
                             int K, int R, const int64_t *sb3, const int64_t *sc2, const int64_t *sd2,

@@ -12,7 +12,8 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+# $T2SP_ORACLE_LIBRARY names another build of the same file (the sanitizer build of `make -C oracle asan`)
+_LIB_PATH = os.environ.get("T2SP_ORACLE_LIBRARY") or os.path.join(_HERE, "liboracle.so")
 
 ACC_F32, ACC_F32_FMA, ACC_F64 = 0, 1, 2
 ORDER_GOLDEN, ORDER_URE = 0, 1

@@ -4,7 +4,8 @@ import os
 import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB = os.path.join(_HERE, "libt2sp_mi355x.so")
+# $T2SP_LIBRARY names another build of the same library (the sanitizer build of `make -C t2sp_amd/csrc asan`)
+_LIB = os.environ.get("T2SP_LIBRARY") or os.path.join(_HERE, "libt2sp_mi355x.so")
 _lib = None
 
 

@@ -721,14 +721,22 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
 
 // Fallback for shapes the vector loaders cannot take (K or N not a multiple
 // of 4, or operands not 16-byte aligned): one thread per output, sequential k.
-__global__ void sgemm_scalar_kernel(const GemmArgs g, int bt) {
+// at: A is stored K x M (element (r, k) at k * lda + r); bt: B is stored N x K.
+__global__ void sgemm_scalar_kernel(const GemmArgs g, int bt, int at) {
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
-    const int r = blockIdx.y;
     if (c >= g.N) return;
-    float acc = 0.f;
-    for (int k = 0; k < g.K; k++)
-        acc = fmaf(g.A[(int64_t)r * g.lda + k], bt ? g.B[(int64_t)c * g.ldb + k] : g.B[(int64_t)k * g.ldb + c], acc);
-    gemm_store1(g, r, c, acc);
+    for (int r = blockIdx.y; r < g.M; r += gridDim.y) {
+        float acc = 0.f;
+        for (int k = 0; k < g.K; k++)
+            acc = fmaf(at ? g.A[(int64_t)k * g.lda + r] : g.A[(int64_t)r * g.lda + k],
+                       bt ? g.B[(int64_t)c * g.ldb + k] : g.B[(int64_t)k * g.ldb + c], acc);
+        gemm_store1(g, r, c, acc);
+    }
+}
+
+static int launch_scalar(const GemmArgs &g, bool bt, bool at, hipStream_t stream) {
+    hipLaunchKernelGGL(sgemm_scalar_kernel, dim3((g.N + 255) / 256, g.M < 65535 ? g.M : 65535), dim3(256), 0, stream, g, bt ? 1 : 0, at ? 1 : 0);
+    return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
 }
 
 // Zero-padded copy of a row-major rows x cols matrix into rows_p x cols_p (leading dimension cols_p).
@@ -1172,7 +1180,9 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         // spread over the CUs than they have)
         const bool lds_split = workspace && workspace_bytes >= plan_gemm(g.M, g.N, g.K).scratch_bytes;
         const bool too_few = (int64_t)p.tiles_m * p.tiles_n < cus / 2 && g.K >= 4096 && !can_split && lds_split;
-        if (!big_tiles && !tiled_better && !too_few && g.K >= 64)
+        // (the plain form's grid is tiles_m x tiles_n: a thin, very wide product goes on to the other kernels)
+        const bool grid_ok = bt || p.tiles_n <= 65535;
+        if (!big_tiles && !tiled_better && !too_few && grid_ok && g.K >= 64)
             return bt ? launch_d16_bt(g, stream) : launch_d16(g, stream, workspace, workspace_bytes);
     }
     if ((cfg == T2SP_CFG_AUTO || cfg == T2SP_CFG_DIRECT) && !bt && !g.scale && !g.tiled &&
@@ -1214,8 +1224,7 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
     }
     if (cfg == T2SP_CFG_SCALAR || !vec_ok) {
-        hipLaunchKernelGGL(sgemm_scalar_kernel, dim3((g.N + 255) / 256, g.M), dim3(256), 0, stream, g, bt ? 1 : 0);
-        return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+        return launch_scalar(g, bt, false, stream);
     }
     int splits = 1;
     bool phased = false;
@@ -1290,6 +1299,7 @@ extern "C" size_t t2sp_sgemm_workspace_bytes(int M, int N, int K) {
 extern "C" int t2sp_sgemm_f32(const float *A, const float *B, float *C, int M, int N, int K,
                               int64_t lda, int64_t ldb, int64_t ldc, int cfg, float *workspace,
                               size_t workspace_bytes, void *stream) {
+    if (lda < 0 || ldb < 0 || ldc < 0) return T2SP_ERR_SHAPE;   // the loaders' offsets are unsigned
     t2sp::GemmArgs g{};
     g.A = A; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K;
     g.lda = lda; g.ldb = ldb; g.ldc = ldc;
@@ -1301,7 +1311,7 @@ extern "C" int t2sp_sgemm_f32_tiled(const float *A, const float *B, float *C, in
                                     int64_t lda, int64_t ldb, int jjj, int iii, int jj, int ii,
                                     const int64_t *strides6, int cfg, float *workspace,
                                     size_t workspace_bytes, void *stream) {
-    if (jjj <= 0 || iii <= 0 || jj <= 0 || ii <= 0 || !strides6) return T2SP_ERR_SHAPE;
+    if (jjj <= 0 || iii <= 0 || jj <= 0 || ii <= 0 || !strides6 || lda < 0 || ldb < 0) return T2SP_ERR_SHAPE;
     t2sp::GemmArgs g{};
     g.A = A; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K;
     g.lda = lda; g.ldb = ldb; g.ldc = 0;
@@ -1326,7 +1336,7 @@ extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, fl
                                  int64_t lda, const float *B, int64_t ldb, float beta, const float *Cin,
                                  int64_t ldcin, float *C, int64_t ldc, int cfg, float *workspace,
                                  size_t workspace_bytes, void *stream) {
-    if (M <= 0 || N <= 0 || K <= 0) return T2SP_ERR_SHAPE;
+    if (M <= 0 || N <= 0 || K <= 0 || lda < 0 || ldb < 0 || ldc < 0 || (Cin && ldcin < 0)) return T2SP_ERR_SHAPE;
     const float *a = A;
     int64_t la = lda;
     auto aligned16 = [](const void *p) { return ((uintptr_t)p & 15) == 0; };
@@ -1349,7 +1359,16 @@ extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, fl
     (void)t256; (void)room;
     if (transa && !native_at) {
         // A is stored K x M: bring it to M x K first (the loaders of the other kernels want k contiguous in A)
-        if (!workspace || workspace_bytes < (size_t)M * K * sizeof(float)) return T2SP_ERR_SHAPE;
+        if (!workspace || workspace_bytes < (size_t)M * K * sizeof(float)) {
+            // no room to re-lay A and a shape the 128-bit loaders cannot take as it lies (M, N or a
+            // leading dimension not a multiple of 4, unaligned operands): one thread per output
+            if (cfg != T2SP_CFG_AUTO && cfg != T2SP_CFG_SCALAR) return T2SP_ERR_SHAPE;
+            t2sp::GemmArgs s{};
+            s.A = A; s.B = B; s.C = C; s.M = M; s.N = N; s.K = K;
+            s.lda = lda; s.ldb = ldb; s.ldc = ldc;
+            s.scale = 1; s.alpha = alpha; s.beta = Cin ? beta : 0.f; s.Cin = Cin ? Cin : C; s.ldcin = Cin ? ldcin : ldc;
+            return t2sp::launch_scalar(s, transb != 0, true, (hipStream_t)stream);
+        }
         const int ext[2] = {K, M};
         const int64_t ss[2] = {lda, 1}, ds[2] = {1, K};
         const int rc = t2sp_relayout_f32(A, workspace, 2, ext, ss, ds, stream);

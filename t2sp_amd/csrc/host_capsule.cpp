@@ -33,12 +33,22 @@
 
 using namespace t2sp;
 
+// The design constant is kept per calling thread, so that two threads that run different designs
+// do not race between their set and their call; a thread that has never stated one uses the value
+// stated last by any thread, then the environment.
 static std::atomic<int> g_capsule_cii{0};
+static thread_local int tl_capsule_cii = 0;
 
-extern "C" int t2sp_capsule_design(int cii) { return g_capsule_cii.exchange(cii < 0 ? 0 : cii); }
+extern "C" int t2sp_capsule_design(int cii) {
+    const int v = cii < 0 ? 0 : cii;
+    const int prev_global = g_capsule_cii.exchange(v);
+    const int prev = tl_capsule_cii > 0 ? tl_capsule_cii : prev_global;
+    tl_capsule_cii = v;
+    return prev;
+}
 
 static int capsule_cii() {
-    int cii = g_capsule_cii.load();
+    int cii = tl_capsule_cii > 0 ? tl_capsule_cii : g_capsule_cii.load();
     if (cii <= 0)
         if (const char *e = getenv("T2SP_CAPSULE_CII")) cii = atoi(e);
     return cii;

@@ -28,9 +28,18 @@
 
 using namespace t2sp;
 
+// Kept per calling thread (two threads with different designs do not race between set and call);
+// a thread that has never stated one uses the value stated last by any thread, then the environment.
 static std::atomic<int> g_conv_total_oy{0};
+static thread_local int tl_conv_total_oy = 0;
 
-extern "C" int t2sp_conv_design(int total_oy) { return g_conv_total_oy.exchange(total_oy < 0 ? 0 : total_oy); }
+extern "C" int t2sp_conv_design(int total_oy) {
+    const int v = total_oy < 0 ? 0 : total_oy;
+    const int prev_global = g_conv_total_oy.exchange(v);
+    const int prev = tl_conv_total_oy > 0 ? tl_conv_total_oy : prev_global;
+    tl_conv_total_oy = v;
+    return prev;
+}
 
 namespace {
 struct Logical4 {
@@ -161,7 +170,7 @@ static int conv_impl(halide_buffer_t *I, halide_buffer_t *K, halide_buffer_t *O,
         if (s2 < 0 || s2 % (KYX - 1) || root < 0 || root * root != disc || (sum + root) % 2)
             return report(halide_error_code_constraint_violated, op, "no map OY x OX has O.extent.1 outputs and I.extent.1 inputs under a 3 x 3 kernel");
         const int64_t big = (sum + root) / 2, small = (sum - root) / 2;
-        int hint = g_conv_total_oy.load();
+        int hint = tl_conv_total_oy > 0 ? tl_conv_total_oy : g_conv_total_oy.load();
         if (hint <= 0)
             if (const char *e = getenv("T2SP_CONV_TOTAL_OY")) hint = atoi(e);
         if (big == small) {

@@ -324,9 +324,10 @@ static int launch_mttkrp(MttkrpArgs g, hipStream_t stream) {
 
 static bool mttkrp_fast(int I, int J, const int64_t *sb3, const int64_t *sc2, const int64_t *sd2,
                         const int64_t *sa2, const float *B, const float *C, const float *A) {
-    (void)sd2;
     // (the loaders reach a tile's rows with 32-bit offsets: see LOADER_MAX_LD, and j within a row of C likewise)
+    // (and with unsigned ones: strides that step backwards take the kernel without requirements)
     return J % 16 == 0 && I % 4 == 0 && sb3[1] == 1 && sc2[0] == 1 && sa2[0] == 1 && sb3[0] % 4 == 0 &&
+           sb3[0] >= 0 && sb3[2] >= 0 && sc2[1] >= 0 && sd2[0] >= 0 && sd2[1] >= 0 && sa2[1] >= 0 &&
            sb3[0] < LOADER_MAX_LD && sc2[1] < LOADER_MAX_LD && J < LOADER_MAX_LD &&
            sb3[2] % 4 == 0 && sc2[1] % 4 == 0 && sa2[1] % 4 == 0 && ((uintptr_t)B % 16 == 0) &&
            ((uintptr_t)C % 16 == 0) && ((uintptr_t)A % 16 == 0);

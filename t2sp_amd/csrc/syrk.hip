@@ -672,6 +672,7 @@ extern "C" size_t t2sp_ssyrk_folded_workspace_bytes(int trans, int N, int K) {
 extern "C" int t2sp_ssyrk_f32(int upper, int trans, int N, int K, float alpha, const float *A, int64_t lda,
                               float beta, const float *Cin, int64_t ldcin, float *C, int64_t ldc, int mirror,
                               int cfg, float *workspace, size_t workspace_bytes, void *stream) {
+    if (lda < 0 || ldc < 0 || (Cin && ldcin < 0)) return T2SP_ERR_SHAPE;   // the loaders' offsets are unsigned
     t2sp::SyrkArgs g{};
     g.A = A; g.lda = lda; g.N = N; g.K = K; g.alpha = alpha; g.beta = beta;
     g.Cin = beta != 0.f ? Cin : nullptr; g.ldcin = ldcin;
@@ -684,7 +685,7 @@ extern "C" int t2sp_ssyrk_f32_folded(int trans, int N, int K, float alpha, const
                                      const float *Cin, int64_t ldcin, float *Out, int iii, int ii,
                                      const int64_t *strides6, int cfg, float *workspace, size_t workspace_bytes,
                                      void *stream) {
-    if (iii <= 0 || ii <= 0 || !strides6 || N <= 0) return T2SP_ERR_SHAPE;
+    if (iii <= 0 || ii <= 0 || !strides6 || N <= 0 || lda < 0 || (Cin && ldcin < 0)) return T2SP_ERR_SHAPE;
     const int B = iii * ii;
     if (N % B || (N / B) % 2) return T2SP_ERR_SHAPE;   // an even number of whole blocks (syrk.cpp:80-82: i < I/2)
     t2sp::SyrkArgs g{};

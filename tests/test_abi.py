@@ -377,3 +377,32 @@ def test_argv_forms_of_scalar_entries_reject_null_buffers():
     assert L.gbmv3_argv(args) == -12
     L.qrd_argv.argtypes = [ctypes.c_void_p]
     assert L.qrd_argv(None) == -12
+
+
+def test_design_constants_belong_to_the_calling_thread():
+    """t2sp_capsule_design / t2sp_conv_design: a thread's own value wins over another thread's; a thread that has
+    stated none sees the one stated last by any thread."""
+    import threading
+    L = t2sp_amd.lib()
+    seen = {}
+    try:
+        assert L.t2sp_capsule_design(16) in (0, 4, 5, 16)
+        ready, go = threading.Event(), threading.Event()
+
+        def other():
+            seen["inherited"] = L.t2sp_capsule_design(32)      # returns what this thread would have used: main's 16
+            ready.set()
+            go.wait(10)
+            seen["own"] = L.t2sp_capsule_design(32)            # still its own 32 after main has set 4
+
+        t = threading.Thread(target=other)
+        t.start()
+        assert ready.wait(10)
+        assert L.t2sp_capsule_design(4) == 16                  # main's own 16, not the other thread's 32
+        go.set()
+        t.join(10)
+        assert seen == {"inherited": 16, "own": 32}
+        assert L.t2sp_conv_design(60) == 0 and L.t2sp_conv_design(0) == 60
+    finally:
+        L.t2sp_capsule_design(0)
+        L.t2sp_conv_design(0)

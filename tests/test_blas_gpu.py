@@ -107,13 +107,47 @@ def test_transposed_a_as_it_lies_without_workspace(shape):
         assert rc == 0
         torch.cuda.synchronize()
         assert torch.equal(C.double(), ref)
-    # rows of A that are not 16-byte aligned cannot be read that way: the workspace is required then
-    if M % 4 == 0:
+    # rows of A that are not 16-byte aligned cannot be read 128 bits at a time: without a workspace the
+    # one-thread-per-output kernel reads the transposed A as it lies
+    if M % 4 == 0 and M * N * K <= 2 ** 28:
         Atp = torch.zeros(K, M + 2, device="cuda")
-        C = torch.empty(M, N, device="cuda")
-        rc = L.t2sp_sgemm_ex_f32(1, 0, M, N, K, 1.0, Atp.data_ptr(), M + 2, B.data_ptr(), N, 0.0, None, 0, C.data_ptr(), N, 0,
-                                 None, 0, None)
-        assert rc != 0
+        Atp[:, :M] = At
+        C = torch.full((M, N), float("nan"), device="cuda")
+        rc = L.t2sp_sgemm_ex_f32(1, 0, M, N, K, 2.0, Atp.data_ptr(), M + 2, B.data_ptr(), N, -3.0, C0.data_ptr(), N,
+                                 C.data_ptr(), N, 0, None, 0, None)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert torch.equal(C.double(), ref)
+
+
+@pytest.mark.parametrize("transb", [0, 1])
+@pytest.mark.parametrize("shape", [(2265, 588, 512), (1562, 512, 3968), (37, 19, 23)])
+def test_transposed_a_no_workspace_sizes_not_multiples_of_four(shape, transb):
+    """A stored K x M with M or N not a multiple of 4 and no workspace to re-lay it into: computed by the
+    one-thread-per-output kernel (as the untransposed forms are for such shapes), not refused.  Integer data:
+    exact.  With the workspace the same call re-lays A and takes the fast kernels: same values."""
+    import torch
+    M, N, K = shape
+    L = t2sp_amd.lib()
+    g = torch.Generator(device="cpu").manual_seed(M * 3 + N * 5 + K)
+    At = torch.randint(-2, 3, (K, M), generator=g).float().cuda()
+    B = torch.randint(-2, 3, (K, N), generator=g).float().cuda()
+    C0 = torch.randint(-4, 5, (M, N), generator=g).float().cuda()
+    ref = 2.0 * (At.double().t() @ B.double()) - 3.0 * C0.double()
+    Bd, ldb = (B.t().contiguous(), K) if transb else (B, N)
+    nbytes = L.t2sp_sgemm_ex_workspace_bytes(1, M, N, K)
+    ws = torch.empty(max(nbytes // 4, 1), device="cuda")
+    for w, nb in ((None, 0), (ws.data_ptr(), nbytes)):
+        C = torch.full((M, N), float("nan"), device="cuda")
+        rc = L.t2sp_sgemm_ex_f32(1, transb, M, N, K, 2.0, At.data_ptr(), M, Bd.data_ptr(), ldb, -3.0, C0.data_ptr(), N,
+                                 C.data_ptr(), N, 0, w, nb, None)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert torch.equal(C.double(), ref)
+    # a forced fast configuration cannot take the shape without the workspace and says so
+    C = torch.empty(M, N, device="cuda")
+    assert L.t2sp_sgemm_ex_f32(1, transb, M, N, K, 1.0, At.data_ptr(), M, Bd.data_ptr(), ldb, 0.0, None, 0, C.data_ptr(), N,
+                               1, None, 0, None) != 0   # T2SP_CFG_256x256
 
 
 @pytest.mark.parametrize("K", [4, 20, 36, 60, 64, 68, 100, 132, 1000, 4104])
