@@ -197,12 +197,13 @@ def cpu_baseline_sgemm_1024(oracle, A, B):
             "sample": "golden loop (i,j,k order, scalar accumulator), the full 1024^3 problem, single thread, %.1f s" % dt}
 
 
-def check_conv(oracle, tensors, cpu_seconds):
+def check_conv(oracle, tensors, cpu_seconds, ure=True):
     """configs[2]: parity on two images x 24 output channels; CPU: the golden loop order (ci -> kx -> ky per
     output, conv-run-fpga.cpp:73-93), one thread, on a declared sample of output channels of one image."""
     I, W, O = tensors
     N, CO = I.shape[0], W.shape[0]
     imgs, cos = [0, N - 1], slice(100, 124)
+    ure = cpu_seconds and ure
     In, Wn = I[imgs].cpu().numpy(), W.cpu().numpy()
     # device layout [n][c][h][w] with w = the reference's y: the oracle indexes (n, ci, y, x)
     ref = oracle.conv(In.transpose(0, 1, 3, 2), Wn.transpose(0, 1, 3, 2), co_range=(cos.start, cos.stop))[:, cos]
@@ -221,24 +222,48 @@ def check_conv(oracle, tensors, cpu_seconds):
         out["cpu_baseline"] = {"value": round(flop / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
                                "sample": "sampled: golden order per output, single thread, %d of %d output channels of 1 of %d "
                                          "images, %.1f s; extrapolated full problem: %.0f s" % (n_co, CO, N, dt, dt * CO / n_co * N)}
+        if ure:
+            # the spec executed as one serial loop nest in its own order (conv.cpp:30,59-65: ci outermost, then
+            # kx, ky, then the output tile loops, cii innermost; CII = 8 as in the GPU constant set), what a
+            # host-target build of the merged UREs runs
+            t0 = time.perf_counter()
+            oracle.conv(one, Wt, co_range=(0, n_co), threads=1, order=oracle.ORDER_URE, cii=8)
+            dtu = time.perf_counter() - t0
+            out["cpu_baseline"]["ure_order"] = {
+                "value": round(flop / dtu / 1e12, 6), "unit": "TFLOP/s", "cores": 1,
+                "sample": "sampled: spec loop nest (conv.cpp:30,59-65, CII = 8), single thread, the same %d output channels of "
+                          "1 image, %.1f s" % (n_co, dtu)}
     return out
 
 
-def check_capsule(oracle, tensors, cpu_seconds):
+def check_capsule(oracle, tensors, cpu_seconds, images=None):
     """configs[3]: parity on every vote; CPU: the golden loop order (kx -> ky -> mk -> ci per vote,
-    capsule-run-fpga.cpp:78-104), one thread, the full problem."""
+    capsule-run-fpga.cpp:78-104), one thread, the full problem.  `images`: check (and time) only these."""
     P, W, V = tensors
+    if images is not None:
+        P, V = P[images], V[images]
     Pn, Wn = P.cpu().numpy(), W.cpu().numpy()
     # device layout P [n][ci][h][w][mx][mk] with w = the reference's y: the oracle indexes (n, ci, y, x, mx, mk)
     Pt, Wt = Pn.transpose(0, 1, 3, 2, 4, 5), Wn.transpose(0, 1, 3, 2, 4, 5)
     t0 = time.perf_counter()
     ref = oracle.capsule(Pt, Wt, threads=1)
     dt = time.perf_counter() - t0
-    out = {"parity": parity_of(V.cpu().numpy().transpose(0, 1, 3, 2, 4, 5), ref, "all %d votes against the CPU oracle (golden order)" % ref.size)}
+    what = ("all %d votes" % ref.size) if images is None else ("the %d votes of images %s" % (ref.size, list(images)))
+    out = {"parity": parity_of(V.cpu().numpy().transpose(0, 1, 3, 2, 4, 5), ref, what + " against the CPU oracle (golden order)")}
     if cpu_seconds:
         flop = 2.0 * ref.size * Pn.shape[1] * 9 * 4
         out["cpu_baseline"] = {"value": round(flop / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
-                               "sample": "golden order per vote, single thread, the full problem, %.1f s" % dt}
+                               "sample": "golden order per vote, single thread, %s, %.1f s" % (
+                                   "the full problem" if images is None else "sampled: %d images" % len(images), dt)}
+        if images is None:
+            # the spec's own loop order (capsule.cpp:28,60-66: mk outermost, then ci, kx, ky, then the output tile
+            # loops, cii innermost; CII = 4 as in the GPU constant set), one serial loop nest
+            t0 = time.perf_counter()
+            oracle.capsule(Pt, Wt, threads=1, order=oracle.ORDER_URE, cii=4)
+            dtu = time.perf_counter() - t0
+            out["cpu_baseline"]["ure_order"] = {
+                "value": round(flop / dtu / 1e12, 6), "unit": "TFLOP/s", "cores": 1,
+                "sample": "spec loop nest (capsule.cpp:28,60-66, CII = 4), single thread, the full problem, %.1f s" % dtu}
     return out
 
 
@@ -265,6 +290,33 @@ def check_mttkrp(oracle, tensors, cpu_seconds):
         out["cpu_baseline"] = {"value": round(flop / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
                                "sample": "sampled: two-step order of util.h:498-515, single thread, %d of %d rows i, %.1f s; "
                                          "extrapolated full problem: %.0f s" % (n_rows, I, dt, dt * I / n_rows)}
+    return out
+
+
+def published_shapes(torch, t2sp_amd, oracle, bench_ops, steps):
+    """The problem sizes of the reference's own README tables (measured there on FPGAs and Intel GPUs): capsule
+    at N = 64, 256 and 4096 (capsule/README.md:13-16), conv I(4,256,64,64) * K(256,256,3,3) (conv/README.md:15-16),
+    SGEMM 2048^3 and A(10240,16384) * B(16384,8192) (gemm/README.md:9-12).  Each with parity on a sample."""
+    import numpy as np
+    out = {}
+    for n in (64, 256, 4096):
+        e = bench_ops.capsule_case(torch, steps, 3, PEAK_FP32_MFMA_TFLOPS, n, 0, 0,
+                                   "P(%d,32,15,15,4,4) * W(32,32,3,3,4,4), stride 2 (capsule/README.md:13-16)" % n, graph=False)
+        e.update(check_capsule(oracle, e.pop("_tensors"), None, images=[0, n // 2, n - 1]))
+        out["capsule_n%d" % n] = e
+    e = bench_ops.conv_case(torch, max(steps, 50), 5, PEAK_FP32_MFMA_TFLOPS, 4, 256, 256, 64, 64,
+                            "I(4,256,64,64) * K(256,256,3,3) (conv/README.md:15-16)")
+    e.update(check_conv(oracle, e.pop("_tensors"), None))
+    out["conv_n4_256ch_64x64"] = e
+    for (m, n, k, src) in ((2048, 2048, 2048, "gemm/README.md:12"), (10240, 8192, 16384, "gemm/README.md:9")):
+        c = sgemm_case(torch, t2sp_amd, m, n, k, max(steps, 50) if m == 2048 else steps, 5, min_warm_ms=100.0)
+        tf = c["flop"] / (c["avg_ms"] * 1e-3) / 1e12
+        out["sgemm_%dx%dx%d" % (m, n, k)] = {
+            "TFLOP/s": round(tf, 3), "frac_of_peak": round(tf / PEAK_FP32_MFMA_TFLOPS, 4), "avg_launch_ms": round(c["avg_ms"], 4),
+            "workload": "A(%d,%d) * B(%d,%d) (%s)" % (m, k, k, n, src),
+            "parity": parity_of(c["C"][:16].cpu().numpy(), oracle.gemm(c["A"][:16].cpu().numpy(), c["B"].cpu().numpy()),
+                                "rows 0-15 against the CPU oracle (golden order)")}
+        del c
     return out
 
 
@@ -377,6 +429,7 @@ def main():
             more[name].update(check(oracle, tensors, None if args.no_cpu else args.cpu_seconds / 4))
             del tensors
         others.update(more)
+        others["reference_published_shapes"] = published_shapes(torch, t2sp_amd, oracle, bench_ops, max(5, args.steps // 2))
         out["others"] = others
         if not args.no_cpu:
             out["end_to_end"] = end_to_end_gemm(torch, t2sp_amd, M, N, K)

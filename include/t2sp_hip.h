@@ -33,6 +33,7 @@ extern "C" {
 #define T2SP_CFG_32x128 4 /* sgemm: one wavefront per tile, for problems with few outputs; mttkrp: the 256x64 tile for small ranks */
 #define T2SP_CFG_DIRECT 5 /* small problems (sgemm, capsule): one small tile per workgroup, reduction split over its waves, operands global -> registers */
 #define T2SP_CFG_DIRECT16 6 /* sgemm, conv, capsule: the direct form on 16x16 MFMA tiles, rows (and column blocks) per workgroup chosen to fill the CUs evenly */
+#define T2SP_CFG_256x128 7 /* sgemm, capsule: four waves of 64x128, two workgroups per CU; for outputs of at most 128 columns */
 #define T2SP_CFG_SCALAR 99
 
 #define T2SP_MAX_DIMS 10

@@ -38,8 +38,11 @@ def _entry(tf, peak, ms, **extra):
 
 
 def conv_config3(torch, steps, warmup, peak):
+    return conv_case(torch, steps, warmup, peak, 64, 256, 256, 56, 56, "N=64 CI=CO=256 56x56 out 3x3 NCHW, seeds 1,2 (configs[2])")
+
+
+def conv_case(torch, steps, warmup, peak, N, CI, CO, OH, OW, workload, cfg=0):
     L = lib()
-    N, CI, CO, OH, OW = 64, 256, 256, 56, 56
     I = ops.fill_uniform(torch.empty(N, CI, OH + 2, OW + 2, device="cuda"), 1)
     W = ops.fill_uniform(torch.empty(CO, CI, 3, 3, device="cuda"), 2)
     O = torch.empty(N, CO, OH, OW, device="cuda")
@@ -49,20 +52,25 @@ def conv_config3(torch, steps, warmup, peak):
     ws = torch.empty(max(nbytes // 4, 1), device="cuda")
 
     def launch():
-        rc = L.t2sp_conv2d_f32(I.data_ptr(), W.data_ptr(), O.data_ptr(), N, CI, CO, OH, OW, 3, 3, si, sw, so, 0,
+        rc = L.t2sp_conv2d_f32(I.data_ptr(), W.data_ptr(), O.data_ptr(), N, CI, CO, OH, OW, 3, 3, si, sw, so, cfg,
                                ws.data_ptr(), nbytes, s)
         assert rc == 0, rc
 
     ms = _time(torch, launch, steps, warmup)
     flop = 2.0 * N * CO * OH * OW * CI * 9
-    e = _entry(flop / ms / 1e9, peak, ms, workload="N=64 CI=CO=256 56x56 out 3x3 NCHW, seeds 1,2 (configs[2])")
+    e = _entry(flop / ms / 1e9, peak, ms, workload=workload)
     e["_tensors"] = (I, W, O)
     return e
 
 
 def capsule_config4(torch, steps, warmup, peak, cfg=0, splits=0):
+    return capsule_case(torch, steps, warmup, peak, 32, cfg, splits,
+                        "N=32 CI=CO=32 15x15->7x7 3x3 s2 4x4 poses, seeds 1,2 (configs[3])")
+
+
+def capsule_case(torch, steps, warmup, peak, N, cfg, splits, workload, graph=True):
     L = lib()
-    N, CI, CO = 32, 32, 32
+    CI, CO = 32, 32
     P = ops.fill_uniform(torch.empty(N, CI, 15, 15, 4, 4, device="cuda"), 1)
     W = ops.fill_uniform(torch.empty(CO, CI, 3, 3, 4, 4, device="cuda"), 2)
     V = torch.empty(N, CO, 7, 7, 4, 4, device="cuda")
@@ -77,12 +85,11 @@ def capsule_config4(torch, steps, warmup, peak, cfg=0, splits=0):
                                 nbytes, s)
         assert rc == 0, rc
 
-    ms = _time(torch, launch, max(steps, 200), max(warmup, 20))
+    ms = _time(torch, launch, max(steps, 200) if N <= 256 else steps, max(warmup, 20) if N <= 256 else warmup)
     flop = 2.0 * N * CO * 49 * 16 * CI * 9 * 4
-    e = _entry(flop / ms / 1e9, peak, ms, workload="N=32 CI=CO=32 15x15->7x7 3x3 s2 4x4 poses, seeds 1,2 (configs[3])",
-               note="back-to-back launches; the library's own choice is one direct kernel without a split-reduction "
-                    "pass" if cfg == 0 else "forced cfg %d splits %d" % (cfg, splits))
-    if cfg == 0:
+    e = _entry(flop / ms / 1e9, peak, ms, workload=workload,
+               note="back-to-back launches; the library's own choice of kernel" if cfg == 0 else "forced cfg %d splits %d" % (cfg, splits))
+    if cfg == 0 and graph:
         e.update(_graph_replay(torch, launch_on=lambda st: L.t2sp_capsule_f32(
             P.data_ptr(), W.data_ptr(), V.data_ptr(), dims, sp, sw, sv, cfg, splits, ws.data_ptr(), nbytes, st), out=V))
     e["_tensors"] = (P, W, V)
@@ -122,7 +129,7 @@ def _graph_replay(torch, launch_on, out, per_graph=100, replays=20):
     return {"graph_replay_us_per_launch": round(us, 3), "graph_replays_equal_plain_launch": same}
 
 
-def mttkrp_config5(torch, steps, warmup, peak):
+def mttkrp_config5(torch, steps, warmup, peak, cfg=0, splits=0):
     L = lib()
     I = J = K = 512
     R = 256
@@ -130,14 +137,14 @@ def mttkrp_config5(torch, steps, warmup, peak):
     C = ops.fill_uniform(torch.empty(R, J, device="cuda"), 2).t()
     D = ops.fill_uniform(torch.empty(R, K, device="cuda"), 3).t()
     A = torch.empty(R, I, device="cuda").t()
-    nbytes = L.t2sp_mttkrp_workspace_bytes(I, J, K, R, 0, 0)
+    nbytes = L.t2sp_mttkrp_workspace_bytes(I, J, K, R, cfg, splits)
     ws = torch.empty(max(nbytes // 4, 1), device="cuda")
     sb, sc, sd, sa = (i64 * 3)(*B.stride()), (i64 * 2)(*C.stride()), (i64 * 2)(*D.stride()), (i64 * 2)(*A.stride())
     s = torch.cuda.current_stream().cuda_stream
 
     def launch():
         rc = L.t2sp_mttkrp_f32(B.data_ptr(), C.data_ptr(), D.data_ptr(), A.data_ptr(), I, J, K, R, sb, sc, sd, sa,
-                               0, 0, ws.data_ptr(), nbytes, s)
+                               cfg, splits, ws.data_ptr(), nbytes, s)
         assert rc == 0, rc
 
     ms = _time(torch, launch, steps, warmup)
@@ -412,3 +419,63 @@ def _run_all(torch, steps, warmup, peak, capsule_cfg=0, capsule_splits=0):
             "ssymv_16384": ssymv_case(torch, steps, warmup, peak),
             "pairhmm_224x224": pairhmm_case(torch, steps, warmup, peak),
             "qrd_128x128_b16384": qrd_case(torch, steps, warmup, peak)}
+
+
+def main(argv=None):
+    """One benchmark case with a forced kernel choice, a few launches, one JSON line: the program the
+    tile-choice counter runs under profiles/ put behind `rocprofv3 ... --`.
+
+        python3 -m t2sp_amd.bench_ops conv --cfg 1          # configs[2] on one launch of 256 x 256 tiles
+        python3 -m t2sp_amd.bench_ops mttkrp --cfg 2 --splits 64
+        python3 -m t2sp_amd.bench_ops capsule --batch 4096 --cfg 2
+        python3 -m t2sp_amd.bench_ops sgemm --shape 8192 8192 8192 --cfg 2
+
+    --cfg takes the T2SP_CFG_* numbers of include/t2sp_hip.h (0 = the library's own plan)."""
+    import argparse
+    import json
+    import torch
+    ap = argparse.ArgumentParser(description=main.__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("case", choices=["sgemm", "conv", "capsule", "mttkrp"])
+    ap.add_argument("--cfg", type=int, default=0)
+    ap.add_argument("--splits", type=int, default=0)
+    ap.add_argument("--batch", type=int, default=0, help="capsule / conv batch (default: the benchmark configuration's)")
+    ap.add_argument("--map", type=int, nargs=2, default=[56, 56], help="conv output map OH OW")
+    ap.add_argument("--shape", type=int, nargs=3, default=[8192, 8192, 8192], help="sgemm M N K")
+    ap.add_argument("--no-workspace", action="store_true", help="sgemm: pass no workspace")
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    a = ap.parse_args(argv)
+    peak = 157.3
+    if a.case == "conv":
+        n = a.batch or 64
+        e = conv_case(torch, a.steps, a.warmup, peak, n, 256, 256, a.map[0], a.map[1],
+                      "N=%d CI=CO=256 %dx%d out 3x3, cfg %d" % (n, a.map[0], a.map[1], a.cfg), a.cfg)
+    elif a.case == "capsule":
+        n = a.batch or 32
+        e = capsule_case(torch, a.steps, a.warmup, peak, n, a.cfg, a.splits, "N=%d cfg %d splits %d" % (n, a.cfg, a.splits), graph=False)
+    elif a.case == "mttkrp":
+        e = mttkrp_config5(torch, a.steps, a.warmup, peak, a.cfg, a.splits)
+        e["workload"] += ", cfg %d splits %d" % (a.cfg, a.splits)
+    else:
+        L = lib()
+        M, N, K = a.shape
+        A = ops.fill_uniform(torch.empty(M, K, device="cuda"), 1)
+        B = ops.fill_uniform(torch.empty(K, N, device="cuda"), 2)
+        C = torch.empty(M, N, device="cuda")
+        nbytes = 0 if a.no_workspace else L.t2sp_sgemm_workspace_bytes(M, N, K)
+        ws = torch.empty(max(nbytes // 4, 1), device="cuda")
+        s = torch.cuda.current_stream().cuda_stream
+
+        def launch():
+            rc = L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, a.cfg,
+                                  ws.data_ptr() if nbytes else None, nbytes, s)
+            assert rc == 0, rc
+
+        ms = _time(torch, launch, a.steps, a.warmup)
+        e = _entry(2.0 * M * N * K / ms / 1e9, peak, ms, workload="SGEMM %dx%dx%d cfg %d" % (M, N, K, a.cfg))
+    e.pop("_tensors", None)
+    print(json.dumps(e))
+
+
+if __name__ == "__main__":
+    main()

@@ -543,6 +543,7 @@ using CapsM = TileCfg<128, 128, 16, 4, 1, STYLE_RC>;
 using CapsS = TileCfg<64, 128, 16, 2, 1, STYLE_RC>;
 using CapsL = TileCfg<256, 256, 16, 4, 2, STYLE_RC>;
 using CapsW = TileCfg<32, 128, 16, 1, 1, STYLE_RC>;   // one wave per tile
+using CapsT = TileCfg<256, 128, 16, 4, 1, STYLE_RC>;  // four waves of 64 x 128: outputs of at most 128 columns, large batches
 
 constexpr int DIRECT_MAX_KRED = 16384;   // its per-wave offset tables must fit in LDS
 constexpr int DIRECT_MAX_TILES = 4096;  // beyond this the LDS-tiled kernels win (operands shared)
@@ -578,7 +579,7 @@ static CapsulePlan plan_capsule(int rows, int cols, int kred, int cfg, int split
         const int64_t t256 = (int64_t)((rows + 255) / 256) * ((cols + 255) / 256);
         cfg = (t256 >= machine().cus * 25 / 32 && cols > 128) ? T2SP_CFG_256x256 : (t128 >= 24 ? T2SP_CFG_128x128 : T2SP_CFG_64x128);
     }
-    const int bm = cfg == T2SP_CFG_256x256 ? 256 : cfg == T2SP_CFG_128x128 ? 128 : cfg == T2SP_CFG_64x128 ? 64 : 32;
+    const int bm = (cfg == T2SP_CFG_256x256 || cfg == T2SP_CFG_256x128) ? 256 : cfg == T2SP_CFG_128x128 ? 128 : cfg == T2SP_CFG_64x128 ? 64 : 32;
     const int bn = cfg == T2SP_CFG_256x256 ? 256 : 128;
     const int tiles = ((rows + bm - 1) / bm) * ((cols + bn - 1) / bn);
     const int ktiles = (kred + 15) / 16;
@@ -799,6 +800,7 @@ extern "C" int t2sp_capsule_f32(const float *P, const float *W, float *V, const 
         case T2SP_CFG_DIRECT: return launch_capsule_direct(g, (hipStream_t)stream);
         case T2SP_CFG_DIRECT16: return launch_capsule_direct16(g, (hipStream_t)stream);
         case T2SP_CFG_256x256: return launch_capsule<CapsL>(g, (hipStream_t)stream);
+        case T2SP_CFG_256x128: return launch_capsule<CapsT>(g, (hipStream_t)stream);
         case T2SP_CFG_128x128: return launch_capsule<CapsM>(g, (hipStream_t)stream);
         case T2SP_CFG_64x128: return launch_capsule<CapsS>(g, (hipStream_t)stream);
         case T2SP_CFG_32x128: return launch_capsule<CapsW>(g, (hipStream_t)stream);

@@ -875,6 +875,7 @@ using GemmL = TileCfg<256, 256, 16, 4, 2, STYLE_RC>;  // 8 waves, 64x128 per wav
 using GemmM = TileCfg<128, 128, 16, 4, 1, STYLE_RC>;  // 4 waves, 32x128 per wave
 using GemmS = TileCfg<64, 128, 16, 2, 1, STYLE_RC>;   // 2 waves, 32x128 per wave
 using GemmW = TileCfg<32, 128, 16, 1, 1, STYLE_RC>;   // 1 wave per tile
+using GemmT = TileCfg<256, 128, 16, 4, 1, STYLE_RC>;  // 4 waves, 64x128 per wave: tall products of at most 128 columns
 using GemmLT = TileCfg<256, 256, 16, 4, 2, STYLE_KC>;  // B^T forms: both operands k-contiguous
 using GemmMT = TileCfg<128, 128, 16, 2, 2, STYLE_KC>;
 using GemmST = TileCfg<64, 64, 16, 2, 1, STYLE_KC>;
@@ -1171,8 +1172,13 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         const bool big_tiles = t256 >= cus * 25 / 32 && fill256 >= 0.6;
         // 2304^3, 2560^3: the 16 x 16 form is 7-11 % ahead.  With B transposed it stores element by element and
         // whole rounds of 128 x 128 tiles are 4-10 % ahead of it (1024 x 4096 x 512, 2048^3, 4096 x 1024 x 1024).
+        // Whole rounds of 128 x 128 tiles beat it in both forms (plain form, 14 shapes with 256 or 512 tiles
+        // and K from 256 to 4096: +4 to +13 %, 2048^3 139 -> 146 TFLOP/s), and so do many rounds of them
+        // under an output of at most 128 columns, whatever K (65536 x 128 x 256: 89 -> 114; 802816 x 128 x
+        // 1152: 112 -> 130); 384 tiles (one and a half rounds) stay with the 16 x 16 form.
         const bool tiled_better = (t128 >= 2 * cus - cus / 16 && g.K >= 2048 && fill128 >= 0.6) ||
-                                  (bt && t128 % cus == 0 && fill128 >= 0.9);
+                                  (t128 % cus == 0 && fill128 >= 0.9) ||
+                                  (g.N <= 128 && t128 >= 2 * cus - cus / 16 && fill128 >= 0.9);
         // (with room for the planes the 16 x 16 form splits such a reduction over workgroups itself)
         const GemmD16Split sp = plan_gemm_d16_split(g.M, g.N, g.K, p);
         const bool can_split = !bt && sp.shift && workspace && workspace_bytes >= sp.scratch_bytes && ((uintptr_t)workspace % 16 == 0);
@@ -1254,6 +1260,7 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
     switch (cfg) {
         case T2SP_CFG_256x256: return launch<GemmL, false>(g, stream, 1, workspace, workspace_bytes, phased);
         case T2SP_CFG_128x128: return launch<GemmM, false>(g, stream, splits, workspace, workspace_bytes, phased);
+        case T2SP_CFG_256x128: return launch<GemmT, false>(g, stream);
         case T2SP_CFG_64x128: return launch<GemmS, false>(g, stream, splits, workspace);
         case T2SP_CFG_32x128: return launch<GemmW, false>(g, stream);
         default: return T2SP_ERR_SHAPE;
