@@ -172,7 +172,62 @@ struct PoseWeightRcLoader {
     }
 };
 
+// Weights that are dense behind their output channel (W[co][ci][kh][kw][mk][my] with nothing
+// between the inner five: the reduction index k = (ci, kh, kw, mk) then counts groups of four floats
+// from the channel's first): the 16 k-rows of a tile are 256 contiguous bytes per channel, so 16
+// adjacent lanes load one channel's piece (two cache lines) where the general loader above has
+// every lane of a load in a different line (a channel is CI*KH*KW*64 bytes from the next: 64 lines
+// per instruction, as many tag look-ups in the first-level cache).  No window walk either: a k-tile
+// further on is 256 bytes further on for every lane, a scalar offset of the buffer load.  A lane
+// writes its four columns of one k-row; the 16 lanes of a channel write 16 consecutive k-rows, which
+// the tile's row padding (TileCfg BPAD = 4) spreads over the banks.
 template <class Cfg, bool KPAD>
+struct DenseWeightRcLoader {
+    static_assert(Cfg::LDB % 32 == 4, "k-rows 4 banks apart");
+    uint32_t off[Cfg::B_VEC];     // the slot's (channel, k-row) from W, bytes
+    v4f reg[2][Cfg::B_VEC];
+    int k0;
+    const CapsuleArgs &g;
+    __device__ DenseWeightRcLoader(const CapsuleArgs &g_, int n0, int k_begin, const int *) : k0(k_begin), g(g_) {
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            const int f = threadIdx.x + i * Cfg::NTHREADS;
+            int co = (n0 >> 2) + f / Cfg::BK;
+            if (co * 4 >= g.COLS) co = 0;           // a column past the end reads the first: never stored
+            off[i] = 4u * (uint32_t)(co * (int)g.sw[0] + 4 * (f % Cfg::BK));
+        }
+    }
+    static constexpr bool HAS_TAIL_FETCH = KPAD;   // as in PoseKcLoader
+    template <int S>
+    __device__ __forceinline__ void fetch() {
+        const bool go = KPAD || k0 + 2 * Cfg::BK <= g.KRED;
+        const __amdgpu_buffer_rsrc_t rsrc = whole_buffer(g.W);
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) reg[S][i] = buffer_load<v4f>(rsrc, off[i], 16u * (uint32_t)k0);
+        k0 += go ? Cfg::BK : 0;
+    }
+    template <int S>
+    __device__ __forceinline__ void fetch_tail() {
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            const int k = (threadIdx.x + i * Cfg::NTHREADS) % Cfg::BK;
+            const bool ok = k0 + k < g.KRED;
+            const v4f v = *reinterpret_cast<const v4f *>(reinterpret_cast<const char *>(g.W) + (ok ? off[i] + 16u * (uint32_t)k0 : 0u));
+            reg[S][i] = ok ? v : v4f{0.f, 0.f, 0.f, 0.f};
+        }
+        k0 += Cfg::BK;
+    }
+    template <int S>
+    __device__ __forceinline__ void commit(float *stage) const {
+#pragma unroll
+        for (int i = 0; i < Cfg::B_VEC; i++) {
+            const int f = threadIdx.x + i * Cfg::NTHREADS;
+            *reinterpret_cast<v4f *>(stage + (f % Cfg::BK) * Cfg::LDB + 4 * (f / Cfg::BK)) = reg[S][i];
+        }
+    }
+};
+
+template <class Cfg, bool KPAD, bool WDENSE>
 __global__ void __launch_bounds__(Cfg::NTHREADS) capsule_kernel(const CapsuleArgs g) {
     extern __shared__ __align__(16) float smem[];
     int *tab_p = reinterpret_cast<int *>(smem + Cfg::SMEM_FLOATS);
@@ -186,7 +241,7 @@ __global__ void __launch_bounds__(Cfg::NTHREADS) capsule_kernel(const CapsuleArg
     int kt0, kt1;
     split_range((g.KRED + Cfg::BK - 1) / Cfg::BK, g.splits, split, kt0, kt1);
     PoseKcLoader<Cfg, KPAD> la(g, m0, kt0 * Cfg::BK, tab_p);
-    PoseWeightRcLoader<Cfg, KPAD> lb(g, n0, kt0 * Cfg::BK, tab_w);
+    std::conditional_t<WDENSE, DenseWeightRcLoader<Cfg, KPAD>, PoseWeightRcLoader<Cfg, KPAD>> lb(g, n0, kt0 * Cfg::BK, tab_w);
     Accum<Cfg> acc;
     mainloop<Cfg>(acc, la, lb, kt1 - kt0, smem, tail_from_for<Cfg>(g.KRED - kt0 * Cfg::BK));
     if (g.splits == 1) {
@@ -539,11 +594,12 @@ __global__ void capsule_scalar_kernel(const CapsuleGenericArgs g) {
     }
 }
 
-using CapsM = TileCfg<128, 128, 16, 4, 1, STYLE_RC>;
-using CapsS = TileCfg<64, 128, 16, 2, 1, STYLE_RC>;
-using CapsL = TileCfg<256, 256, 16, 4, 2, STYLE_RC>;
-using CapsW = TileCfg<32, 128, 16, 1, 1, STYLE_RC>;   // one wave per tile
-using CapsT = TileCfg<256, 128, 16, 4, 1, STYLE_RC>;  // four waves of 64 x 128: outputs of at most 128 columns, large batches
+// (k-rows of the weight tile padded by 4 floats: see DenseWeightRcLoader; harmless to the general loader)
+using CapsM = TileCfg<128, 128, 16, 4, 1, STYLE_RC, STYLE_KC, 4>;
+using CapsS = TileCfg<64, 128, 16, 2, 1, STYLE_RC, STYLE_KC, 4>;
+using CapsL = TileCfg<256, 256, 16, 4, 2, STYLE_RC, STYLE_KC, 4>;
+using CapsW = TileCfg<32, 128, 16, 1, 1, STYLE_RC, STYLE_KC, 4>;   // one wave per tile
+using CapsT = TileCfg<256, 128, 16, 4, 1, STYLE_RC, STYLE_KC, 4>;  // four waves of 64 x 128: outputs of at most 128 columns, large batches
 
 constexpr int DIRECT_MAX_KRED = 16384;   // its per-wave offset tables must fit in LDS
 constexpr int DIRECT_MAX_TILES = 4096;  // beyond this the LDS-tiled kernels win (operands shared)
@@ -565,7 +621,16 @@ static CapsulePlan plan_capsule(int rows, int cols, int kred, int cfg, int split
         const bool rounds_ok = t32 <= cus || t32 >= cus + cus / 2;
         // With 4-row poses the 16 x 16 form spreads any batch up to a few hundred evenly over the
         // CUs and was the fastest kernel at every batch from 8 to 256 (13-131 us against 19-152 us).
-        if (mx == 4 && t32 <= DIRECT_MAX_TILES && kred <= DIRECT_MAX_KRED) cfg = T2SP_CFG_DIRECT16;
+        // From a few hundred images on, rounds of 128 x 128 LDS tiles (one tile per CU at a time: the time
+        // goes with ceil(tiles / CUs)) are ahead when their last round is nearly full: N = 320 (490
+        // tiles, 0.96 of two rounds) 126 against 119 TFLOP/s, N = 640 (0.96 of four) 127 against 82,
+        // N = 768 (0.92 of five) 122 against 72; behind when it is not: N = 256 and 512 (0.77) 102
+        // against 126 and 103 against 120.
+        const int64_t t128 = (int64_t)((rows + 127) / 128) * ((cols + 127) / 128);
+        const double last_round_fill = (double)t128 / (double)(((t128 + cus - 1) / cus) * cus);
+        const bool lds_rounds = cols <= 128 && t128 >= cus && last_round_fill >= 0.85;
+        if (lds_rounds) cfg = T2SP_CFG_128x128;
+        else if (mx == 4 && t32 <= DIRECT_MAX_TILES && kred <= DIRECT_MAX_KRED) cfg = T2SP_CFG_DIRECT16;
         else if (t32 >= cus * 25 / 64 && t32 <= DIRECT_MAX_TILES && rounds_ok && kred <= DIRECT_MAX_KRED) cfg = T2SP_CFG_DIRECT;
     }
     if (cfg == T2SP_CFG_DIRECT || cfg == T2SP_CFG_DIRECT16) {
@@ -704,12 +769,15 @@ static int launch_capsule_direct(CapsuleArgs g, hipStream_t stream) {
     return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
 }
 
+// w_dense: the weights' inner five dimensions are contiguous and their byte offsets fit 32 bits
 template <class Cfg>
-static int launch_capsule(CapsuleArgs g, hipStream_t stream) {
+static int launch_capsule(CapsuleArgs g, hipStream_t stream, bool w_dense) {
     g.tiles_m = g.Mp / Cfg::BM;
     g.tiles_n = g.Np / Cfg::BN;
     const size_t smem = Cfg::SMEM_FLOATS * sizeof(float) + 2 * (size_t)g.KH * g.KW * sizeof(int);
-    auto kern = (g.KRED % (2 * Cfg::BK)) ? capsule_kernel<Cfg, true> : capsule_kernel<Cfg, false>;
+    const bool kpad = g.KRED % (2 * Cfg::BK);
+    auto kern = w_dense ? (kpad ? capsule_kernel<Cfg, true, true> : capsule_kernel<Cfg, false, true>)
+                        : (kpad ? capsule_kernel<Cfg, true, false> : capsule_kernel<Cfg, false, false>);
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * g.splits), dim3(Cfg::NTHREADS), smem, stream, g);
@@ -796,14 +864,16 @@ extern "C" int t2sp_capsule_f32(const float *P, const float *W, float *V, const 
     for (int i = 0; i < 5; i++) { g.sp[i] = sp6[i]; g.sw[i] = sw6[i]; g.sv[i] = sv6[i]; }
     g.ROWS = (int)rows; g.COLS = (int)cols; g.KRED = (int)kred;
     g.splits = p.splits; g.Mp = p.Mp; g.Np = p.Np; g.scratch = workspace;
+    const bool w_dense = byte_offsets_fit && sw6[4] == 4 && sw6[3] == 16 && sw6[2] == 16 * (int64_t)d[6] &&
+                         sw6[1] == 16 * (int64_t)d[6] * d[5];
     switch (p.cfg) {
         case T2SP_CFG_DIRECT: return launch_capsule_direct(g, (hipStream_t)stream);
         case T2SP_CFG_DIRECT16: return launch_capsule_direct16(g, (hipStream_t)stream);
-        case T2SP_CFG_256x256: return launch_capsule<CapsL>(g, (hipStream_t)stream);
-        case T2SP_CFG_256x128: return launch_capsule<CapsT>(g, (hipStream_t)stream);
-        case T2SP_CFG_128x128: return launch_capsule<CapsM>(g, (hipStream_t)stream);
-        case T2SP_CFG_64x128: return launch_capsule<CapsS>(g, (hipStream_t)stream);
-        case T2SP_CFG_32x128: return launch_capsule<CapsW>(g, (hipStream_t)stream);
+        case T2SP_CFG_256x256: return launch_capsule<CapsL>(g, (hipStream_t)stream, w_dense);
+        case T2SP_CFG_256x128: return launch_capsule<CapsT>(g, (hipStream_t)stream, w_dense);
+        case T2SP_CFG_128x128: return launch_capsule<CapsM>(g, (hipStream_t)stream, w_dense);
+        case T2SP_CFG_64x128: return launch_capsule<CapsS>(g, (hipStream_t)stream, w_dense);
+        case T2SP_CFG_32x128: return launch_capsule<CapsW>(g, (hipStream_t)stream, w_dense);
         default: return T2SP_ERR_SHAPE;
     }
 }

@@ -283,7 +283,6 @@ template <> struct VecOf<2> { typedef float type __attribute__((ext_vector_type(
 template <> struct VecOf<4> { typedef float type __attribute__((ext_vector_type(4))); };
 
 // Timeline stamps of this kernel (100 MHz wall clock, one set per wave), compiled in only by
-// `make trace-lib`; python -m t2sp_amd.d16_timeline reads them back.
 // What the loop of the 16 x 16 form needs of the arguments.  The kernel takes these as leading
 // scalar parameters, which the dispatcher preloads into scalar registers before the first wave
 // starts (the build sets -amdgpu-kernarg-preload-count): a wave that has to fetch them from the
@@ -395,14 +394,33 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     const int lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
     // a grid of tiles_m x tiles_n: no division on the way to the first loads (every instruction before
     // them is fetched through a cold instruction cache at each launch)
-    const int tm = blockIdx.x, tn = blockIdx.y;
+    int tm = blockIdx.x, tn = blockIdx.y, share = 0;
+    if (split_shift) {
+        // The reduction is split over 2^split_shift workgroups per tile (tiny outputs with a long
+        // reduction).  Workgroup ids are dealt round-robin to the dies, each with its own L2, so the
+        // share of k is taken from the id's die: a die then walks 1/nxcd of k for every tile and
+        // fetches its slabs of A and B once, instead of every die fetching all of both (256 x 256 x
+        // 16384: 155 MB fetched for 34 MB of operands before).
+        const int lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+        const int S = 1 << split_shift, nx = g.nxcd;
+        int tile;
+        if (nx > 1 && S >= nx && S % nx == 0) {
+            const int rest = lin / nx, per = S / nx;
+            share = lin % nx + nx * (rest % per);
+            tile = rest / per;
+        } else {
+            share = lin & (S - 1);
+            tile = lin >> split_shift;
+        }
+        tn = tile / (int)gridDim.x;
+        tm = tile - tn * (int)gridDim.x;
+    }
     const int m0 = tm * rows_per_tile, n0 = tn * 16 * NB;
     const int m_end = min(m0 + rows_per_tile, M);
     const int steps = K >> 4;
-    // blockIdx.z: the workgroup's share of the reduction when it is split over 2^split_shift
-    // workgroups per tile (tiny outputs with a long reduction); its waves split that share again
+    // the workgroup's share of the reduction; its waves split that share again
     static_assert(NW == 4, "shares of the reduction by shifts");
-    const int z0 = (int)(((int64_t)steps * blockIdx.z) >> split_shift), z1 = (int)(((int64_t)steps * (blockIdx.z + 1)) >> split_shift);
+    const int z0 = (int)(((int64_t)steps * share) >> split_shift), z1 = (int)(((int64_t)steps * (share + 1)) >> split_shift);
     const int s0 = z0 + (((z1 - z0) * wave) >> 2), s1 = z0 + (((z1 - z0) * (wave + 1)) >> 2);
     const GemmHot hot{A, B, M, N, lda, ldb};
     sgemm_d16_wave<MB, NB, BUF>(hot, 0, m0, n0, s0, s1 - s0, steps, red + wave * MB * NB * 64);
@@ -447,7 +465,7 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
             if (row < m_end && col_ok) {
                 if (split_shift) {
                     // a partial sum: plane blockIdx.z of the workspace, M x N; the kernel that adds the planes scales and stores
-                    *reinterpret_cast<vnb *>(g.scratch + ((int64_t)blockIdx.z * M + row) * N + col) = out;
+                    *reinterpret_cast<vnb *>(g.scratch + ((int64_t)share * M + row) * N + col) = out;
                     continue;
                 }
                 if (g.scale) {
@@ -464,11 +482,48 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
         }
     }
 }
+// 4 x 4 transpose across the four lanes of a quad: lane e of a quad (e = lane & 3) enters with v[r]
+// = X[r][e] and leaves with v[j] = X[e][j].  Two butterfly stages, lanes e and e ^ 1 on the register
+// pairs (0,1) and (2,3), then lanes e and e ^ 2 on the pairs (0,2) and (1,3): each lane sends the
+// element of the pair that belongs to its partner through a quad-permute DPP move and keeps the
+// other.  16 vector instructions, no LDS.
+__device__ __forceinline__ float quad_swap(float x, bool by_two) {
+    const int xi = __builtin_bit_cast(int, x);
+    // quad_perm [1,0,3,2] = 0xB1, [2,3,0,1] = 0x4E
+    const int yi = by_two ? __builtin_amdgcn_update_dpp(xi, xi, 0x4E, 0xf, 0xf, false)
+                          : __builtin_amdgcn_update_dpp(xi, xi, 0xB1, 0xf, 0xf, false);
+    return __builtin_bit_cast(float, yi);
+}
+__device__ __forceinline__ v4f quad_transpose(v4f v, int e) {
+    const bool odd = e & 1, high = e & 2;
+    // stage 1: 2 x 2 blocks (registers r, r + 1) x (lanes e, e ^ 1)
+    {
+        const float s01 = odd ? v[0] : v[1], s23 = odd ? v[2] : v[3];
+        const float r01 = quad_swap(s01, false), r23 = quad_swap(s23, false);
+        v[0] = odd ? r01 : v[0];
+        v[1] = odd ? v[1] : r01;
+        v[2] = odd ? r23 : v[2];
+        v[3] = odd ? v[3] : r23;
+    }
+    // stage 2: (registers r, r + 2) x (lanes e, e ^ 2)
+    {
+        const float s02 = high ? v[0] : v[2], s13 = high ? v[1] : v[3];
+        const float r02 = quad_swap(s02, true), r13 = quad_swap(s13, true);
+        v[0] = high ? r02 : v[0];
+        v[2] = high ? v[2] : r02;
+        v[1] = high ? r13 : v[1];
+        v[3] = high ? v[3] : r13;
+    }
+    return v;
+}
+
 // The same form for B stored transposed (N x K, k contiguous: C = A * B^T, the layout of a weight
 // matrix): both operands are read as A is above, 4 consecutive k of one row (of A) or column (of
 // the product) per lane and 128-bit load, element j feeding MFMA j; accumulator block nb holds the
-// 16 adjacent columns n0 + 16 nb ..; the exchange through LDS that sums the waves' partial tiles
-// also turns a lane's four rows of one column into four adjacent columns of one row.
+// 16 adjacent columns n0 + 16 nb ..; the waves' partial tiles are summed through LDS as in the
+// first form (128-bit, lane-contiguous, no bank conflicts), and a 4 x 4 transpose inside each quad of
+// lanes then turns a lane's four rows of one column into four adjacent columns of one row, so that C
+// is written 128 bits at a time.
 template <int MB, int NB>
 __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     sgemm_direct16_bt_kernel(const float *A, const float *B, int M, int N, int K, int lda, int ldb, int tiles_m, int rows_per_tile,
@@ -537,20 +592,15 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
 #undef T2SP_GEMM_D16BT_ISSUE
 #undef T2SP_GEMM_D16BT_MMA
 
-    // A lane holds four rows of one column of each block; the partial blocks go to LDS row by row
-    // ([wave][block][row][column], one float per lane and store) so that they come back as four
-    // adjacent columns of one row per lane: 128-bit reads, and 128-bit stores to C where its rows allow.
-    // (row rho of a block starts at float 16 rho + 16 (rho / 4): the four row groups a store instruction
-    // writes then fall into four different sets of banks)
-    constexpr int BLK = 16 * 16 + 4 * 16;
-    float *mine = smem + wave * MB * NB * BLK + (4 * lq) * 16 + 16 * lq + li;
+    // A lane holds four rows (4 lq + r) of one column (li) of each block.  After the sum over the
+    // waves, quad_transpose gives lane li = 4c + e the four adjacent columns 4c .. 4c + 3 of row 4 lq + e.
+    v4f *red = reinterpret_cast<v4f *>(smem);            // [wave][mb][nb][lane]
+    v4f *mine = red + wave * MB * NB * 64 + lane;
 #pragma unroll
     for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) mine[(mb * NB + nb) * BLK + r * 16] = acc[mb][nb][r];
-    const int orow = lane >> 2, ocol = (lane & 3) * 4;              // this lane's row and first column inside a block
+        for (int nb = 0; nb < NB; nb++) mine[(mb * NB + nb) * 64] = acc[mb][nb];
+    const int orow = 4 * lq + (li & 3), ocol = li & ~3;             // this lane's row and first column inside a block
     const bool vec_ok = !g.tiled && g.ldc % 4 == 0 && ((uintptr_t)g.C % 16 == 0) &&
                         (!g.scale || g.beta == 0.f || (g.ldcin % 4 == 0 && ((uintptr_t)g.Cin % 16 == 0)));
     // beta * Cin of this wave's blocks: requested before the exchange (see sgemm_direct16_kernel)
@@ -570,11 +620,12 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
 #pragma unroll
     for (int i = 0; i < PER_WAVE; i++) {                 // sum the partial blocks of the waves in wave order
         const int pr = wave + i * NW;
-        if (pr >= MB * NB) break;
-        const v4f *src = reinterpret_cast<const v4f *>(smem + pr * BLK + orow * 16 + 16 * (orow >> 2) + ocol);
+        if (pr >= MB * NB) break;                        // the same for every lane of the wave
+        const v4f *src = red + pr * 64 + lane;
         v4f sum = src[0];
 #pragma unroll
-        for (int wv = 1; wv < NW; wv++) sum += src[wv * MB * NB * (BLK / 4)];
+        for (int wv = 1; wv < NW; wv++) sum += src[wv * MB * NB * 64];
+        sum = quad_transpose(sum, li & 3);
         const int mb = pr / NB, nb = pr - mb * NB;
         const int row = m0 + 16 * mb + orow, col = n0 + 16 * nb + ocol;
         if (row >= m_end) continue;
@@ -975,35 +1026,59 @@ static GemmD16Plan plan_gemm_d16(int M, int N) {
     return best;
 }
 
-// Tiny outputs with a long reduction: the tiles of the plan above leave most CUs idle, so each goes
-// to 2^shift workgroups that each reduce a share of k into a plane of the workspace, and a second
-// kernel adds the planes in order.  As many shares as fit one round of workgroups and leave each
-// workgroup 32 steps of 16 k (8 per wave) or more; not at all where the time saved would not pay
-// for the second launch.  Measured with every tile and split forced (256 x 256 x 16384,
-// 128 x 128 x 4096, 64 x 64 x 65536, ...): the small tiles of the plan above, split this way, are
-// within a few per cent of the best choice everywhere, and larger tiles with deeper splits are not
-// better: a step costs its MFMAs or its loads whichever is longer, and with few tiles the time is
-// that of one workgroup.
+// Tiny outputs with a long reduction: the tiles of the plan above leave most CUs idle, so each tile
+// goes to 2^shift workgroups that each reduce a share of k into a plane of the workspace, and a
+// second kernel adds the planes in order.  Tile and depth are chosen together, by estimated time:
+//   steps per wave x a step's MFMAs (16 x 16 x 4, 32 cycles each) or its loads, whichever is longer
+//   (measured 0.345 us for the six loads of a 32 x 32 step), + the planes written and read back.
+// Shares of k follow the dies (see sgemm_direct16_kernel), so a depth that is a multiple of the die
+// count fetches every operand once; with that, 64-column tiles (128-bit loads of B, half the loads
+// per MFMA) beat the smallest tile wherever 8 shares of them fill the chip.  Measured with tile and
+// depth forced, 13 combinations each: 256 x 256 x 16384 32.7 -> 25.6 us (32 x 64 tiles, 8 shares),
+// 256 x 256 x 65536 96 -> 68 us, 512 x 256 x 16384 56 -> 43 us; 128 x 128 x 4096 and 64 x 64 x 65536
+// keep 32 x 32 tiles with 8 and 32 shares.  At least 32 steps of 16 k per workgroup (8 per wave), and
+// no split where the time saved would not pay for the second launch.
 struct GemmD16Split {
     int shift;                 // 0: no split
     size_t scratch_bytes;
+    GemmD16Plan tile;          // the tile to split (valid when shift > 0)
 };
-static GemmD16Split plan_gemm_d16_split(int M, int N, int K, const GemmD16Plan &p) {
-    const int cus = machine().cus;
-    const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
-    GemmD16Split r{0, 0};
-    if (tiles <= 0 || tiles > cus / 2 || K % 16) return r;
+static GemmD16Split plan_gemm_d16_split(int M, int N, int K, const GemmD16Plan &unsplit) {
+    const int cus = machine().cus, nx = machine().xcds;
+    GemmD16Split r{0, 0, unsplit};
+    if ((int64_t)unsplit.tiles_m * unsplit.tiles_n <= 0 || (int64_t)unsplit.tiles_m * unsplit.tiles_n > cus / 2 || K % 16) return r;
     const int steps = K / 16;
-    int shift = 0;
-    while (shift < 5 && (tiles << (shift + 1)) <= cus && (steps >> (shift + 1)) >= 32) shift++;
-    if (!shift) return r;
-    // a step of the tile: its MFMAs (16 x 16 x 4, 32 cycles each) or its loads (measured 0.345 us for 32 x 32)
-    const double mfma_us = 4.0 * p.mb * p.nb * 32.0 / 2400.0 * 1.03, load_us = (p.mb + 4) * 0.0575;
-    const double step_us = mfma_us > load_us ? mfma_us : load_us;
-    const double saved_us = (steps / 4.0) * step_us * (1.0 - 1.0 / (1 << shift));
-    if (saved_us < 8.0) return r;                                         // the second launch and its pass over the planes
-    r.shift = shift;
-    r.scratch_bytes = ((size_t)M * N << shift) * sizeof(float);
+    auto step_us = [](int mb, int nb) {
+        const double mfma_us = 4.0 * mb * nb * 32.0 / 2400.0 * 1.03, load_us = (mb + 4) * 0.0575;
+        return mfma_us > load_us ? mfma_us : load_us;
+    };
+    double best = 1e300;
+    for (int nb = 2; nb <= 4; nb += 2)
+        for (int mb = 2; mb <= 4; mb++) {
+            const int tiles_m = (M + 16 * mb - 1) / (16 * mb), tiles_n = (N + 16 * nb - 1) / (16 * nb);
+            const int64_t tiles = (int64_t)tiles_m * tiles_n;
+            if (tiles > cus / 2 || tiles_n > 65535) continue;
+            int shift = 0;
+            while (shift < 5 && (tiles << (shift + 1)) <= cus && (steps >> (shift + 1)) >= 32) shift++;
+            if (!shift) continue;
+            const int S = 1 << shift;
+            const double planes_us = (double)S * M * N * 8.0 / 3.0e6;          // written, then read, at about 3 TB/s
+            const double apart = (nx > 1 && S % nx) ? 1.15 : 1.0;               // dies share slabs of k
+            const double t = (double)steps / S / 4.0 * step_us(mb, nb) * apart + planes_us;
+            if (t < best) {
+                best = t;
+                r.shift = shift;
+                r.tile = GemmD16Plan{mb, nb, (M + tiles_m - 1) / tiles_m, tiles_m, tiles_n, t};
+            }
+        }
+    if (!r.shift) return r;
+    const double unsplit_us = (steps / 4.0) * step_us(unsplit.mb, unsplit.nb);
+    if (unsplit_us - best < 8.0) {                                          // the second launch and its pass over the planes
+        r.shift = 0;
+        r.tile = unsplit;
+        return r;
+    }
+    r.scratch_bytes = ((size_t)M * N << r.shift) * sizeof(float);
     return r;
 }
 
@@ -1019,6 +1094,7 @@ static int launch_d16_t(GemmArgs g, const GemmD16Plan &p, hipStream_t stream, in
     g.tiles_m = p.tiles_m;
     g.tiles_n = p.tiles_n;
     g.scratch = scratch;
+    g.nxcd = machine().xcds;
     const size_t smem = (size_t)GEMM_D16_WAVES * MB * NB * 64 * sizeof(v4f);
     // one workgroup per CU at most, or a short reduction: the form whose loop has no vector arithmetic
     // (see sgemm_d16_wave; measured with several rounds: 2048 x 1024 x 512 20.7 -> 18.8 us,
@@ -1039,10 +1115,11 @@ static int launch_d16_t(GemmArgs g, const GemmD16Plan &p, hipStream_t stream, in
 }
 
 static int launch_d16(const GemmArgs &g, hipStream_t stream, float *workspace = nullptr, size_t workspace_bytes = 0) {
-    const GemmD16Plan p = plan_gemm_d16(g.M, g.N);
-    GemmD16Split sp = plan_gemm_d16_split(g.M, g.N, g.K, p);
+    const GemmD16Plan whole = plan_gemm_d16(g.M, g.N);
+    GemmD16Split sp = plan_gemm_d16_split(g.M, g.N, g.K, whole);
     if (!workspace || workspace_bytes < sp.scratch_bytes || ((uintptr_t)workspace % 16)) sp.shift = 0;
     const int shift = sp.shift;
+    const GemmD16Plan p = shift ? sp.tile : whole;
 #define T2SP_D16_CASE(MBV, NBV) if (p.mb == MBV && p.nb == NBV) return launch_d16_t<MBV, NBV>(g, p, stream, shift, workspace);
     T2SP_D16_CASE(2, 2) T2SP_D16_CASE(3, 2) T2SP_D16_CASE(4, 2) T2SP_D16_CASE(5, 2) T2SP_D16_CASE(6, 2)
     T2SP_D16_CASE(7, 2) T2SP_D16_CASE(8, 2) T2SP_D16_CASE(2, 4) T2SP_D16_CASE(3, 4) T2SP_D16_CASE(4, 4)
@@ -1076,7 +1153,7 @@ template <int MB, int NB>
 static int launch_d16_bt_t(GemmArgs g, const GemmD16Plan &p, hipStream_t stream) {
     g.tiles_m = p.tiles_m;
     g.tiles_n = p.tiles_n;
-    const size_t smem = (size_t)GEMM_D16_WAVES * MB * NB * (16 * 16 + 4 * 16) * sizeof(float);
+    const size_t smem = (size_t)GEMM_D16_WAVES * MB * NB * 64 * sizeof(v4f);
     auto kern = sgemm_direct16_bt_kernel<MB, NB>;
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;

@@ -53,7 +53,10 @@ enum : int { STYLE_KC = 0, STYLE_RC = 1 };
 
 typedef float v2f __attribute__((ext_vector_type(2)));
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int BSTYLE_, int ASTYLE_ = STYLE_KC>
+// BPAD_: floats of padding per k-row of an RC Y tile, for loaders whose lanes write one column
+// group of consecutive k-rows each (rows a whole number of banks apart would collide); loaders that
+// write consecutive columns of one k-row need none.
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int BSTYLE_, int ASTYLE_ = STYLE_KC, int BPAD_ = 0>
 struct TileCfg {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, BSTYLE = BSTYLE_, ASTYLE = ASTYLE_;
     static constexpr int NTHREADS = WM * WN * 64;
@@ -62,7 +65,8 @@ struct TileCfg {
     static constexpr int MT = TM / 32;          // 32-row accumulator tiles per wave
     static constexpr int NT = TN / 32;          // 32-col accumulator tiles per wave
     static constexpr int LDA = (ASTYLE == STYLE_RC) ? BM : BK + 4;   // floats per row of the X tile
-    static constexpr int LDB = (BSTYLE == STYLE_RC) ? BN : BK + 4;
+    static constexpr int LDB = (BSTYLE == STYLE_RC) ? BN + BPAD_ : BK + 4;
+    static_assert(BPAD_ % 4 == 0, "rows of the tile stay 16-byte aligned");
     static constexpr int A_STAGE = (ASTYLE == STYLE_RC) ? BK * LDA : BM * LDA;    // floats
     static constexpr int A_READS = (ASTYLE == STYLE_RC) ? 4 * (MT / 2) : MT;      // LDS reads of X per k-slice
     static constexpr int B_STAGE = (BSTYLE == STYLE_RC) ? BK * LDB : BN * LDB;

@@ -273,14 +273,19 @@ __device__ __forceinline__ void syrk_store_upper(const SyrkArgs &g, int r, int c
 }
 
 template <int MB, int NB, int MODE, int NW, int R>
-__global__ void __launch_bounds__(NW * 64) ssyrk_direct16_kernel(const SyrkArgs g, int rows_per_tile, int tiles_m) {
+__global__ void __launch_bounds__(NW * 64)
+    ssyrk_direct16_kernel(const float *A_hot, int N_hot, int K_hot, int lda_hot, int rows_per_tile, int tiles_m, const SyrkArgs g) {
+    // What the way to the first loads needs comes as leading scalar parameters, which the dispatcher
+    // preloads into scalar registers before the first wave starts (the build sets
+    // -amdgpu-kernarg-preload-count); the rest of the arguments is read from the argument buffer
+    // while the loop runs.  See sgemm_direct16_kernel.
     extern __shared__ __align__(16) float smem[];
     v4f *red = reinterpret_cast<v4f *>(smem);            // [wave][mb][nb][lane]
     // workgroup id -> (row tile, column tile) over the tiles that touch the upper triangle only,
     // row by row: launching the empty ones too and letting them exit leaves whole XCDs with little
     // work, because the round-robin deal of ids to XCDs then lines up with the row tiles
     int tm = 0, rest = blockIdx.x;
-    const int tiles_n = (g.N + 16 * NB - 1) / (16 * NB);
+    const int tiles_n = (N_hot + 16 * NB - 1) / (16 * NB);
     for (; tm < tiles_m; tm++) {
         const int count = tiles_n - (tm * rows_per_tile) / (16 * NB);
         if (rest < count) break;
@@ -290,17 +295,17 @@ __global__ void __launch_bounds__(NW * 64) ssyrk_direct16_kernel(const SyrkArgs 
     const int m0 = tm * rows_per_tile, n0 = tn * 16 * NB;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
-    const int m_end = min(m0 + rows_per_tile, g.N);
-    const int steps = g.K >> 4;
+    const int m_end = min(m0 + rows_per_tile, N_hot);
+    const int steps = K_hot >> 4;
     const int s0 = (int)((int64_t)steps * wave / NW), s1 = (int)((int64_t)steps * (wave + 1) / NW);
     const int nsteps = s1 - s0;
 
     uint32_t a_off[MB], b_off[NB];
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++) a_off[mb] = 4u * (uint32_t)(min(m0 + 16 * mb + li, g.N - 1) * (int)g.lda + 4 * lq);
+    for (int mb = 0; mb < MB; mb++) a_off[mb] = 4u * (uint32_t)(min(m0 + 16 * mb + li, N_hot - 1) * lda_hot + 4 * lq);
 #pragma unroll
-    for (int nb = 0; nb < NB; nb++) b_off[nb] = 4u * (uint32_t)(min(n0 + 16 * nb + li, g.N - 1) * (int)g.lda + 4 * lq);
-    const char *a_base = reinterpret_cast<const char *>(g.A + 16 * s0);
+    for (int nb = 0; nb < NB; nb++) b_off[nb] = 4u * (uint32_t)(min(n0 + 16 * nb + li, N_hot - 1) * lda_hot + 4 * lq);
+    const char *a_base = reinterpret_cast<const char *>(A_hot + 16 * s0);
     int issued = 0;
 
     v4f ra[R][MB], rb[R][NB];
@@ -436,7 +441,7 @@ static SyrkD16Plan plan_syrk_d16(int N) {
 template <int MB, int NB>
 static int launch_syrk_d16_t(const SyrkArgs &g, const SyrkD16Plan &p, hipStream_t stream) {
     const size_t smem = (size_t)SYRK_D16_WAVES * MB * NB * 64 * sizeof(v4f);
-    void (*kern)(const SyrkArgs, int, int);
+    void (*kern)(const float *, int, int, int, int, int, const SyrkArgs);
     switch (g.mode) {
         case SYRK_FLAT_SYM: kern = ssyrk_direct16_kernel<MB, NB, SYRK_FLAT_SYM, SYRK_D16_WAVES, SYRK_D16_RING>; break;
         case SYRK_FLAT_FULL: kern = ssyrk_direct16_kernel<MB, NB, SYRK_FLAT_FULL, SYRK_D16_WAVES, SYRK_D16_RING>; break;
@@ -444,8 +449,8 @@ static int launch_syrk_d16_t(const SyrkArgs &g, const SyrkD16Plan &p, hipStream_
     }
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3((unsigned)p.needed), dim3(SYRK_D16_WAVES * 64), smem, stream, g, p.rows_per_tile,
-                       p.tiles_m);
+    hipLaunchKernelGGL(kern, dim3((unsigned)p.needed), dim3(SYRK_D16_WAVES * 64), smem, stream, g.A, g.N, g.K, (int)g.lda,
+                       p.rows_per_tile, p.tiles_m, g);
     return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
 }
 

@@ -211,3 +211,28 @@ def test_packed_form_needs_its_design_constant_and_consistent_extents(oracle):
     other = np.zeros_like(V10)
     t2sp_amd.capsule_packed(P2, W2, other, 16)
     assert not np.array_equal(other, V10)
+
+
+@pytest.mark.parametrize("batch", [320, 4096])
+def test_large_batches_on_lds_tiles_sampled_images(oracle, batch):
+    """The reference's published capsule sizes go up to N = 4096 (capsule/README.md:13): rounds of 128 x 128 LDS
+    tiles with the weights' 16 k-rows loaded as 256 contiguous bytes per channel.  Sampled images against the
+    oracle, every image against the same images computed in a batch of their own (other kernel, same bits not
+    required: 1e-5), and a weight tensor with a gap between its channels (the general loader) against the dense one."""
+    import torch
+    N, CI, CO = batch, 32, 32
+    P = t2sp_amd.fill_uniform(torch.empty(N, CI, 15, 15, 4, 4, device="cuda"), 11)
+    W = t2sp_amd.fill_uniform(torch.empty(CO, CI, 3, 3, 4, 4, device="cuda"), 12)
+    V = t2sp_amd.capsule(P, W)
+    assert not torch.isnan(V).any()
+    imgs = [0, 1, N // 2, N - 2, N - 1]
+    # device layout [n][c][h][w][mx][mk] with w = the reference's y: the oracle indexes (n, ci, y, x, mx, mk)
+    ref = oracle.capsule(P[imgs].cpu().numpy().transpose(0, 1, 3, 2, 4, 5), W.cpu().numpy().transpose(0, 1, 3, 2, 4, 5))
+    assert rel_fro(V[imgs].cpu().numpy().transpose(0, 1, 3, 2, 4, 5), ref)[0] <= TOL
+    small = t2sp_amd.capsule(P[:48].contiguous(), W)
+    assert rel_fro(V[:48].cpu().numpy(), small.cpu().numpy())[0] <= TOL
+    if batch == 320:
+        Wg = torch.zeros(CO, CI, 3, 4, 4, 4, device="cuda")[:, :, :, :3]      # a gap after every kernel row
+        Wg.copy_(W)
+        assert not Wg.is_contiguous()
+        assert torch.equal(t2sp_amd.capsule(P, Wg), V) or rel_fro(t2sp_amd.capsule(P, Wg).cpu().numpy(), V.cpu().numpy())[0] <= 1e-6

@@ -308,7 +308,9 @@ def test_direct16_kernel_small_products(oracle, torch_cuda, shape):
                             None) == -8
 
 
-@pytest.mark.parametrize("shape", [(256, 256, 16384), (128, 128, 4096), (100, 132, 4096), (64, 64, 32768), (40, 520, 2048)])
+@pytest.mark.parametrize("shape", [(256, 256, 16384), (128, 128, 4096), (100, 132, 4096), (64, 64, 32768), (40, 520, 2048),
+                                   # 64-column tiles with 8 and 16 shares of k dealt to the dies, ragged against them
+                                   (512, 256, 16384), (250, 260, 16384), (512, 256, 65536), (96, 160, 32768)])
 def test_tiny_outputs_split_their_reduction_over_workgroups(oracle, torch_cuda, shape):
     """Outputs of a few tiles with a long reduction: given the workspace the library asks for, every tile
     goes to several workgroups that reduce a share of k each, and a second kernel adds their planes; the
@@ -378,3 +380,20 @@ def test_config2_full_size_sampled_rows_and_identity(oracle, torch_cuda, shape):
     if K == N:
         eye = torch.eye(K, device="cuda")
         assert torch.equal(t2sp_amd.gemm(A, eye), A)
+
+
+def test_thin_and_very_wide_product(torch_cuda):
+    """64 x 2^22 x 64: more column tiles of the one-launch form than a grid's second dimension holds, so the
+    library's own choice must fall through to a kernel that can take the shape.  Integer data: exact."""
+    torch = torch_cuda
+    M, N, K = 64, 1 << 22, 64
+    L = t2sp_amd.lib()
+    g = torch.Generator().manual_seed(7)
+    A = torch.randint(-2, 3, (M, K), generator=g).float().cuda()
+    B = torch.randint(-2, 3, (K, N), generator=g, dtype=torch.int8).cuda().float()
+    C = torch.full((M, N), float("nan"), device="cuda")
+    assert L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, None, 0, None) == 0
+    torch.cuda.synchronize()
+    cols = torch.cat([torch.arange(0, 4096), torch.arange(N - 4096, N), torch.randint(0, N, (4096,), generator=g)]).cuda()
+    assert torch.equal(C[:, cols].double(), A.double() @ B[:, cols].double())
+    assert not torch.isnan(C).any()
