@@ -20,7 +20,7 @@ def test_constant_fixture_exact():
     assert V.shape == (2, 8, 7, 7, 4, 4) and (V == 1152).all()
 
 
-@pytest.mark.parametrize("cfg,splits", [(0, 0), (5, 0), (6, 0), (2, 1), (2, 3), (3, 2), (4, 2), (1, 2), (99, 0)])
+@pytest.mark.parametrize("cfg,splits", [(0, 0), (5, 0), (6, 0), (2, 1), (2, 3), (3, 2), (4, 2), (1, 2), (7, 1), (7, 2), (99, 0)])
 def test_tiny_constants_parity_golden_and_ure_order(oracle, cfg, splits):
     """The TINY sizes of capsule/const-parameters.h:43-52 with N=4 (capsule-run-fpga.cpp:37-39):
     16 -> 16 channels, 15x15 -> 7x7, against both reduction orders the reference uses."""
@@ -70,7 +70,7 @@ def test_short_and_odd_reductions_ragged_columns(oracle, ci, co, n, cfg):
 
 
 @pytest.mark.parametrize("ci", [1, 2, 3, 5, 9, 17])
-@pytest.mark.parametrize("cfg,splits", [(2, 1), (3, 1), (4, 1), (2, 2), (1, 1)])
+@pytest.mark.parametrize("cfg,splits", [(2, 1), (3, 1), (4, 1), (2, 2), (1, 1), (7, 1)])
 def test_lds_tile_kernels_reduction_tails_exact(ci, cfg, splits):
     """The LDS-tiled kernels with reductions of CI * 36 = 36 .. 612 rows, none a whole number of pairs of
     16-row tiles (guarded fetches only for the last tiles; with a split, per slice).  Integer data: exact

@@ -14,7 +14,7 @@ from conftest import rel_fro
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-5
-CFGS = [0, 1, 2, 3]
+CFGS = [0, 1, 2, 3, 7]      # T2SP_CFG_AUTO, _256x256, _128x128, _64x128, _256x128
 
 
 @pytest.fixture(scope="module")
