@@ -37,6 +37,10 @@ extern "C" {
 #define T2SP_CFG_SCALAR 99
 
 #define T2SP_MAX_DIMS 10
+/* Largest extent of any one dimension (rows, columns, reduction length, pixels, ...) the thin layer
+ * and its planners take: the tile arithmetic rounds extents up in 32 bits.  Larger values get
+ * T2SP_ERR_SHAPE (or 0 from the *_workspace_bytes and *_plan calls). */
+#define T2SP_MAX_EXTENT (1 << 30)
 
 /* C[i,j] = sum_k A[i,k] * B[k,j], fp32, row-major with leading dimensions in
  * elements, which must not be negative here and in the BLAS, SYRK and MTTKRP forms below

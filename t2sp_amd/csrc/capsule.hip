@@ -675,15 +675,20 @@ static Direct16Plan plan_direct16_for(int rows, int cols, int nb, int max_mb) {
     p.nb = nb;
     p.tiles_n = (cols + 16 * nb - 1) / (16 * nb);
     const int cus = machine().cus;
-    for (int rounds = 1;; rounds++) {
-        const int want_m = (rounds * cus) / p.tiles_n > 0 ? (rounds * cus) / p.tiles_n : 1;
-        int rpt = ((rows + want_m - 1) / want_m + 3) / 4 * 4;
+    // (the first candidate is the least number of rounds whose tiles could be short enough; 64-bit: the
+    // product of rounds and CUs has no bound a 32-bit integer would hold for the tallest matrices)
+    const int64_t least_m = (rows + 16 * max_mb - 1) / (16 * max_mb);
+    int64_t rounds = (least_m * p.tiles_n + cus - 1) / cus - 1;
+    if (rounds < 1) rounds = 1;
+    for (;; rounds++) {
+        const int64_t want_m = (rounds * cus) / p.tiles_n > 0 ? (rounds * cus) / p.tiles_n : 1;
+        int rpt = (int)(((rows + want_m - 1) / want_m + 3) / 4 * 4);
         if (rpt < 64) rpt = 64;
         if (rpt <= 16 * max_mb) {
             p.rows_per_tile = rpt;
             p.mb = (rpt + 15) / 16;
             p.tiles_m = (rows + rpt - 1) / rpt;
-            p.rounds = rounds;
+            p.rounds = (int)(rounds < INT32_MAX ? rounds : INT32_MAX);
             return p;
         }
     }
@@ -695,7 +700,7 @@ static Direct16Plan plan_direct16_for(int rows, int cols, int nb, int max_mb) {
 static Direct16Plan plan_direct16(int rows, int cols) {
     const Direct16Plan wide = plan_direct16_for(rows, cols, 2, D16_MAX_MB);
     const Direct16Plan tall = plan_direct16_for(rows, cols, 1, D16_MAX_MB_TALL);
-    return tall.rounds * tall.mb < wide.rounds * wide.mb * 2 ? tall : wide;
+    return (int64_t)tall.rounds * tall.mb < (int64_t)wide.rounds * wide.mb * 2 ? tall : wide;
 }
 static int direct16_tab_entries(int kred) {
     const int steps = (kred / 4 + 3) / 4;
@@ -817,7 +822,7 @@ static bool capsule_fast(const int *d, const int64_t *sp6, const int64_t *sw6, c
 // tile, row blocks, column blocks, tiles along rows and columns, rounds of workgroups.  For tests
 // of the planner.
 extern "C" int t2sp_capsule_direct16_plan(int rows, int cols, int *out6) {
-    if (rows <= 0 || cols <= 0 || !out6) return 0;
+    if (rows <= 0 || cols <= 0 || !out6 || rows > T2SP_MAX_EXTENT || cols > T2SP_MAX_EXTENT) return 0;
     const t2sp::Direct16Plan p = t2sp::plan_direct16(rows, cols);
     out6[0] = p.rows_per_tile; out6[1] = p.mb; out6[2] = p.nb; out6[3] = p.tiles_m; out6[4] = p.tiles_n; out6[5] = p.rounds;
     return 1;
@@ -827,7 +832,9 @@ extern "C" size_t t2sp_capsule_workspace_bytes(const int *dims11, int cfg, int s
     const int *d = dims11;
     if (!d) return 0;
     const int64_t rows = (int64_t)d[0] * d[3] * d[4] * d[8], cols = (int64_t)d[2] * 4, kred = (int64_t)d[1] * d[5] * d[6] * 4;
-    if (rows <= 0 || rows > INT32_MAX || cols > INT32_MAX || kred > INT32_MAX) return 0;
+    for (int i = 0; i < 11; i++)
+        if (d[i] <= 0) return 0;
+    if (rows <= 0 || rows > T2SP_MAX_EXTENT || cols > T2SP_MAX_EXTENT || kred > T2SP_MAX_EXTENT) return 0;
     return t2sp::plan_capsule((int)rows, (int)cols, (int)kred, cfg, splits, dims11[8]).scratch_bytes;
 }
 
@@ -841,7 +848,7 @@ extern "C" int t2sp_capsule_f32(const float *P, const float *W, float *V, const 
         if (d[i] <= 0) return T2SP_ERR_SHAPE;
     const int64_t rows = (int64_t)d[0] * d[3] * d[4] * d[8], cols = (int64_t)d[2] * 4,
                   kred = (int64_t)d[1] * d[5] * d[6] * 4;
-    if (rows > INT32_MAX / 2 || cols > INT32_MAX / 2 || kred > INT32_MAX / 2) return T2SP_ERR_SHAPE;
+    if (rows > T2SP_MAX_EXTENT || cols > T2SP_MAX_EXTENT || kred > T2SP_MAX_EXTENT) return T2SP_ERR_SHAPE;
     bool byte_offsets_fit = false;
     if (cfg == T2SP_CFG_SCALAR || !capsule_fast(d, sp6, sw6, sv6, P, W, V, &byte_offsets_fit)) {
         CapsuleGenericArgs a{P, W, V, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], d[8], d[9], d[10], {}, {}, {}};

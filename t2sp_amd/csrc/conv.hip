@@ -626,7 +626,7 @@ static size_t conv_padded_weight_bytes(int CO, int kred) {
 // pixels as (tile configuration, first pixel, end pixel, splits of the reduction) quadruples; P is
 // the number of output pixels N*OH*round_up4(OW).  For tests of the planner.
 extern "C" int t2sp_conv2d_plan(int CO, int P, int KRED, int *stages16) {
-    if (CO <= 0 || P <= 0 || KRED <= 0 || !stages16) return 0;
+    if (CO <= 0 || P <= 0 || KRED <= 0 || !stages16 || CO > T2SP_MAX_EXTENT || P > T2SP_MAX_EXTENT || KRED > T2SP_MAX_EXTENT) return 0;
     const t2sp::ConvPlan p = t2sp::plan_conv(CO, P, KRED);
     for (int i = 0; i < p.n; i++) {
         stages16[4 * i] = p.st[i].cfg; stages16[4 * i + 1] = p.st[i].p_begin;
@@ -636,7 +636,7 @@ extern "C" int t2sp_conv2d_plan(int CO, int P, int KRED, int *stages16) {
 }
 
 extern "C" int t2sp_conv2d_direct16_plan(int CO, int P, int KRED, int *out4, double *times2) {
-    if (CO <= 0 || P <= 0 || KRED <= 0 || !out4 || !times2) return 0;
+    if (CO <= 0 || P <= 0 || KRED <= 0 || !out4 || !times2 || CO > T2SP_MAX_EXTENT || P > T2SP_MAX_EXTENT || KRED > T2SP_MAX_EXTENT) return 0;
     const t2sp::ConvD16Plan d = t2sp::plan_conv_d16(CO, P, KRED);
     const t2sp::ConvPlan l = t2sp::plan_conv(CO, P, KRED);
     out4[0] = d.mb; out4[1] = d.rows_per_tile; out4[2] = d.tiles_m; out4[3] = d.tiles_n;
@@ -646,10 +646,10 @@ extern "C" int t2sp_conv2d_direct16_plan(int CO, int P, int KRED, int *out4, dou
 
 extern "C" size_t t2sp_conv2d_workspace_bytes(int N, int CI, int CO, int OH, int OW, int KH, int KW) {
     if (N <= 0 || CI <= 0 || CO <= 0 || OH <= 0 || OW <= 0 || KH <= 0 || KW <= 0) return 0;
-    if ((int64_t)N * OH * OW > INT32_MAX || (int64_t)CI * KH * KW > INT32_MAX) return 0;
+    if (CO > T2SP_MAX_EXTENT || (int64_t)N * OH * OW > T2SP_MAX_EXTENT || (int64_t)CI * KH * KW > T2SP_MAX_EXTENT) return 0;
     // padded weight rows when their length is not a multiple of 4, then the planes of a split rest
     const int64_t owp = (OW + 3) / 4 * 4;
-    if ((int64_t)N * OH * owp > INT32_MAX) return 0;
+    if ((int64_t)N * OH * owp > T2SP_MAX_EXTENT) return 0;
     return t2sp::conv_padded_weight_bytes(CO, CI * KH * KW) +
            t2sp::plan_conv(CO, (int)(N * OH * owp), CI * KH * KW).scratch_bytes;
 }
@@ -661,7 +661,8 @@ extern "C" int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, 
     using namespace t2sp;
     if (N <= 0 || CI <= 0 || CO <= 0 || OH <= 0 || OW <= 0 || KH <= 0 || KW <= 0 || !si4 || !sw4 || !so4)
         return T2SP_ERR_SHAPE;
-    if ((int64_t)N * OH * OW > INT32_MAX || (int64_t)CI * KH * KW > INT32_MAX) return T2SP_ERR_SHAPE;
+    if (CO > T2SP_MAX_EXTENT || OW > T2SP_MAX_EXTENT || (int64_t)N * OH * OW > T2SP_MAX_EXTENT || (int64_t)CI * KH * KW > T2SP_MAX_EXTENT)
+        return T2SP_ERR_SHAPE;
     const int64_t in_span = (int64_t)(N - 1) * si4[0] + (int64_t)(CI - 1) * si4[1] +
                             (int64_t)(OH + KH - 2) * si4[2] + (OW + KW - 2);
     hipStream_t st = (hipStream_t)stream;
@@ -690,7 +691,7 @@ extern "C" int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, 
     const bool out_ok = so4[3] == 1 && (ragged ? ((uintptr_t)O % 4 == 0)
                                                 : (so4[0] % 4 == 0 && so4[1] % 4 == 0 && so4[2] % 4 == 0 && (uintptr_t)O % 16 == 0));
     const bool fast = cfg != T2SP_CFG_SCALAR && si4[3] == 1 && out_ok && w_dense && sw_o % 4 == 0 && sw_o < t2sp::LOADER_MAX_LD && si4[0] >= 0 && si4[1] >= 0 && si4[2] >= 0 && OW >= 4 &&
-                      (int64_t)N * OH * owp <= INT32_MAX && (kred % 4 == 0 || padded) && KH * KW <= 4096 &&
+                      (int64_t)N * OH * owp <= T2SP_MAX_EXTENT && (kred % 4 == 0 || padded) && KH * KW <= 4096 &&
                       in_span < INT32_MAX && ((uintptr_t)W % 16 == 0) && ((uintptr_t)I % 4 == 0);
     if (!fast) {
         ConvGenericArgs a{I, W_given, O, N, CI, CO, OH, OW, KH, KW, {}, {}, {}};

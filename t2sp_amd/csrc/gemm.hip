@@ -1349,8 +1349,12 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
 // The launch plan of the LDS-tiled kernels for an M x N x K product on the current machine(): tile
 // edge (256 or 128; 0 when the product would not take whole rounds of these tiles) and the launches
 // as (first tile, tiles, splits of the reduction) triples.  For tests of the planner.
+static inline bool gemm_extents_ok(int M, int N, int K) {
+    return M > 0 && N > 0 && K > 0 && M <= T2SP_MAX_EXTENT && N <= T2SP_MAX_EXTENT && K <= T2SP_MAX_EXTENT;
+}
+
 extern "C" int t2sp_sgemm_plan(int M, int N, int K, int *tile_edge, int *phases12) {
-    if (M <= 0 || N <= 0 || K <= 0 || !tile_edge || !phases12) return 0;
+    if (!gemm_extents_ok(M, N, K) || !tile_edge || !phases12) return 0;
     const t2sp::GemmPlan p = t2sp::plan_gemm(M, N, K);
     *tile_edge = 0;
     if (!p.phased) return 0;
@@ -1369,7 +1373,7 @@ extern "C" int t2sp_sgemm_plan(int M, int N, int K, int *tile_edge, int *phases1
 extern "C" int t2sp_sgemm_tail_from(int k_len) { return t2sp::tail_from_for<t2sp::GemmL>(k_len); }
 
 extern "C" size_t t2sp_sgemm_workspace_bytes(int M, int N, int K) {
-    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    if (!gemm_extents_ok(M, N, K)) return 0;
     if (K % 4 == 0 && N % 4 == 0) {
         const size_t tiled = t2sp::plan_gemm(M, N, K).scratch_bytes;
         const size_t one_launch = t2sp::plan_gemm_d16_split(M, N, K, t2sp::plan_gemm_d16(M, N)).scratch_bytes;
@@ -1384,6 +1388,7 @@ extern "C" int t2sp_sgemm_f32(const float *A, const float *B, float *C, int M, i
                               int64_t lda, int64_t ldb, int64_t ldc, int cfg, float *workspace,
                               size_t workspace_bytes, void *stream) {
     if (lda < 0 || ldb < 0 || ldc < 0) return T2SP_ERR_SHAPE;   // the loaders' offsets are unsigned
+    if (M > T2SP_MAX_EXTENT || N > T2SP_MAX_EXTENT || K > T2SP_MAX_EXTENT) return T2SP_ERR_SHAPE;
     t2sp::GemmArgs g{};
     g.A = A; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K;
     g.lda = lda; g.ldb = ldb; g.ldc = ldc;
@@ -1396,6 +1401,7 @@ extern "C" int t2sp_sgemm_f32_tiled(const float *A, const float *B, float *C, in
                                     const int64_t *strides6, int cfg, float *workspace,
                                     size_t workspace_bytes, void *stream) {
     if (jjj <= 0 || iii <= 0 || jj <= 0 || ii <= 0 || !strides6 || lda < 0 || ldb < 0) return T2SP_ERR_SHAPE;
+    if (M > T2SP_MAX_EXTENT || N > T2SP_MAX_EXTENT || K > T2SP_MAX_EXTENT) return T2SP_ERR_SHAPE;
     t2sp::GemmArgs g{};
     g.A = A; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K;
     g.lda = lda; g.ldb = ldb; g.ldc = 0;
@@ -1405,7 +1411,7 @@ extern "C" int t2sp_sgemm_f32_tiled(const float *A, const float *B, float *C, in
 }
 
 extern "C" size_t t2sp_sgemm_ex_workspace_bytes(int transa, int M, int N, int K) {
-    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    if (!gemm_extents_ok(M, N, K)) return 0;
     // the re-laid A of the transposed form (required), then the planes of a split reduction (optional)
     const size_t pad_t = t2sp::gemm_pad_bytes(M, N, K, true), pad_n = t2sp::gemm_pad_bytes(M, N, K, false);
     const bool padded = K % 4 || N % 4;
@@ -1420,7 +1426,7 @@ extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, fl
                                  int64_t lda, const float *B, int64_t ldb, float beta, const float *Cin,
                                  int64_t ldcin, float *C, int64_t ldc, int cfg, float *workspace,
                                  size_t workspace_bytes, void *stream) {
-    if (M <= 0 || N <= 0 || K <= 0 || lda < 0 || ldb < 0 || ldc < 0 || (Cin && ldcin < 0)) return T2SP_ERR_SHAPE;
+    if (!gemm_extents_ok(M, N, K) || lda < 0 || ldb < 0 || ldc < 0 || (Cin && ldcin < 0)) return T2SP_ERR_SHAPE;
     const float *a = A;
     int64_t la = lda;
     auto aligned16 = [](const void *p) { return ((uintptr_t)p & 15) == 0; };

@@ -286,11 +286,11 @@ static MttkrpPlan plan_mttkrp(int I, int J, int K, int R, int cfg, int splits) {
     int bm = 64, bn = 64;
     for (const Cand &c : cands)
         if (c.cfg == cfg) { bm = c.bm; bn = c.bn; }
-    const int tiles = ((I + bm - 1) / bm) * ((R + bn - 1) / bn);
+    const int64_t tiles = (int64_t)((I + bm - 1) / bm) * ((R + bn - 1) / bn);
     const int64_t ktiles = (int64_t)K * (J / 16);
     if (splits <= 0) {
         const int cus = machine().cus;
-        splits = tiles >= cus * 25 / 32 ? 1 : (cus + tiles / 2) / tiles;
+        splits = tiles >= cus * 25 / 32 ? 1 : (int)((cus + tiles / 2) / tiles);
         if (splits > ktiles / 16) splits = (int)(ktiles / 16);
         if (splits < 1) splits = 1;
     }
@@ -366,6 +366,7 @@ static size_t mttkrp_pad_bytes(int I, int J, int K, int R) {
 
 extern "C" size_t t2sp_mttkrp_workspace_bytes(int I, int J, int K, int R, int cfg, int splits) {
     if (I <= 0 || J <= 0 || K <= 0 || R <= 0) return 0;
+    if (I > T2SP_MAX_EXTENT || R > T2SP_MAX_EXTENT || J > T2SP_MAX_EXTENT || (int64_t)K * ((J + 15) / 16 * 16) > T2SP_MAX_EXTENT) return 0;
     if (J % 16 == 0 && I % 4 == 0) return t2sp::plan_mttkrp(I, J, K, R, cfg, splits).scratch_bytes;
     // padded copies of B and C and a temporary result, then the planes of the padded product
     return t2sp::mttkrp_pad_bytes(I, J, K, R) +
@@ -378,7 +379,7 @@ extern "C" int t2sp_mttkrp_f32(const float *B, const float *C, const float *D, f
                                float *workspace, size_t workspace_bytes, void *stream) {
     using namespace t2sp;
     if (I <= 0 || J <= 0 || K <= 0 || R <= 0 || !sb3 || !sc2 || !sd2 || !sa2) return T2SP_ERR_SHAPE;
-    if ((int64_t)K * J > INT32_MAX) return T2SP_ERR_SHAPE;
+    if (I > T2SP_MAX_EXTENT || R > T2SP_MAX_EXTENT || J > T2SP_MAX_EXTENT || (int64_t)K * J > T2SP_MAX_EXTENT) return T2SP_ERR_SHAPE;
     const bool fast = mttkrp_fast(I, J, sb3, sc2, sd2, sa2, B, C, A);
     if (cfg == T2SP_CFG_AUTO && !fast && sb3[1] == 1 && sc2[0] == 1 && sa2[0] == 1 && workspace &&
         ((uintptr_t)workspace % 16 == 0) && workspace_bytes >= mttkrp_pad_bytes(I, J, K, R) &&

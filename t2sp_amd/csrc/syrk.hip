@@ -650,14 +650,14 @@ __global__ void __launch_bounds__(256) syrk_fold_kernel(const float *flat, float
 // How SYRK with tiles of edge b splits its last, partial round on the current machine(): tiles of
 // the triangle, tiles of the tail that is split, splits per tail tile.  For tests of the planner.
 extern "C" int t2sp_ssyrk_plan(int N, int K, int b, int *total_tail_splits) {
-    if (N <= 0 || K <= 0 || b <= 0 || !total_tail_splits) return 0;
+    if (N <= 0 || K <= 0 || b <= 0 || !total_tail_splits || N > T2SP_MAX_EXTENT || K > T2SP_MAX_EXTENT || b > 256) return 0;
     const t2sp::SyrkTail t = t2sp::plan_syrk_tail(N, K, b, 16);
     total_tail_splits[0] = (int)t.total; total_tail_splits[1] = (int)t.tail; total_tail_splits[2] = t.splits;
     return 1;
 }
 
 extern "C" size_t t2sp_ssyrk_workspace_bytes(int trans, int N, int K) {
-    if (N <= 0 || K <= 0) return 0;
+    if (N <= 0 || K <= 0 || N > T2SP_MAX_EXTENT || K > T2SP_MAX_EXTENT) return 0;
     // the re-laid A of the transposed form (required), then room for the planes of a split last
     // round with any of the tile sizes (optional: without it the last round runs unsplit)
     size_t planes = 0;
@@ -670,7 +670,7 @@ extern "C" size_t t2sp_ssyrk_workspace_bytes(int trans, int N, int K) {
 }
 
 extern "C" size_t t2sp_ssyrk_folded_workspace_bytes(int trans, int N, int K) {
-    if (N <= 0 || K <= 0) return 0;
+    if (N <= 0 || K <= 0 || N > T2SP_MAX_EXTENT || K > T2SP_MAX_EXTENT) return 0;
     return (size_t)N * N * sizeof(float) + t2sp_ssyrk_workspace_bytes(trans, N, K);
 }
 
@@ -678,6 +678,7 @@ extern "C" int t2sp_ssyrk_f32(int upper, int trans, int N, int K, float alpha, c
                               float beta, const float *Cin, int64_t ldcin, float *C, int64_t ldc, int mirror,
                               int cfg, float *workspace, size_t workspace_bytes, void *stream) {
     if (lda < 0 || ldc < 0 || (Cin && ldcin < 0)) return T2SP_ERR_SHAPE;   // the loaders' offsets are unsigned
+    if (N > T2SP_MAX_EXTENT || K > T2SP_MAX_EXTENT) return T2SP_ERR_SHAPE;
     t2sp::SyrkArgs g{};
     g.A = A; g.lda = lda; g.N = N; g.K = K; g.alpha = alpha; g.beta = beta;
     g.Cin = beta != 0.f ? Cin : nullptr; g.ldcin = ldcin;
@@ -691,6 +692,7 @@ extern "C" int t2sp_ssyrk_f32_folded(int trans, int N, int K, float alpha, const
                                      const int64_t *strides6, int cfg, float *workspace, size_t workspace_bytes,
                                      void *stream) {
     if (iii <= 0 || ii <= 0 || !strides6 || N <= 0 || lda < 0 || (Cin && ldcin < 0)) return T2SP_ERR_SHAPE;
+    if (N > T2SP_MAX_EXTENT || K > T2SP_MAX_EXTENT || iii > T2SP_MAX_EXTENT || ii > T2SP_MAX_EXTENT || (int64_t)iii * ii > T2SP_MAX_EXTENT) return T2SP_ERR_SHAPE;
     const int B = iii * ii;
     if (N % B || (N / B) % 2) return T2SP_ERR_SHAPE;   // an even number of whole blocks (syrk.cpp:80-82: i < I/2)
     t2sp::SyrkArgs g{};

@@ -166,3 +166,52 @@ def test_unguarded_loop_bodies_only_fetch_whole_k_tiles():
         tiles = -(-k_len // 16)
         if k_len >= 64:
             assert t >= tiles - 5
+
+
+def test_planners_take_extreme_extents(lib):
+    """Every planner and workspace query with extents from 1 up to 2^31 - 1, in random combinations: each must
+    return (0 / no plan beyond T2SP_MAX_EXTENT = 2^30 per dimension) without overflowing its 32-bit tile arithmetic
+    or looping for long.  `make -C t2sp_amd/csrc asan-check` runs this under UndefinedBehaviorSanitizer, which is
+    what turns an overflow into a failure; it found four, all fixed."""
+    import random
+    import time
+    L = lib
+    L.t2sp_set_machine(256, 8)
+    i32, sz = ctypes.c_int, ctypes.c_size_t
+    for f in (L.t2sp_sgemm_workspace_bytes, L.t2sp_sgemm_ex_workspace_bytes, L.t2sp_conv2d_workspace_bytes,
+              L.t2sp_ssyrk_workspace_bytes, L.t2sp_mttkrp_workspace_bytes, L.t2sp_capsule_workspace_bytes):
+        f.restype = sz
+    L.t2sp_sgemm_workspace_bytes.argtypes = [i32] * 3
+    L.t2sp_sgemm_ex_workspace_bytes.argtypes = [i32] * 4
+    L.t2sp_conv2d_workspace_bytes.argtypes = [i32] * 7
+    L.t2sp_ssyrk_workspace_bytes.argtypes = [i32] * 3
+    L.t2sp_mttkrp_workspace_bytes.argtypes = [i32] * 6
+    L.t2sp_conv2d_direct16_plan.argtypes = [i32] * 3 + [ctypes.POINTER(i32), ctypes.POINTER(ctypes.c_double)]
+    rng = random.Random(1)
+    edge = [1, 2, 3, 4, 15, 16, 17, 63, 64, 65, 127, 128, 255, 256, 257, 1023, 4096, 65535, 65536, 1 << 20,
+            (1 << 22) - 1, 1 << 22, 1 << 30, (1 << 30) + 1, (1 << 31) - 1]
+
+    def pick():
+        return rng.choice(edge) if rng.random() < 0.7 else rng.randint(1, 1 << 20)
+
+    t0 = time.time()
+    for _ in range(3000):
+        M, N, K = pick(), pick(), pick()
+        te, ph = i32(), (i32 * 12)()
+        n = L.t2sp_sgemm_plan(M, N, K, ctypes.byref(te), ph)
+        assert 0 <= n <= 4 and (max(M, N, K) <= 1 << 30 or n == 0)
+        if max(M, N, K) > 1 << 30:
+            assert L.t2sp_sgemm_workspace_bytes(M, N, K) == 0
+        else:
+            L.t2sp_sgemm_workspace_bytes(M, N, K)
+        L.t2sp_sgemm_ex_workspace_bytes(rng.randint(0, 1), M, N, K)
+        assert 0 <= L.t2sp_conv2d_plan(pick(), pick(), pick(), (i32 * 16)()) <= 4
+        L.t2sp_conv2d_direct16_plan(pick(), pick(), pick(), (i32 * 4)(), (ctypes.c_double * 2)())
+        L.t2sp_ssyrk_plan(pick(), pick(), rng.choice([64, 128, 256]), (i32 * 3)())
+        L.t2sp_ssyrk_workspace_bytes(rng.randint(0, 1), pick(), pick())
+        L.t2sp_capsule_direct16_plan(pick(), pick(), (i32 * 6)())
+        L.t2sp_mttkrp_workspace_bytes(pick(), pick(), pick(), pick(), 0, 0)
+        L.t2sp_capsule_workspace_bytes((i32 * 11)(pick() % 70000 + 1, pick() % 4096 + 1, pick() % 4096 + 1, 7, 7, 3, 3, 2, 4, 4, 4), 0, 0)
+        L.t2sp_conv2d_workspace_bytes(pick() % 4096 + 1, pick() % 4096 + 1, pick() % 4096 + 1, pick() % 4096 + 1,
+                                      pick() % 4096 + 1, 3, 3)
+    assert time.time() - t0 < 60
