@@ -66,8 +66,16 @@ int check_buffer_typed(const halide_buffer_t *b, const char *op, const char *nam
             snprintf(msg, sizeof msg, "%s dimension %d has negative stride", name, d);
             return report(halide_error_code_constraint_violated, op, msg);
         }
+        // (a buffer of more than 2^40 elements, or one that spans more, is refused before the products
+        // below could leave 64 bits: Halide's own limit is 2^31 - 1 bytes, halide_error_code_buffer_extents_too_large)
+        constexpr int64_t LIMIT = (int64_t)1 << 40;
+        const int64_t reach = (int64_t)(b->dim[d].extent > 0 ? b->dim[d].extent - 1 : 0) * b->dim[d].stride;
+        if ((b->dim[d].extent > 0 && elements > LIMIT / b->dim[d].extent) || reach > LIMIT || spn + reach > LIMIT) {
+            snprintf(msg, sizeof msg, "%s is larger than 2^40 elements at dimension %d", name, d);
+            return report(halide_error_code_buffer_extents_too_large, op, msg);
+        }
         elements *= b->dim[d].extent;
-        spn += (int64_t)(b->dim[d].extent > 0 ? b->dim[d].extent - 1 : 0) * b->dim[d].stride;
+        spn += reach;
     }
     if (b->dimensions > 0 && b->dim[0].stride != 1) {
         snprintf(msg, sizeof msg, "%s.stride.0 is %d, must be 1", name, b->dim[0].stride);

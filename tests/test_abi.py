@@ -406,3 +406,75 @@ def test_design_constants_belong_to_the_calling_thread():
     finally:
         L.t2sp_capsule_design(0)
         L.t2sp_conv_design(0)
+
+
+def test_entries_survive_random_buffers():
+    """Every operator entry with randomly shaped halide_buffer_t arguments (ranks 0 to 11, extents from -1 to
+    2^31 - 1, strides from -1 to 2^31 - 1, NULL buffers and hosts, both dirty flags): each call must come back
+    with 0 or a negative halide_error_code_t from the argument checks, which read nothing beyond `dimensions`
+    entries of `dim` and overflow no product.  `make -C t2sp_amd/csrc asan-check` runs this under
+    AddressSanitizer and UndefinedBehaviorSanitizer; it found the element count of a buffer leaving 64 bits."""
+    import random
+    from t2sp_amd.buffer import halide_dimension_t
+    L = t2sp_amd.lib()
+    rng = random.Random(7)
+    store = np.zeros(1 << 12, np.float32)
+    keep = []
+
+    def R(want=None, u8=False):
+        nd = want if (want is not None and rng.random() < 0.9) else rng.choice([0, 1, 2, 3, 4, 6, 10, 11])
+        dims = (halide_dimension_t * max(nd, 1))()
+        for d in range(nd):
+            dims[d].min = rng.choice([0, 0, 0, 1, -3])
+            dims[d].extent = rng.choice([0, 1, 2, 3, 4, 4, 7, 8, 16, 64, 225, 1024, -1, 1 << 20, (1 << 31) - 1])
+            dims[d].stride = 1 if (d == 0 and rng.random() < 0.9) else rng.choice([0, 1, 2, 4, 16, 64, 1024, -1, 1 << 20, (1 << 31) - 1])
+        b = halide_buffer_t()
+        b.host = store.ctypes.data if rng.random() < 0.8 else None
+        b.flags = rng.choice([0, 0, 1, 2, 3])
+        b.type.code, b.type.bits, b.type.lanes = (1, 8, 1) if u8 else (2, 32, 1)
+        if rng.random() < 0.03:
+            b.type.bits = 64
+        b.dimensions = nd
+        b.dim = dims
+        keep.append((b, dims))
+        return ctypes.byref(b) if rng.random() < 0.95 else None
+
+    vp, f32 = ctypes.c_void_p, ctypes.c_float
+    seen = set()
+    for _ in range(4000):
+        del keep[:]
+        fn = rng.choice(["gemm", "GEMM", "conv", "capsule", "mttkrp", "syrk", "ger", "gbmv3", "symv", "pairhmm", "qrd"])
+        f = getattr(L, fn)
+        f.restype = ctypes.c_int
+        if fn in ("gemm", "GEMM"):
+            f.argtypes = [vp] * 3
+            rc = f(R(2), R(2), R(rng.choice([2, 6])))
+        elif fn == "conv":
+            k = rng.choice([2, 4])
+            f.argtypes = [vp] * 3
+            rc = f(R(k), R(k), R(rng.choice([2, 4, 10])))
+        elif fn == "capsule":
+            k = rng.choice([2, 6])
+            f.argtypes = [vp] * 3
+            rc = f(R(k), R(k), R(rng.choice([2, 6, 10])))
+        elif fn == "qrd":
+            f.argtypes = [vp] * 3
+            rc = f(R(3), R(3), R(3))
+        elif fn == "mttkrp":
+            f.argtypes = [vp] * 4
+            rc = f(R(3), R(2), R(2), R(2))
+        elif fn == "ger":
+            f.argtypes = [vp] * 4
+            rc = f(R(2), R(1), R(1), R(rng.choice([2, 6])))
+        elif fn == "syrk":
+            f.argtypes = [ctypes.c_int, f32, f32] + [vp] * 3
+            rc = f(rng.randint(0, 1), 1.5, 0.5, R(2), R(2), R(rng.choice([2, 6])))
+        elif fn in ("gbmv3", "symv"):
+            f.argtypes = [f32, f32] + [vp] * 4
+            rc = f(1.5, 0.5, R(2), R(1), R(1), R(rng.choice([1, 3])))
+        else:
+            f.argtypes = [vp] * 10
+            rc = f(R(2, True), R(2, True), *[R(2) for _ in range(7)], R(rng.choice([2, 4])))
+        assert rc <= 0, (fn, rc)
+        seen.add(rc)
+    assert {-43, -28, -12, -8, -6}.issubset(seen)
