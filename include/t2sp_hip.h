@@ -41,6 +41,8 @@ extern "C" {
  * and its planners take: the tile arithmetic rounds extents up in 32 bits.  Larger values get
  * T2SP_ERR_SHAPE (or 0 from the *_workspace_bytes and *_plan calls). */
 #define T2SP_MAX_EXTENT (1 << 30)
+/* Largest magnitude of any stride or leading dimension, in elements; beyond it T2SP_ERR_SHAPE. */
+#define T2SP_MAX_STRIDE ((int64_t)1 << 31)
 
 /* C[i,j] = sum_k A[i,k] * B[k,j], fp32, row-major with leading dimensions in
  * elements, which must not be negative here and in the BLAS, SYRK and MTTKRP forms below

@@ -849,6 +849,12 @@ extern "C" int t2sp_capsule_f32(const float *P, const float *W, float *V, const 
     const int64_t rows = (int64_t)d[0] * d[3] * d[4] * d[8], cols = (int64_t)d[2] * 4,
                   kred = (int64_t)d[1] * d[5] * d[6] * 4;
     if (rows > T2SP_MAX_EXTENT || cols > T2SP_MAX_EXTENT || kred > T2SP_MAX_EXTENT) return T2SP_ERR_SHAPE;
+    // the image an output map of OH x OW reads under stride S, and the number of votes
+    if ((int64_t)(d[3] - 1) * d[7] + d[5] > T2SP_MAX_EXTENT || (int64_t)(d[4] - 1) * d[7] + d[6] > T2SP_MAX_EXTENT ||
+        rows * cols > ((int64_t)1 << 40))
+        return T2SP_ERR_SHAPE;
+    for (int i = 0; i < 6; i++)
+        if (!strides_in_range(sp6[i], sw6[i], sv6[i])) return T2SP_ERR_SHAPE;
     bool byte_offsets_fit = false;
     if (cfg == T2SP_CFG_SCALAR || !capsule_fast(d, sp6, sw6, sv6, P, W, V, &byte_offsets_fit)) {
         CapsuleGenericArgs a{P, W, V, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], d[8], d[9], d[10], {}, {}, {}};

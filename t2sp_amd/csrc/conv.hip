@@ -663,6 +663,8 @@ extern "C" int t2sp_conv2d_f32(const float *I, const float *W, float *O, int N, 
         return T2SP_ERR_SHAPE;
     if (CO > T2SP_MAX_EXTENT || OW > T2SP_MAX_EXTENT || (int64_t)N * OH * OW > T2SP_MAX_EXTENT || (int64_t)CI * KH * KW > T2SP_MAX_EXTENT)
         return T2SP_ERR_SHAPE;
+    for (int d = 0; d < 4; d++)
+        if (!strides_in_range(si4[d], sw4[d], so4[d])) return T2SP_ERR_SHAPE;
     const int64_t in_span = (int64_t)(N - 1) * si4[0] + (int64_t)(CI - 1) * si4[1] +
                             (int64_t)(OH + KH - 2) * si4[2] + (OW + KW - 2);
     hipStream_t st = (hipStream_t)stream;

@@ -1388,7 +1388,7 @@ extern "C" int t2sp_sgemm_f32(const float *A, const float *B, float *C, int M, i
                               int64_t lda, int64_t ldb, int64_t ldc, int cfg, float *workspace,
                               size_t workspace_bytes, void *stream) {
     if (lda < 0 || ldb < 0 || ldc < 0) return T2SP_ERR_SHAPE;   // the loaders' offsets are unsigned
-    if (M > T2SP_MAX_EXTENT || N > T2SP_MAX_EXTENT || K > T2SP_MAX_EXTENT) return T2SP_ERR_SHAPE;
+    if (M > T2SP_MAX_EXTENT || N > T2SP_MAX_EXTENT || K > T2SP_MAX_EXTENT || !t2sp::strides_in_range(lda, ldb, ldc)) return T2SP_ERR_SHAPE;
     t2sp::GemmArgs g{};
     g.A = A; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K;
     g.lda = lda; g.ldb = ldb; g.ldc = ldc;
@@ -1401,7 +1401,10 @@ extern "C" int t2sp_sgemm_f32_tiled(const float *A, const float *B, float *C, in
                                     const int64_t *strides6, int cfg, float *workspace,
                                     size_t workspace_bytes, void *stream) {
     if (jjj <= 0 || iii <= 0 || jj <= 0 || ii <= 0 || !strides6 || lda < 0 || ldb < 0) return T2SP_ERR_SHAPE;
-    if (M > T2SP_MAX_EXTENT || N > T2SP_MAX_EXTENT || K > T2SP_MAX_EXTENT) return T2SP_ERR_SHAPE;
+    if (M > T2SP_MAX_EXTENT || N > T2SP_MAX_EXTENT || K > T2SP_MAX_EXTENT || !t2sp::strides_in_range(lda, ldb)) return T2SP_ERR_SHAPE;
+    for (int d = 0; d < 6; d++)
+        if (!t2sp::stride_in_range(strides6[d])) return T2SP_ERR_SHAPE;
+    if (jjj > T2SP_MAX_EXTENT || iii > T2SP_MAX_EXTENT || jj > T2SP_MAX_EXTENT || ii > T2SP_MAX_EXTENT) return T2SP_ERR_SHAPE;
     t2sp::GemmArgs g{};
     g.A = A; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K;
     g.lda = lda; g.ldb = ldb; g.ldc = 0;
@@ -1427,6 +1430,7 @@ extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, fl
                                  int64_t ldcin, float *C, int64_t ldc, int cfg, float *workspace,
                                  size_t workspace_bytes, void *stream) {
     if (!gemm_extents_ok(M, N, K) || lda < 0 || ldb < 0 || ldc < 0 || (Cin && ldcin < 0)) return T2SP_ERR_SHAPE;
+    if (!t2sp::strides_in_range(lda, ldb, ldc, ldcin)) return T2SP_ERR_SHAPE;
     const float *a = A;
     int64_t la = lda;
     auto aligned16 = [](const void *p) { return ((uintptr_t)p & 15) == 0; };

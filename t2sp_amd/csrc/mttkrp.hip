@@ -380,6 +380,7 @@ extern "C" int t2sp_mttkrp_f32(const float *B, const float *C, const float *D, f
     using namespace t2sp;
     if (I <= 0 || J <= 0 || K <= 0 || R <= 0 || !sb3 || !sc2 || !sd2 || !sa2) return T2SP_ERR_SHAPE;
     if (I > T2SP_MAX_EXTENT || R > T2SP_MAX_EXTENT || J > T2SP_MAX_EXTENT || (int64_t)K * J > T2SP_MAX_EXTENT) return T2SP_ERR_SHAPE;
+    if (!strides_in_range(sb3[0], sb3[1], sb3[2], sc2[0], sc2[1], sd2[0], sd2[1], sa2[0], sa2[1])) return T2SP_ERR_SHAPE;
     const bool fast = mttkrp_fast(I, J, sb3, sc2, sd2, sa2, B, C, A);
     if (cfg == T2SP_CFG_AUTO && !fast && sb3[1] == 1 && sc2[0] == 1 && sa2[0] == 1 && workspace &&
         ((uintptr_t)workspace % 16 == 0) && workspace_bytes >= mttkrp_pad_bytes(I, J, K, R) &&

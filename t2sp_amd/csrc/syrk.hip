@@ -678,7 +678,7 @@ extern "C" int t2sp_ssyrk_f32(int upper, int trans, int N, int K, float alpha, c
                               float beta, const float *Cin, int64_t ldcin, float *C, int64_t ldc, int mirror,
                               int cfg, float *workspace, size_t workspace_bytes, void *stream) {
     if (lda < 0 || ldc < 0 || (Cin && ldcin < 0)) return T2SP_ERR_SHAPE;   // the loaders' offsets are unsigned
-    if (N > T2SP_MAX_EXTENT || K > T2SP_MAX_EXTENT) return T2SP_ERR_SHAPE;
+    if (N > T2SP_MAX_EXTENT || K > T2SP_MAX_EXTENT || !t2sp::strides_in_range(lda, ldc, ldcin)) return T2SP_ERR_SHAPE;
     t2sp::SyrkArgs g{};
     g.A = A; g.lda = lda; g.N = N; g.K = K; g.alpha = alpha; g.beta = beta;
     g.Cin = beta != 0.f ? Cin : nullptr; g.ldcin = ldcin;
@@ -693,6 +693,9 @@ extern "C" int t2sp_ssyrk_f32_folded(int trans, int N, int K, float alpha, const
                                      void *stream) {
     if (iii <= 0 || ii <= 0 || !strides6 || N <= 0 || lda < 0 || (Cin && ldcin < 0)) return T2SP_ERR_SHAPE;
     if (N > T2SP_MAX_EXTENT || K > T2SP_MAX_EXTENT || iii > T2SP_MAX_EXTENT || ii > T2SP_MAX_EXTENT || (int64_t)iii * ii > T2SP_MAX_EXTENT) return T2SP_ERR_SHAPE;
+    if (!t2sp::strides_in_range(lda, ldcin)) return T2SP_ERR_SHAPE;
+    for (int d = 0; d < 6; d++)
+        if (!t2sp::stride_in_range(strides6[d])) return T2SP_ERR_SHAPE;
     const int B = iii * ii;
     if (N % B || (N / B) % 2) return T2SP_ERR_SHAPE;   // an even number of whole blocks (syrk.cpp:80-82: i < I/2)
     t2sp::SyrkArgs g{};

@@ -408,6 +408,20 @@ def test_design_constants_belong_to_the_calling_thread():
         L.t2sp_conv_design(0)
 
 
+def _gpu_present():
+    try:
+        import torch
+        return torch.cuda.is_available()
+    except Exception:
+        return False
+
+
+# The two walks below hand the entries buffers that describe more memory than they own: without a device every
+# call ends in the argument checks or at "no device"; with one, a combination that passes the checks would run.
+only_without_gpu = pytest.mark.skipif(_gpu_present(), reason="argument-check walk with fake buffers: CPU only")
+
+
+@only_without_gpu
 def test_entries_survive_random_buffers():
     """Every operator entry with randomly shaped halide_buffer_t arguments (ranks 0 to 11, extents from -1 to
     2^31 - 1, strides from -1 to 2^31 - 1, NULL buffers and hosts, both dirty flags): each call must come back
@@ -478,3 +492,69 @@ def test_entries_survive_random_buffers():
         assert rc <= 0, (fn, rc)
         seen.add(rc)
     assert {-43, -28, -12, -8, -6}.issubset(seen)
+
+
+@only_without_gpu
+def test_thin_layer_entries_survive_random_extents_and_strides():
+    """The plain-pointer entries (t2sp_sgemm_f32, t2sp_sgemm_ex_f32, t2sp_conv2d_f32, t2sp_capsule_f32,
+    t2sp_mttkrp_f32, t2sp_ssyrk_f32) with extents up to 2^31 - 1, strides and leading dimensions from -4 to 2^40,
+    every tile configuration and workspaces of 0 to 2^40 bytes: each call returns 0 or a negative code, and under
+    `make -C t2sp_amd/csrc asan-check` (UndefinedBehaviorSanitizer) no extent x stride product leaves 64 bits.
+    That walk found `M * lda` overflowing for a leading dimension of 2^40; strides beyond T2SP_MAX_STRIDE = 2^31
+    are now refused with T2SP_ERR_SHAPE at every entry."""
+    import random
+    L = t2sp_amd.lib()
+    rng = random.Random(3)
+    i64, f32, sz = ctypes.c_int64, ctypes.c_float, ctypes.c_size_t
+    ext = [1, 2, 3, 4, 5, 15, 16, 17, 63, 64, 100, 128, 255, 256, 1000, 1024, 4096, 65535, 65536, 1 << 20, 1 << 22,
+           1 << 30, (1 << 31) - 1]
+    strd = [0, 1, 2, 3, 4, 16, 100, 1024, 4096, 1 << 20, 1 << 22, (1 << 22) + 4, 1 << 31, (1 << 31) + 1, 1 << 40, -1, -4]
+    ptrs = [0x1000, 0x1004, 0x1010, 0x7f0000000000, 0x7f0000000010]
+    cfgs = [0, 0, 0, 1, 2, 3, 4, 5, 6, 7, 99]
+
+    def e():
+        return rng.choice(ext) if rng.random() < 0.8 else rng.randint(1, 5000)
+
+    def s():
+        return rng.choice(strd)
+
+    def p():
+        return rng.choice(ptrs)
+
+    def arr(n, last=None):
+        v = [s() for _ in range(n)]
+        if last is not None:
+            v[-1] = last
+        return (i64 * n)(*v)
+
+    beyond = 0
+    for _ in range(6000):
+        k = rng.randint(0, 5)
+        ws = rng.choice([None, 0x7f1000000000])
+        wsb = sz(rng.choice([0, 1 << 10, 1 << 30, 1 << 40]) if ws else 0)
+        cfg = rng.choice(cfgs)
+        if k == 0:
+            ld = (s(), s(), s())
+            rc = L.t2sp_sgemm_f32(p(), p(), p(), e(), e(), e(), i64(ld[0]), i64(ld[1]), i64(ld[2]), cfg, ws, wsb, None)
+            if max(ld) > 1 << 31:
+                beyond += 1
+                assert rc == -8
+        elif k == 1:
+            rc = L.t2sp_sgemm_ex_f32(rng.randint(0, 1), rng.randint(0, 1), e(), e(), e(), f32(1.0), p(), i64(s()), p(), i64(s()),
+                                     f32(0.5), rng.choice([None, p()]), i64(s()), p(), i64(s()), cfg, ws, wsb, None)
+        elif k == 2:
+            rc = L.t2sp_conv2d_f32(p(), p(), p(), e() % 5000 + 1, e() % 5000 + 1, e() % 5000 + 1, e() % 5000 + 1,
+                                   e() % 5000 + 1, rng.choice([1, 3, 7]), rng.choice([1, 3, 7]), arr(4, 1), arr(4, 1),
+                                   arr(4, rng.choice([1, 2])), cfg, ws, wsb, None)
+        elif k == 3:
+            d = (ctypes.c_int * 11)(e() % 5000 + 1, e() % 300 + 1, e() % 300 + 1, rng.choice([7, 7, 1 << 20, 1 << 30]), 7, 3, 3,
+                                    rng.choice([2, 2, 1 << 20]), 4, 4, 4)
+            rc = L.t2sp_capsule_f32(p(), p(), p(), d, arr(6, 1), arr(6, 1), arr(6, 1), cfg, rng.choice([0, 1, 3]), ws, wsb, None)
+        elif k == 4:
+            rc = L.t2sp_mttkrp_f32(p(), p(), p(), p(), e(), e(), e(), e(), arr(3), arr(2), arr(2), arr(2), cfg,
+                                   rng.choice([0, 1, 8]), ws, wsb, None)
+        else:
+            rc = L.t2sp_ssyrk_f32(rng.randint(0, 1), rng.randint(0, 1), e(), e(), f32(1.0), p(), i64(s()), f32(0.5),
+                                  rng.choice([None, p()]), i64(s()), p(), i64(s()), rng.randint(0, 2), cfg, ws, wsb, None)
+        assert rc <= 0, (k, rc)
+    assert beyond > 50
