@@ -178,6 +178,16 @@ int t2sp_qrd_f32(const float *A, float *Q, float *R, int m, int n, int batch, in
                  int64_t a_batch_stride, int64_t q_col_stride, int64_t q_batch_stride, int64_t r_row_stride,
                  int64_t r_batch_stride, void *stream);
 
+/* The same with the kernel stated.  T2SP_QRD_ORDERED: every sum over ascending k, one fused multiply-add per
+ * term, as the reference's loop (t2sp_qrd_f32).  T2SP_QRD_PANELS: panels of four pivots with the later columns
+ * updated on the matrix cores; Gram-Schmidt's column-by-column values up to rounding (sums in another order),
+ * so Q agrees with the ordered kernel to a few 2^-24 * cond(A), R to a few 2^-24. */
+#define T2SP_QRD_ORDERED 1
+#define T2SP_QRD_PANELS 2
+int t2sp_qrd_variant_f32(const float *A, float *Q, float *R, int m, int n, int batch, int64_t a_row_stride,
+                         int64_t a_batch_stride, int64_t q_col_stride, int64_t q_batch_stride,
+                         int64_t r_row_stride, int64_t r_batch_stride, int variant, void *stream);
+
 /* O[n,co,h,w] = sum_{ci,kh,kw} I[n,ci,h+kh,w+kw] * W[co,ci,kh,kw], stride 1, valid
  * padding, fp32.  si4/sw4/so4 are element strides of the logical indices
  * (n,ci,h,w), (co,ci,kh,kw), (n,co,h,w); "w" is the innermost spatial axis (the

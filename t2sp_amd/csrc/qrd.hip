@@ -262,6 +262,279 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2)
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same factorisation in panels of four pivots, with the work on the later columns moved to
+// the matrix cores.  Lanes own columns as above.  For the four columns u_0..u_3 of a panel:
+//   1. Gram-Schmidt among the four (a quad of lanes): the steps above, the pivot's values taken
+//      from the pivot's lane by a quad broadcast inside the multiply-add (DPP), no LDS;
+//   2. the owners write u to LDS once (four lanes, 128-bit stores);
+//   3. y_i = u_i . t_j for every column j of the wave: v_mfma_f32_4x4x1 (16 blocks of 4 x 4 x 1)
+//      with A = u_i[k] read back from LDS (lane l supplies i = l % 4) and B = t_j[k], the lane's
+//      own register; block b, lane j, register i then holds y_i of column 4 b + j.  In the
+//      owning quad these are the inner products of the panel's columns with each other;
+//   4. r_i = y_i / |u_i| - sum_{l<i} (q_i . q_l) r_l, q = u / |u|: what Gram-Schmidt's column by
+//      column order computes, because t_j^(i) = t_j - sum_{l<i} r_l q_l.  The q_i . q_l are not
+//      zero in floating point (four nearly parallel columns), and this term is what keeps the
+//      panel form as accurate as the column form; r_i is row 4 P + i of R;
+//   5. t_j -= sum_i r_i q_i: the same instruction with A = u_i[k0 + l % 4] (rows along lanes: the
+//      transposed read of the LDS copy), B = -r_i / |u_i| and C = D = four rows of t_j.
+// Sums run in another order than the reference's loop (two or four partial sums per inner
+// product), so results agree with it to rounding error times cond(A), not bit for bit.  A wave
+// that owns the panel does 1-5, the other wave of a 128-column matrix 3-5 after a barrier.
+template <int II>
+__device__ __forceinline__ float qrd_quad_lane(float v) {        // the value lane II of this lane's quad holds
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), II * 0x55, 0xf, 0xf, true));
+}
+
+// acc += (the value lane II of this lane's quad holds in a) * b, one instruction: the compiler does not fold a DPP
+// move into the multiply-add by itself.  Callers keep two vector-ALU instructions between a write of `a` and this.
+template <int II>
+__device__ __forceinline__ void qrd_fmac_quad_lane(float &acc, float a, float b) {
+    static_assert(II >= 0 && II < 4, "a quad has four lanes");
+    if (II == 0) asm volatile("v_fmac_f32_dpp %0, %1, %2 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(a), "v"(b));
+    if (II == 1) asm volatile("v_fmac_f32_dpp %0, %1, %2 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(a), "v"(b));
+    if (II == 2) asm volatile("v_fmac_f32_dpp %0, %1, %2 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(a), "v"(b));
+    if (II == 3) asm volatile("v_fmac_f32_dpp %0, %1, %2 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(a), "v"(b));
+}
+
+// The sum of x over the 16 lanes that share lane % 4, in every lane: two rotations inside the rows of 16 lanes,
+// then the two swaps of half rows and half waves (the builtins of the swaps returned the first operand twice
+// with this compiler, hence the instructions by name).
+__device__ __forceinline__ float qrd_sum_over_quads(float x) {
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x124, 0xf, 0xf, true));   // row_ror:4
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x128, 0xf, 0xf, true));   // row_ror:8
+    float a = x, b = x;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    x = a + b;
+    a = x;
+    b = x;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    return a + b;
+}
+
+// One Gram-Schmidt step among the four columns of a panel held spread over the wave: lane l has RPL rows (those of
+// its quad l / 4) of column l % 4, so the pivot's values sit in lane II of the same quad and an inner product is
+// RPL multiply-adds and a sum over the quads.  ir_mine: 1 / |u| of this lane's column once it has been the pivot;
+// r_in_panel: R(pivot, this lane's column).
+template <int II, int RPL>
+__device__ __forceinline__ void qrd_spread_step(float (&c)[RPL], int sub, float &r_in_panel, float &ir_mine) {
+    float x0 = 0.f, x1 = 0.f;
+    asm volatile("s_nop 1");
+#pragma unroll
+    for (int e = 0; e < RPL; e += 2) {
+        qrd_fmac_quad_lane<II>(x0, c[e], c[e]);
+        qrd_fmac_quad_lane<II>(x1, c[e + 1], c[e + 1]);
+    }
+    const float x = qrd_sum_over_quads(x0 + x1);
+    const float xi = qrd_quad_lane<II>(x);
+    const float root = sqrtf(xi);
+    const float ir = 1.0f / root;
+    r_in_panel = sub < II ? 0.f : sub == II ? root : ir * x;
+    if (sub == II) ir_mine = ir;
+    if (II < 3) {
+        float s = sub > II ? -x / xi : 0.f;
+        asm volatile("s_nop 1" : "+v"(s));
+#pragma unroll
+        for (int e = 0; e < RPL; e++) qrd_fmac_quad_lane<II>(c[e], c[e], s);
+    }
+}
+
+template <int MR, int ROLE>
+__device__ __forceinline__ void qrd_panel_wave(const QrdArgs &g, float *lds_u, float *lds_s) {
+    constexpr int LD = MR + 4, G4 = MR / 4;              // LD: the four columns of a panel start 4 banks apart
+    const int lane = threadIdx.x & 63, quad = lane >> 2, sub = lane & 3;
+    const int j = (ROLE == QRD_SECOND ? 64 : 0) + lane;
+    const int64_t b = blockIdx.x;
+    const float *a = g.A + b * g.a_batch;
+    float *q = g.Q + b * g.q_batch, *r = g.R + b * g.r_batch;
+
+    qrd_v4f t[G4];
+    const float *aj = a + (j < g.n ? j : g.n - 1);
+    const int rows = j < g.n ? g.m : 0;
+#pragma unroll
+    for (int k = 0; k < MR; k++) {
+        const float v = aj[(int64_t)(k < g.m ? k : g.m - 1) * g.a_row];
+        t[k / 4][k % 4] = k < rows ? v : 0.f;
+    }
+    float my_ir = 0.f;
+
+    // steps 3 to 5 for panel P, whose columns lie in U (the owner has written them and S)
+    // Loads run one chunk of 16 rows ahead of the matrix instructions that use them (the fences keep the
+    // scheduler from sinking them back to their uses, where every instruction would wait for LDS).
+    auto inner_products = [&](const float *U) {
+        const float *ua = U + sub * LD;
+        qrd_v4f y0 = {0.f, 0.f, 0.f, 0.f}, y1 = y0, y2 = y0, y3 = y0;
+        qrd_v4f ahead[2][4];
+        auto fetch = [&](qrd_v4f (&d)[4], int g0) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) d[e] = *reinterpret_cast<const qrd_v4f *>(ua + 4 * (g0 + e));
+        };
+        fetch(ahead[0], 0);
+#pragma unroll
+        for (int g0 = 0; g0 < G4; g0 += 4) {
+            const int cur = (g0 / 4) & 1;
+            if (g0 + 4 < G4) fetch(ahead[cur ^ 1], g0 + 4);
+#pragma unroll
+            for (int gg = 0; gg < 4; gg++) {
+                y0 = __builtin_amdgcn_mfma_f32_4x4x1f32(ahead[cur][gg][0], t[g0 + gg][0], y0, 0, 0, 0);
+                y1 = __builtin_amdgcn_mfma_f32_4x4x1f32(ahead[cur][gg][1], t[g0 + gg][1], y1, 0, 0, 0);
+                y2 = __builtin_amdgcn_mfma_f32_4x4x1f32(ahead[cur][gg][2], t[g0 + gg][2], y2, 0, 0, 0);
+                y3 = __builtin_amdgcn_mfma_f32_4x4x1f32(ahead[cur][gg][3], t[g0 + gg][3], y3, 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        return (y0 + y1) + (y2 + y3);
+    };
+    auto rows_of_r_and_update = [&](int P, const float *U, const float *S, qrd_v4f y, bool in_panel, bool update) {
+        const qrd_v4f s0 = *reinterpret_cast<const qrd_v4f *>(S), s1 = *reinterpret_cast<const qrd_v4f *>(S + 4),
+                      s2 = *reinterpret_cast<const qrd_v4f *>(S + 8), ir = *reinterpret_cast<const qrd_v4f *>(S + 16);
+        const float g10 = ir[1] * ir[0] * s0[1], g20 = ir[2] * ir[0] * s0[2], g21 = ir[2] * ir[1] * s1[2];
+        const float g30 = ir[3] * ir[0] * s0[3], g31 = ir[3] * ir[1] * s1[3], g32 = ir[3] * ir[2] * s2[3];
+        float rr[4];
+        rr[0] = ir[0] * y[0];
+        rr[1] = __builtin_fmaf(-g10, rr[0], ir[1] * y[1]);
+        rr[2] = __builtin_fmaf(-g21, rr[1], __builtin_fmaf(-g20, rr[0], ir[2] * y[2]));
+        rr[3] = __builtin_fmaf(-g32, rr[2], __builtin_fmaf(-g31, rr[1], __builtin_fmaf(-g30, rr[0], ir[3] * y[3])));
+        const bool later = j >= 4 * (P + 1);
+        float c[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int p = 4 * P + i;
+            if (p < g.n && j < g.n) r[(int64_t)p * g.r_row + j] = later ? rr[i] : in_panel ? S[20 + 4 * i + sub] : 0.f;
+            c[i] = later ? -ir[i] * rr[i] : 0.f;
+        }
+        if (!update) return;
+        const float *ub = U + sub;
+        float ahead[2][4][4];
+        auto fetch = [&](float (&d)[4][4], int g0) {
+#pragma unroll
+            for (int gg = 0; gg < 4; gg++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) d[gg][i] = ub[i * LD + 4 * (g0 + gg)];
+        };
+        fetch(ahead[0], 0);
+#pragma unroll
+        for (int g0 = 0; g0 < G4; g0 += 4) {
+            const int cur = (g0 / 4) & 1;
+            if (g0 + 4 < G4) fetch(ahead[cur ^ 1], g0 + 4);
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int gg = 0; gg < 4; gg++)
+                    t[g0 + gg] = __builtin_amdgcn_mfma_f32_4x4x1f32(ahead[cur][gg][i], c[i], t[g0 + gg], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // The whole panel P for the wave that owns its columns (quad Pw of this wave).  The four owners write their
+    // columns to LDS, the wave reads them back spread over all lanes (RPL rows of one column each), orthogonalises
+    // them there, writes them back and the owners reload theirs: a step among four columns then costs 2 RPL
+    // multiply-adds instead of 2 MR.
+    auto own_panel = [&](int P, bool with_other_wave, bool need_products, bool update) {
+        constexpr int RPL = MR / 16;
+        const int Pw = P & 15, buf = with_other_wave ? P & 1 : 0;
+        float *U = lds_u + buf * 4 * LD, *S = lds_s + buf * 48;
+        const bool in_panel = quad == Pw;
+        if (in_panel) {
+#pragma unroll
+            for (int gq = 0; gq < G4; gq++) *reinterpret_cast<qrd_v4f *>(U + sub * LD + 4 * gq) = t[gq];
+        }
+        __builtin_amdgcn_wave_barrier();                   // one wave's LDS accesses stay in program order
+        float c[RPL];
+        float *mine = U + sub * LD + RPL * quad;
+#pragma unroll
+        for (int e = 0; e < RPL; e += 4) {
+            const qrd_v4f v = *reinterpret_cast<const qrd_v4f *>(mine + e);
+            c[e] = v[0], c[e + 1] = v[1], c[e + 2] = v[2], c[e + 3] = v[3];
+        }
+        float rp[4] = {0.f, 0.f, 0.f, 0.f}, ir_mine = 0.f;
+        const int left = g.n - 4 * P;                      // uniform: only the last panel has fewer than four pivots
+        qrd_spread_step<0, RPL>(c, sub, rp[0], ir_mine);
+        if (left > 1) qrd_spread_step<1, RPL>(c, sub, rp[1], ir_mine);
+        if (left > 2) qrd_spread_step<2, RPL>(c, sub, rp[2], ir_mine);
+        if (left > 3) qrd_spread_step<3, RPL>(c, sub, rp[3], ir_mine);
+#pragma unroll
+        for (int e = 0; e < RPL; e += 4) {
+            const qrd_v4f v = {c[e], c[e + 1], c[e + 2], c[e + 3]};
+            *reinterpret_cast<qrd_v4f *>(mine + e) = v;
+        }
+        if (quad == 0) {
+            S[16 + sub] = ir_mine;
+#pragma unroll
+            for (int i = 0; i < 4; i++) S[20 + 4 * i + sub] = rp[i];
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (in_panel) {
+#pragma unroll
+            for (int gq = 0; gq < G4; gq++) t[gq] = *reinterpret_cast<const qrd_v4f *>(U + sub * LD + 4 * gq);
+            my_ir = S[16 + sub];
+        }
+        if (!need_products) {                              // the last panel of the matrix: nothing after it
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (4 * P + i < g.n && j < g.n) r[(int64_t)(4 * P + i) * g.r_row + j] = in_panel ? S[20 + 4 * i + sub] : 0.f;
+            return;
+        }
+        const qrd_v4f y = inner_products(U);
+        if (in_panel) *reinterpret_cast<qrd_v4f *>(S + 4 * sub) = y;   // S[4 l + i] = u_i . u_l
+        if (with_other_wave) __syncthreads(); else __builtin_amdgcn_wave_barrier();
+        rows_of_r_and_update(P, U, S, y, in_panel, update);
+        __builtin_amdgcn_wave_barrier();
+    };
+
+    const int panels = (g.n + 3) / 4;
+    if (ROLE == QRD_FIRST) {
+        for (int P = 0; P < 16; P++) own_panel(P, true, true, P < 15);
+    } else if (ROLE == QRD_SECOND) {
+        for (int P = 0; P < 16; P++) {
+            __syncthreads();
+            const float *U = lds_u + (P & 1) * 4 * LD;
+            const qrd_v4f y = inner_products(U);
+            rows_of_r_and_update(P, U, lds_s + (P & 1) * 48, y, false, true);
+        }
+        for (int P = 16; P < panels; P++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (4 * P + i < g.n) r[(int64_t)(4 * P + i) * g.r_row + lane] = 0.f;   // under the columns of the wave that has left
+            own_panel(P, false, P + 1 < panels, P + 1 < panels);
+        }
+    } else {
+        for (int P = 0; P < panels; P++) own_panel(P, false, P + 1 < panels, P + 1 < panels);
+    }
+
+    if (j >= g.n) return;
+    float *qj = q + (int64_t)j * g.q_col;
+    int m_out = g.m;
+    asm volatile("" : "+s"(m_out));
+    if (m_out % 4 == 0 && g.q_col % 4 == 0 && g.q_batch % 4 == 0 && (reinterpret_cast<uintptr_t>(g.Q) & 15) == 0) {
+#pragma unroll
+        for (int k = 0; k < MR; k += 4)
+            if (k < m_out) *reinterpret_cast<qrd_v4f *>(qj + k) = my_ir * t[k / 4];
+    } else {
+#pragma unroll
+        for (int k = 0; k < MR; k++)
+            if (k < m_out) qj[k] = my_ir * t[k / 4][k % 4];
+    }
+}
+
+template <int MR, int NW>
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) qrd_panel_kernel(const QrdArgs g) {
+    __shared__ __align__(16) float lds_u[2 * 4 * (MR + 4)];
+    __shared__ __align__(16) float lds_s[2 * 48];
+    if (NW == 1) {
+        qrd_panel_wave<MR, QRD_ALONE>(g, lds_u, lds_s);
+    } else if (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6) == 0) {
+        qrd_panel_wave<MR, QRD_FIRST>(g, lds_u, lds_s);
+    } else {
+        qrd_panel_wave<MR, QRD_SECOND>(g, lds_u, lds_s);
+    }
+}
+
+template <int MR, int NW>
+static int launch_qrd_panels(const QrdArgs &g, hipStream_t stream) {
+    hipLaunchKernelGGL((qrd_panel_kernel<MR, NW>), dim3((unsigned)g.batch), dim3(64 * NW), 0, stream, g);
+    return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+}
+
 template <int MR, int NW, int CACHE, int KEEP>
 static int launch_qrd(const QrdArgs &g, hipStream_t stream) {
     hipLaunchKernelGGL((qrd_kernel<MR, NW, CACHE, KEEP>), dim3((unsigned)g.batch), dim3(64 * NW), 0, stream, g);
@@ -269,6 +542,23 @@ static int launch_qrd(const QrdArgs &g, hipStream_t stream) {
 }
 
 }  // namespace t2sp
+
+extern "C" int t2sp_qrd_variant_f32(const float *A, float *Q, float *R, int m, int n, int batch, int64_t a_row_stride,
+                                    int64_t a_batch_stride, int64_t q_col_stride, int64_t q_batch_stride,
+                                    int64_t r_row_stride, int64_t r_batch_stride, int variant, void *stream) {
+    using namespace t2sp;
+    if (variant == T2SP_QRD_ORDERED)
+        return t2sp_qrd_f32(A, Q, R, m, n, batch, a_row_stride, a_batch_stride, q_col_stride, q_batch_stride, r_row_stride,
+                            r_batch_stride, stream);
+    if (variant != T2SP_QRD_PANELS) return T2SP_ERR_SHAPE;
+    if (m <= 0 || n <= 0 || batch < 0 || m > T2SP_QRD_MAX_DIM || n > T2SP_QRD_MAX_DIM) return T2SP_ERR_SHAPE;
+    if (a_row_stride < n || q_col_stride < m || r_row_stride < n) return T2SP_ERR_SHAPE;
+    if (batch == 0) return T2SP_OK;
+    QrdArgs g{A, Q, R, m, n, batch, a_row_stride, a_batch_stride, q_col_stride, q_batch_stride, r_row_stride, r_batch_stride};
+    hipStream_t s = (hipStream_t)stream;
+    if (n <= 64) return m <= 64 ? launch_qrd_panels<64, 1>(g, s) : launch_qrd_panels<128, 1>(g, s);
+    return m <= 64 ? launch_qrd_panels<64, 2>(g, s) : launch_qrd_panels<128, 2>(g, s);
+}
 
 extern "C" int t2sp_qrd_f32(const float *A, float *Q, float *R, int m, int n, int batch, int64_t a_row_stride,
                             int64_t a_batch_stride, int64_t q_col_stride, int64_t q_batch_stride,
