@@ -20,8 +20,17 @@ extern "C" {
  *   R: float32 (J, I, BATCH) with I = J: row i contiguous over j, zeros left of the diagonal
  *      (qrd-run-fpga.cpp:583-596).
  * K, J <= 128 (the reference's pipeline is built for 128 x 128).  Returns 0 or a negative
- * halide_error_code_t. */
+ * halide_error_code_t.  Results satisfy the reference's acceptance test |Q R - a| < 0.005
+ * (qrd-run-fpga.cpp:627-640) with either kernel of t2sp_qrd_design(). */
 int qrd(struct halide_buffer_t *a, struct halide_buffer_t *Q, struct halide_buffer_t *R);
+
+/* Which of the two kernels qrd() runs (T2SP_QRD_AUTO, T2SP_QRD_ORDERED, T2SP_QRD_PANELS of t2sp_hip.h: 0, 1, 2;
+ * anything else counts as 0): the ordered kernel sums as the reference's loop does and matches a CPU
+ * restatement of it bit for bit, the panel kernel is the faster one and matches to rounding error times
+ * cond(A).  The value belongs to the calling thread; a thread that has stated none uses the value stated
+ * last by any thread, then the environment variable T2SP_QRD_VARIANT (0, 1 or 2), then 0.  Returns the
+ * value it replaces.  No counterpart in the reference, which has one pipeline. */
+int t2sp_qrd_design(int variant);
 
 /* qrd() that returns the kernel time in ns (negative error code on failure). */
 double qrd_ns(struct halide_buffer_t *a, struct halide_buffer_t *Q, struct halide_buffer_t *R);

@@ -164,24 +164,30 @@ int t2sp_pairhmm_f32(const uint8_t *H, const uint8_t *R, const float *delta, con
                      const float *beta_gap, float *O, int num_haps, int hap_len, int num_reads, int read_len,
                      int64_t h_stride, int64_t r_stride, int hh, int rr, const int64_t *so4, void *stream);
 
-/* QR factorisation of `batch` m x n matrices by modified Gram-Schmidt, column by column, every
- * inner product summed over ascending k: R(i,i) = sqrt(X_i), R(i,j) = X_j / sqrt(X_i),
- * Q(:,i) = t_i / sqrt(X_i), t_j -= (X_j / X_i) * t_i with X_j = <t_i, t_j>
- * (t2s/tests/performance/qrd/qrd.cpp:51-63; the spec's fast_inverse_sqrt is an exact 1/sqrt here).
+/* QR factorisation of `batch` m x n matrices by modified Gram-Schmidt: R(i,i) = sqrt(X_i),
+ * R(i,j) = X_j / sqrt(X_i), Q(:,i) = t_i / sqrt(X_i), t_j -= (X_j / X_i) * t_i with X_j = <t_i, t_j>
+ * (t2s/tests/performance/qrd/qrd.cpp:51-63; the spec's fast_inverse_sqrt, an approximation that differs
+ * from target to target, is 1/sqrt to an ulp or better here).
  * A(k, j) at k*a_row_stride + j (the spec's a(j, k, b), qrd.cpp:46-48); Q(k, i) at i*q_col_stride + k
  * (QDeserializer(k, j, b)); R(i, j) at i*r_row_stride + j, zero left of the diagonal
  * (RDeserializer(j, i, b), qrd-run-fpga.cpp:583-596); the batch strides separate matrices.
- * 1 <= m, n <= T2SP_QRD_MAX_DIM (the reference's pipeline is built for 128 x 128).  Vector
- * arithmetic with the columns in registers, no MFMA; the unit of work is the matrix. */
+ * 1 <= m, n <= T2SP_QRD_MAX_DIM (the reference's pipeline is built for 128 x 128).  The columns
+ * stay in registers; the unit of work is the matrix.  Two kernels, see t2sp_qrd_variant_f32. */
 #define T2SP_QRD_MAX_DIM 128
 int t2sp_qrd_f32(const float *A, float *Q, float *R, int m, int n, int batch, int64_t a_row_stride,
                  int64_t a_batch_stride, int64_t q_col_stride, int64_t q_batch_stride, int64_t r_row_stride,
                  int64_t r_batch_stride, void *stream);
 
-/* The same with the kernel stated.  T2SP_QRD_ORDERED: every sum over ascending k, one fused multiply-add per
- * term, as the reference's loop (t2sp_qrd_f32).  T2SP_QRD_PANELS: panels of four pivots with the later columns
- * updated on the matrix cores; Gram-Schmidt's column-by-column values up to rounding (sums in another order),
- * so Q agrees with the ordered kernel to a few 2^-24 * cond(A), R to a few 2^-24. */
+/* The same with the kernel stated.
+ *   T2SP_QRD_ORDERED: every sum over ascending k with one fused multiply-add per term, the order of the reference's
+ *     loop; results equal a CPU restatement in that order bit for bit.
+ *   T2SP_QRD_PANELS: panels of four pivots, the later columns updated on the matrix cores, 1 / sqrt from the
+ *     hardware's estimate and a Newton step.  The values are those of Gram-Schmidt's column-by-column order up to
+ *     rounding (sums in another order), so R agrees with the ordered kernel to a few 2^-24 in norm and Q to a
+ *     few 2^-24 * cond(A), as two roundings of the same algorithm do.  A column of zero norm makes every later
+ *     column undefined (the ordered kernel confines the NaNs to the columns the reference's loop would).
+ *   T2SP_QRD_AUTO: the faster one, T2SP_QRD_PANELS; t2sp_qrd_f32 is this call with T2SP_QRD_AUTO. */
+#define T2SP_QRD_AUTO 0
 #define T2SP_QRD_ORDERED 1
 #define T2SP_QRD_PANELS 2
 int t2sp_qrd_variant_f32(const float *A, float *Q, float *R, int m, int n, int batch, int64_t a_row_stride,

@@ -86,6 +86,7 @@ def _declare(L):
     L.qrd_ns.restype = ctypes.c_double
     L.t2sp_qrd_f32.argtypes = [vp, vp, vp, i32, i32, i32] + [i64] * 6 + [vp]
     L.t2sp_qrd_variant_f32.argtypes = [vp, vp, vp, i32, i32, i32] + [i64] * 6 + [i32, vp]
+    L.t2sp_qrd_design.argtypes = [i32]
     L.t2sp_host_malloc.argtypes = [ctypes.c_size_t]
     L.t2sp_host_malloc.restype = ctypes.c_void_p
     L.t2sp_host_free.argtypes = [ctypes.c_void_p]

@@ -281,9 +281,10 @@ def pairhmm_case(torch, steps, warmup, peak):
 def qrd_case(torch, steps, warmup, peak):
     """Not one of the headline benchmark configurations: the batched QR pipeline (t2s/tests/performance/qrd) at the
     size its README reports, 16384 matrices of 128 x 128 (23.3 K matrices/s on the FPGA).  The unit of work
-    is the matrix.  No matrix product: modified Gram-Schmidt takes m*n^2 fused multiply-adds per matrix
-    (one inner product and one update per pair of columns), so the roof is the vector issue rate,
-    256 CUs x 64 lanes x 2.4 GHz = 39.3e12 lane-instructions/s."""
+    is the matrix; modified Gram-Schmidt takes m*n^2 multiply-adds per matrix (one inner product and one
+    update per pair of columns).  The default kernel does them in panels of four pivots on the matrix cores
+    (v_mfma_f32_4x4x1, whose rate is the fp32 MFMA peak), the ordered kernel one by one on the vector ALUs
+    (roof: 256 CUs x 64 lanes x 2.4 GHz = 39.3e12 lane-instructions/s); 3.2 GB move per call."""
     L = lib()
     batch, m, n = 16384, 128, 128
     A = ops.fill_uniform(torch.empty(batch, m, n, device="cuda"), 1)
@@ -291,15 +292,19 @@ def qrd_case(torch, steps, warmup, peak):
     R = torch.empty(batch, n, n, device="cuda")
     s = torch.cuda.current_stream().cuda_stream
 
-    def launch():
-        rc = L.t2sp_qrd_f32(A.data_ptr(), Q.data_ptr(), R.data_ptr(), m, n, batch, n, m * n, m, m * n, n, n * n, s)
+    def launch(variant):
+        rc = L.t2sp_qrd_variant_f32(A.data_ptr(), Q.data_ptr(), R.data_ptr(), m, n, batch, n, m * n, m, m * n, n, n * n, variant, s)
         assert rc == 0, rc
 
-    ms = _time(torch, launch, steps, warmup)
-    rate = batch / ms * 1e3
-    return {"Mmatrices/s": round(rate / 1e6, 3), "avg_launch_ms": round(ms, 5), "bound": "vector issue",
-            "frac_of_vector_issue_peak": round(rate * m * n * n / 39.3e12, 4),
+    ms = _time(torch, lambda: launch(ops.QRD_AUTO), steps, warmup)
+    ms_ordered = _time(torch, lambda: launch(ops.QRD_ORDERED), steps, warmup)
+    rate, rate_ordered = batch / ms * 1e3, batch / ms_ordered * 1e3
+    return {"Mmatrices/s": round(rate / 1e6, 3), "avg_launch_ms": round(ms, 5), "bound": "mfma",
+            "TFLOP/s": round(rate * 2 * m * n * n / 1e12, 2), "frac_of_peak": round(rate * 2 * m * n * n / 1e12 / peak, 4),
             "GB/s": round(rate * (m * n + n * m + n * n) * 4 / 1e9, 1),
+            "frac_of_hbm_peak": round(rate * (m * n + n * m + n * n) * 4 / 8e12, 4),
+            "ordered_kernel": {"Mmatrices/s": round(rate_ordered / 1e6, 3), "avg_launch_ms": round(ms_ordered, 5), "bound": "vector issue",
+                               "frac_of_vector_issue_peak": round(rate_ordered * m * n * n / 39.3e12, 4)},
             "workload": "16384 matrices of 128 x 128 (the size of the reference's README)"}
 
 

@@ -10,9 +10,33 @@
 #include "runtime.hpp"
 #include "t2sp_hip.h"
 
+#include <stdlib.h>
+
+#include <atomic>
 #include <initializer_list>
 
 using namespace t2sp;
+
+// The kernel choice is kept per calling thread, like the design constants of the other entries;
+// stored as variant + 1 so that zero means "never stated".
+static std::atomic<int> g_qrd_variant{0};
+static thread_local int tl_qrd_variant = 0;
+
+static int known_variant(int v) { return v == T2SP_QRD_ORDERED || v == T2SP_QRD_PANELS ? v : T2SP_QRD_AUTO; }
+
+static int qrd_variant() {
+    const int stored = tl_qrd_variant > 0 ? tl_qrd_variant : g_qrd_variant.load();
+    if (stored > 0) return stored - 1;
+    if (const char *e = getenv("T2SP_QRD_VARIANT")) return known_variant(atoi(e));
+    return T2SP_QRD_AUTO;
+}
+
+extern "C" int t2sp_qrd_design(int variant) {
+    const int prev = qrd_variant();
+    tl_qrd_variant = known_variant(variant) + 1;
+    g_qrd_variant.store(tl_qrd_variant);
+    return prev;
+}
 
 // Large batches on dense host buffers go through the device in panels of matrices, so that the
 // upload of the next panel and the download of the previous one overlap with the kernel of the
@@ -43,8 +67,8 @@ static int qrd_panels(halide_buffer_t *a, halide_buffer_t *Q, halide_buffer_t *R
         (void)hipEventRecord(ps.up[p], ps.in);
         (void)hipStreamWaitEvent(api_stream(), ps.up[p], 0);
         (void)hipEventRecord(ps.k0[p], api_stream());
-        const int err = t2sp_qrd_f32(da + b0 * ea, dq + b0 * eq, dr + b0 * er, m, n, (int)nb, n, (int64_t)ea, m, (int64_t)eq, n,
-                                     (int64_t)er, api_stream());
+        const int err = t2sp_qrd_variant_f32(da + b0 * ea, dq + b0 * eq, dr + b0 * er, m, n, (int)nb, n, (int64_t)ea, m, (int64_t)eq, n,
+                                             (int64_t)er, qrd_variant(), api_stream());
         if (err) return fail(err, "kernel launch failed");
         (void)hipEventRecord(ps.k1[p], api_stream());
         (void)hipStreamWaitEvent(ps.out, ps.k1[p], 0);
@@ -97,8 +121,8 @@ extern "C" int qrd(halide_buffer_t *a, halide_buffer_t *Q, halide_buffer_t *R) {
     if ((err = dq.output(Q, sq, op))) return err;
     if ((err = dr.output(R, sr, op))) return err;
     KernelTimer timer;
-    err = t2sp_qrd_f32(da.ptr(), dq.ptr(), dr.ptr(), m, n, batch, a->dim[1].stride, a->dim[2].stride, Q->dim[1].stride,
-                       Q->dim[2].stride, R->dim[1].stride, R->dim[2].stride, api_stream());
+    err = t2sp_qrd_variant_f32(da.ptr(), dq.ptr(), dr.ptr(), m, n, batch, a->dim[1].stride, a->dim[2].stride, Q->dim[1].stride,
+                               Q->dim[2].stride, R->dim[1].stride, R->dim[2].stride, qrd_variant(), api_stream());
     if (err) return report(err, op, "kernel launch failed");
     if ((err = timer.stop_and_sync(op))) return err;
     if ((err = dq.finish(op))) return err;

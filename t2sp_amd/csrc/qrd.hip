@@ -327,21 +327,36 @@ __device__ __forceinline__ void qrd_spread_step(float (&c)[RPL], int sub, float 
     }
     const float x = qrd_sum_over_quads(x0 + x1);
     const float xi = qrd_quad_lane<II>(x);
-    const float root = sqrtf(xi);
-    const float ir = 1.0f / root;
+    // 1 / sqrt from the hardware's estimate and one Newton step, the root from it and one correction: a dozen
+    // dependent instructions where the correctly rounded root and quotient take some fifty, on the one chain of
+    // the panel that nothing else hides.  Exact for exact squares; otherwise within an ulp or two.
+    float ir = __builtin_amdgcn_rsqf(xi);
+    ir = __builtin_fmaf(0.5f * ir, __builtin_fmaf(-xi * ir, ir, 1.0f), ir);
+    float root = xi * ir;
+    root = __builtin_fmaf(0.5f * ir, __builtin_fmaf(-root, root, xi), root);
     r_in_panel = sub < II ? 0.f : sub == II ? root : ir * x;
     if (sub == II) ir_mine = ir;
     if (II < 3) {
-        float s = sub > II ? -x / xi : 0.f;
+        float s = sub > II ? -(x * ir) * ir : 0.f;
         asm volatile("s_nop 1" : "+v"(s));
 #pragma unroll
         for (int e = 0; e < RPL; e++) qrd_fmac_quad_lane<II>(c[e], c[e], s);
     }
 }
 
+// LDS of one panel: the four columns as U[i][k] (row stride LD: the columns start 4 banks apart) for the inner
+// products, the same values as UT[k][i] for the update, and S: 0..11 u_i . u_l at [4 l + i], 16..19 1 / |u_i|,
+// 20..35 R(4 P + i, 4 P + l) at [20 + 4 i + l].
+template <int MR>
+struct QrdPanelLds {
+    static constexpr int LD = MR + 4, U = 0, UT = 4 * LD, S = UT + 4 * MR, FLOATS = S + 48;
+};
+
 template <int MR, int ROLE>
-__device__ __forceinline__ void qrd_panel_wave(const QrdArgs &g, float *lds_u, float *lds_s) {
-    constexpr int LD = MR + 4, G4 = MR / 4;              // LD: the four columns of a panel start 4 banks apart
+__device__ __forceinline__ void qrd_panel_wave(const QrdArgs &g, float *lds) {
+    using Lds = QrdPanelLds<MR>;
+    constexpr int LD = Lds::LD, G4 = MR / 4;
+    constexpr int CH = 2;                                // row groups per chunk of LDS loads, fetched one chunk ahead
     const int lane = threadIdx.x & 63, quad = lane >> 2, sub = lane & 3;
     const int j = (ROLE == QRD_SECOND ? 64 : 0) + lane;
     const int64_t b = blockIdx.x;
@@ -356,26 +371,26 @@ __device__ __forceinline__ void qrd_panel_wave(const QrdArgs &g, float *lds_u, f
         const float v = aj[(int64_t)(k < g.m ? k : g.m - 1) * g.a_row];
         t[k / 4][k % 4] = k < rows ? v : 0.f;
     }
-    float my_ir = 0.f;
+    const bool q_vectors = g.m % 4 == 0 && g.q_col % 4 == 0 && g.q_batch % 4 == 0 && (reinterpret_cast<uintptr_t>(g.Q) & 15) == 0;
 
-    // steps 3 to 5 for panel P, whose columns lie in U (the owner has written them and S)
-    // Loads run one chunk of 16 rows ahead of the matrix instructions that use them (the fences keep the
-    // scheduler from sinking them back to their uses, where every instruction would wait for LDS).
-    auto inner_products = [&](const float *U) {
-        const float *ua = U + sub * LD;
+    // Steps 3 to 5 for panel P, whose columns the owner has written to LDS.  Loads run one chunk of rows ahead of
+    // the matrix instructions that use them (the fences keep the scheduler from sinking them back to their uses,
+    // where every instruction would wait for LDS); one 128-bit load feeds four matrix instructions in both passes.
+    auto inner_products = [&](const float *L) {
+        const float *ua = L + Lds::U + sub * LD;
         qrd_v4f y0 = {0.f, 0.f, 0.f, 0.f}, y1 = y0, y2 = y0, y3 = y0;
-        qrd_v4f ahead[2][4];
-        auto fetch = [&](qrd_v4f (&d)[4], int g0) {
+        qrd_v4f ahead[2][CH];
+        auto fetch = [&](qrd_v4f (&d)[CH], int g0) {
 #pragma unroll
-            for (int e = 0; e < 4; e++) d[e] = *reinterpret_cast<const qrd_v4f *>(ua + 4 * (g0 + e));
+            for (int e = 0; e < CH; e++) d[e] = *reinterpret_cast<const qrd_v4f *>(ua + 4 * (g0 + e));
         };
         fetch(ahead[0], 0);
 #pragma unroll
-        for (int g0 = 0; g0 < G4; g0 += 4) {
-            const int cur = (g0 / 4) & 1;
-            if (g0 + 4 < G4) fetch(ahead[cur ^ 1], g0 + 4);
+        for (int g0 = 0; g0 < G4; g0 += CH) {
+            const int cur = (g0 / CH) & 1;
+            if (g0 + CH < G4) fetch(ahead[cur ^ 1], g0 + CH);
 #pragma unroll
-            for (int gg = 0; gg < 4; gg++) {
+            for (int gg = 0; gg < CH; gg++) {
                 y0 = __builtin_amdgcn_mfma_f32_4x4x1f32(ahead[cur][gg][0], t[g0 + gg][0], y0, 0, 0, 0);
                 y1 = __builtin_amdgcn_mfma_f32_4x4x1f32(ahead[cur][gg][1], t[g0 + gg][1], y1, 0, 0, 0);
                 y2 = __builtin_amdgcn_mfma_f32_4x4x1f32(ahead[cur][gg][2], t[g0 + gg][2], y2, 0, 0, 0);
@@ -385,7 +400,10 @@ __device__ __forceinline__ void qrd_panel_wave(const QrdArgs &g, float *lds_u, f
         }
         return (y0 + y1) + (y2 + y3);
     };
-    auto rows_of_r_and_update = [&](int P, const float *U, const float *S, qrd_v4f y, bool in_panel, bool update) {
+    // next_u: where the columns of panel P + 1 go if this wave owns them (else null): its four lanes store each
+    // group of rows as soon as the update has finished it, under the matrix instructions of the groups after it.
+    auto rows_of_r_and_update = [&](int P, const float *L, qrd_v4f y, bool in_panel, bool update, float *next_u) {
+        const float *S = L + Lds::S;
         const qrd_v4f s0 = *reinterpret_cast<const qrd_v4f *>(S), s1 = *reinterpret_cast<const qrd_v4f *>(S + 4),
                       s2 = *reinterpret_cast<const qrd_v4f *>(S + 8), ir = *reinterpret_cast<const qrd_v4f *>(S + 16);
         const float g10 = ir[1] * ir[0] * s0[1], g20 = ir[2] * ir[0] * s0[2], g21 = ir[2] * ir[1] * s1[2];
@@ -404,43 +422,48 @@ __device__ __forceinline__ void qrd_panel_wave(const QrdArgs &g, float *lds_u, f
             c[i] = later ? -ir[i] * rr[i] : 0.f;
         }
         if (!update) return;
-        const float *ub = U + sub;
-        float ahead[2][4][4];
-        auto fetch = [&](float (&d)[4][4], int g0) {
+        const float *ut = L + Lds::UT + 4 * sub;
+        qrd_v4f ahead[2][CH];
+        auto fetch = [&](qrd_v4f (&d)[CH], int g0) {
 #pragma unroll
-            for (int gg = 0; gg < 4; gg++)
-#pragma unroll
-                for (int i = 0; i < 4; i++) d[gg][i] = ub[i * LD + 4 * (g0 + gg)];
+            for (int gg = 0; gg < CH; gg++) d[gg] = *reinterpret_cast<const qrd_v4f *>(ut + 16 * (g0 + gg));
         };
         fetch(ahead[0], 0);
 #pragma unroll
-        for (int g0 = 0; g0 < G4; g0 += 4) {
-            const int cur = (g0 / 4) & 1;
-            if (g0 + 4 < G4) fetch(ahead[cur ^ 1], g0 + 4);
+        for (int g0 = 0; g0 < G4; g0 += CH) {
+            const int cur = (g0 / CH) & 1;
+            if (g0 + CH < G4) fetch(ahead[cur ^ 1], g0 + CH);
 #pragma unroll
             for (int i = 0; i < 4; i++)
 #pragma unroll
-                for (int gg = 0; gg < 4; gg++)
+                for (int gg = 0; gg < CH; gg++)
                     t[g0 + gg] = __builtin_amdgcn_mfma_f32_4x4x1f32(ahead[cur][gg][i], c[i], t[g0 + gg], 0, 0, 0);
+            if (next_u && quad == ((P + 1) & 15)) {
+#pragma unroll
+                for (int gg = 0; gg < CH; gg++) *reinterpret_cast<qrd_v4f *>(next_u + sub * LD + 4 * (g0 + gg)) = t[g0 + gg];
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    // The whole panel P for the wave that owns its columns (quad Pw of this wave).  The four owners write their
-    // columns to LDS, the wave reads them back spread over all lanes (RPL rows of one column each), orthogonalises
-    // them there, writes them back and the owners reload theirs: a step among four columns then costs 2 RPL
-    // multiply-adds instead of 2 MR.
+    auto publish = [&](float *u) {                         // the first panel a wave owns
+        if (quad == 0) {
+#pragma unroll
+            for (int gq = 0; gq < G4; gq++) *reinterpret_cast<qrd_v4f *>(u + sub * LD + 4 * gq) = t[gq];
+        }
+    };
+    // The whole panel P for the wave that owns its columns (quad P % 16 of this wave).  The four owners write
+    // their columns to LDS and the wave reads them back spread over all lanes (RPL rows of one column each);
+    // there the four are orthogonalised (a step costs 2 RPL multiply-adds instead of 2 MR), their inner products
+    // with each other taken, the columns of Q stored and u written back to LDS in both layouts.  The owners'
+    // registers keep the old values from then on: nothing reads them (their update factors are zero).
     auto own_panel = [&](int P, bool with_other_wave, bool need_products, bool update) {
         constexpr int RPL = MR / 16;
-        const int Pw = P & 15, buf = with_other_wave ? P & 1 : 0;
-        float *U = lds_u + buf * 4 * LD, *S = lds_s + buf * 48;
-        const bool in_panel = quad == Pw;
-        if (in_panel) {
-#pragma unroll
-            for (int gq = 0; gq < G4; gq++) *reinterpret_cast<qrd_v4f *>(U + sub * LD + 4 * gq) = t[gq];
-        }
+        float *L = lds + (with_other_wave ? P & 1 : 0) * Lds::FLOATS;
+        float *S = L + Lds::S;
+        const bool in_panel = quad == (P & 15);
         __builtin_amdgcn_wave_barrier();                   // one wave's LDS accesses stay in program order
         float c[RPL];
-        float *mine = U + sub * LD + RPL * quad;
+        float *mine = L + Lds::U + sub * LD + RPL * quad;
 #pragma unroll
         for (int e = 0; e < RPL; e += 4) {
             const qrd_v4f v = *reinterpret_cast<const qrd_v4f *>(mine + e);
@@ -452,44 +475,72 @@ __device__ __forceinline__ void qrd_panel_wave(const QrdArgs &g, float *lds_u, f
         if (left > 1) qrd_spread_step<1, RPL>(c, sub, rp[1], ir_mine);
         if (left > 2) qrd_spread_step<2, RPL>(c, sub, rp[2], ir_mine);
         if (left > 3) qrd_spread_step<3, RPL>(c, sub, rp[3], ir_mine);
+        if (need_products) {
 #pragma unroll
-        for (int e = 0; e < RPL; e += 4) {
-            const qrd_v4f v = {c[e], c[e + 1], c[e + 2], c[e + 3]};
-            *reinterpret_cast<qrd_v4f *>(mine + e) = v;
+            for (int e = 0; e < RPL; e += 4) {
+                const qrd_v4f v = {c[e], c[e + 1], c[e + 2], c[e + 3]};
+                *reinterpret_cast<qrd_v4f *>(mine + e) = v;
+            }
+#pragma unroll
+            for (int e = 0; e < RPL; e++) L[Lds::UT + 4 * (RPL * quad + e) + sub] = c[e];
+            // u_l . u_(this lane's column) for l = 0, 1, 2 (used for l below the column)
+            float d0 = 0.f, d1 = 0.f, d2 = 0.f;
+            asm volatile("s_nop 1");
+#pragma unroll
+            for (int e = 0; e < RPL; e++) {
+                qrd_fmac_quad_lane<0>(d0, c[e], c[e]);
+                qrd_fmac_quad_lane<1>(d1, c[e], c[e]);
+                qrd_fmac_quad_lane<2>(d2, c[e], c[e]);
+            }
+            d0 = qrd_sum_over_quads(d0);
+            d1 = qrd_sum_over_quads(d1);
+            d2 = qrd_sum_over_quads(d2);
+            if (quad == 0) S[sub] = d0, S[4 + sub] = d1, S[8 + sub] = d2;
         }
         if (quad == 0) {
             S[16 + sub] = ir_mine;
 #pragma unroll
             for (int i = 0; i < 4; i++) S[20 + 4 * i + sub] = rp[i];
         }
-        __builtin_amdgcn_wave_barrier();
-        if (in_panel) {
+        if (4 * P + sub < g.n) {                           // Q(:, 4 P + sub), rows RPL * quad ..
+            float *qc = q + (int64_t)(4 * P + sub) * g.q_col + RPL * quad;
+            if (q_vectors) {
 #pragma unroll
-            for (int gq = 0; gq < G4; gq++) t[gq] = *reinterpret_cast<const qrd_v4f *>(U + sub * LD + 4 * gq);
-            my_ir = S[16 + sub];
+                for (int e = 0; e < RPL; e += 4)
+                    if (RPL * quad + e < g.m) {
+                        const qrd_v4f v = {ir_mine * c[e], ir_mine * c[e + 1], ir_mine * c[e + 2], ir_mine * c[e + 3]};
+                        *reinterpret_cast<qrd_v4f *>(qc + e) = v;
+                    }
+            } else {
+#pragma unroll
+                for (int e = 0; e < RPL; e++)
+                    if (RPL * quad + e < g.m) qc[e] = ir_mine * c[e];
+            }
         }
+        __builtin_amdgcn_wave_barrier();
         if (!need_products) {                              // the last panel of the matrix: nothing after it
 #pragma unroll
             for (int i = 0; i < 4; i++)
                 if (4 * P + i < g.n && j < g.n) r[(int64_t)(4 * P + i) * g.r_row + j] = in_panel ? S[20 + 4 * i + sub] : 0.f;
             return;
         }
-        const qrd_v4f y = inner_products(U);
-        if (in_panel) *reinterpret_cast<qrd_v4f *>(S + 4 * sub) = y;   // S[4 l + i] = u_i . u_l
+        const qrd_v4f y = inner_products(L);
         if (with_other_wave) __syncthreads(); else __builtin_amdgcn_wave_barrier();
-        rows_of_r_and_update(P, U, S, y, in_panel, update);
+        float *next_u = update ? lds + (with_other_wave ? (P + 1) & 1 : 0) * Lds::FLOATS + Lds::U : nullptr;
+        rows_of_r_and_update(P, L, y, in_panel, update, next_u);
         __builtin_amdgcn_wave_barrier();
     };
 
     const int panels = (g.n + 3) / 4;
     if (ROLE == QRD_FIRST) {
+        publish(lds + Lds::U);
         for (int P = 0; P < 16; P++) own_panel(P, true, true, P < 15);
     } else if (ROLE == QRD_SECOND) {
         for (int P = 0; P < 16; P++) {
             __syncthreads();
-            const float *U = lds_u + (P & 1) * 4 * LD;
-            const qrd_v4f y = inner_products(U);
-            rows_of_r_and_update(P, U, lds_s + (P & 1) * 48, y, false, true);
+            const float *L = lds + (P & 1) * Lds::FLOATS;
+            const qrd_v4f y = inner_products(L);
+            rows_of_r_and_update(P, L, y, false, true, P == 15 && panels > 16 ? lds + Lds::U : nullptr);
         }
         for (int P = 16; P < panels; P++) {
 #pragma unroll
@@ -498,34 +549,20 @@ __device__ __forceinline__ void qrd_panel_wave(const QrdArgs &g, float *lds_u, f
             own_panel(P, false, P + 1 < panels, P + 1 < panels);
         }
     } else {
+        publish(lds + Lds::U);
         for (int P = 0; P < panels; P++) own_panel(P, false, P + 1 < panels, P + 1 < panels);
-    }
-
-    if (j >= g.n) return;
-    float *qj = q + (int64_t)j * g.q_col;
-    int m_out = g.m;
-    asm volatile("" : "+s"(m_out));
-    if (m_out % 4 == 0 && g.q_col % 4 == 0 && g.q_batch % 4 == 0 && (reinterpret_cast<uintptr_t>(g.Q) & 15) == 0) {
-#pragma unroll
-        for (int k = 0; k < MR; k += 4)
-            if (k < m_out) *reinterpret_cast<qrd_v4f *>(qj + k) = my_ir * t[k / 4];
-    } else {
-#pragma unroll
-        for (int k = 0; k < MR; k++)
-            if (k < m_out) qj[k] = my_ir * t[k / 4][k % 4];
     }
 }
 
 template <int MR, int NW>
-__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) qrd_panel_kernel(const QrdArgs g) {
-    __shared__ __align__(16) float lds_u[2 * 4 * (MR + 4)];
-    __shared__ __align__(16) float lds_s[2 * 48];
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(MR > 64 ? 2 : 4))) qrd_panel_kernel(const QrdArgs g) {
+    __shared__ __align__(16) float lds[2 * QrdPanelLds<MR>::FLOATS];
     if (NW == 1) {
-        qrd_panel_wave<MR, QRD_ALONE>(g, lds_u, lds_s);
+        qrd_panel_wave<MR, QRD_ALONE>(g, lds);
     } else if (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6) == 0) {
-        qrd_panel_wave<MR, QRD_FIRST>(g, lds_u, lds_s);
+        qrd_panel_wave<MR, QRD_FIRST>(g, lds);
     } else {
-        qrd_panel_wave<MR, QRD_SECOND>(g, lds_u, lds_s);
+        qrd_panel_wave<MR, QRD_SECOND>(g, lds);
     }
 }
 
@@ -547,15 +584,16 @@ extern "C" int t2sp_qrd_variant_f32(const float *A, float *Q, float *R, int m, i
                                     int64_t a_batch_stride, int64_t q_col_stride, int64_t q_batch_stride,
                                     int64_t r_row_stride, int64_t r_batch_stride, int variant, void *stream) {
     using namespace t2sp;
-    if (variant == T2SP_QRD_ORDERED)
-        return t2sp_qrd_f32(A, Q, R, m, n, batch, a_row_stride, a_batch_stride, q_col_stride, q_batch_stride, r_row_stride,
-                            r_batch_stride, stream);
-    if (variant != T2SP_QRD_PANELS) return T2SP_ERR_SHAPE;
+    if (variant != T2SP_QRD_AUTO && variant != T2SP_QRD_ORDERED && variant != T2SP_QRD_PANELS) return T2SP_ERR_SHAPE;
     if (m <= 0 || n <= 0 || batch < 0 || m > T2SP_QRD_MAX_DIM || n > T2SP_QRD_MAX_DIM) return T2SP_ERR_SHAPE;
     if (a_row_stride < n || q_col_stride < m || r_row_stride < n) return T2SP_ERR_SHAPE;
     if (batch == 0) return T2SP_OK;
     QrdArgs g{A, Q, R, m, n, batch, a_row_stride, a_batch_stride, q_col_stride, q_batch_stride, r_row_stride, r_batch_stride};
     hipStream_t s = (hipStream_t)stream;
+    if (variant == T2SP_QRD_ORDERED) {
+        if (n <= 64) return m <= 64 ? launch_qrd<64, 1, 0, 16>(g, s) : launch_qrd<128, 1, 0, 32>(g, s);
+        return m <= 64 ? launch_qrd<64, 2, 64, 16>(g, s) : launch_qrd<128, 2, 80, 32>(g, s);
+    }
     if (n <= 64) return m <= 64 ? launch_qrd_panels<64, 1>(g, s) : launch_qrd_panels<128, 1>(g, s);
     return m <= 64 ? launch_qrd_panels<64, 2>(g, s) : launch_qrd_panels<128, 2>(g, s);
 }
@@ -563,12 +601,6 @@ extern "C" int t2sp_qrd_variant_f32(const float *A, float *Q, float *R, int m, i
 extern "C" int t2sp_qrd_f32(const float *A, float *Q, float *R, int m, int n, int batch, int64_t a_row_stride,
                             int64_t a_batch_stride, int64_t q_col_stride, int64_t q_batch_stride,
                             int64_t r_row_stride, int64_t r_batch_stride, void *stream) {
-    using namespace t2sp;
-    if (m <= 0 || n <= 0 || batch < 0 || m > T2SP_QRD_MAX_DIM || n > T2SP_QRD_MAX_DIM) return T2SP_ERR_SHAPE;
-    if (a_row_stride < n || q_col_stride < m || r_row_stride < n) return T2SP_ERR_SHAPE;
-    if (batch == 0) return T2SP_OK;
-    QrdArgs g{A, Q, R, m, n, batch, a_row_stride, a_batch_stride, q_col_stride, q_batch_stride, r_row_stride, r_batch_stride};
-    hipStream_t s = (hipStream_t)stream;
-    if (n <= 64) return m <= 64 ? launch_qrd<64, 1, 0, 16>(g, s) : launch_qrd<128, 1, 0, 32>(g, s);
-    return m <= 64 ? launch_qrd<64, 2, 64, 16>(g, s) : launch_qrd<128, 2, 80, 32>(g, s);
+    return t2sp_qrd_variant_f32(A, Q, R, m, n, batch, a_row_stride, a_batch_stride, q_col_stride, q_batch_stride, r_row_stride,
+                                r_batch_stride, T2SP_QRD_AUTO, stream);
 }

@@ -194,17 +194,26 @@ def pairhmm(H, R, delta, zeta, eta, alpha_match, alpha_gap, beta_match, beta_gap
     return out
 
 
-def qrd(A, out=None):
+QRD_AUTO, QRD_ORDERED, QRD_PANELS = 0, 1, 2
+
+
+def qrd(A, out=None, variant=QRD_AUTO):
     """A = Q R for every matrix of a batch through the `qrd` entry point (include/qrd-interface.h).
 
     A: (BATCH, K, J), numpy order of the reference's a(J, K, BATCH): K rows, J columns, both at
     most 128.  Returns (Q, R): Q (BATCH, J, K) with Q[b, j] the j-th column (numpy order of
     Q(K, J, BATCH)), R (BATCH, J, J) with R[b, i] the i-th row, zero left of the diagonal
-    (t2s/tests/performance/qrd/qrd-run-fpga.cpp:572-596)."""
+    (t2s/tests/performance/qrd/qrd-run-fpga.cpp:572-596).  `variant` picks the kernel
+    (t2sp_qrd_design): QRD_ORDERED sums in the reference's order, QRD_PANELS / QRD_AUTO is faster."""
     batch, m, n = A.shape
     Q, R = out if out is not None else (_empty_like_kind(A, (batch, n, m)), _empty_like_kind(A, (batch, n, n)))
     a, q, r = HalideBuffer.wrap(A), HalideBuffer.wrap(Q), HalideBuffer.wrap(R)
-    _check("qrd", lib().qrd(a.ref, q.ref, r.ref))
+    L = lib()
+    previous = L.t2sp_qrd_design(int(variant))
+    try:
+        _check("qrd", L.qrd(a.ref, q.ref, r.ref))
+    finally:
+        L.t2sp_qrd_design(previous)
     return Q, R
 
 

@@ -46,6 +46,8 @@ def test_hip_path_matches_the_fixtures():
     ph = t2sp_amd.pairhmm(*o.pairhmm_inputs(**mk.PAIRHMM))
     assert np.array_equal(ph, FIX["pairhmm_fused"])
     assert rel_fro(ph, FIX["pairhmm"])[0] <= TOL
-    Q, R = t2sp_amd.qrd(o.fill_uniform(*mk.QRD))
+    Q, R = t2sp_amd.qrd(o.fill_uniform(*mk.QRD), variant=t2sp_amd.ops.QRD_ORDERED)
     assert np.array_equal(Q, FIX["qrd_q_fused"]) and np.array_equal(R, FIX["qrd_r_fused"])
+    assert rel_fro(Q, FIX["qrd_q"])[0] <= TOL and rel_fro(R, FIX["qrd_r"])[0] <= TOL
+    Q, R = t2sp_amd.qrd(o.fill_uniform(*mk.QRD))                           # the default (panel) kernel
     assert rel_fro(Q, FIX["qrd_q"])[0] <= TOL and rel_fro(R, FIX["qrd_r"])[0] <= TOL

@@ -67,12 +67,18 @@ def test_syrk_and_mttkrp_random_shapes(oracle, seed):
 @pytest.mark.parametrize("seed", range(3))
 def test_qrd_random_shapes(oracle, seed):
     """Random row and column counts up to 128 (one wave or two per matrix, padded registers, vector
-    and scalar stores of Q): bit for bit against the oracle's fused variant."""
+    and scalar stores of Q): the ordered kernel bit for bit against the oracle's fused variant, the panel
+    kernel within what separates two roundings of Gram-Schmidt (2 * 2^-24 * cond(A) for Q, per matrix)."""
     rnd = random.Random(400 + seed)
     for _ in range(12):
         n = rnd.randrange(1, 129)
         m = rnd.randrange(n, 129)
         A = oracle.fill_uniform((rnd.randrange(1, 5), m, n), 7 + seed)
-        Q, R = t2sp_amd.qrd(A)
+        Q, R = t2sp_amd.qrd(A, variant=t2sp_amd.ops.QRD_ORDERED)
         Qf, Rf = oracle.qrd(A, acc=oracle.ACC_F32_FMA)
         assert np.array_equal(Q, Qf, equal_nan=True) and np.array_equal(R, Rf, equal_nan=True), (m, n)
+        Q, R = t2sp_amd.qrd(A, variant=t2sp_amd.ops.QRD_PANELS)
+        for b in range(A.shape[0]):
+            cond = np.linalg.cond(A[b].astype(np.float64))
+            assert rel_fro(Q[b], Qf[b])[0] <= max(1e-6, 2.0 * 2.0 ** -24 * cond), (m, n, cond)
+            assert rel_fro(R[b], Rf[b])[0] <= max(TOL, 0.1 * 2.0 ** -24 * cond), (m, n, cond)
