@@ -399,11 +399,13 @@ __device__ __forceinline__ void qrd_spread_step(float (&c)[RPL], int sub, float 
 }
 
 // LDS of one panel: the four columns as U[i][k] (row stride LD: the columns start 4 banks apart) for the inner
-// products, the same values as UT[k][i] for the update, and S: 0..11 u_i . u_l at [4 l + i], 16..19 1 / |u_i|,
-// 20..35 R(4 P + i, 4 P + l) at [20 + 4 i + l].
+// products, the same values as UT[k][i] for the update (row k at 4 (k + k / 16) floats: the panel wave writes it
+// one value per lane, quad q rows RPL q .., and the shift by k / 16 puts its 64 lanes on 64 banks), and S:
+// 0..11 u_i . u_l at [4 l + i], 16..19 1 / |u_i|, 20..35 R(4 P + i, 4 P + l) at [20 + 4 i + l].
 template <int MR>
 struct QrdPanelLds {
-    static constexpr int LD = MR + 4, U = 0, UT = 4 * LD, S = UT + 4 * MR, FLOATS = S + 48;
+    static constexpr int LD = MR + 4, U = 0, UT = 4 * LD, S = UT + 4 * (MR + MR / 16), FLOATS = S + 48;
+    __device__ static constexpr int ut_row(int k) { return 4 * (k + (k >> 4)); }
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -520,7 +522,7 @@ __device__ __forceinline__ void qrd_pipe_columns(const QrdArgs &g, float *lds) {
             float *next_u = lds + Lds::RAW + (k & 1) * Lds::RAW_FLOATS + sub * LD;
             qrd_v4f ring[DEPTH];
 #pragma unroll
-            for (int gq = 0; gq < DEPTH; gq++) ring[gq] = *reinterpret_cast<const qrd_v4f *>(ut + 16 * gq);
+            for (int gq = 0; gq < DEPTH; gq++) ring[gq] = *reinterpret_cast<const qrd_v4f *>(ut + Pan::ut_row(4 * gq));
 #pragma unroll
             for (int g0 = 0; g0 < G4; g0 += 2) {           // two groups side by side: each one's four instructions form a chain
                 const qrd_v4f a0 = ring[g0 % DEPTH], a1 = ring[(g0 + 1) % DEPTH];
@@ -530,8 +532,8 @@ __device__ __forceinline__ void qrd_pipe_columns(const QrdArgs &g, float *lds) {
                     t[g0 + 1] = __builtin_amdgcn_mfma_f32_4x4x1f32(a1[i], c[i], t[g0 + 1], 0, 0, 0);
                 }
                 if (g0 + DEPTH < G4) {
-                    ring[g0 % DEPTH] = *reinterpret_cast<const qrd_v4f *>(ut + 16 * (g0 + DEPTH));
-                    ring[(g0 + 1) % DEPTH] = *reinterpret_cast<const qrd_v4f *>(ut + 16 * (g0 + 1 + DEPTH));
+                    ring[g0 % DEPTH] = *reinterpret_cast<const qrd_v4f *>(ut + Pan::ut_row(4 * (g0 + DEPTH)));
+                    ring[(g0 + 1) % DEPTH] = *reinterpret_cast<const qrd_v4f *>(ut + Pan::ut_row(4 * (g0 + 1 + DEPTH)));
                 }
                 if (hand_over) {
                     *reinterpret_cast<qrd_v4f *>(next_u + 4 * g0) = t[g0];
@@ -589,7 +591,7 @@ __device__ __forceinline__ void qrd_pipe_panels(const QrdArgs &g, float *lds) {
                 *reinterpret_cast<qrd_v4f *>(mine + e) = v;
             }
 #pragma unroll
-            for (int e = 0; e < RPL; e++) L[Pan::UT + 4 * (RPL * quad + e) + sub] = c[e];
+            for (int e = 0; e < RPL; e++) L[Pan::UT + Pan::ut_row(RPL * quad + e) + sub] = c[e];
             float d[3] = {0.f, 0.f, 0.f}, d1[3] = {0.f, 0.f, 0.f};   // u_l . u_(this lane's column) for l = 0, 1, 2
             qrd_dot(QrdLane<0>{}, d[0], d1[0], c, c);
             qrd_dot(QrdLane<1>{}, d[1], d1[1], c, c);

@@ -148,6 +148,11 @@ def test_thin_layer_rejects_bad_shapes():
     assert L.t2sp_qrd_f32(None, None, None, 129, 8, 1, 8, 8 * 129, 129, 8 * 129, 8, 64, None) == -8
     assert L.t2sp_qrd_f32(None, None, None, 16, 8, 1, 7, 128, 16, 128, 8, 64, None) == -8        # row stride below the row length
     assert L.t2sp_qrd_f32(None, None, None, 16, 8, 0, 8, 128, 16, 128, 8, 64, None) == 0
+    assert L.t2sp_qrd_variant_f32(None, None, None, 16, 8, 0, 8, 128, 16, 128, 8, 64, 1, None) == 0
+    assert L.t2sp_qrd_variant_f32(None, None, None, 16, 8, 0, 8, 128, 16, 128, 8, 64, 3, None) == -8   # no such kernel
+    assert L.t2sp_qrd_variant_f32(None, None, None, 16, 8, 1, 7, 128, 16, 128, 8, 64, 2, None) == -8
+    previous = L.t2sp_qrd_design(1)                        # the kernel choice of qrd(): per thread, returns what it replaces
+    assert L.t2sp_qrd_design(2) == 1 and L.t2sp_qrd_design(7) == 2 and L.t2sp_qrd_design(previous) == 0
     assert L.t2sp_mttkrp_workspace_bytes(512, 512, 512, 256, 1, 128) == 128 * 512 * 256 * 4
 
 
