@@ -170,6 +170,21 @@ def test_full_batch_reconstructs_and_is_orthonormal(variant):
     assert (torch.tril(R, -1) == 0).all()
 
 
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_a_matrix_factors_the_same_in_any_batch(variant):
+    """One workgroup per matrix, no state shared between them: the factors of a matrix are the same bits whether
+    it is alone, in a batch that does not fill the machine, or among 40000 others (more workgroups than one
+    launch round holds several times over)."""
+    import torch
+    A = t2sp_amd.fill_uniform(torch.empty(40000, 128, 128, device="cuda"), 17)
+    Q, R = t2sp_amd.qrd(A, variant=variant)
+    for lo, hi in ((0, 1), (39999, 40000), (1000, 1257), (20000, 21030)):
+        q, r = t2sp_amd.qrd(A[lo:hi].contiguous(), variant=variant)
+        assert torch.equal(q, Q[lo:hi]) and torch.equal(r, R[lo:hi]), (lo, hi)
+    err = (torch.bmm(Q[::97].transpose(1, 2), R[::97]) - A[::97]).abs().amax().item()
+    assert err < 1e-4
+
+
 def test_error_codes(oracle):
     A = oracle.fill_uniform((2, 16, 8), 5)
     with pytest.raises(t2sp_amd.T2spError) as e:           # bytes are not float32
