@@ -50,7 +50,7 @@ __global__ void __launch_bounds__(64 * GBMV_ROWS_PER_WG) sgbmv3_kernel(const Gbm
         if (VEC) {
 #pragma unroll 4
             for (int k = lane * 4; k < g.K; k += 256) {
-                const gbmv_v4f av = *reinterpret_cast<const gbmv_v4f *>(a + k);
+                const gbmv_v4f av = __builtin_nontemporal_load(reinterpret_cast<const gbmv_v4f *>(a + k));   // read once: a stream
                 const gbmv_v4f_u xv = *reinterpret_cast<const gbmv_v4f_u *>(x + k);
                 s0 += av[0] * xv[0];
                 s1 += av[1] * xv[1];
@@ -74,7 +74,7 @@ static int launch_gbmv(const GbmvArgs &g, hipStream_t stream) {
     if (g.I <= 0 || g.K <= 0 || g.t_iii <= 0 || g.t_ii <= 0) return T2SP_ERR_SHAPE;
     const bool vec = g.K % 4 == 0 && g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.x % 4 == 0);
     int64_t blocks = ((int64_t)g.I + GBMV_ROWS_PER_WG - 1) / GBMV_ROWS_PER_WG;
-    if (blocks > 256 * 32) blocks = 256 * 32;            // grid-stride beyond 32 workgroups per CU
+    if (blocks > (1 << 24)) blocks = 1 << 24;            // one row per wave; the loop only serves sizes beyond the grid limit
     auto kern = vec ? sgbmv3_kernel<true> : sgbmv3_kernel<false>;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(64 * GBMV_ROWS_PER_WG), 0, stream, g);
     return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;

@@ -58,8 +58,8 @@ __global__ void __launch_bounds__(SYMV_THREADS) ssymv_block_kernel(const SymvArg
 #pragma unroll
     for (int s = 0; s < SYMV_STEPS; s++) {
         const int row = row0 + s * 8 + rg;
-        a[s] = (col_in && row < g.N) ? *reinterpret_cast<const symv_v4f *>(g.A + (int64_t)row * g.lda + col)
-                                     : symv_v4f{0.f, 0.f, 0.f, 0.f};
+        a[s] = (col_in && row < g.N) ? __builtin_nontemporal_load(reinterpret_cast<const symv_v4f *>(g.A + (int64_t)row * g.lda + col))
+                                     : symv_v4f{0.f, 0.f, 0.f, 0.f};          // the triangle is read once: a stream
     }
     const symv_v4f xc = col_in ? *reinterpret_cast<const symv_v4f *>(g.x + col) : symv_v4f{0.f, 0.f, 0.f, 0.f};
     symv_v4f cacc = {0.f, 0.f, 0.f, 0.f};
