@@ -285,6 +285,11 @@ int t2sp_capsule_direct16_plan(int rows, int cols, int *out6);
 int t2sp_relayout_f32(const float *src, float *dst, int nd, const int *extents,
                       const int64_t *src_strides, const int64_t *dst_strides, void *stream);
 
+/* dst[0..n) = src[0..n), both dense, as a stream past the caches (what a device-to-device copy reaches on this
+ * machine is the practical ceiling of the HBM-bound entries above; bench.py measures it with this call).  The
+ * buffers must not overlap.  No counterpart in the reference. */
+int t2sp_copy_f32(const float *src, float *dst, int64_t n, void *stream);
+
 /* x[i] = u(seed, i), i in [0,n): the seeded uniform[-1,1) generator shared with
  * the CPU checker (same bits for the same seed and index).  The reference's
  * drivers fill their inputs with unseeded random() (gemm-run-fpga.cpp:57-67);

@@ -99,6 +99,7 @@ def _declare(L):
     L.t2sp_conv2d_workspace_bytes.argtypes = [i32] * 7
     L.t2sp_conv2d_workspace_bytes.restype = ctypes.c_size_t
     L.t2sp_relayout_f32.argtypes = [vp, vp, i32, p32, p64, p64, vp]
+    L.t2sp_copy_f32.argtypes = [vp, vp, i64, vp]
     L.capsule.argtypes = [bp, bp, bp]
     L.t2sp_capsule_with_cfg.argtypes = [bp, bp, bp, i32, i32]
     L.t2sp_capsule_design.argtypes = [i32]

@@ -386,14 +386,24 @@ def sgemm_tiny_output(torch, steps, warmup, peak):
 
 
 def copy_rate(torch):
-    """What a plain device-to-device copy of 256 MiB reaches on this box (torch's copy kernel; read + write
-    bytes per second): the measured ceiling next to the nominal 8 TB/s that `frac_of_hbm_peak` of the three
-    matrix-vector entries is quoted against."""
+    """What a plain device-to-device copy of 256 MiB reaches on this box (read + write bytes per second), with
+    the library's streaming copy (128-bit nontemporal loads and stores, one per thread) and with torch's copy
+    kernel: the measured ceiling next to the nominal 8 TB/s that `frac_of_hbm_peak` of the three matrix-vector
+    entries is quoted against."""
     n = 64 << 20
     src, dst = torch.empty(n, device="cuda"), torch.empty(n, device="cuda")
-    ms = _time(torch, lambda: dst.copy_(src), 20, 5)
+    s = torch.cuda.current_stream().cuda_stream
+    L = lib()
+
+    def launch():
+        rc = L.t2sp_copy_f32(src.data_ptr(), dst.data_ptr(), n, s)
+        assert rc == 0, rc
+
+    ms = _time(torch, launch, 50, 10)
+    ms_torch = _time(torch, lambda: dst.copy_(src), 20, 5)
     gbs = 8.0 * n / ms / 1e6
     return {"GB/s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / 8000.0, 4), "avg_launch_ms": round(ms, 5),
+            "torch_copy_GB/s": round(8.0 * n / ms_torch / 1e6, 1),
             "workload": "device copy of 64 Mi floats (256 MiB read, 256 MiB written)"}
 
 

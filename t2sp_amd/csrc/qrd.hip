@@ -466,7 +466,7 @@ __device__ __forceinline__ void qrd_pipe_columns(const QrdArgs &g, float *lds) {
     const int rows = j < g.n ? g.m : 0;
 #pragma unroll
     for (int k = 0; k < MR; k++) {
-        const float v = aj[(int64_t)(k < g.m ? k : g.m - 1) * g.a_row];
+        const float v = __builtin_nontemporal_load(aj + (int64_t)(k < g.m ? k : g.m - 1) * g.a_row);   // A, Q, R: each touched once
         t[k / 4][k % 4] = k < rows ? v : 0.f;
     }
     const int panels = (g.n + 3) / 4;
@@ -546,8 +546,8 @@ __device__ __forceinline__ void qrd_pipe_columns(const QrdArgs &g, float *lds) {
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int p = 4 * k + i;
-            if (p < g.n && j < g.n && !in_next) r[(int64_t)p * g.r_row + j] = rr[i];
-            if (WAVE == 1 && p < g.n && k >= 16) r[(int64_t)p * g.r_row + lane] = 0.f;   // under the columns of the wave that has left
+            if (p < g.n && j < g.n && !in_next) __builtin_nontemporal_store(rr[i], r + (int64_t)p * g.r_row + j);
+            if (WAVE == 1 && p < g.n && k >= 16) __builtin_nontemporal_store(0.f, r + (int64_t)p * g.r_row + lane);   // under the columns of the wave that has left
         }
         if (k + 1 < panels) qrd_lds_barrier();
     }
@@ -613,12 +613,12 @@ __device__ __forceinline__ void qrd_pipe_panels(const QrdArgs &g, float *lds) {
                 for (int e = 0; e < RPL; e += 4)
                     if (RPL * quad + e < g.m) {
                         const qrd_v4f v = {ir_mine * c[e], ir_mine * c[e + 1], ir_mine * c[e + 2], ir_mine * c[e + 3]};
-                        *reinterpret_cast<qrd_v4f *>(qc + e) = v;
+                        __builtin_nontemporal_store(v, reinterpret_cast<qrd_v4f *>(qc + e));
                     }
             } else {
 #pragma unroll
                 for (int e = 0; e < RPL; e++)
-                    if (RPL * quad + e < g.m) qc[e] = ir_mine * c[e];
+                    if (RPL * quad + e < g.m) __builtin_nontemporal_store(ir_mine * c[e], qc + e);
             }
         }
     };

@@ -149,6 +149,8 @@ def test_thin_layer_rejects_bad_shapes():
     assert L.t2sp_qrd_f32(None, None, None, 16, 8, 1, 7, 128, 16, 128, 8, 64, None) == -8        # row stride below the row length
     assert L.t2sp_qrd_f32(None, None, None, 16, 8, 0, 8, 128, 16, 128, 8, 64, None) == 0
     assert L.t2sp_qrd_variant_f32(None, None, None, 16, 8, 0, 8, 128, 16, 128, 8, 64, 1, None) == 0
+    assert L.t2sp_copy_f32(None, None, -1, None) == -8 and L.t2sp_copy_f32(None, None, 8, None) == -8
+    assert L.t2sp_copy_f32(None, None, 0, None) == 0
     assert L.t2sp_qrd_variant_f32(None, None, None, 16, 8, 0, 8, 128, 16, 128, 8, 64, 3, None) == -8   # no such kernel
     assert L.t2sp_qrd_variant_f32(None, None, None, 16, 8, 1, 7, 128, 16, 128, 8, 64, 2, None) == -8
     previous = L.t2sp_qrd_design(1)                        # the kernel choice of qrd(): per thread, returns what it replaces
