@@ -465,8 +465,9 @@ static ConvD16Plan plan_conv_d16(int CO, int P, int KRED) {
         const double loads_per_mfma = (double)(mb + 4) / (4.0 * mb * 4);
         // a workgroup alone on its CU: 4 waves at the rate of this form (measured: 0.92 of the MFMA
         // rate at 4 x 4 blocks, less with fewer MFMAs per load) + launch, first loads, exchange
-        // (5 and 6 row blocks run 6 % under that: their operand ring leaves the registers little room)
-        const double wg = 2.0 * (16.0 * mb) * 64.0 * KRED / 614e9 * (1.0 + 1.5 * loads_per_mfma) / 1.09 * (mb >= 5 ? 1.06 : 1.0);
+        // (5 and 6 row blocks run 6 % under that: their operand ring leaves the registers little room).
+        // Calibrated on 14 shapes of 256 -> 256 channels, 3 x 3 (1 to 8 rounds): within 1 % of the measured times.
+        const double wg = 2.0 * (16.0 * mb) * 64.0 * KRED / 614e9 * (1.0 + 1.5 * loads_per_mfma) / 1.13 * (mb >= 5 ? 1.06 : 1.0);
         const double time = (double)((tiles + cus - 1) / cus) * (wg + 2.5e-6) + 3e-6;
         if (time < best.time) best = ConvD16Plan{mb, rpt, tiles_m, tiles_n, time};
     }
@@ -556,7 +557,10 @@ static ConvPlan plan_conv(int CO, int P, int KRED) {
         const int64_t ptiles = rounds * per_round / tiles_m(c);
         const int p1 = (int)(p0 + ptiles * c.bn < P ? p0 + ptiles * c.bn : P);
         p.st[p.n++] = ConvStage{c.cfg, p0, p1, 1};
-        p.time += (double)rounds * (c.bm == 64 ? 2.0 : 1.0) * 2.0 * c.bm * c.bn * KRED / (614e9 * c.eff * CONV_SUSTAINED) + 3e-6;
+        // a single round of 128 x 128 tiles leaves each CU one workgroup, one wave per SIMD, with nothing to cover
+        // its waits (148.8 us measured against 145.2 from the rate of several rounds, N = 4, 64 x 64)
+        const double alone = rounds == 1 && c.bm == 128 ? 1.025 : 1.0;
+        p.time += alone * (double)rounds * (c.bm == 64 ? 2.0 : 1.0) * 2.0 * c.bm * c.bn * KRED / (614e9 * c.eff * CONV_SUSTAINED) + 3e-6;
         p0 = p1;
     }
     if (p0 >= P) return p;
@@ -579,7 +583,8 @@ static ConvPlan plan_conv(int CO, int P, int KRED) {
             const double busy = per_cu * waves >= 4 ? 1.0 : per_cu * waves / 4.0;
             const double wg = 2.0 * c.bm * c.bn * KRED / (614e9 * c.eff * CONV_SUSTAINED) / sp;     // one workgroup's MFMA time (256 flop/clk at 2.4 GHz)
             const double planes = sp > 1 ? (double)t * sp * c.bm * c.bn * 8.0 / 3e12 + 8e-6 : 0.0;
-            const double time = wg * (double)per_cu / busy + planes;
+            const double alone = per_cu == 1 && c.bm == 128 ? 1.025 : 1.0;      // one wave per SIMD, as for a single whole round
+            const double time = alone * wg * (double)per_cu / busy + planes;
             if (time < best_time) { best_time = time; tail = ConvStage{c.cfg, p0, P, sp}; }
         }
     }
