@@ -821,6 +821,34 @@ static bool capsule_fast(const int *d, const int64_t *sp6, const int64_t *sw6, c
 // The tile of the 16 x 16 direct form for rows x cols votes on the current machine(): rows per
 // tile, row blocks, column blocks, tiles along rows and columns, rounds of workgroups.  For tests
 // of the planner.
+namespace t2sp {
+// Many images under an output of at most 128 columns run as rounds of 128 x 128 LDS tiles, one tile per CU at
+// a time, so a last round that is not full costs a whole round all the same.  When the images of that round
+// are cheaper in the one-launch 16 x 16 form (3 us + their flop at 118 TFLOP/s, measured at 24 to 160 images)
+// than a round (its flop at 0.85 of a CU's MFMA rate: 72 us at the benchmark's channel counts, measured
+// 72.3 to 73.5), the automatic plan is two launches: whole rounds of LDS tiles over the first images, then its
+// own plan for the rest.  Returns the number of images of the first launch, 0 for a single launch.  Only from
+// two whole rounds on: below that the 16 x 16 form alone is as fast (N = 192: 100 us against about 93 in two
+// launches, N = 256: 117 against about 121).  And only when the estimate for the rest is under 0.6 of a round:
+// behind a long launch of LDS tiles the second kernel runs slower than on its own (N = 768, 100 images left:
+// 81 us instead of 51, 367 us in two launches against 358 in one; N = 384, 512, 1024, 2048, with 11 to 50
+// images left: 175, 231, 456, 909 us against 214, 242, 497, 920).
+static int capsule_staged_images(const int *d, int64_t rows, int64_t cols, int64_t kred) {
+    const int cus = machine().cus;
+    if (cols > 128 || d[8] != 4) return 0;
+    const int64_t rows_per_image = (int64_t)d[3] * d[4] * d[8];
+    const int64_t t128 = (rows + 127) / 128;
+    const int64_t rounds = t128 / cus;
+    if (rounds < 2 || t128 % cus == 0) return 0;
+    const int64_t first = rounds * cus * 128 / rows_per_image;          // images whose tiles fill `rounds` rounds
+    const int64_t rest = d[0] - first;
+    if (first < 1 || rest < 1) return 0;
+    const double round_s = 2.0 * 128.0 * 128.0 * (double)kred / (614e9 * 0.85);
+    const double rest_s = 3e-6 + (double)rest * 2.0 * (double)rows_per_image * (double)cols * (double)kred / 118e12;
+    return rest_s + 3e-6 < 0.6 * round_s ? (int)first : 0;
+}
+}  // namespace t2sp
+
 extern "C" int t2sp_capsule_direct16_plan(int rows, int cols, int *out6) {
     if (rows <= 0 || cols <= 0 || !out6 || rows > T2SP_MAX_EXTENT || cols > T2SP_MAX_EXTENT) return 0;
     const t2sp::Direct16Plan p = t2sp::plan_direct16(rows, cols);
@@ -835,6 +863,12 @@ extern "C" size_t t2sp_capsule_workspace_bytes(const int *dims11, int cfg, int s
     for (int i = 0; i < 11; i++)
         if (d[i] <= 0) return 0;
     if (rows <= 0 || rows > T2SP_MAX_EXTENT || cols > T2SP_MAX_EXTENT || kred > T2SP_MAX_EXTENT) return 0;
+    if (cfg == T2SP_CFG_AUTO && splits <= 0) {
+        if (const int first = t2sp::capsule_staged_images(d, rows, cols, kred)) {   // the rest's plan is what may need room
+            const int64_t rest_rows = (int64_t)(d[0] - first) * d[3] * d[4] * d[8];
+            return t2sp::plan_capsule((int)rest_rows, (int)cols, (int)kred, cfg, splits, dims11[8]).scratch_bytes;
+        }
+    }
     return t2sp::plan_capsule((int)rows, (int)cols, (int)kred, cfg, splits, dims11[8]).scratch_bytes;
 }
 
@@ -863,6 +897,18 @@ extern "C" int t2sp_capsule_f32(const float *P, const float *W, float *V, const 
         const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
         hipLaunchKernelGGL(capsule_scalar_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
         return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+    }
+    if (cfg == T2SP_CFG_AUTO && splits <= 0 && byte_offsets_fit) {
+        if (const int first = capsule_staged_images(d, rows, cols, kred)) {
+            int d1[11], d2[11];
+            for (int i = 0; i < 11; i++) d1[i] = d2[i] = d[i];
+            d1[0] = first;
+            d2[0] = d[0] - first;
+            const int rc = t2sp_capsule_f32(P, W, V, d1, sp6, sw6, sv6, T2SP_CFG_128x128, 1, nullptr, 0, stream);
+            if (rc != T2SP_OK) return rc;
+            return t2sp_capsule_f32(P + (int64_t)first * sp6[0], W, V + (int64_t)first * sv6[0], d2, sp6, sw6, sv6, T2SP_CFG_AUTO, 0,
+                                    workspace, workspace_bytes, stream);
+        }
     }
     CapsulePlan p = plan_capsule((int)rows, (int)cols, (int)kred, cfg, splits, d[8]);
     if (p.cfg == T2SP_CFG_DIRECT && !(byte_offsets_fit && direct_smem_bytes((int)kred) <= 160 * 1024))
