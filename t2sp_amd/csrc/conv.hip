@@ -468,7 +468,7 @@ static ConvD16Plan plan_conv_d16(int CO, int P, int KRED) {
         // (5 and 6 row blocks run 6 % under that: their operand ring leaves the registers little room).
         // Calibrated on 14 shapes of 256 -> 256 channels, 3 x 3 (1 to 8 rounds): within 1 % of the measured times.
         const double wg = 2.0 * (16.0 * mb) * 64.0 * KRED / 614e9 * (1.0 + 1.5 * loads_per_mfma) / 1.13 * (mb >= 5 ? 1.06 : 1.0);
-        const double time = (double)((tiles + cus - 1) / cus) * (wg + 2.5e-6) + 3e-6;
+        const double time = (double)((tiles + cus - 1) / cus) * (wg + 1.8e-6) + 3e-6;
         if (time < best.time) best = ConvD16Plan{mb, rpt, tiles_m, tiles_n, time};
     }
     return best;
@@ -600,8 +600,21 @@ static ConvPlan plan_conv(int CO, int P, int KRED) {
 // Short reductions (1 x 1 kernels over few channels) leave the 16 x 16 form nothing to amortise its
 // set-up and its narrow stores with; above 288 reduction rows (3 x 3 over 32 channels) the estimates decide.
 static bool conv_prefers_d16(int CO, int P, int KRED, const ConvPlan &lds) {
-    // within 3 % the staged plan is taken: over many rounds it tends to beat its estimate, the 16 x 16 form not
-    return KRED > CONV_SHORT_KRED && plan_conv_d16(CO, P, KRED).time < 0.97 * lds.time;
+    // Up to 64 output channels the LDS tiles are the 2-wave 64 x 128 ones, and a CU does not run two of their
+    // workgroups any faster than one after the other (measured, 64 channels, tile counts from 64 to 1536 and
+    // reductions of 64, 288, 576 and 1152: 64..256 tiles take one tile's time, 320..1024 nearly twice that).  The
+    // 16 x 16 form is ahead at every reduction length up to two tiles per CU (1.1 to 6 times), and up to three
+    // per CU from 3 x 3 over 32 channels on; beyond that the two are within a few per cent and the estimates decide.
+    if (CO <= 64) {
+        const int cus = machine().cus;
+        const int64_t t64 = ((int64_t)P + 127) / 128;
+        if (t64 <= 2 * cus || (t64 <= 3 * cus + cus / 16 && KRED >= CONV_SHORT_KRED)) return true;
+    }
+    // within 3 % the staged plan is taken where the 16 x 16 form needs more than six rounds of CUs: over many
+    // rounds the staged plan tends to beat its estimate, the 16 x 16 form not
+    const ConvD16Plan d = plan_conv_d16(CO, P, KRED);
+    const bool few = (int64_t)d.tiles_m * d.tiles_n <= 6 * (int64_t)machine().cus;
+    return KRED > CONV_SHORT_KRED && d.time < (few ? 1.0 : 0.97) * lds.time;
 }
 
 using ConvL = TileCfg<256, 256, 16, 4, 2, STYLE_RC>;

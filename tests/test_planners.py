@@ -101,8 +101,10 @@ def test_conv_never_leaves_half_of_a_cu_idle_when_a_split_fills_it(lib, cus):
 
 def test_conv_takes_the_one_launch_form_for_small_convolutions_only(lib):
     """On the full machine: the benchmark convolution and other many-round shapes keep the staged LDS-tile
-    plan, small and middle-sized ones with a reduction of at least 288 rows take the 16 x 16 form, short
-    reductions (1 x 1 kernels over 64 channels) never do; its tiles cover CO with at most 6 row blocks."""
+    plan, small and middle-sized ones with a reduction of more than 288 rows take the 16 x 16 form, shorter
+    reductions only with up to 64 output channels (where the LDS tiles are the two-wave ones, which a CU
+    runs one workgroup after the other) and up to two or three tiles per CU; its tiles cover CO with at
+    most 6 row blocks."""
     lib.t2sp_set_machine(256, 8)
     lib.t2sp_conv2d_direct16_plan.argtypes = [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_void_p]
     out, times = (ctypes.c_int * 4)(), (ctypes.c_double * 2)()
@@ -120,6 +122,11 @@ def test_conv_takes_the_one_launch_form_for_small_convolutions_only(lib):
     assert not takes(64, 64, 256, 56, 56, 1)
     for shape in ((32, 64, 64, 30, 30), (8, 256, 256, 14, 14), (16, 144, 144, 28, 28), (4, 128, 128, 28, 28), (1, 256, 256, 56, 56)):
         assert takes(*shape), shape
+    # up to 64 output channels: measured against the 64 x 128 LDS tiles at 64..1536 tiles and four reductions
+    for shape in ((1, 64, 64, 224, 224), (16, 32, 64, 64, 64), (4, 64, 64, 56, 56, 1), (2, 16, 32, 128, 128), (24, 32, 64, 64, 64)):
+        assert takes(*shape), shape
+    for shape in ((128, 32, 64, 64, 64), (24, 64, 64, 64, 64, 1), (64, 32, 64, 64, 64)):
+        assert not takes(*shape), shape
     lib.t2sp_set_machine(0, 0)
 
 
