@@ -869,6 +869,15 @@ static GemmPhases plan_phases(int64_t tiles, int K, int bk, int bm, int bn, bool
         first += take;
         rest -= take;
     }
+    // a short reduction does not repay the split (its planes and second launch cost more than the part of a
+    // round it saves: 114688 x 128 x 288, 896 tiles of 128 x 128: 93 us split, 75 as one launch)
+    const double unsplit = (double)(full / GEMM_CUS) + 1.0;
+    if (p.scratch_bytes > 0 && unsplit <= p.rounds) {
+        p = GemmPhases{};
+        p.n = 1;
+        p.ph[0] = GemmPhase{0, (int)tiles, 1};
+        p.rounds = unsplit;
+    }
     return p;
 }
 
@@ -887,10 +896,13 @@ static int launch(GemmArgs g, hipStream_t stream, int splits = 1, float *scratch
     const bool edge = (g.M % Cfg::BM) || (g.N % Cfg::BN) || (g.K % (2 * Cfg::BK));
     const size_t smem = Cfg::SMEM_FLOATS * sizeof(float);
     auto kern = edge ? sgemm_kernel<Cfg, true, BT> : sgemm_kernel<Cfg, false, BT>;
+    // (the largest request a launch below can make: one workgroup per CU)
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)smem) != hipSuccess)
+                            (int)lds_request(smem, Cfg::BM == 128 ? 1 : 0)) != hipSuccess)
         return T2SP_ERR_LAUNCH;
     const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+    // LDS asked for a launch of `groups` workgroups: what the kernel needs, or more where that evens the CUs out
+    auto lds_for = [&](int64_t groups) { return lds_request(smem, Cfg::BM == 128 ? resident_cap(groups) : 0); };
     if (phased && splits == 1) {
         GemmPhases p = plan_phases(tiles, g.K, Cfg::BK, Cfg::BM, Cfg::BN, true);
         if (scratch && scratch_bytes >= p.scratch_bytes) {
@@ -899,7 +911,8 @@ static int launch(GemmArgs g, hipStream_t stream, int splits = 1, float *scratch
                 g.tile_count = p.ph[i].count;
                 g.splits = p.ph[i].splits;
                 g.compact = g.splits > 1;
-                hipLaunchKernelGGL(kern, dim3((unsigned)(g.tile_count * g.splits)), dim3(Cfg::NTHREADS), smem, stream, g);
+                hipLaunchKernelGGL(kern, dim3((unsigned)(g.tile_count * g.splits)), dim3(Cfg::NTHREADS),
+                                   lds_for((int64_t)g.tile_count * g.splits), stream, g);
                 if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
                 if (g.splits > 1) {
                     GemmCompactMap<Cfg::BM, Cfg::BN, !BT> map{GemmOutMap{g}};
@@ -913,7 +926,7 @@ static int launch(GemmArgs g, hipStream_t stream, int splits = 1, float *scratch
     g.tile_first = 0;
     g.tile_count = (int)tiles;
     g.compact = 0;
-    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * g.splits), dim3(Cfg::NTHREADS), smem, stream, g);
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * g.splits), dim3(Cfg::NTHREADS), lds_for(tiles * g.splits), stream, g);
     if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
     if (g.splits > 1) {
         GemmOutMap map{g};
@@ -1234,7 +1247,24 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         if (bt) return gemm_d16_bt_ok(g) ? launch_d16_bt(g, stream) : T2SP_ERR_SHAPE;
         return gemm_d16_ok(g) ? launch_d16(g, stream, workspace, workspace_bytes) : T2SP_ERR_SHAPE;
     }
-    if (cfg == T2SP_CFG_AUTO && (bt ? gemm_d16_bt_ok(g) : gemm_d16_ok(g))) {
+    // (the loaders address a tile with 32-bit offsets: leading dimensions below LOADER_MAX_LD)
+    const bool vec_ok = g.K % 4 == 0 && (bt || g.N % 4 == 0) && g.lda % 4 == 0 && g.ldb % 4 == 0 &&
+                        g.lda < LOADER_MAX_LD && g.ldb < LOADER_MAX_LD &&
+                        ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
+                        ((uintptr_t)g.C % 16 == 0) && (g.tiled || g.ldc % 4 == 0) &&
+                        (!g.scale || (g.ldcin % 4 == 0 && (uintptr_t)g.Cin % 16 == 0));
+    // A few rows under a very wide output (plain form; measured at 32, 64, 96 and 128 rows, 8192 to 196608
+    // columns, K = 64, 288, 1152, 4096, every kernel forced in turn):
+    //  - up to 32 rows and at least three tiles of 32 x 128 per CU: the one-wave tiles are 4 to 20 % ahead
+    //    of the 16 x 16 form at every K (32 x 196608 x 1152: 208 -> 188 us);
+    //  - a reduction under 128 with more than 3 M outputs is a stream of C: the LDS tiles' wide stores win,
+    //    one-wave tiles up to 96 rows (96 x 196608 x 64: 67 -> 36 us), whole rounds of 128 x 128 above.
+    const int64_t t32w = (int64_t)((g.M + 31) / 32) * ((g.N + 127) / 128);
+    const bool stream_of_c = g.K < 128 && (int64_t)g.M * g.N >= (3 << 20);
+    const bool one_wave_tiles = cfg == T2SP_CFG_AUTO && !bt && vec_ok &&
+                                ((g.M <= 32 && t32w >= 3 * (int64_t)machine().cus) || (stream_of_c && g.M <= 96));
+    const bool skip_d16 = one_wave_tiles || (cfg == T2SP_CFG_AUTO && !bt && vec_ok && stream_of_c);
+    if (cfg == T2SP_CFG_AUTO && !skip_d16 && (bt ? gemm_d16_bt_ok(g) : gemm_d16_ok(g))) {
         // Measured from 256^2 x 8192 to 3072^2 x 1024: the 16 x 16 form wins whenever 256 x 256 tiles
         // would not fill the chip, except where 128 x 128 tiles do and the reduction is long enough to
         // amortise their prologue, and for tiny outputs with a long reduction (too few tiles even at
@@ -1253,7 +1283,8 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         // and K from 256 to 4096: +4 to +13 %, 2048^3 139 -> 146 TFLOP/s), and so do many rounds of them
         // under an output of at most 128 columns, whatever K (65536 x 128 x 256: 89 -> 114; 802816 x 128 x
         // 1152: 112 -> 130); 384 tiles (one and a half rounds) stay with the 16 x 16 form.
-        const bool tiled_better = (t128 >= 2 * cus - cus / 16 && g.K >= 2048 && fill128 >= 0.6) ||
+        // (tiles a quarter empty lose what they gained: 96 rows, K = 4096, 512 to 1536 tiles: 24 to 29 % behind)
+        const bool tiled_better = (t128 >= 2 * cus - cus / 16 && g.K >= 2048 && fill128 >= 0.85) ||
                                   (t128 % cus == 0 && fill128 >= 0.9) ||
                                   (g.N <= 128 && t128 >= 2 * cus - cus / 16 && fill128 >= 0.9);
         // (with room for the planes the 16 x 16 form splits such a reduction over workgroups itself)
@@ -1272,12 +1303,6 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && gemm_direct_ok(g, cfg == T2SP_CFG_DIRECT))
         return launch_direct(g, stream);
     if (cfg == T2SP_CFG_DIRECT) return T2SP_ERR_SHAPE;
-    // (the loaders address a tile with 32-bit offsets: leading dimensions below LOADER_MAX_LD)
-    const bool vec_ok = g.K % 4 == 0 && (bt || g.N % 4 == 0) && g.lda % 4 == 0 && g.ldb % 4 == 0 &&
-                        g.lda < LOADER_MAX_LD && g.ldb < LOADER_MAX_LD &&
-                        ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
-                        ((uintptr_t)g.C % 16 == 0) && (g.tiled || g.ldc % 4 == 0) &&
-                        (!g.scale || (g.ldcin % 4 == 0 && (uintptr_t)g.Cin % 16 == 0));
     if (cfg == T2SP_CFG_AUTO && !vec_ok && workspace &&
         ((uintptr_t)workspace % 16 == 0) && workspace_bytes >= gemm_pad_bytes(g.M, g.N, g.K, bt)) {
         // K or N not a multiple of 4, or rows that are not 16-byte aligned: multiply zero-padded,
@@ -1311,7 +1336,9 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
     }
     int splits = 1;
     bool phased = false;
-    if (cfg == T2SP_CFG_AUTO) {
+    if (one_wave_tiles) {
+        cfg = T2SP_CFG_32x128;
+    } else if (cfg == T2SP_CFG_AUTO) {
         const GemmPlan p = plan_gemm(g.M, g.N, g.K);
         cfg = p.cfg;
         if (!bt && p.splits > 1 && workspace && workspace_bytes >= p.scratch_bytes) splits = p.splits;

@@ -164,7 +164,7 @@ def test_split_reduction_with_workspace(oracle, torch_cuda, shape):
 
 
 @pytest.mark.parametrize("shape", [(6144, 6144, 4096), (3072, 3072, 2048), (5120, 5120, 512), (4100, 4100, 1024),
-                                   (3000, 7000, 520), (6400, 6400, 256)])
+                                   (3000, 7000, 520), (6400, 6400, 2048)])
 def test_partial_last_round_split_with_workspace(oracle, torch_cuda, shape):
     """Tile counts that are not a multiple of 256: with a workspace the tiles left after the whole
     rounds split their reduction.  The whole result against the run without a workspace, sampled

@@ -36,7 +36,7 @@ def test_dies_follow_from_the_compute_units(lib, cus, xcds):
 
 @pytest.mark.parametrize("cus", CUS)
 @pytest.mark.parametrize("shape", [(8192, 8192, 8192), (6144, 6144, 6144), (5120, 5120, 2048), (4096, 16384, 2048),
-                                   (10240, 10240, 1024), (7168, 7168, 7168)])
+                                   (10240, 10240, 1024), (7168, 7168, 7168), (114688, 128, 288), (5120, 5120, 256)])
 def test_sgemm_launches_whole_rounds_then_a_split_rest(lib, cus, shape):
     lib.t2sp_set_machine(cus, 0)
     M, N, K = shape
@@ -54,8 +54,12 @@ def test_sgemm_launches_whole_rounds_then_a_split_rest(lib, cus, shape):
         elif i == 0 and tiles >= cus and n > 1:
             assert count % cus == 0                 # the unsplit part is whole rounds
     assert covered == tiles
-    if tiles % cus and tiles > cus and K >= 1024:
+    # (a rest of more than half a round saves too little to repay its planes and second launch, and so does
+    # any rest under a short reduction: then everything goes as one launch)
+    if tiles % cus and tiles > cus and K >= 2048 and tiles % cus <= cus // 2:
         assert any(s > 1 for _, _, s in phases), (cus, phases)
+    if tiles > cus and K <= 384:
+        assert phases == [(0, tiles, 1)], (cus, phases)
 
 
 @pytest.mark.parametrize("cus", CUS)
