@@ -275,26 +275,36 @@ static MttkrpPlan plan_mttkrp(int I, int J, int K, int R, int cfg, int splits) {
     // sustained fraction of the 256 x 256 tile's rate, measured
     const Cand cands[4] = {{T2SP_CFG_256x256, 256, 256, 1.0}, {T2SP_CFG_128x128, 128, 128, 0.93},
                            {T2SP_CFG_32x128, 256, 64, 0.85}, {T2SP_CFG_64x128, 64, 64, 0.7}};
+    const int64_t ktiles = (int64_t)K * (J / 16);
+    const int cus = machine().cus;
+    // the reduction split that puts about one workgroup on every CU
+    auto fill = [&](int64_t tiles) {
+        int s = tiles >= cus * 25 / 32 ? 1 : (int)((cus + tiles / 2) / tiles);
+        if (s > ktiles / 16) s = (int)(ktiles / 16);
+        return s < 1 ? 1 : s;
+    };
     if (cfg == T2SP_CFG_AUTO) {
-        // least padded work over sustained rate: a rank of 64 in 256-wide tiles would multiply 4x too much
+        // least estimated time: the padded work over the tile's sustained rate (a rank of 64 in 256-wide tiles
+        // would multiply 4x too much), plus writing and re-reading the planes of the split reduction, which for
+        // few large tiles are many (I = R = 256, J = K = 256: one 256 x 256 tile in 256 shares moves 2 x 67 MB,
+        // 87 us; four 128 x 128 tiles in 64 shares each 75 us).  The large tile keeps a 2 % margin.
         double best = 1e300;
         for (const Cand &c : cands) {
-            const double cost = (double)((I + c.bm - 1) / c.bm * c.bm) * ((R + c.bn - 1) / c.bn * c.bn) / c.eff;
-            if (cost < best) { best = cost; cfg = c.cfg; }
+            const double mp = (double)((I + c.bm - 1) / c.bm * c.bm), np = (double)((R + c.bn - 1) / c.bn * c.bn);
+            const int s = splits > 0 ? splits : fill((int64_t)(mp / c.bm) * (int64_t)(np / c.bn));
+            const double mult = 2.0 * mp * np * (double)J * (double)K / (150e12 * c.eff);
+            const double planes = s > 1 ? 2.0 * s * mp * np * sizeof(float) / 5e12 : 0.0;
+            const double time = (mult + planes) * (c.cfg == T2SP_CFG_256x256 ? 0.98 : 1.0);
+            if (time < best) { best = time; cfg = c.cfg; }
         }
     }
     int bm = 64, bn = 64;
     for (const Cand &c : cands)
         if (c.cfg == cfg) { bm = c.bm; bn = c.bn; }
     const int64_t tiles = (int64_t)((I + bm - 1) / bm) * ((R + bn - 1) / bn);
-    const int64_t ktiles = (int64_t)K * (J / 16);
-    if (splits <= 0) {
-        const int cus = machine().cus;
-        splits = tiles >= cus * 25 / 32 ? 1 : (int)((cus + tiles / 2) / tiles);
-        if (splits > ktiles / 16) splits = (int)(ktiles / 16);
-        if (splits < 1) splits = 1;
-    }
+    if (splits <= 0) splits = fill(tiles);
     if (splits > (ktiles + 1) / 2) splits = (int)((ktiles + 1) / 2);
+    if (splits < 1) splits = 1;
     p.cfg = cfg; p.splits = splits;
     p.Mp = (I + bm - 1) / bm * bm;
     p.Np = (R + bn - 1) / bn * bn;
