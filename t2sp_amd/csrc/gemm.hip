@@ -896,13 +896,16 @@ static int launch(GemmArgs g, hipStream_t stream, int splits = 1, float *scratch
     const bool edge = (g.M % Cfg::BM) || (g.N % Cfg::BN) || (g.K % (2 * Cfg::BK));
     const size_t smem = Cfg::SMEM_FLOATS * sizeof(float);
     auto kern = edge ? sgemm_kernel<Cfg, true, BT> : sgemm_kernel<Cfg, false, BT>;
+    // LDS asked for a launch of `groups` workgroups: what the kernel needs, or more where that evens the CUs out
+    // (the four-wave 128 x 128 tiles of the plain form, three to a CU; the B^T form's tiles measure 3 to 7 % slower
+    // under a cap at every count from 4 to 8 per CU)
+    constexpr bool capped = !BT && Cfg::BM == 128 && Cfg::BN == 128 && Cfg::NTHREADS == 256;
     // (the largest request a launch below can make: one workgroup per CU)
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds_request(smem, Cfg::BM == 128 ? 1 : 0)) != hipSuccess)
+                            (int)lds_request(smem, capped ? 1 : 0)) != hipSuccess)
         return T2SP_ERR_LAUNCH;
     const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
-    // LDS asked for a launch of `groups` workgroups: what the kernel needs, or more where that evens the CUs out
-    auto lds_for = [&](int64_t groups) { return lds_request(smem, Cfg::BM == 128 ? resident_cap(groups) : 0); };
+    auto lds_for = [&](int64_t groups) { return lds_request(smem, capped ? resident_cap(groups) : 0); };
     if (phased && splits == 1) {
         GemmPhases p = plan_phases(tiles, g.K, Cfg::BK, Cfg::BM, Cfg::BN, true);
         if (scratch && scratch_bytes >= p.scratch_bytes) {
