@@ -597,8 +597,9 @@ static ConvPlan plan_conv(int CO, int P, int KRED) {
     return p;
 }
 
-// Short reductions (1 x 1 kernels over few channels) leave the 16 x 16 form nothing to amortise its
-// set-up and its narrow stores with; above 288 reduction rows (3 x 3 over 32 channels) the estimates decide.
+// With more than 64 output channels, short reductions (1 x 1 kernels over few channels) leave the 16 x 16 form
+// nothing to amortise its set-up and its narrow stores with; above 288 reduction rows (3 x 3 over 32 channels)
+// the estimates decide.
 static bool conv_prefers_d16(int CO, int P, int KRED, const ConvPlan &lds) {
     // Up to 64 output channels the LDS tiles are the 2-wave 64 x 128 ones, and a CU does not run two of their
     // workgroups any faster than one after the other (measured, 64 channels, tile counts from 64 to 1536 and
