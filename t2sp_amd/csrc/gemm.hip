@@ -958,7 +958,10 @@ struct GemmPlan {
     bool phased;              // whole rounds, then the remaining tiles with a split reduction
     size_t scratch_bytes;
 };
-static GemmPlan plan_gemm(int M, int N, int K) {
+// two_wave_128: the 128 x 128 tile is the A^T form's, two waves of 64 x 128, which a CU runs well only alone or
+// four at a time (the SIMDs are handed out in a cycle that moves on by one per workgroup); rounds of it are
+// costed a fifth higher.
+static GemmPlan plan_gemm(int M, int N, int K, bool two_wave_128 = false) {
     auto tiles = [&](int bm, int bn) { return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
     GemmPlan p{T2SP_CFG_64x128, 1, false, 0};
     const int cus = machine().cus, nearly_full = cus * 25 / 32;   // 200 of 256: enough tiles to be worth whole rounds
@@ -967,7 +970,7 @@ static GemmPlan plan_gemm(int M, int N, int K) {
         // tile size sustains (measured: 0.94 for 128 x 128)
         const GemmPhases l = plan_phases(tiles(256, 256), K, 16, 256, 256, true);
         const GemmPhases m = plan_phases(tiles(128, 128), K, 16, 128, 128, true);
-        const double cl = l.rounds * 65536.0, cm = m.rounds * 16384.0 / 0.94;
+        const double cl = l.rounds * 65536.0, cm = m.rounds * 16384.0 / (two_wave_128 ? 0.78 : 0.94);
         const bool large = tiles(256, 256) >= nearly_full && cl <= cm;
         p.cfg = large ? T2SP_CFG_256x256 : T2SP_CFG_128x128;
         p.phased = true;
@@ -1230,7 +1233,7 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
             const int cus = machine().cus;
             if (gemm_d16_at_ok(g) && t256 < cus * 25 / 32 && g.K >= 64 && !(t64 < cus / 8 && g.K >= 4096)) return launch_d16_at(g, stream);
         }
-        const GemmPlan p = plan_gemm(g.M, g.N, g.K);
+        const GemmPlan p = plan_gemm(g.M, g.N, g.K, true);
         if (p.phased) {
             const bool phased = workspace && workspace_bytes >= p.scratch_bytes;
             if (p.cfg == T2SP_CFG_256x256) return launch<GemmLA, false>(g, stream, 1, workspace, workspace_bytes, phased);
@@ -1450,7 +1453,11 @@ extern "C" size_t t2sp_sgemm_ex_workspace_bytes(int transa, int M, int N, int K)
     const bool padded = K % 4 || N % 4;
     const size_t pad = padded ? (pad_t > pad_n ? pad_t : pad_n) : 0;
     const int n4 = (int)t2sp::round_up4(N), k4 = (int)(padded ? t2sp::pad_k(K) : K);
-    const size_t tiled = t2sp::plan_gemm(M, n4, k4).scratch_bytes;
+    size_t tiled = t2sp::plan_gemm(M, n4, k4).scratch_bytes;
+    if (transa) {   // taken as it lies, the A^T form may plan other tiles
+        const size_t as_it_lies = t2sp::plan_gemm(M, n4, k4, true).scratch_bytes;
+        if (as_it_lies > tiled) tiled = as_it_lies;
+    }
     const size_t one_launch = t2sp::plan_gemm_d16_split(M, n4, k4, t2sp::plan_gemm_d16(M, n4)).scratch_bytes;
     return t2sp::round_up256(transa ? (size_t)M * K * sizeof(float) : 0) + pad + (tiled > one_launch ? tiled : one_launch);
 }
