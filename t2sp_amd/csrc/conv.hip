@@ -541,8 +541,8 @@ static ConvPlan plan_conv(int CO, int P, int KRED) {
     if (KRED <= CONV_SHORT_KRED) {
         const Cand &c = CO <= 64 ? all[2] : all[1];
         p.st[p.n++] = ConvStage{c.cfg, 0, P, 1};
-        const int64_t per_round = (int64_t)CUS * (c.bm == 64 ? 2 : 1);
-        p.time = (double)((tiles(c, 0) + per_round - 1) / per_round) * (c.bm == 64 ? 2.0 : 1.0) * 2.0 * c.bm * c.bn * KRED /
+        const int64_t per_round = (int64_t)CUS * (c.bm == 64 ? 4 : 1);     // (see the whole rounds below)
+        p.time = (double)((tiles(c, 0) + per_round - 1) / per_round) * (c.bm == 64 ? 4.0 : 1.0) * 2.0 * c.bm * c.bn * KRED /
                      (614e9 * c.eff * CONV_SUSTAINED) + 3e-6;
         return p;
     }
@@ -550,8 +550,10 @@ static ConvPlan plan_conv(int CO, int P, int KRED) {
     for (int i = best; i < 3 && p0 < P; i++) {
         if (i != best && all[i].cfg != T2SP_CFG_128x128) break;
         const Cand &c = all[i];
-        // a round puts a wave on every SIMD: one workgroup per CU, two of the 2-wave ones
-        const int64_t per_round = (int64_t)CUS * (c.bm == 64 ? 2 : 1);
+        // a round loads the four SIMDs of every CU evenly: one workgroup per CU, or four of the 2-wave ones (a CU
+        // hands out its SIMDs in a cycle that moves on by one per workgroup, so two 2-wave workgroups put two
+        // waves on one SIMD and none on another: only four make them level)
+        const int64_t per_round = (int64_t)CUS * (c.bm == 64 ? 4 : 1);
         const int64_t rounds = tiles(c, p0) / per_round;
         if (rounds < 1) continue;
         const int64_t ptiles = rounds * per_round / tiles_m(c);
@@ -560,7 +562,7 @@ static ConvPlan plan_conv(int CO, int P, int KRED) {
         // a single round of 128 x 128 tiles leaves each CU one workgroup, one wave per SIMD, with nothing to cover
         // its waits (148.8 us measured against 145.2 from the rate of several rounds, N = 4, 64 x 64)
         const double alone = rounds == 1 && c.bm == 128 ? 1.025 : 1.0;
-        p.time += alone * (double)rounds * (c.bm == 64 ? 2.0 : 1.0) * 2.0 * c.bm * c.bn * KRED / (614e9 * c.eff * CONV_SUSTAINED) + 3e-6;
+        p.time += alone * (double)rounds * (c.bm == 64 ? 4.0 : 1.0) * 2.0 * c.bm * c.bn * KRED / (614e9 * c.eff * CONV_SUSTAINED) + 3e-6;
         p0 = p1;
     }
     if (p0 >= P) return p;
@@ -584,7 +586,10 @@ static ConvPlan plan_conv(int CO, int P, int KRED) {
             const double wg = 2.0 * c.bm * c.bn * KRED / (614e9 * c.eff * CONV_SUSTAINED) / sp;     // one workgroup's MFMA time (256 flop/clk at 2.4 GHz)
             const double planes = sp > 1 ? (double)t * sp * c.bm * c.bn * 8.0 / 3e12 + 8e-6 : 0.0;
             const double alone = per_cu == 1 && c.bm == 128 ? 1.025 : 1.0;      // one wave per SIMD, as for a single whole round
-            const double time = alone * wg * (double)per_cu / busy + planes;
+            // (2-wave workgroups: two to four on a CU put two waves on its busiest SIMD, see above; measured at a
+            // reduction of 576: 43 us for up to one per CU, 77 to 85 us for two to four)
+            const double units = waves == 2 ? (per_cu == 1 ? 2.0 : per_cu <= 4 ? 4.0 : (double)per_cu) : (double)per_cu / busy;
+            const double time = alone * wg * units + planes;
             if (time < best_time) { best_time = time; tail = ConvStage{c.cfg, p0, P, sp}; }
         }
     }
