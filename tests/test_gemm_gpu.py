@@ -397,3 +397,46 @@ def test_thin_and_very_wide_product(torch_cuda):
     cols = torch.cat([torch.arange(0, 4096), torch.arange(N - 4096, N), torch.randint(0, N, (4096,), generator=g)]).cuda()
     assert torch.equal(C[:, cols].double(), A.double() @ B[:, cols].double())
     assert not torch.isnan(C).any()
+
+
+@pytest.mark.parametrize("shape", [(32, 100352, 64), (32, 100352, 1152), (96, 40000, 64), (128, 30000, 96), (64, 65536, 288),
+                                   (96, 65536, 4096), (4096, 4096, 256), (5120, 4096, 512), (114688, 128, 288), (131072, 128, 288)])
+def test_library_choice_for_thin_wide_and_many_tile_products(oracle, torch_cuda, shape):
+    """Shapes whose automatic route differs from the square products': a few rows under a very wide output
+    (one-wave tiles; a stream of C under a short reduction), 128 x 128 tiles that would be a quarter empty,
+    four and five 128 x 128 tiles per CU (launched with LDS that limits the workgroups per CU), a rest that
+    is not split under a short reduction.  Sampled columns or rows against the oracle, and the whole result
+    against a second run (same bits) and for NaNs left behind."""
+    torch = torch_cuda
+    M, N, K = shape
+    L = t2sp_amd.lib()
+    A = t2sp_amd.fill_uniform(torch.empty(M, K, device="cuda"), 31)
+    B = t2sp_amd.fill_uniform(torch.empty(K, N, device="cuda"), 32)
+    nbytes = L.t2sp_sgemm_workspace_bytes(M, N, K)
+    ws = torch.empty(max(nbytes // 4, 4), device="cuda")
+    outs = []
+    for _ in range(2):
+        C = torch.full((M, N), float("nan"), device="cuda")
+        assert L.t2sp_sgemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, ws.data_ptr(),
+                                ctypes.c_size_t(nbytes), None) == 0
+        torch.cuda.synchronize()
+        outs.append(C)
+    C = outs[0]
+    assert torch.equal(C, outs[1])
+    assert not torch.isnan(C).any()
+    rng = np.random.default_rng(3)
+    if N >= M:
+        cols = np.unique(np.concatenate([[0, 1, N // 2, N - 2, N - 1], rng.integers(0, N, 59)]))
+        ci = torch.as_tensor(cols, device="cuda")
+        rows = np.arange(M) if M <= 128 else np.unique(np.concatenate([[0, M - 1], rng.integers(0, M, 62)]))
+        ri = torch.as_tensor(rows, device="cuda")
+        ref = oracle.gemm(A[ri].cpu().numpy(), np.ascontiguousarray(B[:, ci].cpu().numpy()))
+        got = C[ri][:, ci].cpu().numpy()
+    else:
+        rows = np.unique(np.concatenate([[0, 1, M // 2, M - 129, M - 2, M - 1], rng.integers(0, M, 58)]))
+        ri = torch.as_tensor(rows, device="cuda")
+        ref = oracle.gemm(A[ri].cpu().numpy(), B.cpu().numpy())
+        got = C[ri].cpu().numpy()
+    err, mx = rel_fro(got, ref)
+    print("shape %s rel_fro %.3e max_abs %.3e" % (shape, err, mx))
+    assert err <= TOL
