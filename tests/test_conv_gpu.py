@@ -357,3 +357,22 @@ def test_large_host_buffers_run_in_image_panels(oracle):
     ref = oracle.conv(np.ascontiguousarray(In), np.ascontiguousarray(Wn), co_range=(cos.start, cos.stop))[:, cos]
     got = O[[0, N - 1]][:, cos].transpose(0, 1, 3, 2)
     assert rel_fro(got, ref)[0] <= TOL
+
+
+@pytest.mark.parametrize("shape", [(2, 64, 64, 28, 28, 1), (4, 32, 64, 32, 32, 3), (1, 64, 64, 112, 112, 3), (2, 16, 32, 64, 64, 3),
+                                   (8, 64, 48, 30, 30, 1), (24, 32, 64, 64, 64, 3), (40, 64, 64, 56, 56, 1), (3, 128, 128, 28, 28, 3)])
+def test_library_choice_for_few_output_channels_exact(shape):
+    """Layers of up to 64 output channels, where the automatic choice takes the one-launch 16 x 16 form up to
+    two or three 64 x 128 tiles per CU whatever the reduction length (1 x 1 kernels included) and the staged
+    plan of LDS tiles beyond, and a 128-channel layer at the boundary between the two.  Integer data: exact
+    against the float64 convolution, whichever kernel runs; the same bits twice."""
+    import torch
+    N, CI, CO, OH, OW, KH = shape
+    g = torch.Generator().manual_seed(N * CI + CO)
+    I = torch.randint(-2, 3, (N, CI, OH + KH - 1, OW + KH - 1), generator=g).float().numpy()
+    W = torch.randint(-2, 3, (CO, CI, KH, KH), generator=g).float().numpy()
+    want = torch.nn.functional.conv2d(torch.from_numpy(I).double(), torch.from_numpy(W).double()).numpy()
+    got = run(I, W, cfg=0)
+    assert (got == want).all()
+    assert (run(I, W, cfg=0) == got).all()
+    assert (run(I, W, cfg=3) == want).all()
