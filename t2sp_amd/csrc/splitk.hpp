@@ -36,6 +36,32 @@ __device__ __forceinline__ void store_partial(const Accum<Cfg> &acc, float *scra
     });
 }
 
+// sum (+)= p[s * stride] + ... + p[(s + N - 1) * stride], added in ascending order; the N loads are issued together,
+// so the sum waits for memory once per call and not once per plane.  FIRST: the sum starts with the first value.
+template <int N, bool FIRST>
+__device__ __forceinline__ void add_planes(v4f &sum, const float *p, size_t stride, int s) {
+    v4f v[N];
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] = *reinterpret_cast<const v4f *>(p + (size_t)(s + i) * stride);
+#pragma unroll
+    for (int i = 0; i < N; i++) sum = (FIRST && i == 0) ? v[0] : sum + v[i];
+}
+// The S planes of one group of four values, in ascending order, up to eight loads in flight.
+__device__ __forceinline__ v4f sum_planes(const float *q, size_t stride, int S) {
+    v4f sum = {0.f, 0.f, 0.f, 0.f};
+    const int n = S;
+    int s = 0;
+    if (n >= 8) { add_planes<8, true>(sum, q, stride, 0); s = 8; }
+    else if (n >= 4) { add_planes<4, true>(sum, q, stride, 0); s = 4; }
+    else if (n >= 2) { add_planes<2, true>(sum, q, stride, 0); s = 2; }
+    else if (n >= 1) { add_planes<1, true>(sum, q, stride, 0); s = 1; }
+    for (; n - s >= 8; s += 8) add_planes<8, false>(sum, q, stride, s);
+    if (n - s >= 4) { add_planes<4, false>(sum, q, stride, s); s += 4; }
+    if (n - s >= 2) { add_planes<2, false>(sum, q, stride, s); s += 2; }
+    if (n - s >= 1) add_planes<1, false>(sum, q, stride, s);
+    return sum;
+}
+
 // OutMap: __device__ void store(int row, int col, v4f v) const — writes D[row][col..col+3]
 // (ALONG_COLS) or D[row..row+3][col] (!ALONG_COLS), ignoring out-of-range positions.
 template <bool ALONG_COLS, class OutMap>
@@ -45,17 +71,7 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *scratch
     const size_t groups = plane / 4;
     for (size_t g = (size_t)blockIdx.x * blockDim.x + threadIdx.x; g < groups;
          g += (size_t)gridDim.x * blockDim.x) {
-        const float *p = scratch + g * 4;
-        v4f sum = *reinterpret_cast<const v4f *>(p);
-        int s = 1;
-        for (; s + 3 < S; s += 4) {   // four loads in flight; the additions stay in ascending order
-            const v4f a = *reinterpret_cast<const v4f *>(p + (size_t)s * plane);
-            const v4f b = *reinterpret_cast<const v4f *>(p + (size_t)(s + 1) * plane);
-            const v4f c = *reinterpret_cast<const v4f *>(p + (size_t)(s + 2) * plane);
-            const v4f d = *reinterpret_cast<const v4f *>(p + (size_t)(s + 3) * plane);
-            sum = (((sum + a) + b) + c) + d;
-        }
-        for (; s < S; s++) sum += *reinterpret_cast<const v4f *>(p + (size_t)s * plane);
+        const v4f sum = sum_planes(scratch + g * 4, plane, S);
         int row, col;
         if (ALONG_COLS) {
             row = (int)(g / (Np / 4));

@@ -209,17 +209,7 @@ __global__ void __launch_bounds__(256) ssyrk_split_sum_kernel(const SyrkArgs g) 
     const size_t plane = (size_t)g.tile_count * B * B;
     const size_t groups = plane / 4;
     for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < groups; q += (size_t)gridDim.x * blockDim.x) {
-        const float *p = g.scratch + q * 4;
-        v4f sum = *reinterpret_cast<const v4f *>(p);
-        int s = 1;
-        for (; s + 3 < g.splits; s += 4) {   // four loads in flight; the additions stay in ascending order
-            const v4f a = *reinterpret_cast<const v4f *>(p + (size_t)s * plane);
-            const v4f b = *reinterpret_cast<const v4f *>(p + (size_t)(s + 1) * plane);
-            const v4f c = *reinterpret_cast<const v4f *>(p + (size_t)(s + 2) * plane);
-            const v4f d = *reinterpret_cast<const v4f *>(p + (size_t)(s + 3) * plane);
-            sum = (((sum + a) + b) + c) + d;
-        }
-        for (; s < g.splits; s++) sum += *reinterpret_cast<const v4f *>(p + (size_t)s * plane);
+        const v4f sum = sum_planes(g.scratch + q * 4, plane, g.splits);
         const int colg = (int)(q / (B / 4)), row = (int)(q % (B / 4)) * 4;
         const int t = colg / B, col = colg - t * B;
         int tm, tn;
