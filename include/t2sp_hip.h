@@ -138,9 +138,10 @@ int t2sp_sgbmv3_f32_tiled(float alpha, float beta, const float *A, const float *
  * stored in row-major A (elements above the diagonal are never read).  O is flat, or the
  * reference's 3-D Out(kkk, kk, k) with element strides strides3
  * (t2s/tests/performance/symv/symv-run-fpga.cpp:79).  HBM-bound: the triangle is read once.  With
- * N % 4 == 0, lda % 4 == 0, 16-byte aligned A and x and a workspace of
- * t2sp_ssymv_workspace_bytes(N) it runs on 128 x 128 blocks; otherwise (workspace may be NULL) a
- * slow kernel without requirements.  Replaces the device side of the reference's SYMV pipeline
+ * a workspace of t2sp_ssymv_workspace_bytes(N) it runs on 128 x 128 blocks (128-bit loads when
+ * N % 4 == 0, lda % 4 == 0 and A and x are 16-byte aligned, 32-bit loads at about 0.8 of that rate
+ * otherwise); without one (workspace may be NULL) a slow kernel, a tenth of the rate.  Replaces the
+ * device side of the reference's SYMV pipeline
  * (t2s/tests/performance/symv/symv.cpp:57-72). */
 size_t t2sp_ssymv_workspace_bytes(int N);
 int t2sp_ssymv_f32(float alpha, float beta, const float *A, const float *x, const float *y, float *O, int N,

@@ -58,7 +58,19 @@ __global__ void __launch_bounds__(64 * GBMV_ROWS_PER_WG) sgbmv3_kernel(const Gbm
                 s3 += av[3] * xv[3];
             }
         } else {
-            for (int k = lane; k < g.K; k += 64) s0 += a[k] * x[k];
+            // 32-bit loads, lanes side by side, eight per lane in flight
+            float t0 = 0.f, t1 = 0.f, t2 = 0.f, t3 = 0.f;
+            int k = lane;
+            for (; k + 448 < g.K; k += 512) {
+                const float a0 = __builtin_nontemporal_load(a + k), a1 = __builtin_nontemporal_load(a + k + 64);
+                const float a2 = __builtin_nontemporal_load(a + k + 128), a3 = __builtin_nontemporal_load(a + k + 192);
+                const float a4 = __builtin_nontemporal_load(a + k + 256), a5 = __builtin_nontemporal_load(a + k + 320);
+                const float a6 = __builtin_nontemporal_load(a + k + 384), a7 = __builtin_nontemporal_load(a + k + 448);
+                s0 += a0 * x[k];       s1 += a1 * x[k + 64];  s2 += a2 * x[k + 128]; s3 += a3 * x[k + 192];
+                t0 += a4 * x[k + 256]; t1 += a5 * x[k + 320]; t2 += a6 * x[k + 384]; t3 += a7 * x[k + 448];
+            }
+            for (; k < g.K; k += 64) s0 += a[k] * x[k];
+            s0 += t0; s1 += t1; s2 += t2; s3 += t3;
         }
         const float z = gbmv_wave_sum((s0 + s1) + (s2 + s3));
         if (lane == 0) {

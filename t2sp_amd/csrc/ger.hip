@@ -40,28 +40,42 @@ __device__ __forceinline__ float ger_value(float a, float x, float y) {
     return a + p;
 }
 
-template <bool VEC>
 __global__ void __launch_bounds__(256) sger_kernel(const GerArgs g) {
-    const int kq = (g.K + 3) / 4;                       // groups of four k per row
+    const int kq = g.K / 4;                             // groups of four k per row
     const int64_t total = (int64_t)g.I * kq;
     for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
         const int i = (int)(t / kq), k = (int)(t - (int64_t)i * kq) * 4;
         const float xi = g.x[i];
-        if (VEC) {
-            // A is read once and O written once: both go past the caches as streams (no reuse to keep them for)
-            const ger_v4f a = __builtin_nontemporal_load(reinterpret_cast<const ger_v4f *>(g.A + (int64_t)i * g.lda + k));
-            const ger_v4f y = *reinterpret_cast<const ger_v4f *>(g.y + k);
-            ger_v4f o;
+        // A is read once and O written once: both go past the caches as streams (no reuse to keep them for)
+        const ger_v4f a = __builtin_nontemporal_load(reinterpret_cast<const ger_v4f *>(g.A + (int64_t)i * g.lda + k));
+        const ger_v4f y = *reinterpret_cast<const ger_v4f *>(g.y + k);
+        ger_v4f o;
 #pragma unroll
-            for (int e = 0; e < 4; e++) o[e] = ger_value(a[e], xi, y[e]);
+        for (int e = 0; e < 4; e++) o[e] = ger_value(a[e], xi, y[e]);
+        float *dst = g.tiled ? g.O + ger_tiled_offset(g, i, k) : g.O + (int64_t)i * g.ldo + k;
+        __builtin_nontemporal_store(o, reinterpret_cast<ger_v4f *>(dst));
+    }
+}
+
+// Sizes, leading dimensions or addresses that rule out 128-bit accesses: 32-bit accesses, lanes side by side
+// along k (whole cache lines per load and store all the same); a thread takes GER_ROWS rows of its column so
+// that as many loads are in flight per lane as bytes would be with the wide form.
+constexpr int GER_ROWS = 8;
+__global__ void __launch_bounds__(256) sger_element_kernel(const GerArgs g) {
+    const int k = (int)(blockIdx.x * blockDim.x + threadIdx.x);
+    if (k >= g.K) return;
+    const float yk = g.y[k];
+    for (int64_t i0 = (int64_t)blockIdx.y * GER_ROWS; i0 < g.I; i0 += (int64_t)gridDim.y * GER_ROWS) {
+        float a[GER_ROWS];
+#pragma unroll
+        for (int r = 0; r < GER_ROWS; r++)
+            a[r] = i0 + r < g.I ? __builtin_nontemporal_load(g.A + (i0 + r) * g.lda + k) : 0.f;
+#pragma unroll
+        for (int r = 0; r < GER_ROWS; r++) {
+            if (i0 + r >= g.I) break;
+            const int i = (int)(i0 + r);
             float *dst = g.tiled ? g.O + ger_tiled_offset(g, i, k) : g.O + (int64_t)i * g.ldo + k;
-            __builtin_nontemporal_store(o, reinterpret_cast<ger_v4f *>(dst));
-        } else {
-            for (int e = 0; e < 4 && k + e < g.K; e++) {
-                const float o = ger_value(g.A[(int64_t)i * g.lda + k + e], xi, g.y[k + e]);
-                if (g.tiled) g.O[ger_tiled_offset(g, i, k + e)] = o;
-                else g.O[(int64_t)i * g.ldo + k + e] = o;
-            }
+            __builtin_nontemporal_store(ger_value(a[r], g.x[i], yk), dst);
         }
     }
 }
@@ -78,8 +92,13 @@ static int launch_ger(const GerArgs &g, hipStream_t stream) {
     // One group of four per thread measures best (6.1 against 5.7 TB/s for a plain copy of this size with a
     // grid-stride loop over 64 workgroups per CU); the loop only serves sizes beyond the grid limit.
     if (blocks > (1 << 24)) blocks = 1 << 24;
-    auto kern = (in_vec && out_vec) ? sger_kernel<true> : sger_kernel<false>;
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), 0, stream, g);
+    if (in_vec && out_vec) {
+        hipLaunchKernelGGL(sger_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, g);
+    } else {
+        const int64_t row_groups = ((int64_t)g.I + GER_ROWS - 1) / GER_ROWS;
+        const unsigned bx = (unsigned)((g.K + 255) / 256), by = (unsigned)(row_groups < 65535 ? row_groups : 65535);
+        hipLaunchKernelGGL(sger_element_kernel, dim3(bx, by), dim3(256), 0, stream, g);
+    }
     return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
 }
 

@@ -44,6 +44,10 @@ __device__ __forceinline__ void symv_block(int t, int &bi, int &bj) {
     bj = t - r * (r + 1) / 2;
 }
 
+// VEC: N and lda are multiples of 4 and A and x are 16-byte aligned, so a lane takes four adjacent columns with
+// one 128-bit load.  Otherwise a lane takes columns lane, lane + 32, lane + 64 and lane + 96 of the block with
+// 32-bit loads (lanes side by side: whole cache lines per load all the same), each guarded against N.
+template <bool VEC>
 __global__ void __launch_bounds__(SYMV_THREADS) ssymv_block_kernel(const SymvArgs g) {
     __shared__ float row_part[SYMV_B][33];           // [row][lane], padded against bank conflicts
     __shared__ float col_part[8][SYMV_B];            // [row group][column]
@@ -51,17 +55,30 @@ __global__ void __launch_bounds__(SYMV_THREADS) ssymv_block_kernel(const SymvArg
     symv_block((int)blockIdx.x, bi, bj);
     const bool diag = bi == bj;
     const int lane = threadIdx.x & 31, rg = threadIdx.x >> 5;
-    const int row0 = bi * SYMV_B, col = bj * SYMV_B + lane * 4;
-    const bool col_in = col < g.N;                   // N % 4 == 0: a group of four is in or out
+    const int row0 = bi * SYMV_B, col = bj * SYMV_B + (VEC ? lane * 4 : lane);
+    constexpr int CS = VEC ? 1 : 32;                 // distance between a lane's four columns
+    const bool col_in = col < g.N;                   // VEC: N % 4 == 0, a group of four is in or out
 
     symv_v4f a[SYMV_STEPS];
+    symv_v4f xc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < SYMV_STEPS; s++) {
         const int row = row0 + s * 8 + rg;
-        a[s] = (col_in && row < g.N) ? __builtin_nontemporal_load(reinterpret_cast<const symv_v4f *>(g.A + (int64_t)row * g.lda + col))
-                                     : symv_v4f{0.f, 0.f, 0.f, 0.f};          // the triangle is read once: a stream
+        if (VEC) {
+            a[s] = (col_in && row < g.N) ? __builtin_nontemporal_load(reinterpret_cast<const symv_v4f *>(g.A + (int64_t)row * g.lda + col))
+                                         : symv_v4f{0.f, 0.f, 0.f, 0.f};          // the triangle is read once: a stream
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                a[s][e] = (col + e * CS < g.N && row < g.N) ? __builtin_nontemporal_load(g.A + (int64_t)row * g.lda + col + e * CS) : 0.f;
+        }
     }
-    const symv_v4f xc = col_in ? *reinterpret_cast<const symv_v4f *>(g.x + col) : symv_v4f{0.f, 0.f, 0.f, 0.f};
+    if (VEC) {
+        if (col_in) xc = *reinterpret_cast<const symv_v4f *>(g.x + col);
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) xc[e] = col + e * CS < g.N ? g.x[col + e * CS] : 0.f;
+    }
     symv_v4f cacc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < SYMV_STEPS; s++) {
@@ -71,8 +88,8 @@ __global__ void __launch_bounds__(SYMV_THREADS) ssymv_block_kernel(const SymvArg
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             // on a diagonal block, elements above the diagonal are not part of the input
-            const bool low = !diag || col + e <= row;
-            const bool strict = !diag || col + e < row;
+            const bool low = !diag || col + e * CS <= row;
+            const bool strict = !diag || col + e * CS < row;
             const float v = low ? a[s][e] : 0.f;
             racc += v * xc[e];
             cacc[e] += (strict ? v : 0.f) * xr;
@@ -80,7 +97,7 @@ __global__ void __launch_bounds__(SYMV_THREADS) ssymv_block_kernel(const SymvArg
         row_part[s * 8 + rg][lane] = racc;
     }
 #pragma unroll
-    for (int e = 0; e < 4; e++) col_part[rg][lane * 4 + e] = cacc[e];
+    for (int e = 0; e < 4; e++) col_part[rg][VEC ? lane * 4 + e : lane + e * CS] = cacc[e];
     __syncthreads();
     if (threadIdx.x < SYMV_B) {
         const int t = threadIdx.x;
@@ -122,8 +139,8 @@ __global__ void __launch_bounds__(SYMV_B * SYMV_SUM_WAYS) ssymv_sum_kernel(const
     g.O[off] = g.alpha * sum + g.beta * g.y[k];
 }
 
-// Any N, lda and alignment: one wave per output, a strided walk down the column for the part
-// below the diagonal.  Correct everywhere, slow; the block kernels cover the shapes that matter.
+// Without a workspace for the partial vectors: one wave per output, a strided walk down the column for
+// the part below the diagonal.  Correct everywhere, slow (a tenth of the block kernels' rate).
 __global__ void __launch_bounds__(256) ssymv_scalar_kernel(const SymvArgs g) {
     const int lane = threadIdx.x & 63;
     const int k = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -150,13 +167,13 @@ static int launch_symv(SymvArgs g, size_t workspace_bytes, hipStream_t stream) {
     if (g.N <= 0 || g.t_kkk <= 0 || g.t_kk <= 0) return T2SP_ERR_SHAPE;
     g.nb = (g.N + SYMV_B - 1) / SYMV_B;
     if (g.nb > 2048) return T2SP_ERR_SHAPE;          // keeps the block count within int and the sqrt exact enough
-    const bool blocks_ok = symv_vec_ok(g) && g.W && workspace_bytes >= t2sp_ssymv_workspace_bytes(g.N);
+    const bool blocks_ok = g.W && workspace_bytes >= t2sp_ssymv_workspace_bytes(g.N);
     if (!blocks_ok) {
         hipLaunchKernelGGL(ssymv_scalar_kernel, dim3((unsigned)((g.N + 3) / 4)), dim3(256), 0, stream, g);
         return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
     }
     const int tri = g.nb * (g.nb + 1) / 2;
-    hipLaunchKernelGGL(ssymv_block_kernel, dim3((unsigned)tri), dim3(SYMV_THREADS), 0, stream, g);
+    hipLaunchKernelGGL(symv_vec_ok(g) ? ssymv_block_kernel<true> : ssymv_block_kernel<false>, dim3((unsigned)tri), dim3(SYMV_THREADS), 0, stream, g);
     hipLaunchKernelGGL(ssymv_sum_kernel, dim3((unsigned)g.nb), dim3(SYMV_B * SYMV_SUM_WAYS), 0, stream, g);
     return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
 }

@@ -75,6 +75,21 @@ def test_gbmv3_large_on_device(oracle):
     assert rel_fro(O.cpu().numpy(), want)[0] <= TOL
 
 
+@pytest.mark.parametrize("I,K,lda", [(30001, 1023, 1023), (30000, 1022, 1024), (999, 4100 + 3, 4104)])
+def test_gbmv3_odd_sizes_on_device(oracle, I, K, lda):
+    """Band widths and leading dimensions that rule out 128-bit loads: 32-bit loads, eight per lane in flight."""
+    import torch
+    L = t2sp_amd.lib()
+    A = t2sp_amd.fill_uniform(torch.empty(I, lda, device="cuda"), 124)
+    x = t2sp_amd.fill_uniform(torch.empty(I + K - 1, device="cuda"), 125)
+    y = t2sp_amd.fill_uniform(torch.empty(I, device="cuda"), 126)
+    O = torch.full((I,), float("nan"), device="cuda")
+    assert L.t2sp_sgbmv3_f32(0.75, 1.25, A.data_ptr(), x.data_ptr(), y.data_ptr(), O.data_ptr(), I, K, lda, None) == 0
+    torch.cuda.synchronize()
+    want = oracle.gbmv3(np.ascontiguousarray(A[:, :K].cpu().numpy()), x.cpu().numpy(), y.cpu().numpy(), 0.75, 1.25)
+    assert rel_fro(O.cpu().numpy(), want)[0] <= TOL
+
+
 def test_gbmv3_error_codes():
     A = np.zeros((8, 16), np.float32)
     with pytest.raises(t2sp_amd.T2spError) as e:       # x must span I + K - 1 = 23
@@ -161,6 +176,30 @@ def test_symv_full_size_on_device_and_without_workspace(oracle):
     torch.cuda.synchronize()
     want2 = oracle.symv(A[:M, :M].cpu().numpy(), x[:M].cpu().numpy(), y[:M].cpu().numpy(), 0.5, 2.0)
     assert rel_fro(O2.cpu().numpy(), want2)[0] <= TOL
+
+
+@pytest.mark.parametrize("N,lda", [(4099, 4099), (4098, 4100), (4097, 4104), (129, 131)])
+def test_symv_odd_sizes_take_the_block_kernels(oracle, N, lda):
+    """N or lda not a multiple of 4: with a workspace the block kernels run all the same, on 32-bit loads
+    (a lane's four columns 32 apart), every element guarded against N.  Elements above the diagonal are NaN:
+    they are loaded on diagonal blocks and must not reach a sum."""
+    import torch
+    L = t2sp_amd.lib()
+    A = t2sp_amd.fill_uniform(torch.empty(N, lda, device="cuda"), 146)
+    iu = torch.triu_indices(N, N, 1, device="cuda")
+    A[iu[0], iu[1]] = float("nan")
+    x = t2sp_amd.fill_uniform(torch.empty(N, device="cuda"), 147)
+    y = t2sp_amd.fill_uniform(torch.empty(N, device="cuda"), 148)
+    O = torch.full((N,), float("nan"), device="cuda")
+    nbytes = L.t2sp_ssymv_workspace_bytes(N)
+    ws = torch.empty(nbytes // 4, device="cuda")
+    assert L.t2sp_ssymv_f32(0.5, 2.0, A.data_ptr(), x.data_ptr(), y.data_ptr(), O.data_ptr(), N, lda, ws.data_ptr(),
+                            nbytes, None) == 0
+    torch.cuda.synchronize()
+    want = oracle.symv(np.ascontiguousarray(A[:, :N].cpu().numpy()), x.cpu().numpy(), y.cpu().numpy(), 0.5, 2.0)
+    got = O.cpu().numpy()
+    assert np.isfinite(got).all()
+    assert rel_fro(got, want)[0] <= TOL
 
 
 def test_symv_error_codes():

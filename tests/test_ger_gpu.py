@@ -57,6 +57,23 @@ def test_full_size_on_device(oracle):
     assert (O.cpu().numpy() == want).all()
 
 
+@pytest.mark.parametrize("I,K,lda", [(2049, 4099, 4099), (2050, 4098, 4100), (70001, 37, 37)])
+def test_odd_sizes_on_device_bit_exact(oracle, I, K, lda):
+    """Sizes and leading dimensions that rule out 128-bit accesses take the kernel of 32-bit accesses (eight rows
+    per thread, the last group of rows short); whole result against the oracle, padding columns untouched."""
+    import torch
+    L = t2sp_amd.lib()
+    A = t2sp_amd.fill_uniform(torch.empty(I, lda, device="cuda"), 104)
+    x = t2sp_amd.fill_uniform(torch.empty(I, device="cuda"), 105)
+    y = t2sp_amd.fill_uniform(torch.empty(K, device="cuda"), 106)
+    O = torch.full((I, lda), float("nan"), device="cuda")
+    assert L.t2sp_sger_f32(A.data_ptr(), x.data_ptr(), y.data_ptr(), O.data_ptr(), I, K, lda, lda, None) == 0
+    torch.cuda.synchronize()
+    want = oracle.ger(np.ascontiguousarray(A[:, :K].cpu().numpy()), x.cpu().numpy(), y.cpu().numpy())
+    assert (O[:, :K].cpu().numpy() == want).all()
+    assert torch.isnan(O[:, K:]).all()
+
+
 def test_error_codes():
     A = np.zeros((8, 16), np.float32)
     with pytest.raises(t2sp_amd.T2spError) as e:
