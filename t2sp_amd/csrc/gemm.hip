@@ -1217,9 +1217,50 @@ static int launch_d16_at(GemmArgs g, hipStream_t stream) {
     return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
 }
 
+// C[i][j..j+3] += alpha * sum_{k0 <= k < K} A(i, k) * B(k, j..j+3): the last 4, 8 or 12 steps of a reduction whose
+// length is not a multiple of 16, added to a product that a kernel of 16-k steps has computed over [0, k0).
+// A(i, k) = A[i * a_i + k * a_k]; B(k, j) = B[k * b_k + j * b_j].  One thread per four columns of one row.
+__global__ void __launch_bounds__(256) gemm_ktail_kernel(const float *A, int64_t a_i, int64_t a_k, const float *B, int64_t b_k,
+                                                         int64_t b_j, float *C, int64_t ldc, int M, int N, int k0, int K,
+                                                         float alpha) {
+    const int nq = N / 4;
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= (int64_t)M * nq) return;
+    const int i = (int)(t / nq), j = (int)(t - (int64_t)i * nq) * 4;
+    v4f sum = {0.f, 0.f, 0.f, 0.f};
+    for (int k = k0; k < K; k++) {
+        const float a = A[i * a_i + k * a_k];
+        v4f b;
+        if (b_j == 1) b = *reinterpret_cast<const v4f *>(B + k * b_k + j);
+        else b = v4f{B[k * b_k + j * b_j], B[k * b_k + (j + 1) * b_j], B[k * b_k + (j + 2) * b_j], B[k * b_k + (j + 3) * b_j]};
+        sum += a * b;
+    }
+    v4f *c = reinterpret_cast<v4f *>(C + (int64_t)i * ldc + j);
+    *c = *c + alpha * sum;
+}
+
 static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *workspace = nullptr,
                     size_t workspace_bytes = 0) {
     if (g.M <= 0 || g.N <= 0 || g.K <= 0) return T2SP_ERR_SHAPE;
+    // Small outputs whose reduction is not a multiple of 16: the one-launch kernels step 16 k at a time, and without
+    // them such a product falls to a few LDS tiles with a split reduction (256 x 256 x 16388: 78 us against 25 us
+    // at K = 16384).  The product over the first K - K % 16 steps goes the usual way; one more pass adds the rest.
+    if (cfg == T2SP_CFG_AUTO && g.K % 16 != 0 && g.K % 4 == 0 && g.K > 64 && !g.tiled && g.N % 4 == 0 && g.ldc % 4 == 0 &&
+        ((uintptr_t)g.C % 16 == 0) && (int64_t)g.M * g.N <= (1 << 21)) {
+        GemmArgs h = g;
+        h.K = g.K - g.K % 16;
+        // (the direct kernel of 8-k steps takes its shapes as they are: 1000^3 20.9 us, 23.8 this way)
+        const bool direct = !bt && !g.at && !g.scale && g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && gemm_direct_ok(g, false);
+        if (!direct && (g.at ? gemm_d16_at_ok(h) : bt ? gemm_d16_bt_ok(h) : gemm_d16_ok(h))) {
+            const int rc = dispatch(h, cfg, bt, stream, workspace, workspace_bytes);
+            if (rc != T2SP_OK) return rc;
+            const int64_t groups = (int64_t)g.M * (g.N / 4);
+            hipLaunchKernelGGL(gemm_ktail_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, stream, g.A,
+                               g.at ? (int64_t)1 : g.lda, g.at ? g.lda : (int64_t)1, g.B, bt ? (int64_t)1 : g.ldb,
+                               bt ? g.ldb : (int64_t)1, g.C, g.ldc, g.M, g.N, h.K, g.K, g.scale ? g.alpha : 1.f);
+            return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+        }
+    }
     if (g.at) {
         // A^T * B with both operands as they lie (the caller has checked the alignment the 128-bit
         // loads need).  Any K: k is the row index of both operands.
@@ -1409,8 +1450,12 @@ extern "C" size_t t2sp_sgemm_workspace_bytes(int M, int N, int K) {
     if (!gemm_extents_ok(M, N, K)) return 0;
     if (K % 4 == 0 && N % 4 == 0) {
         const size_t tiled = t2sp::plan_gemm(M, N, K).scratch_bytes;
-        const size_t one_launch = t2sp::plan_gemm_d16_split(M, N, K, t2sp::plan_gemm_d16(M, N)).scratch_bytes;
-        return tiled > one_launch ? tiled : one_launch;
+        // (a reduction that is not a multiple of 16 may run as the product over its first K - K % 16 steps + a pass for the rest)
+        const int k16 = K > 64 ? K - K % 16 : K;
+        const size_t one_launch = t2sp::plan_gemm_d16_split(M, N, k16, t2sp::plan_gemm_d16(M, N)).scratch_bytes;
+        const size_t tiled16 = k16 != K ? t2sp::plan_gemm(M, N, k16).scratch_bytes : 0;
+        const size_t most = tiled > one_launch ? tiled : one_launch;
+        return most > tiled16 ? most : tiled16;
     }
     // padded copies of the operands, then the planes for the padded product
     return t2sp::gemm_pad_bytes(M, N, K, false) +
@@ -1458,7 +1503,12 @@ extern "C" size_t t2sp_sgemm_ex_workspace_bytes(int transa, int M, int N, int K)
         const size_t as_it_lies = t2sp::plan_gemm(M, n4, k4, true).scratch_bytes;
         if (as_it_lies > tiled) tiled = as_it_lies;
     }
-    const size_t one_launch = t2sp::plan_gemm_d16_split(M, n4, k4, t2sp::plan_gemm_d16(M, n4)).scratch_bytes;
+    const int k16 = k4 > 64 ? k4 - k4 % 16 : k4;     // (see t2sp_sgemm_workspace_bytes)
+    const size_t one_launch = t2sp::plan_gemm_d16_split(M, n4, k16, t2sp::plan_gemm_d16(M, n4)).scratch_bytes;
+    if (k16 != k4) {
+        const size_t tiled16 = t2sp::plan_gemm(M, n4, k16).scratch_bytes;
+        if (tiled16 > tiled) tiled = tiled16;
+    }
     return t2sp::round_up256(transa ? (size_t)M * K * sizeof(float) : 0) + pad + (tiled > one_launch ? tiled : one_launch);
 }
 

@@ -1,5 +1,7 @@
 """GPU parity tests of the BLAS-form SGEMM (include/blas-gemm.h): the `next` row that wraps the
 SGEMM path the way t2s/peppers/blas/level3/gemm/release/a10/blas-gemm.cpp does."""
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -306,3 +308,32 @@ def test_lds_tile_loaders_rows_far_apart(form, cfg):
     torch.cuda.synchronize()
     assert torch.equal(C.double(), want)
     del big
+
+
+@pytest.mark.parametrize("K", [68, 1000, 4104, 16388])
+@pytest.mark.parametrize("MN", [(256, 256), (512, 384), (132, 1000)])
+@pytest.mark.parametrize("form", ["NN", "NT", "TN"])
+def test_small_outputs_with_a_reduction_off_the_16_grid_exact(form, MN, K):
+    """Small outputs whose K is a multiple of 4 but not of 16: the product over the first K - K % 16 steps takes
+    the one-launch kernels (or their split over workgroups, with the workspace), and one more pass adds the
+    last 4, 8 or 12 steps.  All three operand layouts, alpha, beta and C in place.  Integer data: exact."""
+    import torch
+    M, N = MN
+    L = t2sp_amd.lib()
+    g = torch.Generator().manual_seed(K + M)
+    A = torch.randint(-2, 3, (M, K), generator=g).float().cuda()
+    B = torch.randint(-2, 3, (K, N), generator=g).float().cuda()
+    C0 = torch.randint(-4, 5, (M, N), generator=g).float().cuda()
+    want = 2.0 * (A.double() @ B.double()) - 3.0 * C0.double()
+    ta, tb = form[0] == "T", form[1] == "T"
+    Ad = A.t().contiguous() if ta else A
+    Bd = B.t().contiguous() if tb else B
+    nbytes = L.t2sp_sgemm_ex_workspace_bytes(int(ta), M, N, K)
+    ws = torch.empty(max(nbytes // 4, 4), device="cuda")
+    for w, nb in ((None, 0), (ws.data_ptr(), nbytes)):
+        C = C0.clone()
+        rc = L.t2sp_sgemm_ex_f32(int(ta), int(tb), M, N, K, 2.0, Ad.data_ptr(), M if ta else K, Bd.data_ptr(), K if tb else N, -3.0,
+                                 C.data_ptr(), N, C.data_ptr(), N, 0, w, ctypes.c_size_t(nb), None)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert torch.equal(C.double(), want)
