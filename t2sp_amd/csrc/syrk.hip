@@ -501,6 +501,10 @@ static SyrkTail plan_syrk_tail(int N, int K, int b, int bk) {
     return t;
 }
 
+static bool syrk_one_per_cu(int bm, int K, int64_t per_cu) {
+    return bm == 128 && (K >= 1024 || (K >= 512 && per_cu >= 3 && per_cu % 2 == 1));
+}
+
 template <class Cfg>
 static int launch_syrk(SyrkArgs g, hipStream_t stream, float *scratch = nullptr, size_t scratch_bytes = 0) {
     g.tiles = (g.N + Cfg::BM - 1) / Cfg::BM;
@@ -513,14 +517,20 @@ static int launch_syrk(SyrkArgs g, hipStream_t stream, float *scratch = nullptr,
         case SYRK_FLAT_FULL: kern = edge ? ssyrk_kernel<Cfg, true, SYRK_FLAT_FULL> : ssyrk_kernel<Cfg, false, SYRK_FLAT_FULL>; break;
         default: kern = edge ? ssyrk_kernel<Cfg, true, SYRK_FOLDED> : ssyrk_kernel<Cfg, false, SYRK_FOLDED>; break;
     }
-    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
-        return T2SP_ERR_LAUNCH;
     SyrkTail tail = plan_syrk_tail(g.N, g.K, Cfg::BM, Cfg::BK);
     if (!scratch || scratch_bytes < tail.scratch_bytes) tail.tail = 0;
     g.tile_first = 0;
     g.tile_count = (int)(tail.total - tail.tail);
     g.splits = 1;
-    hipLaunchKernelGGL(kern, dim3((unsigned)g.tile_count), dim3(Cfg::NTHREADS), smem, stream, g);
+    // Two workgroups of the 128 x 128 tiles fit a CU, and the dispatcher fills both slots of a CU at once: the
+    // last tiles then pile up on the CUs that came free first (820 tiles, K = 4096: 974 us, 767 with one per
+    // CU; 2080 tiles, K = 8192: 4200 / 3709 us).  One per CU (enough LDS asked for) costs 4 to 8 % at K = 256,
+    // where a second workgroup covers the other's start and end, and nothing from K = 1024 on.
+    const int64_t per_cu = ((int64_t)g.tile_count + machine().cus - 1) / machine().cus;
+    const size_t lds = lds_request(smem, syrk_one_per_cu(Cfg::BM, g.K, per_cu) ? 1 : 0);
+    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return T2SP_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3((unsigned)g.tile_count), dim3(Cfg::NTHREADS), lds, stream, g);
     if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
     if (tail.tail == 0) return T2SP_OK;
     g.tile_first = g.tile_count;
@@ -578,34 +588,48 @@ static int dispatch_syrk(SyrkArgs g, int trans, int cfg, float *workspace, size_
         workspace_bytes -= used;
     }
     if (cfg == T2SP_CFG_DIRECT16) return syrk_d16_ok(g) ? launch_syrk_d16(g, stream) : T2SP_ERR_SHAPE;
-    if (cfg == T2SP_CFG_AUTO && g.N <= SYRK_D16_MAX_N && g.K >= 64 && syrk_d16_ok(g)) return launch_syrk_d16(g, stream);
     const bool out_ok = g.mode == SYRK_FOLDED ||
                         (g.ldc % 4 == 0 && (uintptr_t)g.C % 16 == 0 &&
                          (!g.Cin || (g.ldcin % 4 == 0 && (uintptr_t)g.Cin % 16 == 0)));
     const bool vec_ok = out_ok && g.K % 4 == 0 && g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && g.lda < LOADER_MAX_LD;
+    // Estimated cost of each LDS tile size, in units of one output element's reduction at the 256 tile's rate: the
+    // number of rounds of 256 tiles (a last round whose reduction is split over the CUs counts 1/splits, plus a
+    // little for adding the planes) times the tile's area over the fraction of the 256 tile's rate that the size
+    // sustains (measured: 128 tiles one to a CU run at its rate, two to a CU, for short reductions, at 0.93 of it;
+    // 64 tiles at 0.78 for long reductions; their finer grain wastes less of an unsplit last round).
+    auto cost = [&](int b, double eff) {
+        const SyrkTail t = plan_syrk_tail(g.N, g.K, b, 16);
+        const bool split = t.tail > 0 && workspace && workspace_bytes >= t.scratch_bytes;
+        const int cus = machine().cus;
+        const double rounds = split ? (double)((t.total - t.tail) / cus) + 1.0 / t.splits + 0.03
+                                    : (double)((t.total + cus - 1) / cus);
+        return rounds * b * b / eff;
+    };
+    // (short reductions: a tile is mostly its start and its stores, and the small tiles lose the least to them:
+    // K = 256, N = 2560 ... 8192: 64 tiles 4 to 18 % ahead of the next choice)
+    const double c256 = cost(256, 1.0), c128 = cost(128, g.K >= 1024 ? 0.99 : 0.93),
+                 c64 = cost(64, g.K <= 256 ? 0.95 : g.K <= 512 ? 0.85 : 0.78);
+    if (cfg == T2SP_CFG_AUTO && g.N <= SYRK_D16_MAX_N && g.K >= 64 && syrk_d16_ok(g)) {
+        // The one-launch form up to N = 2048.  Above, it sustains about 122 TFLOP/s of the triangle's work whatever
+        // the shape, and the LDS tiles pass it where their rounds come out even (measured at N = 2560 ... 5120:
+        // K = 256 25 to 75 % ahead, K = 1024 up to 21 %; K = 4096: N = 4096 and 5120 15 and 11 % ahead, N = 2560
+        // 4 % behind): short reductions take the tiles, long ones whichever is estimated faster.
+        bool d16 = true;
+        if (g.N > 2048 && vec_ok) {
+            const double best = c256 <= c128 && c256 <= c64 ? c256 : (c128 <= c64 ? c128 : c64);
+            const double t_lds = best * 2.0 * g.K / (614e9 * 0.965), t_d16 = (double)g.N * (g.N + 1.0) * g.K / 122e12;
+            d16 = g.K > 1024 && t_d16 <= t_lds;
+        }
+        if (d16) return launch_syrk_d16(g, stream);
+    }
     if (cfg == T2SP_CFG_SCALAR || !vec_ok) {
         auto kern = g.mode == SYRK_FLAT_SYM ? ssyrk_scalar_kernel<SYRK_FLAT_SYM>
                     : g.mode == SYRK_FLAT_FULL ? ssyrk_scalar_kernel<SYRK_FLAT_FULL> : ssyrk_scalar_kernel<SYRK_FOLDED>;
         hipLaunchKernelGGL(kern, dim3((g.N + 255) / 256, g.N), dim3(256), 0, stream, g);
         return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
     }
-    if (cfg == T2SP_CFG_AUTO) {
-        // Estimated time of each tile size: the number of rounds of 256 tiles (a last round whose
-        // reduction is split over the CUs counts 1/splits, plus a little for adding the planes)
-        // times the work of one tile over the fraction of the MFMA rate that tile size sustains
-        // (measured: the 128 and 64 tiles run at about 0.93 and 0.78 of the 256 tile's rate, and
-        // their finer grain wastes less of an unsplit last round).
-        auto cost = [&](int b, double eff) {
-            const SyrkTail t = plan_syrk_tail(g.N, g.K, b, 16);
-            const bool split = t.tail > 0 && workspace && workspace_bytes >= t.scratch_bytes;
-            const int cus = machine().cus;
-            const double rounds = split ? (double)((t.total - t.tail) / cus) + 1.0 / t.splits + 0.03
-                                        : (double)((t.total + cus - 1) / cus);
-            return rounds * b * b / eff;
-        };
-        const double c256 = cost(256, 1.0), c128 = cost(128, 0.93), c64 = cost(64, 0.78);
+    if (cfg == T2SP_CFG_AUTO)
         cfg = (c256 <= c128 && c256 <= c64) ? T2SP_CFG_256x256 : (c128 <= c64 ? T2SP_CFG_128x128 : T2SP_CFG_64x128);
-    }
     switch (cfg) {
         case T2SP_CFG_256x256: return launch_syrk<SyrkL>(g, stream, workspace, workspace_bytes);
         case T2SP_CFG_128x128: return launch_syrk<SyrkM>(g, stream, workspace, workspace_bytes);
