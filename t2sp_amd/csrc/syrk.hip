@@ -455,7 +455,7 @@ static int launch_syrk_d16(const SyrkArgs &g, hipStream_t stream) {
     return T2SP_ERR_SHAPE;
 }
 
-constexpr int SYRK_D16_MAX_N = 5120;   // measured: from about 6144 on the LDS tiles' operand reuse wins
+constexpr int SYRK_D16_MAX_N = 5120;   // measured: from about 6144 on the LDS tiles' operand reuse wins at every K (see dispatch for 2048 < N)
 
 static bool syrk_d16_ok(const SyrkArgs &g) {
     return g.K % 16 == 0 && g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && (int64_t)g.N * g.lda < (1 << 30);
