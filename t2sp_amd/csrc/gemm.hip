@@ -1340,7 +1340,9 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         // (without it, and without room for the planes of the LDS tiles' split either, it still has more tiles to
         // spread over the CUs than they have)
         const bool lds_split = workspace && workspace_bytes >= plan_gemm(g.M, g.N, g.K).scratch_bytes;
-        const bool too_few = (int64_t)p.tiles_m * p.tiles_n < cus / 2 && g.K >= 4096 && !can_split && lds_split;
+        // (plain form only: the B^T form's LDS tiles do not split their reduction, and a few of them unsplit are far
+        // slower than the 16 x 16 form's many small tiles: 256 x 256 x 16384 485 against 114 us)
+        const bool too_few = !bt && (int64_t)p.tiles_m * p.tiles_n < cus / 2 && g.K >= 4096 && !can_split && lds_split;
         // (the plain form's grid is tiles_m x tiles_n: a thin, very wide product goes on to the other kernels)
         const bool grid_ok = bt || p.tiles_n <= 65535;
         if (!big_tiles && !tiled_better && !too_few && grid_ok && g.K >= 64)
@@ -1509,7 +1511,9 @@ extern "C" size_t t2sp_sgemm_ex_workspace_bytes(int transa, int M, int N, int K)
         const size_t tiled16 = t2sp::plan_gemm(M, n4, k16).scratch_bytes;
         if (tiled16 > tiled) tiled = tiled16;
     }
-    return t2sp::round_up256(transa ? (size_t)M * K * sizeof(float) : 0) + pad + (tiled > one_launch ? tiled : one_launch);
+    // (and for B brought from N x K to K x N where the plain form would split a tiny output's reduction)
+    const size_t b_relaid = one_launch ? t2sp::round_up256((size_t)n4 * k4 * sizeof(float)) : 0;
+    return t2sp::round_up256(transa ? (size_t)M * K * sizeof(float) : 0) + pad + b_relaid + (tiled > one_launch ? tiled : one_launch);
 }
 
 extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, float alpha, const float *A,
@@ -1560,12 +1564,33 @@ extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, fl
         workspace = relaid <= workspace_bytes ? workspace + relaid / sizeof(float) : nullptr;
         workspace_bytes = relaid <= workspace_bytes ? workspace_bytes - relaid : 0;
     }
+    // A tiny output under a long reduction with B stored N x K: the plain form splits such a reduction over
+    // workgroups, the B^T form does not (256 x 256 x 16384: 25 us against 114 us).  With room for it B is brought
+    // to K x N first (16 MB moved there: a few microseconds).
+    const float *b = B;
+    int64_t lb = ldb;
+    bool bt = transb != 0;
+    if (bt && !native_at && cfg == T2SP_CFG_AUTO && K % 16 == 0 && N % 4 == 0 && workspace && aligned16(workspace)) {
+        const t2sp::GemmD16Split sp = t2sp::plan_gemm_d16_split(M, N, K, t2sp::plan_gemm_d16(M, N));
+        const size_t relaid = t2sp::round_up256((size_t)N * K * sizeof(float));
+        if (sp.shift > 0 && workspace_bytes >= relaid + sp.scratch_bytes) {
+            const int ext[2] = {N, K};
+            const int64_t ss[2] = {ldb, 1}, ds[2] = {1, N};
+            const int rc = t2sp_relayout_f32(B, workspace, 2, ext, ss, ds, stream);
+            if (rc != T2SP_OK) return rc;
+            b = workspace;
+            lb = N;
+            bt = false;
+            workspace += relaid / sizeof(float);
+            workspace_bytes -= relaid;
+        }
+    }
     t2sp::GemmArgs g{};
-    g.A = a; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K;
-    g.lda = la; g.ldb = ldb; g.ldc = ldc;
+    g.A = a; g.B = b; g.C = C; g.M = M; g.N = N; g.K = K;
+    g.lda = la; g.ldb = lb; g.ldc = ldc;
     g.tiled = 0;
     g.at = native_at ? 1 : 0;
     g.scale = 1; g.alpha = alpha; g.beta = beta; g.Cin = Cin ? Cin : C; g.ldcin = Cin ? ldcin : ldc;
     if (!Cin) g.beta = 0.f;
-    return t2sp::dispatch(g, cfg, transb != 0, (hipStream_t)stream, workspace, workspace_bytes);
+    return t2sp::dispatch(g, cfg, bt, (hipStream_t)stream, workspace, workspace_bytes);
 }

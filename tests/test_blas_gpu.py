@@ -337,3 +337,30 @@ def test_small_outputs_with_a_reduction_off_the_16_grid_exact(form, MN, K):
         assert rc == 0
         torch.cuda.synchronize()
         assert torch.equal(C.double(), want)
+
+
+@pytest.mark.parametrize("shape", [(256, 256, 16384), (128, 128, 4096), (64, 64, 65536), (100, 132, 8192)])
+@pytest.mark.parametrize("transa", [0, 1])
+def test_tiny_outputs_with_b_transposed_exact(shape, transa):
+    """A tiny output under a long reduction with B stored N x K: with the workspace B is first brought to K x N
+    and the product then splits its reduction over workgroups like the plain form; without one it runs the
+    one-launch B^T kernel.  alpha, beta, C in place; A as it lies or transposed too.  Integer data: exact."""
+    import torch
+    M, N, K = shape
+    L = t2sp_amd.lib()
+    g = torch.Generator().manual_seed(M + K)
+    A = torch.randint(-2, 3, (M, K), generator=g).float().cuda()
+    Bt = torch.randint(-2, 3, (N, K), generator=g).float().cuda()
+    C0 = torch.randint(-4, 5, (M, N), generator=g).float().cuda()
+    want = 2.0 * (A.double() @ Bt.double().t()) - 3.0 * C0.double()
+    Ad = A.t().contiguous() if transa else A
+    nbytes = L.t2sp_sgemm_ex_workspace_bytes(transa, M, N, K)
+    assert nbytes >= N * K * 4
+    ws = torch.empty(nbytes // 4, device="cuda")
+    for w, nb in ((ws.data_ptr(), nbytes), (None, 0) if not transa else (ws.data_ptr(), M * K * 4)):
+        C = C0.clone()
+        rc = L.t2sp_sgemm_ex_f32(transa, 1, M, N, K, 2.0, Ad.data_ptr(), M if transa else K, Bt.data_ptr(), K, -3.0,
+                                 C.data_ptr(), N, C.data_ptr(), N, 0, w, ctypes.c_size_t(nb), None)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert torch.equal(C.double(), want)
