@@ -1540,8 +1540,15 @@ extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, fl
     // (rows too far apart for the LDS-tile loaders' 32-bit offsets: only the 16 x 16 form, where it reaches)
     const bool at_far = lda >= t2sp::LOADER_MAX_LD || ldb >= t2sp::LOADER_MAX_LD;
     const bool at_far_ok = K % 16 == 0 && (int64_t)K * lda < (1 << 30) && (int64_t)K * ldb < (1 << 30);
-    const bool native_at = at_possible && (cfg == T2SP_CFG_AUTO || cfg == T2SP_CFG_DIRECT16) && (!at_far || at_far_ok);
-    (void)t256; (void)room;
+    bool native_at = at_possible && (cfg == T2SP_CFG_AUTO || cfg == T2SP_CFG_DIRECT16) && (!at_far || at_far_ok);
+    (void)t256;
+    // A tiny output under a long reduction: the plain form splits the reduction over workgroups, the A^T form's
+    // kernels do not do that as well (256 x 256 x 16384: 131 us against 26 us; 64 x 64 x 65536: 454 against 20), so
+    // with room for it A is brought to M x K after all.
+    if (native_at && cfg == T2SP_CFG_AUTO && room && K % 16 == 0 && aligned16(workspace)) {
+        const t2sp::GemmD16Split sp = t2sp::plan_gemm_d16_split(M, N, K, t2sp::plan_gemm_d16(M, N));
+        if (sp.shift > 0 && workspace_bytes >= t2sp::round_up256((size_t)M * K * sizeof(float)) + sp.scratch_bytes) native_at = false;
+    }
     if (transa && !native_at) {
         // A is stored K x M: bring it to M x K first (the loaders of the other kernels want k contiguous in A)
         if (!workspace || workspace_bytes < (size_t)M * K * sizeof(float)) {
