@@ -1227,16 +1227,25 @@ __global__ void __launch_bounds__(256) gemm_ktail_kernel(const float *A, int64_t
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= (int64_t)M * nq) return;
     const int i = (int)(t / nq), j = (int)(t - (int64_t)i * nq) * 4;
-    v4f sum = {0.f, 0.f, 0.f, 0.f};
-    for (int k = k0; k < K; k++) {
-        const float a = A[i * a_i + k * a_k];
-        v4f b;
-        if (b_j == 1) b = *reinterpret_cast<const v4f *>(B + k * b_k + j);
-        else b = v4f{B[k * b_k + j * b_j], B[k * b_k + (j + 1) * b_j], B[k * b_k + (j + 2) * b_j], B[k * b_k + (j + 3) * b_j]};
-        sum += a * b;
-    }
+    // all loads first (up to 12 steps: the count is the same for every thread), then the sums in ascending k
+    float a[12];
+    v4f b[12];
     v4f *c = reinterpret_cast<v4f *>(C + (int64_t)i * ldc + j);
-    *c = *c + alpha * sum;
+    const v4f c0 = *c;
+#pragma unroll
+    for (int u = 0; u < 12; u++) {
+        const int k = k0 + u;
+        if (k < K) {
+            a[u] = A[i * a_i + k * a_k];
+            if (b_j == 1) b[u] = *reinterpret_cast<const v4f *>(B + k * b_k + j);
+            else b[u] = v4f{B[k * b_k + j * b_j], B[k * b_k + (j + 1) * b_j], B[k * b_k + (j + 2) * b_j], B[k * b_k + (j + 3) * b_j]};
+        }
+    }
+    v4f sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < 12; u++)
+        if (k0 + u < K) sum += a[u] * b[u];
+    *c = c0 + alpha * sum;
 }
 
 static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *workspace = nullptr,
@@ -1244,9 +1253,14 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
     if (g.M <= 0 || g.N <= 0 || g.K <= 0) return T2SP_ERR_SHAPE;
     // Small outputs whose reduction is not a multiple of 16: the one-launch kernels step 16 k at a time, and without
     // them such a product falls to a few LDS tiles with a split reduction (256 x 256 x 16388: 78 us against 25 us
-    // at K = 16384).  The product over the first K - K % 16 steps goes the usual way; one more pass adds the rest.
+    // at K = 16384; 768 x 2944 x 4684: 279 us, 1.6 times hipBLASLt's time).  The product over the first K - K % 16
+    // steps goes the usual way; one more pass adds the rest (it reads and writes C once: outputs of up to 2 M
+    // elements, up to 8 M under a reduction long enough to dwarf that).
     if (cfg == T2SP_CFG_AUTO && g.K % 16 != 0 && g.K % 4 == 0 && g.K > 64 && !g.tiled && g.N % 4 == 0 && g.ldc % 4 == 0 &&
-        ((uintptr_t)g.C % 16 == 0) && (int64_t)g.M * g.N <= (1 << 21)) {
+        ((uintptr_t)g.C % 16 == 0) &&
+        ((int64_t)g.M * g.N <= (1 << 21) ||
+         ((int64_t)g.M * g.N <= (1 << 23) && g.K >= 512 &&
+          (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) < machine().cus * 25 / 32))) {   // (nearly a round of 128 x 128 tiles takes the tail as it comes)
         GemmArgs h = g;
         h.K = g.K - g.K % 16;
         // (the direct kernel of 8-k steps takes its shapes as they are: 1000^3 20.9 us, 23.8 this way)
@@ -1307,10 +1321,12 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
     //  - a reduction under 128 with more than 3 M outputs is a stream of C: the LDS tiles' wide stores win,
     //    one-wave tiles up to 96 rows (96 x 196608 x 64: 67 -> 36 us), whole rounds of 128 x 128 above.
     const int64_t t32w = (int64_t)((g.M + 31) / 32) * ((g.N + 127) / 128);
+    //    (and up to K = 256 from 4 M outputs on: 2624 x 2816 x 192 43 -> 29 us).
     const bool stream_of_c = g.K < 128 && (int64_t)g.M * g.N >= (3 << 20);
+    const bool short_k_wide = g.K <= 256 && (int64_t)g.M * g.N >= (4 << 20) && g.M > 128 && g.N > 128;
     const bool one_wave_tiles = cfg == T2SP_CFG_AUTO && !bt && vec_ok &&
                                 ((g.M <= 32 && t32w >= 3 * (int64_t)machine().cus) || (stream_of_c && g.M <= 96));
-    const bool skip_d16 = one_wave_tiles || (cfg == T2SP_CFG_AUTO && !bt && vec_ok && stream_of_c);
+    const bool skip_d16 = one_wave_tiles || (cfg == T2SP_CFG_AUTO && !bt && vec_ok && (stream_of_c || short_k_wide));
     if (cfg == T2SP_CFG_AUTO && !skip_d16 && (bt ? gemm_d16_bt_ok(g) : gemm_d16_ok(g))) {
         // Measured from 256^2 x 8192 to 3072^2 x 1024: the 16 x 16 form wins whenever 256 x 256 tiles
         // would not fill the chip, except where 128 x 128 tiles do and the reduction is long enough to
