@@ -35,27 +35,44 @@ __global__ void relayout_kernel(const RelayoutArgs a) {
         a.dst[dof] = a.src[so];
     }
 }
-// A 2-D box whose source is contiguous along one dimension and whose destination is contiguous along the other (a
-// transpose): 64 x 64 tiles through LDS, read along the source's rows and written along the destination's, so
-// that both sides move whole cache lines (the element-wise kernel above reads a different line per lane).
-// Dimension `c` is the one contiguous in the source (extent nc, destination stride dc), dimension `r` the one
-// contiguous in the destination (extent nr, source stride sr).
-__global__ void __launch_bounds__(256) transpose_tile_kernel(const float *src, float *dst, int nr, int nc, int64_t sr, int64_t dc) {
+// A box whose source is contiguous along one dimension (c) and whose destination is contiguous along another
+// (r): a transpose, batched over the remaining dimensions.  64 x 64 tiles of (r, c) go through LDS, read along
+// the source's rows and written along the destination's, so that both sides move whole cache lines (the
+// element-wise kernel above reads a different line per lane).  One workgroup per tile and batch entry.
+__global__ void __launch_bounds__(256) transpose_tile_kernel(const RelayoutArgs a, int r, int c) {
     __shared__ float tile[64][65];
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-    const int tiles_c = (nc + 63) / 64;
-    const int64_t t = blockIdx.x;
-    const int r0 = (int)(t / tiles_c) * 64, c0 = (int)(t % tiles_c) * 64;
+    const int nr = a.ext[r], nc = a.ext[c];
+    const int tiles_c = (nc + 63) / 64, tiles_r = (nr + 63) / 64;
+    int64_t t = blockIdx.x;
+    const int c0 = (int)(t % tiles_c) * 64;
+    t /= tiles_c;
+    const int r0 = (int)(t % tiles_r) * 64;
+    t /= tiles_r;
+    int64_t so = 0, dof = 0;              // the batch entry's offsets
+#pragma unroll
+    for (int d = 0; d < T2SP_MAX_DIMS; d++) {
+        if (d < a.nd && d != r && d != c) {
+            const int64_t q = t / a.ext[d];
+            const int i = (int)(t - q * a.ext[d]);
+            t = q;
+            so += i * a.ss[d];
+            dof += i * a.ds[d];
+        }
+    }
+    const float *src = a.src + so;
+    float *dst = a.dst + dof;
+    const int64_t sr = a.ss[r], dc = a.ds[c];
 #pragma unroll
     for (int k = 0; k < 16; k++) {
-        const int r = r0 + ty + 4 * k, c = c0 + tx;
-        if (r < nr && c < nc) tile[ty + 4 * k][tx] = __builtin_nontemporal_load(src + (int64_t)r * sr + c);
+        const int ri = r0 + ty + 4 * k, ci = c0 + tx;
+        if (ri < nr && ci < nc) tile[ty + 4 * k][tx] = __builtin_nontemporal_load(src + ri * sr + ci);
     }
     __syncthreads();
 #pragma unroll
     for (int k = 0; k < 16; k++) {
-        const int c = c0 + ty + 4 * k, r = r0 + tx;
-        if (r < nr && c < nc) dst[(int64_t)c * dc + r] = tile[tx][ty + 4 * k];
+        const int ci = c0 + ty + 4 * k, ri = r0 + tx;
+        if (ri < nr && ci < nc) dst[ci * dc + ri] = tile[tx][ty + 4 * k];
     }
 }
 // A plain copy: one 128-bit group per thread, read and written as a stream (nontemporal): 6.8 TB/s for 256 MiB
@@ -98,17 +115,17 @@ extern "C" int t2sp_relayout_f32(const float *src, float *dst, int nd, const int
         a.total *= extents[d];
     }
     if (a.total == 0) return T2SP_OK;
-    if (nd == 2 && a.ext[0] > 1 && a.ext[1] > 1) {
-        // r: contiguous in the destination, c: contiguous in the source
-        const int r = a.ds[0] == 1 && a.ss[1] == 1 ? 0 : (a.ds[1] == 1 && a.ss[0] == 1 ? 1 : -1);
-        if (r >= 0 && a.ss[r] >= 0 && a.ds[1 - r] >= 0) {
-            const int nr = a.ext[r], nc = a.ext[1 - r];
-            const int64_t tiles = (int64_t)((nr + 63) / 64) * ((nc + 63) / 64);
-            if (tiles <= INT32_MAX) {
-                hipLaunchKernelGGL(transpose_tile_kernel, dim3((unsigned)tiles), dim3(256), 0, (hipStream_t)stream, src, dst, nr, nc,
-                                   a.ss[r], a.ds[1 - r]);
-                return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
-            }
+    // r: a dimension contiguous in the destination, c: one contiguous in the source; both long enough to fill tiles
+    int r = -1, c = -1;
+    for (int d = 0; d < nd; d++) {
+        if (r < 0 && a.ds[d] == 1 && a.ext[d] >= 16) r = d;
+        if (c < 0 && a.ss[d] == 1 && a.ext[d] >= 16) c = d;
+    }
+    if (r >= 0 && c >= 0 && r != c && a.ss[r] != 1) {
+        const int64_t tiles = (int64_t)((a.ext[r] + 63) / 64) * ((a.ext[c] + 63) / 64) * (a.total / a.ext[r] / a.ext[c]);
+        if (tiles <= INT32_MAX) {
+            hipLaunchKernelGGL(transpose_tile_kernel, dim3((unsigned)tiles), dim3(256), 0, (hipStream_t)stream, a, r, c);
+            return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
         }
     }
     int64_t blocks = (a.total + 255) / 256;

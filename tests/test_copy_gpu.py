@@ -55,11 +55,13 @@ def test_relayout_transposes_bit_exact(shape, padded):
         assert (dst[C] == -1.0).all() and (dst[:C, R:] == -1.0).all()
 
 
-def test_relayout_general_box_bit_exact():
-    """A 4-D permutation with padded strides (the element-wise kernel)."""
+@pytest.mark.parametrize("dims", [(5, 6, 7, 9), (3, 6, 40, 70), (2, 3, 130, 65), (4, 1, 16, 16)])
+def test_relayout_general_box_bit_exact(dims):
+    """A 4-D permutation with padded strides: the element-wise kernel for short extents, and tiles of the two
+    dimensions that are contiguous in source and destination, batched over the other two, for long ones."""
     import torch
     L = t2sp_amd.lib()
-    a, b, c, d = 5, 6, 7, 9
+    a, b, c, d = dims
     src = torch.arange(a * b * c * (d + 2), dtype=torch.float32, device="cuda").reshape(a, b, c, d + 2)
     dst = torch.full((d, b, a, c + 1), -1.0, device="cuda")
     i64 = ctypes.c_int64
