@@ -457,6 +457,55 @@ static int launch_syrk_d16(const SyrkArgs &g, hipStream_t stream) {
 
 constexpr int SYRK_D16_MAX_N = 5120;   // measured: from about 6144 on the LDS tiles' operand reuse wins at every K (see dispatch for 2048 < N)
 
+// C(r, c) += alpha * sum_{k0 <= k < K} A[r][k] * A[c][k] wherever the output form writes C: the last 4, 8 or 12
+// steps of a reduction that is not a multiple of 16, after the one-launch kernel (steps of 16 k) has written the
+// product over [0, k0) with its alpha, beta and Cin.  Flat forms.  One workgroup per 64 x 64 tile of C: the two
+// panels of A (64 rows x up to 12 k each) go through LDS, a thread adds to four rows of four adjacent columns.
+__global__ void __launch_bounds__(256) ssyrk_ktail_kernel(const SyrkArgs g, int k0) {
+    typedef float tv4 __attribute__((ext_vector_type(4)));
+    __shared__ float pr[64][13], pc[64][13];
+    const int tiles = (g.N + 63) / 64;
+    const int r0 = (int)(blockIdx.x / tiles) * 64, c0 = (int)(blockIdx.x % tiles) * 64;
+    const bool full = g.mode == SYRK_FLAT_FULL;
+    const bool want_upper = full || g.upper || g.mirror, want_lower = full || !g.upper || g.mirror;
+    if ((!want_upper && c0 > r0 + 63) || (!want_lower && c0 + 63 < r0)) return;      // nothing of this tile is written
+    const int T = g.K - k0;                                                           // 4, 8 or 12
+    for (int idx = threadIdx.x; idx < 2 * 64 * (T / 4); idx += 256) {
+        const int which = idx / (64 * (T / 4)), rest = idx - which * 64 * (T / 4);
+        const int row = rest / (T / 4), q = rest - row * (T / 4);
+        const int src = min((which ? c0 : r0) + row, g.N - 1);
+        const tv4 v = *reinterpret_cast<const tv4 *>(g.A + (int64_t)src * g.lda + k0 + 4 * q);
+        float *dst = which ? &pc[row][4 * q] : &pr[row][4 * q];
+        dst[0] = v[0]; dst[1] = v[1]; dst[2] = v[2]; dst[3] = v[3];
+    }
+    __syncthreads();
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const bool vec = (g.ldc & 3) == 0 && ((uintptr_t)g.C & 15) == 0;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int rl = ty + 16 * k, r = r0 + rl, c = c0 + 4 * tx;
+        if (r >= g.N || c >= g.N) continue;
+        tv4 sum = {0.f, 0.f, 0.f, 0.f};
+        for (int t = 0; t < T; t++) {
+            const float a = pr[rl][t];
+#pragma unroll
+            for (int e = 0; e < 4; e++) sum[e] += a * pc[4 * tx + e][t];
+        }
+        bool w[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) w[e] = c + e < g.N && (c + e == r || (c + e > r ? want_upper : want_lower));
+        float *dst = g.C + (int64_t)r * g.ldc + c;
+        if (w[0] && w[1] && w[2] && w[3] && vec) {
+            tv4 *p = reinterpret_cast<tv4 *>(dst);
+            *p = *p + g.alpha * sum;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (w[e]) dst[e] += g.alpha * sum[e];
+        }
+    }
+}
+
 static bool syrk_d16_ok(const SyrkArgs &g) {
     return g.K % 16 == 0 && g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && (int64_t)g.N * g.lda < (1 << 30);
 }
@@ -588,6 +637,20 @@ static int dispatch_syrk(SyrkArgs g, int trans, int cfg, float *workspace, size_
         workspace_bytes -= used;
     }
     if (cfg == T2SP_CFG_DIRECT16) return syrk_d16_ok(g) ? launch_syrk_d16(g, stream) : T2SP_ERR_SHAPE;
+    // Up to N = 2048 with K a multiple of 4 but not of 16: the one-launch kernel steps 16 k at a time, and the LDS
+    // tiles that took such shapes are few and slow (N = 768, K = 1028: 39 us against 13 us at K = 1024).  The
+    // product over the first K - K % 16 steps goes to the one-launch kernel; a second pass adds the rest.
+    if (cfg == T2SP_CFG_AUTO && g.K % 16 != 0 && g.K % 4 == 0 && g.K > 64 && g.N <= 2048 && g.mode != SYRK_FOLDED) {
+        SyrkArgs h = g;
+        h.K = g.K - g.K % 16;
+        if (syrk_d16_ok(h)) {
+            const int rc = launch_syrk_d16(h, stream);
+            if (rc != T2SP_OK) return rc;
+            const int side = (g.N + 63) / 64;
+            hipLaunchKernelGGL(ssyrk_ktail_kernel, dim3((unsigned)(side * side)), dim3(256), 0, stream, g, h.K);
+            return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+        }
+    }
     const bool out_ok = g.mode == SYRK_FOLDED ||
                         (g.ldc % 4 == 0 && (uintptr_t)g.C % 16 == 0 &&
                          (!g.Cin || (g.ldcin % 4 == 0 && (uintptr_t)g.Cin % 16 == 0)));
@@ -601,8 +664,18 @@ static int dispatch_syrk(SyrkArgs g, int trans, int cfg, float *workspace, size_
         const SyrkTail t = plan_syrk_tail(g.N, g.K, b, 16);
         const bool split = t.tail > 0 && workspace && workspace_bytes >= t.scratch_bytes;
         const int cus = machine().cus;
-        const double rounds = split ? (double)((t.total - t.tail) / cus) + 1.0 / t.splits + 0.03
-                                    : (double)((t.total + cus - 1) / cus);
+        double rounds = split ? (double)((t.total - t.tail) / cus) + 1.0 / t.splits + 0.03
+                              : (double)((t.total + cus - 1) / cus);
+        // the 64 tiles are two-wave workgroups: one alone on a CU runs at half the CU's rate, and two to four take
+        // the time of four (a CU hands out its SIMDs in a cycle that moves on by one per workgroup); with long
+        // enough reductions that is what a few of them per CU cost (N = 2048, K = 1028: 86 us against 73 us on
+        // 128 tiles; N = 1024: 39 us, N = 1536: 57 us)
+        if (b == 64 && g.K >= 512) {
+            const int64_t main_tiles = split ? t.total - t.tail : t.total;
+            const int64_t per = (main_tiles + cus - 1) / cus;
+            const double units = per <= 0 ? 0.0 : per == 1 ? 2.0 : per <= 4 ? 4.0 : (double)per;
+            rounds = units + (split ? 2.0 / t.splits + 0.03 : 0.0);
+        }
         return rounds * b * b / eff;
     };
     // (short reductions: a tile is mostly its start and its stores, and the small tiles lose the least to them:

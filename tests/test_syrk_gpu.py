@@ -220,3 +220,33 @@ def test_thin_layer_folded_with_and_without_workspace(oracle, III, II, I, K):
         assert (np.isnan(got) == ~written).all()
         assert rel_fro(got[written], want[written])[0] <= TOL
     assert (outs[0][written] == outs[1][written]).all()
+
+
+@pytest.mark.parametrize("N,K", [(100, 68), (768, 1028), (1030, 520), (257, 4104), (2048, 76)])
+def test_reduction_off_the_16_grid_every_flat_form_exact(N, K):
+    """K a multiple of 4 but not of 16 up to N = 2048: the one-launch kernel multiplies over the first
+    K - K % 16 steps and a second pass adds the last 4, 8 or 12 to whatever the output form writes: either
+    triangle alone (the other keeps C), the mirrored pair, the full matrix with C read at every element; alpha,
+    beta and C in place.  Integer data: exact; N that ends inside the pass's 64 x 64 tiles."""
+    import torch
+    L = t2sp_amd.lib()
+    g = torch.Generator().manual_seed(N + K)
+    A = torch.randint(-2, 3, (N, K), generator=g).float().cuda()
+    C0 = torch.randint(-4, 5, (N, N), generator=g).float().cuda()
+    prod = 2.0 * (A.double() @ A.double().t())
+    for upper in (1, 0):
+        tri = torch.triu if upper else torch.tril
+        csym = tri(C0.double()) + tri(C0.double(), 1 if upper else -1).t()
+        for mirror in (0, 1, 2):
+            C = C0.clone()
+            rc = L.t2sp_ssyrk_f32(upper, 0, N, K, 2.0, A.data_ptr(), K, -3.0, C.data_ptr(), N, C.data_ptr(), N, mirror, 0,
+                                  None, 0, None)
+            assert rc == 0
+            torch.cuda.synchronize()
+            if mirror == 0:
+                want = tri(prod - 3.0 * C0.double()) + (torch.tril(C0.double(), -1) if upper else torch.triu(C0.double(), 1))
+            elif mirror == 1:
+                want = prod - 3.0 * csym
+            else:
+                want = prod - 3.0 * C0.double()
+            assert torch.equal(C.double(), want), (upper, mirror)
