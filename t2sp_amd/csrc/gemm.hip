@@ -1217,35 +1217,40 @@ static int launch_d16_at(GemmArgs g, hipStream_t stream) {
     return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
 }
 
-// C[i][j..j+3] += alpha * sum_{k0 <= k < K} A(i, k) * B(k, j..j+3): the last 4, 8 or 12 steps of a reduction whose
-// length is not a multiple of 16, added to a product that a kernel of 16-k steps has computed over [0, k0).
-// A(i, k) = A[i * a_i + k * a_k]; B(k, j) = B[k * b_k + j * b_j].  One thread per four columns of one row.
+// C[i][j] += alpha * sum_{k0 <= k < K} A(i, k) * B(k, j): the last 4, 8 or 12 steps of a reduction whose length is
+// not a multiple of 16, added to a product that a kernel of 16-k steps has computed over [0, k0).
+// A(i, k) = A[i * a_i + k * a_k]; B(k, j) = B[k * b_k + j * b_j] (either stride 1: the three operand layouts).
+// One workgroup per 64 x 64 tile of C: the two panels (64 x up to 12) go through LDS, read with the lanes along
+// whichever index is contiguous; a thread adds to four rows of four adjacent columns (N % 4 == 0, rows of C aligned).
 __global__ void __launch_bounds__(256) gemm_ktail_kernel(const float *A, int64_t a_i, int64_t a_k, const float *B, int64_t b_k,
                                                          int64_t b_j, float *C, int64_t ldc, int M, int N, int k0, int K,
                                                          float alpha) {
-    const int nq = N / 4;
-    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= (int64_t)M * nq) return;
-    const int i = (int)(t / nq), j = (int)(t - (int64_t)i * nq) * 4;
-    // all loads first (up to 12 steps: the count is the same for every thread), then the sums in ascending k
-    float a[12];
-    v4f b[12];
-    v4f *c = reinterpret_cast<v4f *>(C + (int64_t)i * ldc + j);
-    const v4f c0 = *c;
-#pragma unroll
-    for (int u = 0; u < 12; u++) {
-        const int k = k0 + u;
-        if (k < K) {
-            a[u] = A[i * a_i + k * a_k];
-            if (b_j == 1) b[u] = *reinterpret_cast<const v4f *>(B + k * b_k + j);
-            else b[u] = v4f{B[k * b_k + j * b_j], B[k * b_k + (j + 1) * b_j], B[k * b_k + (j + 2) * b_j], B[k * b_k + (j + 3) * b_j]};
-        }
+    __shared__ float pa[64][13], pb[64][13];
+    const int tiles_n = (N + 63) / 64;
+    const int i0 = (int)(blockIdx.x / tiles_n) * 64, j0 = (int)(blockIdx.x % tiles_n) * 64;
+    const int T = K - k0;
+    for (int idx = threadIdx.x; idx < 64 * T; idx += 256) {
+        // lanes along k where k is contiguous, along the row or column index where that is
+        const int ra = a_k == 1 ? idx / T : idx % 64, ta = a_k == 1 ? idx % T : idx / 64;
+        const int cb = b_k == 1 ? idx / T : idx % 64, tb = b_k == 1 ? idx % T : idx / 64;
+        pa[ra][ta] = A[(int64_t)min(i0 + ra, M - 1) * a_i + (int64_t)(k0 + ta) * a_k];
+        pb[cb][tb] = B[(int64_t)(k0 + tb) * b_k + (int64_t)min(j0 + cb, N - 1) * b_j];
     }
-    v4f sum = {0.f, 0.f, 0.f, 0.f};
+    __syncthreads();
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
 #pragma unroll
-    for (int u = 0; u < 12; u++)
-        if (k0 + u < K) sum += a[u] * b[u];
-    *c = c0 + alpha * sum;
+    for (int q = 0; q < 4; q++) {
+        const int il = ty + 16 * q, i = i0 + il, j = j0 + 4 * tx;
+        if (i >= M || j >= N) continue;
+        v4f sum = {0.f, 0.f, 0.f, 0.f};
+        for (int t = 0; t < T; t++) {
+            const float a = pa[il][t];
+#pragma unroll
+            for (int e = 0; e < 4; e++) sum[e] += a * pb[4 * tx + e][t];
+        }
+        v4f *c = reinterpret_cast<v4f *>(C + (int64_t)i * ldc + j);
+        *c = *c + alpha * sum;
+    }
 }
 
 static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *workspace = nullptr,
@@ -1268,8 +1273,8 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         if (!direct && (g.at ? gemm_d16_at_ok(h) : bt ? gemm_d16_bt_ok(h) : gemm_d16_ok(h))) {
             const int rc = dispatch(h, cfg, bt, stream, workspace, workspace_bytes);
             if (rc != T2SP_OK) return rc;
-            const int64_t groups = (int64_t)g.M * (g.N / 4);
-            hipLaunchKernelGGL(gemm_ktail_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, stream, g.A,
+            const int64_t tiles = (int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64);
+            hipLaunchKernelGGL(gemm_ktail_kernel, dim3((unsigned)tiles), dim3(256), 0, stream, g.A,
                                g.at ? (int64_t)1 : g.lda, g.at ? g.lda : (int64_t)1, g.B, bt ? (int64_t)1 : g.ldb,
                                bt ? g.ldb : (int64_t)1, g.C, g.ldc, g.M, g.N, h.K, g.K, g.scale ? g.alpha : 1.f);
             return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
