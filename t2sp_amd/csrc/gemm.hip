@@ -527,7 +527,7 @@ __device__ __forceinline__ v4f quad_transpose(v4f v, int e) {
 template <int MB, int NB>
 __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     sgemm_direct16_bt_kernel(const float *A, const float *B, int M, int N, int K, int lda, int ldb, int tiles_m, int rows_per_tile,
-                             const GemmArgs g) {
+                             int split_shift, const GemmArgs g) {
     constexpr int NW = GEMM_D16_WAVES, R = GEMM_D16_RING;
     extern __shared__ __align__(16) float smem[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -536,7 +536,11 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     const int m0 = tm * rows_per_tile, n0 = tn * 16 * NB;
     const int m_end = min(m0 + rows_per_tile, M);
     const int steps = K >> 4;
-    const int s0 = (int)((int64_t)steps * wave / NW), s1 = (int)((int64_t)steps * (wave + 1) / NW);
+    // split_shift > 0: workgroup blockIdx.y of 2^split_shift reduces its share of k into plane blockIdx.y of the
+    // workspace (tiny outputs under a long reduction, as in sgemm_direct16_kernel); its waves split that share again
+    const int share = blockIdx.y;
+    const int z0 = (int)(((int64_t)steps * share) >> split_shift), z1 = (int)(((int64_t)steps * (share + 1)) >> split_shift);
+    const int s0 = z0 + (int)((int64_t)(z1 - z0) * wave / NW), s1 = z0 + (int)((int64_t)(z1 - z0) * (wave + 1) / NW);
     const int nsteps = s1 - s0;
 
     uint32_t a_off[MB], b_off[NB];
@@ -606,7 +610,7 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     // beta * Cin of this wave's blocks: requested before the exchange (see sgemm_direct16_kernel)
     constexpr int PER_WAVE = (MB * NB + NW - 1) / NW;
     v4f cin[PER_WAVE];
-    const bool with_cin = vec_ok && g.scale && g.beta != 0.f;
+    const bool with_cin = vec_ok && g.scale && g.beta != 0.f && !split_shift;
     if (with_cin) {
 #pragma unroll
         for (int i = 0; i < PER_WAVE; i++) {
@@ -629,6 +633,10 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
         const int mb = pr / NB, nb = pr - mb * NB;
         const int row = m0 + 16 * mb + orow, col = n0 + 16 * nb + ocol;
         if (row >= m_end) continue;
+        if (split_shift) {          // a partial sum (N % 4 == 0): the kernel that adds the planes scales and stores
+            if (col + 4 <= N) *reinterpret_cast<v4f *>(g.scratch + ((int64_t)share * M + row) * N + col) = sum;
+            continue;
+        }
         if (vec_ok && col + 4 <= N) {
             v4f out = sum;
             if (g.scale) {
@@ -1169,20 +1177,32 @@ static bool gemm_d16_bt_ok(const GemmArgs &g) {
            (int64_t)g.M * g.lda < (1 << 30) && (int64_t)g.N * g.ldb < (1 << 30);
 }
 template <int MB, int NB>
-static int launch_d16_bt_t(GemmArgs g, const GemmD16Plan &p, hipStream_t stream) {
+static int launch_d16_bt_t(GemmArgs g, const GemmD16Plan &p, hipStream_t stream, int split_shift = 0, float *scratch = nullptr) {
     g.tiles_m = p.tiles_m;
     g.tiles_n = p.tiles_n;
+    g.scratch = scratch;
     const size_t smem = (size_t)GEMM_D16_WAVES * MB * NB * 64 * sizeof(v4f);
     auto kern = sgemm_direct16_bt_kernel<MB, NB>;
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(GEMM_D16_WAVES * 64), smem, stream, g.A, g.B, g.M, g.N, g.K,
-                       (int)g.lda, (int)g.ldb, p.tiles_m, p.rows_per_tile, g);
-    return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n, 1 << split_shift), dim3(GEMM_D16_WAVES * 64), smem, stream, g.A, g.B, g.M, g.N,
+                       g.K, (int)g.lda, (int)g.ldb, p.tiles_m, p.rows_per_tile, split_shift, g);
+    if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
+    if (split_shift) {
+        GemmOutMap map{g};
+        if (launch_splitk_reduce<true>(scratch, 1 << split_shift, g.M, g.N, map, stream) != hipSuccess) return T2SP_ERR_LAUNCH;
+    }
+    return T2SP_OK;
 }
-static int launch_d16_bt(const GemmArgs &g, hipStream_t stream) {
-    const GemmD16Plan p = plan_gemm_d16_bt(g.M, g.N);
-#define T2SP_D16_CASE(MBV, NBV) if (p.mb == MBV && p.nb == NBV) return launch_d16_bt_t<MBV, NBV>(g, p, stream);
+// (with room for the planes, a tiny output under a long reduction splits it over workgroups: tile and depth as the
+// plain form plans them, its tiles being ones this form has too)
+static int launch_d16_bt(const GemmArgs &g, hipStream_t stream, float *workspace = nullptr, size_t workspace_bytes = 0) {
+    const GemmD16Plan whole = plan_gemm_d16_bt(g.M, g.N);
+    GemmD16Split sp = plan_gemm_d16_split(g.M, g.N, g.K, plan_gemm_d16(g.M, g.N));     // (decided as for the plain form)
+    if (!workspace || workspace_bytes < sp.scratch_bytes || ((uintptr_t)workspace % 16) || g.N % 4 || g.tiled) sp.shift = 0;
+    const int shift = sp.shift;
+    const GemmD16Plan p = shift ? sp.tile : whole;
+#define T2SP_D16_CASE(MBV, NBV) if (p.mb == MBV && p.nb == NBV) return launch_d16_bt_t<MBV, NBV>(g, p, stream, shift, workspace);
     T2SP_D16_CASE(2, 2) T2SP_D16_CASE(3, 2) T2SP_D16_CASE(4, 2) T2SP_D16_CASE(5, 2) T2SP_D16_CASE(6, 2)
     T2SP_D16_CASE(7, 2) T2SP_D16_CASE(8, 2) T2SP_D16_CASE(2, 3) T2SP_D16_CASE(3, 3) T2SP_D16_CASE(4, 3)
     T2SP_D16_CASE(5, 3) T2SP_D16_CASE(6, 3) T2SP_D16_CASE(7, 3) T2SP_D16_CASE(8, 3) T2SP_D16_CASE(2, 4)
@@ -1221,10 +1241,11 @@ static int launch_d16_at(GemmArgs g, hipStream_t stream) {
 // not a multiple of 16, added to a product that a kernel of 16-k steps has computed over [0, k0).
 // A(i, k) = A[i * a_i + k * a_k]; B(k, j) = B[k * b_k + j * b_j] (either stride 1: the three operand layouts).
 // One workgroup per 64 x 64 tile of C: the two panels (64 x up to 12) go through LDS, read with the lanes along
-// whichever index is contiguous; a thread adds to four rows of four adjacent columns (N % 4 == 0, rows of C aligned).
+// whichever index is contiguous; a thread adds to four rows of four adjacent columns; C(i, j) at C[i * c_i + j * c_j]
+// (128-bit accesses where c_j is 1 and rows are aligned).
 __global__ void __launch_bounds__(256) gemm_ktail_kernel(const float *A, int64_t a_i, int64_t a_k, const float *B, int64_t b_k,
-                                                         int64_t b_j, float *C, int64_t ldc, int M, int N, int k0, int K,
-                                                         float alpha) {
+                                                         int64_t b_j, float *C, int64_t c_i, int64_t c_j, int M, int N, int k0,
+                                                         int K, float alpha) {
     __shared__ float pa[64][13], pb[64][13];
     const int tiles_n = (N + 63) / 64;
     const int i0 = (int)(blockIdx.x / tiles_n) * 64, j0 = (int)(blockIdx.x % tiles_n) * 64;
@@ -1248,8 +1269,15 @@ __global__ void __launch_bounds__(256) gemm_ktail_kernel(const float *A, int64_t
 #pragma unroll
             for (int e = 0; e < 4; e++) sum[e] += a * pb[4 * tx + e][t];
         }
-        v4f *c = reinterpret_cast<v4f *>(C + (int64_t)i * ldc + j);
-        *c = *c + alpha * sum;
+        float *dst = C + (int64_t)i * c_i + (int64_t)j * c_j;
+        if (c_j == 1 && j + 3 < N && (c_i & 3) == 0 && ((uintptr_t)C & 15) == 0) {
+            v4f *c = reinterpret_cast<v4f *>(dst);
+            *c = *c + alpha * sum;
+        } else {      // C(i, j) at any two strides, or a ragged last group
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (j + e < N) dst[e * c_j] += alpha * sum[e];
+        }
     }
 }
 
@@ -1261,11 +1289,15 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
     // at K = 16384; 768 x 2944 x 4684: 279 us, 1.6 times hipBLASLt's time).  The product over the first K - K % 16
     // steps goes the usual way; one more pass adds the rest (it reads and writes C once: outputs of up to 2 M
     // elements, up to 8 M under a reduction long enough to dwarf that).
-    if (cfg == T2SP_CFG_AUTO && g.K % 16 != 0 && g.K % 4 == 0 && g.K > 64 && !g.tiled && g.N % 4 == 0 && g.ldc % 4 == 0 &&
-        ((uintptr_t)g.C % 16 == 0) &&
+    // (a "tiled" output that is just a matrix at two strides, as the transposed result of the A^T * B^T form is, counts as flat)
+    const bool strided_c = g.tiled && g.t_jj == 1 && g.t_ii == 1 && g.t_jjj >= g.N && g.t_iii >= g.M && !(g.scale && g.beta != 0.f);
+    if (cfg == T2SP_CFG_AUTO && g.K % 16 != 0 && g.K % 4 == 0 && g.K > 64 && g.N % 4 == 0 &&
+        (strided_c || (!g.tiled && g.ldc % 4 == 0 && ((uintptr_t)g.C % 16 == 0))) &&
         ((int64_t)g.M * g.N <= (1 << 21) ||
-         ((int64_t)g.M * g.N <= (1 << 23) && g.K >= 512 &&
-          (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) < machine().cus * 25 / 32))) {   // (nearly a round of 128 x 128 tiles takes the tail as it comes)
+         (g.K >= 512 &&
+          (g.at ? (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256) < machine().cus * 25 / 32    // (the A^T form's 128 x 128 tiles are two-wave ones: whatever would take its one-launch kernel)
+                : ((int64_t)g.M * g.N <= (1 << 23) &&
+                   (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) < machine().cus * 25 / 32))))) {   // (nearly a round of 128 x 128 tiles takes the tail as it comes)
         GemmArgs h = g;
         h.K = g.K - g.K % 16;
         // (the direct kernel of 8-k steps takes its shapes as they are: 1000^3 20.9 us, 23.8 this way)
@@ -1274,9 +1306,16 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
             const int rc = dispatch(h, cfg, bt, stream, workspace, workspace_bytes);
             if (rc != T2SP_OK) return rc;
             const int64_t tiles = (int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64);
-            hipLaunchKernelGGL(gemm_ktail_kernel, dim3((unsigned)tiles), dim3(256), 0, stream, g.A,
-                               g.at ? (int64_t)1 : g.lda, g.at ? g.lda : (int64_t)1, g.B, bt ? (int64_t)1 : g.ldb,
-                               bt ? g.ldb : (int64_t)1, g.C, g.ldc, g.M, g.N, h.K, g.K, g.scale ? g.alpha : 1.f);
+            const int64_t a_i = g.at ? (int64_t)1 : g.lda, a_k = g.at ? g.lda : (int64_t)1;
+            const int64_t b_k = bt ? (int64_t)1 : g.ldb, b_j = bt ? g.ldb : (int64_t)1;
+            const int64_t c_i = strided_c ? g.s[1] : g.ldc, c_j = strided_c ? g.s[0] : (int64_t)1;
+            const float alpha = g.scale ? g.alpha : 1.f;
+            if (c_j != 1 && c_i == 1)      // a transposed result: the pass runs on C^T = B^T * A^T, whose rows are contiguous
+                hipLaunchKernelGGL(gemm_ktail_kernel, dim3((unsigned)tiles), dim3(256), 0, stream, g.B, b_j, b_k, g.A, a_k, a_i, g.C,
+                                   c_j, c_i, g.N, g.M, h.K, g.K, alpha);
+            else
+                hipLaunchKernelGGL(gemm_ktail_kernel, dim3((unsigned)tiles), dim3(256), 0, stream, g.A, a_i, a_k, g.B, b_k, b_j, g.C,
+                                   c_i, c_j, g.M, g.N, h.K, g.K, alpha);
             return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
         }
     }
@@ -1310,7 +1349,7 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         return launch<GemmMA, false>(g, stream, sp, workspace);
     }
     if (cfg == T2SP_CFG_DIRECT16) {
-        if (bt) return gemm_d16_bt_ok(g) ? launch_d16_bt(g, stream) : T2SP_ERR_SHAPE;
+        if (bt) return gemm_d16_bt_ok(g) ? launch_d16_bt(g, stream, workspace, workspace_bytes) : T2SP_ERR_SHAPE;
         return gemm_d16_ok(g) ? launch_d16(g, stream, workspace, workspace_bytes) : T2SP_ERR_SHAPE;
     }
     // (the loaders address a tile with 32-bit offsets: leading dimensions below LOADER_MAX_LD)
@@ -1367,7 +1406,7 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         // (the plain form's grid is tiles_m x tiles_n: a thin, very wide product goes on to the other kernels)
         const bool grid_ok = bt || p.tiles_n <= 65535;
         if (!big_tiles && !tiled_better && !too_few && grid_ok && g.K >= 64)
-            return bt ? launch_d16_bt(g, stream) : launch_d16(g, stream, workspace, workspace_bytes);
+            return bt ? launch_d16_bt(g, stream, workspace, workspace_bytes) : launch_d16(g, stream, workspace, workspace_bytes);
     }
     if ((cfg == T2SP_CFG_AUTO || cfg == T2SP_CFG_DIRECT) && !bt && !g.scale && !g.tiled &&
         g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && gemm_direct_ok(g, cfg == T2SP_CFG_DIRECT))
@@ -1532,20 +1571,58 @@ extern "C" size_t t2sp_sgemm_ex_workspace_bytes(int transa, int M, int N, int K)
         const size_t tiled16 = t2sp::plan_gemm(M, n4, k16).scratch_bytes;
         if (tiled16 > tiled) tiled = tiled16;
     }
-    // (and for B brought from N x K to K x N where the plain form would split a tiny output's reduction)
-    const size_t b_relaid = one_launch ? t2sp::round_up256((size_t)n4 * k4 * sizeof(float)) : 0;
+    // (and for B brought from N x K to K x N: where the plain form would split a tiny output's reduction, and when
+    // both operands are transposed)
+    const size_t b_relaid = (one_launch || transa) ? t2sp::round_up256((size_t)n4 * k4 * sizeof(float)) : 0;
     return t2sp::round_up256(transa ? (size_t)M * K * sizeof(float) : 0) + pad + b_relaid + (tiled > one_launch ? tiled : one_launch);
 }
 
-extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, float alpha, const float *A,
-                                 int64_t lda, const float *B, int64_t ldb, float beta, const float *Cin,
+extern "C" int t2sp_sgemm_ex_f32(int transa, int transb_given, int M, int N, int K, float alpha, const float *A,
+                                 int64_t lda, const float *B_given, int64_t ldb_given, float beta, const float *Cin,
                                  int64_t ldcin, float *C, int64_t ldc, int cfg, float *workspace,
                                  size_t workspace_bytes, void *stream) {
+    int transb = transb_given;
+    const float *B = B_given;
+    int64_t ldb = ldb_given;
+
     if (!gemm_extents_ok(M, N, K) || lda < 0 || ldb < 0 || ldc < 0 || (Cin && ldcin < 0)) return T2SP_ERR_SHAPE;
     if (!t2sp::strides_in_range(lda, ldb, ldc, ldcin)) return T2SP_ERR_SHAPE;
     const float *a = A;
     int64_t la = lda;
     auto aligned16 = [](const void *p) { return ((uintptr_t)p & 15) == 0; };
+    // Both operands transposed: the A^T form's kernels take A as it lies and are as fast as the plain form's, the
+    // B^T form's one-launch kernel stores element by element, so with room for it B (N x K) is brought to K x N and the
+    // product runs as A^T * B, rather than A re-laid and the product run as A * B^T (measured on random shapes:
+    // 1.5 to 2.1 times hipBLASLt's time that way).
+    // Small and middle-sized outputs without a C to read: A^T * B^T = (B * A)^T, and B (N x K) times A (K x M) is a plain
+    // product of the operands as they lie; its result goes out transposed, element by element (fine up to a few
+    // million outputs).  No operand is moved.
+    if (transa && transb && cfg == T2SP_CFG_AUTO && (!Cin || beta == 0.f) && (int64_t)M * N <= (4 << 20) && M % 4 == 0 && K % 4 == 0 &&
+        lda % 4 == 0 && ldb % 4 == 0 && aligned16(A) && aligned16(B) && aligned16(C) && (int64_t)N * ldb < (1 << 30) &&
+        (int64_t)K * lda < (1 << 30)) {
+        t2sp::GemmArgs g{};
+        g.A = B; g.B = A; g.C = C; g.M = N; g.N = M; g.K = K;
+        g.lda = ldb; g.ldb = lda; g.ldc = 0;
+        g.tiled = 1; g.t_jjj = M; g.t_iii = N; g.t_jj = 1; g.t_ii = 1;
+        g.s[0] = ldc; g.s[1] = 1;                 // column m of the swapped product is row m of C
+        g.scale = 1; g.alpha = alpha; g.beta = 0.f; g.Cin = C; g.ldcin = ldc;
+        return t2sp::dispatch(g, cfg, false, (hipStream_t)stream, workspace, workspace_bytes);
+    }
+    if (transa && transb && cfg == T2SP_CFG_AUTO && M % 4 == 0 && N % 4 == 0 && lda % 4 == 0 && ldc % 4 == 0 && aligned16(A) &&
+        aligned16(C) && (!Cin || (ldcin % 4 == 0 && aligned16(Cin))) && workspace && aligned16(workspace)) {
+        const size_t relaid = t2sp::round_up256((size_t)N * K * sizeof(float));
+        if (workspace_bytes >= relaid) {
+            const int ext[2] = {N, K};
+            const int64_t ss[2] = {ldb, 1}, ds[2] = {1, N};
+            const int rc = t2sp_relayout_f32(B, workspace, 2, ext, ss, ds, stream);
+            if (rc != T2SP_OK) return rc;
+            B = workspace;
+            ldb = N;
+            transb = 0;
+            workspace += relaid / sizeof(float);
+            workspace_bytes -= relaid;
+        }
+    }
     // A stored K x M is taken as it lies when B is not transposed too and rows of all operands
     // can be read and written 128 bits at a time
     const bool at_possible = transa && !transb && (cfg == T2SP_CFG_AUTO || cfg == T2SP_CFG_DIRECT16) && M % 4 == 0 && N % 4 == 0 && lda % 4 == 0 &&
@@ -1592,27 +1669,9 @@ extern "C" int t2sp_sgemm_ex_f32(int transa, int transb, int M, int N, int K, fl
         workspace = relaid <= workspace_bytes ? workspace + relaid / sizeof(float) : nullptr;
         workspace_bytes = relaid <= workspace_bytes ? workspace_bytes - relaid : 0;
     }
-    // A tiny output under a long reduction with B stored N x K: the plain form splits such a reduction over
-    // workgroups, the B^T form does not (256 x 256 x 16384: 25 us against 114 us).  With room for it B is brought
-    // to K x N first (16 MB moved there: a few microseconds).
     const float *b = B;
     int64_t lb = ldb;
-    bool bt = transb != 0;
-    if (bt && !native_at && cfg == T2SP_CFG_AUTO && K % 16 == 0 && N % 4 == 0 && workspace && aligned16(workspace)) {
-        const t2sp::GemmD16Split sp = t2sp::plan_gemm_d16_split(M, N, K, t2sp::plan_gemm_d16(M, N));
-        const size_t relaid = t2sp::round_up256((size_t)N * K * sizeof(float));
-        if (sp.shift > 0 && workspace_bytes >= relaid + sp.scratch_bytes) {
-            const int ext[2] = {N, K};
-            const int64_t ss[2] = {ldb, 1}, ds[2] = {1, N};
-            const int rc = t2sp_relayout_f32(B, workspace, 2, ext, ss, ds, stream);
-            if (rc != T2SP_OK) return rc;
-            b = workspace;
-            lb = N;
-            bt = false;
-            workspace += relaid / sizeof(float);
-            workspace_bytes -= relaid;
-        }
-    }
+    const bool bt = transb != 0;
     t2sp::GemmArgs g{};
     g.A = a; g.B = b; g.C = C; g.M = M; g.N = N; g.K = K;
     g.lda = la; g.ldb = lb; g.ldc = ldc;

@@ -364,3 +364,34 @@ def test_tiny_outputs_with_b_transposed_exact(shape, transa):
         assert rc == 0
         torch.cuda.synchronize()
         assert torch.equal(C.double(), want)
+
+
+@pytest.mark.parametrize("shape", [(256, 700, 3404), (512, 2340, 512), (844, 204, 2528), (132, 68, 100), (1332, 5528, 64), (2048, 2052, 1028)])
+def test_both_operands_transposed_exact(shape):
+    """A stored K x M and B stored N x K.  Without a C to read, outputs of up to 4 M elements run as the plain
+    product B * A of the operands as they lie, written out transposed (reductions off the 16 grid through the
+    second pass, which then adds at the transposed positions too); with beta, or beyond that size, B is re-laid and
+    the A^T form takes A as it lies, given the room, else A is re-laid.  alpha throughout.  Integer data: exact;
+    a canary frame around C stays."""
+    import torch
+    M, N, K = shape
+    L = t2sp_amd.lib()
+    g = torch.Generator().manual_seed(M + N + K)
+    At = torch.randint(-2, 3, (K, M), generator=g).float().cuda()
+    Bt = torch.randint(-2, 3, (N, K), generator=g).float().cuda()
+    C0 = torch.randint(-4, 5, (M, N), generator=g).float().cuda()
+    prod = At.double().t() @ Bt.double().t()
+    nbytes = L.t2sp_sgemm_ex_workspace_bytes(1, M, N, K)
+    ws = torch.empty(max(nbytes // 4, 4), device="cuda")
+    for beta in (0.0, -3.0):
+        for w, nb in ((ws.data_ptr(), nbytes), (ws.data_ptr(), M * K * 4)):
+            frame = torch.full((M + 2, N + 8), 7.0, device="cuda")
+            C = frame[1:M + 1, 4:N + 4]
+            C.copy_(C0)
+            rc = L.t2sp_sgemm_ex_f32(1, 1, M, N, K, 2.0, At.data_ptr(), M, Bt.data_ptr(), K, beta, C.data_ptr(), N + 8,
+                                     C.data_ptr(), N + 8, 0, w, ctypes.c_size_t(nb), None)
+            assert rc == 0
+            torch.cuda.synchronize()
+            assert torch.equal(C.double(), 2.0 * prod + beta * C0.double()), (beta, nb)
+            C.fill_(7.0)
+            assert (frame == 7.0).all()
