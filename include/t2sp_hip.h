@@ -70,13 +70,15 @@ int t2sp_sgemm_f32_tiled(const float *A, const float *B, float *C, int M, int N,
 
 /* BLAS form, row-major: C = alpha * op(A) * op(B) + beta * Cin with op(X) = X or X^T (transa /
  * transb non-zero: A stored K x M, B stored N x K).  Cin may be NULL (beta is then ignored) or
- * equal to C (in place).  Every form but A^T * B^T reads both operands as they lie: B^T through
- * k-contiguous tiles, A^T (with M, N and the leading dimensions multiples of 4 and 16-byte
- * aligned pointers) through row-contiguous ones, for any K; small and middle-sized products of
- * each form have a one-launch kernel of their own (T2SP_CFG_DIRECT16 forces it).  Otherwise a transposed A is first
- * re-laid into `workspace` when there is room for it (M * K floats) and read as it lies by a
- * one-thread-per-output kernel when there is not (slow, like every shape the 128-bit loaders cannot
- * take without a workspace); the rest of t2sp_sgemm_ex_workspace_bytes is
+ * equal to C (in place).  The forms with one operand transposed read both operands as they lie:
+ * B^T through k-contiguous tiles, A^T (with M, N and the leading dimensions multiples of 4 and
+ * 16-byte aligned pointers) through row-contiguous ones, for any K; small and middle-sized products of
+ * each form have a one-launch kernel of their own (T2SP_CFG_DIRECT16 forces it).  A^T * B^T without a
+ * C to read and with at most 4 M outputs runs as the plain product B * A of the operands as they lie,
+ * written out transposed; otherwise one operand is first re-laid into `workspace` when there is room
+ * for it (B, N * K floats, for the A^T kernels; else A, M * K floats), and a transposed A that can be
+ * neither taken as it lies nor re-laid is read by a one-thread-per-output kernel (slow, like every
+ * shape the 128-bit loaders cannot take without a workspace); the rest of t2sp_sgemm_ex_workspace_bytes is
  * optional room for the planes of a split reduction, as in t2sp_sgemm_f32.  Device side of the reference's 8-argument
  * gemm(opa, opb, alpha, beta, A, B, C, O) pipeline behind its BLAS wrapper
  * (t2s/peppers/blas/level3/gemm/release/a10/blas-gemm.cpp:28-47). */
