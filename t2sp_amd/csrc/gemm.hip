@@ -659,7 +659,8 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
 // ends with four adjacent columns of each of its rows and stores 128 bits at a time.
 template <int MB, bool BUF>
 __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
-    sgemm_direct16_at_kernel(const float *A, const float *B, int M, int N, int K, int lda, int ldb, int tiles_m, const GemmArgs g) {
+    sgemm_direct16_at_kernel(const float *A, const float *B, int M, int N, int K, int lda, int ldb, int tiles_m, int split_shift,
+                             const GemmArgs g) {
     constexpr int NW = GEMM_D16_WAVES, R = GEMM_D16_RING, NB = 4;
     extern __shared__ __align__(16) float smem[];
     v4f *red = reinterpret_cast<v4f *>(smem);            // [wave][mb][nb][lane]
@@ -668,7 +669,11 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     const int tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
     const int m0 = tm * 16 * MB, n0 = tn * 64;
     const int steps = K >> 4;
-    const int s0 = (int)((int64_t)steps * wave / NW), s1 = (int)((int64_t)steps * (wave + 1) / NW);
+    // split_shift > 0: workgroup blockIdx.y of 2^split_shift reduces its share of k into plane blockIdx.y of the
+    // workspace (tiny outputs under a long reduction, as in sgemm_direct16_kernel); its waves split that share again
+    const int share = blockIdx.y;
+    const int z0 = (int)(((int64_t)steps * share) >> split_shift), z1 = (int)(((int64_t)steps * (share + 1)) >> split_shift);
+    const int s0 = z0 + (int)((int64_t)(z1 - z0) * wave / NW), s1 = z0 + (int)((int64_t)(z1 - z0) * (wave + 1) / NW);
     const int nsteps = s1 - s0;
 
     // a lane's MB adjacent rows (MB = 4: one 128-bit load; MB = 2: 64 bits) and 4 adjacent columns
@@ -743,7 +748,7 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     // beta * Cin is requested before the exchange (see sgemm_direct16_kernel); MB <= NW: one row block per wave
     static_assert(MB <= NW, "a wave sums one row block");
     v4f cin[4];
-    const bool with_cin = g.scale && g.beta != 0.f && wave < MB;
+    const bool with_cin = g.scale && g.beta != 0.f && wave < MB && !split_shift;
     if (with_cin) {
 #pragma unroll
         for (int r = 0; r < 4; r++) {
@@ -767,6 +772,10 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
             const int orow = m0 + MB * (4 * lq + r) + mb;
             v4f out = {sum[0][r], sum[1][r], sum[2][r], sum[3][r]};
             if (orow < M && col_ok) {
+                if (split_shift) {      // a partial sum: the kernel that adds the planes scales and stores
+                    *reinterpret_cast<v4f *>(g.scratch + ((int64_t)share * M + orow) * N + col) = out;
+                    continue;
+                }
                 if (g.scale) {
                     out = out * g.alpha;
                     if (g.beta != 0.f) out += cin[r] * g.beta;
@@ -1073,7 +1082,10 @@ struct GemmD16Split {
 static GemmD16Split plan_gemm_d16_split(int M, int N, int K, const GemmD16Plan &unsplit) {
     const int cus = machine().cus, nx = machine().xcds;
     GemmD16Split r{0, 0, unsplit};
-    if ((int64_t)unsplit.tiles_m * unsplit.tiles_n <= 0 || (int64_t)unsplit.tiles_m * unsplit.tiles_n > cus / 2 || K % 16) return r;
+    // (tiny = at most half as many 64 x 64 tiles as CUs, whatever the unsplit plan would cut the output into: 384 x 384
+    // unsplit is 144 tiles of 32 x 32, 176 us at K = 32768, against 36 of 64 x 64 in four shares each)
+    const int64_t t64 = (int64_t)((M + 63) / 64) * ((N + 63) / 64);
+    if ((int64_t)unsplit.tiles_m * unsplit.tiles_n <= 0 || t64 > cus / 2 || K % 16) return r;
     const int steps = K / 16;
     auto step_us = [](int mb, int nb) {
         const double mfma_us = 4.0 * mb * nb * 32.0 / 2400.0 * 1.03, load_us = (mb + 4) * 0.0575;
@@ -1099,7 +1111,8 @@ static GemmD16Split plan_gemm_d16_split(int M, int N, int K, const GemmD16Plan &
             }
         }
     if (!r.shift) return r;
-    const double unsplit_us = (steps / 4.0) * step_us(unsplit.mb, unsplit.nb);
+    const int64_t unsplit_rounds = ((int64_t)unsplit.tiles_m * unsplit.tiles_n + cus - 1) / cus;
+    const double unsplit_us = (steps / 4.0) * step_us(unsplit.mb, unsplit.nb) * (double)unsplit_rounds;
     if (unsplit_us - best < 8.0) {                                          // the second launch and its pass over the planes
         r.shift = 0;
         r.tile = unsplit;
@@ -1218,7 +1231,7 @@ static bool gemm_d16_at_ok(const GemmArgs &g) {
            (int64_t)g.K * g.lda < (1 << 30) && (int64_t)g.K * g.ldb < (1 << 30) &&
            (!g.scale || (g.ldcin % 4 == 0 && (uintptr_t)g.Cin % 16 == 0));
 }
-static int launch_d16_at(GemmArgs g, hipStream_t stream) {
+static int launch_d16_at(GemmArgs g, hipStream_t stream, float *workspace = nullptr, size_t workspace_bytes = 0) {
     const int cus = machine().cus;
     const int64_t t64 = (int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64), t32 = (int64_t)((g.M + 31) / 32) * ((g.N + 63) / 64);
     // 32-row tiles when they fill the CUs and 64-row tiles would leave most of them idle
@@ -1232,9 +1245,24 @@ static int launch_d16_at(GemmArgs g, hipStream_t stream) {
                        : (buf ? sgemm_direct16_at_kernel<4, true> : sgemm_direct16_at_kernel<4, false>);
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
         return T2SP_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(GEMM_D16_WAVES * 64), smem, stream, g.A, g.B, g.M, g.N, g.K, (int)g.lda,
-                       (int)g.ldb, g.tiles_m, g);
-    return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+    // a tiny output under a long reduction: as many shares of k per tile as fill the CUs, at least 32 steps each,
+    // given room for their planes
+    int shift = 0;
+    const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+    if (tiles <= cus / 2 && workspace && ((uintptr_t)workspace % 16 == 0)) {
+        while ((tiles << (shift + 1)) <= cus && ((g.K >> 4) >> (shift + 1)) >= 32 &&
+               ((size_t)g.M * g.N << (shift + 1)) * sizeof(float) <= workspace_bytes)
+            shift++;
+    }
+    g.scratch = workspace;
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n, 1 << shift), dim3(GEMM_D16_WAVES * 64), smem, stream, g.A, g.B, g.M, g.N, g.K,
+                       (int)g.lda, (int)g.ldb, g.tiles_m, shift, g);
+    if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
+    if (shift) {
+        GemmOutMap map{g};
+        if (launch_splitk_reduce<true>(workspace, 1 << shift, g.M, g.N, map, stream) != hipSuccess) return T2SP_ERR_LAUNCH;
+    }
+    return T2SP_OK;
 }
 
 // C[i][j] += alpha * sum_{k0 <= k < K} A(i, k) * B(k, j): the last 4, 8 or 12 steps of a reduction whose length is
@@ -1324,13 +1352,16 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         // loads need).  Any K: k is the row index of both operands.
         if (bt || (cfg != T2SP_CFG_AUTO && cfg != T2SP_CFG_DIRECT16)) return T2SP_ERR_SHAPE;
         if (cfg == T2SP_CFG_DIRECT16 || g.lda >= LOADER_MAX_LD || g.ldb >= LOADER_MAX_LD)
-            return gemm_d16_at_ok(g) ? launch_d16_at(g, stream) : T2SP_ERR_SHAPE;
+            return gemm_d16_at_ok(g) ? launch_d16_at(g, stream, workspace, workspace_bytes) : T2SP_ERR_SHAPE;
         {
             // small and middle-sized products: the one-launch form, as for the other layouts
             const int64_t t256 = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
             const int64_t t64 = (int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64);
             const int cus = machine().cus;
-            if (gemm_d16_at_ok(g) && t256 < cus * 25 / 32 && g.K >= 64 && !(t64 < cus / 8 && g.K >= 4096)) return launch_d16_at(g, stream);
+            // (a tiny output under a long reduction needs the room for two planes at least to split it there)
+            const bool can_split = workspace && workspace_bytes >= (size_t)g.M * g.N * 2 * sizeof(float);
+            if (gemm_d16_at_ok(g) && t256 < cus * 25 / 32 && g.K >= 64 && (can_split || !(t64 < cus / 8 && g.K >= 4096)))
+                return launch_d16_at(g, stream, workspace, workspace_bytes);
         }
         const GemmPlan p = plan_gemm(g.M, g.N, g.K, true);
         if (p.phased) {
@@ -1638,15 +1669,8 @@ extern "C" int t2sp_sgemm_ex_f32(int transa, int transb_given, int M, int N, int
     // (rows too far apart for the LDS-tile loaders' 32-bit offsets: only the 16 x 16 form, where it reaches)
     const bool at_far = lda >= t2sp::LOADER_MAX_LD || ldb >= t2sp::LOADER_MAX_LD;
     const bool at_far_ok = K % 16 == 0 && (int64_t)K * lda < (1 << 30) && (int64_t)K * ldb < (1 << 30);
-    bool native_at = at_possible && (cfg == T2SP_CFG_AUTO || cfg == T2SP_CFG_DIRECT16) && (!at_far || at_far_ok);
-    (void)t256;
-    // A tiny output under a long reduction: the plain form splits the reduction over workgroups, the A^T form's
-    // kernels do not do that as well (256 x 256 x 16384: 131 us against 26 us; 64 x 64 x 65536: 454 against 20), so
-    // with room for it A is brought to M x K after all.
-    if (native_at && cfg == T2SP_CFG_AUTO && room && K % 16 == 0 && aligned16(workspace)) {
-        const t2sp::GemmD16Split sp = t2sp::plan_gemm_d16_split(M, N, K, t2sp::plan_gemm_d16(M, N));
-        if (sp.shift > 0 && workspace_bytes >= t2sp::round_up256((size_t)M * K * sizeof(float)) + sp.scratch_bytes) native_at = false;
-    }
+    const bool native_at = at_possible && (cfg == T2SP_CFG_AUTO || cfg == T2SP_CFG_DIRECT16) && (!at_far || at_far_ok);
+    (void)t256; (void)room;
     if (transa && !native_at) {
         // A is stored K x M: bring it to M x K first (the loaders of the other kernels want k contiguous in A)
         if (!workspace || workspace_bytes < (size_t)M * K * sizeof(float)) {
