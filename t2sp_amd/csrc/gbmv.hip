@@ -58,19 +58,24 @@ __global__ void __launch_bounds__(64 * GBMV_ROWS_PER_WG) sgbmv3_kernel(const Gbm
                 s3 += av[3] * xv[3];
             }
         } else {
-            // 32-bit loads, lanes side by side, eight per lane in flight
-            float t0 = 0.f, t1 = 0.f, t2 = 0.f, t3 = 0.f;
-            int k = lane;
-            for (; k + 448 < g.K; k += 512) {
-                const float a0 = __builtin_nontemporal_load(a + k), a1 = __builtin_nontemporal_load(a + k + 64);
-                const float a2 = __builtin_nontemporal_load(a + k + 128), a3 = __builtin_nontemporal_load(a + k + 192);
-                const float a4 = __builtin_nontemporal_load(a + k + 256), a5 = __builtin_nontemporal_load(a + k + 320);
-                const float a6 = __builtin_nontemporal_load(a + k + 384), a7 = __builtin_nontemporal_load(a + k + 448);
-                s0 += a0 * x[k];       s1 += a1 * x[k + 64];  s2 += a2 * x[k + 128]; s3 += a3 * x[k + 192];
-                t0 += a4 * x[k + 256]; t1 += a5 * x[k + 320]; t2 += a6 * x[k + 384]; t3 += a7 * x[k + 448];
+            // K or lda not a multiple of 4: the row starts at any 4-byte boundary.  The first elements up to a 16-byte
+            // boundary and the last ones after the last whole group of four go one per lane; the groups between are
+            // read like the aligned form's, 128 bits per lane
+            const int head = (int)((4 - ((reinterpret_cast<uintptr_t>(a) >> 2) & 3)) & 3);
+            const int h = head < g.K ? head : g.K;
+            const int groups = (g.K - h) >> 2, rest = g.K - h - 4 * groups;
+            if (lane < h) s0 += a[lane] * x[lane];
+            if (lane < rest) s1 += a[h + 4 * groups + lane] * x[h + 4 * groups + lane];
+#pragma unroll 4
+            for (int q = lane; q < groups; q += 64) {
+                const int k = h + 4 * q;
+                const gbmv_v4f av = __builtin_nontemporal_load(reinterpret_cast<const gbmv_v4f *>(a + k));
+                const gbmv_v4f_u xv = *reinterpret_cast<const gbmv_v4f_u *>(x + k);
+                s0 += av[0] * xv[0];
+                s1 += av[1] * xv[1];
+                s2 += av[2] * xv[2];
+                s3 += av[3] * xv[3];
             }
-            for (; k < g.K; k += 64) s0 += a[k] * x[k];
-            s0 += t0; s1 += t1; s2 += t2; s3 += t3;
         }
         const float z = gbmv_wave_sum((s0 + s1) + (s2 + s3));
         if (lane == 0) {
