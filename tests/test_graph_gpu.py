@@ -108,3 +108,43 @@ def test_capsule_mttkrp_and_syrk_in_a_graph():
     ws = torch.empty(max(nb // 4, 1), device="cuda")
     assert replays_equal(torch, lambda st: L.t2sp_ssyrk_f32(1, 0, Ns, Ks, 1.0, As.data_ptr(), Ks, 0.0, None, 0, Cs.data_ptr(), Ns, 1, 0,
                                                             ws.data_ptr(), nb, st), Cs)
+
+
+@pytest.mark.parametrize("form,shape", [("NN", (516, 260, 1036)), ("NT", (256, 256, 16384)), ("TN", (256, 384, 8200)), ("TT", (260, 132, 2060)),
+                                        ("TT-beta", (260, 132, 2048)), ("NN", (4096, 4096, 256))])
+def test_multi_launch_sgemm_routes_in_a_graph(form, shape):
+    """Routes of several launches: the pass for a reduction off the 16 grid in every operand layout, the split of the
+    transposed forms with its sum kernel, the transposed result of the A^T * B^T form, B re-laid for it when a C is
+    read, and a launch that asks for more LDS than it needs (four 128 x 128 tiles per CU)."""
+    import torch
+    L = t2sp_amd.lib()
+    M, N, K = shape
+    ta, tb = form[0] == "T", form[1] == "T"
+    beta = 0.5 if form.endswith("beta") else 0.0
+    A = t2sp_amd.fill_uniform(torch.empty((K, M) if ta else (M, K), device="cuda"), 1)
+    B = t2sp_amd.fill_uniform(torch.empty((N, K) if tb else (K, N), device="cuda"), 2)
+    C0 = t2sp_amd.fill_uniform(torch.empty(M, N, device="cuda"), 3)
+    C = torch.empty(M, N, device="cuda")
+    nb = L.t2sp_sgemm_ex_workspace_bytes(int(ta), M, N, K)
+    ws = torch.empty(max(nb // 4, 4), device="cuda")
+
+    def launch(st):
+        assert L.t2sp_sgemm_ex_f32(int(ta), int(tb), M, N, K, 1.5, A.data_ptr(), M if ta else K, B.data_ptr(), K if tb else N, beta,
+                                   C0.data_ptr(), N, C.data_ptr(), N, 0, ws.data_ptr(), ctypes.c_size_t(nb), st) == 0
+    assert replays_equal(torch, launch, C)
+
+
+def test_syrk_routes_in_a_graph():
+    """SYRK's pass for a reduction off the 16 grid, and its 128 x 128 tiles one workgroup to a CU with the split rest."""
+    import torch
+    L = t2sp_amd.lib()
+    for N, K in ((768, 1028), (4096, 2048)):
+        A = t2sp_amd.fill_uniform(torch.empty(N, K, device="cuda"), 4)
+        C = torch.empty(N, N, device="cuda")
+        nb = L.t2sp_ssyrk_workspace_bytes(0, N, K)
+        ws = torch.empty(max(nb // 4, 4), device="cuda")
+
+        def launch(st):
+            assert L.t2sp_ssyrk_f32(1, 0, N, K, ctypes.c_float(0.5), A.data_ptr(), i64(K), ctypes.c_float(0.0), None, i64(0), C.data_ptr(),
+                                    i64(N), 1, 0, ws.data_ptr(), ctypes.c_size_t(nb), st) == 0
+        assert replays_equal(torch, launch, C)
