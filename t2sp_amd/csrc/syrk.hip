@@ -753,7 +753,11 @@ extern "C" size_t t2sp_ssyrk_workspace_bytes(int trans, int N, int K) {
         if (t.scratch_bytes > planes) planes = t.scratch_bytes;
     }
     // and, when K is not a multiple of 4, a zero-padded copy of A
-    return (trans ? (size_t)N * K * sizeof(float) : 0) + (K % 4 ? t2sp::syrk_padded_a_bytes(N, K) : 0) + planes;
+    const size_t own = (trans ? (size_t)N * K * sizeof(float) : 0) + (K % 4 ? t2sp::syrk_padded_a_bytes(N, K) : 0) + planes;
+    // (small results under a long reduction may run as an SGEMM: its planes)
+    const double nk = (double)N * K;
+    const size_t as_gemm = ((N <= 512 && K >= 1024) || (trans && nk * N * 7.2e-15 < 8e-6 + nk * 2e-12)) ? t2sp_sgemm_ex_workspace_bytes(trans ? 1 : 0, N, N, K) : 0;
+    return own > as_gemm ? own : as_gemm;
 }
 
 extern "C" size_t t2sp_ssyrk_folded_workspace_bytes(int trans, int N, int K) {
@@ -766,6 +770,24 @@ extern "C" int t2sp_ssyrk_f32(int upper, int trans, int N, int K, float alpha, c
                               int cfg, float *workspace, size_t workspace_bytes, void *stream) {
     if (lda < 0 || ldc < 0 || (Cin && ldcin < 0)) return T2SP_ERR_SHAPE;   // the loaders' offsets are unsigned
     if (N > T2SP_MAX_EXTENT || K > T2SP_MAX_EXTENT || !t2sp::strides_in_range(lda, ldc, ldcin)) return T2SP_ERR_SHAPE;
+    // A small result under a long reduction, wanted as the whole matrix: the SYRK kernels have few tiles for it and
+    // do not split a reduction over workgroups; the SGEMM forms do (A * A^T is its B^T form with both operands A, and
+    // A stored K x N its A^T form: no operand is re-laid), and at this size twice the multiplications cost less than
+    // idle CUs (N = 156, K = 7900: 48 -> 20 us).  Both halves come out the same to the bit: element (i, j) and
+    // element (j, i) add the same products in the same order.
+    const bool whole = mirror == 2 || (mirror == 1 && (beta == 0.f || !Cin));
+    // (and A stored K x N under a short reduction, up to N = 2048: the A^T form takes it as it lies, where the SYRK
+    // kernels need it re-laid first; N = 1324, K = 340: 34 -> 20 us)
+    // (where the other half of the multiplications, at about 130 TFLOP/s, costs less than re-laying A and its launch)
+    const double nk = (double)N * K;
+    const bool small_long = N <= 512 && K >= 1024, transposed_short = trans && K >= 64 && nk * N * 7.2e-15 < 8e-6 + nk * 2e-12;
+    if (cfg == T2SP_CFG_AUTO && whole && N > 0 && (small_long || transposed_short) && K % 4 == 0 && N % 4 == 0 && lda % 4 == 0 && ldc % 4 == 0 &&
+        ((uintptr_t)A % 16 == 0) && ((uintptr_t)C % 16 == 0) && (beta == 0.f || !Cin || (ldcin % 4 == 0 && (uintptr_t)Cin % 16 == 0)) &&
+        workspace && ((uintptr_t)workspace % 16 == 0)) {
+        const bool with_c = mirror == 2 && beta != 0.f && Cin;
+        return t2sp_sgemm_ex_f32(trans ? 1 : 0, trans ? 0 : 1, N, N, K, alpha, A, lda, A, lda, with_c ? beta : 0.f, with_c ? Cin : nullptr,
+                                 ldcin, C, ldc, T2SP_CFG_AUTO, workspace, workspace_bytes, stream);
+    }
     t2sp::SyrkArgs g{};
     g.A = A; g.lda = lda; g.N = N; g.K = K; g.alpha = alpha; g.beta = beta;
     g.Cin = beta != 0.f ? Cin : nullptr; g.ldcin = ldcin;

@@ -250,3 +250,31 @@ def test_reduction_off_the_16_grid_every_flat_form_exact(N, K):
             else:
                 want = prod - 3.0 * C0.double()
             assert torch.equal(C.double(), want), (upper, mirror)
+
+
+@pytest.mark.parametrize("N,K,trans", [(156, 7900, 0), (128, 4096, 0), (512, 1024, 0), (740, 1112, 1), (1324, 340, 1), (260, 2048, 1)])
+def test_small_whole_results_through_the_sgemm_forms_exact(N, K, trans):
+    """A small result under a long reduction, and A stored K x N under a short one, wanted as the whole matrix, run
+    as products of the SGEMM forms (with both operands A): mirror = 2 with C read at every element, mirror = 1
+    without a C.  Integer data: exact; both halves equal to the bit; one triangle alone (mirror = 0) must still
+    leave the other untouched (it takes the SYRK kernels)."""
+    import torch
+    L = t2sp_amd.lib()
+    g = torch.Generator().manual_seed(N + K)
+    A = torch.randint(-2, 3, (N, K), generator=g).float().cuda()
+    Ad = A.t().contiguous() if trans else A
+    C0 = torch.randint(-4, 5, (N, N), generator=g).float().cuda()
+    prod = 2.0 * (A.double() @ A.double().t())
+    nbytes = L.t2sp_ssyrk_workspace_bytes(trans, N, K)
+    ws = torch.empty(max(nbytes // 4, 4), device="cuda")
+    lda = N if trans else K
+    for mirror, beta, want in ((2, -3.0, prod - 3.0 * C0.double()), (1, 0.0, prod),
+                               (0, 0.0, torch.triu(prod) + torch.tril(C0.double(), -1))):
+        C = C0.clone()
+        rc = L.t2sp_ssyrk_f32(1, trans, N, K, ctypes.c_float(2.0), Ad.data_ptr(), ctypes.c_int64(lda), ctypes.c_float(beta), C.data_ptr(),
+                              ctypes.c_int64(N), C.data_ptr(), ctypes.c_int64(N), mirror, 0, ws.data_ptr(), ctypes.c_size_t(nbytes), None)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert torch.equal(C.double(), want), mirror
+        if mirror:
+            assert torch.equal(C, C.t()) or beta != 0.0
