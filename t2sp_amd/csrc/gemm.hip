@@ -443,6 +443,10 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
         }
     }
     __syncthreads();
+    // (the reference's tiled output with its innermost extent a multiple of NB, unit stride there and every other
+    // stride a multiple of NB: a lane's NB adjacent columns start at a multiple of NB and go out as one store)
+    const bool tiled_vec = g.tiled && g.s[0] == 1 && g.t_jjj % NB == 0 && ((g.s[1] | g.s[2] | g.s[3] | g.s[4] | g.s[5]) % NB) == 0 &&
+                           ((uintptr_t)g.C % (4 * NB)) == 0;
     // sum the partial tiles of the waves in wave order
 #pragma unroll
     for (int i = 0; i < PER_WAVE; i++) {
@@ -474,6 +478,8 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
                 }
                 if (!g.tiled) {
                     *reinterpret_cast<vnb *>(g.C + (int64_t)row * g.ldc + col) = out;
+                } else if (tiled_vec) {      // the NB adjacent columns lie inside one innermost tile, at an aligned address
+                    *reinterpret_cast<vnb *>(g.C + tiled_offset(g, row, col)) = out;
                 } else {
 #pragma unroll
                     for (int nb = 0; nb < NB; nb++) g.C[tiled_offset(g, row, col + nb)] = out[nb];
