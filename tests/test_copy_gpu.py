@@ -3,6 +3,7 @@ against.  Bit-exact by nature; the cases cover the 128-bit path, the scalar path
 the edges."""
 import ctypes
 
+import numpy as np
 import pytest
 
 import t2sp_amd
@@ -73,3 +74,61 @@ def test_relayout_general_box_bit_exact(dims):
     torch.cuda.synchronize()
     assert torch.equal(dst[:, :, :, :c], src[:, :, :, :d].permute(3, 1, 0, 2))
     assert (dst[:, :, :, c] == -1.0).all()
+
+
+def _relayout_against_torch(ext, perm_s, perm_d, pad_s, pad_d):
+    """Lays a box of extents `ext` out twice (dimension perm[0] fastest, its rows padded), re-lays one into the
+    other on the device and compares with torch's strided copy; the destination's padding must stay untouched."""
+    import torch
+    L = t2sp_amd.lib()
+    nd = len(ext)
+
+    def strides(perm, pad):
+        st, s = [0] * nd, 1
+        for k, d in enumerate(perm):
+            st[d] = s
+            s *= ext[d]
+            if k == 0:
+                s += pad
+        return st, s
+    ss, ns = strides(perm_s, pad_s)
+    ds, nds = strides(perm_d, pad_d)
+    src = torch.arange(ns, dtype=torch.float32, device="cuda")
+    dst = torch.full((nds,), -1.0, device="cuda")
+    want = dst.clone()
+    torch.as_strided(want, ext, ds).copy_(torch.as_strided(src, ext, ss))
+    i64 = ctypes.c_int64
+    assert L.t2sp_relayout_f32(src.data_ptr(), dst.data_ptr(), nd, (ctypes.c_int * nd)(*ext), (i64 * nd)(*ss),
+                               (i64 * nd)(*ds), None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(dst, want), (ext, ss, ds)
+
+
+def test_relayout_random_boxes_bit_exact():
+    """Boxes of 2 to 6 dimensions in random orders on both sides, extents that end inside tiles and inside the
+    lanes' runs, padded rows: whichever kernel the library picks, the result equals torch's strided copy."""
+    import random
+    rng = random.Random(7)
+    for _ in range(120):
+        nd = rng.randint(2, 6)
+        ext = [rng.choice([1, 2, 3, 5, 7, 8, 13, 16, 33, 70, 129, 300]) for _ in range(nd)]
+        while np.prod(ext) > 3_000_000:
+            ext[rng.randrange(nd)] = 2
+        ps, pd = list(range(nd)), list(range(nd))
+        rng.shuffle(ps)
+        rng.shuffle(pd)
+        _relayout_against_torch(ext, ps, pd, rng.choice([0, 0, 3]), rng.choice([0, 0, 2]))
+
+
+@pytest.mark.parametrize("consts", [
+    dict(COOO=8, COO=1, CO=4, YYY=7, XXX=1, YY=2, XX=2, Y=4, X=28, N=3),
+    dict(COOO=8, COO=2, CO=2, YYY=8, XXX=2, YY=2, XX=1, Y=3, X=5, N=2),
+    dict(COOO=4, COO=4, CO=4, YYY=4, XXX=4, YY=1, XX=1, Y=1, X=1, N=4),
+])
+def test_relayout_into_the_convolutions_tiled_output_bit_exact(consts):
+    """Flat (n, co, x, y) with y fastest into the reference's 10-D tiled output O(cooo, yyy, xxx, coo, yy, xx, y,
+    x, co, n) (conv-run-fpga.cpp:63-66): destination runs of 8 channels by a few pixels, source runs along y."""
+    c = consts
+    ext = [c[k] for k in ("COOO", "YYY", "XXX", "COO", "YY", "XX", "Y", "X", "CO", "N")]
+    # fastest-first orders: the destination's is the listed one, the source's is y, x, channels, n
+    _relayout_against_torch(ext, [1, 4, 6, 2, 5, 7, 0, 3, 8, 9], list(range(10)), 0, 0)
