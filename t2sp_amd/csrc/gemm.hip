@@ -40,7 +40,12 @@ struct GemmArgs {
     int tile_first, tile_count, compact;
     // A is stored transposed (K x M, lda >= M): taken as it lies by the kernels whose X tile is RC
     int at;
+    // > 0: the operands are zero-padded copies, N columns wide, of a product whose C has n_store columns at any
+    // leading dimension and alignment: the one-launch kernels store C's own columns one element at a time, and
+    // dispatch() launches nothing else (it returns GEMM_NOT_TAKEN)
+    int n_store;
 };
+constexpr int GEMM_NOT_TAKEN = 1;
 
 __device__ __forceinline__ int64_t tiled_offset(const GemmArgs &g, int row, int col) {
     const int jjj = col % g.t_jjj, cj = col / g.t_jjj;
@@ -430,7 +435,7 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
     // and written by its own workgroup only, so C may be updated in place)
     constexpr int PER_WAVE = (MB + NW - 1) / NW;
     vnb cin[PER_WAVE][4];
-    const bool with_cin = g.scale && g.beta != 0.f && !split_shift;
+    const bool with_cin = g.scale && g.beta != 0.f && !split_shift && !g.n_store;
     if (with_cin) {
 #pragma unroll
         for (int i = 0; i < PER_WAVE; i++) {
@@ -470,6 +475,12 @@ __global__ void __launch_bounds__(GEMM_D16_WAVES * 64)
                 if (split_shift) {
                     // a partial sum: plane blockIdx.z of the workspace, M x N; the kernel that adds the planes scales and stores
                     *reinterpret_cast<vnb *>(g.scratch + ((int64_t)share * M + row) * N + col) = out;
+                    continue;
+                }
+                if (g.n_store) {             // C narrower than the padded operands, rows at any alignment
+#pragma unroll
+                    for (int nb = 0; nb < NB; nb++)
+                        if (col + nb < g.n_store) gemm_store1(g, row, col + nb, out[nb]);
                     continue;
                 }
                 if (g.scale) {
@@ -823,6 +834,29 @@ __global__ void __launch_bounds__(256) gemm_pad_copy_kernel(const float *src, in
     }
 }
 
+// Two such copies in one launch (the operands of one product): grid rows [0, a_rows_p) are A's, the rest B's.  A thread
+// writes four adjacent elements of a padded row (padded widths are multiples of 4, the copies 16-byte aligned) from
+// four guarded 32-bit loads; no division anywhere.
+__global__ void __launch_bounds__(256) gemm_pad_copy2_kernel(const float *a, int64_t lda, float *a2, int a_rows, int a_cols, int a_rows_p,
+                                                             int a_cols_p, const float *b, int64_t ldb, float *b2, int b_rows,
+                                                             int b_cols, int b_rows_p, int b_cols_p) {
+    const int c = 4 * (blockIdx.x * 256 + threadIdx.x);
+    for (int y = blockIdx.y; y < a_rows_p + b_rows_p; y += gridDim.y) {
+        const bool is_a = y < a_rows_p;
+        const int r = is_a ? y : y - a_rows_p;
+        const int rows = is_a ? a_rows : b_rows, cols = is_a ? a_cols : b_cols, cols_p = is_a ? a_cols_p : b_cols_p;
+        if (c >= cols_p) continue;
+        const float *src = (is_a ? a + (int64_t)r * lda : b + (int64_t)r * ldb) + c;
+        v4f v{0.f, 0.f, 0.f, 0.f};
+        if (r < rows) {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (c + e < cols) v[e] = src[e];
+        }
+        *reinterpret_cast<v4f *>((is_a ? a2 : b2) + (int64_t)r * cols_p + c) = v;
+    }
+}
+
 // The product computed on padded operands goes to the caller's C, with the BLAS form's scaling.
 __global__ void __launch_bounds__(256) gemm_unpad_kernel(const float *src, int64_t ld, const GemmArgs g) {
     const int64_t total = (int64_t)g.M * g.N;
@@ -1129,10 +1163,11 @@ static GemmD16Split plan_gemm_d16_split(int M, int N, int K, const GemmD16Plan &
 }
 
 static bool gemm_d16_ok(const GemmArgs &g) {
-    return g.K % 16 == 0 && g.N % 4 == 0 && g.ldb % 4 == 0 && (g.tiled || g.ldc % 4 == 0) && g.lda % 4 == 0 &&
-           ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) && ((uintptr_t)g.C % 16 == 0) &&
-           (int64_t)g.M * g.lda < (1 << 30) && (int64_t)g.K * g.ldb < (1 << 30) &&
-           (!g.scale || (g.ldcin % 4 == 0 && (uintptr_t)g.Cin % 16 == 0));
+    const bool c_ok = g.n_store || ((g.tiled || g.ldc % 4 == 0) && ((uintptr_t)g.C % 16 == 0) &&
+                                    (!g.scale || (g.ldcin % 4 == 0 && (uintptr_t)g.Cin % 16 == 0)));
+    return g.K % 16 == 0 && g.N % 4 == 0 && g.ldb % 4 == 0 && c_ok && g.lda % 4 == 0 &&
+           ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
+           (int64_t)g.M * g.lda < (1 << 30) && (int64_t)g.K * g.ldb < (1 << 30);
 }
 
 template <int MB, int NB>
@@ -1163,7 +1198,7 @@ static int launch_d16_t(GemmArgs g, const GemmD16Plan &p, hipStream_t stream, in
 static int launch_d16(const GemmArgs &g, hipStream_t stream, float *workspace = nullptr, size_t workspace_bytes = 0) {
     const GemmD16Plan whole = plan_gemm_d16(g.M, g.N);
     GemmD16Split sp = plan_gemm_d16_split(g.M, g.N, g.K, whole);
-    if (!workspace || workspace_bytes < sp.scratch_bytes || ((uintptr_t)workspace % 16)) sp.shift = 0;
+    if (!workspace || workspace_bytes < sp.scratch_bytes || ((uintptr_t)workspace % 16) || g.n_store) sp.shift = 0;
     const int shift = sp.shift;
     const GemmD16Plan p = shift ? sp.tile : whole;
 #define T2SP_D16_CASE(MBV, NBV) if (p.mb == MBV && p.nb == NBV) return launch_d16_t<MBV, NBV>(g, p, stream, shift, workspace);
@@ -1218,7 +1253,7 @@ static int launch_d16_bt_t(GemmArgs g, const GemmD16Plan &p, hipStream_t stream,
 static int launch_d16_bt(const GemmArgs &g, hipStream_t stream, float *workspace = nullptr, size_t workspace_bytes = 0) {
     const GemmD16Plan whole = plan_gemm_d16_bt(g.M, g.N);
     GemmD16Split sp = plan_gemm_d16_split(g.M, g.N, g.K, plan_gemm_d16(g.M, g.N));     // (decided as for the plain form)
-    if (!workspace || workspace_bytes < sp.scratch_bytes || ((uintptr_t)workspace % 16) || g.N % 4 || g.tiled) sp.shift = 0;
+    if (!workspace || workspace_bytes < sp.scratch_bytes || ((uintptr_t)workspace % 16) || g.N % 4 || g.tiled || g.n_store) sp.shift = 0;
     const int shift = sp.shift;
     const GemmD16Plan p = shift ? sp.tile : whole;
 #define T2SP_D16_CASE(MBV, NBV) if (p.mb == MBV && p.nb == NBV) return launch_d16_bt_t<MBV, NBV>(g, p, stream, shift, workspace);
@@ -1334,8 +1369,13 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
                    (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) < machine().cus * 25 / 32))))) {   // (nearly a round of 128 x 128 tiles takes the tail as it comes)
         GemmArgs h = g;
         h.K = g.K - g.K % 16;
-        // (the direct kernel of 8-k steps takes its shapes as they are: 1000^3 20.9 us, 23.8 this way)
-        const bool direct = !bt && !g.at && !g.scale && g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && gemm_direct_ok(g, false);
+        // (the direct kernel of 8-k steps, 64 x 64 tiles, takes the shapes that fill one round of CUs with them as they
+        // are: 1000^3 20.9 us, 23.8 this way; 672 x 1320 x 1952, 231 tiles, 36.5 against 38.  Where its tiles leave CUs
+        // idle the one-launch form's choice of tile is worth more than the second pass costs: 888 x 1380 x 3032, 308
+        // tiles, 117 us against 75; 3636 x 512 x 1168, 456 tiles, 51 against 44; 136 x 4068 x 2608, 192 tiles, 46 against 38)
+        const int64_t t64 = (int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64);
+        const bool direct = !bt && !g.at && !g.scale && g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && gemm_direct_ok(g, false) &&
+                            t64 <= machine().cus && t64 >= machine().cus * 27 / 32;
         if (!direct && (g.at ? gemm_d16_at_ok(h) : bt ? gemm_d16_bt_ok(h) : gemm_d16_ok(h))) {
             const int rc = dispatch(h, cfg, bt, stream, workspace, workspace_bytes);
             if (rc != T2SP_OK) return rc;
@@ -1433,7 +1473,7 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
                                   (g.N <= 128 && t128 >= 2 * cus - cus / 16 && fill128 >= 0.9);
         // (with room for the planes the 16 x 16 form splits such a reduction over workgroups itself)
         const GemmD16Split sp = plan_gemm_d16_split(g.M, g.N, g.K, p);
-        const bool can_split = !bt && sp.shift && workspace && workspace_bytes >= sp.scratch_bytes && ((uintptr_t)workspace % 16 == 0);
+        const bool can_split = !bt && !g.n_store && sp.shift && workspace && workspace_bytes >= sp.scratch_bytes && ((uintptr_t)workspace % 16 == 0);
         // (without it, and without room for the planes of the LDS tiles' split either, it still has more tiles to
         // spread over the CUs than they have)
         const bool lds_split = workspace && workspace_bytes >= plan_gemm(g.M, g.N, g.K).scratch_bytes;
@@ -1445,6 +1485,7 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         if (!big_tiles && !tiled_better && !too_few && grid_ok && g.K >= 64)
             return bt ? launch_d16_bt(g, stream, workspace, workspace_bytes) : launch_d16(g, stream, workspace, workspace_bytes);
     }
+    if (g.n_store) return GEMM_NOT_TAKEN;
     if ((cfg == T2SP_CFG_AUTO || cfg == T2SP_CFG_DIRECT) && !bt && !g.scale && !g.tiled &&
         g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && gemm_direct_ok(g, cfg == T2SP_CFG_DIRECT))
         return launch_direct(g, stream);
@@ -1457,21 +1498,37 @@ static int dispatch(GemmArgs g, int cfg, bool bt, hipStream_t stream, float *wor
         // copy the result out.  Moving the matrices twice costs little next to the product.  (A K or
         // M, N that is merely not a multiple of the tile needs none of this: the guarded kernels
         // run at the rate of the unguarded ones.)
-        const int kp = (int)pad_k(g.K), np = bt ? g.N : (int)round_up4(g.N);
+        // A that the loaders can read where it lies (only N or the rows of B and C are off the grid) is not copied
+        const bool a_as_it_lies = g.K % 16 == 0 && g.lda % 4 == 0 && g.lda < LOADER_MAX_LD && ((uintptr_t)g.A % 16 == 0);
+        const int kp = a_as_it_lies ? g.K : (int)pad_k(g.K), np = bt ? g.N : (int)round_up4(g.N);
         float *a2 = workspace;
-        float *b2 = a2 + round_up256((size_t)g.M * kp * sizeof(float)) / sizeof(float);
-        float *c2 = b2 + round_up256((size_t)(bt ? (int64_t)g.N * kp : (int64_t)kp * np) * sizeof(float)) / sizeof(float);
+        float *b2 = a2 + round_up256((size_t)g.M * pad_k(g.K) * sizeof(float)) / sizeof(float);
+        float *c2 = b2 + round_up256((size_t)(bt ? (int64_t)g.N * pad_k(g.K) : (int64_t)pad_k(g.K) * np) * sizeof(float)) / sizeof(float);
         const size_t used = gemm_pad_bytes(g.M, g.N, g.K, bt);
         auto blocks = [](int64_t n) { return dim3((unsigned)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192)); };
-        hipLaunchKernelGGL(gemm_pad_copy_kernel, blocks((int64_t)g.M * kp), dim3(256), 0, stream, g.A, g.lda, a2, g.M, g.K, g.M, kp);
-        if (bt)
-            hipLaunchKernelGGL(gemm_pad_copy_kernel, blocks((int64_t)g.N * kp), dim3(256), 0, stream, g.B, g.ldb, b2, g.N, g.K, g.N, kp);
-        else
-            hipLaunchKernelGGL(gemm_pad_copy_kernel, blocks((int64_t)kp * np), dim3(256), 0, stream, g.B, g.ldb, b2, g.K, g.N, kp, np);
+        // both copies in one launch
+        const int b_rows = bt ? g.N : g.K, b_cols = bt ? g.K : g.N, b_rows_p = bt ? g.N : kp, b_cols_p = bt ? kp : np;
+        const int a_rows_p = a_as_it_lies ? 0 : g.M;
+        const int widest = kp > b_cols_p ? kp : b_cols_p, grid_rows = a_rows_p + b_rows_p;
+        hipLaunchKernelGGL(gemm_pad_copy2_kernel, dim3((unsigned)((widest + 1023) / 1024), (unsigned)(grid_rows < 65535 ? grid_rows : 65535)),
+                           dim3(256), 0, stream, g.A, g.lda, a2, g.M, g.K, a_rows_p, kp, g.B, g.ldb, b2, b_rows, b_cols, b_rows_p, b_cols_p);
         if (hipGetLastError() != hipSuccess) return T2SP_ERR_LAUNCH;
-        GemmArgs h{};
-        h.A = a2; h.B = b2; h.C = c2; h.M = g.M; h.N = np; h.K = kp;
-        h.lda = kp; h.ldb = bt ? kp : np; h.ldc = np;
+        GemmArgs h = g;
+        h.A = a_as_it_lies ? g.A : a2; h.B = b2; h.N = np; h.K = kp;
+        h.lda = a_as_it_lies ? g.lda : kp; h.ldb = bt ? kp : np;
+        const bool c_as_it_lies = np == g.N && !g.tiled && g.ldc % 4 == 0 && ((uintptr_t)g.C % 16 == 0) &&
+                                  (!g.scale || (g.ldcin % 4 == 0 && (uintptr_t)g.Cin % 16 == 0));
+        if (c_as_it_lies)          // only K, or the rows of A and B, were off the grid
+            return dispatch(h, T2SP_CFG_AUTO, bt, stream, workspace + used / sizeof(float), workspace_bytes - used);
+        if (!g.tiled) {
+            // the one-launch kernels store into C as it lies, whatever its width and alignment
+            h.n_store = g.N;
+            const int rc = dispatch(h, T2SP_CFG_AUTO, bt, stream, workspace + used / sizeof(float), workspace_bytes - used);
+            if (rc != GEMM_NOT_TAKEN) return rc;
+        }
+        h = GemmArgs{};
+        h.A = a_as_it_lies ? g.A : a2; h.B = b2; h.C = c2; h.M = g.M; h.N = np; h.K = kp;
+        h.lda = a_as_it_lies ? g.lda : kp; h.ldb = bt ? kp : np; h.ldc = np;
         const int rc = dispatch(h, T2SP_CFG_AUTO, bt, stream, workspace + used / sizeof(float), workspace_bytes - used);
         if (rc != T2SP_OK) return rc;
         hipLaunchKernelGGL(gemm_unpad_kernel, blocks((int64_t)g.M * g.N), dim3(256), 0, stream, c2, (int64_t)np, g);

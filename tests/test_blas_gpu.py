@@ -29,11 +29,15 @@ def test_alpha_beta_and_transposes(oracle, opa, opb, shape):
 
 
 @pytest.mark.parametrize("opa,opb", [(0, 0), (0, 1), (1, 0), (1, 1)])
-@pytest.mark.parametrize("shape", [(1001, 1003, 1005), (640, 513, 2050), (77, 130, 257)])
+@pytest.mark.parametrize("shape", [(1001, 1003, 1005), (640, 513, 2050), (77, 130, 257), (640, 512, 2050), (300, 1001, 1024),
+                                   (4099, 4101, 1030)])
 def test_odd_sizes_run_on_padded_copies(oracle, opa, opb, shape):
     """K or N not a multiple of 4: the operands are multiplied as zero-padded, aligned copies (as the
     reference's wrapper pads to tile multiples, blas-gemm.cpp:28-31); integer data, so the result is
-    exact whatever the order, with alpha, beta and C applied on the way out; inputs untouched."""
+    exact whatever the order, with alpha, beta and C applied on the way out; inputs untouched.  The
+    shapes cover the one-launch kernels storing into C as it lies, only K off the grid (C written in
+    place by any kernel), only N off it (A read where it lies) and an output large enough for the LDS
+    tiles, whose product goes through a padded C."""
     M, N, K = shape
     rng = np.random.default_rng(5)
     A = rng.integers(-2, 3, (M, K)).astype(np.float32)
