@@ -608,7 +608,8 @@ static int dispatch_syrk(SyrkArgs g, int trans, int cfg, float *workspace, size_
     if (g.N <= 0 || g.K <= 0) return T2SP_ERR_SHAPE;
     if (trans) {
         // A is stored K x N: bring it to N x K first (the MFMA loaders want k contiguous)
-        const size_t relaid = (size_t)g.N * g.K * sizeof(float);
+        // (a whole number of 128-bit groups, so that what follows it in the workspace stays aligned)
+        const size_t relaid = ((size_t)g.N * g.K + 3) / 4 * 4 * sizeof(float);
         if (!workspace || workspace_bytes < relaid) return T2SP_ERR_SHAPE;
         const int ext[2] = {g.K, g.N};
         const int64_t ss[2] = {g.lda, 1}, ds[2] = {1, g.K};
@@ -616,7 +617,7 @@ static int dispatch_syrk(SyrkArgs g, int trans, int cfg, float *workspace, size_
         if (rc != T2SP_OK) return rc;
         g.A = workspace;
         g.lda = g.K;
-        workspace += (size_t)g.N * g.K;      // what is left may hold the planes of a split last round
+        workspace += relaid / sizeof(float);      // what is left may hold the planes of a split last round
         workspace_bytes -= relaid;
     }
     // A the 128-bit loaders cannot read where it lies (K or its leading dimension not a multiple of 4,
@@ -640,7 +641,12 @@ static int dispatch_syrk(SyrkArgs g, int trans, int cfg, float *workspace, size_
     // Up to N = 2048 with K a multiple of 4 but not of 16: the one-launch kernel steps 16 k at a time, and the LDS
     // tiles that took such shapes are few and slow (N = 768, K = 1028: 39 us against 13 us at K = 1024).  The
     // product over the first K - K % 16 steps goes to the one-launch kernel; a second pass adds the rest.
-    if (cfg == T2SP_CFG_AUTO && g.K % 16 != 0 && g.K % 4 == 0 && g.K > 64 && g.N <= 2048 && g.mode != SYRK_FOLDED) {
+    // (and at any N where C's rows are not 16-byte aligned: the LDS tiles cannot store there, and the kernel of one thread
+    // per output that was left is a hundred times slower: N = 2921, K = 632: 12.4 ms)
+    const bool out_ok = g.mode == SYRK_FOLDED ||
+                        (g.ldc % 4 == 0 && (uintptr_t)g.C % 16 == 0 &&
+                         (!g.Cin || (g.ldcin % 4 == 0 && (uintptr_t)g.Cin % 16 == 0)));
+    if (cfg == T2SP_CFG_AUTO && g.K % 16 != 0 && g.K % 4 == 0 && g.K > 64 && (g.N <= 2048 || !out_ok) && g.mode != SYRK_FOLDED) {
         SyrkArgs h = g;
         h.K = g.K - g.K % 16;
         if (syrk_d16_ok(h)) {
@@ -651,9 +657,6 @@ static int dispatch_syrk(SyrkArgs g, int trans, int cfg, float *workspace, size_
             return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
         }
     }
-    const bool out_ok = g.mode == SYRK_FOLDED ||
-                        (g.ldc % 4 == 0 && (uintptr_t)g.C % 16 == 0 &&
-                         (!g.Cin || (g.ldcin % 4 == 0 && (uintptr_t)g.Cin % 16 == 0)));
     const bool vec_ok = out_ok && g.K % 4 == 0 && g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && g.lda < LOADER_MAX_LD;
     // Estimated cost of each LDS tile size, in units of one output element's reduction at the 256 tile's rate: the
     // number of rounds of 256 tiles (a last round whose reduction is split over the CUs counts 1/splits, plus a
@@ -682,7 +685,8 @@ static int dispatch_syrk(SyrkArgs g, int trans, int cfg, float *workspace, size_
     // K = 256, N = 2560 ... 8192: 64 tiles 4 to 18 % ahead of the next choice)
     const double c256 = cost(256, 1.0), c128 = cost(128, g.K >= 1024 ? 0.99 : 0.93),
                  c64 = cost(64, g.K <= 256 ? 0.95 : g.K <= 512 ? 0.85 : 0.78);
-    if (cfg == T2SP_CFG_AUTO && g.N <= SYRK_D16_MAX_N && g.K >= 64 && syrk_d16_ok(g)) {
+    // (an output the LDS tiles cannot store to goes to the one-launch kernel, which stores element by element, at any N)
+    if (cfg == T2SP_CFG_AUTO && (g.N <= SYRK_D16_MAX_N || !vec_ok) && g.K >= 64 && syrk_d16_ok(g)) {
         // The one-launch form up to N = 2048.  Above, it sustains about 122 TFLOP/s of the triangle's work whatever
         // the shape, and the LDS tiles pass it where their rounds come out even (measured at N = 2560 ... 5120:
         // K = 256 25 to 75 % ahead, K = 1024 up to 21 %; K = 4096: N = 4096 and 5120 15 and 11 % ahead, N = 2560
@@ -753,7 +757,7 @@ extern "C" size_t t2sp_ssyrk_workspace_bytes(int trans, int N, int K) {
         if (t.scratch_bytes > planes) planes = t.scratch_bytes;
     }
     // and, when K is not a multiple of 4, a zero-padded copy of A
-    const size_t own = (trans ? (size_t)N * K * sizeof(float) : 0) + (K % 4 ? t2sp::syrk_padded_a_bytes(N, K) : 0) + planes;
+    const size_t own = (trans ? ((size_t)N * K + 3) / 4 * 4 * sizeof(float) : 0) + (K % 4 ? t2sp::syrk_padded_a_bytes(N, K) : 0) + planes;
     // (small results under a long reduction may run as an SGEMM: its planes)
     const double nk = (double)N * K;
     const size_t as_gemm = ((N <= 512 && K >= 1024) || (trans && nk * N * 7.2e-15 < 8e-6 + nk * 2e-12)) ? t2sp_sgemm_ex_workspace_bytes(trans ? 1 : 0, N, N, K) : 0;

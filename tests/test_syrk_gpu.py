@@ -278,3 +278,31 @@ def test_small_whole_results_through_the_sgemm_forms_exact(N, K, trans):
         assert torch.equal(C.double(), want), mirror
         if mirror:
             assert torch.equal(C, C.t()) or beta != 0.0
+
+
+@pytest.mark.parametrize("N,K,trans", [(2921, 632, 0), (2357, 152, 0), (5335, 48, 0), (1319, 625, 1), (253, 2489, 1), (2705, 604, 1),
+                                       (593, 97, 1)])
+def test_rows_of_c_off_the_128_bit_grid_exact(N, K, trans):
+    """N not a multiple of 4 with C stored at leading dimension N: its rows are not 16-byte aligned, so the LDS
+    tiles cannot store there; the one-launch kernel (element stores) takes such outputs at any N, with the tail
+    pass for K off the 16 grid and a padded copy of A for K off the 4 grid; A stored K x N is re-laid first and
+    what follows it in the workspace must stay aligned.  Integer data: exact, for the mirrored pair without a C,
+    the full matrix with C read everywhere, and one triangle alone."""
+    import torch
+    L = t2sp_amd.lib()
+    g = torch.Generator().manual_seed(N + K)
+    A = torch.randint(-2, 3, (N, K), generator=g).float().cuda()
+    Ad = A.t().contiguous() if trans else A
+    C0 = torch.randint(-4, 5, (N, N), generator=g).float().cuda()
+    prod = 2.0 * (A.double() @ A.double().t())
+    nbytes = L.t2sp_ssyrk_workspace_bytes(trans, N, K)
+    ws = torch.empty(max(nbytes // 4, 4), device="cuda")
+    lda = N if trans else K
+    for mirror, beta, want in ((1, 0.0, prod), (2, -3.0, prod - 3.0 * C0.double()),
+                               (0, 0.0, torch.triu(prod) + torch.tril(C0.double(), -1))):
+        C = C0.clone()
+        rc = L.t2sp_ssyrk_f32(1, trans, N, K, ctypes.c_float(2.0), Ad.data_ptr(), ctypes.c_int64(lda), ctypes.c_float(beta), C.data_ptr(),
+                              ctypes.c_int64(N), C.data_ptr(), ctypes.c_int64(N), mirror, 0, ws.data_ptr(), ctypes.c_size_t(nbytes), None)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert torch.equal(C.double(), want), mirror
