@@ -280,6 +280,11 @@ int t2sp_conv2d_plan(int CO, int P, int KRED, int *stages16);
 int t2sp_conv2d_direct16_plan(int CO, int P, int KRED, int *out4, double *times2);
 int t2sp_ssyrk_plan(int N, int K, int b, int *total_tail_splits);
 int t2sp_capsule_direct16_plan(int rows, int cols, int *out6);
+/* The tile t2sp_relayout_f32's multi-dimensional kernel would take for a box: its extent along each of the nd
+ * dimensions, and the lanes (of 64) in use when reading and when writing; returns 1 when the box goes to that
+ * kernel, 0 when it goes to the transpose or the element-wise one. */
+int t2sp_relayout_plan(int nd, const int *extents, const int64_t *src_strides, const int64_t *dst_strides,
+                       int *tile_extents, int *lanes2);
 
 /* dst[sum_d c_d*dst_strides[d]] = src[sum_d c_d*src_strides[d]] for every coordinate c of the
  * box `extents` (nd <= T2SP_MAX_DIMS, dimension 0 fastest).  Device-side replacement of the

@@ -309,6 +309,18 @@ bool plan_pack(const RelayoutArgs &r, PackArgs &a) {
     }
     return stride <= PACK_LDS && tile_span_fits();
 }
+// A box for transpose_tile_kernel: r, a dimension contiguous in the destination, and c, one contiguous in the source,
+// both long enough to fill tiles.
+bool relayout_is_transpose(const RelayoutArgs &a, int *r_out, int *c_out) {
+    int r = -1, c = -1;
+    for (int d = 0; d < a.nd; d++) {
+        if (r < 0 && a.ds[d] == 1 && a.ext[d] >= 16) r = d;
+        if (c < 0 && a.ss[d] == 1 && a.ext[d] >= 16) c = d;
+    }
+    if (r_out) *r_out = r;
+    if (c_out) *c_out = c;
+    return r >= 0 && c >= 0 && r != c && a.ss[r] != 1;
+}
 // A plain copy: one 128-bit group per thread, read and written as a stream (nontemporal): 6.8 TB/s for 256 MiB
 // on the MI355X, against 6.1 without the hint and 5.3 to 5.8 with a grid-stride loop over fewer workgroups.
 typedef float copy_v4f __attribute__((ext_vector_type(4)));
@@ -336,6 +348,27 @@ extern "C" int t2sp_copy_f32(const float *src, float *dst, int64_t n, void *stre
     return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
 }
 
+// The tile the multi-dimensional kernel would take for a box (for tests of the planner, which runs on the host):
+// tile_extents[d] for each of the nd dimensions (1 for those outside the tile), lanes2 = the lanes in use when reading and
+// when writing.  Returns 1 when t2sp_relayout_f32 takes that kernel for the box, 0 when it takes another.
+extern "C" int t2sp_relayout_plan(int nd, const int *extents, const int64_t *src_strides, const int64_t *dst_strides,
+                                  int *tile_extents, int *lanes2) {
+    if (nd <= 0 || nd > T2SP_MAX_DIMS || !extents || !src_strides || !dst_strides || !tile_extents || !lanes2) return 0;
+    RelayoutArgs a{};
+    a.nd = nd; a.total = 1;
+    for (int d = 0; d < nd; d++) {
+        if (extents[d] <= 0) return 0;
+        a.ext[d] = extents[d]; a.ss[d] = src_strides[d]; a.ds[d] = dst_strides[d];
+        a.total *= extents[d];
+    }
+    if (relayout_is_transpose(a, nullptr, nullptr) || a.total < 4096) return 0;
+    PackArgs pk;
+    if (!plan_pack(a, pk)) return 0;
+    for (int d = 0, k = 0; d < nd; d++) tile_extents[d] = extents[d] > 1 ? pk.te[k++] : 1;
+    lanes2[0] = pk.rd.p_lo; lanes2[1] = pk.wr.p_lo;
+    return 1;
+}
+
 extern "C" int t2sp_relayout_f32(const float *src, float *dst, int nd, const int *extents,
                                  const int64_t *src_strides, const int64_t *dst_strides,
                                  void *stream) {
@@ -349,13 +382,8 @@ extern "C" int t2sp_relayout_f32(const float *src, float *dst, int nd, const int
         a.total *= extents[d];
     }
     if (a.total == 0) return T2SP_OK;
-    // r: a dimension contiguous in the destination, c: one contiguous in the source; both long enough to fill tiles
     int r = -1, c = -1;
-    for (int d = 0; d < nd; d++) {
-        if (r < 0 && a.ds[d] == 1 && a.ext[d] >= 16) r = d;
-        if (c < 0 && a.ss[d] == 1 && a.ext[d] >= 16) c = d;
-    }
-    if (r >= 0 && c >= 0 && r != c && a.ss[r] != 1) {
+    if (relayout_is_transpose(a, &r, &c)) {
         const int64_t tiles = (int64_t)((a.ext[r] + 63) / 64) * ((a.ext[c] + 63) / 64) * (a.total / a.ext[r] / a.ext[c]);
         if (tiles <= INT32_MAX) {
             hipLaunchKernelGGL(transpose_tile_kernel, dim3((unsigned)tiles), dim3(256), 0, (hipStream_t)stream, a, r, c);

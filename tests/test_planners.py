@@ -227,3 +227,60 @@ def test_planners_take_extreme_extents(lib):
         L.t2sp_conv2d_workspace_bytes(pick() % 4096 + 1, pick() % 4096 + 1, pick() % 4096 + 1, pick() % 4096 + 1,
                                       pick() % 4096 + 1, 3, 3)
     assert time.time() - t0 < 60
+
+
+def _relayout_plan(L, ext, ss, ds):
+    nd = len(ext)
+    i64 = ctypes.c_int64
+    L.t2sp_relayout_plan.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(i64), ctypes.POINTER(i64),
+                                     ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
+    te, lanes = (ctypes.c_int * nd)(), (ctypes.c_int * 2)()
+    took = L.t2sp_relayout_plan(nd, (ctypes.c_int * nd)(*ext), (i64 * nd)(*ss), (i64 * nd)(*ds), te, lanes)
+    return took, list(te), list(lanes)
+
+
+def _strides(ext, order):
+    st, s = [0] * len(ext), 1
+    for d in order:
+        st[d] = s
+        s *= ext[d]
+    return st
+
+
+def test_relayout_tiles_cover_the_runs_of_both_sides(lib):
+    """The multi-dimensional relayout tile: for the convolution's 10-D tiled output (8 channels, then 7 pixels
+    innermost; source rows along the pixels) it is whole along the destination's channel and pixel groups and
+    along the source's row, so that 56 of 64 lanes work on both sides; it never exceeds 4096 elements or a
+    dimension's extent; plain transposes and tiny boxes go to the other kernels."""
+    # cooo, yyy, xxx, coo, yy, xx, y, x, co, n  (fastest first in the destination); source order y.., x.., channels, n
+    ext = [8, 7, 1, 1, 2, 2, 4, 28, 32, 16]
+    src_order = [1, 4, 6, 2, 5, 7, 0, 3, 8, 9]
+    took, te, lanes = _relayout_plan(lib, ext, _strides(ext, src_order), _strides(ext, range(10)))
+    assert took == 1
+    assert te[0] == 8 and te[1] == 7 and te[4] == 2 and te[6] == 4          # channels x the whole source row of 56
+    assert lanes == [56, 56]
+    elems = 1
+    for t, e in zip(te, ext):
+        assert 1 <= t <= e
+        elems *= t
+    assert 2048 < elems <= 4096
+    # a 2-D transpose belongs to the 64 x 64 tile kernel, a box under 4096 elements to the element-wise one
+    assert _relayout_plan(lib, [1000, 300], [300, 1], [1, 1000])[0] == 0
+    assert _relayout_plan(lib, [8, 7, 5], _strides([8, 7, 5], [1, 2, 0]), _strides([8, 7, 5], [0, 1, 2]))[0] == 0
+    # strides that are not positive are not for it
+    assert _relayout_plan(lib, [64, 64, 8], [0, 64, 4096], [1, 64, 4096])[0] == 0
+    import random
+    rng = random.Random(3)
+    for _ in range(300):
+        nd = rng.randint(2, 8)
+        ext = [rng.choice([1, 2, 3, 4, 7, 8, 15, 16, 33, 100, 1000]) for _ in range(nd)]
+        so, do = list(range(nd)), list(range(nd))
+        rng.shuffle(so)
+        rng.shuffle(do)
+        took, te, lanes = _relayout_plan(lib, ext, _strides(ext, so), _strides(ext, do))
+        if took:
+            elems = 1
+            for t, e in zip(te, ext):
+                assert 1 <= t <= e
+                elems *= t
+            assert elems <= 4096 and 1 <= lanes[0] <= 64 and 1 <= lanes[1] <= 64
