@@ -286,6 +286,17 @@ int t2sp_capsule_direct16_plan(int rows, int cols, int *out6);
 int t2sp_relayout_plan(int nd, const int *extents, const int64_t *src_strides, const int64_t *dst_strides,
                        int *tile_extents, int *lanes2);
 
+/* The capsule convolution on the reference's packed 2-D operands, read where they lie (the call form of
+ * t2s/tests/performance/capsule/capsule-run-gpu.cpp:38-39,67-69, layouts of capsule.cpp:52-53):
+ * P2(ci + CI*mk + CI*4*mx + CI*16*nn, iy + 15*ix + 225*n) with row stride ldp,
+ * W2(co + CO*my, cii + CII*ky + CII*3*kx + CII*9*ci_o + CI*9*mk) with row stride ldw, and
+ * V(co + CO*my + CO*4*mx + CO*16*nn, oy + 7*ox + 49*n) with row stride ldv.
+ * Returns 1, having launched nothing, when the library's plan for the size is another kernel or the operands
+ * do not suit this one: the caller then re-lays them (t2sp_relayout_f32) and calls t2sp_capsule_f32, which is
+ * what the operator entry `capsule` does. */
+int t2sp_capsule_packed_f32(const float *P2, int64_t ldp, const float *W2, int64_t ldw, float *V, int64_t ldv,
+                            int N, int NN, int CI, int CO, int CII, void *stream);
+
 /* dst[sum_d c_d*dst_strides[d]] = src[sum_d c_d*src_strides[d]] for every coordinate c of the
  * box `extents` (nd <= T2SP_MAX_DIMS, dimension 0 fastest).  Device-side replacement of the
  * host serializer/deserializer loops the reference's generated interface runs around its

@@ -28,6 +28,15 @@ struct CapsuleArgs {
     int ROWS, COLS, KRED;   // N*OH*OW*MX, CO*4, CI*KH*KW*4
     int tiles_m, tiles_n, splits, Mp, Np;
     float *scratch;
+    // The reference's packed 2-D operands read where they lie by the 16 x 16 direct kernel (pk_nn > 0):
+    //   P(ci + CI*mk + CI*4*mx + CI*16*nn, iy + 15*ix + 225*n), W(co + CO*my, cii + CII*ky + CII*3*kx + CII*9*ci_o + CI*9*mk).
+    // Image n_total = nn + pk_nn * n lies at nn * pk_p_nn + n * sp[0] (votes: nn * pk_v_nn + n * sv[0]).  A lane's four
+    // reduction values are four adjacent ci (contiguous in both operands) instead of the four mk, so a "pose row" is
+    // (ci / 4, mk, kh, kw), walked with ci / 4 fastest; sp[2], sp[3] and sw[2], sw[3] are the strides of the window,
+    // sp[4] that of mx, sw[4] the row stride of W (one ci further), and column c of the product is W's column c.
+    // The votes go to V(column + 4*CO*mx + 16*CO*nn, pixel), column by column as W has them.
+    int pk_nn, pk_cii;
+    int64_t pk_p_nn, pk_v_nn;
 };
 
 struct CapsuleOutMap {
@@ -421,7 +430,7 @@ __device__ __forceinline__ void direct16_wave(const CapsuleArgs &g, int mb0, int
     for (int nb = 0; nb < NB; nb++) {
         const int col = n0 + 16 * nb + li;
         const int co = col < g.COLS ? col >> 2 : 0;
-        w_lane[nb] = 4u * (uint32_t)(co * (int)g.sw[0] + (li & 3));
+        w_lane[nb] = g.pk_nn > 0 ? 4u * (uint32_t)(col < g.COLS ? col : 0) : 4u * (uint32_t)(co * (int)g.sw[0] + (li & 3));
     }
     const char *p_base = reinterpret_cast<const char *>(g.P);
     const char *w_base[4];
@@ -519,9 +528,10 @@ __global__ void __launch_bounds__(D16_WAVES * D16_ROWSPLIT * 64)
     if (wave == NW * RS - 1 && lane < 4 * MB) {
         const int t = lane;
         const int pix = pix0 + (t < pix_n ? t : 0);
-        const int w = pix % g.OW, hn = pix / g.OW, h = hn % g.OH, n = hn / g.OH;
-        pix_p[t] = 4u * (uint32_t)(int)(n * g.sp[0] + h * g.S * g.sp[2] + w * g.S * g.sp[3]);
-        pix_v[t] = t < pix_n ? 4u * (uint32_t)(int)(n * g.sv[0] + h * g.sv[2] + w * g.sv[3]) : ~0u;
+        const int w = pix % g.OW, hn = pix / g.OW, h = hn % g.OH, nt = hn / g.OH;
+        const int group = g.pk_nn > 0 ? g.pk_nn : 1, nn = nt % group, n = nt / group;      // (nn = 0 for tensors with one image index)
+        pix_p[t] = 4u * (uint32_t)(int)(nn * g.pk_p_nn + n * g.sp[0] + h * g.S * g.sp[2] + w * g.S * g.sp[3]);
+        pix_v[t] = t < pix_n ? 4u * (uint32_t)(int)(nn * g.pk_v_nn + n * g.sv[0] + h * g.sv[2] + w * g.sv[3]) : ~0u;
     }
     // steps [s0, s1) of 4 pose rows each belong to share kq; byte offsets of its pose rows, filled
     // by the first wave of the pair (rows past the end repeat the last one)
@@ -532,6 +542,14 @@ __global__ void __launch_bounds__(D16_WAVES * D16_ROWSPLIT * 64)
     if (rh == 0)
         for (int i = lane; i < 4 * nsteps + 4 * R; i += 64) {
             const int q = min(4 * s0 + i, Q - 1);
+            if (g.pk_nn > 0) {
+                const int c4n = g.CI >> 2, c4 = q % c4n, t1 = q / c4n, mk = t1 & 3, t2 = t1 >> 2;
+                const int kh = t2 / g.KW, kw = t2 - kh * g.KW;
+                const int ci = 4 * c4, w_row = ci % g.pk_cii + g.pk_cii * (g.KH * g.KW * (ci / g.pk_cii)) + g.CI * g.KH * g.KW * mk;
+                tab[i] = uint2{4u * (uint32_t)(ci + g.CI * mk + kh * (int)g.sp[2] + kw * (int)g.sp[3]),
+                               4u * (uint32_t)(w_row * (int)g.sw[4] + kh * (int)g.sw[2] + kw * (int)g.sw[3])};
+                continue;
+            }
             const int c = q / (g.KH * g.KW), r = q - c * (g.KH * g.KW);
             const int kh = r / g.KW, kw = r - kh * g.KW;
             tab[i] = uint2{4u * (uint32_t)(c * (int)g.sp[1] + kh * (int)g.sp[2] + kw * (int)g.sp[3]),
@@ -555,7 +573,7 @@ __global__ void __launch_bounds__(D16_WAVES * D16_ROWSPLIT * 64)
         const uint32_t pv = pix_v[4 * mb + lq];
         const int col = n0 + 16 * nb + li;
         if (pv != ~0u && col < g.COLS) {
-            const uint32_t v_lane = 4u * (uint32_t)((col >> 2) * (int)g.sv[1] + (li & 3));
+            const uint32_t v_lane = g.pk_nn > 0 ? 4u * (uint32_t)col : 4u * (uint32_t)((col >> 2) * (int)g.sv[1] + (li & 3));
 #pragma unroll
             for (int r = 0; r < 4; r++) *reinterpret_cast<float *>(v_base + (pv + v_lane + r * mx_stride)) = sum[r];
         }
@@ -935,4 +953,38 @@ extern "C" int t2sp_capsule_f32(const float *P, const float *W, float *V, const 
         case T2SP_CFG_32x128: return launch_capsule<CapsW>(g, (hipStream_t)stream, w_dense);
         default: return T2SP_ERR_SHAPE;
     }
+}
+
+// The 16 x 16 direct kernel on the reference's packed operands, read where they lie (capsule.cpp:52-53; the
+// layouts are spelled out at CapsuleArgs::pk_nn): P2 with row stride ldp, W2 with row stride ldw, and the GPU flow's
+// V(co + CO*my + CO*4*mx + CO*16*nn, oy + 7*ox + 49*n) with row stride ldv.  7 x 7 votes of 3 x 3 windows at stride
+// 2, 4 x 4 poses.  Returns 1, having launched nothing, when the library's plan for this size is another kernel or
+// the operands do not suit this one (the caller re-lays them and calls t2sp_capsule_f32).
+extern "C" int t2sp_capsule_packed_f32(const float *P2, int64_t ldp, const float *W2, int64_t ldw, float *V, int64_t ldv,
+                                       int N, int NN, int CI, int CO, int CII, void *stream) {
+    using namespace t2sp;
+    constexpr int OYX = 7, KYX = 3, S = 2, IYX = 15, M = 4;
+    if (N <= 0 || NN <= 0 || CI <= 0 || CO <= 0 || CII <= 0 || ldp <= 0 || ldw <= 0 || ldv <= 0) return T2SP_ERR_SHAPE;
+    const int64_t nt = (int64_t)N * NN, rows = nt * OYX * OYX * M, cols = (int64_t)CO * M, kred = (int64_t)CI * KYX * KYX * M;
+    if (rows > T2SP_MAX_EXTENT || cols > T2SP_MAX_EXTENT || kred > T2SP_MAX_EXTENT) return 1;
+    if (CI % 4 || CII % 4 || CI % CII || ldp % 4 || ldw % 4 || ldv % 4 || ((uintptr_t)P2 % 16) || ((uintptr_t)W2 % 16) || ((uintptr_t)V % 16))
+        return 1;
+    // 32-bit byte offsets
+    const int64_t span_p = (int64_t)IYX * IYX * N * ldp, span_w = (int64_t)CI * KYX * KYX * M * ldw, span_v = (int64_t)OYX * OYX * N * ldv;
+    if (span_p >= (1 << 30) || span_w >= (1 << 30) || span_v >= (1 << 30)) return 1;
+    const int d[11] = {(int)nt, CI, CO, OYX, OYX, KYX, KYX, S, M, M, M};
+    if (capsule_staged_images(d, rows, cols, kred)) return 1;
+    const CapsulePlan p = plan_capsule((int)rows, (int)cols, (int)kred, T2SP_CFG_AUTO, 0, M);
+    if (p.cfg != T2SP_CFG_DIRECT16 || direct16_smem_bytes(D16_MAX_MB, 2, (int)kred) > 160 * 1024) return 1;
+    CapsuleArgs g{};
+    g.P = P2; g.W = W2; g.V = V;
+    g.N = (int)nt; g.CI = CI; g.CO = CO; g.OH = OYX; g.OW = OYX; g.KH = KYX; g.KW = KYX; g.S = S; g.MX = M;
+    // h is the x of the reference's names, w its y (the pipeline's pixel index is oy + OY*ox, capsule.cpp:38-39)
+    g.sp[0] = (int64_t)IYX * IYX * ldp; g.sp[2] = IYX * ldp; g.sp[3] = ldp; g.sp[4] = (int64_t)M * CI;
+    g.sw[2] = (int64_t)CII * KYX * ldw; g.sw[3] = (int64_t)CII * ldw; g.sw[4] = ldw;
+    g.sv[0] = (int64_t)OYX * OYX * ldv; g.sv[2] = OYX * ldv; g.sv[3] = ldv; g.sv[4] = (int64_t)CO * M;
+    g.pk_nn = NN; g.pk_cii = CII; g.pk_p_nn = (int64_t)M * M * CI; g.pk_v_nn = (int64_t)CO * M * M;
+    g.ROWS = (int)rows; g.COLS = (int)cols; g.KRED = (int)kred;
+    g.splits = 1; g.Mp = p.Mp; g.Np = p.Np;
+    return launch_capsule_direct16(g, (hipStream_t)stream);
 }

@@ -1,6 +1,8 @@
 """GPU parity tests of the capsule convolution path through `capsule`
 (include/capsule-interface.h).  Arrays are indexed P (n,ci,y,x,mx,mk), W (co,ci,ky,kx,mk,my),
 V (n,co,y,x,mx,my), the oracle's convention."""
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -184,7 +186,9 @@ def test_reference_packed_call_form(oracle, design, N):
     V2 = np.full((49 * N, TCO * 16 * c["NN"]), np.nan, np.float32)
     t2sp_amd.capsule_packed(P2, W2, V2, c["CII"])
     got = V2.reshape(N, 7, 7, c["NN"], 4, 4, TCO).transpose(0, 3, 6, 2, 1, 4, 5).reshape(NT, TCO, 7, 7, 4, 4)
-    assert (got == votes).all()
+    # (for this output the packed operands are read where they lie, four adjacent ci per lane where the other forms
+    # read four mk: the same products added in another order)
+    assert rel_fro(got, ref)[0] <= TOL and rel_fro(got, votes)[0] <= TOL
 
 
 def test_packed_form_needs_its_design_constant_and_consistent_extents(oracle):
@@ -242,3 +246,43 @@ def test_large_batches_on_lds_tiles_sampled_images(oracle, batch):
         Wg.copy_(W)
         assert not Wg.is_contiguous()
         assert torch.equal(t2sp_amd.capsule(P, Wg), V) or rel_fro(t2sp_amd.capsule(P, Wg).cpu().numpy(), V.cpu().numpy())[0] <= 1e-6
+
+
+@pytest.mark.parametrize("design,N", [("TINY", 4), ("GPU", 2), ("S10", 3), ("A10", 2)])
+def test_packed_operands_read_where_they_lie_exact(oracle, design, N):
+    """t2sp_capsule_packed_f32: the one-launch kernel on the reference's packed P and W (capsule.cpp:52-53) and the
+    GPU flow's 2-D V, nothing re-laid, for the four constant sets (CII = 4, 16 and 32: the weights' rows are ordered
+    by it), a row stride of V wider than its rows, device tensors.  Integer data, so the sums are exact whatever
+    their order; V's padding stays untouched; operands the kernel cannot take are declined (return value 1) with
+    nothing written."""
+    import torch
+    c = CAPSULE_DESIGNS[design]
+    TCI, TCO, NN = c["CII"] * c["CI"], c["COOO"] * c["COO"] * c["CO"], c["NN"]
+    NT = NN * N
+    rng = np.random.default_rng(N + TCI)
+    P = rng.integers(-2, 3, (NT, TCI, 15, 15, 4, 4)).astype(np.float32)
+    W = rng.integers(-2, 3, (TCO, TCI, 3, 3, 4, 4)).astype(np.float32)
+    ref = oracle.capsule(P, W)
+    P2, W2 = pack_capsule_inputs(P, W, NN, c["CII"])
+    L = t2sp_amd.lib()
+    i64 = ctypes.c_int64
+    L.t2sp_capsule_packed_f32.argtypes = [ctypes.c_void_p, i64, ctypes.c_void_p, i64, ctypes.c_void_p, i64] + [ctypes.c_int] * 5 + [ctypes.c_void_p]
+    dP, dW = torch.from_numpy(P2).cuda(), torch.from_numpy(W2).cuda()
+    ldv = TCO * 16 * NN + 8
+    dV = torch.full((49 * N, ldv), -7.0, device="cuda")
+    rc = L.t2sp_capsule_packed_f32(dP.data_ptr(), P2.shape[1], dW.data_ptr(), W2.shape[1], dV.data_ptr(), ldv, N, NN, TCI, TCO,
+                                   c["CII"], None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    V2 = dV.cpu().numpy()
+    got = V2[:, :TCO * 16 * NN].reshape(N, 7, 7, NN, 4, 4, TCO).transpose(0, 3, 6, 2, 1, 4, 5).reshape(NT, TCO, 7, 7, 4, 4)
+    assert (got == ref).all()
+    assert (V2[:, TCO * 16 * NN:] == -7.0).all()
+    # a row stride of P that is not a multiple of 4, or a CII that does not divide into groups of 4: declined
+    dV.fill_(-7.0)
+    assert L.t2sp_capsule_packed_f32(dP.data_ptr(), P2.shape[1] + 1, dW.data_ptr(), W2.shape[1], dV.data_ptr(), ldv, N, NN, TCI, TCO,
+                                     c["CII"], None) == 1
+    assert L.t2sp_capsule_packed_f32(dP.data_ptr(), P2.shape[1], dW.data_ptr(), W2.shape[1], dV.data_ptr(), ldv, N, NN, TCI, TCO,
+                                     2, None) == 1
+    torch.cuda.synchronize()
+    assert (dV == -7.0).all()
