@@ -284,3 +284,24 @@ def test_relayout_tiles_cover_the_runs_of_both_sides(lib):
                 assert 1 <= t <= e
                 elems *= t
             assert elems <= 4096 and 1 <= lanes[0] <= 64 and 1 <= lanes[1] <= 64
+
+
+def test_packed_capsule_entry_declines_before_any_launch(lib):
+    """t2sp_capsule_packed_f32 checks its operands on the host: sizes that are not positive are errors, strides or
+    addresses off the 128-bit grid, a CII that is not a multiple of 4 or does not divide CI, and batches the library
+    plans another kernel for (thousands of images: LDS tiles) are declined with 1; nothing is launched in either case,
+    so the call is safe without a device."""
+    lib.t2sp_set_machine(256, 8)
+    i64 = ctypes.c_int64
+    f = lib.t2sp_capsule_packed_f32
+    f.argtypes = [ctypes.c_void_p, i64, ctypes.c_void_p, i64, ctypes.c_void_p, i64] + [ctypes.c_int] * 5 + [ctypes.c_void_p]
+    P, W, V = 0x10000, 0x20000, 0x30000          # never dereferenced on these paths
+    ldp, ldw, ldv = 16 * 16 * 32, 4 * 32, 32 * 16 * 16
+    assert f(P, ldp, W, ldw, V, ldv, 0, 16, 32, 32, 4, None) == -8
+    assert f(P, ldp, W, ldw, V, 0, 2, 16, 32, 32, 4, None) == -8
+    assert f(P, ldp + 2, W, ldw, V, ldv, 2, 16, 32, 32, 4, None) == 1
+    assert f(P + 4, ldp, W, ldw, V, ldv, 2, 16, 32, 32, 4, None) == 1
+    assert f(P, ldp, W, ldw, V, ldv, 2, 16, 32, 32, 6, None) == 1
+    assert f(P, ldp, W, ldw, V, ldv, 2, 16, 32, 32, 64, None) == 1
+    assert f(P, ldp, W, ldw, V, ldv, 2, 16, 30, 32, 2, None) == 1
+    assert f(P, ldp, W, ldw, V, ldv, 256, 16, 32, 32, 4, None) == 1          # 4096 images: rounds of LDS tiles
