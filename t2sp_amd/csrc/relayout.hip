@@ -101,12 +101,13 @@ struct PackArgs {
     int lstride[T2SP_MAX_DIMS];                       // a tile element's place in LDS: sum digit * lstride
     int n_tile;                                       // dimensions with te > 1
     unsigned tiles;                                   // tiles of the whole box
+    int even;                                         // the lanes' steps along both split dimensions divide the tile's extent
     PackOrder rd, wr;
 };
 constexpr int PACK_TILE = 4096, PACK_LDS = PACK_TILE + 128, PACK_TABLE = 128, PACK_BATCH = 8;
 struct PackTable {
-    int off[PACK_TABLE];          // -1: outside the box (offsets inside a tile fit 31 bits: plan_pack checks)
-    int lds[PACK_TABLE];
+    int2 ol[PACK_TABLE];          // .x: offset in the tensor, -1: outside the box (offsets inside a tile fit 31 bits:
+                                  // plan_pack checks); .y: place in the LDS tile
     int split[PACK_TABLE];        // this entry's position along the split dimension
 };
 struct PackShared {
@@ -139,8 +140,7 @@ __device__ __forceinline__ PackLane pack_offsets(const PackArgs &a, const PackOr
             off += i * (int)stride[d];
             l += i * a.lstride[d];
         }
-        tb.off[h] = ok ? off : -1;
-        tb.lds[h] = l;
+        tb.ol[h] = int2{ok ? off : -1, l};
         tb.split[h] = split;
     }
     PackLane r{0, 0, 0, 1 << 30, (int)(threadIdx.x & 63) < o.p_lo};
@@ -201,34 +201,72 @@ __global__ void __launch_bounds__(256) pack_tile_kernel(const PackArgs) {
             __syncthreads();
         }
         const float *src = a.src + base_s + rl.off;
+        float *dst = a.dst + base_d + wl.off;
         // eight loads in flight per lane: one at a time, a tile's few dozen steps would cost a memory latency each
-        for (int h0 = wave; h0 < r_hi; h0 += 4 * PACK_BATCH) {
-            float v[PACK_BATCH];
-            bool in[PACK_BATCH];
+        if (!edge && a.even) {
+            // a whole tile whose split dimensions divide evenly: every table entry and every lane in use is inside
+            // the box, and the loops are a table read, a load and a store (the checks below are most of the
+            // instructions of the general loops)
+            if (rl.ok)
+                for (int h0 = wave; h0 < r_hi; h0 += 4 * PACK_BATCH) {
+                    float v[PACK_BATCH];
+                    int at[PACK_BATCH];
 #pragma unroll
-            for (int u = 0; u < PACK_BATCH; u++) {
-                const int h = h0 + 4 * u;
-                in[u] = false;
-                if (h < r_hi) {
-                    const int o = sh.rd.off[h];
-                    in[u] = rl.ok && o >= 0 && rl.split + sh.rd.split[h] < rl.split_end;
-                    if (in[u]) v[u] = __builtin_nontemporal_load(src + o);
+                    for (int u = 0; u < PACK_BATCH; u++) {
+                        const int h = h0 + 4 * u;
+                        if (h < r_hi) {
+                            const int2 e = sh.rd.ol[h];
+                            at[u] = e.y;
+                            v[u] = __builtin_nontemporal_load(src + e.x);
+                        }
+                    }
+#pragma unroll
+                    for (int u = 0; u < PACK_BATCH; u++)
+                        if (h0 + 4 * u < r_hi) sh.tile[rl.lds + at[u]] = v[u];
+                }
+            __syncthreads();
+            if (wl.ok) {
+#pragma unroll 4
+                for (int h = wave; h < w_hi; h += 4) {
+                    const int2 e = sh.wr.ol[h];
+                    __builtin_nontemporal_store(sh.tile[wl.lds + e.y], dst + e.x);
                 }
             }
+        } else {
+            for (int h0 = wave; h0 < r_hi; h0 += 4 * PACK_BATCH) {
+                float v[PACK_BATCH];
+                bool in[PACK_BATCH];
 #pragma unroll
-            for (int u = 0; u < PACK_BATCH; u++)
-                if (in[u]) sh.tile[rl.lds + sh.rd.lds[h0 + 4 * u]] = v[u];
-        }
-        __syncthreads();
-        float *dst = a.dst + base_d + wl.off;
+                for (int u = 0; u < PACK_BATCH; u++) {
+                    const int h = h0 + 4 * u;
+                    in[u] = false;
+                    if (h < r_hi) {
+                        const int o = sh.rd.ol[h].x;
+                        in[u] = rl.ok && o >= 0 && rl.split + sh.rd.split[h] < rl.split_end;
+                        if (in[u]) v[u] = __builtin_nontemporal_load(src + o);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < PACK_BATCH; u++)
+                    if (in[u]) sh.tile[rl.lds + sh.rd.ol[h0 + 4 * u].y] = v[u];
+            }
+            __syncthreads();
 #pragma unroll 4
-        for (int h = wave; h < w_hi; h += 4) {
-            const int o = sh.wr.off[h];
-            if (wl.ok && o >= 0 && wl.split + sh.wr.split[h] < wl.split_end)
-                __builtin_nontemporal_store(sh.tile[wl.lds + sh.wr.lds[h]], dst + o);
+            for (int h = wave; h < w_hi; h += 4) {
+                const int2 e = sh.wr.ol[h];
+                if (wl.ok && e.x >= 0 && wl.split + sh.wr.split[h] < wl.split_end)
+                    __builtin_nontemporal_store(sh.tile[wl.lds + e.y], dst + e.x);
+            }
         }
         __syncthreads();                   // the tile and rem are free for the next round
     }
+}
+// A tile extent of at most `want` along a dimension of extent `ext`: a divisor of ext where one lies above want / 2,
+// so that no tile reaches over the edge (whole tiles take the kernel's loops without checks): 15 -> 5 rather than 8.
+int whole_tiles_extent(int ext, int want) {
+    for (int t = want; t > want / 2 && t > 1; t--)
+        if (ext % t == 0) return t;
+    return want;
 }
 // Chooses the tile of pack_tile_kernel; false when the box does not suit it (a stride that is not positive,
 // a table or tile beyond its LDS array).
@@ -257,6 +295,7 @@ bool plan_pack(const RelayoutArgs &r, PackArgs &a) {
             const int d = order[k];
             int want = 64 / p;
             if (want > a.ext[d]) want = a.ext[d];
+            want = whole_tiles_extent(a.ext[d], want);
             if (want > a.te[d]) a.te[d] = want;
             p *= a.te[d];
             if (a.te[d] < a.ext[d]) break;
@@ -276,6 +315,8 @@ bool plan_pack(const RelayoutArgs &r, PackArgs &a) {
         if (a.te[d] == a.ext[d]) continue;
         int64_t grow = PACK_TILE / elems * a.te[d];
         if (grow > a.ext[d]) grow = a.ext[d];
+        grow = whole_tiles_extent(a.ext[d], (int)grow);
+        if (grow <= a.te[d]) continue;
         elems = elems / a.te[d] * grow;
         a.te[d] = (int)grow;
     }
@@ -299,6 +340,8 @@ bool plan_pack(const RelayoutArgs &r, PackArgs &a) {
         if (rest > PACK_TABLE) return false;
         o->p_hi = (int)rest;
     }
+    a.even = (!a.rd.split_q || a.te[a.rd.dim[a.rd.n_lo]] % a.rd.split_q == 0) &&
+             (!a.wr.split_q || a.te[a.wr.dim[a.wr.n_lo]] % a.wr.split_q == 0);
     // LDS places: dense over the lanes of the source order, then an odd pitch so that the destination
     // order's lanes, which step through the rest, fall into different banks
     int64_t stride = 1;
