@@ -96,6 +96,35 @@ def capsule_case(torch, steps, warmup, peak, N, cfg, splits, workload, graph=Tru
     return e
 
 
+def capsule_packed_case(torch, steps, warmup, peak, N=8, NN=16):
+    """The capsule kernel on the reference's packed 2-D P and W and the GPU flow's 2-D V (capsule.cpp:52-53,
+    capsule-run-gpu.cpp:38-39,67-69), read and written where they lie; checked against the N-D call on the same data."""
+    L = lib()
+    CI = CO = 32
+    CII = 4
+    NT = N * NN
+    P = ops.fill_uniform(torch.empty(NT, CI, 15, 15, 4, 4, device="cuda"), 1)
+    W = ops.fill_uniform(torch.empty(CO, CI, 3, 3, 4, 4, device="cuda"), 2)
+    P2 = P.reshape(N, NN, CI, 15, 15, 4, 4).permute(0, 4, 3, 1, 5, 6, 2).contiguous().reshape(N * 225, NN * 16 * CI)
+    W2 = W.reshape(CO, CI // CII, CII, 3, 3, 4, 4).permute(5, 1, 4, 3, 2, 6, 0).contiguous().reshape(4 * CI * 9, 4 * CO)
+    V2 = torch.empty(49 * N, CO * 16 * NN, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    L.t2sp_capsule_packed_f32.argtypes = [ctypes.c_void_p, i64, ctypes.c_void_p, i64, ctypes.c_void_p, i64] + [ctypes.c_int] * 5 + [ctypes.c_void_p]
+
+    def launch():
+        rc = L.t2sp_capsule_packed_f32(P2.data_ptr(), P2.shape[1], W2.data_ptr(), W2.shape[1], V2.data_ptr(), V2.shape[1], N, NN, CI,
+                                       CO, CII, s)
+        assert rc == 0, rc
+
+    ms = _time(torch, launch, max(steps, 100), max(warmup, 10))
+    flop = 2.0 * NT * CO * 49 * 16 * CI * 9 * 4
+    e = _entry(flop / ms / 1e9, peak, ms, workload="%d images, CI=CO=32, packed P and W, 2-D V: nothing re-laid" % NT)
+    ref = ops.capsule(P, W)
+    got = V2.reshape(N, 7, 7, NN, 4, 4, CO).permute(0, 3, 6, 2, 1, 4, 5).reshape(NT, CO, 7, 7, 4, 4)
+    e["parity"] = {"rel_frobenius_against_the_n_d_call": float(((got - ref).norm() / ref.norm()).item())}
+    return e
+
+
 def _graph_replay(torch, launch_on, out, per_graph=100, replays=20):
     """The same launch recorded 100 times in a row into one HIP graph (the kernels allocate nothing and clear
     nothing, so the graph holds kernel nodes only) and replayed: the launch interval without the host in the
@@ -425,6 +454,7 @@ def _run_all(torch, steps, warmup, peak, capsule_cfg=0, capsule_splits=0):
             "sgemm_1024_a_transposed": sgemm_transposed_1024(torch, steps, warmup, peak, 1, 0),
             "sgemm_256x256x16384": sgemm_tiny_output(torch, steps, warmup, peak),
             "capsule": capsule_config4(torch, steps, warmup, peak, capsule_cfg, capsule_splits),
+            "capsule_packed_128": capsule_packed_case(torch, steps, warmup, peak),
             "mttkrp": mttkrp_config5(torch, steps, warmup, peak),
             "ssyrk_8192": ssyrk_case(torch, steps, warmup, peak, 8192, 8192, ""),
             "ssyrk_768x1024": ssyrk_case(torch, max(steps, 200), max(warmup, 20), peak, 768, 1024,
