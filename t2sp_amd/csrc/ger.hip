@@ -80,6 +80,104 @@ __global__ void __launch_bounds__(256) sger_element_kernel(const GerArgs g) {
     }
 }
 
+// The tiled output with a short innermost extent (KKK = 8 in the reference's GPU constants, 2 in its TINY set): four
+// adjacent k of a row are 16 or 32 contiguous bytes of the output and the next four lie KKK*III floats further, so
+// sger_kernel's stores, lanes side by side along k, write a different cache line every lane or two (8192 x 8192 with
+// KKK = 8: 2.4 TB/s against 6.2 for the flat output).  Here a workgroup takes rows of whole iii groups by columns of
+// whole kkk groups, reads them along k as the flat kernel does, lays the results out in LDS as the output has them,
+// runs of KKK*III floats for each (ii, kk), and writes each run with lanes side by side.  Needs the two innermost
+// output dimensions (kkk, iii) at strides 1 and KKK, and I, K whole multiples of the tile.
+struct GerTile {
+    int iic, kkc;      // ii groups and kk groups of a tile
+    int run_stride;    // floats between runs in LDS: KKK*III plus a few to spread them over the banks
+    int tpr_pad, tpu_pad;
+};
+// GRID: 256 is a multiple of the threads a row of the tile takes and of those a run takes, so a thread keeps its
+// column (and its place in a run) and steps through rows (runs) by additions; otherwise each element's row and
+// column come from divisions, which at four or more per 16 bytes make the kernel instruction-bound.
+template <bool VEC, bool GRID>
+__global__ void __launch_bounds__(256) sger_tiled_lds_kernel(const GerArgs g, const GerTile t, int tiles) {
+    extern __shared__ __align__(16) float lds_tile[];
+    __shared__ int64_t run_at[256];                   // where each run of the tile starts in the output
+    const int III = g.t_iii, KKK = g.t_kkk, run = KKK * III;
+    const int rows = III * t.iic, cols = KKK * t.kkc, col_tiles = g.K / cols, runs = t.iic * t.kkc;
+    constexpr int W = VEC ? 4 : 1;
+    const int tpr = cols / W, tpu = run / W;          // threads per row of the tile, per run
+    for (int tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+        const int ct = tile % col_tiles, rt = tile / col_tiles;
+        const int i0 = rt * rows, k0 = ct * cols;
+        if ((int)threadIdx.x < runs) {
+            const int q = threadIdx.x, kc = q / t.iic, ic = q - kc * t.iic;
+            run_at[q] = ger_tiled_offset(g, i0 + ic * III, k0 + kc * KKK);
+        }
+        auto element = [&](int r, int c, int ic, int iii, int kc, int kkk) {
+            const float xi = g.x[i0 + r];
+            float *at = lds_tile + kkk + KKK * iii + t.run_stride * (ic + t.iic * kc);
+            if (VEC) {
+                const ger_v4f a = __builtin_nontemporal_load(reinterpret_cast<const ger_v4f *>(g.A + (int64_t)(i0 + r) * g.lda + k0 + c));
+                const ger_v4f y = *reinterpret_cast<const ger_v4f *>(g.y + k0 + c);
+                ger_v4f o;
+#pragma unroll
+                for (int e = 0; e < 4; e++) o[e] = ger_value(a[e], xi, y[e]);
+                *reinterpret_cast<ger_v4f *>(at) = o;
+            } else {
+                *at = ger_value(__builtin_nontemporal_load(g.A + (int64_t)(i0 + r) * g.lda + k0 + c), xi, g.y[k0 + c]);
+            }
+        };
+        if (GRID) {
+            // (tpr_pad, tpu_pad: the powers of two from tpr and tpu up; the threads past a row's or a run's end idle)
+            const int step = 256 / t.tpr_pad, c = ((int)threadIdx.x % t.tpr_pad) * W, kc = c / KKK, kkk = c - kc * KKK;
+            int r = threadIdx.x / t.tpr_pad, ic = r / III, iii = r - ic * III;
+            if (c < cols)
+                for (; r < rows; r += step) {
+                    element(r, c, ic, iii, kc, kkk);
+                    iii += step;
+                    while (iii >= III) { iii -= III; ic++; }
+                }
+        } else {
+            for (int idx = threadIdx.x; idx < rows * tpr; idx += 256) {
+                const int r = idx / tpr, c = (idx - r * tpr) * W;
+                const int kc = c / KKK, ic = r / III;
+                element(r, c, ic, r - ic * III, kc, c - kc * KKK);
+            }
+        }
+        __syncthreads();
+        auto put = [&](int q, int p) {
+            float *dst = g.O + run_at[q] + p;
+            if (VEC)
+                __builtin_nontemporal_store(*reinterpret_cast<const ger_v4f *>(lds_tile + t.run_stride * q + p), reinterpret_cast<ger_v4f *>(dst));
+            else
+                __builtin_nontemporal_store(lds_tile[t.run_stride * q + p], dst);
+        };
+        if (GRID) {
+            const int p = ((int)threadIdx.x % t.tpu_pad) * W;
+            if (p < run)
+                for (int q = threadIdx.x / t.tpu_pad; q < runs; q += 256 / t.tpu_pad) put(q, p);
+        } else {
+            for (int idx = threadIdx.x; idx < runs * tpu; idx += 256) {
+                const int q = idx / tpu;
+                put(q, (idx - q * tpu) * W);
+            }
+        }
+        __syncthreads();
+    }
+}
+// The tile of sger_tiled_lds_kernel: whole kk groups first, then whole ii groups, up to 4096 floats; false when the
+// output or the sizes do not suit it.
+static bool plan_ger_tile(const GerArgs &g, GerTile &t) {
+    if (!g.tiled || g.s[0] != 1 || g.s[1] != g.t_kkk) return false;
+    const int64_t run = (int64_t)g.t_kkk * g.t_iii;
+    if (run > 4096 || g.I % (g.t_iii * g.t_ii) || g.K % (g.t_kkk * g.t_kk)) return false;
+    t.kkc = 1;
+    for (int d = 1; d <= g.t_kk; d++)
+        if (g.t_kk % d == 0 && run * d <= 4096) t.kkc = d;
+    t.iic = 1;
+    for (int d = 1; d <= g.t_ii; d++)
+        if (g.t_ii % d == 0 && run * t.kkc * d <= 4096) t.iic = d;
+    t.run_stride = (int)run + (g.t_kkk % 4 == 0 ? g.t_kkk : 0);
+    return g.t_kkk * t.kkc >= 16 && t.iic * t.kkc <= 256;          // a row of a tile is at least 64 contiguous bytes of A
+}
+
 static int launch_ger(const GerArgs &g, hipStream_t stream) {
     if (g.I <= 0 || g.K <= 0) return T2SP_ERR_SHAPE;
     const bool in_vec = g.K % 4 == 0 && g.lda % 4 == 0 && ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.y % 16 == 0);
@@ -92,6 +190,25 @@ static int launch_ger(const GerArgs &g, hipStream_t stream) {
     // One group of four per thread measures best (6.1 against 5.7 TB/s for a plain copy of this size with a
     // grid-stride loop over 64 workgroups per CU); the loop only serves sizes beyond the grid limit.
     if (blocks > (1 << 24)) blocks = 1 << 24;
+    GerTile gt{};
+    if (plan_ger_tile(g, gt)) {
+        const int64_t tiles = (int64_t)(g.I / (g.t_iii * gt.iic)) * (g.K / (g.t_kkk * gt.kkc));
+        const size_t lds = (size_t)gt.run_stride * gt.iic * gt.kkc * sizeof(float);
+        // 128-bit accesses: groups of four k inside a kkk group, every run and row on the 16-byte grid
+        const bool vec = in_vec && g.t_kkk % 4 == 0 && ((uintptr_t)g.O % 16 == 0) && g.s[2] % 4 == 0 && g.s[3] % 4 == 0 &&
+                         g.s[4] % 4 == 0 && g.s[5] % 4 == 0;
+        if (tiles <= INT32_MAX) {
+            const unsigned grid = (unsigned)(tiles < (1 << 20) ? tiles : (1 << 20));
+            const int w = vec ? 4 : 1, tpr = g.t_kkk * gt.kkc / w, tpu = g.t_kkk * g.t_iii / w;
+            const bool fits = tpr <= 256 && tpu <= 256;
+            for (gt.tpr_pad = 1; gt.tpr_pad < tpr; gt.tpr_pad *= 2) {}
+            for (gt.tpu_pad = 1; gt.tpu_pad < tpu; gt.tpu_pad *= 2) {}
+            auto kern = vec ? (fits ? sger_tiled_lds_kernel<true, true> : sger_tiled_lds_kernel<true, false>)
+                            : (fits ? sger_tiled_lds_kernel<false, true> : sger_tiled_lds_kernel<false, false>);
+            hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, stream, g, gt, (int)tiles);
+            return hipGetLastError() == hipSuccess ? T2SP_OK : T2SP_ERR_LAUNCH;
+        }
+    }
     if (in_vec && out_vec) {
         hipLaunchKernelGGL(sger_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, g);
     } else {
