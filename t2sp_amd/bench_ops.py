@@ -208,6 +208,32 @@ def ssyrk_case(torch, steps, warmup, peak, N, K, note):
                   **{"TFLOP/s_reference_count": round(2.0 * N * N * K / ms / 1e9, 3)})
 
 
+def sger_8192_tiled(torch, steps, warmup, peak):
+    """GER as the reference calls it: Out(kkk, iii, ii, kk, k, i) with the GPU constants of ger/const-parameters.h
+    (KKK = 8, III = 16, II = 4, KK = 4; ger-run-fpga.cpp:60), same size and traffic as the flat case."""
+    L = lib()
+    N, III, II, KKK, KK = 8192, 16, 4, 8, 4
+    A = ops.fill_uniform(torch.empty(N, N, device="cuda"), 1)
+    x = ops.fill_uniform(torch.empty(N, device="cuda"), 2)
+    y = ops.fill_uniform(torch.empty(N, device="cuda"), 3)
+    O = torch.empty(N // (III * II), N // (KKK * KK), KK, II, III, KKK, device="cuda")     # dimensions reversed, as numpy has them
+    s6 = (i64 * 6)(*reversed(O.stride()))
+    s = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        rc = L.t2sp_sger_f32_tiled(A.data_ptr(), x.data_ptr(), y.data_ptr(), O.data_ptr(), N, N, N, KKK, III, II, KK, s6, s)
+        assert rc == 0, rc
+
+    ms = _time(torch, launch, steps, warmup)
+    nbytes = 8.0 * N * N + 8.0 * N
+    flat = torch.empty(N, N, device="cuda")
+    assert L.t2sp_sger_f32(A.data_ptr(), x.data_ptr(), y.data_ptr(), flat.data_ptr(), N, N, N, N, s) == 0
+    same = torch.equal(O.permute(0, 3, 4, 1, 2, 5).reshape(N, N), flat)      # (i, ii, iii) rows by (k, kk, kkk) columns
+    return _entry(2.0 * N * N / ms / 1e9, peak, ms, workload="I=K=8192, the reference's tiled output, GPU constants",
+                  **{"bound": "hbm", "GB/s": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / 8000.0, 4),
+                     "equals_flat_result": bool(same)})
+
+
 def sger_8192(torch, steps, warmup, peak):
     """Not one of the headline benchmark configurations: the GER pipeline (t2s/tests/performance/ger) on an 8192 x 8192
     matrix.  It moves 8 bytes per element (A in, Out out; x and y are negligible) for 2 flop, so its
@@ -460,6 +486,7 @@ def _run_all(torch, steps, warmup, peak, capsule_cfg=0, capsule_splits=0):
             "ssyrk_768x1024": ssyrk_case(torch, max(steps, 200), max(warmup, 20), peak, 768, 1024,
                                          " (the size of peppers/blas/level3/syrk/release/s10)"),
             "sger_8192": sger_8192(torch, steps, warmup, peak),
+            "sger_8192_tiled": sger_8192_tiled(torch, steps, warmup, peak),
             "sgbmv3_131072x1024": sgbmv3_case(torch, steps, warmup, peak),
             "ssymv_16384": ssymv_case(torch, steps, warmup, peak),
             "pairhmm_224x224": pairhmm_case(torch, steps, warmup, peak),
