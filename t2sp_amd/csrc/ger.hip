@@ -174,6 +174,19 @@ static bool plan_ger_tile(const GerArgs &g, GerTile &t) {
     t.iic = 1;
     for (int d = 1; d <= g.t_ii; d++)
         if (g.t_ii % d == 0 && run * t.kkc * d <= 4096) t.iic = d;
+    // Small constants (a whole kkk x kk block under 128 bytes of a row, as in the reference's TINY set): the tile spans
+    // several blocks along k, up to 256 bytes of a row, and then several along i; the runs' addresses are computed run
+    // by run, so a tile may cross blocks, and in the dense output the runs of a tile then follow one another.
+    if (g.t_kkk * g.t_kk < 32 && t.kkc == g.t_kk && t.iic == g.t_ii) {
+        const int k_blocks = g.K / (g.t_kkk * g.t_kk), i_blocks = g.I / (g.t_iii * g.t_ii);
+        int m = 1, n = 1;
+        for (int d = 1; d <= k_blocks && g.t_kkk * g.t_kk * d <= 64; d++)
+            if (k_blocks % d == 0 && run * g.t_kk * d * g.t_ii <= 4096 && g.t_kk * d * g.t_ii <= 256) m = d;
+        for (int d = 1; d <= i_blocks; d++)
+            if (i_blocks % d == 0 && run * g.t_kk * m * g.t_ii * d <= 4096 && g.t_kk * m * g.t_ii * d <= 256) n = d;
+        t.kkc = g.t_kk * m;
+        t.iic = g.t_ii * n;
+    }
     t.run_stride = (int)run + (g.t_kkk % 4 == 0 ? g.t_kkk : 0);
     return g.t_kkk * t.kkc >= 16 && t.iic * t.kkc <= 256;          // a row of a tile is at least 64 contiguous bytes of A
 }

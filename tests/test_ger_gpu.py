@@ -43,12 +43,14 @@ def test_padded_rows_and_tiled_with_odd_inner_extent(oracle):
 
 
 @pytest.mark.parametrize("tiles,I,K,pad", [((3, 2, 6, 4), 30, 168, 0), ((16, 4, 8, 4), 192, 96, 4), ((14, 32, 16, 32), 448, 1024, 0),
-                                           ((7, 3, 12, 5), 42, 240, 8), ((5, 1, 4, 4), 35, 64, 0), ((64, 8, 8, 2), 1024, 64, 0)])
+                                           ((7, 3, 12, 5), 42, 240, 8), ((5, 1, 4, 4), 35, 64, 0), ((64, 8, 8, 2), 1024, 64, 0), ((2, 2, 2, 2), 256, 512, 0),
+                                           ((4, 4, 4, 4), 160, 96, 4), ((3, 2, 2, 3), 36, 180, 0)])
 def test_tiled_output_through_lds_bit_exact(oracle, tiles, I, K, pad):
     """The tiled output's kernel that lays a tile out in LDS as the output has it (rows of whole iii groups by
     columns of whole kkk groups, runs of KKK*III floats written side by side): innermost extents on and off the
     4-element grid, runs that are not a power of two long (threads past a run's end idle), one ii group or several
-    per tile, A with padded rows.  Against the oracle's tiling of the flat result, bit for bit."""
+    per tile, small constants whose tiles span several blocks along k and i, A with padded rows.  Against the oracle's
+    tiling of the flat result, bit for bit."""
     III, II, KKK, KK = tiles
     Ap = oracle.fill_uniform((I, K + pad), 101)
     A, x, y = Ap[:, :K], oracle.fill_uniform((I,), 102), oracle.fill_uniform((K,), 103)
